@@ -1,0 +1,513 @@
+"""HIP source emitters for elementwise kernels (gfx950).
+
+Three kernel shapes are produced from one loop body:
+
+``flat``     every array operand walks memory linearly (contiguous, or a single
+             broadcast element): 128-bit vector loads/stores, grid-stride over
+             vectors, scalar tail.
+``tiled2d``  two-dimensional problems where each operand is contiguous along
+             one of the two axes (row-major operands, row/column broadcasts and
+             transposed operands): transposed operands go through an LDS tile
+             so that every global access is coalesced.
+``generic``  anything else: CIndexer/CArray addressing per element, the same
+             semantics as the reference's kernel template
+             (cupy/_core/_kernel.pyx:78-107,709-728) including ``continue`` in
+             the body and outputs that are read before they are written.
+
+The body sees the names the reference provides: the parameters, ``i`` (linear
+index) and ``_ind``.
+"""
+import re
+
+BLOCK = 256
+
+
+class Operand:
+    """One kernel parameter as the emitters see it.
+
+    kind        'array' (broadcast, iterated), 'raw' (CArray handed to the body
+                untouched), 'scalar' (by value) or 'indexer'
+    name        identifier used by the body
+    store_t     C type of an element in memory / of the scalar argument
+    var_t       C type of the variable the body sees
+    is_out      True for output arrays
+    read_out    outputs only: load the old element before running the body
+    cast_in     callable(expr) -> expr converting a loaded element to var_t
+    cast_out    callable(expr) -> expr converting the variable to store_t
+    ndim, c_contiguous, index_32   CArray template arguments (raw / generic)
+    """
+
+    def __init__(self, kind, name, store_t, var_t=None, is_out=False,
+                 read_out=False, cast_in=None, cast_out=None, ndim=0,
+                 c_contiguous=False, index_32=True, is_const=True):
+        self.kind = kind
+        self.name = name
+        self.store_t = store_t
+        self.var_t = var_t or store_t
+        self.is_out = is_out
+        self.read_out = read_out
+        self.cast_in = cast_in or (lambda e: e)
+        self.cast_out = cast_out or (lambda e: e)
+        self.ndim = ndim
+        self.c_contiguous = c_contiguous
+        self.index_32 = index_32
+        self.is_const = is_const
+
+    def key(self):
+        return (self.kind, self.name, self.store_t, self.var_t, self.is_out,
+                self.read_out, self.ndim, self.c_contiguous, self.index_32,
+                self.is_const, self.cast_in('@'), self.cast_out('@'))
+
+
+_ident_cache = {}
+
+
+def uses_identifier(code, ident):
+    """True if ``ident`` appears in ``code`` as a whole word."""
+    key = (code, ident)
+    hit = _ident_cache.get(key)
+    if hit is None:
+        hit = re.search(r'(?<![A-Za-z0-9_])%s(?![A-Za-z0-9_])' % re.escape(ident),
+                        code) is not None
+        if len(_ident_cache) < 4096:
+            _ident_cache[key] = hit
+    return hit
+
+
+def output_is_write_only(operation, name):
+    """Conservative test that the body assigns ``name`` unconditionally before
+    any other use: its first occurrence is ``name = ...`` as a statement at
+    brace depth 0 that is not governed by ``if``/``else``/a loop.  Anything
+    else (compound assignment, assignment inside a branch, a read) makes the
+    emitter load the previous value first, which reproduces reference
+    semantics where the variable is a reference to the element in memory."""
+    m = re.search(r'(?<![A-Za-z0-9_])%s(?![A-Za-z0-9_])' % re.escape(name), operation)
+    if m is None:
+        return False
+    head = operation[:m.start()]
+    tail = operation[m.end():]
+    if not re.match(r'\s*=(?!=)', tail):
+        return False
+    if head.count('{') != head.count('}'):
+        return False
+    if head.count('(') != head.count(')'):
+        return False
+    stmt_start = max(head.rfind(';'), head.rfind('}'))
+    stmt_head = head[stmt_start + 1:]
+    return stmt_head.strip() == ''
+
+
+def body_needs_generic(operation):
+    """Bodies that steer the element loop themselves need the one-element-per-
+    iteration loop of the generic kernel."""
+    return (uses_identifier(operation, 'continue')
+            or uses_identifier(operation, 'return')
+            or uses_identifier(operation, 'break')
+            or uses_identifier(operation, 'goto'))
+
+
+def _param_decl(op):
+    if op.kind == 'array':
+        const = 'const ' if (op.is_const and not op.is_out) else ''
+        return '%s%s* _p_%s' % (const, op.store_t, op.name)
+    if op.kind == 'raw':
+        const = 'const ' if op.is_const else ''
+        return '%sCArray<%s, %d, %d, %d> %s' % (
+            const, op.store_t, op.ndim, op.c_contiguous, op.index_32, op.name)
+    if op.kind == 'scalar':
+        return 'const %s %s' % (op.store_t, op.name)
+    if op.kind == 'indexer':
+        return 'CIndexer<%d, %d> %s' % (op.ndim, op.index_32, op.name)
+    raise AssertionError(op.kind)
+
+
+def _header(typedefs, preamble):
+    return ('#include <cupy/carray.cuh>\n' + typedefs + '\n' + preamble + '\n')
+
+
+def _element_code(operands, operation, load_expr, store_stmt, indent):
+    """Per-element code: declare the body variables from ``load_expr(op)``,
+    run the body, hand results to ``store_stmt(op, value_expr)``."""
+    pad = ' ' * indent
+    lines = []
+    for op in operands:
+        if op.kind != 'array':
+            continue
+        if not op.is_out:
+            lines.append('%sconst %s %s(%s);' % (
+                pad, op.var_t, op.name, op.cast_in(load_expr(op))))
+        elif op.read_out:
+            lines.append('%s%s %s(%s);' % (
+                pad, op.var_t, op.name, op.cast_in(load_expr(op))))
+        else:
+            lines.append('%s%s %s;' % (pad, op.var_t, op.name))
+    lines.append('%s{ %s; }' % (pad, operation))
+    for op in operands:
+        if op.kind == 'array' and op.is_out:
+            lines.append(pad + store_stmt(op, op.cast_out(op.name)))
+    return '\n'.join(lines)
+
+
+def emit_flat(name, operands, operation, typedefs='', preamble='',
+              loop_prep='', after_loop='', vec=4, unroll=1, idx64=False,
+              bcast=(), stream_hint=True, block=BLOCK):
+    """Kernel for operands that are all contiguous.
+
+    ``bcast`` names array operands that hold a single element broadcast over
+    the whole index space.  Trailing parameters of the kernel: the array
+    pointers / scalars / raw arrays in operand order, then ``_n`` (element
+    count) and, when the body uses it, ``_ind``.
+    """
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    uidx_t = 'ptrdiff_t' if idx64 else 'unsigned int'
+    arrays = [op for op in operands if op.kind == 'array']
+    iter_arrays = [op for op in arrays if op.name not in bcast]
+    needs_ind = any(op.kind == 'indexer' for op in operands)
+    params = ', '.join([_param_decl(op) for op in operands if op.kind != 'indexer']
+                       + ['const %s _n' % idx_t]
+                       + [_param_decl(op) for op in operands if op.kind == 'indexer'])
+    nt = 'true' if stream_hint else 'false'
+    use_i = uses_identifier(operation, 'i')
+    set_ind = '_ind.set(i);' if needs_ind and uses_identifier(operation, '_ind') else ''
+
+    def bcast_decls():
+        out = []
+        for op in arrays:
+            if op.name in bcast and not op.is_out:
+                out.append('  const %s _b_%s = _p_%s[0];' % (
+                    op.store_t, op.name, op.name))
+        return '\n'.join(out)
+
+    def vec_load_expr(suffix):
+        def f(op):
+            if op.name in bcast:
+                return '_b_%s' % op.name
+            return '_l_%s%s.v[_k]' % (op.name, suffix)
+        return f
+
+    def vec_store_stmt(suffix):
+        def f(op, value):
+            return '_l_%s%s.v[_k] = %s;' % (op.name, suffix, value)
+        return f
+
+    def vec_block(suffix, base_expr, indent):
+        pad = ' ' * indent
+        lines = []
+        return lines
+
+    # --- vector part: `unroll` vectors per thread per trip -----------------------
+    body = []
+    body.append('  const %s _nvec = _n / %d;' % (idx_t, vec))
+    body.append('  const %s _gstride = (%s)gridDim.x * %d;' % (idx_t, idx_t, block * unroll))
+    body.append('  for (%s _v0 = (%s)blockIdx.x * %d + threadIdx.x; _v0 < _nvec; '
+                '_v0 += _gstride) {' % (idx_t, idx_t, block * unroll))
+    if unroll > 1:
+        body.append('    if (_v0 + %d < _nvec) {' % ((unroll - 1) * block))
+        # all loads first, so that `unroll` independent requests are in flight
+        for u in range(unroll):
+            for op in iter_arrays:
+                if (not op.is_out) or op.read_out:
+                    body.append(
+                        '      cupy::Vec<%s, %d> _l_%s_%d = cupy::load_vec<%s, %d, %s>('
+                        '_p_%s + (_v0 + %d) * %d);' % (
+                            op.store_t, vec, op.name, u, op.store_t, vec, nt,
+                            op.name, u * block, vec))
+                else:
+                    body.append('      cupy::Vec<%s, %d> _l_%s_%d;' % (
+                        op.store_t, vec, op.name, u))
+        for u in range(unroll):
+            body.append('      {')
+            body.append('        const %s _base = (_v0 + %d) * %d;' % (idx_t, u * block, vec))
+            body.append('#pragma unroll')
+            body.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
+            if use_i or set_ind:
+                body.append('          const ptrdiff_t i = _base + _k; %s' % set_ind)
+            body.append(_element_code(
+                operands, operation, vec_load_expr('_%d' % u),
+                vec_store_stmt('_%d' % u), 10))
+            body.append('        }')
+            for op in iter_arrays:
+                if op.is_out:
+                    body.append(
+                        '        cupy::store_vec<%s, %d, %s>(_p_%s + _base, _l_%s_%d);' % (
+                            op.store_t, vec, nt, op.name, op.name, u))
+            body.append('      }')
+        body.append('    } else {')
+        body.append('      for (%s _v = _v0; _v < _nvec; _v += %d) {' % (idx_t, block))
+        inner_pad = 8
+    else:
+        body.append('    {')
+        body.append('      const %s _v = _v0; {' % idx_t)
+        inner_pad = 8
+    pad = ' ' * inner_pad
+    body.append('%sconst %s _base = _v * %d;' % (pad, idx_t, vec))
+    for op in iter_arrays:
+        if (not op.is_out) or op.read_out:
+            body.append('%scupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>('
+                        '_p_%s + _base);' % (pad, op.store_t, vec, op.name,
+                                             op.store_t, vec, nt, op.name))
+        else:
+            body.append('%scupy::Vec<%s, %d> _l_%s;' % (pad, op.store_t, vec, op.name))
+    body.append('#pragma unroll')
+    body.append('%sfor (int _k = 0; _k < %d; ++_k) {' % (pad, vec))
+    if use_i or set_ind:
+        body.append('%s  const ptrdiff_t i = _base + _k; %s' % (pad, set_ind))
+    body.append(_element_code(operands, operation, vec_load_expr(''),
+                              vec_store_stmt(''), inner_pad + 2))
+    body.append('%s}' % pad)
+    for op in iter_arrays:
+        if op.is_out:
+            body.append('%scupy::store_vec<%s, %d, %s>(_p_%s + _base, _l_%s);' % (
+                pad, op.store_t, vec, nt, op.name, op.name))
+    body.append('      }')
+    body.append('    }')
+    body.append('  }')
+
+    # --- scalar tail ----------------------------------------------------------------
+    def tail_load(op):
+        if op.name in bcast:
+            return '_b_%s' % op.name
+        return '_p_%s[_t]' % op.name
+
+    def tail_store(op, value):
+        return '_p_%s[_t] = %s;' % (op.name, value)
+
+    tail = []
+    tail.append('  for (%s _t = _nvec * %d + (%s)blockIdx.x * %d + threadIdx.x; _t < _n; '
+                '_t += (%s)gridDim.x * %d) {' % (idx_t, vec, idx_t, block, idx_t, block))
+    if use_i or set_ind:
+        tail.append('    const ptrdiff_t i = _t; %s' % set_ind)
+    tail.append(_element_code(operands, operation, tail_load, tail_store, 4))
+    tail.append('  }')
+
+    src = [_header(typedefs, preamble)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        block, name, params))
+    src.append('  %s;' % loop_prep)
+    b = bcast_decls()
+    if b:
+        src.append(b)
+    if vec > 1:
+        src.extend(body)
+    else:
+        src.append('  const %s _nvec = 0;' % idx_t)
+    src.extend(tail)
+    src.append('  %s;' % after_loop)
+    src.append('}')
+    del uidx_t, vec_block
+    return '\n'.join(src) + '\n'
+
+
+def emit_generic(name, operands, operation, typedefs='', preamble='',
+                 loop_prep='', after_loop='', block=128):
+    """Reference-semantics kernel: one element per loop trip, operands
+    addressed through CArray/CIndexer, body variables are references into
+    memory (so ``continue``, partial writes and in-place reads all behave as
+    in the reference)."""
+    parts = []
+    for op in operands:
+        if op.kind == 'array':
+            const = 'const ' if (op.is_const and not op.is_out) else ''
+            parts.append('%sCArray<%s, %d, %d, %d> _raw_%s' % (
+                const, op.store_t, op.ndim, op.c_contiguous, op.index_32, op.name))
+        else:
+            parts.append(_param_decl(op))
+    params = ', '.join(parts)
+    lines = []
+    for op in operands:
+        if op.kind != 'array':
+            continue
+        same = op.cast_in('@') == '@' and op.cast_out('@') == '@' and \
+            op.store_t == op.var_t
+        if same or op.var_t == op.store_t:
+            if op.is_out:
+                lines.append('    %s &%s = _raw_%s[_ind.get()];' % (
+                    op.var_t, op.name, op.name))
+            else:
+                lines.append('    const %s &%s = _raw_%s[_ind.get()];' % (
+                    op.var_t, op.name, op.name))
+        elif op.is_out:
+            if op.read_out:
+                lines.append('    %s %s(%s);' % (op.var_t, op.name, op.cast_in(
+                    '_raw_%s[_ind.get()]' % op.name)))
+            else:
+                lines.append('    %s %s;' % (op.var_t, op.name))
+        else:
+            lines.append('    const %s %s(%s);' % (op.var_t, op.name, op.cast_in(
+                '_raw_%s[_ind.get()]' % op.name)))
+    lines.append('    %s;' % operation)
+    for op in operands:
+        if op.kind == 'array' and op.is_out and op.var_t != op.store_t:
+            lines.append('    _raw_%s[_ind.get()] = %s;' % (
+                op.name, op.cast_out(op.name)))
+    src = [_header(typedefs, preamble)]
+    src.append('extern "C" __global__ void %s(%s) {' % (name, params))
+    src.append('  %s;' % loop_prep)
+    src.append('#pragma unroll 1')
+    src.append('  CUPY_FOR(i, _ind.size()) {')
+    src.append('    _ind.set(i);')
+    src.extend(lines)
+    src.append('  }')
+    src.append('  %s;' % after_loop)
+    src.append('}')
+    del block
+    return '\n'.join(src) + '\n'
+
+
+def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
+                 loop_prep='', after_loop='', layouts=None, vec=4, tile=64,
+                 idx64=False, stream_hint=True):
+    """Kernel for a 2-d index space (rows r, columns c) where every array
+    operand is contiguous along one axis.
+
+    ``layouts[name]`` is 'R' (unit or zero stride along columns; any stride
+    along rows) or 'C' (unit stride along rows, any stride along columns: a
+    transposed operand).  'C' inputs are staged through an LDS tile: the tile is
+    read from memory along rows (coalesced) and consumed along columns.  Outputs
+    must be 'R'.
+
+    Work split: a workgroup of 256 threads owns a ``tile`` x ``tile`` block.
+    For 'R' operands thread (ty, tx) handles ``vec`` consecutive columns
+    starting at tx*vec of rows ty, ty+TY, ...  Kernel parameters after the
+    operands: ``_nr, _nc`` (extent), then per array its row stride and column
+    stride in elements.
+    """
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    arrays = [op for op in operands if op.kind == 'array']
+    needs_ind = any(op.kind == 'indexer' for op in operands)
+    tx_n = tile // vec            # threads across the columns of a tile
+    ty_n = BLOCK // tx_n          # rows covered per pass
+    passes = tile // ty_n
+    assert tx_n * ty_n == BLOCK and passes * ty_n == tile
+    nt = 'true' if stream_hint else 'false'
+    use_i = uses_identifier(operation, 'i')
+    set_ind = '_ind.set(i);' if needs_ind and uses_identifier(operation, '_ind') else ''
+
+    parts = [_param_decl(op) for op in operands if op.kind != 'indexer']
+    parts += ['const %s _nr' % idx_t, 'const %s _nc' % idx_t]
+    for op in arrays:
+        parts += ['const %s _sr_%s' % (idx_t, op.name),
+                  'const %s _sc_%s' % (idx_t, op.name)]
+    parts += [_param_decl(op) for op in operands if op.kind == 'indexer']
+    params = ', '.join(parts)
+
+    c_ops = [op for op in arrays if layouts[op.name] == 'C']
+    for op in c_ops:
+        assert not op.is_out, 'transposed outputs are not handled by tiled2d'
+
+    src = [_header(typedefs, preamble)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, params))
+    src.append('  %s;' % loop_prep)
+    for op in c_ops:
+        # +1 element of padding per tile row keeps the column-wise reads off a
+        # single LDS bank.
+        src.append('  __shared__ %s _t_%s[%d][%d];' % (
+            op.store_t, op.name, tile, tile + 1))
+    src.append('  const int _tx = threadIdx.x %% %d;' % tx_n)
+    src.append('  const int _ty = threadIdx.x / %d;' % tx_n)
+    src.append('  const %s _ntr = (_nr + %d) / %d;' % (idx_t, tile - 1, tile))
+    src.append('  const %s _ntc = (_nc + %d) / %d;' % (idx_t, tile - 1, tile))
+    src.append('  for (%s _tile = blockIdx.x; _tile < _ntr * _ntc; _tile += gridDim.x) {' % idx_t)
+    src.append('    const %s _r0 = (_tile / _ntc) * %d;' % (idx_t, tile))
+    src.append('    const %s _c0 = (_tile %% _ntc) * %d;' % (idx_t, tile))
+    if c_ops:
+        # Stage transposed operands: walk the tile with rows as the fast
+        # direction.  Thread (ty, tx): rows r0 + tx*vec .. +vec, column c0 + ty (+TY..).
+        src.append('    {')
+        src.append('      const %s _rr = _r0 + _tx * %d;' % (idx_t, vec))
+        src.append('      const bool _rfull = _rr + %d <= _nr;' % vec)
+        src.append('#pragma unroll')
+        src.append('      for (int _p = 0; _p < %d; ++_p) {' % passes)
+        src.append('        const %s _cc = _c0 + _ty + _p * %d;' % (idx_t, ty_n))
+        src.append('        if (_cc < _nc) {')
+        for op in c_ops:
+            src.append('          if (_rfull) {')
+            src.append('            cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>('
+                       '_p_%s + _rr + (ptrdiff_t)_cc * _sc_%s);' % (
+                           op.store_t, vec, op.store_t, vec, nt, op.name, op.name))
+            src.append('#pragma unroll')
+            src.append('            for (int _k = 0; _k < %d; ++_k) '
+                       '_t_%s[_tx * %d + _k][_ty + _p * %d] = _lv.v[_k];' % (
+                           vec, op.name, vec, ty_n))
+            src.append('          } else {')
+            src.append('            for (int _k = 0; _k < %d; ++_k) if (_rr + _k < _nr) '
+                       '_t_%s[_tx * %d + _k][_ty + _p * %d] = '
+                       '_p_%s[_rr + _k + (ptrdiff_t)_cc * _sc_%s];' % (
+                           vec, op.name, vec, ty_n, op.name, op.name))
+            src.append('          }')
+        src.append('        }')
+        src.append('      }')
+        src.append('    }')
+        src.append('    __syncthreads();')
+    # Consume: thread (ty, tx) handles row r0 + ty + p*TY, columns c0 + tx*vec ..
+    src.append('    const %s _cb = _c0 + _tx * %d;' % (idx_t, vec))
+    src.append('    const bool _cfull = _cb + %d <= _nc;' % vec)
+    src.append('#pragma unroll')
+    src.append('    for (int _p = 0; _p < %d; ++_p) {' % passes)
+    src.append('      const int _lr = _ty + _p * %d;' % ty_n)
+    src.append('      const %s _r = _r0 + _lr;' % idx_t)
+    src.append('      if (_r < _nr && _cb < _nc) {')
+
+    def r_ptr(op):
+        return '(_p_%s + (ptrdiff_t)_r * _sr_%s + (ptrdiff_t)_cb * _sc_%s)' % (
+            op.name, op.name, op.name)
+
+    # full-width path ------------------------------------------------------------------
+    src.append('        if (_cfull) {')
+    for op in arrays:
+        if layouts[op.name] == 'R':
+            if (not op.is_out) or op.read_out:
+                src.append('          cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+                src.append('          if (_sc_%s == 1) _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
+                    op.name, op.name, op.store_t, vec, nt, r_ptr(op)))
+                src.append('          else { const %s _bv = *%s;' % (op.store_t, r_ptr(op)))
+                src.append('#pragma unroll')
+                src.append('            for (int _k = 0; _k < %d; ++_k) _l_%s.v[_k] = _bv; }' % (
+                    vec, op.name))
+            else:
+                src.append('          cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+
+    def full_load(op):
+        if layouts[op.name] == 'C':
+            return '_t_%s[_lr][_tx * %d + _k]' % (op.name, vec)
+        return '_l_%s.v[_k]' % op.name
+
+    def full_store(op, value):
+        return '_l_%s.v[_k] = %s;' % (op.name, value)
+
+    src.append('#pragma unroll')
+    src.append('          for (int _k = 0; _k < %d; ++_k) {' % vec)
+    if use_i or set_ind:
+        src.append('            const ptrdiff_t i = (ptrdiff_t)_r * _nc + _cb + _k; %s' % set_ind)
+    src.append(_element_code(operands, operation, full_load, full_store, 12))
+    src.append('          }')
+    for op in arrays:
+        if op.is_out:
+            src.append('          cupy::store_vec<%s, %d, %s>(%s, _l_%s);' % (
+                op.store_t, vec, nt, r_ptr(op), op.name))
+    src.append('        } else {')
+
+    # ragged right edge ----------------------------------------------------------------
+    def edge_load(op):
+        if layouts[op.name] == 'C':
+            return '_t_%s[_lr][_tx * %d + _k]' % (op.name, vec)
+        return '%s[(ptrdiff_t)_k * _sc_%s]' % (r_ptr(op), op.name)
+
+    def edge_store(op, value):
+        return '%s[(ptrdiff_t)_k * _sc_%s] = %s;' % (r_ptr(op), op.name, value)
+
+    src.append('          for (int _k = 0; _k < %d && _cb + _k < _nc; ++_k) {' % vec)
+    if use_i or set_ind:
+        src.append('            const ptrdiff_t i = (ptrdiff_t)_r * _nc + _cb + _k; %s' % set_ind)
+    src.append(_element_code(operands, operation, edge_load, edge_store, 12))
+    src.append('          }')
+    src.append('        }')
+    src.append('      }')
+    src.append('    }')
+    if c_ops:
+        src.append('    __syncthreads();')
+    src.append('  }')
+    src.append('  %s;' % after_loop)
+    src.append('}')
+    return '\n'.join(src) + '\n'

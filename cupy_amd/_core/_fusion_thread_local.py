@@ -1,0 +1,22 @@
+"""Thread-local switch telling ufuncs and reductions that a ``cupy.fuse``
+trace is in progress (reference: cupy/_core/_fusion_thread_local.pyx:1-46)."""
+import threading
+
+thread_local = threading.local()
+
+
+def is_fusing():
+    return getattr(thread_local, 'history', None) is not None
+
+
+def is_old_fusing():
+    return getattr(thread_local, 'is_old_fusing', False)
+
+
+def call_ufunc(fusion_op, *args, **kwargs):
+    return thread_local.history.call_ufunc(fusion_op, *args, **kwargs)
+
+
+def call_reduction(fusion_op, *args, **kwargs):
+    from cupy_amd._core import fusion
+    return fusion._call_reduction(fusion_op, *args, **kwargs)

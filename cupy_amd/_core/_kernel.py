@@ -1,0 +1,1334 @@
+"""ElementwiseKernel, ufunc and their shared host machinery.
+
+Public behaviour follows the reference's cupy/_core/_kernel.pyx
+(ParameterInfo :464-525, type resolution :557-604, broadcasting :607-640,
+output handling :646-706, ElementwiseKernel :743-1002, ufunc :1147-1493,
+loop selection :1532-1753); what happens below the call surface -- stride
+canonicalisation into launch plans, the HIP emitters, argument packing -- is
+specific to this implementation.
+"""
+import struct
+import threading
+import warnings
+
+import numpy
+
+from cupy_amd._core import _carray
+from cupy_amd._core import _codegen_elementwise as _cg
+from cupy_amd._core import _fusion_thread_local
+from cupy_amd._core import _scalar
+from cupy_amd._core import internal
+from cupy_amd._core._dtype import get_dtype, _raise_if_invalid_cast
+from cupy_amd._core._scalar import CScalar, get_typename as _get_typename
+from cupy_amd._core.core import ndarray, _convert_from_cupy_like
+from cupy_amd.cuda import compiler
+from cupy_amd.cuda import device as _device
+from cupy_amd.cuda import stream as _stream
+
+_INT32_MAX = (1 << 31) - 1
+
+
+# ---------------------------------------------------------------------------------
+# parameters and type placeholders
+# ---------------------------------------------------------------------------------
+
+class ParameterInfo:
+    """One entry of an ``in_params`` / ``out_params`` string:
+    ``[raw] [_non_const] <dtype name | single-letter placeholder> <name>``."""
+
+    def __init__(self, param, is_const):
+        self.name = None
+        self.dtype = None
+        self.ctype = None
+        self.raw = False
+        self.is_const = is_const
+        s = tuple(i for i in param.split() if len(i) != 0)
+        if len(s) < 2:
+            raise Exception('Syntax error: %s' % param)
+        t, self.name = s[-2:]
+        if t == 'CIndexer':
+            pass
+        elif len(t) == 1:
+            self.ctype = t
+        else:
+            dtype = get_dtype(t)
+            self.dtype = dtype
+            self.ctype = _get_typename(dtype)
+        for i in s[:-2]:
+            if i == 'raw':
+                self.raw = True
+            elif i == '_non_const':
+                self.is_const = False
+            else:
+                raise Exception('Unknown keyword "%s"' % i)
+
+    def _key(self):
+        return (self.name, self.dtype, self.ctype, self.raw, self.is_const)
+
+    def __hash__(self):
+        return hash(self._key())
+
+    def __eq__(self, other):
+        return isinstance(other, ParameterInfo) and self._key() == other._key()
+
+    def __repr__(self):
+        return '<ParameterInfo name=%r dtype=%r ctype=%r raw=%r is_const=%r>' % (
+            self._key())
+
+
+_param_info_memo = {}
+
+
+def _get_param_info(s, is_const):
+    key = (s, is_const)
+    ret = _param_info_memo.get(key)
+    if ret is None:
+        if len(s) == 0:
+            ret = ()
+        else:
+            ret = tuple(ParameterInfo(i, is_const) for i in s.strip().split(','))
+        _param_info_memo[key] = ret
+    return ret
+
+
+class _TypeMap:
+    """Resolved type placeholders: pairs (placeholder, dtype)."""
+
+    def __init__(self, pairs):
+        self._pairs = tuple(pairs)
+
+    def __hash__(self):
+        return hash(self._pairs)
+
+    def __eq__(self, other):
+        return isinstance(other, _TypeMap) and self._pairs == other._pairs
+
+    def __str__(self):
+        return '<_TypeMap {}>'.format(self._pairs)
+
+    def get_typedef_code(self):
+        return ''.join('typedef %s %s;\n' % (_get_typename(t), name)
+                       for name, t in self._pairs)
+
+
+def _decide_params_type_core(in_params, out_params, in_args_dtype, out_args_dtype):
+    """Binds single-letter type placeholders from the dtypes of the array
+    arguments (outputs first) and checks fixed-dtype parameters."""
+    type_dict = {}
+    if out_args_dtype:
+        assert len(out_params) == len(out_args_dtype)
+        for p, a in zip(out_params, out_args_dtype):
+            if a is None:
+                raise TypeError('Output arguments must be cupy.ndarray')
+            if p.dtype is not None:
+                if get_dtype(a) != get_dtype(p.dtype):
+                    raise TypeError(
+                        'Type is mismatched. %s %s %s' % (p.name, a, p.dtype))
+            elif p.ctype in type_dict:
+                t = type_dict[p.ctype]
+                if get_dtype(t) != get_dtype(a):
+                    raise TypeError('Type is mismatched. %s %s %s %s' % (
+                        p.name, a, t, p.ctype))
+            else:
+                type_dict[p.ctype] = a
+    assert len(in_params) == len(in_args_dtype)
+    for p, a in zip(in_params, in_args_dtype):
+        if a is None:
+            continue
+        if p.dtype is not None:
+            if numpy.dtype(a) != numpy.dtype(p.dtype):
+                raise TypeError(
+                    'Type is mismatched. %s %s %s' % (p.name, a, p.dtype))
+        elif p.ctype in type_dict:
+            t = type_dict[p.ctype]
+            if numpy.dtype(t) != numpy.dtype(a):
+                raise TypeError('Type is mismatched. %s %s %s %s' % (
+                    p.name, a, t, p.ctype))
+        else:
+            type_dict[p.ctype] = a
+    in_types = tuple(type_dict[p.ctype] if p.dtype is None else p.dtype
+                     for p in in_params)
+    out_types = tuple(type_dict[p.ctype] if p.dtype is None else p.dtype
+                      for p in out_params)
+    type_map = _TypeMap(sorted(type_dict.items(), key=lambda kv: kv[0]))
+    return in_types, out_types, type_map
+
+
+_decide_memo = {}
+
+
+def _decide_params_type(in_params, out_params, in_args_dtype, out_args_dtype):
+    key = (in_params, out_params, in_args_dtype, out_args_dtype)
+    ret = _decide_memo.get(key)
+    if ret is None:
+        ret = _decide_params_type_core(
+            in_params, out_params, in_args_dtype, out_args_dtype)
+        _decide_memo[key] = ret
+    return ret
+
+
+# ---------------------------------------------------------------------------------
+# argument handling
+# ---------------------------------------------------------------------------------
+
+def _check_peer_access(arr, device_id):
+    if arr.data.device_id == device_id:
+        return
+    raise ValueError(
+        'The device where the array resides ({}) is different from the current '
+        'device ({}). Peer access is unavailable between these devices.'.format(
+            arr.data.device_id, device_id))
+
+
+def _preprocess_arg(dev_id, arg):
+    if type(arg) is ndarray:
+        s = arg
+    else:
+        s = _convert_from_cupy_like(arg, error=False)
+    if s is not None:
+        if s.data.device_id != dev_id:
+            _check_peer_access(s, dev_id)
+        return s
+    return CScalar(arg)
+
+
+def _preprocess_args(dev_id, args):
+    return [_preprocess_arg(dev_id, a) for a in args]
+
+
+def _preprocess_optional_args(dev_id, args):
+    return [None if a is None else _preprocess_arg(dev_id, a) for a in args]
+
+
+def _broadcast(args, params, use_size):
+    """Broadcasts the non-raw arrays of ``args`` against each other.
+    Returns (new args, broadcast shape)."""
+    value = []
+    any_nonraw_array = False
+    for a, p in zip(args, params):
+        if not p.raw and isinstance(a, ndarray):
+            any_nonraw_array = True
+            value.append(a)
+        else:
+            value.append(None)
+    if use_size:
+        if any_nonraw_array:
+            raise ValueError('Specified \'size\' can be used only '
+                             'if all of the ndarray are \'raw\'.')
+    else:
+        if not any_nonraw_array:
+            raise ValueError('Loop size is undecided.')
+    shape = internal._broadcast_core(value)
+    for i, a in enumerate(value):
+        if a is None:
+            value[i] = args[i]
+    return value, shape
+
+
+def _get_out_args_from_optionals(subtype, out_args, out_types, out_shape, casting, obj):
+    out_args = list(out_args)
+    while len(out_args) < len(out_types):
+        out_args.append(None)
+    for i, a in enumerate(out_args):
+        if a is None:
+            arr = ndarray._new_contiguous(out_shape, out_types[i])
+            if subtype is not ndarray:
+                arr = arr._retype(subtype, obj)
+            out_args[i] = arr
+            continue
+        if not isinstance(a, ndarray):
+            raise TypeError('Output arguments type must be cupy.ndarray')
+        if a._shape != out_shape:
+            raise ValueError('Out shape is mismatched')
+        out_type = get_dtype(out_types[i])
+        _raise_if_invalid_cast(out_type, a.dtype, casting, 'output operand')
+    return out_args
+
+
+def _copy_in_args_if_needed(in_args, out_args):
+    """Inputs that overlap an explicit output (without being that very array)
+    are copied first, so the kernel never reads what it has already written."""
+    for i, a in enumerate(in_args):
+        if isinstance(a, ndarray):
+            for out in out_args:
+                if a is not out and _carray.may_share_bounds(a, out):
+                    in_args[i] = a.copy()
+                    break
+
+
+def _get_out_args_with_params(out_args, out_types, out_shape, out_params,
+                              is_size_specified):
+    if not out_args:
+        for p in out_params:
+            if p.raw and not is_size_specified:
+                raise ValueError('Output array size is Undecided')
+        return [ndarray._new_contiguous(out_shape, t) for t in out_types]
+    for a, p in zip(out_args, out_params):
+        if not isinstance(a, ndarray):
+            raise TypeError('Output arguments type must be cupy.ndarray')
+        if not p.raw and a._shape != out_shape:
+            raise ValueError('Out shape is mismatched')
+    return out_args
+
+
+# ---------------------------------------------------------------------------------
+# launch plans
+# ---------------------------------------------------------------------------------
+
+def _canonical_dims(arrays, shape):
+    """Merges axes that every array walks back to back and drops unit axes.
+    Returns (shape, [strides per array]) of the equivalent smaller problem."""
+    cshape = []
+    cstrides = [[] for _ in arrays]
+    for d, ext in enumerate(shape):
+        if ext == 1:
+            continue
+        if cshape:
+            for cs, a in zip(cstrides, arrays):
+                if cs[-1] != a._strides[d] * ext:
+                    break
+            else:
+                cshape[-1] *= ext
+                for cs, a in zip(cstrides, arrays):
+                    cs[-1] = a._strides[d]
+                continue
+        cshape.append(ext)
+        for cs, a in zip(cstrides, arrays):
+            cs.append(a._strides[d])
+    return tuple(cshape), [tuple(cs) for cs in cstrides]
+
+
+def _max_vector_width(itemsizes):
+    """Elements per thread such that the narrowest operand moves 16 bytes and
+    the widest at most 64."""
+    v = 16 // min(itemsizes)
+    while v > 1 and v * max(itemsizes) > 64:
+        v //= 2
+    return max(v, 1)
+
+
+def _aligned(ptr, nbytes):
+    return ptr % nbytes == 0
+
+
+_grid_limit_memo = {}
+
+
+def _grid_limit(dev_id, blocks_per_cu):
+    key = (dev_id, blocks_per_cu)
+    g = _grid_limit_memo.get(key)
+    if g is None:
+        g = _device.get_compute_units(dev_id) * blocks_per_cu
+        _grid_limit_memo[key] = g
+    return g
+
+
+# Tunables of the flat elementwise kernel (vectors per thread per trip, resident
+# workgroups per CU the grid is capped at, non-temporal hint).
+FLAT_UNROLL = 2
+FLAT_BLOCKS_PER_CU = 16
+FLAT_STREAM_HINT = True
+TILED_BLOCKS_PER_CU = 8
+
+
+class _ElementwisePlanner:
+    """Builds, memoises and launches the kernels of one elementwise operation
+    (an ElementwiseKernel, or one loop of a ufunc)."""
+
+    def __init__(self, name, params, operation, preamble, loop_prep, after_loop,
+                 options, is_ufunc):
+        self.name = name
+        self.params = params          # ParameterInfo of inputs + outputs
+        self.operation = operation
+        self.preamble = preamble
+        self.loop_prep = loop_prep
+        self.after_loop = after_loop
+        self.options = tuple(options)
+        self.is_ufunc = is_ufunc
+        self._memo = {}
+        self._codes = {}
+        self._lock = threading.Lock()
+        self._force_generic = _cg.body_needs_generic(operation) or \
+            _cg.body_needs_generic(loop_prep) or _cg.body_needs_generic(after_loop)
+        self._uses_ind = _cg.uses_identifier(operation, '_ind') or \
+            _cg.uses_identifier(loop_prep, '_ind') or \
+            _cg.uses_identifier(after_loop, '_ind')
+        self._uses_i = _cg.uses_identifier(operation, 'i')
+
+    # One operand description per kernel parameter -------------------------------------
+    def _make_operands(self, args, nin, var_types, casts, force_read_out):
+        ops = []
+        for idx, (p, a) in enumerate(zip(self.params, args)):
+            is_out = idx >= nin
+            if isinstance(a, ndarray):
+                store_t = _get_typename(a.dtype)
+                if p.raw:
+                    ops.append(_cg.Operand(
+                        'raw', p.name, store_t, ndim=a.ndim,
+                        c_contiguous=a._c_contiguous, index_32=a._index_32_bits,
+                        is_const=p.is_const, is_out=is_out))
+                else:
+                    cast_in, cast_out = casts[idx] if casts else (None, None)
+                    read_out = False
+                    if is_out:
+                        read_out = force_read_out or not _cg.output_is_write_only(
+                            self.operation, p.name)
+                    elif not p.is_const:
+                        # a `_non_const` input is written by the body
+                        is_out = True
+                        read_out = True
+                    ops.append(_cg.Operand(
+                        'array', p.name, store_t, var_types[idx], is_out=is_out,
+                        read_out=read_out, cast_in=cast_in, cast_out=cast_out,
+                        ndim=a.ndim, c_contiguous=a._c_contiguous,
+                        index_32=a._index_32_bits, is_const=p.is_const))
+            else:
+                ops.append(_cg.Operand(
+                    'scalar', p.name, _get_typename(a.descr), is_const=True))
+        return ops
+
+    def launch(self, dev_id, args, nin, shape, var_types, typedefs, casts=None,
+               force_generic=False, force_read_out=False, stream=None,
+               block_size=None, kernel_name=None):
+        """Plans and launches.  ``args``: preprocessed inputs then outputs
+        (ndarrays already broadcast to ``shape``, CScalars already typed)."""
+        params = self.params
+        arrays = [a for a, p in zip(args, params)
+                  if isinstance(a, ndarray) and not p.raw]
+        size = internal.prod(shape)
+        stream_ptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
+        mode = 'generic'
+        cshape = cstrides = None
+        if not (force_generic or self._force_generic) and arrays:
+            cshape, cstrides = _canonical_dims(arrays, shape)
+            nd = len(cshape)
+            if nd <= 1:
+                ok = True
+                for a, cs in zip(arrays, cstrides):
+                    if nd == 1 and cs[0] != a.dtype.itemsize and cs[0] != 0:
+                        ok = False
+                        break
+                if ok:
+                    mode = 'flat'
+            elif nd == 2 and not self._uses_ind:
+                mode = self._classify_2d(arrays, cstrides, args, nin)
+        if mode == 'flat':
+            return self._launch_flat(
+                dev_id, args, nin, arrays, cstrides, size, var_types, typedefs,
+                casts, force_read_out, stream_ptr, kernel_name)
+        if mode in ('tiled', 'tiled_t'):
+            return self._launch_tiled(
+                dev_id, args, nin, arrays, cshape, cstrides, var_types, typedefs,
+                casts, force_read_out, stream_ptr, kernel_name, mode == 'tiled_t')
+        return self._launch_generic(
+            dev_id, args, nin, shape, var_types, typedefs, casts, force_read_out,
+            stream_ptr, block_size or 128, kernel_name)
+
+    # -- flat ---------------------------------------------------------------------------
+    def _launch_flat(self, dev_id, args, nin, arrays, cstrides, size, var_types,
+                     typedefs, casts, force_read_out, stream_ptr, kernel_name):
+        params = self.params
+        bcast = []
+        itemsizes = []
+        ai = 0
+        for a, p in zip(args, params):
+            if isinstance(a, ndarray) and not p.raw:
+                cs = cstrides[ai]
+                ai += 1
+                if size > 1 and (len(cs) == 1 and cs[0] == 0):
+                    bcast.append(p.name)
+                else:
+                    itemsizes.append(a.dtype.itemsize)
+        if not itemsizes:
+            itemsizes = [arrays[0].dtype.itemsize]
+        vec = _max_vector_width(itemsizes)
+        # every iterated array must sit on a boundary of its vector
+        ai = 0
+        for a, p in zip(args, params):
+            if isinstance(a, ndarray) and not p.raw:
+                if p.name not in bcast:
+                    while vec > 1 and not _aligned(
+                            a.data.ptr, min(16, vec * a.dtype.itemsize)):
+                        vec //= 2
+                ai += 1
+        if size < vec * 64:
+            vec = 1
+        idx64 = size > _INT32_MAX - (1 << 24)
+        unroll = FLAT_UNROLL if vec > 1 else 1
+        operands = self._make_operands(args, nin, var_types, casts, force_read_out)
+        if self._uses_ind:
+            operands.append(_cg.Operand('indexer', '_ind', '', ndim=1,
+                                        index_32=not idx64))
+        key = ('flat', tuple(o.key() for o in operands), typedefs, vec, unroll,
+               idx64, tuple(bcast), dev_id)
+        entry = self._memo.get(key)
+        if entry is None:
+            name = kernel_name or self.name
+            code = _cg.emit_flat(
+                name, operands, self.operation, typedefs, self.preamble,
+                self.loop_prep, self.after_loop, vec=vec, unroll=unroll,
+                idx64=idx64, bcast=tuple(bcast), stream_hint=FLAT_STREAM_HINT)
+            fn = compiler.compile_with_cache(code, self.options).get_function(name)
+            fmt = self._arg_format(operands, 'q' if idx64 else 'i', flat=True)
+            entry = (fn, struct.Struct(fmt), code)
+            with self._lock:
+                entry = self._memo.setdefault(key, entry)
+            self._remember_code(args, entry[2])
+        fn, packer, _ = entry
+        vals = self._flat_values(args)
+        vals.append(size)
+        if self._uses_ind:
+            vals.extend((size, size, 0))
+        blob = packer.pack(*vals)
+        nvec = size // vec
+        per_block = _cg.BLOCK * unroll
+        grid = max(1, min((max(nvec, size - nvec * vec) + per_block - 1) // per_block,
+                          _grid_limit(dev_id, FLAT_BLOCKS_PER_CU)))
+        fn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+
+    def _flat_values(self, args):
+        """Argument values for kernels that take plain pointers: data pointer
+        per iterated array, CArray fields per raw array, scalar values."""
+        out = []
+        for a, p in zip(args, self.params):
+            if isinstance(a, ndarray):
+                out.append(a.data.ptr)
+                if p.raw:
+                    out.append(a.size)
+                    out.extend(a._shape)
+                    out.extend(a._strides)
+            else:
+                out.append(a._struct_value())
+        return out
+
+    def _arg_format(self, operands, idx_code, flat):
+        """struct format of the kernel's argument block."""
+        fmt = ['@']
+        for o in operands:
+            if o.kind == 'array':
+                fmt.append('P' if flat else 'PP')
+            elif o.kind == 'raw':
+                fmt.append('P' + 'q' * (1 + 2 * o.ndim))
+            elif o.kind == 'scalar':
+                fmt.append(_scalar_struct_code(o.store_t))
+        fmt.append(idx_code)
+        for o in operands:
+            if o.kind == 'indexer':
+                fmt.append('q' * (1 + 2 * o.ndim))
+        return ''.join(fmt)
+
+    # -- tiled 2-d -----------------------------------------------------------------------
+    def _classify_2d(self, arrays, cstrides, args, nin):
+        """'tiled' if every array is contiguous (or broadcast) along the
+        columns, 'tiled_t' if that holds after swapping the two axes,
+        'generic' otherwise.  Transposed ('C') operands are allowed as inputs."""
+        def classify(swap):
+            ok = True
+            any_c = False
+            for a, cs in zip(arrays, cstrides):
+                s0, s1 = (cs[1], cs[0]) if swap else cs
+                item = a.dtype.itemsize
+                if s1 == item or s1 == 0:
+                    if s0 % item:
+                        ok = False
+                elif s0 == item and s1 % item == 0:
+                    any_c = True
+                    if any(a is o for o in args[nin:]):
+                        ok = False
+                else:
+                    ok = False
+                if not ok:
+                    break
+            return ok, any_c
+        ok, _ = classify(False)
+        if ok:
+            # outputs must be unit stride along columns
+            for o in args[nin:]:
+                for a, cs in zip(arrays, cstrides):
+                    if a is o and cs[1] != a.dtype.itemsize:
+                        ok = False
+            if ok:
+                return 'tiled'
+        if self._uses_i:
+            return 'generic'
+        ok, _ = classify(True)
+        if ok:
+            for o in args[nin:]:
+                for a, cs in zip(arrays, cstrides):
+                    if a is o and cs[0] != a.dtype.itemsize:
+                        ok = False
+            if ok:
+                return 'tiled_t'
+        return 'generic'
+
+    def _launch_tiled(self, dev_id, args, nin, arrays, cshape, cstrides, var_types,
+                      typedefs, casts, force_read_out, stream_ptr, kernel_name, swap):
+        params = self.params
+        if swap:
+            cshape = (cshape[1], cshape[0])
+            cstrides = [(cs[1], cs[0]) for cs in cstrides]
+        nr, nc = cshape
+        layouts = {}
+        itemsizes = [a.dtype.itemsize for a in arrays]
+        vec = _max_vector_width(itemsizes)
+        names = [p.name for a, p in zip(args, params)
+                 if isinstance(a, ndarray) and not p.raw]
+        for a, cs, nm in zip(arrays, cstrides, names):
+            item = a.dtype.itemsize
+            layouts[nm] = 'R' if (cs[1] == item or cs[1] == 0) else 'C'
+        # alignment of every vector access
+        while vec > 1:
+            ok = True
+            for a, cs, nm in zip(arrays, cstrides, names):
+                item = a.dtype.itemsize
+                nb = min(16, vec * item)
+                if not _aligned(a.data.ptr, nb):
+                    ok = False
+                elif layouts[nm] == 'R':
+                    if cs[1] != 0 and cs[0] % nb:
+                        ok = False
+                elif cs[1] % nb:
+                    ok = False
+            if ok:
+                break
+            vec //= 2
+        tile = 64
+        if tile // vec > _cg.BLOCK:
+            vec = max(vec, tile // _cg.BLOCK)
+        span = 0
+        for a, cs in zip(arrays, cstrides):
+            span = max(span, abs(cs[0]) * nr + abs(cs[1]) * nc)
+        idx64 = span > _INT32_MAX or nr * nc > _INT32_MAX
+        operands = self._make_operands(args, nin, var_types, casts, force_read_out)
+        key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
+               tuple(sorted(layouts.items())), dev_id)
+        entry = self._memo.get(key)
+        if entry is None:
+            name = kernel_name or self.name
+            code = _cg.emit_tiled2d(
+                name, operands, self.operation, typedefs, self.preamble,
+                self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
+                tile=tile, idx64=idx64, stream_hint=FLAT_STREAM_HINT)
+            fn = compiler.compile_with_cache(code, self.options).get_function(name)
+            ic = 'q' if idx64 else 'i'
+            fmt = ['@']
+            for o in operands:
+                if o.kind == 'array':
+                    fmt.append('P')
+                elif o.kind == 'raw':
+                    fmt.append('P' + 'q' * (1 + 2 * o.ndim))
+                elif o.kind == 'scalar':
+                    fmt.append(_scalar_struct_code(o.store_t))
+            fmt.append(ic * (2 + 2 * len(arrays)))
+            entry = (fn, struct.Struct(''.join(fmt)), code)
+            with self._lock:
+                entry = self._memo.setdefault(key, entry)
+            self._remember_code(args, entry[2])
+        fn, packer, _ = entry
+        vals = self._flat_values(args)
+        vals.extend((nr, nc))
+        for a, cs in zip(arrays, cstrides):
+            item = a.dtype.itemsize
+            vals.extend((cs[0] // item, cs[1] // item))
+        blob = packer.pack(*vals)
+        ntiles = ((nr + tile - 1) // tile) * ((nc + tile - 1) // tile)
+        grid = max(1, min(ntiles, 0x7fffffff))
+        fn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+
+    # -- generic ---------------------------------------------------------------------------
+    def _launch_generic(self, dev_id, args, nin, shape, var_types, typedefs, casts,
+                        force_read_out, stream_ptr, block_size, kernel_name):
+        params = self.params
+        arrays_idx = [i for i, (a, p) in enumerate(zip(args, params))
+                      if isinstance(a, ndarray) and not p.raw]
+        args = list(args)
+        if arrays_idx:
+            arrays = [args[i] for i in arrays_idx]
+            cshape, cstrides = _canonical_dims(arrays, shape)
+            if len(cshape) != len(shape):
+                if len(cshape) == 0:
+                    cshape = (1,)
+                    cstrides = [(a.dtype.itemsize,) for a in arrays]
+                for i, cs in zip(arrays_idx, cstrides):
+                    args[i] = args[i]._view(cshape, cs)
+                shape = cshape
+        indexer = _carray.Indexer(shape)
+        operands = self._make_operands(args, nin, var_types, casts, force_read_out)
+        operands.append(_cg.Operand('indexer', '_ind', '', ndim=indexer.ndim,
+                                    index_32=indexer._index_32_bits))
+        key = ('generic', tuple(o.key() for o in operands), typedefs, dev_id)
+        entry = self._memo.get(key)
+        if entry is None:
+            name = kernel_name or self.name
+            code = _cg.emit_generic(
+                name, operands, self.operation, typedefs, self.preamble,
+                self.loop_prep, self.after_loop)
+            fn = compiler.compile_with_cache(code, self.options).get_function(name)
+            fmt = ['@']
+            for o in operands:
+                if o.kind in ('array', 'raw'):
+                    fmt.append('P' + 'q' * (1 + 2 * o.ndim))
+                elif o.kind == 'scalar':
+                    fmt.append(_scalar_struct_code(o.store_t))
+                else:
+                    fmt.append('q' * (1 + 2 * o.ndim))
+            entry = (fn, struct.Struct(''.join(fmt)), code)
+            with self._lock:
+                entry = self._memo.setdefault(key, entry)
+            self._remember_code(args, entry[2])
+        fn, packer, _ = entry
+        vals = []
+        for a in args:
+            if isinstance(a, ndarray):
+                vals.append(a.data.ptr)
+                vals.append(a.size)
+                vals.extend(a._shape)
+                vals.extend(a._strides)
+            else:
+                vals.append(a._struct_value())
+        vals.append(indexer.size)
+        vals.extend(indexer.shape)
+        vals.extend((0,) * indexer.ndim)
+        blob = packer.pack(*vals)
+        size = indexer.size
+        block = max(1, min(block_size, size))
+        # enough workgroups to fill the device several times over; the kernel
+        # loops over what is left
+        grid = max(1, min((size + block - 1) // block,
+                          _grid_limit(dev_id, 32) * max(1, 256 // block)))
+        fn.launch_packed((grid, 1, 1), (block, 1, 1), blob, 0, stream_ptr)
+
+    def _remember_code(self, args, code):
+        in_types = tuple(a.dtype for a in args if isinstance(a, ndarray))
+        if in_types not in self._codes:
+            self._codes[in_types] = code
+
+
+_SCALAR_CODES = {
+    'bool': '?', 'signed char': 'b', 'unsigned char': 'B', 'short': 'h',
+    'unsigned short': 'H', 'int': 'i', 'unsigned int': 'I', 'long long': 'q',
+    'unsigned long long': 'Q', 'float16': '2s', 'float': '4s', 'double': '8s',
+}
+
+
+def _scalar_struct_code(ctype):
+    """struct code for a by-value scalar; floats travel as their bytes with an
+    explicit alignment pad handled by the native-alignment '@' mode."""
+    code = _SCALAR_CODES[ctype]
+    if code == '2s':
+        return 'e'
+    if code == '4s':
+        return 'f'
+    if code == '8s':
+        return 'd'
+    return code
+
+
+# ---------------------------------------------------------------------------------
+# ElementwiseKernel
+# ---------------------------------------------------------------------------------
+
+class ElementwiseKernel:
+    """User-defined elementwise kernel.
+
+    The loop body ``operation`` is HIP C++ operating on one element; array
+    parameters are broadcast against each other unless marked ``raw``.  The
+    kernel is generated and compiled for gfx950 on first use for each
+    combination of argument types and memory layouts, cached in the process and
+    on disk.
+
+    Args:
+        in_params (str): Input argument list, e.g. ``'float32 x, T y'``.
+        out_params (str): Output argument list.
+        operation (str): The body of the loop.
+        name (str): Name of the kernel function (shows up in profiles).
+        reduce_dims (bool): Merge contiguous axes before launching.
+        preamble (str): Code inserted before the kernel.
+        no_return (bool): ``__call__`` returns ``None``.
+        return_tuple (bool): ``__call__`` always returns a tuple.
+        options (tuple): Extra hiprtc options.
+        loop_prep (str): Code run by every thread before the loop.
+        after_loop (str): Code run by every thread after the loop.
+    """
+
+    def __init__(self, in_params, out_params, operation, name='kernel',
+                 reduce_dims=True, preamble='', no_return=False,
+                 return_tuple=False, **kwargs):
+        if not compiler.is_valid_kernel_name(name):
+            raise ValueError('Invalid kernel name: "%s"' % name)
+        self.in_params = _get_param_info(in_params, True)
+        self.out_params = _get_param_info(out_params, False)
+        self.nin = len(self.in_params)
+        self.nout = len(self.out_params)
+        self.nargs = self.nin + self.nout
+        param_rest = _get_param_info('CIndexer _ind', False)
+        self.params = self.in_params + self.out_params + param_rest
+        self.operation = operation
+        self.name = name
+        self.__name__ = name
+        self.reduce_dims = reduce_dims
+        self.preamble = preamble
+        self.no_return = no_return
+        self.return_tuple = return_tuple
+        self.kwargs = dict(kwargs)
+        options = kwargs.pop('options', ())
+        loop_prep = kwargs.pop('loop_prep', '')
+        after_loop = kwargs.pop('after_loop', '')
+        if kwargs:
+            raise TypeError('Wrong arguments %s' % kwargs)
+        names = [p.name for p in self.in_params + self.out_params]
+        if 'i' in names:
+            raise ValueError('Can not use \'i\' as a parameter name')
+        self._params_type_memo = {}
+        self._planner = _ElementwisePlanner(
+            name, self.in_params + self.out_params, operation, preamble,
+            loop_prep, after_loop, options, is_ufunc=False)
+        self._cached_codes = self._planner._codes
+
+    def __call__(self, *args, **kwargs):
+        """Compiles (if needed) and launches the kernel.
+
+        Args:
+            args: Inputs, optionally followed by the outputs.
+            size (int): Number of loop iterations; required if and only if no
+                non-raw array is among the arguments.
+            stream: Stream to launch on (default: current stream).
+            block_size (int): Threads per workgroup of the strided fallback
+                kernel (default 128).
+        """
+        size = kwargs.pop('size', -1)
+        stream = kwargs.pop('stream', None)
+        block_size = kwargs.pop('block_size', 128)
+        if len(kwargs):
+            raise TypeError('Wrong arguments %s' % kwargs)
+        if block_size <= 0:
+            raise ValueError('block_size must be greater than zero')
+        n_args = len(args)
+        if n_args != self.nin and n_args != self.nargs:
+            raise TypeError(
+                'Wrong number of arguments for {!r}. '
+                'It must be either {} or {} (with outputs), '
+                'but given {}.'.format(self.name, self.nin, self.nargs, n_args))
+        for arg in args:
+            if hasattr(arg, '__cupy_override_elementwise_kernel__'):
+                return arg.__cupy_override_elementwise_kernel__(
+                    self, *args, size=size, stream=stream, block_size=block_size)
+        dev_id = _device.get_device_id()
+        arg_list = _preprocess_args(dev_id, args)
+        out_args = arg_list[self.nin:]
+        bargs, shape = _broadcast(arg_list, self.params, size != -1)
+        in_args = bargs[:self.nin]
+
+        in_ndarray_types = tuple(
+            a.dtype if isinstance(a, ndarray) else None for a in in_args)
+        out_ndarray_types = tuple(
+            a.dtype if isinstance(a, ndarray) else None for a in out_args)
+        in_types, out_types, type_map = self._decide_params_type(
+            in_ndarray_types, out_ndarray_types)
+
+        is_size_specified = False
+        if size != -1:
+            shape = (int(size),)
+            is_size_specified = True
+
+        out_args = _get_out_args_with_params(
+            out_args, out_types, shape, self.out_params, is_size_specified)
+        if self.no_return:
+            ret = None
+        elif not self.return_tuple and self.nout == 1:
+            ret = out_args[0]
+        else:
+            ret = tuple(out_args)
+        if 0 in shape:
+            return ret
+
+        for i, x in enumerate(in_args):
+            if type(x) is CScalar:
+                x.apply_dtype(in_types[i])
+
+        inout_args = in_args + out_args
+        var_types = [p.ctype for p in self.in_params + self.out_params]
+        self._planner.launch(
+            dev_id, inout_args, self.nin, shape, var_types,
+            type_map.get_typedef_code(), stream=stream, block_size=block_size,
+            force_generic=not self.reduce_dims and False)
+        return ret
+
+    def _decide_params_type(self, in_args_dtype, out_args_dtype):
+        key = (in_args_dtype, out_args_dtype)
+        ret = self._params_type_memo.get(key)
+        if ret is None:
+            ret = _decide_params_type_core(
+                self.in_params, self.out_params, in_args_dtype, out_args_dtype)
+            self._params_type_memo[key] = ret
+        return ret
+
+    @property
+    def cached_codes(self):
+        """dict: input dtypes -> generated source (for debugging)."""
+        if len(self._cached_codes) == 0:
+            warnings.warn(
+                'No codes are cached because compilation is deferred until '
+                'the first function call.')
+        return dict(self._cached_codes.items())
+
+    @property
+    def cached_code(self):
+        """``next(iter(self.cached_codes.values()))``."""
+        codes = self._cached_codes
+        if len(codes) > 1:
+            warnings.warn(
+                'The input types of the kernel could not be inferred. '
+                'Please use `.cached_codes` instead.')
+        return next(iter(codes.values()))
+
+
+# ---------------------------------------------------------------------------------
+# ufunc
+# ---------------------------------------------------------------------------------
+
+def fix_cast_expr(src_type, dst_type, expr):
+    """Expression converting ``expr`` of ``src_type`` for use as ``dst_type``."""
+    src_kind = get_dtype(src_type).kind
+    dst_kind = get_dtype(dst_type).kind
+    if src_kind == dst_kind:
+        return expr
+    if src_kind == 'b':
+        return '((%s) ? 1 : 0)' % expr
+    return expr
+
+
+def _get_kind_score(kind):
+    if issubclass(kind, numpy.bool_):
+        return 0
+    if issubclass(kind, (numpy.integer, int)):
+        return 1
+    if issubclass(kind, (numpy.inexact, float, complex)):
+        return 2
+    return 3
+
+
+def _check_should_use_weak_scalar(in_types, weaks):
+    """With the first-matching-loop strategy a weak Python scalar may only take
+    part in loop selection when it is not of a higher kind than the arrays
+    (so that ``uint8 array + 0.`` does not pick up a float64 loop by way of
+    the scalar alone)."""
+    if weaks is None:
+        return False
+    max_array_kind = -1
+    max_scalar_kind = -1
+    for in_t, w_t in zip(in_types, weaks):
+        if w_t:
+            max_scalar_kind = max(max_scalar_kind, _get_kind_score(w_t))
+        else:
+            max_array_kind = max(max_array_kind, _get_kind_score(in_t.type))
+    all_scalars_or_arrays = max_scalar_kind == -1 or max_array_kind == -1
+    return not all_scalars_or_arrays and max_array_kind >= max_scalar_kind
+
+
+class _Op:
+    """One typed loop of a ufunc / reduction: input and output dtypes plus the
+    routine (code) or an ``error_func`` raising for a forbidden combination."""
+
+    def __init__(self, in_types, out_types, routine, error_func):
+        if error_func is None:
+            assert routine is not None
+        else:
+            assert callable(error_func)
+        self.in_types = in_types
+        self.out_types = out_types
+        self.nin = len(in_types)
+        self.nout = len(out_types)
+        self.routine = routine
+        self.error_func = error_func
+        self._in_dtypes = tuple(get_dtype(t) for t in in_types)
+        self._out_dtypes = tuple(get_dtype(t) for t in out_types)
+
+    @staticmethod
+    def _from(typ, routine, error_func):
+        types = typ.split('->')
+        if len(types) == 1:
+            in_types = out_types = tuple(types)
+        else:
+            in_types, out_types = map(tuple, types)
+        in_types = tuple(get_dtype(t).type for t in in_types)
+        out_types = tuple(get_dtype(t).type for t in out_types)
+        return _Op(in_types, out_types, routine, error_func)
+
+    def check_valid(self):
+        if self.error_func is not None:
+            self.error_func()
+
+    def resolve_dtypes(self, in_args, out_args):
+        return self._in_dtypes, self._out_dtypes
+
+    def __repr__(self):
+        return '_Op(%s -> %s)' % (self.in_types, self.out_types)
+
+
+class _Ops:
+
+    def __init__(self, ops):
+        assert len(ops) > 0
+        nin = ops[0].nin
+        nout = ops[0].nout
+        for op in ops:
+            if op.nin != nin or op.nout != nout:
+                raise ValueError(f'invalid op {op}, wrong nin or nout.')
+        self.ops = ops
+        self.nin = nin
+        self.nout = nout
+
+    @staticmethod
+    def from_tuples(ops, routine):
+        ops_ = []
+        for t in ops:
+            if isinstance(t, tuple):
+                typ, rt = t
+                if rt is None:
+                    rt = routine
+                elif isinstance(rt, tuple):
+                    rt = tuple(r1 or r2 for r1, r2 in zip(rt, routine))
+                elif not isinstance(rt, str):
+                    if not callable(rt):
+                        raise ValueError(f'invalid op {t}, expected callable {rt}')
+                    ops_.append(_Op._from(typ, None, rt))
+                    continue
+            else:
+                if not isinstance(t, str):
+                    raise ValueError(f'invalid op {t}, expected string')
+                typ, rt = t, routine
+            ops_.append(_Op._from(typ, rt, None))
+        return _Ops(tuple(ops_))
+
+    def guess_routine(self, name, cache, in_args, dtype, out_ops):
+        if dtype is None:
+            weaks_l = []
+            in_types_l = []
+            any_weak = False
+            for a in in_args:
+                if type(a) is CScalar:
+                    t = a.descr
+                    weak_t = a.weak_t
+                    if weak_t is not False:
+                        any_weak = True
+                elif isinstance(a, ndarray):
+                    t = a.dtype
+                    weak_t = False
+                else:
+                    raise RuntimeError(f'Need array or CScalar got {type(a)}')
+                in_types_l.append(t)
+                weaks_l.append(weak_t)
+            in_types = tuple(in_types_l)
+            weaks = tuple(weaks_l) if any_weak else None
+            if not _check_should_use_weak_scalar(in_types, weaks):
+                weaks = (False,) * len(in_args)
+            op = cache.get((in_types, weaks), ())
+            if op == ():
+                op = self._guess_routine_from_in_types(in_types, weaks)
+                cache[(in_types, weaks)] = op
+        else:
+            op = cache.get(dtype, ())
+            if op == ():
+                ops_ = out_ops or self
+                op = ops_._guess_routine_from_dtype(dtype)
+                cache[dtype] = op
+        if op is not None:
+            op.check_valid()
+            return op
+        if dtype is None:
+            dtype = in_types
+        raise TypeError('Wrong type (%s) of arguments for %s' % (dtype, name))
+
+    def _guess_routine_from_in_types(self, in_types, weaks=None):
+        """First loop every input can be safely cast to.  A weak Python scalar
+        that cannot be cast safely is still accepted when it would not change
+        the loop's type under NumPy's promotion (NEP 50)."""
+        can_cast = numpy.can_cast
+        for op in self.ops:
+            op_types = op.in_types
+            for i in range(self.nin):
+                it = in_types[i]
+                ot = op_types[i]
+                weak_t = weaks[i] if weaks is not None else False
+                if not can_cast(it, ot):
+                    if not weak_t:
+                        break
+                    try:
+                        if numpy.result_type(weak_t(0), ot) != ot:
+                            break
+                    except TypeError:
+                        break
+            else:
+                return op
+        return None
+
+    def _guess_routine_from_dtype(self, dtype):
+        for op in self.ops:
+            for t in op.out_types:
+                if t != dtype:
+                    break
+            else:
+                return op
+        return None
+
+
+class ufunc:
+    """Universal function: typed loops selected the way NumPy selects them,
+    broadcasting, ``out=``, ``dtype=``, ``casting=`` and ``_where=``.
+
+    Attributes:
+        name (str), nin (int), nout (int), nargs (int), types (list of str)
+    """
+
+    def __init__(self, name, nin, nout, ops, preamble='', loop_prep='', doc='',
+                 default_casting=None, *, out_ops=None, cutensor_op=None,
+                 scatter_op=None):
+        self.name = name
+        self.__name__ = name
+        self.nin = nin
+        self.nout = nout
+        self.nargs = nin + nout
+        self._ops = ops
+        self._out_ops = out_ops
+        self._preamble = preamble
+        self._loop_prep = loop_prep
+        self._doc = doc
+        self.__doc__ = doc
+        self._default_casting = 'same_kind' if default_casting is None \
+            else default_casting
+        self._scatter_op = scatter_op
+        _in_params = tuple(ParameterInfo('T in%d' % i, True) for i in range(nin))
+        _out_params = tuple(ParameterInfo('T out%d' % i, False) for i in range(nout))
+        self._params = _in_params + _out_params
+        self._params_with_where = (
+            _in_params + (ParameterInfo('T _where', True),) + _out_params)
+        self._routine_cache = {}
+        self._planners = {}
+        self._kernel_memo = self._planners
+
+    def __repr__(self):
+        return '<ufunc \'%s\'>' % self.name
+
+    @property
+    def types(self):
+        """Type signatures ``'ff->f'`` of the loops, in selection order."""
+        types = []
+        for op in self._ops.ops:
+            in_str = ''.join(get_dtype(t).char for t in op.in_types)
+            out_str = ''.join(get_dtype(t).char for t in op.out_types)
+            types.append('%s->%s' % (in_str, out_str))
+        return types
+
+    def __call__(self, *args, **kwargs):
+        """Applies the function elementwise.
+
+        Args:
+            args: Inputs (arrays or scalars), optionally followed by outputs.
+            out (cupy.ndarray or tuple): Output array(s).
+            dtype: Selects the loop by its output type.
+            casting (str): Rule for casting results into given outputs
+                (default ``'same_kind'``).
+        """
+        for arg in args:
+            if hasattr(arg, '__cupy_override_elementwise_kernel__'):
+                return arg.__cupy_override_elementwise_kernel__(
+                    self, *args, **kwargs)
+        if _fusion_thread_local.is_fusing():
+            return _fusion_thread_local.call_ufunc(self, *args, **kwargs)
+
+        out = kwargs.pop('out', None)
+        where = kwargs.pop('_where', None)
+        has_where = where is not None
+        dtype = kwargs.pop('dtype', None)
+        casting = kwargs.pop('casting', self._default_casting)
+        if dtype is not None:
+            dtype = get_dtype(dtype).type
+        if kwargs:
+            raise TypeError('Wrong arguments %s' % kwargs)
+
+        n_args = len(args)
+        if not (self.nin <= n_args <= self.nargs):
+            raise TypeError(
+                'Wrong number of arguments for {!r}. '
+                'It must be either {} or {} (with outputs), '
+                'but given {}.'.format(self.name, self.nin, self.nargs, n_args))
+        in_args = args[:self.nin]
+        out_args = args[self.nin:]
+        if out is not None:
+            if out_args:
+                raise ValueError('Cannot specify \'out\' as both '
+                                 'a positional and keyword argument')
+            if isinstance(out, tuple):
+                if len(out) != self.nout:
+                    raise ValueError(
+                        "The 'out' tuple must have exactly one entry per "
+                        "ufunc output")
+                out_args = out
+            else:
+                if 1 != self.nout:
+                    raise ValueError("'out' must be a tuple of arrays")
+                out_args = out,
+
+        dev_id = _device.get_device_id()
+        in_args = _preprocess_args(dev_id, in_args)
+        out_args = _preprocess_optional_args(dev_id, out_args)
+        given_out_args = [o for o in out_args if o is not None]
+
+        if has_where:
+            where_args = _preprocess_args(dev_id, (where,))
+            x = where_args[0]
+            if isinstance(x, ndarray):
+                if x.dtype != bool:
+                    raise TypeError(
+                        f'Cannot cast array data from {x.dtype!r} to '
+                        f'{get_dtype(bool)!r} according to the rule \'safe\'')
+            else:
+                where_args[0] = CScalar(bool(x.value))
+        else:
+            where_args = []
+
+        _copy_in_args_if_needed(in_args, given_out_args)
+        _copy_in_args_if_needed(where_args, given_out_args)
+        inout_args = in_args + where_args + given_out_args
+        shape = internal._broadcast_core(inout_args)
+        n_in = len(in_args)
+        in_args = inout_args[:n_in]
+        where_args = inout_args[n_in:n_in + len(where_args)]
+
+        op = self._ops.guess_routine(
+            self.name, self._routine_cache, in_args, dtype, self._out_ops)
+
+        subtype = ndarray
+        template = None
+        for in_arg in in_args:
+            t = type(in_arg)
+            if t is not ndarray and issubclass(t, ndarray):
+                subtype = t
+                template = in_arg
+                break
+
+        core_in_dtypes, core_out_dtypes = op.resolve_dtypes(in_args, out_args)
+        out_args = _get_out_args_from_optionals(
+            subtype, out_args, core_out_dtypes, shape, casting, template)
+        ret = out_args[0] if self.nout == 1 else tuple(out_args)
+        if 0 in shape:
+            return ret
+
+        for i, t in enumerate(core_in_dtypes):
+            if type(in_args[i]) is CScalar:
+                in_args[i].apply_dtype(t)
+
+        planner = self._get_planner(op, has_where)
+        all_args = in_args + where_args + out_args
+        nin_total = n_in + len(where_args)
+        # Body variables carry the loop's types; elements are converted on load
+        # and store when the array's dtype differs.
+        var_types = ['in%d_type' % i for i in range(n_in)]
+        casts = []
+        for i, a in enumerate(in_args):
+            if isinstance(a, ndarray):
+                lt = core_in_dtypes[i]
+                casts.append((_make_cast(a.dtype, lt), None))
+            else:
+                casts.append((None, None))
+        if has_where:
+            var_types.append('bool')
+            casts.append((None, None))
+        for i, a in enumerate(out_args):
+            var_types.append('out%d_type' % i)
+            lt = core_out_dtypes[i]
+            casts.append((_make_cast(a.dtype, lt), _make_cast(lt, a.dtype)))
+        typedefs = ''.join(
+            ['typedef %s in%d_type;\n' % (_get_typename(t), i)
+             for i, t in enumerate(core_in_dtypes)]
+            + ['typedef %s out%d_type;\n' % (_get_typename(t), i)
+               for i, t in enumerate(core_out_dtypes)])
+        planner.launch(
+            dev_id, all_args, nin_total, shape, var_types, typedefs, casts=casts,
+            force_generic=False, force_read_out=has_where,
+            kernel_name=self._get_name_with_type(all_args, has_where))
+        return ret
+
+    def _get_planner(self, op, has_where):
+        key = (op, has_where)
+        planner = self._planners.get(key)
+        if planner is None:
+            routine = op.routine
+            if has_where:
+                # masked-out elements keep the previous contents of the output
+                names = ['out%d' % i for i in range(self.nout)]
+                saves = ' '.join('const out%d_type _keep%d = %s;' % (i, i, n)
+                                 for i, n in enumerate(names))
+                restores = ' '.join('%s = _keep%d;' % (n, i)
+                                    for i, n in enumerate(names))
+                routine = '%s %s; if (!_where) { %s }' % (saves, routine, restores)
+                params = self._params_with_where
+            else:
+                params = self._params
+            planner = _ElementwisePlanner(
+                self.name, params, routine, self._preamble, self._loop_prep, '',
+                (), is_ufunc=True)
+            planner = self._planners.setdefault(key, planner)
+        return planner
+
+    def _get_name_with_type(self, args, has_where):
+        name = self.name
+        if has_where:
+            name += '_where'
+        words = []
+        for a in args:
+            if isinstance(a, ndarray):
+                words.append(a.dtype.name)
+            else:
+                words.append(a.descr.name.rstrip('0123456789'))
+        return '{}__{}'.format(name, '_'.join(words))
+
+    def outer(self, A, B, **kwargs):
+        """Applies the ufunc to all pairs of elements of ``A`` and ``B``."""
+        from cupy_amd._core.core import array
+        A = array(A, copy=False)
+        B = array(B, copy=False)
+        A = A.reshape(A.shape + (1,) * B.ndim)
+        B = B.reshape((1,) * (A.ndim - B.ndim) + B.shape) if B.ndim else B
+        return self(A, B, **kwargs)
+
+    def at(self, a, indices, b=None):
+        raise NotImplementedError(f'`{self.name}.at` is not supported yet')
+
+    def reduce(self, array, axis=0, dtype=None, out=None, keepdims=False):
+        if self.name == 'cupy_add':
+            return array.sum(axis, dtype, out, keepdims)
+        if self.name == 'cupy_multiply':
+            return array.prod(axis, dtype, out, keepdims)
+        raise NotImplementedError(f'`{self.name}.reduce` is not supported yet')
+
+    def accumulate(self, array, axis=0, dtype=None, out=None):
+        raise NotImplementedError(
+            f'`{self.name}.accumulate` is not supported yet')
+
+    def reduceat(self, array, indices, axis=0, dtype=None, out=None):
+        raise NotImplementedError(
+            f'`{self.name}.reduceat` is not supported yet')
+
+
+def _make_cast(src_dtype, dst_dtype):
+    """Callable(expr) applying the conversion quirks between two dtypes, or
+    None when a plain C++ conversion does."""
+    src = get_dtype(src_dtype)
+    dst = get_dtype(dst_dtype)
+    if src.kind == dst.kind or src.kind != 'b':
+        return None
+    return lambda e: fix_cast_expr(src, dst, e)
+
+
+def create_ufunc(name, ops, routine=None, preamble='', doc='',
+                 default_casting=None, loop_prep='', out_ops=None,
+                 cutensor_op=None, scatter_op=None, promote_types=None):
+    """Builds a ufunc from loop signatures (``'ff->f'`` or
+    ``('ff->f', routine)``) and a default routine."""
+    ops_ = _Ops.from_tuples(ops, routine)
+    _out_ops = None if out_ops is None else _Ops.from_tuples(out_ops, routine)
+    return ufunc(name, ops_.nin, ops_.nout, ops_, preamble, loop_prep, doc,
+                 default_casting=default_casting, out_ops=_out_ops,
+                 cutensor_op=cutensor_op, scatter_op=scatter_op)

@@ -1,0 +1,207 @@
+"""Run-time compilation of generated HIP source for gfx950 with hiprtc.
+
+Counterpart of the reference's cupy/cuda/compiler.py (``_compile_with_cache_hip``
+:1003-1087, ``_NVRTCProgram`` :832-880, ``CompileException`` :793-829,
+``is_valid_kernel_name`` :883-884) and of ``compile_with_cache`` in
+cupy/_core/core.pyx:2621-2643.  Two cache levels: an in-process memo of loaded
+modules per device, and code objects on disk.
+"""
+import ctypes
+import hashlib
+import os
+import re
+import sys
+import threading
+
+from cupy_amd import _dryrun
+from cupy_amd import _rt
+from cupy_amd.cuda import _compiler_cache
+from cupy_amd.cuda import device as _device
+from cupy_amd.cuda import function as _function
+
+_INCLUDE_DIR = os.path.join(os.path.dirname(os.path.dirname(
+    os.path.abspath(__file__))), 'include')
+
+_kernel_name_re = re.compile(r'^[a-zA-Z_][a-zA-Z_0-9]*$')
+
+# Options every generated kernel is compiled with.
+#  * -ffp-contract=off: a*b+c must round twice, like the NumPy loops the
+#    results are compared with.
+#  * no denormal flushing (the default), for the same reason.
+#  * packed-FP32 instructions are switched off.
+_BASE_OPTIONS = (
+    '-std=c++17', '-O3', '-ffp-contract=off',
+    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+)
+
+
+def is_valid_kernel_name(name):
+    return _kernel_name_re.match(name) is not None
+
+
+class CompileException(Exception):
+    """hiprtc rejected the source; ``str()`` is the compiler log."""
+
+    def __init__(self, msg, source, name, options, backend='hiprtc'):
+        self._msg = msg
+        self.source = source
+        self.name = name
+        self.options = options
+        self.backend = backend
+        super().__init__()
+
+    def __reduce__(self):
+        return (type(self), (self._msg, self.source, self.name, self.options,
+                             self.backend))
+
+    def __repr__(self):
+        return str(self)
+
+    def __str__(self):
+        return self.get_message()
+
+    def get_message(self):
+        return self._msg
+
+    def dump(self, f):
+        lines = self.source.split('\n')
+        digits = len(str(len(lines)))
+        f.write('%s compilation error: %s\n' % (self.backend, self))
+        f.write('-----\nName: %s\nOptions: %s\nSource:\n' % (
+            self.name, ' '.join(self.options)))
+        for i, line in enumerate(lines):
+            f.write('%*d\t%s\n' % (digits, i + 1, line.rstrip()))
+        f.write('-----\n')
+        f.flush()
+
+
+_rtc_version = None
+
+
+def get_rtc_version():
+    global _rtc_version
+    if _rtc_version is None:
+        major = ctypes.c_int(0)
+        minor = ctypes.c_int(0)
+        _rt.check(_rt.lib.rt_rtc_version(ctypes.byref(major), ctypes.byref(minor)))
+        _rtc_version = (major.value, minor.value)
+    return _rtc_version
+
+
+_header_digest = None
+
+
+def _get_header_digest():
+    """Hash of the bundled device headers: part of every cache key."""
+    global _header_digest
+    if _header_digest is None:
+        h = hashlib.sha1()
+        for root, _, files in sorted(os.walk(_INCLUDE_DIR)):
+            for name in sorted(files):
+                with open(os.path.join(root, name), 'rb') as f:
+                    h.update(name.encode())
+                    h.update(f.read())
+        _header_digest = h.hexdigest()
+    return _header_digest
+
+
+def get_arch(device_id=None):
+    """Target processor for hiprtc, e.g. ``gfx950`` (feature suffixes dropped
+    so the code object loads whatever the sramecc/xnack setting)."""
+    if _dryrun.enabled():
+        return 'gfx950'
+    return _device.get_device_properties(device_id)['arch'].split(':')[0]
+
+
+def compile_source(source, options=(), arch='gfx950', name='kernel.hip'):
+    """Compiles HIP source to a gfx950 code object (bytes); no caching."""
+    opts = ('--offload-arch=' + arch,) + _BASE_OPTIONS + (
+        '-I' + _INCLUDE_DIR,) + tuple(options)
+    enc = [o.encode() for o in opts]
+    c_opts = (ctypes.c_char_p * len(enc))(*enc)
+    code = ctypes.c_void_p()
+    size = ctypes.c_size_t(0)
+    log = ctypes.c_void_p()
+    status = _rt.lib.rt_compile(
+        source.encode(), name.encode(), len(enc), c_opts, 0, None, None,
+        ctypes.byref(code), ctypes.byref(size), ctypes.byref(log))
+    try:
+        log_text = ctypes.string_at(log.value).decode(errors='replace') \
+            if log.value else ''
+        if status != 0:
+            if _rt.RT_ERR_RTC_BASE <= status < _rt.RT_ERR_POOL_OOM:
+                exc = CompileException(log_text or _rt.lib.rt_error_string(
+                    status).decode(), source, name, opts)
+                if os.environ.get('CUPY_DUMP_CUDA_SOURCE_ON_ERROR', '0') not in ('', '0'):
+                    exc.dump(sys.stderr)
+                raise exc
+            _rt.check(status)
+        return ctypes.string_at(code.value, size.value)
+    finally:
+        if code.value:
+            _rt.lib.rt_free_buffer(code)
+        if log.value:
+            _rt.lib.rt_free_buffer(log)
+
+
+def _cache_key(source, options, arch):
+    h = hashlib.sha1()
+    for part in (arch, repr(_BASE_OPTIONS), repr(tuple(options)),
+                 repr(get_rtc_version()), _get_header_digest(), source):
+        h.update(part.encode())
+        h.update(b'\0')
+    return h.hexdigest() + '.hsaco'
+
+
+_disk_cache = None
+_module_memo = {}
+_memo_lock = threading.Lock()
+# compile statistics, for tests and the launch-latency report
+stats = {'memo_hit': 0, 'disk_hit': 0, 'compiled': 0}
+
+
+def _get_disk_cache():
+    global _disk_cache
+    if _disk_cache is None or _disk_cache.cache_dir != _compiler_cache.get_cache_dir():
+        _disk_cache = _compiler_cache.DiskKernelCache(
+            extra_read_dirs=(_compiler_cache.bundled_cache_dir(),))
+    return _disk_cache
+
+
+def get_code_object(source, options=()):
+    """Code object for ``source`` through the disk cache."""
+    arch = get_arch()
+    key = _cache_key(source, options, arch)
+    use_disk = os.environ.get('CUPY_CACHE_IN_MEMORY', '0') in ('', '0')
+    payload = _get_disk_cache().load(key) if use_disk else None
+    if payload is None:
+        payload = compile_source(source, options, arch)
+        stats['compiled'] += 1
+        if use_disk:
+            save_src = os.environ.get('CUPY_CACHE_SAVE_CUDA_SOURCE', '0') not in ('', '0')
+            _get_disk_cache().save(key, payload, source if save_src else None)
+    else:
+        stats['disk_hit'] += 1
+    return payload
+
+
+def compile_with_cache(source, options=()):
+    """Loaded module for ``source`` on the current device (memoised)."""
+    options = tuple(options)
+    dev = _device.get_device_id()
+    key = (dev, source, options)
+    mod = _module_memo.get(key)
+    if mod is not None:
+        stats['memo_hit'] += 1
+        return mod
+    code = get_code_object(source, options)
+    mod = _function.Module()
+    mod.load(code)
+    with _memo_lock:
+        mod = _module_memo.setdefault(key, mod)
+    return mod
+
+
+def clear_memo():
+    with _memo_lock:
+        _module_memo.clear()

@@ -1,0 +1,179 @@
+"""Loaded code objects and kernel launch.
+
+Counterpart of the reference's cupy/cuda/function.pyx (``Module`` :174-208,
+``Function`` :134-171, ``_launch`` :92-131, argument conversion :53-82).
+"""
+import ctypes
+import struct
+
+import numpy
+
+from cupy_amd import _dryrun
+from cupy_amd import _rt
+from cupy_amd.cuda import stream as _stream
+
+# hipFunction_attribute values
+_FUNC_ATTRIBUTES = {
+    'max_threads_per_block': 0,
+    'shared_size_bytes': 1,
+    'const_size_bytes': 2,
+    'local_size_bytes': 3,
+    'num_regs': 4,
+    'ptx_version': 5,
+    'binary_version': 6,
+    'cache_mode_ca': 7,
+    'max_dynamic_shared_size_bytes': 8,
+    'preferred_shared_memory_carveout': 9,
+}
+
+
+def _arg_to_bytes(arg):
+    """Bytes of one kernel argument passed by value."""
+    if hasattr(arg, '_kernel_arg_bytes'):      # ndarray, Indexer, CScalar
+        return arg._kernel_arg_bytes()
+    if isinstance(arg, bool):
+        return struct.pack('?', arg)
+    if isinstance(arg, int):
+        return struct.pack('q', arg) if arg < (1 << 63) else struct.pack('Q', arg)
+    if isinstance(arg, float):
+        return struct.pack('d', arg)
+    if isinstance(arg, complex):
+        return struct.pack('dd', arg.real, arg.imag)
+    if isinstance(arg, numpy.generic):
+        return arg.tobytes()
+    if isinstance(arg, numpy.ndarray):
+        if arg.size != 1:
+            raise TypeError(
+                'You are trying to pass a numpy.ndarray of shape %s as a kernel '
+                'parameter. Only numpy.ndarrays of size one can be passed by '
+                'value. If you meant to pass a pointer to __global__ memory, '
+                'you need to pass a cupy.ndarray instead.' % (arg.shape,))
+        return arg.tobytes()
+    if hasattr(arg, 'ptr'):                    # MemoryPointer and friends
+        return struct.pack('Q', int(arg.ptr))
+    raise TypeError('Unsupported type %s' % type(arg))
+
+
+class Module:
+    """A code object loaded on the current device."""
+
+    def __init__(self):
+        self.ptr = 0
+        self.code = None
+
+    def __del__(self):
+        ptr, self.ptr = getattr(self, 'ptr', 0), 0
+        if ptr:
+            try:
+                _rt.lib.rt_module_unload(ptr)
+            except Exception:
+                pass
+
+    def load(self, code):
+        self.code = bytes(code)
+        if _dryrun.enabled():
+            return
+        p = ctypes.c_void_p()
+        _rt.check(_rt.lib.rt_module_load(self.code, ctypes.byref(p)))
+        self.ptr = p.value or 0
+
+    def get_function(self, name):
+        return Function(self, name)
+
+    def get_global_var(self, name):
+        """(device address, size in bytes) of a ``__device__`` variable."""
+        if _dryrun.enabled():
+            return 0, 0
+        p = ctypes.c_void_p()
+        n = ctypes.c_size_t(0)
+        _rt.check(_rt.lib.rt_module_get_global(
+            self.ptr, name.encode(), ctypes.byref(p), ctypes.byref(n)))
+        return p.value or 0, n.value
+
+
+class Function:
+    """A ``__global__`` function of a module (keeps the module alive)."""
+
+    def __init__(self, module, name):
+        self.module = module
+        self.name = name
+        self.ptr = 0
+        if _dryrun.enabled():
+            if ('\x00' + name + '\x00').encode() not in b'\x00' + module.code:
+                if name.encode() not in module.code:
+                    raise _rt.HIPError(500, 'no kernel named %r' % name)
+            return
+        p = ctypes.c_void_p()
+        _rt.check(_rt.lib.rt_module_get_function(
+            module.ptr, name.encode(), ctypes.byref(p)))
+        self.ptr = p.value or 0
+
+    def get_attribute(self, name):
+        if _dryrun.enabled():
+            return 0
+        v = ctypes.c_int(0)
+        _rt.check(_rt.lib.rt_func_get_attribute(
+            _FUNC_ATTRIBUTES[name], self.ptr, ctypes.byref(v)))
+        return v.value
+
+    @property
+    def attributes(self):
+        out = {}
+        for name in _FUNC_ATTRIBUTES:
+            try:
+                out[name] = self.get_attribute(name)
+            except _rt.HIPError:
+                pass
+        return out
+
+    def max_active_blocks_per_cu(self, block_size, dynamic_smem=0):
+        if _dryrun.enabled():
+            return 8
+        v = ctypes.c_int(0)
+        _rt.check(_rt.lib.rt_occupancy_max_active_blocks(
+            self.ptr, block_size, dynamic_smem, ctypes.byref(v)))
+        return v.value
+
+    # -- launch -----------------------------------------------------------------
+    def launch_packed(self, grid, block, arg_block, shared_mem=0, stream_ptr=None):
+        """Launch with the argument block already laid out (bytes-like)."""
+        if stream_ptr is None:
+            stream_ptr = _stream.get_current_stream_ptr()
+        gx, gy, gz = grid
+        bx, by, bz = block
+        if _dryrun.enabled():
+            _dryrun.record_launch(self.name, grid, block, shared_mem, bytes(arg_block))
+            return
+        status = _rt.lib.rt_launch_packed(
+            self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr,
+            arg_block, len(arg_block))
+        if status != 0:
+            _rt.check(status)
+
+    def __call__(self, grid, block, args, shared_mem=0, stream=None):
+        """Launch with one Python object per kernel parameter."""
+        grid = tuple(grid) + (1,) * (3 - len(grid))
+        block = tuple(block) + (1,) * (3 - len(block))
+        bufs = [ctypes.create_string_buffer(b, len(b))
+                for b in map(_arg_to_bytes, args)]
+        stream_ptr = (_stream.get_current_stream_ptr() if stream is None
+                      else stream.ptr)
+        if _dryrun.enabled():
+            _dryrun.record_launch(self.name, grid, block, shared_mem,
+                                  b''.join(b.raw for b in bufs))
+            return
+        params = (ctypes.c_void_p * max(len(bufs), 1))(
+            *[ctypes.addressof(b) for b in bufs])
+        _rt.check(_rt.lib.rt_launch(
+            self.ptr, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+            shared_mem, stream_ptr, params))
+
+    def linear_launch(self, size, args, shared_mem=0, block_max_size=128,
+                      stream=None):
+        """1-D launch of ``size`` threads in blocks of at most
+        ``block_max_size``; the grid is capped so that grid*block stays within
+        the 2**32-1 work-items one dispatch may hold (kernels loop)."""
+        block = max(1, min(block_max_size, size))
+        grid = max(1, min((size + block - 1) // block, 0x7fffffff,
+                          0xffffffff // block))
+        self((grid,), (block,), args, shared_mem, stream)

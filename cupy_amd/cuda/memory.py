@@ -1,0 +1,456 @@
+"""Device memory: allocations, pointers and the caching pool.
+
+Python face of the native pool in ``csrc/pool.cpp``.  API and behaviour follow
+the reference's ``cupy/cuda/memory.pyx`` (Memory :105-124, MemoryPointer
+:458-765, PooledMemory :943-1038, SingleDeviceMemoryPool :1217-1563,
+MemoryPool :1566-1737, allocator registry :892-940).
+"""
+import contextlib
+import ctypes
+import gc
+import threading
+import warnings
+import weakref
+
+from cupy_amd import _dryrun
+from cupy_amd import _rt
+from cupy_amd.cuda import device as _device
+from cupy_amd.cuda import stream as _stream
+
+_allocation_unit_size = 512
+
+
+class OutOfMemoryError(MemoryError):
+    """Raised when the pool (or its limit) cannot satisfy a request
+    (reference: memory.pyx:55-81)."""
+
+    def __init__(self, size, total, limit=0):
+        self._size, self._total, self._limit = size, total, limit
+        if limit == 0:
+            msg = ('Out of memory allocating {:,} bytes '
+                   '(allocated so far: {:,} bytes).'.format(size, total))
+        else:
+            msg = ('Out of memory allocating {:,} bytes '
+                   '(allocated so far: {:,} bytes, '
+                   'limit set to: {:,} bytes).'.format(size, total, limit))
+        super().__init__(msg)
+
+    def __reduce__(self):
+        return (type(self), (self._size, self._total, self._limit))
+
+
+class BaseMemory:
+    """A piece of device memory: ``ptr``, ``size``, ``device_id``."""
+    ptr = 0
+    size = 0
+    device_id = 0
+
+    def __int__(self):
+        return self.ptr
+
+    @property
+    def device(self):
+        return _device.Device(self.device_id)
+
+
+class Memory(BaseMemory):
+    """An allocation straight from the driver, freed when collected."""
+
+    def __init__(self, size):
+        self.size = size
+        self.device_id = _device.get_device_id()
+        self.ptr = 0
+        if size > 0:
+            if _dryrun.enabled():
+                self.ptr = _dryrun.fake_alloc(size)
+            else:
+                p = ctypes.c_void_p()
+                _rt.check(_rt.lib.rt_malloc(ctypes.byref(p), size))
+                self.ptr = p.value or 0
+
+    def __del__(self):
+        ptr, self.ptr = getattr(self, 'ptr', 0), 0
+        if ptr and type(self) is Memory and not _dryrun.enabled():
+            try:
+                _rt.lib.rt_free(ptr)
+            except Exception:
+                pass
+
+
+class UnownedMemory(BaseMemory):
+    """Memory owned by somebody else (``owner`` is kept alive)."""
+
+    def __init__(self, ptr, size, owner, device_id=-1):
+        if device_id < 0:
+            device_id = _device.get_device_id()
+        self.ptr = ptr
+        self.size = size
+        self.device_id = device_id
+        self._owner = owner
+
+
+class PooledMemory(BaseMemory):
+    """A block handed out by a pool; returns to the pool when collected or on
+    ``free()`` (a second ``free()`` does nothing)."""
+
+    def __init__(self, ptr, size, device_id, pool):
+        self.ptr = ptr
+        self.size = size
+        self.device_id = device_id
+        self._pool = weakref.ref(pool)
+
+    def free(self):
+        ptr, self.ptr = self.ptr, 0
+        if not ptr:
+            return
+        pool = self._pool()
+        if pool is not None:
+            pool._free(ptr, self.size)
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _as_host_address(obj):
+    if isinstance(obj, int):
+        return obj
+    if isinstance(obj, ctypes.c_void_p):
+        return obj.value or 0
+    if hasattr(obj, 'ctypes'):          # numpy array
+        return obj.ctypes.data
+    return ctypes.cast(obj, ctypes.c_void_p).value or 0
+
+
+class MemoryPointer:
+    """Address inside a ``BaseMemory``: ``ptr == mem.ptr + offset``."""
+    __slots__ = ('mem', 'ptr', 'device_id')
+
+    def __init__(self, mem, offset):
+        self.mem = mem
+        self.ptr = mem.ptr + offset
+        self.device_id = mem.device_id
+
+    def __int__(self):
+        return self.ptr
+
+    def __repr__(self):
+        return '<MemoryPointer 0x%x device=%d mem=%r>' % (
+            self.ptr, self.device_id, self.mem)
+
+    @property
+    def device(self):
+        return _device.Device(self.device_id)
+
+    def __add__(self, offset):
+        return MemoryPointer(self.mem, self.ptr - self.mem.ptr + int(offset))
+
+    __radd__ = __add__
+
+    def __iadd__(self, offset):
+        self.ptr += int(offset)
+        return self
+
+    def __sub__(self, offset):
+        return self + (-int(offset))
+
+    def __isub__(self, offset):
+        self.ptr -= int(offset)
+        return self
+
+    # -- copies ---------------------------------------------------------------
+    def copy_from_device(self, src, size):
+        if size > 0 and not _dryrun.enabled():
+            _rt.check(_rt.lib.rt_memcpy(self.ptr, src.ptr, size, _rt.MEMCPY_D2D))
+
+    def copy_from_device_async(self, src, size, stream=None):
+        if size > 0 and not _dryrun.enabled():
+            sptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
+            _rt.check(_rt.lib.rt_memcpy_async(
+                self.ptr, src.ptr, size, _rt.MEMCPY_D2D, sptr))
+
+    def copy_from_host(self, mem, size):
+        if size > 0 and not _dryrun.enabled():
+            _rt.check(_rt.lib.rt_memcpy(
+                self.ptr, _as_host_address(mem), size, _rt.MEMCPY_H2D))
+
+    def copy_from_host_async(self, mem, size, stream=None):
+        if size > 0 and not _dryrun.enabled():
+            sptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
+            _rt.check(_rt.lib.rt_memcpy_async(
+                self.ptr, _as_host_address(mem), size, _rt.MEMCPY_H2D, sptr))
+
+    def copy_from(self, mem, size):
+        if isinstance(mem, MemoryPointer):
+            self.copy_from_device(mem, size)
+        else:
+            self.copy_from_host(mem, size)
+
+    def copy_from_async(self, mem, size, stream=None):
+        if isinstance(mem, MemoryPointer):
+            self.copy_from_device_async(mem, size, stream)
+        else:
+            self.copy_from_host_async(mem, size, stream)
+
+    def copy_to_host(self, mem, size):
+        if _dryrun.enabled():
+            _dryrun.forbid('copying device memory to the host')
+        if size > 0:
+            _rt.check(_rt.lib.rt_memcpy(
+                _as_host_address(mem), self.ptr, size, _rt.MEMCPY_D2H))
+
+    def copy_to_host_async(self, mem, size, stream=None):
+        if _dryrun.enabled():
+            _dryrun.forbid('copying device memory to the host')
+        if size > 0:
+            sptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
+            _rt.check(_rt.lib.rt_memcpy_async(
+                _as_host_address(mem), self.ptr, size, _rt.MEMCPY_D2H, sptr))
+
+    def memset(self, value, size):
+        if size > 0 and not _dryrun.enabled():
+            _rt.check(_rt.lib.rt_memset(self.ptr, value, size))
+
+    def memset_async(self, value, size, stream=None):
+        if size > 0 and not _dryrun.enabled():
+            sptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
+            _rt.check(_rt.lib.rt_memset_async(self.ptr, value, size, sptr))
+
+
+def _malloc(size):
+    """Plain driver allocation wrapped as a pointer (no pooling)."""
+    return MemoryPointer(Memory(size), 0)
+
+
+def _round_size(size):
+    """Rounds up to the pool's 512-byte allocation unit."""
+    return (size + _allocation_unit_size - 1) // _allocation_unit_size \
+        * _allocation_unit_size
+
+
+def _parse_limit_string(limit=None):
+    """``'1073741824'`` -> size, ``'70.5%'`` -> fraction (value of
+    ``CUPY_GPU_MEMORY_LIMIT``)."""
+    import os
+    if limit is None:
+        limit = os.environ.get('CUPY_GPU_MEMORY_LIMIT')
+    size = None
+    fraction = None
+    if limit is not None:
+        if limit.endswith('%'):
+            fraction = float(limit[:-1]) / 100.0
+        else:
+            size = int(limit)
+    return {'size': size, 'fraction': fraction}
+
+
+class SingleDeviceMemoryPool:
+    """Caching pool of one device.
+
+    ``allocator`` is a callable ``size -> MemoryPointer`` used to obtain fresh
+    memory; by default the native core calls ``hipMalloc`` itself.
+    """
+
+    def __init__(self, allocator=None):
+        self._device_id = _device.get_device_id()
+        self._handle = ctypes.c_void_p()
+        self._live = {}      # address -> MemoryPointer from a Python allocator
+        self._callbacks = None
+        if allocator is None and _dryrun.enabled():
+            allocator = _malloc
+        if allocator is None or allocator is _malloc and not _dryrun.enabled():
+            _rt.check(_rt.lib.rt_pool_create(ctypes.byref(self._handle)))
+        else:
+            live = self._live
+
+            def alloc_cb(ctx, size, out):
+                try:
+                    memptr = allocator(size)
+                except Exception:
+                    return 1
+                live[memptr.ptr] = memptr
+                out[0] = memptr.ptr
+                return 0
+
+            def free_cb(ctx, address, size):
+                live.pop(address, None)
+
+            self._callbacks = (_rt.POOL_ALLOC_FN(alloc_cb), _rt.POOL_FREE_FN(free_cb))
+            _rt.check(_rt.lib.rt_pool_create_with_allocator(
+                ctypes.byref(self._handle), self._callbacks[0],
+                self._callbacks[1], None))
+        limit = _parse_limit_string()
+        if limit['size'] is not None or limit['fraction'] is not None:
+            self.set_limit(**limit)
+
+    def __del__(self):
+        handle, self._handle = getattr(self, '_handle', None), None
+        if handle:
+            try:
+                _rt.lib.rt_pool_destroy(handle)
+            except Exception:
+                pass
+
+    # -- allocation -------------------------------------------------------------
+    def malloc(self, size):
+        if size == 0:
+            return MemoryPointer(Memory(0), 0)
+        rounded = _round_size(size)
+        stream_ident = _stream.get_current_stream_ptr()
+        addr = ctypes.c_uint64(0)
+        lib = _rt.lib
+        status = lib.rt_pool_malloc(self._handle, rounded, stream_ident, ctypes.byref(addr))
+        if status == _rt.RT_ERR_POOL_OOM:
+            # Last resort before giving up: collect garbage cycles that may be
+            # keeping arrays (and so pool blocks) alive.
+            gc.collect()
+            status = lib.rt_pool_malloc(
+                self._handle, rounded, stream_ident, ctypes.byref(addr))
+            if status == _rt.RT_ERR_POOL_OOM:
+                raise OutOfMemoryError(rounded, self.total_bytes(), self.get_limit())
+        _rt.check(status)
+        mem = PooledMemory(addr.value, rounded, self._device_id, self)
+        return MemoryPointer(mem, 0)
+
+    def _free(self, ptr, size):
+        handle = self._handle
+        if handle:
+            _rt.lib.rt_pool_free(handle, ptr)
+
+    def free_all_blocks(self, stream=None):
+        if stream is None:
+            _rt.check(_rt.lib.rt_pool_free_all_blocks(self._handle, 1, 0))
+        else:
+            _rt.check(_rt.lib.rt_pool_free_all_blocks(self._handle, 0, stream.ptr))
+
+    def free_all_free(self):
+        warnings.warn('free_all_free is deprecated. Use free_all_blocks instead.',
+                      DeprecationWarning)
+        self.free_all_blocks()
+
+    # -- statistics ---------------------------------------------------------------
+    def _stats(self):
+        vals = [ctypes.c_size_t(0) for _ in range(4)]
+        _rt.check(_rt.lib.rt_pool_stats(self._handle, *[ctypes.byref(v) for v in vals]))
+        return tuple(v.value for v in vals)
+
+    def used_bytes(self):
+        return self._stats()[0]
+
+    def free_bytes(self):
+        return self._stats()[1]
+
+    def total_bytes(self):
+        return self._stats()[2]
+
+    def n_free_blocks(self):
+        return self._stats()[3]
+
+    # -- limit -----------------------------------------------------------------------
+    def set_limit(self, size=None, fraction=None):
+        if size is None:
+            if fraction is None:
+                size = 0
+            else:
+                if not 0 <= fraction <= 1:
+                    raise ValueError('memory limit fraction out of range: %r' % fraction)
+                _, total = _device.Device(self._device_id).mem_info
+                size = int(fraction * total)
+        else:
+            if fraction is not None:
+                raise ValueError('size and fraction cannot be specified at one time')
+            if size < 0:
+                raise ValueError('memory limit size out of range: %r' % size)
+        _rt.check(_rt.lib.rt_pool_set_limit(self._handle, int(size)))
+
+    def get_limit(self):
+        v = ctypes.c_size_t(0)
+        _rt.check(_rt.lib.rt_pool_get_limit(self._handle, ctypes.byref(v)))
+        return v.value
+
+
+class MemoryPool:
+    """Pool for every device of the process; one ``SingleDeviceMemoryPool`` per
+    device, created on first use."""
+
+    def __init__(self, allocator=None):
+        self._allocator = allocator
+        self._pools = {}
+        self._lock = threading.Lock()
+
+    def _pool(self):
+        dev = _device.get_device_id()
+        pool = self._pools.get(dev)
+        if pool is None:
+            with self._lock:
+                pool = self._pools.get(dev)
+                if pool is None:
+                    pool = SingleDeviceMemoryPool(self._allocator)
+                    self._pools[dev] = pool
+        return pool
+
+    def malloc(self, size):
+        return self._pool().malloc(size)
+
+    def free_all_blocks(self, stream=None):
+        self._pool().free_all_blocks(stream)
+
+    def free_all_free(self):
+        self._pool().free_all_free()
+
+    def n_free_blocks(self):
+        return self._pool().n_free_blocks()
+
+    def used_bytes(self):
+        return self._pool().used_bytes()
+
+    def free_bytes(self):
+        return self._pool().free_bytes()
+
+    def total_bytes(self):
+        return self._pool().total_bytes()
+
+    def set_limit(self, size=None, fraction=None):
+        self._pool().set_limit(size, fraction)
+
+    def get_limit(self):
+        return self._pool().get_limit()
+
+
+# -- allocator registry ------------------------------------------------------------
+_current_allocator = _malloc
+_thread_local = threading.local()
+
+
+def alloc(size):
+    """Allocates through the current allocator (thread-local override first)."""
+    return get_allocator()(size)
+
+
+def set_allocator(allocator=None):
+    """Sets the process-wide allocator; ``None`` means plain driver allocation."""
+    global _current_allocator
+    if getattr(_thread_local, 'allocator', None) is not None:
+        raise ValueError('Can\'t change the global allocator inside '
+                         '`using_allocator` context manager')
+    _current_allocator = _malloc if allocator is None else allocator
+
+
+def get_allocator():
+    override = getattr(_thread_local, 'allocator', None)
+    return _current_allocator if override is None else override
+
+
+@contextlib.contextmanager
+def using_allocator(allocator=None):
+    """Thread-local, nestable allocator override."""
+    if allocator is None:
+        allocator = _malloc
+    previous = getattr(_thread_local, 'allocator', None)
+    _thread_local.allocator = allocator
+    try:
+        yield
+    finally:
+        _thread_local.allocator = previous
