@@ -30,3 +30,79 @@ cuda.set_allocator(_default_memory_pool.malloc)
 def get_default_memory_pool():
     """The pool that backs every ``ndarray`` allocation by default."""
     return _default_memory_pool
+
+from cupy_amd._core._reduction import (  # noqa
+    ReductionKernel, create_reduction_func)
+from cupy_amd._core.fusion import fuse  # noqa
+from cupy_amd._core._routines_math import sum, prod, nansum  # noqa
+from cupy_amd._core._routines_statistics import (  # noqa
+    amax, amin, argmax, argmin)
+from cupy_amd._core._routines_logic import all, any  # noqa
+from cupy_amd._creation import (  # noqa
+    empty, empty_like, zeros, zeros_like, ones, ones_like, full, full_like, arange)
+
+max = amax
+min = amin
+
+
+def mean(a, axis=None, dtype=None, out=None, keepdims=False):
+    """Arithmetic mean along the given axes."""
+    return a.mean(axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+
+
+def where(condition, x=None, y=None):
+    """Elementwise selection ``condition ? x : y``."""
+    if x is None or y is None:
+        raise NotImplementedError('where() with one argument is not supported')
+    return _ufuncs_module._where_ufunc(condition.astype('?', copy=False), x, y)
+
+
+def clip(a, a_min, a_max, out=None):
+    """Limits the values of an array to ``[a_min, a_max]``."""
+    return _ufuncs_module._clip(a, a_min, a_max, out=out)
+
+
+def transpose(a, axes=None):
+    return a.transpose(axes)
+
+
+def reshape(a, newshape, order='C'):
+    return a.reshape(newshape, order=order)
+
+
+def ravel(a, order='C'):
+    return a.ravel(order)
+
+
+def broadcast_to(array, shape):
+    """Read-only zero-stride view of ``array`` with the given shape."""
+    shape = tuple(shape) if isinstance(shape, (tuple, list)) else (shape,)
+    if array.ndim > len(shape):
+        raise ValueError('input operand has more dimensions than allowed by '
+                         'the axis remapping')
+    off = len(shape) - array.ndim
+    strides = [0] * len(shape)
+    for i, (ext, st) in enumerate(zip(array.shape, array.strides)):
+        if ext == shape[off + i]:
+            strides[off + i] = st
+        elif ext != 1:
+            raise ValueError(
+                'operands could not be broadcast together with remapped shapes '
+                '[original->remapped]: {} and requested shape {}'.format(
+                    array.shape, shape))
+    return array._view(shape, tuple(strides))
+
+
+def copy(a, order='K'):
+    from cupy_amd._core import _fusion_thread_local
+    if _fusion_thread_local.is_fusing():
+        return _ufuncs_module.elementwise_copy(a)
+    return a.copy(order=order)
+
+
+def copyto(dst, src, casting='same_kind', where=None):
+    """Copies ``src`` into ``dst`` (broadcasting), optionally under a mask."""
+    if where is None:
+        _ufuncs_module.elementwise_copy(src, dst, casting=casting)
+    else:
+        _ufuncs_module.elementwise_copy(src, dst, casting=casting, _where=where)

@@ -159,7 +159,6 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
     count) and, when the body uses it, ``_ind``.
     """
     idx_t = 'ptrdiff_t' if idx64 else 'int'
-    uidx_t = 'ptrdiff_t' if idx64 else 'unsigned int'
     arrays = [op for op in operands if op.kind == 'array']
     iter_arrays = [op for op in arrays if op.name not in bcast]
     needs_ind = any(op.kind == 'indexer' for op in operands)
@@ -189,11 +188,6 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
         def f(op, value):
             return '_l_%s%s.v[_k] = %s;' % (op.name, suffix, value)
         return f
-
-    def vec_block(suffix, base_expr, indent):
-        pad = ' ' * indent
-        lines = []
-        return lines
 
     # --- vector part: `unroll` vectors per thread per trip -----------------------
     body = []
@@ -294,7 +288,6 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
     src.extend(tail)
     src.append('  %s;' % after_loop)
     src.append('}')
-    del uidx_t, vec_block
     return '\n'.join(src) + '\n'
 
 
@@ -350,7 +343,6 @@ def emit_generic(name, operands, operation, typedefs='', preamble='',
     src.append('  }')
     src.append('  %s;' % after_loop)
     src.append('}')
-    del block
     return '\n'.join(src) + '\n'
 
 

@@ -1,0 +1,474 @@
+"""HIP source emitters for reduction kernels (gfx950, wave64).
+
+A reduction is stated as in the reference (cupy/_core/_reduction.pyx:44-126):
+``pre_map_expr`` over the input element(s), ``reduce_expr`` over ``a`` and
+``b`` of type ``_type_reduce``, ``post_map_expr`` storing the final value, an
+``identity``, and ``_J`` = position of the element along the reduced axes.
+Where the reference has one template (strided per-thread accumulation followed
+by an LDS tree with a barrier per level, one launch geometry formula), this
+module has three kernels, chosen by the host from the canonical 2-d form
+``in[i, j]`` (i = output index, j = reduce index) of the problem:
+
+``rows``     the reduce axis is contiguous in memory.  A group of G lanes
+             (G = 1..64, or a whole 256-thread workgroup) owns a row, reads it
+             with 128-bit loads into per-lane accumulators and combines them
+             with wave64 cross-lane exchanges -- no LDS and no barrier unless a
+             workgroup shares the row.  Long rows with few outputs are split
+             across workgroups (grid.y) into partial results.
+``cols``     the output axis is contiguous (e.g. ``axis=0`` of a C-order
+             matrix).  Threads own ``V`` adjacent output columns and walk down
+             the reduce axis, TY row-slices per workgroup and grid.y slices per
+             launch; slices are combined through cross-lane exchanges, LDS and,
+             across workgroups, a partial-result buffer.
+``generic``  any strides: CIndexer addressing, same thread layout as ``cols``.
+
+Partial results are combined by a second ``cols`` launch that reads
+``_type_reduce`` values (``partial_in``) -- deterministic, no atomics.
+"""
+BLOCK = 256
+WAVE = 64
+
+
+class RArg:
+    """Kernel parameter of a reduction.
+
+    kind     'in' (iterated input array), 'out' (output array), 'raw' (CArray
+             passed through), 'scalar'
+    name     identifier used by the expressions
+    store_t  element type in memory / scalar type
+    var_t    type of the variable the expressions see
+    bcast_r  'in' only: the array does not vary along the reduce axis
+    bcast_o  'in' only: the array does not vary along the output axis
+    """
+
+    def __init__(self, kind, name, store_t, var_t=None, is_const=True, ndim=0,
+                 c_contiguous=False, index_32=True, bcast_r=False, bcast_o=False):
+        self.kind = kind
+        self.name = name
+        self.store_t = store_t
+        self.var_t = var_t or store_t
+        self.is_const = is_const
+        self.ndim = ndim
+        self.c_contiguous = c_contiguous
+        self.index_32 = index_32
+        self.bcast_r = bcast_r
+        self.bcast_o = bcast_o
+
+    def key(self):
+        return (self.kind, self.name, self.store_t, self.var_t, self.is_const,
+                self.ndim, self.c_contiguous, self.index_32, self.bcast_r,
+                self.bcast_o)
+
+
+def _prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr):
+    return '''#include <cupy/carray.cuh>
+%s
+%s
+#define REDUCE(a, b) (%s)
+#define POST_MAP(a) (%s)
+typedef %s _type_reduce;
+// lets the host learn sizeof(_type_reduce) (size of this variable) when it has
+// to allocate a buffer of partial results
+__device__ __attribute__((used)) char _cupy_type_reduce_probe[sizeof(_type_reduce)];
+struct _ReduceOp {
+  __device__ __forceinline__ _type_reduce operator()(
+      const _type_reduce& a, const _type_reduce& b) const {
+    return REDUCE(a, b);
+  }
+};
+''' % (typedefs, preamble, reduce_expr, post_map_expr, reduce_type)
+
+
+def _raw_param(a):
+    const = 'const ' if a.is_const else ''
+    return '%sCArray<%s, %d, %d, %d> %s' % (
+        const, a.store_t, a.ndim, a.c_contiguous, a.index_32, a.name)
+
+
+def _fast_params(args, idx_t, partial_in, partial_out):
+    """Parameter list of the rows / cols kernels."""
+    parts = []
+    for a in args:
+        if a.kind == 'in':
+            if partial_in:
+                parts.append('const _type_reduce* __restrict__ _p_%s' % a.name)
+            else:
+                parts.append('const %s* __restrict__ _p_%s' % (a.store_t, a.name))
+        elif a.kind == 'out':
+            parts.append('%s* __restrict__ _p_%s' % (a.store_t, a.name))
+        elif a.kind == 'raw':
+            parts.append(_raw_param(a))
+        else:
+            parts.append('const %s %s' % (a.store_t, a.name))
+    parts.append('const %s _n_out' % idx_t)
+    parts.append('const %s _n_red' % idx_t)
+    for a in args:
+        if a.kind == 'in':
+            parts.append('const %s _so_%s' % (idx_t, a.name))   # stride along i
+            parts.append('const %s _sr_%s' % (idx_t, a.name))   # stride along j
+        elif a.kind == 'out':
+            parts.append('const %s _so_%s' % (idx_t, a.name))
+    if partial_out:
+        parts.append('_type_reduce* __restrict__ _partials')
+    return ', '.join(parts)
+
+
+def _identity_decl(identity):
+    return '_type_reduce(%s)' % identity
+
+
+def _finish(args, partial_out, pad, i_expr='_i', s_expr='_s', split_expr='blockIdx.y'):
+    """Code storing one finished value: either into the partial buffer or
+    through POST_MAP into the output element(s)."""
+    lines = []
+    if partial_out:
+        lines.append('%s_partials[(ptrdiff_t)%s * _n_out + %s] = %s;' % (
+            pad, split_expr, i_expr, s_expr))
+    else:
+        for a in args:
+            if a.kind == 'out':
+                lines.append('%s%s &%s = _p_%s[(ptrdiff_t)%s * _so_%s];' % (
+                    pad, a.var_t, a.name, a.name, i_expr, a.name))
+        lines.append('%sPOST_MAP(%s);' % (pad, s_expr))
+    return lines
+
+
+def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
+              reduce_type, typedefs='', preamble='', group=64, vec=4,
+              idx64=False, partial_out=False, stream_hint=False, unroll=2):
+    """Reduce-axis-contiguous kernel.  ``group`` lanes per row (power of two up
+    to 64) or 256 for a workgroup per row.  With ``partial_out`` the reduce
+    range is cut into gridDim.y chunks of ``_chunk`` elements (an extra kernel
+    parameter) and each (chunk, row) writes one ``_type_reduce`` partial."""
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    nt = 'true' if stream_hint else 'false'
+    ins = [a for a in args if a.kind == 'in']
+    params = _fast_params(args, idx_t, False, partial_out)
+    if partial_out:
+        params += ', const %s _chunk' % idx_t
+    block_mode = group >= BLOCK
+    lanes = BLOCK if block_mode else group
+    src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, params))
+    if block_mode:
+        src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (BLOCK // WAVE))
+        src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
+        src.append('  const int _lane = threadIdx.x;')
+        src.append('  const %s _first = blockIdx.x;' % idx_t)
+        src.append('  const %s _step = gridDim.x;' % idx_t)
+    else:
+        src.append('  const int _lane = threadIdx.x %% %d;' % group)
+        src.append('  const %s _first = ((%s)blockIdx.x * %d + threadIdx.x) / %d;' % (
+            idx_t, idx_t, BLOCK, group))
+        src.append('  const %s _step = (%s)gridDim.x * %d;' % (idx_t, idx_t, BLOCK // group))
+    if partial_out:
+        src.append('  const %s _j_begin = (%s)blockIdx.y * _chunk;' % (idx_t, idx_t))
+        src.append('  const %s _j_end = (_j_begin + _chunk < _n_red) ? (_j_begin + _chunk) : _n_red;' % idx_t)
+    else:
+        src.append('  const %s _j_begin = 0;' % idx_t)
+        src.append('  const %s _j_end = _n_red;' % idx_t)
+    # inputs that do not vary along the output axis keep the same per-lane
+    # elements for every row when the row fits one trip: hoisting is left to
+    # the compiler (the loads are loop-invariant and the pointers const).
+    src.append('  for (%s _i = _first; _i < _n_out; _i += _step) {' % idx_t)
+    for a in ins:
+        src.append('    const %s* _row_%s = _p_%s + (ptrdiff_t)_i * _so_%s;' % (
+            a.store_t, a.name, a.name, a.name))
+    src.append('    _type_reduce _acc[%d];' % vec)
+    src.append('#pragma unroll')
+    src.append('    for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (
+        vec, _identity_decl(identity)))
+    if vec > 1:
+        src.append('    const %s _j_vend = _j_begin + (_j_end - _j_begin) / %d * %d;' % (
+            idx_t, vec, vec))
+        src.append('#pragma unroll %d' % unroll)
+        src.append('    for (%s _j = _j_begin + _lane * %d; _j < _j_vend; _j += %d) {' % (
+            idx_t, vec, lanes * vec))
+        for a in ins:
+            if a.bcast_r:
+                src.append('      const %s _b_%s = _row_%s[0];' % (a.store_t, a.name, a.name))
+            else:
+                src.append('      const cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>('
+                           '_row_%s + _j);' % (a.store_t, vec, a.name, a.store_t, vec,
+                                               nt, a.name))
+        src.append('#pragma unroll')
+        src.append('      for (int _k = 0; _k < %d; ++_k) {' % vec)
+        src.append('        const IndexT _J = _j + _k;')
+        for a in ins:
+            val = ('_b_%s' % a.name) if a.bcast_r else ('_l_%s.v[_k]' % a.name)
+            src.append('        const %s %s(%s);' % (a.var_t, a.name, val))
+        src.append('        _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+        src.append('        _acc[_k] = REDUCE(_acc[_k], _a);')
+        src.append('      }')
+        src.append('    }')
+    else:
+        src.append('    const %s _j_vend = _j_begin;' % idx_t)
+    # ragged tail (and the whole row when vec == 1)
+    src.append('    for (%s _j = _j_vend + _lane; _j < _j_end; _j += %d) {' % (idx_t, lanes))
+    src.append('      const IndexT _J = _j;')
+    for a in ins:
+        val = ('_row_%s[0]' % a.name) if a.bcast_r else ('_row_%s[_j]' % a.name)
+        src.append('      const %s %s(%s);' % (a.var_t, a.name, val))
+    src.append('      _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+    src.append('      _acc[0] = REDUCE(_acc[0], _a);')
+    src.append('    }')
+    src.append('    _type_reduce _s = _acc[0];')
+    if vec > 1:
+        src.append('#pragma unroll')
+        src.append('    for (int _k = 1; _k < %d; ++_k) _s = REDUCE(_s, _acc[_k]);' % vec)
+    if block_mode:
+        src.append('    _s = cupy::group_allreduce<%d>(_s, _ReduceOp());' % WAVE)
+        src.append('    if ((threadIdx.x %% %d) == 0) _sm[threadIdx.x / %d] = _s;' % (WAVE, WAVE))
+        src.append('    __syncthreads();')
+        src.append('    if (threadIdx.x == 0) {')
+        src.append('      _s = _sm[0];')
+        src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[_w]);' % (BLOCK // WAVE))
+        src.extend(_finish(args, partial_out, '      '))
+        src.append('    }')
+        src.append('    __syncthreads();')
+    else:
+        if group > 1:
+            src.append('    _s = cupy::group_allreduce<%d>(_s, _ReduceOp());' % group)
+        src.append('    if (_lane == 0) {')
+        src.extend(_finish(args, partial_out, '      '))
+        src.append('    }')
+    src.append('  }')
+    src.append('}')
+    return '\n'.join(src) + '\n'
+
+
+def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
+              reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
+              partial_in=False, partial_out=False, stream_hint=False, unroll=4):
+    """Output-axis-contiguous kernel.  Thread layout: ``tx`` threads across
+    the output axis (each owning ``vec`` adjacent outputs) times 256/tx slices
+    of the reduce axis; gridDim.y further slices.  ``partial_in``: the single
+    input holds ``_type_reduce`` values that are combined as they are."""
+    assert tx in (1, 2, 4, 8, 16, 32, 64)
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    nt = 'true' if stream_hint else 'false'
+    ins = [a for a in args if a.kind == 'in']
+    ty = BLOCK // tx
+    waves = BLOCK // WAVE
+    params = _fast_params(args, idx_t, partial_in, partial_out)
+    src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, params))
+    src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (
+        waves * tx * vec))
+    src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
+    src.append('  const int _tx = threadIdx.x %% %d;' % tx)
+    src.append('  const int _ty = threadIdx.x / %d;' % tx)
+    src.append('  const %s _c = ((%s)blockIdx.x * %d + _tx) * %d;' % (idx_t, idx_t, tx, vec))
+    src.append('  _type_reduce _acc[%d];' % vec)
+    src.append('#pragma unroll')
+    src.append('  for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (vec, _identity_decl(identity)))
+    src.append('  if (_c < _n_out) {')
+    src.append('    const bool _full = _c + %d <= _n_out;' % vec)
+    src.append('    if (_full) {')
+    src.append('#pragma unroll %d' % unroll)
+    src.append('      for (%s _j = (%s)blockIdx.y * %d + _ty; _j < _n_red; _j += (%s)gridDim.y * %d) {' % (
+        idx_t, idx_t, ty, idx_t, ty))
+    for a in ins:
+        if partial_in:
+            # partial results may have any size: plain element reads
+            src.append('        const _type_reduce* _l_%s = _p_%s + (ptrdiff_t)_j * _sr_%s + _c;' % (
+                a.name, a.name, a.name))
+        elif a.bcast_o:
+            src.append('        const %s _b_%s = _p_%s[(ptrdiff_t)_j * _sr_%s];' % (
+                a.store_t, a.name, a.name, a.name))
+        else:
+            src.append('        const cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>('
+                       '_p_%s + (ptrdiff_t)_j * _sr_%s + _c);' % (
+                           a.store_t, vec, a.name, a.store_t, vec, nt, a.name, a.name))
+    src.append('        const IndexT _J = _j;')
+    src.append('#pragma unroll')
+    src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
+    if partial_in:
+        a = ins[0]
+        src.append('          _acc[_k] = REDUCE(_acc[_k], _l_%s[_k]);' % a.name)
+    else:
+        for a in ins:
+            val = ('_b_%s' % a.name) if a.bcast_o else ('_l_%s.v[_k]' % a.name)
+            src.append('          const %s %s(%s);' % (a.var_t, a.name, val))
+        src.append('          _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+        src.append('          _acc[_k] = REDUCE(_acc[_k], _a);')
+    src.append('        }')
+    src.append('      }')
+    src.append('    } else {')
+    src.append('      for (%s _j = (%s)blockIdx.y * %d + _ty; _j < _n_red; _j += (%s)gridDim.y * %d) {' % (
+        idx_t, idx_t, ty, idx_t, ty))
+    src.append('        const IndexT _J = _j;')
+    src.append('        for (int _k = 0; _k < %d && _c + _k < _n_out; ++_k) {' % vec)
+    if partial_in:
+        a = ins[0]
+        src.append('          _acc[_k] = REDUCE(_acc[_k], _p_%s[(ptrdiff_t)_j * _sr_%s + _c + _k]);' % (
+            a.name, a.name))
+    else:
+        for a in ins:
+            if a.bcast_o:
+                val = '_p_%s[(ptrdiff_t)_j * _sr_%s]' % (a.name, a.name)
+            else:
+                val = '_p_%s[(ptrdiff_t)_j * _sr_%s + _c + _k]' % (a.name, a.name)
+            src.append('          const %s %s(%s);' % (a.var_t, a.name, val))
+        src.append('          _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+        src.append('          _acc[_k] = REDUCE(_acc[_k], _a);')
+    src.append('        }')
+    src.append('      }')
+    src.append('    }')
+    src.append('  }')
+    # combine the row-slices held by the lanes of one wave, then the waves
+    if tx < WAVE:
+        src.append('#pragma unroll')
+        src.append('  for (int _k = 0; _k < %d; ++_k) {' % vec)
+        src.append('#pragma unroll')
+        src.append('    for (int _m = %d; _m < %d; _m <<= 1) {' % (tx, WAVE))
+        src.append('      _type_reduce _o = cupy::shfl_xor(_acc[_k], _m);')
+        src.append('      _acc[_k] = REDUCE(_acc[_k], _o);')
+        src.append('    }')
+        src.append('  }')
+    src.append('  const int _wave = threadIdx.x / %d;' % WAVE)
+    src.append('  if ((threadIdx.x %% %d) < %d) {' % (WAVE, tx))
+    src.append('#pragma unroll')
+    src.append('    for (int _k = 0; _k < %d; ++_k) _sm[(_wave * %d + _tx) * %d + _k] = _acc[_k];' % (
+        vec, tx, vec))
+    src.append('  }')
+    src.append('  __syncthreads();')
+    src.append('  if (threadIdx.x < %d && _c < _n_out) {' % tx)
+    src.append('    for (int _k = 0; _k < %d && _c + _k < _n_out; ++_k) {' % vec)
+    src.append('      _type_reduce _s = _sm[_tx * %d + _k];' % vec)
+    src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[(_w * %d + _tx) * %d + _k]);' % (
+        waves, tx, vec))
+    src.append('      const %s _i = _c + _k;' % idx_t)
+    src.extend(_finish(args, partial_out, '      '))
+    src.append('    }')
+    src.append('  }')
+    src.append('}')
+    return '\n'.join(src) + '\n'
+
+
+def emit_generic(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
+                 reduce_type, typedefs='', preamble='', tx=64, in_ndim=1,
+                 out_ndim=1, in_index_32=True, out_index_32=True,
+                 partial_out=False, partial_in=False):
+    """Any-stride kernel.  The inputs are views whose leading axes are the
+    reduced ones; element (i, J) of the problem has linear index
+    ``i + J * _out_ind.size()`` in ``_in_ind`` (the reference's convention,
+    cupy/_core/_reduction.pyx:75-93), so expressions may also use ``_in_ind``,
+    ``_out_ind``, ``_i`` and ``_j``."""
+    assert tx in (1, 2, 4, 8, 16, 32, 64)
+    ty = BLOCK // tx
+    waves = BLOCK // WAVE
+    parts = []
+    for a in args:
+        if a.kind in ('in', 'out'):
+            const = 'const ' if (a.kind == 'in' and a.is_const) else ''
+            parts.append('%sCArray<%s, %d, %d, %d> _raw_%s' % (
+                const, a.store_t, a.ndim, a.c_contiguous, a.index_32, a.name))
+        elif a.kind == 'raw':
+            parts.append(_raw_param(a))
+        else:
+            parts.append('const %s %s' % (a.store_t, a.name))
+    parts.append('CIndexer<%d, %d> _in_ind' % (in_ndim, in_index_32))
+    parts.append('CIndexer<%d, %d> _out_ind' % (out_ndim, out_index_32))
+    if partial_out:
+        parts.append('_type_reduce* _partials')
+    params = ', '.join(parts)
+    src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, params))
+    src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (
+        waves * tx))
+    src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
+    src.append('  const int _tx = threadIdx.x %% %d;' % tx)
+    src.append('  const int _ty = threadIdx.x / %d;' % tx)
+    src.append('  const ptrdiff_t _n_out = _out_ind.size();')
+    src.append('  const ptrdiff_t _n_red = _n_out ? _in_ind.size() / _n_out : 0;')
+    src.append('  for (ptrdiff_t _i_base = (ptrdiff_t)blockIdx.x * %d; _i_base < _n_out; '
+               '_i_base += (ptrdiff_t)gridDim.x * %d) {' % (tx, tx))
+    src.append('    const ptrdiff_t _i = _i_base + _tx;')
+    src.append('    _type_reduce _s = %s;' % _identity_decl(identity))
+    src.append('    if (_i < _n_out) {')
+    src.append('      for (ptrdiff_t _Jl = (ptrdiff_t)blockIdx.y * %d + _ty; _Jl < _n_red; '
+               '_Jl += (ptrdiff_t)gridDim.y * %d) {' % (ty, ty))
+    src.append('        const IndexT _J = _Jl;')
+    src.append('        const ptrdiff_t _j = _i + _Jl * _n_out;')
+    src.append('        _in_ind.set(_j);')
+    for a in args:
+        if a.kind == 'in':
+            if a.is_const:
+                src.append('        const %s %s(_raw_%s[_in_ind.get()]);' % (
+                    a.var_t, a.name, a.name))
+            else:
+                src.append('        %s &%s = _raw_%s[_in_ind.get()];' % (
+                    a.var_t, a.name, a.name))
+    src.append('        _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+    src.append('        _s = REDUCE(_s, _a);')
+    src.append('      }')
+    src.append('    }')
+    if tx < WAVE:
+        src.append('#pragma unroll')
+        src.append('    for (int _m = %d; _m < %d; _m <<= 1) {' % (tx, WAVE))
+        src.append('      _type_reduce _o = cupy::shfl_xor(_s, _m);')
+        src.append('      _s = REDUCE(_s, _o);')
+        src.append('    }')
+    src.append('    if ((threadIdx.x %% %d) < %d) _sm[(threadIdx.x / %d) * %d + _tx] = _s;' % (
+        WAVE, tx, WAVE, tx))
+    src.append('    __syncthreads();')
+    src.append('    if (threadIdx.x < %d && _i < _n_out) {' % tx)
+    src.append('      _s = _sm[_tx];')
+    src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[_w * %d + _tx]);' % (
+        waves, tx))
+    if partial_out:
+        src.append('      _partials[(ptrdiff_t)blockIdx.y * _n_out + _i] = _s;')
+    else:
+        src.append('      _out_ind.set(_i);')
+        for a in args:
+            if a.kind == 'out':
+                src.append('      %s &%s = _raw_%s[_out_ind.get()];' % (
+                    a.var_t, a.name, a.name))
+        src.append('      POST_MAP(_s);')
+    src.append('    }')
+    src.append('    __syncthreads();')
+    src.append('  }')
+    src.append('}')
+    del partial_in
+    return '\n'.join(src) + '\n'
+
+
+def emit_finalize_generic(name, args, identity, reduce_expr, post_map_expr,
+                          reduce_type, typedefs='', preamble='', out_ndim=1,
+                          out_index_32=True):
+    """Second pass after a split ``generic`` launch: combines
+    ``_partials[s][i]`` over s and applies POST_MAP through the strided
+    output views.  One thread per output."""
+    parts = []
+    for a in args:
+        if a.kind == 'out':
+            parts.append('CArray<%s, %d, %d, %d> _raw_%s' % (
+                a.store_t, a.ndim, a.c_contiguous, a.index_32, a.name))
+        elif a.kind == 'raw':
+            parts.append(_raw_param(a))
+        elif a.kind == 'scalar':
+            parts.append('const %s %s' % (a.store_t, a.name))
+    parts.append('CIndexer<%d, %d> _out_ind' % (out_ndim, out_index_32))
+    parts.append('const _type_reduce* _partials')
+    parts.append('const int _n_split')
+    params = ', '.join(parts)
+    src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, params))
+    src.append('  const ptrdiff_t _n_out = _out_ind.size();')
+    src.append('  CUPY_FOR(_i, _n_out) {')
+    src.append('    _type_reduce _s = %s;' % _identity_decl(identity))
+    src.append('    for (int _sp = 0; _sp < _n_split; ++_sp) '
+               '_s = REDUCE(_s, _partials[(ptrdiff_t)_sp * _n_out + _i]);')
+    src.append('    _out_ind.set(_i);')
+    for a in args:
+        if a.kind == 'out':
+            src.append('    %s &%s = _raw_%s[_out_ind.get()];' % (a.var_t, a.name, a.name))
+    src.append('    POST_MAP(_s);')
+    src.append('  }')
+    src.append('}')
+    return '\n'.join(src) + '\n'

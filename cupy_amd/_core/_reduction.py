@@ -1,0 +1,835 @@
+"""ReductionKernel, simple reductions (sum, argmax, ...) and their launch
+planning.
+
+The call surface and semantics follow the reference's
+cupy/_core/_reduction.pyx (axis handling :147-176, ``_call`` :309-427,
+``create_reduction_func`` / ``_SimpleReductionKernel`` :557-708,
+``ReductionKernel`` :716-917).  The geometry is not the reference's
+``_get_block_specs`` (:239-253): the problem is brought into a canonical
+``(n_out, n_red)`` form and one of the kernels of ``_codegen_reduction`` is
+launched, split over the grid with a second combining pass when there are too
+few outputs to fill 256 CUs.
+"""
+import struct
+import threading
+import warnings
+
+import numpy
+
+from cupy_amd import _dryrun
+from cupy_amd._core import _carray
+from cupy_amd._core import _codegen_reduction as _cg
+from cupy_amd._core import _kernel
+from cupy_amd._core import internal
+from cupy_amd._core._codegen_elementwise import uses_identifier
+from cupy_amd._core._dtype import get_dtype
+from cupy_amd._core._kernel import (
+    _get_param_info, _decide_params_type, _preprocess_args, _broadcast,
+    _get_out_args_from_optionals, _get_out_args_with_params,
+    _check_peer_access, _scalar_struct_code, _max_vector_width, _aligned)
+from cupy_amd._core._scalar import CScalar, get_typename as _get_typename
+from cupy_amd._core.core import ndarray, _convert_from_cupy_like
+from cupy_amd.cuda import compiler
+from cupy_amd.cuda import device as _device
+from cupy_amd.cuda import memory as _memory
+from cupy_amd.cuda import stream as _stream
+
+_INT32_MAX = (1 << 31) - 1
+
+# Tunables: workgroups a launch should at least consist of, as a multiple of
+# the CU count, before the reduce axis is split across workgroups.
+TARGET_BLOCKS_PER_CU = 8
+MIN_BLOCKS_PER_CU = 2
+ROWS_BLOCK_MODE_BYTES = 16384   # rows at least this long get a whole workgroup
+ROWS_STREAM_HINT = False
+COLS_STREAM_HINT = False
+
+
+def _get_axis(axis, ndim):
+    """(reduce axes, remaining axes), each sorted ascending."""
+    if axis is None:
+        return tuple(range(ndim)), ()
+    if isinstance(axis, (tuple, list)):
+        axis = tuple(axis)
+    else:
+        axis = axis,
+    reduce_axis = tuple(sorted(
+        internal._normalize_axis_index(dim, ndim) for dim in axis))
+    out_axis = tuple(dim for dim in range(ndim) if dim not in reduce_axis)
+    if len(reduce_axis) + len(out_axis) != ndim:
+        raise ValueError("duplicate value in 'axis'")
+    return reduce_axis, out_axis
+
+
+def _get_out_shape(shape, reduce_axis, out_axis, keepdims):
+    if keepdims:
+        out_shape = list(shape)
+        for i in reduce_axis:
+            out_shape[i] = 1
+        return tuple(out_shape)
+    return tuple(shape[i] for i in out_axis)
+
+
+def _sort_axis(axis, strides):
+    """Axes in decreasing order of |stride| (stable)."""
+    return tuple(sorted(axis, key=lambda i: -abs(strides[i])))
+
+
+def _merge_dims(shape, strides_list):
+    """Like ``_kernel._canonical_dims`` for explicit stride lists."""
+    cshape = []
+    cstrides = [[] for _ in strides_list]
+    for d, ext in enumerate(shape):
+        if ext == 1:
+            continue
+        if cshape:
+            for cs, st in zip(cstrides, strides_list):
+                if cs[-1] != st[d] * ext:
+                    break
+            else:
+                cshape[-1] *= ext
+                for cs, st in zip(cstrides, strides_list):
+                    cs[-1] = st[d]
+                continue
+        cshape.append(ext)
+        for cs, st in zip(cstrides, strides_list):
+            cs.append(st[d])
+    return cshape, cstrides
+
+
+_known_type_sizes = {
+    'bool': 1, 'signed char': 1, 'unsigned char': 1, 'short': 2,
+    'unsigned short': 2, 'int': 4, 'unsigned int': 4, 'long long': 8,
+    'unsigned long long': 8, 'float16': 2, 'float': 4, 'double': 8,
+}
+
+
+class _AbstractReductionKernel:
+
+    def __init__(self, name, identity, in_params, out_params):
+        assert name is not None
+        assert identity is not None
+        self.name = name
+        self.__name__ = name
+        self.identity = identity
+        self.in_params = _get_param_info(in_params, True)
+        self.out_params = _get_param_info(out_params, False)
+        self._cached_codes = {}
+        self._memo = {}
+        self._lock = threading.Lock()
+
+    # Hooks of the concrete classes -----------------------------------------------------
+    def _get_expressions_and_types(self, in_args, out_args, dtype):
+        raise NotImplementedError
+
+    def _get_out_args(self, out_args, out_types, out_shape):
+        raise NotImplementedError
+
+    def _get_preamble_options(self):
+        raise NotImplementedError
+
+    def _in_var_type(self, index, param):
+        raise NotImplementedError
+
+    # -----------------------------------------------------------------------------------
+    def _call(self, in_args, out_args, a_shape, axis, dtype, keepdims, reduce_dims,
+              device_id, stream, sort_reduce_axis=True):
+        if dtype is not None:
+            dtype = get_dtype(dtype).type
+        (map_expr, reduce_expr, post_map_expr, in_types, out_types, reduce_type,
+         type_pairs) = self._get_expressions_and_types(in_args, out_args, dtype)
+
+        ndim = len(a_shape)
+        reduce_axis, out_axis = _get_axis(axis, ndim)
+        if (len(in_args) == 1 and sort_reduce_axis
+                and isinstance(in_args[0], ndarray)
+                and not in_args[0]._c_contiguous):
+            # sums do not care about the order: walking the reduced axes from
+            # the largest stride to the smallest lets them merge
+            reduce_axis = _sort_axis(reduce_axis, in_args[0]._strides)
+
+        out_shape = _get_out_shape(a_shape, reduce_axis, out_axis, keepdims)
+        out_args = self._get_out_args(out_args, out_types, out_shape)
+        ret = out_args[0]
+        if ret.size == 0:
+            return ret
+        if self.identity == '' and 0 in a_shape:
+            raise ValueError(('zero-size array to reduction operation'
+                              ' %s which has no identity') % self.name)
+
+        in_size = internal.prod(a_shape)
+        out_size = internal.prod(out_shape)
+        index_t = 'long long' if in_size // max(out_size, 1) > _INT32_MAX else 'int'
+        for x, t in zip(in_args, in_types):
+            if type(x) is CScalar:
+                x.apply_dtype(t)
+
+        typedefs = ''.join('typedef %s %s;\n' % (_get_typename(t), n)
+                           for n, t in type_pairs)
+        typedefs += 'typedef %s IndexT;\n' % index_t
+
+        self._launch(in_args, out_args, a_shape, reduce_axis, out_axis, keepdims,
+                     map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                     device_id, stream)
+        return ret
+
+    # -- planning ---------------------------------------------------------------------------
+    def _launch(self, in_args, out_args, a_shape, reduce_axis, out_axis, keepdims,
+                map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                device_id, stream):
+        stream_ptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
+        in_params = self.in_params
+        out_params = self.out_params
+        n_r = len(reduce_axis)
+        perm = reduce_axis + out_axis
+        need_perm = any(i != p for i, p in enumerate(perm))
+        has_raw = any(p.raw for p in in_params + out_params)
+        if need_perm and has_raw:
+            raise NotImplementedError('Illegal conditions')
+
+        red_shape = tuple(a_shape[i] for i in reduce_axis)
+        kept_shape = tuple(a_shape[i] for i in out_axis)
+        in_arr_idx = [i for i, (a, p) in enumerate(zip(in_args, in_params))
+                      if isinstance(a, ndarray) and not p.raw]
+        out_arr_idx = [i for i, (a, p) in enumerate(zip(out_args, out_params))
+                       if not p.raw]
+        # strides of every iterated array along the reduced / kept axes
+        in_red_strides = []
+        in_kept_strides = []
+        for i in in_arr_idx:
+            st = in_args[i]._strides
+            in_red_strides.append(tuple(st[d] for d in reduce_axis))
+            in_kept_strides.append(tuple(st[d] for d in out_axis))
+        out_kept_strides = []
+        for i in out_arr_idx:
+            o = out_args[i]
+            st = o._strides
+            if keepdims:
+                st = tuple(st[d] for d in out_axis)
+            out_kept_strides.append(tuple(st))
+
+        rshape, rstrides = _merge_dims(red_shape, in_red_strides)
+        oshape, ostrides = _merge_dims(kept_shape, in_kept_strides + out_kept_strides)
+        o_in = ostrides[:len(in_arr_idx)]
+        o_out = ostrides[len(in_arr_idx):]
+
+        exprs = (map_expr, reduce_expr, post_map_expr)
+        needs_indexers = any(
+            uses_identifier(e, n) for e in exprs + (self._get_preamble_options()[0],)
+            for n in ('_in_ind', '_out_ind', '_i', '_j'))
+        canonical = (len(rshape) <= 1 and len(oshape) <= 1 and not has_raw
+                     and not needs_indexers and in_arr_idx)
+        if canonical:
+            n_red = rshape[0] if rshape else 1
+            n_out = oshape[0] if oshape else 1
+            ins = [in_args[i] for i in in_arr_idx]
+            outs = [out_args[i] for i in out_arr_idx]
+            sr = [(rs[0] if rs else 0) for rs in rstrides]
+            so_in = [(os_[0] if os_ else 0) for os_ in o_in]
+            so_out = [(os_[0] if os_ else 0) for os_ in o_out]
+            rows_ok = n_red > 1 and all(
+                s == a.dtype.itemsize or s == 0 for s, a in zip(sr, ins)) and all(
+                s % a.dtype.itemsize == 0 for s, a in zip(so_in, ins)) and all(
+                s % a.dtype.itemsize == 0 for s, a in zip(so_out, outs))
+            cols_ok = all(
+                s == a.dtype.itemsize or s == 0 or n_out == 1
+                for s, a in zip(so_in, ins)) and all(
+                s == a.dtype.itemsize or n_out == 1
+                for s, a in zip(so_out, outs)) and all(
+                s % a.dtype.itemsize == 0 for s, a in zip(sr, ins))
+            plan_args = (in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
+                         so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
+                         reduce_type, typedefs, device_id, stream_ptr)
+            if rows_ok:
+                return self._launch_rows(*plan_args)
+            if cols_ok:
+                return self._launch_cols(*plan_args)
+        # generic: views with the reduced axes in front, merged where possible
+        g_in = list(in_args)
+        for k, i in enumerate(in_arr_idx):
+            shape = tuple(rshape) + tuple(oshape)
+            strides = tuple(rstrides[k]) + tuple(o_in[k])
+            g_in[i] = in_args[i]._view(shape, strides)
+        g_out = list(out_args)
+        for k, i in enumerate(out_arr_idx):
+            g_out[i] = out_args[i]._view(tuple(oshape), tuple(o_out[k]))
+        in_shape = tuple(rshape) + tuple(oshape)
+        if not in_arr_idx:
+            in_shape = red_shape + kept_shape
+            oshape = kept_shape
+        return self._launch_generic(
+            g_in, g_out, in_shape, tuple(oshape), internal.prod(rshape) if in_arr_idx
+            else internal.prod(red_shape), map_expr, reduce_expr, post_map_expr,
+            reduce_type, typedefs, device_id, stream_ptr)
+
+    # -- helpers ----------------------------------------------------------------------------
+    def _rargs(self, in_args, out_args, bcast_r=None, bcast_o=None):
+        rargs = []
+        k = 0
+        for idx, (a, p) in enumerate(zip(in_args, self.in_params)):
+            if isinstance(a, ndarray):
+                st = _get_typename(a.dtype)
+                if p.raw:
+                    rargs.append(_cg.RArg(
+                        'raw', p.name, st, is_const=p.is_const, ndim=a.ndim,
+                        c_contiguous=a._c_contiguous, index_32=a._index_32_bits))
+                else:
+                    rargs.append(_cg.RArg(
+                        'in', p.name, st, self._in_var_type(idx, p),
+                        is_const=p.is_const, ndim=a.ndim,
+                        c_contiguous=a._c_contiguous, index_32=a._index_32_bits,
+                        bcast_r=bool(bcast_r and bcast_r[k]),
+                        bcast_o=bool(bcast_o and bcast_o[k])))
+                    k += 1
+            else:
+                rargs.append(_cg.RArg('scalar', p.name, _get_typename(a.descr)))
+        for idx, (a, p) in enumerate(zip(out_args, self.out_params)):
+            st = _get_typename(a.dtype)
+            if p.raw:
+                rargs.append(_cg.RArg(
+                    'raw', p.name, st, is_const=False, ndim=a.ndim,
+                    c_contiguous=a._c_contiguous, index_32=a._index_32_bits))
+            else:
+                rargs.append(_cg.RArg(
+                    'out', p.name, st, self._out_var_type(idx, p), is_const=False,
+                    ndim=a.ndim, c_contiguous=a._c_contiguous,
+                    index_32=a._index_32_bits))
+        return rargs
+
+    def _out_var_type(self, index, param):
+        return param.ctype
+
+    def _compile(self, key, emit, in_args):
+        """Memoised (function, module, code) for a kernel variant."""
+        entry = self._memo.get(key)
+        if entry is None:
+            name, code = emit()
+            preamble, options = self._get_preamble_options()
+            mod = compiler.compile_with_cache(code, options)
+            fn = mod.get_function(name)
+            entry = (fn, mod, code)
+            with self._lock:
+                entry = self._memo.setdefault(key, entry)
+            in_types = tuple(a.dtype.char for a in in_args if isinstance(a, ndarray))
+            if in_types not in self._cached_codes:
+                self._cached_codes[in_types] = code
+        return entry
+
+    def _reduce_type_size(self, reduce_type, mod):
+        size = _known_type_sizes.get(reduce_type)
+        if size is not None:
+            return size
+        if _dryrun.enabled():
+            return 64
+        _, nbytes = mod.get_global_var('_cupy_type_reduce_probe')
+        return nbytes
+
+    @staticmethod
+    def _fast_format(rargs, ic, extra=''):
+        fmt = ['@']
+        for a in rargs:
+            if a.kind in ('in', 'out'):
+                fmt.append('P')
+            elif a.kind == 'raw':
+                fmt.append('P' + 'q' * (1 + 2 * a.ndim))
+            else:
+                fmt.append(_scalar_struct_code(a.store_t))
+        fmt.append(ic * 2)
+        for a in rargs:
+            if a.kind == 'in':
+                fmt.append(ic * 2)
+            elif a.kind == 'out':
+                fmt.append(ic)
+        fmt.append(extra)
+        return ''.join(fmt)
+
+    def _fast_values(self, in_args, out_args, n_out, n_red, so_in, sr, so_out):
+        vals = []
+        for a in in_args:
+            vals.append(a.data.ptr if isinstance(a, ndarray) else a._struct_value())
+        for a in out_args:
+            vals.append(a.data.ptr)
+        vals.extend((n_out, n_red))
+        k = 0
+        for a, p in zip(in_args, self.in_params):
+            if isinstance(a, ndarray) and not p.raw:
+                item = a.dtype.itemsize
+                vals.extend((so_in[k] // item, sr[k] // item))
+                k += 1
+        for k, a in enumerate(out_args):
+            vals.append(so_out[k] // a.dtype.itemsize)
+        return vals
+
+    def _finalize_partials(self, partials, n_split, out_args, out_arr_idx, n_out,
+                           so_out, in_args, reduce_expr, post_map_expr, reduce_type,
+                           typedefs, device_id, stream_ptr):
+        """Second pass: combine ``partials[s][i]`` over s, then POST_MAP."""
+        preamble, _ = self._get_preamble_options()
+        tx = max(1, min(64, internal.clp2(n_out)))
+        rargs = [_cg.RArg('in', '_partial_in', '_type_reduce')]
+        rargs += [r for r in self._rargs(in_args, out_args) if r.kind in ('scalar', 'out')]
+        idx64 = n_split * n_out > _INT32_MAX
+        key = ('final', tuple(r.key() for r in rargs), typedefs, reduce_expr,
+               post_map_expr, reduce_type, tx, idx64, device_id)
+
+        def emit():
+            name = self.name + '_combine'
+            return name, _cg.emit_cols(
+                name, rargs, self.identity, '_partial_in', reduce_expr,
+                post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=1,
+                idx64=idx64, partial_in=True)
+        fn, _, _ = self._compile(key, emit, in_args)
+        ic = 'q' if idx64 else 'i'
+        fmt = ['@P']
+        vals = [partials.ptr]
+        for a, p in zip(in_args, self.in_params):
+            if not isinstance(a, ndarray):
+                fmt.append(_scalar_struct_code(_get_typename(a.descr)))
+                vals.append(a._struct_value())
+        for a in out_args:
+            fmt.append('P')
+            vals.append(a.data.ptr)
+        fmt.append(ic * 4)
+        vals.extend((n_out, n_split, 1, n_out))
+        for k, a in enumerate(out_args):
+            fmt.append(ic)
+            vals.append(so_out[k] // a.dtype.itemsize)
+        blob = struct.pack(''.join(fmt), *vals)
+        grid = (n_out + tx - 1) // tx
+        fn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+
+    # -- rows ---------------------------------------------------------------------------------
+    def _launch_rows(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
+                     so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
+                     reduce_type, typedefs, device_id, stream_ptr):
+        preamble, _ = self._get_preamble_options()
+        ins = [in_args[i] for i in in_arr_idx]
+        cus = _device.get_compute_units(device_id)
+        vec = _max_vector_width([a.dtype.itemsize for a in ins])
+        while vec > 1:
+            ok = True
+            for a, s_o, s_r in zip(ins, so_in, sr):
+                if s_r == 0:
+                    continue
+                nb = min(16, vec * a.dtype.itemsize)
+                if not _aligned(a.data.ptr, nb) or (n_out > 1 and s_o % nb):
+                    ok = False
+            if ok and n_red >= vec:
+                break
+            vec //= 2
+        bcast_r = [s == 0 for s in sr]
+        max_item = max(a.dtype.itemsize for a in ins)
+        lanes_needed = (n_red + vec - 1) // vec
+        # geometry
+        if n_red * max_item >= ROWS_BLOCK_MODE_BYTES:
+            group = _cg.BLOCK
+        else:
+            group = max(1, min(64, internal.clp2(lanes_needed)))
+        n_split = 1
+        chunk = n_red
+        if group == _cg.BLOCK and n_out < cus * MIN_BLOCKS_PER_CU:
+            trip = _cg.BLOCK * vec
+            want = (cus * TARGET_BLOCKS_PER_CU + n_out - 1) // n_out
+            most = max(1, n_red // (trip * 4))
+            n_split = max(1, min(want, most, 65535))
+            if n_split > 1:
+                chunk = (n_red + n_split - 1) // n_split
+                chunk = (chunk + trip - 1) // trip * trip
+                n_split = (n_red + chunk - 1) // chunk
+        partial = n_split > 1
+        span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
+                   + [abs(s) * n_out for s in so_out] + [n_red + chunk])
+        idx64 = span > _INT32_MAX - (1 << 24)
+        rargs = self._rargs(in_args, out_args, bcast_r=bcast_r)
+        key = ('rows', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
+               post_map_expr, reduce_type, group, vec, idx64, partial, device_id)
+
+        def emit():
+            return self.name, _cg.emit_rows(
+                self.name, rargs, self.identity, map_expr, reduce_expr,
+                post_map_expr, reduce_type, typedefs, preamble, group=group,
+                vec=vec, idx64=idx64, partial_out=partial,
+                stream_hint=ROWS_STREAM_HINT)
+        fn, mod, _ = self._compile(key, emit, in_args)
+        ic = 'q' if idx64 else 'i'
+        vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
+        if group == _cg.BLOCK:
+            gx = min(n_out, 0x7fffffff)
+        else:
+            rows_per_block = _cg.BLOCK // group
+            gx = min((n_out + rows_per_block - 1) // rows_per_block, cus * 64)
+        if partial:
+            rsize = self._reduce_type_size(reduce_type, mod)
+            partials = _memory.alloc(rsize * n_split * n_out)
+            vals.extend((partials.ptr, chunk))
+            blob = struct.pack(self._fast_format(rargs, ic, 'P' + ic), *vals)
+            fn.launch_packed((gx, n_split, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            self._finalize_partials(
+                partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
+                reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
+                stream_ptr)
+        else:
+            blob = struct.pack(self._fast_format(rargs, ic), *vals)
+            fn.launch_packed((gx, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+
+    # -- cols ---------------------------------------------------------------------------------
+    def _launch_cols(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
+                     so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
+                     reduce_type, typedefs, device_id, stream_ptr):
+        preamble, _ = self._get_preamble_options()
+        ins = [in_args[i] for i in in_arr_idx]
+        cus = _device.get_compute_units(device_id)
+        vec = _max_vector_width([a.dtype.itemsize for a in ins])
+        bcast_o = [(s == 0 and n_out > 1) for s in so_in]
+        while vec > 1:
+            ok = n_out >= vec
+            for a, s_o, s_r in zip(ins, so_in, sr):
+                if s_o == 0 and n_out > 1:
+                    continue
+                nb = min(16, vec * a.dtype.itemsize)
+                if not _aligned(a.data.ptr, nb) or (n_red > 1 and s_r % nb):
+                    ok = False
+            if ok:
+                break
+            vec //= 2
+        tx = max(1, min(64, internal.clp2((n_out + vec - 1) // vec)))
+        ty = _cg.BLOCK // tx
+        gx = (n_out + tx * vec - 1) // (tx * vec)
+        want = (cus * TARGET_BLOCKS_PER_CU + gx - 1) // gx
+        most = max(1, n_red // (ty * 8))
+        n_split = max(1, min(want, most, 65535))
+        partial = n_split > 1
+        span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
+                   + [abs(s) * n_out for s in so_out] + [n_red + n_split * ty])
+        idx64 = span > _INT32_MAX - (1 << 24)
+        rargs = self._rargs(in_args, out_args, bcast_o=bcast_o)
+        key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
+               post_map_expr, reduce_type, tx, vec, idx64, partial, device_id)
+
+        def emit():
+            return self.name, _cg.emit_cols(
+                self.name, rargs, self.identity, map_expr, reduce_expr,
+                post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
+                idx64=idx64, partial_out=partial, stream_hint=COLS_STREAM_HINT)
+        fn, mod, _ = self._compile(key, emit, in_args)
+        ic = 'q' if idx64 else 'i'
+        vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
+        if partial:
+            rsize = self._reduce_type_size(reduce_type, mod)
+            partials = _memory.alloc(rsize * n_split * n_out)
+            vals.append(partials.ptr)
+            blob = struct.pack(self._fast_format(rargs, ic, 'P'), *vals)
+            fn.launch_packed((gx, n_split, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            self._finalize_partials(
+                partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
+                reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
+                stream_ptr)
+        else:
+            blob = struct.pack(self._fast_format(rargs, ic), *vals)
+            fn.launch_packed((gx, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+
+    # -- generic ------------------------------------------------------------------------------
+    def _launch_generic(self, in_args, out_args, in_shape, out_shape, n_red,
+                        map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                        device_id, stream_ptr):
+        preamble, _ = self._get_preamble_options()
+        cus = _device.get_compute_units(device_id)
+        n_out = internal.prod(out_shape)
+        in_ind = _carray.Indexer(in_shape)
+        out_ind = _carray.Indexer(out_shape)
+        # threads across the output index: as many as the innermost kept axis
+        # is contiguous for, but no more than needed to leave every thread a
+        # few elements of the reduce axis
+        contiguous = 1
+        nd_in = len(in_shape)
+        nd_out = len(out_shape)
+        for a, p in zip(in_args, self.in_params):
+            if not isinstance(a, ndarray) or p.raw:
+                continue
+            run = 1
+            for j in range(nd_out):
+                if a._strides[nd_in - j - 1] != run * a.dtype.itemsize:
+                    break
+                run *= out_shape[nd_out - j - 1]
+            contiguous = max(contiguous, run)
+        tx = max(min(contiguous, 64), _cg.BLOCK // max(1, n_red))
+        tx = max(1, min(64, internal.flp2(tx), internal.clp2(n_out)))
+        ty = _cg.BLOCK // tx
+        gx = min((n_out + tx - 1) // tx, 0x7fffffff)
+        want = (cus * TARGET_BLOCKS_PER_CU + gx - 1) // gx
+        most = max(1, n_red // (ty * 8))
+        n_split = max(1, min(want, most, 65535))
+        partial = n_split > 1
+        rargs = self._rargs(in_args, out_args)
+        key = ('generic', tuple(r.key() for r in rargs), typedefs, map_expr,
+               reduce_expr, post_map_expr, reduce_type, tx, in_ind.ndim,
+               out_ind.ndim, in_ind._index_32_bits, out_ind._index_32_bits,
+               partial, device_id)
+
+        def emit():
+            return self.name, _cg.emit_generic(
+                self.name, rargs, self.identity, map_expr, reduce_expr,
+                post_map_expr, reduce_type, typedefs, preamble, tx=tx,
+                in_ndim=in_ind.ndim, out_ndim=out_ind.ndim,
+                in_index_32=in_ind._index_32_bits,
+                out_index_32=out_ind._index_32_bits, partial_out=partial)
+        fn, mod, _ = self._compile(key, emit, in_args)
+        fmt = ['@']
+        vals = []
+        for a in list(in_args) + list(out_args):
+            if isinstance(a, ndarray):
+                fmt.append('P' + 'q' * (1 + 2 * a.ndim))
+                vals.append(a.data.ptr)
+                vals.append(a.size)
+                vals.extend(a._shape)
+                vals.extend(a._strides)
+            else:
+                fmt.append(_scalar_struct_code(_get_typename(a.descr)))
+                vals.append(a._struct_value())
+        for ind in (in_ind, out_ind):
+            fmt.append('q' * (1 + 2 * ind.ndim))
+            vals.append(ind.size)
+            vals.extend(ind.shape)
+            vals.extend((0,) * ind.ndim)
+        if not partial:
+            blob = struct.pack(''.join(fmt), *vals)
+            fn.launch_packed((gx, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            return
+        rsize = self._reduce_type_size(reduce_type, mod)
+        partials = _memory.alloc(rsize * n_split * n_out)
+        fmt.append('P')
+        vals.append(partials.ptr)
+        blob = struct.pack(''.join(fmt), *vals)
+        fn.launch_packed((gx, n_split, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+        # second pass through the strided output views
+        frargs = [r for r in rargs if r.kind in ('out', 'raw', 'scalar')]
+        fkey = ('generic_final', tuple(r.key() for r in frargs), typedefs,
+                reduce_expr, post_map_expr, reduce_type, out_ind.ndim,
+                out_ind._index_32_bits, device_id)
+
+        def emit_final():
+            name = self.name + '_combine'
+            return name, _cg.emit_finalize_generic(
+                name, frargs, self.identity, reduce_expr, post_map_expr,
+                reduce_type, typedefs, preamble, out_ndim=out_ind.ndim,
+                out_index_32=out_ind._index_32_bits)
+        ffn, _, _ = self._compile(fkey, emit_final, in_args)
+        fmt = ['@']
+        vals = []
+        # parameter order of emit_finalize_generic: out / raw / scalar in the
+        # order they appear in `frargs`
+        objs = []
+        for a, p in zip(in_args, self.in_params):
+            if isinstance(a, ndarray):
+                if p.raw:
+                    objs.append(a)
+            else:
+                objs.append(a)
+        objs.extend(out_args)
+        for a in objs:
+            if isinstance(a, ndarray):
+                fmt.append('P' + 'q' * (1 + 2 * a.ndim))
+                vals.append(a.data.ptr)
+                vals.append(a.size)
+                vals.extend(a._shape)
+                vals.extend(a._strides)
+            else:
+                fmt.append(_scalar_struct_code(_get_typename(a.descr)))
+                vals.append(a._struct_value())
+        fmt.append('q' * (1 + 2 * out_ind.ndim))
+        vals.append(out_ind.size)
+        vals.extend(out_ind.shape)
+        vals.extend((0,) * out_ind.ndim)
+        fmt.append('Pi')
+        vals.extend((partials.ptr, n_split))
+        blob = struct.pack(''.join(fmt), *vals)
+        grid = max(1, min((n_out + _cg.BLOCK - 1) // _cg.BLOCK, cus * 8))
+        ffn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+
+    # -- debugging aids ------------------------------------------------------------------------
+    @property
+    def cached_codes(self):
+        """dict: input dtype characters -> generated source."""
+        if len(self._cached_codes) == 0:
+            warnings.warn(
+                'No codes are cached because compilation is deferred until '
+                'the first function call.')
+        return dict(self._cached_codes.items())
+
+    @property
+    def cached_code(self):
+        codes = self._cached_codes
+        if len(codes) > 1:
+            warnings.warn(
+                'The input types of the kernel could not be inferred. '
+                'Please use `.cached_codes` instead.')
+        return next(iter(codes.values()))
+
+
+# ---------------------------------------------------------------------------------
+# create_reduction_func
+# ---------------------------------------------------------------------------------
+
+def create_reduction_func(name, ops, routine=None, identity=None, preamble='',
+                          sort_reduce_axis=True):
+    """Builds a one-input reduction from loop signatures and a routine
+    ``(map_expr, reduce_expr, post_map_expr, reduce_type)``."""
+    ops = _kernel._Ops.from_tuples(ops, routine)
+    return _SimpleReductionKernel(name, ops, identity, preamble, sort_reduce_axis)
+
+
+class _SimpleReductionKernel(_AbstractReductionKernel):
+
+    def __init__(self, name, ops, identity, preamble, sort_reduce_axis=True):
+        super().__init__(name, '' if identity is None else str(identity),
+                         'T in0', 'T out0')
+        self._ops = ops
+        self.preamble = preamble
+        self.nin = 1
+        self.nout = 1
+        self._routine_cache = {}
+        self._sort_reduce_axis = sort_reduce_axis
+
+    def __call__(self, a, axis=None, dtype=None, out=None, keepdims=False):
+        if hasattr(a, '__cupy_override_reduction_kernel__'):
+            return a.__cupy_override_reduction_kernel__(
+                self, axis, dtype, out, keepdims)
+        arr = _convert_from_cupy_like(a, error="Argument 'a'")
+        dev_id = _device.get_device_id()
+        _check_peer_access(arr, dev_id)
+        if out is None:
+            out_args = []
+        else:
+            if not isinstance(out, ndarray):
+                raise TypeError("Argument 'out' has incorrect type")
+            _check_peer_access(out, dev_id)
+            out_args = [out]
+        return self._call([arr], out_args, arr._shape, axis, dtype, keepdims,
+                          True, dev_id, None, self._sort_reduce_axis)
+
+    def _get_expressions_and_types(self, in_args, out_args, dtype):
+        op = self._ops.guess_routine(
+            self.name, self._routine_cache, in_args, dtype, self._ops)
+        map_expr, reduce_expr, post_map_expr, reduce_type = op.routine
+        if reduce_type is None:
+            reduce_type = _get_typename(op.out_types[0])
+        if out_args:
+            out_type = out_args[0].dtype.type
+        else:
+            out_type = op.out_types[0]
+        type_pairs = (('type_in0_raw', in_args[0].dtype.type),
+                      ('type_out0_raw', out_type))
+        return (map_expr, reduce_expr, post_map_expr, op.in_types, op.out_types,
+                reduce_type, type_pairs)
+
+    def _get_out_args(self, out_args, out_types, out_shape):
+        return _get_out_args_from_optionals(
+            ndarray, out_args, out_types, out_shape, 'unsafe', None)
+
+    def _get_preamble_options(self):
+        return self.preamble, ()
+
+    def _in_var_type(self, index, param):
+        return 'type_in0_raw'
+
+    def _out_var_type(self, index, param):
+        return 'type_out0_raw'
+
+
+# ---------------------------------------------------------------------------------
+# ReductionKernel
+# ---------------------------------------------------------------------------------
+
+class ReductionKernel(_AbstractReductionKernel):
+    """User-defined reduction kernel.
+
+    Args:
+        in_params (str): Input argument list.
+        out_params (str): Output argument list.
+        map_expr (str): Expression applied to each input element (or tuple of
+            elements of the broadcast inputs).
+        reduce_expr (str): Combines ``a`` and ``b``.
+        post_map_expr (str): Statement storing the reduced value ``a`` into the
+            output parameter.
+        identity (str): Initial value of the reduction.
+        name (str): Kernel name.
+        reduce_type (str): Type of ``a`` / ``b`` (default: first output type).
+        reduce_dims (bool): Merge contiguous axes before launching.
+        preamble (str): Code inserted before the kernel.
+        options (tuple of str): Extra hiprtc options.
+    """
+
+    def __init__(self, in_params, out_params, map_expr, reduce_expr,
+                 post_map_expr, identity, name='reduce_kernel', reduce_type=None,
+                 reduce_dims=True, preamble='', options=()):
+        if not compiler.is_valid_kernel_name(name):
+            raise ValueError('Invalid kernel name: "%s"' % name)
+        super().__init__(name, '' if identity is None else str(identity),
+                         in_params, out_params)
+        self.nin = len(self.in_params)
+        self.nout = len(self.out_params)
+        self.nargs = self.nin + self.nout
+        self.reduce_expr = reduce_expr
+        self.map_expr = map_expr
+        self.post_map_expr = post_map_expr
+        self.options = tuple(options)
+        self.reduce_dims = reduce_dims
+        if reduce_type is None:
+            self.reduce_type = self.out_params[0].ctype
+        else:
+            self.reduce_type = reduce_type
+        self.preamble = preamble
+
+    def __call__(self, *args, **kwargs):
+        """Compiles (if needed) and launches the reduction.
+
+        Args:
+            args: Inputs, optionally followed by the outputs.
+            out (cupy.ndarray): Output array (not together with a positional one).
+            axis (int or tuple of ints): Axes to reduce (default: all).
+            keepdims (bool): Keep reduced axes with length one.
+            stream: Stream to launch on.
+        """
+        out = kwargs.pop('out', None)
+        axis = kwargs.pop('axis', None)
+        keepdims = kwargs.pop('keepdims', False)
+        stream = kwargs.pop('stream', None)
+        if kwargs:
+            raise TypeError('Wrong arguments %s' % kwargs)
+        n_args = len(args)
+        if n_args != self.nin and n_args != self.nargs:
+            raise TypeError('Wrong number of arguments for %s' % self.name)
+        out_args = list(args[self.nin:])
+        if out is not None:
+            if self.nout != 1:
+                raise NotImplementedError('')
+            if len(out_args) != 0:
+                raise ValueError("cannot specify 'out' as both "
+                                 "a positional and keyword argument")
+            out_args = [out]
+        dev_id = _device.get_device_id()
+        in_args = _preprocess_args(dev_id, args[:self.nin])
+        out_args = _preprocess_args(dev_id, out_args)
+        in_args, broad_shape = _broadcast(in_args, self.in_params, False)
+        return self._call(in_args, out_args, broad_shape, axis, None, keepdims,
+                          self.reduce_dims, dev_id, stream, True)
+
+    def _get_expressions_and_types(self, in_args, out_args, dtype):
+        in_ndarray_types = tuple(
+            a.dtype.type if isinstance(a, ndarray) else None for a in in_args)
+        out_ndarray_types = tuple(
+            a.dtype.type if isinstance(a, ndarray) else None for a in out_args)
+        in_types, out_types, type_map = _decide_params_type(
+            self.in_params, self.out_params, in_ndarray_types, out_ndarray_types)
+        return (self.map_expr, self.reduce_expr, self.post_map_expr, in_types,
+                out_types, self.reduce_type, type_map._pairs)
+
+    def _get_out_args(self, out_args, out_types, out_shape):
+        return _get_out_args_with_params(
+            out_args, out_types, out_shape, self.out_params, False)
+
+    def _get_preamble_options(self):
+        return self.preamble, self.options
+
+    def _in_var_type(self, index, param):
+        return param.ctype

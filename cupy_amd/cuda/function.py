@@ -10,6 +10,7 @@ import numpy
 
 from cupy_amd import _dryrun
 from cupy_amd import _rt
+from cupy_amd.cuda import _codeobj
 from cupy_amd.cuda import stream as _stream
 
 # hipFunction_attribute values
@@ -60,6 +61,15 @@ class Module:
     def __init__(self):
         self.ptr = 0
         self.code = None
+        self._metadata = None
+
+    @property
+    def metadata(self):
+        """Per-kernel metadata of the code object (argument layout, register
+        and LDS use)."""
+        if self._metadata is None:
+            self._metadata = _codeobj.kernel_metadata(self.code)
+        return self._metadata
 
     def __del__(self):
         ptr, self.ptr = getattr(self, 'ptr', 0), 0
@@ -98,10 +108,15 @@ class Function:
         self.module = module
         self.name = name
         self.ptr = 0
+        meta = module.metadata.get(name)
+        if meta is None:
+            raise _rt.HIPError(500, 'no kernel named %r in the module' % name)
+        self.meta = meta
+        # size of the explicit arguments, rounded as the packer may leave the
+        # tail padding of the last argument off
+        self._arg_size = meta['explicit_size']
+        self._arg_min = (meta['args'][-1][0] + 1) if meta['args'] else 0
         if _dryrun.enabled():
-            if ('\x00' + name + '\x00').encode() not in b'\x00' + module.code:
-                if name.encode() not in module.code:
-                    raise _rt.HIPError(500, 'no kernel named %r' % name)
             return
         p = ctypes.c_void_p()
         _rt.check(_rt.lib.rt_module_get_function(
@@ -141,6 +156,13 @@ class Function:
             stream_ptr = _stream.get_current_stream_ptr()
         gx, gy, gz = grid
         bx, by, bz = block
+        n = len(arg_block)
+        if n > self._arg_size or n < self._arg_min:
+            raise ValueError(
+                'kernel %s expects an argument block of %d bytes, got %d'
+                % (self.name, self._arg_size, n))
+        if n < self._arg_size:
+            arg_block = bytes(arg_block) + b'\0' * (self._arg_size - n)
         if _dryrun.enabled():
             _dryrun.record_launch(self.name, grid, block, shared_mem, bytes(arg_block))
             return
