@@ -1,0 +1,357 @@
+"""Pool behaviour with a fake allocator that hands out made-up addresses (the
+way the reference tests its pool, tests/cupy_tests/cuda_tests/test_memory.py:
+20-36,291-648): rounding, best fit, split, merge, per-stream arenas,
+free_all_blocks, limits and the byte counters.  No device memory is touched."""
+import threading
+
+import pytest
+
+from cupy_amd.cuda import memory
+from cupy_amd.cuda import stream as stream_module
+
+
+class MockMemory(memory.BaseMemory):
+    cur_ptr = 1 << 20
+
+    def __init__(self, size):
+        self.ptr = MockMemory.cur_ptr
+        MockMemory.cur_ptr += size + (1 << 16)
+        self.size = size
+        self.device_id = 0
+
+
+def mock_alloc(size):
+    return memory.MemoryPointer(MockMemory(size), 0)
+
+
+class FakeStream:
+    def __init__(self, ptr):
+        self.ptr = ptr
+
+    def __enter__(self):
+        self._prev = (getattr(stream_module._tls, 'stream', None),
+                      getattr(stream_module._tls, 'ptr', 0))
+        stream_module._tls.stream = self
+        stream_module._tls.ptr = self.ptr
+        return self
+
+    def __exit__(self, *exc):
+        stream_module._tls.stream, stream_module._tls.ptr = self._prev
+
+
+@pytest.fixture
+def pool(monkeypatch):
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+    return memory.SingleDeviceMemoryPool(allocator=mock_alloc)
+
+
+unit = memory._allocation_unit_size
+stream = FakeStream(0x1234)
+null_stream = FakeStream(0)
+
+
+def test_round_size():
+    assert memory._round_size(unit - 1) == unit
+    assert memory._round_size(unit) == unit
+    assert memory._round_size(unit + 1) == unit * 2
+
+
+def test_alloc_distinct(pool):
+    p1 = pool.malloc(unit * 4)
+    p2 = pool.malloc(unit * 4)
+    p3 = pool.malloc(unit * 8)
+    assert len({p1.ptr, p2.ptr, p3.ptr}) == 3
+
+
+def test_alloc_split(pool):
+    p = pool.malloc(unit * 4)
+    ptr = p.ptr
+    del p
+    head = pool.malloc(unit * 2)
+    tail = pool.malloc(unit * 2)
+    assert ptr == head.ptr
+    assert ptr + unit * 2 == tail.ptr
+
+
+def test_alloc_limit(pool):
+    pool.set_limit(size=unit * 6)
+    p1 = pool.malloc(unit * 5)
+    p2 = pool.malloc(unit * 1)
+    with pytest.raises(memory.OutOfMemoryError):
+        pool.malloc(unit)
+    pool.set_limit(size=unit * 7)
+    p3 = pool.malloc(unit)
+    del p1, p2, p3
+
+
+def test_alloc_limit_fragmented(pool):
+    pool.set_limit(size=unit * 6)
+    p1 = pool.malloc(unit * 5)
+    del p1
+    p2 = pool.malloc(unit * 6)    # the cached 5-unit block is released first
+    del p2
+
+
+def test_free_reuses_block(pool):
+    p1 = pool.malloc(unit * 4)
+    ptr1 = p1.ptr
+    del p1
+    p2 = pool.malloc(unit * 4)
+    assert ptr1 == p2.ptr
+
+
+def test_free_is_per_stream(pool):
+    p1 = pool.malloc(unit * 4)
+    ptr1 = p1.ptr
+    del p1
+    with stream:
+        p2 = pool.malloc(unit * 4)
+    assert ptr1 != p2.ptr
+
+
+def test_free_merge_both_orders(pool):
+    p = pool.malloc(unit * 4)
+    ptr = p.ptr
+    del p
+    head = pool.malloc(unit * 2)
+    tail = pool.malloc(unit * 2)
+    assert ptr == head.ptr
+    del tail
+    del head
+    p = pool.malloc(unit * 4)
+    assert ptr == p.ptr
+    del p
+    head = pool.malloc(unit * 2)
+    tail = pool.malloc(unit * 2)
+    assert ptr == head.ptr
+    del head
+    del tail
+    p = pool.malloc(unit * 4)
+    assert ptr == p.ptr
+
+
+def test_free_different_size(pool):
+    p1 = pool.malloc(unit * 4)
+    ptr1 = p1.ptr
+    del p1
+    p2 = pool.malloc(unit * 8)
+    assert ptr1 != p2.ptr
+
+
+def test_best_fit_takes_smallest_block_that_fits(pool):
+    big = pool.malloc(unit * 8)
+    small = pool.malloc(unit * 3)
+    big_ptr, small_ptr = big.ptr, small.ptr
+    del big, small
+    p = pool.malloc(unit * 2)
+    assert p.ptr == small_ptr
+    q = pool.malloc(unit * 5)
+    assert q.ptr == big_ptr
+
+
+def test_free_all_blocks(pool):
+    p1 = pool.malloc(unit * 4)
+    ptr1 = p1.ptr
+    del p1
+    pool.free_all_blocks()
+    p2 = pool.malloc(unit * 4)
+    assert ptr1 != p2.ptr
+
+
+def test_free_all_blocks_keeps_split_blocks(pool):
+    p = pool.malloc(unit * 4)
+    del p
+    head = pool.malloc(unit * 2)
+    tail = pool.malloc(unit * 2)
+    tailptr = tail.ptr
+    del tail
+    pool.free_all_blocks()
+    p = pool.malloc(unit * 2)
+    assert tailptr == p.ptr
+    del head
+
+
+def test_free_all_blocks_of_one_stream(pool):
+    p1 = pool.malloc(unit * 4)
+    ptr1 = p1.ptr
+    del p1
+    with stream:
+        p2 = pool.malloc(unit * 4)
+        ptr2 = p2.ptr
+        del p2
+    pool.free_all_blocks(stream=null_stream)
+    p3 = pool.malloc(unit * 4)
+    assert ptr1 != p3.ptr and ptr2 != p3.ptr
+    with stream:
+        p4 = pool.malloc(unit * 4)
+        assert ptr1 != p4.ptr and ptr2 == p4.ptr
+
+
+def test_free_all_blocks_all_streams(pool):
+    p1 = pool.malloc(unit * 4)
+    ptr1 = p1.ptr
+    del p1
+    with stream:
+        p2 = pool.malloc(unit * 4)
+        ptr2 = p2.ptr
+        del p2
+    pool.free_all_blocks()
+    p3 = pool.malloc(unit * 4)
+    assert ptr1 != p3.ptr and ptr2 != p3.ptr
+    with stream:
+        p4 = pool.malloc(unit * 4)
+        assert ptr1 != p4.ptr and ptr2 != p4.ptr
+
+
+def test_free_all_free_is_deprecated(pool):
+    p1 = pool.malloc(unit * 4)
+    del p1
+    with pytest.warns(DeprecationWarning):
+        pool.free_all_free()
+    assert pool.n_free_blocks() == 0
+
+
+def test_byte_counters(pool):
+    p1 = pool.malloc(unit * 2)
+    assert (pool.used_bytes(), pool.free_bytes(), pool.total_bytes()) == (unit * 2, 0, unit * 2)
+    p2 = pool.malloc(unit * 4)
+    assert (pool.used_bytes(), pool.free_bytes(), pool.total_bytes()) == (unit * 6, 0, unit * 6)
+    del p2
+    assert (pool.used_bytes(), pool.free_bytes(), pool.total_bytes()) == (unit * 2, unit * 4, unit * 6)
+    del p1
+    assert (pool.used_bytes(), pool.free_bytes(), pool.total_bytes()) == (0, unit * 6, unit * 6)
+    p3 = pool.malloc(unit * 1)
+    assert (pool.used_bytes(), pool.free_bytes(), pool.total_bytes()) == (unit, unit * 5, unit * 6)
+    assert pool.used_bytes() + pool.free_bytes() == pool.total_bytes()
+    del p3
+    pool.free_all_blocks()
+    assert pool.total_bytes() == 0
+
+
+def test_counters_across_streams(pool):
+    p1 = pool.malloc(unit * 4)
+    del p1
+    with stream:
+        p2 = pool.malloc(unit * 2)
+    assert pool.used_bytes() == unit * 2
+    assert pool.free_bytes() == unit * 4
+    assert pool.total_bytes() == unit * 6
+    del p2
+
+
+def test_limit_api(pool, monkeypatch):
+    assert pool.get_limit() == 0
+    pool.set_limit(size=1024)
+    assert pool.get_limit() == 1024
+    pool.set_limit(size=2 ** 33)
+    assert pool.get_limit() == 2 ** 33
+    pool.set_limit(size=0)
+    assert pool.get_limit() == 0
+    with pytest.raises(ValueError):
+        pool.set_limit(size=-1)
+    with pytest.raises(ValueError):
+        pool.set_limit(size=1, fraction=0.5)
+    total = 288 << 30
+    monkeypatch.setattr(memory._device.Device, 'mem_info', property(lambda self: (total, total)))
+    pool.set_limit(fraction=0)
+    assert pool.get_limit() == 0
+    pool.set_limit(fraction=0.5)
+    assert pool.get_limit() == total * 0.5
+    pool.set_limit(fraction=1.0)
+    assert pool.get_limit() == total
+    for bad in (-1, 1.1):
+        with pytest.raises(ValueError):
+            pool.set_limit(fraction=bad)
+
+
+def test_parse_limit_string(golden):
+    for text, size, fraction in golden['limit_strings']:
+        got = memory._parse_limit_string(text)
+        assert got['size'] == size and got['fraction'] == fraction
+
+
+def test_zero_size_and_double_free(pool):
+    mem = pool.malloc(0).mem
+    assert isinstance(mem, memory.Memory) and not isinstance(mem, memory.PooledMemory)
+    mem = pool.malloc(1).mem
+    assert isinstance(mem, memory.PooledMemory)
+    assert pool.n_free_blocks() == 0
+    mem.free()
+    mem.free()
+    assert pool.n_free_blocks() == 1
+    pool.free_all_blocks()
+    assert pool.n_free_blocks() == 0
+
+
+def test_out_of_memory_error_message():
+    e = memory.OutOfMemoryError(1024, 4096, 8192)
+    assert '1,024' in str(e) and '8,192' in str(e)
+    import pickle
+    assert str(pickle.loads(pickle.dumps(e))) == str(e)
+
+
+def test_allocator_registry():
+    calls = []
+
+    def my_alloc(size):
+        calls.append(size)
+        return mock_alloc(size)
+
+    old = memory.get_allocator()
+    try:
+        memory.set_allocator(my_alloc)
+        memory.alloc(100)
+        assert calls == [100]
+        with memory.using_allocator(mock_alloc):
+            memory.alloc(50)
+            assert calls == [100]
+            with pytest.raises(ValueError):
+                memory.set_allocator(my_alloc)
+            with memory.using_allocator(my_alloc):
+                memory.alloc(7)
+            assert calls == [100, 7]
+            assert memory.get_allocator() is mock_alloc
+        assert memory.get_allocator() is my_alloc
+    finally:
+        memory.set_allocator(old)
+
+
+def test_using_allocator_is_thread_local():
+    seen = {}
+
+    def worker():
+        seen['other'] = memory.get_allocator()
+
+    with memory.using_allocator(mock_alloc):
+        t = threading.Thread(target=worker)
+        t.start()
+        t.join()
+        seen['this'] = memory.get_allocator()
+    assert seen['this'] is mock_alloc
+    assert seen['other'] is not mock_alloc
+
+
+def test_threads_hammering_one_pool(pool):
+    errors = []
+
+    def worker(seed):
+        import random
+        rnd = random.Random(seed)
+        held = []
+        try:
+            for _ in range(300):
+                if held and rnd.random() < 0.5:
+                    held.pop(rnd.randrange(len(held)))
+                else:
+                    held.append(pool.malloc(unit * rnd.randint(1, 8)))
+        except Exception as e:       # pragma: no cover
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors
+    assert pool.used_bytes() == 0
+    assert pool.used_bytes() + pool.free_bytes() == pool.total_bytes()
