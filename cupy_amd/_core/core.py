@@ -879,21 +879,19 @@ def array(obj, dtype=None, copy=True, order='K', subok=False, ndmin=0):
         else:
             out = src.astype(dtype)
     else:
-        host = numpy.array(obj, dtype=dtype, copy=None, order='C'
-                           if order in ('K', 'A', 'C', 'k', 'a', 'c', None) else 'F')
-        if host.dtype.char not in _dtype.SUPPORTED_CHARS:
+        host = numpy.asarray(obj, dtype=dtype)
+        if host.dtype.char not in _dtype.SUPPORTED_CHARS or not host.dtype.isnative:
             raise ValueError('Unsupported dtype %s' % host.dtype)
-        f_order = host.ndim > 1 and host.flags.f_contiguous and not host.flags.c_contiguous
-        if f_order:
-            out = ndarray._new_contiguous(host.shape, host.dtype, c_order=False)
-            if out.size:
-                buf = numpy.asfortranarray(host)
-                out.data.copy_from_host(buf.ctypes.data, out.nbytes)
-        else:
-            host = numpy.ascontiguousarray(host)
-            out = ndarray._new_contiguous(host.shape, host.dtype)
-            if out.size:
-                out.set(host)
+        keep_f = (order in ('K', 'A', 'F', 'k', 'a', 'f') and host.ndim > 1
+                  and host.flags.f_contiguous and not host.flags.c_contiguous) \
+            or (order in ('F', 'f') and host.ndim > 1)
+        out = ndarray._new_contiguous(host.shape, host.dtype, c_order=not keep_f)
+        if out.size:
+            # the bytes of an F-ordered array are those of its C-ordered transpose
+            buf = numpy.require(host.T if keep_f else host, requirements='C')
+            # synchronous copy: the data is on the device when it returns,
+            # whichever stream uses it next
+            out.data.copy_from_host(buf.ctypes.data, out.nbytes)
     if out.ndim < ndmin:
         out = out.reshape((1,) * (ndmin - out.ndim) + out._shape)
     return out

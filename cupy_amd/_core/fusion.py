@@ -9,6 +9,7 @@ pre-map function, so the fused function runs on the same emitters (vectorised
 loads, wave64 reductions) as hand-written kernels.
 """
 import functools
+import re
 
 import numpy
 
@@ -614,7 +615,12 @@ class Fusion:
 
     def __init__(self, func, name=None):
         self.func = func
-        self.name = name or func.__name__
+        name = name or getattr(func, '__name__', 'fused')
+        # '<lambda>' and the like are not C identifiers
+        name = re.sub(r'[^a-zA-Z0-9_]', '_', name)
+        if not name or name[0].isdigit():
+            name = '_' + name
+        self.name = name
         self._memo = {}
 
     def __repr__(self):

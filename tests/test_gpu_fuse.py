@@ -1,0 +1,191 @@
+"""cupy.fuse on the GPU.  Each fused function is evaluated four ways -- NumPy,
+eager on the device, the fused Python function on NumPy arrays, the fused
+kernel -- and all must agree (the reference's protocol,
+tests/cupy_tests/core_tests/fusion_tests/fusion_utils.py:14-148, with the
+tolerance of this task instead of its 3e-3)."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from helpers import assert_exact, shaped_random
+from oracle import numpy_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def four_way(func, host_args, exact=True, rtol=1e-5):
+    dev_args = [cp.asarray(a) if isinstance(a, np.ndarray) else a for a in host_args]
+
+    def run(xp, fused, args):
+        f = cp.fuse(func(xp)) if fused else func(xp)
+        return f(*args)
+
+    r_np = run(np, False, host_args)
+    r_eager = run(cp, False, dev_args)
+    r_fused_np = run(np, True, host_args)
+    r_fused = run(cp, True, dev_args)
+    for r in (r_eager, r_fused):
+        got = r.get()
+        assert got.dtype == np.asarray(r_np).dtype, (got.dtype, np.asarray(r_np).dtype)
+        if exact:
+            assert_exact(got, np.asarray(r_np))
+        else:
+            assert np.allclose(got, r_np, rtol=rtol, atol=rtol)
+    assert np.array_equal(np.asarray(r_fused_np), np.asarray(r_np), equal_nan=True)
+
+
+def test_elementwise_chain():
+    x = shaped_random((50, 30), 'float32', 1)
+    y = shaped_random((50, 30), 'float32', 2)
+    four_way(lambda xp: lambda a, b: (a - b) * (a - b) + a, [x, y])
+    four_way(lambda xp: lambda a, b: xp.sqrt(xp.absolute(a)) + b * 2, [x, y])
+    four_way(lambda xp: lambda a, b: xp.maximum(a, b) - xp.minimum(a, 0.5), [x, y])
+
+
+def test_scalars_and_promotion():
+    x = shaped_random((64,), 'int32', 3)
+    four_way(lambda xp: lambda a: a * 2 + 1, [x])
+    four_way(lambda xp: lambda a: a * 2.5, [x])
+    four_way(lambda xp: lambda a, s: a + s, [x, 3])
+    four_way(lambda xp: lambda a, s: a + s, [x, 2.5])
+    h = shaped_random((64,), 'float16', 4)
+    four_way(lambda xp: lambda a: a * 2 + 1, [h])
+    four_way(lambda xp: lambda a, b: a + b, [h, x.astype(np.float32)])
+    four_way(lambda xp: lambda a, s: a * s, [h, np.float32(1.5)])
+
+
+BCAST = [((10,), (1,)), ((3, 1), (1, 4)), ((2, 1, 4), (3, 1)), ((256, 256), (256, 1)),
+         ((5, 6), (6,)), ((0,), (1,))]
+
+
+@pytest.mark.parametrize('sa,sb', BCAST)
+def test_broadcast_shapes(sa, sb):
+    a = shaped_random(sa, 'float32', 5)
+    b = shaped_random(sb, 'float32', 6)
+    four_way(lambda xp: lambda p, q: p * q + q, [a, b])
+
+
+def test_invalid_broadcast():
+    f = cp.fuse(lambda p, q: p + q)
+    with pytest.raises(ValueError):
+        f(cp.zeros((3,), np.float32), cp.zeros((4,), np.float32))
+
+
+def test_power_shortcuts_match_numpy():
+    h = shaped_random((500,), 'float16', 7, scale=3)
+    four_way(lambda xp: lambda a: a ** 2, [h])
+    f = shaped_random((500,), 'float32', 8, scale=3)
+    four_way(lambda xp: lambda a: a ** 2 + a, [f])
+    four_way(lambda xp: lambda a: xp.absolute(a) ** 0.5, [f])
+    i = shaped_random((100,), 'int32', 9, scale=5)
+    four_way(lambda xp: lambda a: a ** 2, [i])
+    four_way(lambda xp: lambda a: a ** 3, [np.abs(i)])
+
+
+def test_non_contiguous_inputs_and_multiple_outputs():
+    x = shaped_random((40, 60), 'float32', 10)
+    y = shaped_random((60, 40), 'float32', 11)
+    d, e = cp.asarray(x), cp.asarray(y)
+    f = cp.fuse(lambda a, b: (a + b, a - b))
+    s, t = f(d, e.T)
+    assert_exact(s.get(), x + y.T)
+    assert_exact(t.get(), x - y.T)
+    g = cp.fuse(lambda a, b: a[...] if False else a * b)
+    assert_exact(g(d[::2, 1::2], e.T[::2, 1::2]).get(), x[::2, 1::2] * y.T[::2, 1::2])
+
+
+def test_in_place_update_of_an_argument():
+    x = shaped_random((100,), 'float32', 12)
+    y = shaped_random((100,), 'float32', 13)
+
+    @cp.fuse()
+    def update(a, b):
+        a += b * 2
+        return a
+
+    d = cp.asarray(x)
+    r = update(d, cp.asarray(y))
+    assert_exact(d.get(), x + y * 2)
+    assert_exact(r.get(), x + y * 2)
+
+
+def test_astype_and_comparison():
+    x = shaped_random((80,), 'float32', 14)
+    four_way(lambda xp: lambda a: (a > 0).astype(np.int32) * 3, [x])
+    four_way(lambda xp: lambda a: a.astype(np.float16) + a.astype(np.float16), [x])
+
+
+# -- reductions ------------------------------------------------------------------------------
+
+def test_fused_sum_over_each_axis():
+    x = shaped_random((37, 53), 'float32', 15, scale=1)
+    y = shaped_random((37, 53), 'float32', 16, scale=1)
+    for axis in (0, 1, -1, None):
+        four_way(lambda xp: lambda a, b: xp.sum(a * b + a, axis=axis), [x, y], exact=False)
+    four_way(lambda xp: lambda a: xp.sum(a), [x], exact=False)
+    i = shaped_random((37, 53), 'int32', 17)
+    four_way(lambda xp: lambda a: xp.sum(a * a, axis=0), [i])
+
+
+def test_fused_config_small(small_configs):
+    c = small_configs
+
+    @cp.fuse()
+    def f(x, y, w):
+        return cp.sum((x - y) ** 2 * w, axis=-1)
+
+    got = f(cp.asarray(c['c5_x']), cp.asarray(c['c5_y']), cp.asarray(c['c5_w']))
+    assert got.dtype == np.float32 and got.shape == (70,)
+    assert np.allclose(got.get(), c['c5_out'], rtol=1e-5)
+    assert np.allclose(got.get(), o.fused_sqdiff_wsum(c['c5_x'], c['c5_y'], c['c5_w']), rtol=1e-5)
+    # the float16 roundings of the pipeline are reproduced: an unrounded float32
+    # evaluation is farther away than the tolerance on at least one row
+    x32, y32 = c['c5_x'].astype(np.float32), c['c5_y'].astype(np.float32)
+    unrounded = ((x32 - y32) ** 2 * c['c5_w']).sum(axis=-1)
+    assert np.abs(got.get() - c['c5_out']).max() < np.abs(unrounded - c['c5_out']).max()
+    # identical inputs: exactly zero
+    z = f(cp.asarray(c['c5_x']), cp.asarray(c['c5_x']), cp.asarray(c['c5_w']))
+    assert_exact(z.get(), np.zeros(70, np.float32))
+
+
+def test_post_reduction_operations():
+    x = shaped_random((30, 200), 'float32', 18, scale=1)
+    four_way(lambda xp: lambda a: xp.sqrt(xp.sum(a * a, axis=1)), [x], exact=False)
+    four_way(lambda xp: lambda a: xp.sum(a, axis=0) * 2 + 1, [x], exact=False)
+
+
+def test_fused_min_max_prod():
+    x = shaped_random((20, 30), 'float32', 19, scale=2)
+    four_way(lambda xp: lambda a: xp.amax(a * 2, axis=1), [x])
+    four_way(lambda xp: lambda a: xp.amin(a + 1, axis=0), [x])
+    four_way(lambda xp: lambda a: xp.prod(a * 0.5 + 1, axis=1), [x], exact=False, rtol=1e-4)
+
+
+def test_reduction_restrictions():
+    @cp.fuse()
+    def two(a):
+        return cp.sum(cp.sum(a, axis=0))
+
+    with pytest.raises(NotImplementedError):
+        two(cp.zeros((3, 3), np.float32))
+
+    @cp.fuse()
+    def mixed(a):
+        return cp.sum(a, axis=0) + a
+
+    with pytest.raises(Exception, match='Shape mismatch'):
+        mixed(cp.zeros((3, 3), np.float32))
+
+
+def test_nested_fused_functions():
+    @cp.fuse()
+    def inner(a, b):
+        return a * b
+
+    @cp.fuse()
+    def outer(a, b):
+        return inner(a, b) + a
+
+    x = shaped_random((64,), 'float32', 20)
+    y = shaped_random((64,), 'float32', 21)
+    assert_exact(outer(cp.asarray(x), cp.asarray(y)).get(), x * y + x)

@@ -1,0 +1,310 @@
+"""Reduction path on the GPU against NumPy: sums (all dtypes, axes, layouts,
+sizes around powers of two), argmax/argmin (ties, NaN, first occurrence),
+min/max/any/all/prod and user ReductionKernels.
+
+Tolerances: integer and index results bit-exact; floating-point sums within
+rtol 1e-5 (fp32) / 1e-12 (fp64) / 1e-3 (fp16) of NumPy, measured against the
+sum of absolute addends (the order of additions differs from NumPy's)."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from helpers import assert_exact, assert_sum_close, shaped_random
+from oracle import numpy_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def check_sum(a, axis=None, keepdims=False, dtype=None, view=None):
+    d = cp.asarray(a)
+    if view is not None:
+        a, d = view(a), view(d)
+    got = d.sum(axis=axis, keepdims=keepdims, dtype=dtype)
+    expect = a.sum(axis=axis, keepdims=keepdims, dtype=dtype)
+    if expect.dtype.kind == 'f':
+        mag = np.abs(a.astype(np.float64)).sum(axis=axis, keepdims=keepdims)
+        assert_sum_close(got.get(), np.asarray(expect), mag, expect.dtype)
+    else:
+        assert_exact(got.get(), np.asarray(expect))
+    return got
+
+
+@pytest.mark.parametrize('dtype', ['bool', 'int8', 'uint8', 'int16', 'uint16', 'int32',
+                                   'uint32', 'int64', 'uint64', 'float16', 'float32', 'float64'])
+def test_sum_all_dtypes(dtype):
+    a = shaped_random((21, 37), dtype, 1, scale=100)
+    for axis in (None, 0, 1, (0, 1), -1):
+        check_sum(a, axis)
+    check_sum(a, 1, keepdims=True)
+    check_sum(a, None, keepdims=True)
+
+
+def test_int8_sums_wrap_like_numpy(small_configs):
+    i8 = small_configs['i8']
+    d = cp.asarray(i8)
+    assert_exact(d.sum(axis=0).get(), small_configs['i8_ax0'])
+    assert_exact(d.sum(axis=1).get(), small_configs['i8_ax1'])
+    assert_exact(d.sum(axis=0, dtype=np.int8).get(), i8.sum(axis=0, dtype=np.int8))
+    assert_exact(d.sum(dtype=np.int8).get(), np.asarray(i8.sum(dtype=np.int8)))
+
+
+@pytest.mark.parametrize('i', range(1, 14))
+def test_sum_sizes_around_powers_of_two(i):
+    for n in (2 ** i - 1, 2 ** i, 2 ** i + 1):
+        a = shaped_random((n,), 'int8', n, scale=100)
+        check_sum(a)
+        f = shaped_random((n,), 'float32', n)
+        check_sum(f)
+
+
+@pytest.mark.parametrize('shape', [(2, 1000), (1000, 2), (65, 1000), (1000, 65), (512, 65536 // 64),
+                                   (513, 1025), (1, 5000), (5000, 1), (3, 70000), (70000, 3)])
+def test_sum_rectangular(shape):
+    a = shaped_random(shape, 'float32', 3)
+    check_sum(a, 0)
+    check_sum(a, 1)
+    check_sum(a)
+    i = shaped_random(shape, 'int32', 4, scale=1000)
+    check_sum(i, 0)
+    check_sum(i, 1)
+
+
+def test_sum_small_config(small_configs):
+    c = small_configs
+    for name, rtol in (('f32', 1e-5), ('f64', 1e-12)):
+        a = c['c3_' + name]
+        d = cp.asarray(a)
+        for axis, key in ((0, 'ax0'), (1, 'ax1'), (None, 'all')):
+            mag = np.abs(a.astype(np.float64)).sum(axis=axis)
+            assert_sum_close(d.sum(axis=axis).get(), c['c3_%s_%s' % (name, key)], mag, a.dtype)
+
+
+TRANSPOSES = [
+    ((2, 3, 4), (1, 0, 2), 0), ((2, 3, 4), (1, 0, 2), 1), ((2, 3, 4), (2, 0, 1), 2),
+    ((2, 3, 4), (2, 1, 0), (0, 2)), ((2, 3, 4, 5), (3, 1, 0, 2), (1, 2)),
+    ((2, 3, 4, 5), (0, 2, 1, 3), (0, 3)), ((2, 3, 4, 5), (1, 3, 0, 2), None),
+    ((6, 0, 4), (1, 0, 2), 2), ((3, 5, 7), (2, 1, 0), (0, 1, 2)),
+]
+
+
+@pytest.mark.parametrize('shape,perm,axis', TRANSPOSES)
+def test_sum_of_transposed_views(shape, perm, axis):
+    a = shaped_random(shape, 'float64', 5)
+    check_sum(a, axis, view=lambda x: x.transpose(perm))
+    check_sum(a, axis, keepdims=True, view=lambda x: x.transpose(perm))
+
+
+def test_sum_strided_and_broadcast_views():
+    a = shaped_random((40, 30, 20), 'float32', 6)
+    check_sum(a, 1, view=lambda x: x[::2, :, ::3])
+    check_sum(a, (0, 2), view=lambda x: x[:, ::-1, 1:])
+    check_sum(a, 0, view=lambda x: x[5:6])
+    b = shaped_random((64, 1, 32), 'float32', 7)
+    d = cp.broadcast_to(cp.asarray(b), (64, 16, 32))
+    e = np.broadcast_to(b, (64, 16, 32))
+    assert_sum_close(d.sum(axis=2).get(), e.sum(axis=2),
+                     np.abs(e.astype(np.float64)).sum(axis=2), np.float32)
+    assert_sum_close(d.sum(axis=1).get(), e.sum(axis=1),
+                     np.abs(e.astype(np.float64)).sum(axis=1), np.float32)
+
+
+def test_sum_many_dims_keepdims():
+    a = shaped_random((2, 3, 2, 3, 2, 3, 2), 'float64', 8)
+    check_sum(a, (1, 3, 4, 6), keepdims=True)
+    check_sum(a, (0, 2, 5))
+
+
+def test_sum_out_and_dtype_arguments():
+    a = shaped_random((30, 50), 'float32', 9)
+    d = cp.asarray(a)
+    out = cp.empty((50,), np.float32)
+    assert d.sum(axis=0, out=out) is out
+    assert_sum_close(out.get(), a.sum(axis=0), np.abs(a).sum(axis=0, dtype=np.float64), np.float32)
+    out64 = cp.empty((30,), np.float64)
+    d.sum(axis=1, out=out64)
+    assert np.allclose(out64.get(), a.sum(axis=1), rtol=1e-5)
+    strided = cp.zeros((30, 2), np.float32)
+    d.sum(axis=1, out=strided[:, 1])
+    assert np.allclose(strided.get()[:, 1], a.sum(axis=1), rtol=1e-5)
+    assert np.all(strided.get()[:, 0] == 0)
+    i = shaped_random((30, 50), 'int32', 10)
+    assert_exact(cp.asarray(i).sum(axis=0, dtype=np.float64).get(), i.sum(axis=0, dtype=np.float64))
+    assert_exact(cp.sum(cp.asarray(i), axis=1).get(), i.sum(axis=1))
+    assert_exact(cp.add.reduce(cp.asarray(i), axis=1).get(), np.add.reduce(i, axis=1))
+
+
+def test_float16_sum_accumulates_in_float32():
+    a = np.full((4096,), 0.1, np.float16)
+    got = cp.asarray(a).sum().get()
+    assert got.dtype == np.float16
+    # accumulating in float16 would stall far below the true value
+    assert abs(float(got) - float(np.float32(a).sum())) <= 1.0
+
+
+def test_prod_min_max_any_all():
+    a = shaped_random((12, 9), 'float32', 11, scale=2)
+    d = cp.asarray(a)
+    for axis in (None, 0, 1):
+        assert np.allclose(d.prod(axis=axis).get(), a.prod(axis=axis), rtol=1e-4)
+        assert_exact(d.max(axis=axis).get(), np.asarray(a.max(axis=axis)))
+        assert_exact(d.min(axis=axis).get(), np.asarray(a.min(axis=axis)))
+        assert_exact((d > 0).any(axis=axis).get(), np.asarray((a > 0).any(axis=axis)))
+        assert_exact((d > -1.9).all(axis=axis).get(), np.asarray((a > -1.9).all(axis=axis)))
+    n = a.copy()
+    n[3, 4] = np.nan
+    dn = cp.asarray(n)
+    assert_exact(dn.max(axis=0).get(), n.max(axis=0))
+    assert_exact(dn.min(axis=1).get(), n.min(axis=1))
+    i = shaped_random((7, 300), 'int16', 12, scale=1000)
+    assert_exact(cp.amax(cp.asarray(i), axis=1).get(), i.max(axis=1))
+    assert_exact(cp.amin(cp.asarray(i)).get(), np.asarray(i.min()))
+    assert np.allclose(d.mean(axis=0).get(), a.mean(axis=0), rtol=1e-5)
+
+
+# -- argmax / argmin ------------------------------------------------------------------------
+
+@pytest.mark.parametrize('dtype', ['bool', 'int8', 'uint8', 'int16', 'int32', 'uint32', 'int64',
+                                   'uint64', 'float16', 'float32', 'float64'])
+def test_arg_extreme_golden_cases(golden, dtype):
+    dt = np.dtype(dtype)
+    for case in golden['argmax_cases']:
+        if case.get('float_only') and dt.kind != 'f':
+            continue
+        a = np.array([float(v) for v in case['values']]).astype(dt)
+        got = cp.asarray(a).argmax()
+        assert got.dtype == np.int64
+        assert int(got.get()) == (case['argmax'] if dt.kind != 'b' else int(np.argmax(a)))
+    for case in golden['argmin_cases']:
+        if case.get('float_only') and dt.kind != 'f':
+            continue
+        a = np.array([float(v) for v in case['values']]).astype(dt)
+        assert int(cp.asarray(a).argmin().get()) == (
+            case['argmin'] if dt.kind != 'b' else int(np.argmin(a)))
+
+
+@pytest.mark.parametrize('shape', [(2, 3), (3, 1000), (1000, 3), (2, 3, 4), (17, 128), (5, 129),
+                                   (300, 2), (9, 4096), (4, 5000)])
+def test_arg_extreme_heavy_ties(shape):
+    a = shaped_random(shape, 'int32', 13, scale=3)
+    d = cp.asarray(a)
+    for axis in list(range(len(shape))) + [None, -1]:
+        assert_exact(d.argmax(axis=axis).get(), np.asarray(a.argmax(axis=axis)))
+        assert_exact(d.argmin(axis=axis).get(), np.asarray(a.argmin(axis=axis)))
+    if len(shape) == 2:
+        assert_exact(d.argmax(axis=1).get(), o.argmax_first(a, 1))
+        assert_exact(d.argmin(axis=0).get(), o.argmin_first(a, 0))
+
+
+def test_arg_extreme_small_config(small_configs):
+    c = small_configs
+    d = cp.asarray(c['c4_i32'])
+    assert_exact(d.argmax(axis=-1).get(), c['c4_i32_argmax'])
+    assert_exact(d.argmin(axis=-1).get(), c['c4_i32_argmin'])
+    assert_exact(cp.asarray(c['c4_f32']).argmax(axis=1).get(), c['c4_f32_argmax'])
+
+
+def test_arg_extreme_nan_positions():
+    a = shaped_random((50, 260), 'float32', 14)
+    a[3, 100] = np.nan
+    a[3, 7] = np.nan          # two NaNs in a row: the first one wins
+    a[9, 259] = np.nan
+    a[20, 0] = np.nan
+    a[:, 33] = np.nan         # a NaN in every row: competes with the others above
+    a[3, 7] = np.nan
+    d = cp.asarray(a)
+    for axis in (0, 1, None):
+        assert_exact(d.argmax(axis=axis).get(), np.asarray(a.argmax(axis=axis)))
+        assert_exact(d.argmin(axis=axis).get(), np.asarray(a.argmin(axis=axis)))
+    h = a.astype(np.float16)
+    assert_exact(cp.asarray(h).argmax(axis=1).get(), h.argmax(axis=1))
+    assert_exact(cp.asarray(a.astype(np.float64)).argmin(axis=0).get(), a.argmin(axis=0))
+    inf = np.array([1.0, np.inf, -np.inf, np.inf, 2.0] * 30, np.float32)
+    assert int(cp.asarray(inf).argmax().get()) == 1
+    assert int(cp.asarray(inf).argmin().get()) == 2
+
+
+def test_arg_extreme_layouts_and_options():
+    a = shaped_random((6, 7, 8), 'float64', 15, scale=2).round()
+    d = cp.asarray(a)
+    for perm in ((1, 0, 2), (2, 1, 0), (0, 2, 1)):
+        for axis in (0, 1, 2, None):
+            assert_exact(d.transpose(perm).argmax(axis=axis).get(),
+                         np.asarray(a.transpose(perm).argmax(axis=axis)))
+    f = np.asfortranarray(a[0])
+    assert_exact(cp.asarray(f).argmax().get(), np.asarray(f.argmax()))   # C-order flattening
+    assert_exact(d[::2, :, ::-1].argmin(axis=2).get(), a[::2, :, ::-1].argmin(axis=2))
+    assert_exact(d.argmax(axis=1, keepdims=True).get(), a.argmax(axis=1, keepdims=True))
+    for dt in (np.int8, np.int16, np.int32, np.int64):
+        assert_exact(d.argmax(axis=2, dtype=dt).get(), a.argmax(axis=2).astype(dt))
+    out = cp.empty((6, 8), np.int64)
+    assert d.argmin(axis=1, out=out) is out
+    assert_exact(out.get(), a.argmin(axis=1))
+    assert_exact(cp.argmax(d, axis=0).get(), a.argmax(axis=0))
+
+
+# -- user reduction kernels --------------------------------------------------------------------
+
+def test_l2norm_kernel():
+    l2 = cp.ReductionKernel('T x', 'T y', 'x * x', 'a + b', 'y = sqrt(a)', '0', 'l2norm')
+    a = np.arange(10, dtype=np.float32).reshape(2, 5)
+    assert np.allclose(l2(cp.asarray(a), axis=1).get(), np.sqrt((a * a).sum(axis=1)), rtol=1e-6)
+    b = shaped_random((33, 700), 'float64', 16)
+    d = cp.asarray(b)
+    for axis in (0, 1, None):
+        assert np.allclose(l2(d, axis=axis).get(), np.sqrt((b * b).sum(axis=axis)), rtol=1e-12)
+    assert np.allclose(l2(d, axis=1, keepdims=True).get(),
+                       np.sqrt((b * b).sum(axis=1, keepdims=True)), rtol=1e-12)
+    out = cp.empty((700,), np.float64)
+    l2(d, out=out, axis=0)
+    assert np.allclose(out.get(), np.sqrt((b * b).sum(axis=0)), rtol=1e-12)
+
+
+def test_multi_input_broadcast_and_scalars():
+    dot = cp.ReductionKernel('T x, T y, T scale', 'T z', 'x * y * scale', 'a + b', 'z = a', '0',
+                             'scaled_dot')
+    x = shaped_random((40, 300), 'float32', 17, scale=1)
+    y = shaped_random((300,), 'float32', 18, scale=1)
+    got = dot(cp.asarray(x), cp.asarray(y), 2.0, axis=1)
+    expect = (x * y * np.float32(2)).sum(axis=1)
+    assert np.allclose(got.get(), expect, rtol=1e-5, atol=1e-4)
+    got0 = dot(cp.asarray(x), cp.asarray(y), 2.0, axis=0)
+    assert np.allclose(got0.get(), (x * y * np.float32(2)).sum(axis=0), rtol=1e-5, atol=1e-4)
+    col = shaped_random((40, 1), 'float32', 19, scale=1)
+    got = dot(cp.asarray(x), cp.asarray(col), 1.0)
+    assert np.allclose(got.get(), (x * col).sum(), rtol=1e-4)
+
+
+def test_reduce_type_identity_and_post_map():
+    # count of positives as int64 even for float input; post map adds a bias
+    cnt = cp.ReductionKernel('T x, int64 bias', 'int64 y', 'x > 0 ? 1 : 0', 'a + b',
+                             'y = a + bias', '0', 'count_pos', reduce_type='long long')
+    a = shaped_random((77, 91), 'float32', 20)
+    assert_exact(cnt(cp.asarray(a), 5, axis=0).get(), (a > 0).sum(axis=0) + 5)
+    assert_exact(cnt(cp.asarray(a), 0).get(), np.asarray((a > 0).sum()))
+    mx = cp.ReductionKernel('T x', 'T y', 'x', 'max(a, b)', 'y = a', '-1e30f', 'my_max')
+    assert_exact(mx(cp.asarray(a), axis=1).get(), a.max(axis=1))
+
+
+def test_raw_input_with_leading_reduce_axes():
+    # raw arrays are legal when the reduced axes come first
+    k = cp.ReductionKernel(
+        'T x, raw T w', 'T y', 'x * w[_j / _out_ind.size()]', 'a + b', 'y = a', '0',
+        'weighted_rows')
+    x = shaped_random((6, 50), 'float64', 21)
+    w = shaped_random((6,), 'float64', 22)
+    got = k(cp.asarray(x), cp.asarray(w), axis=0)
+    assert np.allclose(got.get(), (x * w[:, None]).sum(axis=0), rtol=1e-12)
+    with pytest.raises(NotImplementedError):
+        k(cp.asarray(x), cp.asarray(w), axis=1)
+
+
+def test_large_full_reduction_is_split_and_deterministic():
+    a = shaped_random((3_000_001,), 'float32', 23, scale=1)
+    d = cp.asarray(a)
+    r1 = d.sum().get()
+    r2 = d.sum().get()
+    assert r1 == r2
+    assert abs(float(r1) - o.sum_exact(a)) <= 1e-5 * float(np.abs(a).sum(dtype=np.float64))
+    i = shaped_random((3_000_001,), 'int32', 24, scale=2 ** 30)
+    assert_exact(cp.asarray(i).sum().get(), np.asarray(i.sum()))
+    assert int(cp.asarray(i).argmax().get()) == int(i.argmax())

@@ -1,0 +1,178 @@
+"""The C-ABI shim on a real device, called through ctypes only: memory, copies,
+streams, events, compile -> load -> launch, and the pool on hipMalloc."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from cupy_amd import _rt
+import cupy_amd as cp
+from cupy_amd.cuda import memory
+
+pytestmark = pytest.mark.gpu
+lib = _rt.lib
+
+
+def test_device_queries():
+    n = ctypes.c_int(0)
+    assert lib.rt_init() == 0
+    assert lib.rt_device_count(ctypes.byref(n)) == 0 and n.value >= 1
+    props = _rt.rt_device_props()
+    assert lib.rt_device_get_props(0, ctypes.byref(props)) == 0
+    assert props.arch.decode().startswith('gfx950')
+    assert props.warp_size == 64 and props.compute_units > 0
+    free = ctypes.c_size_t(0)
+    total = ctypes.c_size_t(0)
+    assert lib.rt_mem_info(ctypes.byref(free), ctypes.byref(total)) == 0
+    assert 0 < free.value <= total.value
+
+
+def test_raw_compile_load_launch_round_trip():
+    src = (b'extern "C" __global__ void scale(const float* x, float* y, float a, int n) {'
+           b' int i = blockIdx.x * blockDim.x + threadIdx.x; if (i < n) y[i] = a * x[i]; }')
+    opts = [b'--offload-arch=gfx950', b'-O3']
+    c_opts = (ctypes.c_char_p * len(opts))(*opts)
+    code = ctypes.c_void_p()
+    size = ctypes.c_size_t(0)
+    log = ctypes.c_void_p()
+    assert lib.rt_compile(src, b'scale.hip', len(opts), c_opts, 0, None, None,
+                          ctypes.byref(code), ctypes.byref(size), ctypes.byref(log)) == 0
+    mod = ctypes.c_void_p()
+    assert lib.rt_module_load(code, ctypes.byref(mod)) == 0
+    fn = ctypes.c_void_p()
+    assert lib.rt_module_get_function(mod, b'scale', ctypes.byref(fn)) == 0
+    missing = ctypes.c_void_p()
+    assert lib.rt_module_get_function(mod, b'nope', ctypes.byref(missing)) != 0
+    n = 1000
+    host = np.arange(n, dtype=np.float32)
+    dx = ctypes.c_void_p()
+    dy = ctypes.c_void_p()
+    assert lib.rt_malloc(ctypes.byref(dx), n * 4) == 0
+    assert lib.rt_malloc(ctypes.byref(dy), n * 4) == 0
+    assert lib.rt_memcpy(dx, host.ctypes.data, n * 4, _rt.MEMCPY_H2D) == 0
+    stream = ctypes.c_void_p()
+    assert lib.rt_stream_create(ctypes.byref(stream), 1) == 0
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    assert lib.rt_event_create(ctypes.byref(e0), 0) == 0
+    assert lib.rt_event_create(ctypes.byref(e1), 0) == 0
+    # (a) pointer-array launch
+    a = ctypes.c_float(3.0)
+    cn = ctypes.c_int(n)
+    params = (ctypes.c_void_p * 4)(
+        ctypes.addressof(dx), ctypes.addressof(dy), ctypes.addressof(a), ctypes.addressof(cn))
+    assert lib.rt_event_record(e0, stream) == 0
+    assert lib.rt_launch(fn, 4, 1, 1, 256, 1, 1, 0, stream, params) == 0
+    assert lib.rt_event_record(e1, stream) == 0
+    assert lib.rt_stream_synchronize(stream) == 0
+    ms = ctypes.c_float(-1)
+    assert lib.rt_event_elapsed_ms(ctypes.byref(ms), e0, e1) == 0 and ms.value >= 0
+    out = np.empty(n, np.float32)
+    assert lib.rt_memcpy(out.ctypes.data, dy, n * 4, _rt.MEMCPY_D2H) == 0
+    assert np.array_equal(out, host * 3)
+    # (b) packed argument block
+    import struct
+    blob = struct.pack('@PPfi', dx.value, dy.value, 0.5, n)
+    assert lib.rt_memset_async(dy, 0, n * 4, stream) == 0
+    assert lib.rt_launch_packed(fn, 4, 1, 1, 256, 1, 1, 0, stream, blob, len(blob)) == 0
+    assert lib.rt_memcpy_async(out.ctypes.data, dy, n * 4, _rt.MEMCPY_D2H, stream) == 0
+    assert lib.rt_stream_synchronize(stream) == 0
+    assert np.array_equal(out, host * 0.5)
+    done = ctypes.c_int(0)
+    assert lib.rt_stream_query(stream, ctypes.byref(done)) == 0 and done.value == 1
+    occ = ctypes.c_int(0)
+    assert lib.rt_occupancy_max_active_blocks(fn, 256, 0, ctypes.byref(occ)) == 0 and occ.value > 0
+    regs = ctypes.c_int(0)
+    assert lib.rt_func_get_attribute(4, fn, ctypes.byref(regs)) == 0 and regs.value > 0
+    for e in (e0, e1):
+        assert lib.rt_event_destroy(e) == 0
+    assert lib.rt_stream_destroy(stream) == 0
+    assert lib.rt_free(dx) == 0 and lib.rt_free(dy) == 0
+    assert lib.rt_module_unload(mod) == 0
+    lib.rt_free_buffer(code)
+    lib.rt_free_buffer(log)
+
+
+def test_pinned_host_memory_and_async_copy():
+    n = 1 << 16
+    h = ctypes.c_void_p()
+    assert lib.rt_host_alloc(ctypes.byref(h), n) == 0
+    buf = (ctypes.c_ubyte * n).from_address(h.value)
+    for i in range(0, n, 4096):
+        buf[i] = i // 4096
+    d = ctypes.c_void_p()
+    assert lib.rt_malloc(ctypes.byref(d), n) == 0
+    assert lib.rt_memcpy_async(d, h, n, _rt.MEMCPY_H2D, None) == 0
+    back = np.zeros(n, np.uint8)
+    assert lib.rt_memcpy(back.ctypes.data, d, n, _rt.MEMCPY_D2H) == 0
+    assert back[4096 * 3] == 3 and back[1] == 0
+    assert lib.rt_free(d) == 0
+    assert lib.rt_host_free(h) == 0
+
+
+def test_pool_on_device_memory():
+    pool = memory.SingleDeviceMemoryPool()
+    p = pool.malloc(1000)
+    assert p.ptr % 512 == 0
+    assert pool.used_bytes() == 1024 and pool.total_bytes() == 1024
+    ptr = p.ptr
+    del p
+    assert pool.free_bytes() == 1024
+    q = pool.malloc(600)
+    assert q.ptr == ptr
+    s = cp.cuda.Stream()
+    with s:
+        r = pool.malloc(600)
+        assert r.ptr != ptr
+    del q, r
+    assert pool.n_free_blocks() == 2
+    pool.free_all_blocks()
+    assert pool.total_bytes() == 0
+    pool.set_limit(size=1 << 20)
+    with pytest.raises(memory.OutOfMemoryError):
+        pool.malloc(2 << 20)
+    pool.set_limit(size=0)
+
+
+def test_default_pool_backs_arrays_and_reuses_blocks():
+    pool = cp.get_default_memory_pool()
+    a = cp.zeros((1000,), np.float32)
+    ptr = a.data.ptr
+    used = pool.used_bytes()
+    assert used >= 4096 - 512
+    del a
+    b = cp.empty((1000,), np.float32)
+    assert b.data.ptr == ptr
+    assert isinstance(b.data.mem, memory.PooledMemory)
+    with cp.cuda.using_allocator(memory._malloc):
+        c = cp.empty((10,), np.float32)
+        assert not isinstance(c.data.mem, memory.PooledMemory)
+
+
+def test_streams_events_and_stream_argument():
+    x = np.arange(100000, dtype=np.float32)
+    s = cp.cuda.Stream(non_blocking=True)
+    k = cp.ElementwiseKernel('T x', 'T y', 'y = x + 1', 'plus_one')
+    with s:
+        d = cp.asarray(x)
+        start = cp.cuda.Event()
+        stop = cp.cuda.Event()
+        start.record()
+        y = k(d)
+        stop.record()
+        stop.synchronize()
+        assert cp.cuda.get_elapsed_time(start, stop) >= 0
+        assert cp.cuda.get_current_stream() is s
+        assert np.array_equal(y.get(), x + 1)
+    assert cp.cuda.get_current_stream().ptr == 0
+    d = cp.asarray(x)
+    y = k(d, stream=s)
+    s.synchronize()
+    assert s.done
+    assert np.array_equal(y.get(), x + 1)
+
+
+def test_compile_error_surfaces_as_exception():
+    k = cp.ElementwiseKernel('T x', 'T y', 'y = undefined_function(x)', 'bad_kernel')
+    with pytest.raises(cp.cuda.CompileException) as info:
+        k(cp.zeros((4,), np.float32))
+    assert 'undefined_function' in str(info.value)
