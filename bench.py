@@ -1,0 +1,358 @@
+"""Benchmark of the generated-kernel hot path on one MI355X.
+
+A "step" is one pass over the five benchmark configurations at their full
+shapes (13 operations, inputs resident in HBM, outputs preallocated):
+
+  C1  saxpy via ElementwiseKernel, float32, N = 2**26
+  C2  x.T * y (+ 1): float32 (8192, 8192) transposed view times float16 (1, 8192)
+      row, then add of a Python scalar (two ufunc calls)
+  C3  sum over axis=1, axis=0 and all elements: float32 (16384, 16384) and
+      float64 (8192, 8192)
+  C4  argmax and argmin of int32 (2**20, 128) along the last axis, argmax of
+      float32 (2**16, 4096) along axis 1
+  C5  fused sum((x - y)**2 * w, axis=-1): float16 (2**18, 256) x 2, float32 (256,)
+
+``value`` is the algorithmic bytes of one step divided by the wall time of a
+step (all launches enqueued through the public API, one synchronisation at the
+end of the timed region).  ``per_config`` gives each operation's own figure,
+measured with HIP events on the launch stream; ``roofline`` repeats the entry of
+the operation that takes the largest share of a step.  ``cpu_baseline`` is NumPy
+evaluating the same operations on the same host arrays, single-threaded.
+
+Prints exactly one JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_cases(cp, scale=1):
+    """Returns a list of dicts: name, algorithmic bytes, gpu callable, numpy
+    callable, parity check."""
+    from oracle import numpy_oracle as oracle
+    cases = []
+
+    def add(name, config, nbytes, gpu, cpu, check, kernel):
+        cases.append(dict(name=name, config=config, bytes=int(nbytes), gpu=gpu, cpu=cpu,
+                          check=check, kernel=kernel))
+
+    # ---- C1 ---------------------------------------------------------------------------
+    n1 = (1 << 26) // scale
+    rng = np.random.default_rng(1)
+    x1 = rng.uniform(-1, 1, n1).astype(np.float32)
+    y1 = rng.uniform(-1, 1, n1).astype(np.float32)
+    dx1, dy1 = cp.asarray(x1), cp.asarray(y1)
+    z1 = cp.empty((n1,), np.float32)
+    hz1 = np.empty(n1, np.float32)
+    saxpy = cp.ElementwiseKernel('float32 x, float32 y, float32 a', 'float32 z',
+                                 'z = a * x + y', 'saxpy')
+
+    def cpu_saxpy():
+        np.multiply(np.float32(2.5), x1, out=hz1)
+        np.add(hz1, y1, out=hz1)
+        return hz1
+
+    add('C1 saxpy f32 2^26', 'C1', 12 * n1, lambda: saxpy(dx1, dy1, 2.5, z1), cpu_saxpy,
+        lambda: np.array_equal(z1.get(), oracle.saxpy(2.5, x1, y1)), 'saxpy')
+
+    # ---- C2 ---------------------------------------------------------------------------
+    m = 8192 // (4 if scale > 1 else 1)
+    rng = np.random.default_rng(2)
+    base = rng.standard_normal((m, m), dtype=np.float32)
+    y2 = rng.uniform(0, 2, (1, m)).astype(np.float16)
+    dbase = cp.asarray(base)
+    dx2 = dbase.T
+    dy2 = cp.asarray(y2)
+    tmp2 = cp.empty((m, m), np.float32)
+    out2 = cp.empty((m, m), np.float32)
+    htmp2 = np.empty((m, m), np.float32)
+    hout2 = np.empty((m, m), np.float32)
+    add('C2a x.T*y f32(T)xf16 8192^2', 'C2', 8 * m * m + 2 * m,
+        lambda: cp.multiply(dx2, dy2, tmp2), lambda: np.multiply(base.T, y2, out=htmp2),
+        lambda: np.array_equal(tmp2.get(), base.T * y2),
+        'cupy_multiply__float32_float16_float32')
+    add('C2b tmp+1 f32 8192^2', 'C2', 8 * m * m,
+        lambda: cp.add(tmp2, 1, out2), lambda: np.add(htmp2, 1, out=hout2),
+        lambda: np.array_equal(out2.get(), oracle.broadcast_mul_add(base.T, y2, 1)),
+        'cupy_add__float32_float_float32')
+
+    # ---- C3 ---------------------------------------------------------------------------
+    for dt, n, seed, rtol in ((np.float32, 16384, 3, 1e-5), (np.float64, 8192, 4, 1e-12)):
+        n = n // (4 if scale > 1 else 1)
+        rng = np.random.default_rng(seed)
+        a = rng.standard_normal((n, n), dtype=np.float32) if dt == np.float32 \
+            else rng.standard_normal((n, n))
+        da = cp.asarray(a)
+        item = a.dtype.itemsize
+        for axis in (1, 0, None):
+            oshape = () if axis is None else (n,)
+            out = cp.empty(oshape, dt)
+            hout = np.empty(oshape, dt)
+
+            def gpu(da=da, axis=axis, out=out):
+                return da.sum(axis=axis, out=out)
+
+            def cpu(a=a, axis=axis, hout=hout):
+                return np.sum(a, axis=axis, out=hout)
+
+            def check(a=a, axis=axis, out=out, rtol=rtol):
+                mag = np.abs(a).sum(axis=axis, dtype=np.float64)
+                err = np.abs(out.get().astype(np.float64) - np.sum(a, axis=axis))
+                return bool(np.all(err <= rtol * mag))
+
+            add('C3 sum %s axis=%s %d^2' % (np.dtype(dt).name, axis, n), 'C3',
+                a.nbytes + (item if axis is None else n * item), gpu, cpu, check, 'cupy_sum')
+
+    # ---- C4 ---------------------------------------------------------------------------
+    r4 = (1 << 20) // scale
+    rng = np.random.default_rng(5)
+    a4 = rng.integers(0, 16, (r4, 128), dtype=np.int32)
+    d4 = cp.asarray(a4)
+    o4a = cp.empty((r4,), np.int64)
+    o4b = cp.empty((r4,), np.int64)
+    add('C4 argmax i32 (2^20,128)', 'C4', a4.nbytes + r4 * 8,
+        lambda: d4.argmax(axis=-1, out=o4a), lambda: a4.argmax(axis=-1),
+        lambda: np.array_equal(o4a.get(), oracle.argmax_fast(a4, -1)), 'cupy_argmax')
+    add('C4 argmin i32 (2^20,128)', 'C4', a4.nbytes + r4 * 8,
+        lambda: d4.argmin(axis=-1, out=o4b), lambda: a4.argmin(axis=-1),
+        lambda: np.array_equal(o4b.get(), oracle.argmin_fast(a4, -1)), 'cupy_argmin')
+    r4f = (1 << 16) // scale
+    rng = np.random.default_rng(6)
+    a4f = rng.standard_normal((r4f, 4096), dtype=np.float32)
+    d4f = cp.asarray(a4f)
+    o4f = cp.empty((r4f,), np.int64)
+    add('C4 argmax f32 (2^16,4096)', 'C4', a4f.nbytes + r4f * 8,
+        lambda: d4f.argmax(axis=1, out=o4f), lambda: a4f.argmax(axis=1),
+        lambda: np.array_equal(o4f.get(), a4f.argmax(axis=1)), 'cupy_argmax')
+
+    # ---- C5 ---------------------------------------------------------------------------
+    r5 = (1 << 18) // scale
+    rng = np.random.default_rng(7)
+    x5 = rng.standard_normal((r5, 256)).astype(np.float16)
+    y5 = rng.standard_normal((r5, 256)).astype(np.float16)
+    w5 = rng.uniform(0, 1, 256).astype(np.float32)
+    dx5, dy5, dw5 = cp.asarray(x5), cp.asarray(y5), cp.asarray(w5)
+
+    @cp.fuse(kernel_name='fused_sqdiff_wsum')
+    def fused(x, y, w):
+        return cp.sum((x - y) ** 2 * w, axis=-1)
+
+    res5 = [None]
+
+    def gpu5():
+        res5[0] = fused(dx5, dy5, dw5)
+        return res5[0]
+
+    add('C5 fused sum((x-y)^2*w) f16 (2^18,256)', 'C5',
+        2 * x5.nbytes + w5.nbytes + r5 * 4, gpu5,
+        lambda: np.sum((x5 - y5) ** 2 * w5, axis=-1),
+        lambda: bool(np.allclose(res5[0].get(), oracle.fused_sqdiff_wsum(x5, y5, w5),
+                                 rtol=1e-5, atol=0)), 'fused_sqdiff_wsum')
+    return cases
+
+
+def time_case_events(cp, fn, repeats, inner):
+    """Median over ``repeats`` of the time per call, each sample being
+    ``inner`` back-to-back calls bracketed by two events on the launch stream."""
+    e0 = cp.cuda.Event()
+    e1 = cp.cuda.Event()
+    samples = []
+    for _ in range(repeats):
+        e0.record()
+        for _ in range(inner):
+            fn()
+        e1.record()
+        e1.synchronize()
+        samples.append(cp.cuda.get_elapsed_time(e0, e1) * 1e-3 / inner)
+    return float(np.median(samples)), float(np.min(samples))
+
+
+def launch_latency(cp):
+    """Host enqueue cost (us per call, 2000 asynchronous calls on tiny arrays)
+    and event-bracketed single-call latency on an idle stream."""
+    out = {}
+    x = cp.zeros((1,), np.float32)
+    y = cp.zeros((1,), np.float32)
+    k = cp.ElementwiseKernel('T x', 'T y', 'y = x + 1', 'tiny_add')
+
+    @cp.fuse(kernel_name='tiny_fused')
+    def fz(a):
+        return a * 2 + 1
+
+    pool = cp.get_default_memory_pool()
+
+    def pool_cycle():
+        pool.malloc(4096)
+
+    ops = {'ElementwiseKernel': lambda: k(x, y), 'ufunc_add': lambda: cp.add(x, x, y),
+           'sum': lambda: x.sum(out=y.reshape(())), 'fuse': lambda: fz(x),
+           'pool_malloc_free': pool_cycle}
+    for name, fn in ops.items():
+        for _ in range(20):
+            fn()
+        cp.cuda.Device().synchronize()
+        n = 2000
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        t1 = time.perf_counter()
+        cp.cuda.Device().synchronize()
+        entry = {'host_enqueue_us': round((t1 - t0) / n * 1e6, 2)}
+        if name != 'pool_malloc_free':
+            e0, e1 = cp.cuda.Event(), cp.cuda.Event()
+            lat = []
+            for _ in range(50):
+                cp.cuda.Device().synchronize()
+                e0.record()
+                fn()
+                e1.record()
+                e1.synchronize()
+                lat.append(cp.cuda.get_elapsed_time(e0, e1) * 1e3)
+            entry['single_call_us'] = round(float(np.median(lat)), 2)
+        out[name] = entry
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--scale', type=int, default=1,
+                    help='divide the problem sizes (for quick checks only; the '
+                         'reported figure is then not the benchmark figure)')
+    ap.add_argument('--no-cpu', action='store_true', help='skip the NumPy baseline')
+    ap.add_argument('--no-detail', action='store_true',
+                    help='skip per-operation event timing and launch latency')
+    ap.add_argument('--only', default='', help='run only cases whose name contains this')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py measures one GPU: every operation of this path runs on a '
+              'single device; --gpus %d is not supported.' % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import cupy_amd as cp
+    dev = cp.cuda.Device(0)
+    dev.use()
+    props = cp.cuda.device.get_device_properties(0)
+    log('device:', props['arch'], props['compute_units'], 'CUs')
+    t0 = time.perf_counter()
+    cases = build_cases(cp, args.scale)
+    if args.only:
+        cases = [c for c in cases if args.only in c['name']]
+    log('inputs ready in %.1f s' % (time.perf_counter() - t0))
+
+    def step():
+        for c in cases:
+            c['gpu']()
+
+    # warm-up (compiles / loads kernels, grows the pool)
+    for _ in range(max(args.warmup, 1)):
+        step()
+    dev.synchronize()
+    parity = {}
+    for c in cases:
+        parity[c['name']] = bool(c['check']())
+        if not parity[c['name']]:
+            log('PARITY FAILURE:', c['name'])
+
+    # ---- timed region: exactly `steps` steps ------------------------------------------
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    dev.synchronize()
+    t1 = time.perf_counter()
+    step_s = (t1 - t0) / args.steps
+    total_bytes = sum(c['bytes'] for c in cases)
+    value = total_bytes / step_s / 1e9
+
+    per_config = []
+    roof = None
+    if not args.no_detail:
+        for c in cases:
+            med, mn = time_case_events(cp, c['gpu'], repeats=15, inner=10)
+            gbps = c['bytes'] / med / 1e9
+            per_config.append({
+                'name': c['name'], 'config': c['config'], 'kernel': c['kernel'],
+                'bytes': c['bytes'], 'us': round(med * 1e6, 2), 'min_us': round(mn * 1e6, 2),
+                'gbps': round(gbps, 1), 'frac': round(gbps / HBM_PEAK_GBPS, 4),
+                'parity': parity[c['name']]})
+            log('%-42s %9.1f us  %8.1f GB/s  %5.1f%%' % (
+                c['name'], med * 1e6, gbps, gbps / HBM_PEAK_GBPS * 100))
+        dom = max(per_config, key=lambda e: e['us'])
+        roof = {'bound': 'hbm', 'kernel': dom['kernel'], 'operation': dom['name'],
+                'achieved': dom['gbps'], 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+                'frac': dom['frac'], 'traffic': None,
+                'launch_us': dom['us'], 'algorithmic_bytes': dom['bytes']}
+    else:
+        roof = {'bound': 'hbm', 'achieved': round(value, 1), 'peak': HBM_PEAK_GBPS,
+                'unit': 'GB/s', 'frac': round(value / HBM_PEAK_GBPS, 4), 'traffic': None}
+
+    cpu = None
+    if not args.no_cpu:
+        # NumPy, single-threaded, one warm pass then the best of three passes
+        # over the whole suite (about 10-20 s of CPU work)
+        best = None
+        for _ in range(4):
+            c0 = time.perf_counter()
+            for c in cases:
+                c['cpu']()
+            dt = time.perf_counter() - c0
+            best = dt if best is None else min(best, dt)
+        try:
+            model = [l.split(':', 1)[1].strip() for l in open('/proc/cpuinfo')
+                     if l.startswith('model name')][0]
+        except Exception:
+            model = 'unknown'
+        cpu = {'value': round(total_bytes / best / 1e9, 2), 'unit': 'GB/s', 'cores': 1,
+               'kind': 'port',
+               'sample': 'one full pass of the same 13 operations with NumPy %s on the host '
+                         '(best of 3 after a warm pass, outputs preallocated where NumPy allows); '
+                         '%d host cores visible, CPU: %s' % (np.__version__, os.cpu_count(), model),
+               'seconds_per_pass': round(best, 3)}
+
+    result = {
+        'metric': 'achieved HBM GB/s (elementwise + reduction suite, algorithmic bytes / time)',
+        'value': round(value, 1),
+        'unit': 'GB/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': round(step_s * 1e3, 4),
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'f32/f64/f16/i32 (the element types of the five configurations)',
+        'data': 'synthetic (seeded NumPy RNG, uploaded once)',
+        'config': {'workload': 'C1-C5 of BASELINE.json at full shapes, 13 operations per step'
+                   if args.scale == 1 and not args.only else
+                   'REDUCED run (scale=%d only=%r): not the benchmark figure' % (args.scale, args.only),
+                   'bytes_per_step': total_bytes, 'operations': len(cases)},
+        'frac_of_hbm_peak': round(value / HBM_PEAK_GBPS, 4),
+        'parity_ok': all(parity.values()),
+        'roofline': roof,
+        'cpu_baseline': cpu,
+        'per_config': per_config,
+    }
+    if not args.no_detail:
+        result['launch_us'] = launch_latency(cp)
+    print(json.dumps(result))
+
+
+if __name__ == '__main__':
+    main()

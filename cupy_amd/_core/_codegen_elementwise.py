@@ -401,8 +401,14 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     src.append('  const %s _ntr = (_nr + %d) / %d;' % (idx_t, tile - 1, tile))
     src.append('  const %s _ntc = (_nc + %d) / %d;' % (idx_t, tile - 1, tile))
     src.append('  for (%s _tile = blockIdx.x; _tile < _ntr * _ntc; _tile += gridDim.x) {' % idx_t)
-    src.append('    const %s _r0 = (_tile / _ntc) * %d;' % (idx_t, tile))
-    src.append('    const %s _c0 = (_tile %% _ntc) * %d;' % (idx_t, tile))
+    # Diagonal tile order: consecutive workgroups differ in both the row block
+    # and the column block.  With power-of-two pitches, walking along one axis
+    # only would keep the low address bits of either the transposed reads or the
+    # row-major accesses identical across all concurrently running workgroups,
+    # and with them the memory channel.
+    src.append('    const %s _tr = _tile %% _ntr;' % idx_t)
+    src.append('    const %s _r0 = _tr * %d;' % (idx_t, tile))
+    src.append('    const %s _c0 = ((_tile / _ntr + _tr) %% _ntc) * %d;' % (idx_t, tile))
     if c_ops:
         # Stage transposed operands: walk the tile with rows as the fast
         # direction.  Thread (ty, tx): rows r0 + tx*vec .. +vec, column c0 + ty (+TY..).

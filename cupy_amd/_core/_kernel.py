@@ -17,6 +17,7 @@ from cupy_amd._core import _carray
 from cupy_amd._core import _codegen_elementwise as _cg
 from cupy_amd._core import _fusion_thread_local
 from cupy_amd._core import _scalar
+from cupy_amd._core import _tuning
 from cupy_amd._core import internal
 from cupy_amd._core._dtype import get_dtype, _raise_if_invalid_cast
 from cupy_amd._core._scalar import CScalar, get_typename as _get_typename
@@ -323,14 +324,6 @@ def _grid_limit(dev_id, blocks_per_cu):
     return g
 
 
-# Tunables of the flat elementwise kernel (vectors per thread per trip, resident
-# workgroups per CU the grid is capped at, non-temporal hint).
-FLAT_UNROLL = 2
-FLAT_BLOCKS_PER_CU = 16
-FLAT_STREAM_HINT = True
-TILED_BLOCKS_PER_CU = 8
-
-
 class _ElementwisePlanner:
     """Builds, memoises and launches the kernels of one elementwise operation
     (an ElementwiseKernel, or one loop of a ufunc)."""
@@ -454,20 +447,22 @@ class _ElementwisePlanner:
         if size < vec * 64:
             vec = 1
         idx64 = size > _INT32_MAX - (1 << 24)
-        unroll = FLAT_UNROLL if vec > 1 else 1
+        unroll = _tuning.get('flat_unroll') if vec > 1 else 1
+        block = _tuning.get('flat_block')
+        stream_hint = _tuning.get('flat_stream')
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
         if self._uses_ind:
             operands.append(_cg.Operand('indexer', '_ind', '', ndim=1,
                                         index_32=not idx64))
         key = ('flat', tuple(o.key() for o in operands), typedefs, vec, unroll,
-               idx64, tuple(bcast), dev_id)
+               idx64, tuple(bcast), dev_id, block, stream_hint)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
             code = _cg.emit_flat(
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, vec=vec, unroll=unroll,
-                idx64=idx64, bcast=tuple(bcast), stream_hint=FLAT_STREAM_HINT)
+                idx64=idx64, bcast=tuple(bcast), stream_hint=stream_hint, block=block)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             fmt = self._arg_format(operands, 'q' if idx64 else 'i', flat=True)
             entry = (fn, struct.Struct(fmt), code)
@@ -481,10 +476,10 @@ class _ElementwisePlanner:
             vals.extend((size, size, 0))
         blob = packer.pack(*vals)
         nvec = size // vec
-        per_block = _cg.BLOCK * unroll
+        per_block = block * unroll
         grid = max(1, min((max(nvec, size - nvec * vec) + per_block - 1) // per_block,
-                          _grid_limit(dev_id, FLAT_BLOCKS_PER_CU)))
-        fn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+                          _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu'))))
+        fn.launch_packed((grid, 1, 1), (block, 1, 1), blob, 0, stream_ptr)
 
     def _flat_values(self, args):
         """Argument values for kernels that take plain pointers: data pointer
@@ -600,15 +595,16 @@ class _ElementwisePlanner:
             span = max(span, abs(cs[0]) * nr + abs(cs[1]) * nc)
         idx64 = span > _INT32_MAX or nr * nc > _INT32_MAX
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
+        stream_hint = _tuning.get('tiled_stream')
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
-               tuple(sorted(layouts.items())), dev_id)
+               tuple(sorted(layouts.items())), dev_id, stream_hint)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
             code = _cg.emit_tiled2d(
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
-                tile=tile, idx64=idx64, stream_hint=FLAT_STREAM_HINT)
+                tile=tile, idx64=idx64, stream_hint=stream_hint)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']

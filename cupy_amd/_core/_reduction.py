@@ -20,6 +20,7 @@ from cupy_amd import _dryrun
 from cupy_amd._core import _carray
 from cupy_amd._core import _codegen_reduction as _cg
 from cupy_amd._core import _kernel
+from cupy_amd._core import _tuning
 from cupy_amd._core import internal
 from cupy_amd._core._codegen_elementwise import uses_identifier
 from cupy_amd._core._dtype import get_dtype
@@ -35,14 +36,6 @@ from cupy_amd.cuda import memory as _memory
 from cupy_amd.cuda import stream as _stream
 
 _INT32_MAX = (1 << 31) - 1
-
-# Tunables: workgroups a launch should at least consist of, as a multiple of
-# the CU count, before the reduce axis is split across workgroups.
-TARGET_BLOCKS_PER_CU = 8
-MIN_BLOCKS_PER_CU = 2
-ROWS_BLOCK_MODE_BYTES = 16384   # rows at least this long get a whole workgroup
-ROWS_STREAM_HINT = False
-COLS_STREAM_HINT = False
 
 
 def _get_axis(axis, ndim):
@@ -421,15 +414,15 @@ class _AbstractReductionKernel:
         max_item = max(a.dtype.itemsize for a in ins)
         lanes_needed = (n_red + vec - 1) // vec
         # geometry
-        if n_red * max_item >= ROWS_BLOCK_MODE_BYTES:
+        if n_red * max_item >= _tuning.get('rows_block_mode_bytes'):
             group = _cg.BLOCK
         else:
             group = max(1, min(64, internal.clp2(lanes_needed)))
         n_split = 1
         chunk = n_red
-        if group == _cg.BLOCK and n_out < cus * MIN_BLOCKS_PER_CU:
+        if group == _cg.BLOCK and n_out < cus * _tuning.get('min_blocks_per_cu'):
             trip = _cg.BLOCK * vec
-            want = (cus * TARGET_BLOCKS_PER_CU + n_out - 1) // n_out
+            want = (cus * _tuning.get('target_blocks_per_cu') + n_out - 1) // n_out
             most = max(1, n_red // (trip * 4))
             n_split = max(1, min(want, most, 65535))
             if n_split > 1:
@@ -440,24 +433,51 @@ class _AbstractReductionKernel:
         span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
                    + [abs(s) * n_out for s in so_out] + [n_red + chunk])
         idx64 = span > _INT32_MAX - (1 << 24)
-        rargs = self._rargs(in_args, out_args, bcast_r=bcast_r)
+        batch = _tuning.get('rows_batch')
+        trips = 1
+        batched = (group < _cg.BLOCK and batch >= 1 and n_red <= group * vec
+                   and n_out >= 4 * batch and _tuning.get('rows_trips') >= 1)
+        if batched:
+            # Fewer lanes per row with several loads per lane shorten the
+            # cross-lane butterfly; several rows per group keep loads in
+            # flight.  Both are bounded by a budget of bytes (registers) per
+            # lane.
+            per_trip = sum(vec * a.dtype.itemsize for a, s_o in zip(ins, so_in)
+                           if not (s_o == 0 and n_out > 1))
+            budget = _tuning.get('rows_lane_bytes')
+            while (trips * 2 <= _tuning.get('rows_trips') and group >= 2
+                   and per_trip * trips * 2 <= budget):
+                trips *= 2
+                group //= 2
+            batch = max(1, min(batch, budget // max(1, per_trip * trips)))
+        bcast_o = [(s == 0 and n_out > 1) for s in so_in] if batched else None
+        rargs = self._rargs(in_args, out_args, bcast_r=bcast_r, bcast_o=bcast_o)
         key = ('rows', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
-               post_map_expr, reduce_type, group, vec, idx64, partial, device_id)
+               post_map_expr, reduce_type, group, vec, idx64, partial, device_id,
+               batched, trips, _tuning.signature())
 
         def emit():
+            if batched:
+                return self.name, _cg.emit_rows_batched(
+                    self.name, rargs, self.identity, map_expr, reduce_expr,
+                    post_map_expr, reduce_type, typedefs, preamble, group=group,
+                    vec=vec, trips=trips, batch=batch, idx64=idx64,
+                    stream_hint=_tuning.get('rows_stream'))
             return self.name, _cg.emit_rows(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, group=group,
                 vec=vec, idx64=idx64, partial_out=partial,
-                stream_hint=ROWS_STREAM_HINT)
+                stream_hint=_tuning.get('rows_stream'),
+                unroll=_tuning.get('rows_unroll'))
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
         if group == _cg.BLOCK:
             gx = min(n_out, 0x7fffffff)
         else:
-            rows_per_block = _cg.BLOCK // group
-            gx = min((n_out + rows_per_block - 1) // rows_per_block, cus * 64)
+            rows_per_block = _cg.BLOCK // group * (batch if batched else 1)
+            gx = min((n_out + rows_per_block - 1) // rows_per_block,
+                     cus * _tuning.get('rows_group_rows_per_lane'))
         if partial:
             rsize = self._reduce_type_size(reduce_type, mod)
             partials = _memory.alloc(rsize * n_split * n_out)
@@ -495,7 +515,7 @@ class _AbstractReductionKernel:
         tx = max(1, min(64, internal.clp2((n_out + vec - 1) // vec)))
         ty = _cg.BLOCK // tx
         gx = (n_out + tx * vec - 1) // (tx * vec)
-        want = (cus * TARGET_BLOCKS_PER_CU + gx - 1) // gx
+        want = (cus * _tuning.get('target_blocks_per_cu') + gx - 1) // gx
         most = max(1, n_red // (ty * 8))
         n_split = max(1, min(want, most, 65535))
         partial = n_split > 1
@@ -504,13 +524,15 @@ class _AbstractReductionKernel:
         idx64 = span > _INT32_MAX - (1 << 24)
         rargs = self._rargs(in_args, out_args, bcast_o=bcast_o)
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
-               post_map_expr, reduce_type, tx, vec, idx64, partial, device_id)
+               post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
+               _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
-                idx64=idx64, partial_out=partial, stream_hint=COLS_STREAM_HINT)
+                idx64=idx64, partial_out=partial,
+                stream_hint=_tuning.get('cols_stream'), unroll=_tuning.get('cols_unroll'))
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
@@ -556,7 +578,7 @@ class _AbstractReductionKernel:
         tx = max(1, min(64, internal.flp2(tx), internal.clp2(n_out)))
         ty = _cg.BLOCK // tx
         gx = min((n_out + tx - 1) // tx, 0x7fffffff)
-        want = (cus * TARGET_BLOCKS_PER_CU + gx - 1) // gx
+        want = (cus * _tuning.get('target_blocks_per_cu') + gx - 1) // gx
         most = max(1, n_red // (ty * 8))
         n_split = max(1, min(want, most, 65535))
         partial = n_split > 1

@@ -15,7 +15,7 @@ template <typename T>
 struct min_max_st {
   T value;
   IndexT index;
-  __device__ min_max_st() : index(-1) {}
+  __device__ min_max_st() : value(), index(-1) {}
   __device__ min_max_st(T v) : value(v), index(0) {}
   __device__ min_max_st(T v, IndexT i) : value(v), index(i) {}
 };
@@ -26,30 +26,104 @@ template <> __device__ __forceinline__ bool _mm_isnan<double>(double x) { return
 template <> __device__ __forceinline__ bool _mm_isnan<float16>(float16 x) { return x.isnan(); }
 
 // kMax: larger values win, otherwise smaller ones; kNan: NaN wins over numbers.
-// `index == -1` marks "no element yet".
+// `index == -1` marks "no element yet".  Written with selects on the members
+// (no control flow, operands by value) so that everything stays in registers.
 template <bool kMax, bool kNan, typename T>
-__device__ __forceinline__ min_max_st<T> _mm_pick(
-    const min_max_st<T>& a, const min_max_st<T>& b) {
-  if (a.index == -1) return b;
-  if (b.index == -1) return a;
-  bool a_first;   // a strictly better than b
-  bool tie;
+__device__ __forceinline__ min_max_st<T> _mm_pick(min_max_st<T> a, min_max_st<T> b) {
+  const bool a_valid = a.index != -1;
+  const bool b_valid = b.index != -1;
+  bool a_better = kMax ? (a.value > b.value) : (a.value < b.value);
+  bool tie = a.value == b.value;
   if (kNan) {
     const bool an = _mm_isnan(a.value), bn = _mm_isnan(b.value);
-    if (an | bn) {
-      a_first = an & !bn;
-      tie = an & bn;
-    } else {
-      a_first = kMax ? (a.value > b.value) : (a.value < b.value);
-      tie = a.value == b.value;
-    }
-  } else {
-    a_first = kMax ? (a.value > b.value) : (a.value < b.value);
-    tie = a.value == b.value;
+    a_better = (an & !bn) | (!an & !bn & a_better);
+    tie = tie | (an & bn);
   }
-  if (tie) return (a.index <= b.index) ? a : b;
-  return a_first ? a : b;
+  bool take_a = a_better | (tie & (a.index <= b.index));
+  take_a = (take_a & a_valid) | !b_valid;
+  min_max_st<T> r;
+  r.value = take_a ? a.value : b.value;
+  r.index = take_a ? a.index : b.index;
+  return r;
 }
+
+// ---- argmin / argmax state ---------------------------------------------------
+// For element types of at most 32 bits (and 32-bit reduce indices) value and
+// index are packed into one signed 64-bit key: the high word is an
+// order-preserving image of the value (NaN mapped to the winning extreme), the
+// low word orders equal values by index so that the smallest index wins.  The
+// whole combine is then a 64-bit max or min.  Wider types use (value, index).
+template <typename T> struct _arg_small { static const bool value = false; };
+template <> struct _arg_small<bool> { static const bool value = true; };
+template <> struct _arg_small<signed char> { static const bool value = true; };
+template <> struct _arg_small<unsigned char> { static const bool value = true; };
+template <> struct _arg_small<short> { static const bool value = true; };
+template <> struct _arg_small<unsigned short> { static const bool value = true; };
+template <> struct _arg_small<int> { static const bool value = true; };
+template <> struct _arg_small<unsigned int> { static const bool value = true; };
+template <> struct _arg_small<float> { static const bool value = true; };
+template <> struct _arg_small<float16> { static const bool value = true; };
+
+template <bool kMax> __device__ __forceinline__ int _arg_ord(bool v) { return v ? 1 : 0; }
+template <bool kMax> __device__ __forceinline__ int _arg_ord(signed char v) { return v; }
+template <bool kMax> __device__ __forceinline__ int _arg_ord(unsigned char v) { return v; }
+template <bool kMax> __device__ __forceinline__ int _arg_ord(short v) { return v; }
+template <bool kMax> __device__ __forceinline__ int _arg_ord(unsigned short v) { return v; }
+template <bool kMax> __device__ __forceinline__ int _arg_ord(int v) { return v; }
+template <bool kMax> __device__ __forceinline__ int _arg_ord(unsigned int v) {
+  return static_cast<int>(v ^ 0x80000000u);
+}
+template <bool kMax> __device__ __forceinline__ int _arg_ord(float v) {
+  if (v != v) return kMax ? 0x7fffffff : (-0x7fffffff - 1);
+  v = v + 0.0f;                                  // -0 and +0 must tie
+  const int b = __builtin_bit_cast(int, v);
+  return b ^ ((b >> 31) & 0x7fffffff);
+}
+template <bool kMax> __device__ __forceinline__ int _arg_ord(float16 v) {
+  return _arg_ord<kMax>(static_cast<float>(v));
+}
+
+template <typename T, bool kMax>
+struct arg_key32 {
+  long long k;
+  __device__ arg_key32() : k(kMax ? (-9223372036854775807LL - 1) : 9223372036854775807LL) {}
+  __device__ arg_key32(T v, IndexT i) {
+    const unsigned int low = kMax ? static_cast<unsigned int>(0x7fffffff - static_cast<int>(i))
+                                  : static_cast<unsigned int>(i);
+    k = static_cast<long long>(
+        (static_cast<unsigned long long>(static_cast<unsigned int>(_arg_ord<kMax>(v))) << 32) | low);
+  }
+  __device__ __forceinline__ IndexT index() const {
+    const int low = static_cast<int>(static_cast<unsigned int>(k & 0xffffffffLL));
+    return kMax ? (0x7fffffff - low) : low;
+  }
+};
+template <typename T, bool kMax>
+__device__ __forceinline__ arg_key32<T, kMax> arg_pick(arg_key32<T, kMax> a, arg_key32<T, kMax> b) {
+  arg_key32<T, kMax> r;
+  r.k = kMax ? (a.k > b.k ? a.k : b.k) : (a.k < b.k ? a.k : b.k);
+  return r;
+}
+
+template <typename T, bool kMax>
+struct arg_wide {
+  min_max_st<T> s;
+  __device__ arg_wide() {}
+  __device__ arg_wide(T v, IndexT i) : s(v, i) {}
+  __device__ __forceinline__ IndexT index() const { return s.index; }
+};
+template <typename T, bool kMax>
+__device__ __forceinline__ arg_wide<T, kMax> arg_pick(arg_wide<T, kMax> a, arg_wide<T, kMax> b) {
+  arg_wide<T, kMax> r;
+  r.s = _mm_pick<kMax, true>(a.s, b.s);
+  return r;
+}
+
+template <typename T, bool kMax>
+struct arg_state {
+  typedef typename cupy::conditional<(_arg_small<T>::value && sizeof(IndexT) == 4),
+                                     arg_key32<T, kMax>, arg_wide<T, kMax> >::type type;
+};
 
 template <typename T> __device__ __forceinline__ min_max_st<T> my_min(
     const min_max_st<T>& a, const min_max_st<T>& b) { return _mm_pick<false, false>(a, b); }
@@ -92,26 +166,19 @@ _amax = create_reduction_func(
      'min_max_st<type_in0_raw>'),
     None, _min_max_preamble)
 
-_arg_sigs = tuple('{}->{}'.format(d, r) for r in 'qlihb' for d in '?bBhHiIlLqQ')
+_arg_sigs = tuple('{}->{}'.format(d, r) for r in 'qlihb' for d in '?bBhHiIlLqQ') + (
+    'e->q', 'f->q', 'd->q')
 
 _argmin = create_reduction_func(
-    'cupy_argmin',
-    _arg_sigs + (
-        ('e->q', (None, 'my_argmin_float(a, b)', None, None)),
-        ('f->q', (None, 'my_argmin_float(a, b)', None, None)),
-        ('d->q', (None, 'my_argmin_float(a, b)', None, None))),
-    ('min_max_st<type_in0_raw>(in0, _J)', 'my_argmin(a, b)', 'out0 = a.index',
-     'min_max_st<type_in0_raw>'),
+    'cupy_argmin', _arg_sigs,
+    ('arg_state<type_in0_raw, false>::type(in0, _J)', 'arg_pick(a, b)',
+     'out0 = a.index()', 'arg_state<type_in0_raw, false>::type'),
     None, _min_max_preamble, sort_reduce_axis=False)
 
 _argmax = create_reduction_func(
-    'cupy_argmax',
-    _arg_sigs + (
-        ('e->q', (None, 'my_argmax_float(a, b)', None, None)),
-        ('f->q', (None, 'my_argmax_float(a, b)', None, None)),
-        ('d->q', (None, 'my_argmax_float(a, b)', None, None))),
-    ('min_max_st<type_in0_raw>(in0, _J)', 'my_argmax(a, b)', 'out0 = a.index',
-     'min_max_st<type_in0_raw>'),
+    'cupy_argmax', _arg_sigs,
+    ('arg_state<type_in0_raw, true>::type(in0, _J)', 'arg_pick(a, b)',
+     'out0 = a.index()', 'arg_state<type_in0_raw, true>::type'),
     None, _min_max_preamble, sort_reduce_axis=False)
 
 

@@ -1,0 +1,49 @@
+"""Launch-geometry and code-shape parameters of the emitters, in one place.
+
+The values are the result of measurements on MI355X (256 CUs, wave64, HBM3E):
+streaming kernels do best with one 16-byte access per operand in flight per
+thread (more unrolling lowers the achieved bandwidth), non-temporal accesses,
+and grids large enough that every CU always has several workgroups queued.
+``set(**kw)`` changes a parameter for experiments; kernels are re-planned
+because ``signature()`` is part of every kernel memo key.
+"""
+
+_params = {
+    # flat elementwise kernel
+    'flat_block': 1024,         # threads per workgroup
+    'flat_unroll': 1,           # vectors per thread per trip
+    'flat_blocks_per_cu': 64,   # grid cap, in workgroups per CU
+    'flat_stream': True,        # non-temporal loads/stores
+    # tiled 2-d elementwise kernel
+    'tiled_stream': True,
+    # reductions
+    'rows_stream': True,
+    'rows_unroll': 1,
+    'rows_block_mode_bytes': 32768,   # row length from which a workgroup owns a row
+    'rows_batch': 2,            # short rows handled per lane group at a time
+    'rows_trips': 4,            # ... with up to this many vector loads per lane and row
+    'rows_lane_bytes': 128,     # ... and at most this many bytes in flight per lane
+    'rows_group_rows_per_lane': 64,   # grid cap for sub-wave groups: CUs * this workgroups
+    'cols_stream': True,
+    'cols_unroll': 4,
+    'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
+    'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
+}
+_signature = tuple(sorted(_params.items()))
+
+
+def get(name):
+    return _params[name]
+
+
+def set(**kw):
+    global _signature
+    for k, v in kw.items():
+        if k not in _params:
+            raise KeyError(k)
+        _params[k] = v
+    _signature = tuple(sorted(_params.items()))
+
+
+def signature():
+    return _signature

@@ -188,12 +188,15 @@ def test_launch_plans_of_the_benchmark_shapes():
     saxpy = cp.ElementwiseKernel('float32 x, float32 y, float32 a', 'float32 z',
                                  'z = a * x + y', 'saxpy')
     (l,) = launches_of(lambda: saxpy(x, x, 2.5))
-    assert l[0] == 'saxpy' and l[2] == (256, 1, 1)
+    assert l[0] == 'saxpy' and l[2][0] in (256, 512, 1024)
     assert 'load_vec<float, 4' in saxpy.cached_code
 
-    a = cp.ndarray((2048, 4096), np.float32)
+    a = cp.ndarray((2048, 16384), np.float32)
     (l,) = launches_of(lambda: a.sum(axis=1))
-    assert l[1] == (2048, 1, 1)                       # a workgroup per row
+    assert l[1] == (2048, 1, 1)                       # a workgroup per long row
+    b = cp.ndarray((2048, 1024), np.float32)
+    (l,) = launches_of(lambda: b.sum(axis=1))
+    assert l[1] == (512, 1, 1)                        # a wave per shorter row
     ls = launches_of(lambda: a.sum(axis=0))
     assert [x[0] for x in ls] == ['cupy_sum', 'cupy_sum_combine'] and ls[0][1][1] > 1
     ls = launches_of(lambda: a.sum())
