@@ -347,33 +347,37 @@ def emit_generic(name, operands, operation, typedefs='', preamble='',
 
 
 def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
-                 loop_prep='', after_loop='', layouts=None, vec=4, tile=64,
-                 idx64=False, stream_hint=True):
+                 loop_prep='', after_loop='', layouts=None, vec=4, tile_r=64,
+                 tile_c=64, threads=256, idx64=False, stream_hint=True):
     """Kernel for a 2-d index space (rows r, columns c) where every array
-    operand is contiguous along one axis.
+    operand is contiguous along one of the axes.
 
-    ``layouts[name]`` is 'R' (unit or zero stride along columns; any stride
-    along rows) or 'C' (unit stride along rows, any stride along columns: a
-    transposed operand).  'C' inputs are staged through an LDS tile: the tile is
-    read from memory along rows (coalesced) and consumed along columns.  Outputs
-    must be 'R'.
+    ``layouts[name]`` is
+      'R'   unit stride along columns, any stride (also 0) along rows;
+      'R0'  zero stride along columns (a value per row, broadcast over columns);
+      'C'   unit stride along rows, any stride along columns: a transposed
+            operand.  Inputs only.
+    'C' inputs are staged through an LDS tile: the tile is read from memory
+    along rows (coalesced) and consumed along columns.
 
-    Work split: a workgroup of 256 threads owns a ``tile`` x ``tile`` block.
-    For 'R' operands thread (ty, tx) handles ``vec`` consecutive columns
-    starting at tx*vec of rows ty, ty+TY, ...  Kernel parameters after the
-    operands: ``_nr, _nc`` (extent), then per array its row stride and column
-    stride in elements.
+    Work split: a workgroup of ``threads`` threads owns a ``tile_r`` x ``tile_c``
+    block; tiles are visited in diagonal order.  Every thread handles ``vec``
+    consecutive elements (along rows when staging, along columns otherwise).
+    Interior tiles take an unguarded, fully vectorised path, edge tiles a guarded
+    scalar one.  Kernel parameters after the operands: ``_nr, _nc``, then per
+    array its row stride and column stride in elements.
     """
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     arrays = [op for op in operands if op.kind == 'array']
     needs_ind = any(op.kind == 'indexer' for op in operands)
-    tx_n = tile // vec            # threads across the columns of a tile
-    ty_n = BLOCK // tx_n          # rows covered per pass
-    passes = tile // ty_n
-    assert tx_n * ty_n == BLOCK and passes * ty_n == tile
     nt = 'true' if stream_hint else 'false'
     use_i = uses_identifier(operation, 'i')
     set_ind = '_ind.set(i);' if needs_ind and uses_identifier(operation, '_ind') else ''
+    assert tile_r % vec == 0 and tile_c % vec == 0
+    n_stage = (tile_r // vec) * tile_c          # staging vectors per tile
+    n_work = tile_r * (tile_c // vec)           # compute vectors per tile
+    assert n_stage % threads == 0 and n_work % threads == 0
+    pitch = tile_c + 1                          # odd pitch: column walks spread over banks
 
     parts = [_param_decl(op) for op in operands if op.kind != 'indexer']
     parts += ['const %s _nr' % idx_t, 'const %s _nc' % idx_t]
@@ -387,19 +391,18 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     for op in c_ops:
         assert not op.is_out, 'transposed outputs are not handled by tiled2d'
 
+    def gaddr(op, r, c):
+        return '(_p_%s + (ptrdiff_t)(%s) * _sr_%s + (ptrdiff_t)(%s) * _sc_%s)' % (
+            op.name, r, op.name, c, op.name)
+
     src = [_header(typedefs, preamble)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
-        BLOCK, name, params))
+        threads, name, params))
     src.append('  %s;' % loop_prep)
     for op in c_ops:
-        # +1 element of padding per tile row keeps the column-wise reads off a
-        # single LDS bank.
-        src.append('  __shared__ %s _t_%s[%d][%d];' % (
-            op.store_t, op.name, tile, tile + 1))
-    src.append('  const int _tx = threadIdx.x %% %d;' % tx_n)
-    src.append('  const int _ty = threadIdx.x / %d;' % tx_n)
-    src.append('  const %s _ntr = (_nr + %d) / %d;' % (idx_t, tile - 1, tile))
-    src.append('  const %s _ntc = (_nc + %d) / %d;' % (idx_t, tile - 1, tile))
+        src.append('  __shared__ %s _t_%s[%d];' % (op.store_t, op.name, tile_r * pitch))
+    src.append('  const %s _ntr = (_nr + %d) / %d;' % (idx_t, tile_r - 1, tile_r))
+    src.append('  const %s _ntc = (_nc + %d) / %d;' % (idx_t, tile_c - 1, tile_c))
     src.append('  for (%s _tile = blockIdx.x; _tile < _ntr * _ntc; _tile += gridDim.x) {' % idx_t)
     # Diagonal tile order: consecutive workgroups differ in both the row block
     # and the column block.  With power-of-two pitches, walking along one axis
@@ -407,99 +410,100 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     # row-major accesses identical across all concurrently running workgroups,
     # and with them the memory channel.
     src.append('    const %s _tr = _tile %% _ntr;' % idx_t)
-    src.append('    const %s _r0 = _tr * %d;' % (idx_t, tile))
-    src.append('    const %s _c0 = ((_tile / _ntr + _tr) %% _ntc) * %d;' % (idx_t, tile))
+    src.append('    const %s _r0 = _tr * %d;' % (idx_t, tile_r))
+    src.append('    const %s _c0 = ((_tile / _ntr + _tr) %% _ntc) * %d;' % (idx_t, tile_c))
+    src.append('    const bool _interior = (_r0 + %d <= _nr) && (_c0 + %d <= _nc);' % (
+        tile_r, tile_c))
     if c_ops:
-        # Stage transposed operands: walk the tile with rows as the fast
-        # direction.  Thread (ty, tx): rows r0 + tx*vec .. +vec, column c0 + ty (+TY..).
-        src.append('    {')
-        src.append('      const %s _rr = _r0 + _tx * %d;' % (idx_t, vec))
-        src.append('      const bool _rfull = _rr + %d <= _nr;' % vec)
+        # ---- stage transposed operands: rows are the fast direction -------------------
+        src.append('    if (_interior) {')
         src.append('#pragma unroll')
-        src.append('      for (int _p = 0; _p < %d; ++_p) {' % passes)
-        src.append('        const %s _cc = _c0 + _ty + _p * %d;' % (idx_t, ty_n))
-        src.append('        if (_cc < _nc) {')
+        src.append('      for (int _it = 0; _it < %d; ++_it) {' % (n_stage // threads))
+        src.append('        const int _v = threadIdx.x + _it * %d;' % threads)
+        src.append('        const int _lr = (_v %% %d) * %d;' % (tile_r // vec, vec))
+        src.append('        const int _lc = _v / %d;' % (tile_r // vec))
         for op in c_ops:
-            src.append('          if (_rfull) {')
-            src.append('            cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>('
-                       '_p_%s + _rr + (ptrdiff_t)_cc * _sc_%s);' % (
-                           op.store_t, vec, op.store_t, vec, nt, op.name, op.name))
+            src.append('        { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s);' % (
+                op.store_t, vec, op.store_t, vec, nt, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
             src.append('#pragma unroll')
-            src.append('            for (int _k = 0; _k < %d; ++_k) '
-                       '_t_%s[_tx * %d + _k][_ty + _p * %d] = _lv.v[_k];' % (
-                           vec, op.name, vec, ty_n))
-            src.append('          } else {')
-            src.append('            for (int _k = 0; _k < %d; ++_k) if (_rr + _k < _nr) '
-                       '_t_%s[_tx * %d + _k][_ty + _p * %d] = '
-                       '_p_%s[_rr + _k + (ptrdiff_t)_cc * _sc_%s];' % (
-                           vec, op.name, vec, ty_n, op.name, op.name))
-            src.append('          }')
+            src.append('          for (int _k = 0; _k < %d; ++_k) '
+                       '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (vec, op.name, pitch))
+        src.append('      }')
+        src.append('    } else {')
+        src.append('      for (int _v = threadIdx.x; _v < %d; _v += %d) {' % (
+            tile_r * tile_c, threads))
+        src.append('        const int _lr = _v %% %d;' % tile_r)
+        src.append('        const int _lc = _v / %d;' % tile_r)
+        src.append('        if (_r0 + _lr < _nr && _c0 + _lc < _nc) {')
+        for op in c_ops:
+            src.append('          _t_%s[_lr * %d + _lc] = *%s;' % (
+                op.name, pitch, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
         src.append('        }')
         src.append('      }')
         src.append('    }')
         src.append('    __syncthreads();')
-    # Consume: thread (ty, tx) handles row r0 + ty + p*TY, columns c0 + tx*vec ..
-    src.append('    const %s _cb = _c0 + _tx * %d;' % (idx_t, vec))
-    src.append('    const bool _cfull = _cb + %d <= _nc;' % vec)
-    src.append('#pragma unroll')
-    src.append('    for (int _p = 0; _p < %d; ++_p) {' % passes)
-    src.append('      const int _lr = _ty + _p * %d;' % ty_n)
-    src.append('      const %s _r = _r0 + _lr;' % idx_t)
-    src.append('      if (_r < _nr && _cb < _nc) {')
 
-    def r_ptr(op):
-        return '(_p_%s + (ptrdiff_t)_r * _sr_%s + (ptrdiff_t)_cb * _sc_%s)' % (
-            op.name, op.name, op.name)
-
-    # full-width path ------------------------------------------------------------------
-    src.append('        if (_cfull) {')
-    for op in arrays:
-        if layouts[op.name] == 'R':
-            if (not op.is_out) or op.read_out:
-                src.append('          cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
-                src.append('          if (_sc_%s == 1) _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
-                    op.name, op.name, op.store_t, vec, nt, r_ptr(op)))
-                src.append('          else { const %s _bv = *%s;' % (op.store_t, r_ptr(op)))
-                src.append('#pragma unroll')
-                src.append('            for (int _k = 0; _k < %d; ++_k) _l_%s.v[_k] = _bv; }' % (
-                    vec, op.name))
-            else:
-                src.append('          cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
-
+    # ---- consume: columns are the fast direction ----------------------------------------
     def full_load(op):
-        if layouts[op.name] == 'C':
-            return '_t_%s[_lr][_tx * %d + _k]' % (op.name, vec)
+        lay = layouts[op.name]
+        if lay == 'C':
+            return '_t_%s[_lr * %d + _lc + _k]' % (op.name, pitch)
+        if lay == 'R0':
+            return '_b_%s' % op.name
         return '_l_%s.v[_k]' % op.name
 
     def full_store(op, value):
         return '_l_%s.v[_k] = %s;' % (op.name, value)
 
+    src.append('    if (_interior) {')
     src.append('#pragma unroll')
-    src.append('          for (int _k = 0; _k < %d; ++_k) {' % vec)
+    src.append('      for (int _it = 0; _it < %d; ++_it) {' % (n_work // threads))
+    src.append('        const int _w = threadIdx.x + _it * %d;' % threads)
+    src.append('        const int _lc = (_w %% %d) * %d;' % (tile_c // vec, vec))
+    src.append('        const int _lr = _w / %d;' % (tile_c // vec))
+    src.append('        const %s _r = _r0 + _lr;' % idx_t)
+    src.append('        const %s _c = _c0 + _lc;' % idx_t)
+    for op in arrays:
+        lay = layouts[op.name]
+        if lay == 'R':
+            if (not op.is_out) or op.read_out:
+                src.append('        cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
+                    op.store_t, vec, op.name, op.store_t, vec, nt, gaddr(op, '_r', '_c')))
+            else:
+                src.append('        cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+        elif lay == 'R0':
+            src.append('        const %s _b_%s = *%s;' % (op.store_t, op.name, gaddr(op, '_r', '0')))
+    src.append('#pragma unroll')
+    src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
     if use_i or set_ind:
-        src.append('            const ptrdiff_t i = (ptrdiff_t)_r * _nc + _cb + _k; %s' % set_ind)
-    src.append(_element_code(operands, operation, full_load, full_store, 12))
-    src.append('          }')
+        src.append('          const ptrdiff_t i = (ptrdiff_t)_r * _nc + _c + _k; %s' % set_ind)
+    src.append(_element_code(operands, operation, full_load, full_store, 10))
+    src.append('        }')
     for op in arrays:
         if op.is_out:
-            src.append('          cupy::store_vec<%s, %d, %s>(%s, _l_%s);' % (
-                op.store_t, vec, nt, r_ptr(op), op.name))
-    src.append('        } else {')
+            src.append('        cupy::store_vec<%s, %d, %s>(%s, _l_%s);' % (
+                op.store_t, vec, nt, gaddr(op, '_r', '_c'), op.name))
+    src.append('      }')
+    src.append('    } else {')
 
-    # ragged right edge ----------------------------------------------------------------
     def edge_load(op):
-        if layouts[op.name] == 'C':
-            return '_t_%s[_lr][_tx * %d + _k]' % (op.name, vec)
-        return '%s[(ptrdiff_t)_k * _sc_%s]' % (r_ptr(op), op.name)
+        lay = layouts[op.name]
+        if lay == 'C':
+            return '_t_%s[_lr * %d + _lc]' % (op.name, pitch)
+        return '(*%s)' % gaddr(op, '_r', '_c')
 
     def edge_store(op, value):
-        return '%s[(ptrdiff_t)_k * _sc_%s] = %s;' % (r_ptr(op), op.name, value)
+        return '*%s = %s;' % (gaddr(op, '_r', '_c'), value)
 
-    src.append('          for (int _k = 0; _k < %d && _cb + _k < _nc; ++_k) {' % vec)
+    src.append('      for (int _w = threadIdx.x; _w < %d; _w += %d) {' % (tile_r * tile_c, threads))
+    src.append('        const int _lc = _w %% %d;' % tile_c)
+    src.append('        const int _lr = _w / %d;' % tile_c)
+    src.append('        const %s _r = _r0 + _lr;' % idx_t)
+    src.append('        const %s _c = _c0 + _lc;' % idx_t)
+    src.append('        if (_r < _nr && _c < _nc) {')
     if use_i or set_ind:
-        src.append('            const ptrdiff_t i = (ptrdiff_t)_r * _nc + _cb + _k; %s' % set_ind)
-    src.append(_element_code(operands, operation, edge_load, edge_store, 12))
-    src.append('          }')
+        src.append('          const ptrdiff_t i = (ptrdiff_t)_r * _nc + _c; %s' % set_ind)
+    src.append(_element_code(operands, operation, edge_load, edge_store, 10))
     src.append('        }')
     src.append('      }')
     src.append('    }')

@@ -410,9 +410,11 @@ class _ElementwisePlanner:
                 dev_id, args, nin, arrays, cstrides, size, var_types, typedefs,
                 casts, force_read_out, stream_ptr, kernel_name)
         if mode in ('tiled', 'tiled_t'):
-            return self._launch_tiled(
+            done = self._launch_tiled(
                 dev_id, args, nin, arrays, cshape, cstrides, var_types, typedefs,
                 casts, force_read_out, stream_ptr, kernel_name, mode == 'tiled_t')
+            if done is not None:
+                return
         return self._launch_generic(
             dev_id, args, nin, shape, var_types, typedefs, casts, force_read_out,
             stream_ptr, block_size or 128, kernel_name)
@@ -565,31 +567,50 @@ class _ElementwisePlanner:
         nr, nc = cshape
         layouts = {}
         itemsizes = [a.dtype.itemsize for a in arrays]
-        vec = _max_vector_width(itemsizes)
+        # the widest operand moves 16 bytes per thread, narrower ones less
+        vec = max(1, 16 // max(itemsizes))
         names = [p.name for a, p in zip(args, params)
                  if isinstance(a, ndarray) and not p.raw]
+        n_transposed = 0
+        lds_item = 0
         for a, cs, nm in zip(arrays, cstrides, names):
             item = a.dtype.itemsize
-            layouts[nm] = 'R' if (cs[1] == item or cs[1] == 0) else 'C'
+            if cs[1] == item:
+                layouts[nm] = 'R'
+            elif cs[1] == 0:
+                layouts[nm] = 'R0'
+            else:
+                layouts[nm] = 'C'
+                n_transposed += 1
+                lds_item += item
         # alignment of every vector access
         while vec > 1:
             ok = True
             for a, cs, nm in zip(arrays, cstrides, names):
                 item = a.dtype.itemsize
-                nb = min(16, vec * item)
+                nb = vec * item
+                if layouts[nm] == 'R0':
+                    continue
                 if not _aligned(a.data.ptr, nb):
                     ok = False
                 elif layouts[nm] == 'R':
-                    if cs[1] != 0 and cs[0] % nb:
+                    if cs[0] % nb:
                         ok = False
                 elif cs[1] % nb:
                     ok = False
             if ok:
                 break
             vec //= 2
-        tile = 64
-        if tile // vec > _cg.BLOCK:
-            vec = max(vec, tile // _cg.BLOCK)
+        # Large tiles give long contiguous runs in memory on both the transposed
+        # and the row-major side; they need the LDS for the staged operands.
+        if (nr >= 512 and nc >= 512 and lds_item * 128 * 129 <= 140 * 1024):
+            tile_r = tile_c = 128
+            threads = 1024
+        else:
+            tile_r = tile_c = 64
+            threads = 256
+        if lds_item * tile_r * (tile_c + 1) > 150 * 1024:
+            return None       # too many staged operands for the LDS
         span = 0
         for a, cs in zip(arrays, cstrides):
             span = max(span, abs(cs[0]) * nr + abs(cs[1]) * nc)
@@ -597,14 +618,16 @@ class _ElementwisePlanner:
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
         stream_hint = _tuning.get('tiled_stream')
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
-               tuple(sorted(layouts.items())), dev_id, stream_hint)
+               tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
+               threads)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
             code = _cg.emit_tiled2d(
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
-                tile=tile, idx64=idx64, stream_hint=stream_hint)
+                tile_r=tile_r, tile_c=tile_c, threads=threads, idx64=idx64,
+                stream_hint=stream_hint)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']
@@ -627,9 +650,10 @@ class _ElementwisePlanner:
             item = a.dtype.itemsize
             vals.extend((cs[0] // item, cs[1] // item))
         blob = packer.pack(*vals)
-        ntiles = ((nr + tile - 1) // tile) * ((nc + tile - 1) // tile)
+        ntiles = ((nr + tile_r - 1) // tile_r) * ((nc + tile_c - 1) // tile_c)
         grid = max(1, min(ntiles, 0x7fffffff))
-        fn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+        fn.launch_packed((grid, 1, 1), (threads, 1, 1), blob, 0, stream_ptr)
+        return True
 
     # -- generic ---------------------------------------------------------------------------
     def _launch_generic(self, dev_id, args, nin, shape, var_types, typedefs, casts,
