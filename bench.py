@@ -35,6 +35,26 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch (read + written) from the rocprofv3 FETCH_SIZE and
+# WRITE_SIZE counters, scaled by what the same counters read for the plain copy
+# kernel that --calibrate adds (2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE on this
+# device); the summary of those runs is profiles/pmc_traffic_bench_suite.md.
+# Operations that share a kernel name and launch shape with another one of a
+# different size cannot be told apart in the counter output and are left out.
+MEASURED_TRAFFIC_BYTES = {
+    'C1 saxpy f32 2^26': 536850563 + 268416769,
+    'C2a x.T*y f32(T)xf16 8192^2': 269876044 + 268504827,
+    'C2b tmp+1 f32 8192^2': 268438400 + 268477053,
+    'C3 sum float32 axis=1 16384^2': 1073664650 + 524252,
+    'C3 sum float64 axis=1 8192^2': 536847235 + 262126,
+    'C3 sum float32 axis=0 16384^2': 1073633294 + 2097006,
+    'C3 sum float32 axis=None 16384^2': 1073633294 + 2097006,
+    'C4 argmin i32 (2^20,128)': 536866305 + 8388344,
+    'C4 argmax i32 (2^20,128)': 536866305 + 8388344,
+    'C4 argmax f32 (2^16,4096)': 1073634573 + 524288,
+    'C5 fused sum((x-y)^2*w) f16 (2^18,256)': 268475643 + 1048503,
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -239,6 +259,9 @@ def main():
     ap.add_argument('--no-detail', action='store_true',
                     help='skip per-operation event timing and launch latency')
     ap.add_argument('--only', default='', help='run only cases whose name contains this')
+    ap.add_argument('--calibrate', action='store_true',
+                    help='add a plain copy kernel of known size (256 MiB in, 256 MiB out) to '
+                         'every step, as the yardstick for hardware traffic counters')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: every operation of this path runs on a '
@@ -256,9 +279,21 @@ def main():
         cases = [c for c in cases if args.only in c['name']]
     log('inputs ready in %.1f s' % (time.perf_counter() - t0))
 
+    calib = None
+    if args.calibrate:
+        n_cal = 1 << 26
+        cal_src = cp.zeros((n_cal,), np.float32)
+        cal_dst = cp.empty((n_cal,), np.float32)
+        cal_kernel = cp.ElementwiseKernel('T x', 'T y', 'y = x', 'calib_copy_256MiB')
+
+        def calib():
+            cal_kernel(cal_src, cal_dst)
+
     def step():
         for c in cases:
             c['gpu']()
+        if calib is not None:
+            calib()
 
     # warm-up (compiles / loads kernels, grows the pool)
     for _ in range(max(args.warmup, 1)):
@@ -297,7 +332,8 @@ def main():
         dom = max(per_config, key=lambda e: e['us'])
         roof = {'bound': 'hbm', 'kernel': dom['kernel'], 'operation': dom['name'],
                 'achieved': dom['gbps'], 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                'frac': dom['frac'], 'traffic': None,
+                'frac': dom['frac'],
+                'traffic': MEASURED_TRAFFIC_BYTES.get(dom['name']) if args.scale == 1 else None,
                 'launch_us': dom['us'], 'algorithmic_bytes': dom['bytes']}
     else:
         roof = {'bound': 'hbm', 'achieved': round(value, 1), 'peak': HBM_PEAK_GBPS,
