@@ -16,6 +16,7 @@ import numpy
 from cupy_amd._core import _carray
 from cupy_amd._core import _codegen_elementwise as _cg
 from cupy_amd._core import _fusion_thread_local
+from cupy_amd._core import _launch_plan
 from cupy_amd._core import _scalar
 from cupy_amd._core import _tuning
 from cupy_amd._core import internal
@@ -382,9 +383,10 @@ class _ElementwisePlanner:
 
     def launch(self, dev_id, args, nin, shape, var_types, typedefs, casts=None,
                force_generic=False, force_read_out=False, stream=None,
-               block_size=None, kernel_name=None):
+               block_size=None, kernel_name=None, rec=None):
         """Plans and launches.  ``args``: preprocessed inputs then outputs
-        (ndarrays already broadcast to ``shape``, CScalars already typed)."""
+        (ndarrays already broadcast to ``shape``, CScalars already typed).
+        ``rec``: optional recorder of the launch; argument ``i`` is ref ``i``."""
         params = self.params
         arrays = [a for a, p in zip(args, params)
                   if isinstance(a, ndarray) and not p.raw]
@@ -408,20 +410,21 @@ class _ElementwisePlanner:
         if mode == 'flat':
             return self._launch_flat(
                 dev_id, args, nin, arrays, cstrides, size, var_types, typedefs,
-                casts, force_read_out, stream_ptr, kernel_name)
+                casts, force_read_out, stream_ptr, kernel_name, rec)
         if mode in ('tiled', 'tiled_t'):
             done = self._launch_tiled(
                 dev_id, args, nin, arrays, cshape, cstrides, var_types, typedefs,
-                casts, force_read_out, stream_ptr, kernel_name, mode == 'tiled_t')
+                casts, force_read_out, stream_ptr, kernel_name, mode == 'tiled_t',
+                rec)
             if done is not None:
                 return
         return self._launch_generic(
             dev_id, args, nin, shape, var_types, typedefs, casts, force_read_out,
-            stream_ptr, block_size or 128, kernel_name)
+            stream_ptr, block_size or 128, kernel_name, rec)
 
     # -- flat ---------------------------------------------------------------------------
     def _launch_flat(self, dev_id, args, nin, arrays, cstrides, size, var_types,
-                     typedefs, casts, force_read_out, stream_ptr, kernel_name):
+                     typedefs, casts, force_read_out, stream_ptr, kernel_name, rec):
         params = self.params
         bcast = []
         itemsizes = []
@@ -472,30 +475,29 @@ class _ElementwisePlanner:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
         fn, packer, _ = entry
-        vals = self._flat_values(args)
-        vals.append(size)
+        block_args = self._flat_values(args)
+        block_args.const(size)
         if self._uses_ind:
-            vals.extend((size, size, 0))
-        blob = packer.pack(*vals)
+            block_args.const(size, size, 0)
         nvec = size // vec
         per_block = block * unroll
         grid = max(1, min((max(nvec, size - nvec * vec) + per_block - 1) // per_block,
                           _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu'))))
-        fn.launch_packed((grid, 1, 1), (block, 1, 1), blob, 0, stream_ptr)
+        _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
+                            stream_ptr)
 
     def _flat_values(self, args):
         """Argument values for kernels that take plain pointers: data pointer
         per iterated array, CArray fields per raw array, scalar values."""
-        out = []
-        for a, p in zip(args, self.params):
+        out = _launch_plan.ArgBlock()
+        for ref, (a, p) in enumerate(zip(args, self.params)):
             if isinstance(a, ndarray):
-                out.append(a.data.ptr)
+                out.ptr(ref, a.data.ptr)
                 if p.raw:
-                    out.append(a.size)
-                    out.extend(a._shape)
-                    out.extend(a._strides)
+                    out.const(a.size, *a._shape)
+                    out.const(*a._strides)
             else:
-                out.append(a._struct_value())
+                out.scalar(ref, a)
         return out
 
     def _arg_format(self, operands, idx_code, flat):
@@ -559,7 +561,8 @@ class _ElementwisePlanner:
         return 'generic'
 
     def _launch_tiled(self, dev_id, args, nin, arrays, cshape, cstrides, var_types,
-                      typedefs, casts, force_read_out, stream_ptr, kernel_name, swap):
+                      typedefs, casts, force_read_out, stream_ptr, kernel_name, swap,
+                      rec):
         params = self.params
         if swap:
             cshape = (cshape[1], cshape[0])
@@ -644,20 +647,20 @@ class _ElementwisePlanner:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
         fn, packer, _ = entry
-        vals = self._flat_values(args)
-        vals.extend((nr, nc))
+        block_args = self._flat_values(args)
+        block_args.const(nr, nc)
         for a, cs in zip(arrays, cstrides):
             item = a.dtype.itemsize
-            vals.extend((cs[0] // item, cs[1] // item))
-        blob = packer.pack(*vals)
+            block_args.const(cs[0] // item, cs[1] // item)
         ntiles = ((nr + tile_r - 1) // tile_r) * ((nc + tile_c - 1) // tile_c)
         grid = max(1, min(ntiles, 0x7fffffff))
-        fn.launch_packed((grid, 1, 1), (threads, 1, 1), blob, 0, stream_ptr)
+        _launch_plan.launch(rec, fn, (grid, 1, 1), (threads, 1, 1), packer, block_args,
+                            stream_ptr)
         return True
 
     # -- generic ---------------------------------------------------------------------------
     def _launch_generic(self, dev_id, args, nin, shape, var_types, typedefs, casts,
-                        force_read_out, stream_ptr, block_size, kernel_name):
+                        force_read_out, stream_ptr, block_size, kernel_name, rec):
         params = self.params
         arrays_idx = [i for i, (a, p) in enumerate(zip(args, params))
                       if isinstance(a, ndarray) and not p.raw]
@@ -697,26 +700,24 @@ class _ElementwisePlanner:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
         fn, packer, _ = entry
-        vals = []
-        for a in args:
+        block_args = _launch_plan.ArgBlock()
+        for ref, a in enumerate(args):
             if isinstance(a, ndarray):
-                vals.append(a.data.ptr)
-                vals.append(a.size)
-                vals.extend(a._shape)
-                vals.extend(a._strides)
+                block_args.ptr(ref, a.data.ptr)
+                block_args.const(a.size, *a._shape)
+                block_args.const(*a._strides)
             else:
-                vals.append(a._struct_value())
-        vals.append(indexer.size)
-        vals.extend(indexer.shape)
-        vals.extend((0,) * indexer.ndim)
-        blob = packer.pack(*vals)
+                block_args.scalar(ref, a)
+        block_args.const(indexer.size, *indexer.shape)
+        block_args.const(*((0,) * indexer.ndim))
         size = indexer.size
         block = max(1, min(block_size, size))
         # enough workgroups to fill the device several times over; the kernel
         # loops over what is left
         grid = max(1, min((size + block - 1) // block,
                           _grid_limit(dev_id, 32) * max(1, 256 // block)))
-        fn.launch_packed((grid, 1, 1), (block, 1, 1), blob, 0, stream_ptr)
+        _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
+                            stream_ptr)
 
     def _remember_code(self, args, code):
         in_types = tuple(a.dtype for a in args if isinstance(a, ndarray))
@@ -804,6 +805,7 @@ class ElementwiseKernel:
             name, self.in_params + self.out_params, operation, preamble,
             loop_prep, after_loop, options, is_ufunc=False)
         self._cached_codes = self._planner._codes
+        self._fast_calls = {}
 
     def __call__(self, *args, **kwargs):
         """Compiles (if needed) and launches the kernel.
@@ -829,11 +831,20 @@ class ElementwiseKernel:
                 'Wrong number of arguments for {!r}. '
                 'It must be either {} or {} (with outputs), '
                 'but given {}.'.format(self.name, self.nin, self.nargs, n_args))
+        dev_id = _device.get_device_id()
+        # A call that looks like an earlier one replays that call's launch.
+        fast_key = rec = None
+        if size == -1 and stream is None and block_size == 128:
+            fast_key = _launch_plan.call_signature(args, dev_id)
+            if fast_key is not None:
+                fast = self._fast_calls.get(fast_key)
+                if fast is not None:
+                    return fast.run(args)
+                rec = _launch_plan.Recorder(self.nargs)
         for arg in args:
             if hasattr(arg, '__cupy_override_elementwise_kernel__'):
                 return arg.__cupy_override_elementwise_kernel__(
                     self, *args, size=size, stream=stream, block_size=block_size)
-        dev_id = _device.get_device_id()
         arg_list = _preprocess_args(dev_id, args)
         out_args = arg_list[self.nin:]
         bargs, shape = _broadcast(arg_list, self.params, size != -1)
@@ -871,7 +882,19 @@ class ElementwiseKernel:
         self._planner.launch(
             dev_id, inout_args, self.nin, shape, var_types,
             type_map.get_typedef_code(), stream=stream, block_size=block_size,
-            force_generic=not self.reduce_dims and False)
+            rec=rec)
+        if rec is not None and len(rec.launches) == 1:
+            if self.no_return:
+                ret_refs = None
+            elif not self.return_tuple and self.nout == 1:
+                ret_refs = self.nin
+            else:
+                ret_refs = tuple(range(self.nin, self.nargs))
+            out_specs = () if n_args == self.nargs else tuple(
+                (shape, o.dtype) for o in out_args)
+            _launch_plan.remember(
+                self._fast_calls, fast_key,
+                _launch_plan.FastCall(n_args, out_specs, rec, ret_refs))
         return ret
 
     def _decide_params_type(self, in_args_dtype, out_args_dtype):
@@ -1126,6 +1149,7 @@ class ufunc:
         self._routine_cache = {}
         self._planners = {}
         self._kernel_memo = self._planners
+        self._fast_calls = {}
 
     def __repr__(self):
         return '<ufunc \'%s\'>' % self.name
@@ -1156,6 +1180,26 @@ class ufunc:
                     self, *args, **kwargs)
         if _fusion_thread_local.is_fusing():
             return _fusion_thread_local.call_ufunc(self, *args, **kwargs)
+
+        # A call that looks like an earlier one replays that call's launch.
+        fast_key = rec = fast_args = None
+        nk = len(kwargs)
+        if nk == 0:
+            fast_args = args
+        elif nk == 1 and len(args) == self.nin and 'out' in kwargs:
+            o = kwargs['out']
+            fast_args = args + (o if type(o) is tuple else (o,))
+        if fast_args is not None and self.nin <= len(fast_args) <= self.nargs:
+            fast_key = _launch_plan.call_signature(fast_args, _device.get_device_id())
+            if fast_key is not None:
+                fast = self._fast_calls.get(fast_key)
+                if fast is not None:
+                    ret = fast.run(fast_args)
+                    if ret is not NotImplemented:
+                        return ret
+                    fast_key = None
+                else:
+                    rec = _launch_plan.Recorder(self.nargs)
 
         out = kwargs.pop('out', None)
         where = kwargs.pop('_where', None)
@@ -1208,8 +1252,12 @@ class ufunc:
         else:
             where_args = []
 
+        if rec is not None:
+            before = list(in_args)
         _copy_in_args_if_needed(in_args, given_out_args)
         _copy_in_args_if_needed(where_args, given_out_args)
+        if rec is not None and any(a is not b for a, b in zip(before, in_args)):
+            rec = None          # an input was copied: nothing to replay
         inout_args = in_args + where_args + given_out_args
         shape = internal._broadcast_core(inout_args)
         n_in = len(in_args)
@@ -1267,7 +1315,17 @@ class ufunc:
         planner.launch(
             dev_id, all_args, nin_total, shape, var_types, typedefs, casts=casts,
             force_generic=False, force_read_out=has_where,
-            kernel_name=self._get_name_with_type(all_args, has_where))
+            kernel_name=self._get_name_with_type(all_args, has_where), rec=rec)
+        if rec is not None and len(rec.launches) == 1:
+            n_user = len(fast_args)
+            n_given = n_user - self.nin
+            ret_refs = self.nin if self.nout == 1 else tuple(range(self.nin, self.nargs))
+            out_specs = tuple((shape, o.dtype) for o in out_args[n_given:])
+            overlap = [(i, self.nin + j) for j in range(n_given)
+                       for i in range(self.nin) if isinstance(in_args[i], ndarray)]
+            _launch_plan.remember(
+                self._fast_calls, fast_key,
+                _launch_plan.FastCall(n_user, out_specs, rec, ret_refs, overlap))
         return ret
 
     def _get_planner(self, op, has_where):

@@ -1,0 +1,201 @@
+"""Replay of kernel launches for calls whose arguments look like an earlier call's.
+
+Everything the host path decides for a call of an ElementwiseKernel, a ufunc, a
+reduction or a fused function -- the loop's types, broadcasting, the merged
+axes, the kernel variant, its launch geometry, the layout of its argument
+block, the shapes and types of the outputs and of temporaries -- is a function
+of the arguments' *signature*: for arrays the dtype, shape, strides, device and
+the alignment of the data pointer, for scalars their Python or NumPy type.
+Only data pointers and scalar values change from call to call.  The first call
+with a signature goes through the full path and records what it launched; later
+calls with the same signature patch pointers and scalar values into the recorded
+argument blocks and launch.
+
+The reference repeats its whole per-call path on every call
+(cupy/_core/_kernel.pyx:870-935 for ElementwiseKernel, :1241-1330 for ufuncs,
+cupy/_core/_reduction.pyx:309-427 for reductions); its kernel memo
+(_kernel.pyx:948-975) saves only the compilation.
+"""
+import numpy
+
+from cupy_amd._core import _tuning
+from cupy_amd._core._scalar import CScalar
+from cupy_amd.cuda import memory as _memory
+from cupy_amd.cuda import stream as _stream
+
+
+_float64 = numpy.dtype('float64')
+_float32 = numpy.dtype('float32')
+_bool = numpy.dtype('bool')
+_INT_LIMITS = {
+    numpy.dtype(t): (int(numpy.iinfo(t).min), int(numpy.iinfo(t).max))
+    for t in ('int8', 'int16', 'int32', 'int64', 'uint8', 'uint16', 'uint32', 'uint64')}
+_F32_SAFE = 3.0e38
+_INT64_MIN = -(1 << 63)
+_INT64_MAX = (1 << 63) - 1
+_INF = float('inf')
+
+# Recorded calls kept per kernel object.
+_MAX_PLANS = 256
+
+
+def scalar_value(v, descr):
+    """``v`` as the Python object ``struct.pack`` takes for a kernel parameter
+    of dtype ``descr``; same result (and same errors) as
+    ``CScalar(v).apply_dtype(descr)._struct_value()``."""
+    t = type(v)
+    if t is float:
+        if descr is _float64 or descr == _float64:
+            return v
+        if descr == _float32 and (-_F32_SAFE < v < _F32_SAFE or v != v
+                                  or v == _INF or v == -_INF):
+            return v        # struct rounds to nearest even exactly like NumPy
+    elif t is int:
+        lim = _INT_LIMITS.get(descr)
+        if lim is not None:
+            if lim[0] <= v <= lim[1]:
+                return v
+        elif descr == _float64 and -(1 << 53) <= v <= (1 << 53):
+            return float(v)
+    elif t is bool:
+        if descr == _bool:
+            return v
+    s = CScalar(v)
+    s.apply_dtype(descr)
+    return s._struct_value()
+
+
+class ArgBlock:
+    """Values of one kernel's argument block, in order, with a note of which
+    slots hold the data pointer of which argument and the value of which
+    scalar.  ``ref`` numbers identify the call's arguments: user arguments
+    first, then outputs the call allocates, then temporaries."""
+    __slots__ = ('vals', 'ptrs', 'scalars')
+
+    def __init__(self):
+        self.vals = []
+        self.ptrs = []
+        self.scalars = []
+
+    def ptr(self, ref, address):
+        self.ptrs.append((len(self.vals), ref))
+        self.vals.append(address)
+
+    def scalar(self, ref, cscalar):
+        self.scalars.append((len(self.vals), ref, cscalar.descr))
+        self.vals.append(cscalar._struct_value())
+
+    def const(self, *values):
+        self.vals.extend(values)
+
+
+class Recorder:
+    """Collects the launches and temporaries of one call."""
+    __slots__ = ('n_refs', 'launches', 'temps')
+
+    def __init__(self, n_refs):
+        self.n_refs = n_refs      # user arguments + allocated outputs
+        self.launches = []
+        self.temps = []
+
+    def temp(self, nbytes):
+        """Registers a temporary of ``nbytes``; returns its ref number."""
+        self.temps.append(nbytes)
+        return self.n_refs + len(self.temps) - 1
+
+    def launch(self, fn, grid, block, packer, argblock, shared_mem=0):
+        self.launches.append((fn, grid, block, packer, list(argblock.vals),
+                              tuple(argblock.ptrs), tuple(argblock.scalars),
+                              shared_mem))
+
+
+def launch(rec, fn, grid, block, packer, argblock, stream_ptr, shared_mem=0):
+    """Launches now and, if a recorder is given, notes the launch for replay."""
+    fn.launch_packed(grid, block, packer.pack(*argblock.vals), shared_mem, stream_ptr)
+    if rec is not None:
+        rec.launch(fn, grid, block, packer, argblock, shared_mem)
+
+
+def call_signature(args, dev_id):
+    """Hashable description of everything about ``args`` that launch decisions
+    may depend on, or None if the call must take the full path."""
+    from cupy_amd._core.core import ndarray
+    sig = [dev_id, _tuning.version()]
+    for a in args:
+        t = type(a)
+        if t is ndarray:
+            d = a.data
+            if d.device_id != dev_id:
+                return None
+            sig.append((a.dtype, a._shape, a._strides, d.ptr & 15))
+        elif t is float or t is bool:
+            sig.append(t)
+        elif t is int:
+            if not (_INT64_MIN <= a <= _INT64_MAX):
+                return None
+            sig.append(t)
+        elif isinstance(a, numpy.generic):
+            sig.append(t)
+        else:
+            return None
+    return tuple(sig)
+
+
+def ranges_overlap(a, b):
+    """True if the memory spans of two arrays intersect."""
+    from cupy_amd._core._carray import may_share_bounds
+    return may_share_bounds(a, b)
+
+
+class FastCall:
+    """Recorded call: allocates outputs and temporaries, patches pointers and
+    scalar values, launches."""
+    __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap')
+
+    def __init__(self, n_user, out_specs, rec, ret, overlap=()):
+        self.n_user = n_user
+        self.out_specs = tuple(out_specs)     # (shape, dtype) of allocated outputs
+        self.temps = tuple(rec.temps)
+        self.launches = tuple(rec.launches)
+        self.ret = ret                        # ref, tuple of refs, or None
+        self.overlap = tuple(overlap)         # (input ref, output ref) pairs to check
+
+    def run(self, args, stream_ptr=None):
+        from cupy_amd._core.core import ndarray
+        for i, o in self.overlap:
+            a, b = args[i], args[o]
+            if a is not b and ranges_overlap(a, b):
+                return NotImplemented
+        refs = list(args)
+        for shape, dtype in self.out_specs:
+            refs.append(ndarray._new_contiguous(shape, dtype))
+        n_arr = len(refs)
+        for nbytes in self.temps:
+            refs.append(_memory.alloc(nbytes))
+        if stream_ptr is None:
+            stream_ptr = _stream.get_current_stream_ptr()
+        for fn, grid, block, packer, template, ptrs, scalars, shmem in self.launches:
+            vals = template[:]
+            for slot, ref in ptrs:
+                if ref < n_arr:
+                    vals[slot] = refs[ref].data.ptr
+                else:
+                    vals[slot] = refs[ref].ptr
+            for slot, ref, descr in scalars:
+                vals[slot] = scalar_value(refs[ref], descr)
+            fn.launch_packed(grid, block, packer.pack(*vals), shmem, stream_ptr)
+        ret = self.ret
+        if ret is None:
+            return None
+        if type(ret) is tuple:
+            return tuple(refs[r] for r in ret)
+        return refs[ret]
+
+
+def remember(table, key, fast):
+    """Stores a recorded call; the table is emptied when it grows too large
+    (signatures include shapes, so a loop over many shapes must not pin an
+    unbounded number of entries)."""
+    if len(table) >= _MAX_PLANS:
+        table.clear()
+    table[key] = fast

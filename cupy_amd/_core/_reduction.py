@@ -20,6 +20,7 @@ from cupy_amd import _dryrun
 from cupy_amd._core import _carray
 from cupy_amd._core import _codegen_reduction as _cg
 from cupy_amd._core import _kernel
+from cupy_amd._core import _launch_plan
 from cupy_amd._core import _tuning
 from cupy_amd._core import internal
 from cupy_amd._core._codegen_elementwise import uses_identifier
@@ -110,6 +111,7 @@ class _AbstractReductionKernel:
         self._cached_codes = {}
         self._memo = {}
         self._lock = threading.Lock()
+        self._fast_calls = {}
 
     # Hooks of the concrete classes -----------------------------------------------------
     def _get_expressions_and_types(self, in_args, out_args, dtype):
@@ -126,7 +128,7 @@ class _AbstractReductionKernel:
 
     # -----------------------------------------------------------------------------------
     def _call(self, in_args, out_args, a_shape, axis, dtype, keepdims, reduce_dims,
-              device_id, stream, sort_reduce_axis=True):
+              device_id, stream, sort_reduce_axis=True, rec=None):
         if dtype is not None:
             dtype = get_dtype(dtype).type
         (map_expr, reduce_expr, post_map_expr, in_types, out_types, reduce_type,
@@ -163,13 +165,46 @@ class _AbstractReductionKernel:
 
         self._launch(in_args, out_args, a_shape, reduce_axis, out_axis, keepdims,
                      map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
-                     device_id, stream)
+                     device_id, stream, rec)
         return ret
+
+    def _fast_lookup(self, fast_args, extra, dev_id):
+        """Replays an earlier call with the same argument signature.  Returns
+        (done, result, key, recorder)."""
+        key = _launch_plan.call_signature(fast_args, dev_id)
+        if key is None:
+            return False, None, None, None
+        try:
+            key = key + extra
+            fast = self._fast_calls.get(key)
+        except TypeError:       # unhashable axis / dtype argument
+            return False, None, None, None
+        if fast is not None:
+            ret = fast.run(fast_args)
+            if ret is not NotImplemented:
+                return True, ret, None, None
+            return False, None, None, None
+        nargs = len(self.in_params) + len(self.out_params)
+        return False, None, key, _launch_plan.Recorder(nargs)
+
+    def _fast_remember(self, key, rec, fast_args, ret):
+        if rec is None or not rec.launches or ret is None:
+            return
+        nin = len(self.in_params)
+        n_given = len(fast_args) - nin
+        out_specs = ()
+        if n_given == 0:
+            if len(self.out_params) != 1:
+                return
+            out_specs = ((ret._shape, ret.dtype),)
+        _launch_plan.remember(
+            self._fast_calls, key,
+            _launch_plan.FastCall(len(fast_args), out_specs, rec, nin))
 
     # -- planning ---------------------------------------------------------------------------
     def _launch(self, in_args, out_args, a_shape, reduce_axis, out_axis, keepdims,
                 map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
-                device_id, stream):
+                device_id, stream, rec=None):
         stream_ptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
         in_params = self.in_params
         out_params = self.out_params
@@ -232,7 +267,7 @@ class _AbstractReductionKernel:
                 s % a.dtype.itemsize == 0 for s, a in zip(sr, ins))
             plan_args = (in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                          so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
-                         reduce_type, typedefs, device_id, stream_ptr)
+                         reduce_type, typedefs, device_id, stream_ptr, rec)
             if rows_ok:
                 return self._launch_rows(*plan_args)
             if cols_ok:
@@ -253,7 +288,7 @@ class _AbstractReductionKernel:
         return self._launch_generic(
             g_in, g_out, in_shape, tuple(oshape), internal.prod(rshape) if in_arr_idx
             else internal.prod(red_shape), map_expr, reduce_expr, post_map_expr,
-            reduce_type, typedefs, device_id, stream_ptr)
+            reduce_type, typedefs, device_id, stream_ptr, rec)
 
     # -- helpers ----------------------------------------------------------------------------
     def _rargs(self, in_args, out_args, bcast_r=None, bcast_o=None):
@@ -337,25 +372,29 @@ class _AbstractReductionKernel:
         return ''.join(fmt)
 
     def _fast_values(self, in_args, out_args, n_out, n_red, so_in, sr, so_out):
-        vals = []
-        for a in in_args:
-            vals.append(a.data.ptr if isinstance(a, ndarray) else a._struct_value())
-        for a in out_args:
-            vals.append(a.data.ptr)
-        vals.extend((n_out, n_red))
+        vals = _launch_plan.ArgBlock()
+        nin = len(self.in_params)
+        for ref, a in enumerate(in_args):
+            if isinstance(a, ndarray):
+                vals.ptr(ref, a.data.ptr)
+            else:
+                vals.scalar(ref, a)
+        for j, a in enumerate(out_args):
+            vals.ptr(nin + j, a.data.ptr)
+        vals.const(n_out, n_red)
         k = 0
         for a, p in zip(in_args, self.in_params):
             if isinstance(a, ndarray) and not p.raw:
                 item = a.dtype.itemsize
-                vals.extend((so_in[k] // item, sr[k] // item))
+                vals.const(so_in[k] // item, sr[k] // item)
                 k += 1
         for k, a in enumerate(out_args):
-            vals.append(so_out[k] // a.dtype.itemsize)
+            vals.const(so_out[k] // a.dtype.itemsize)
         return vals
 
     def _finalize_partials(self, partials, n_split, out_args, out_arr_idx, n_out,
                            so_out, in_args, reduce_expr, post_map_expr, reduce_type,
-                           typedefs, device_id, stream_ptr):
+                           typedefs, device_id, stream_ptr, rec, partials_ref):
         """Second pass: combine ``partials[s][i]`` over s, then POST_MAP."""
         preamble, _ = self._get_preamble_options()
         tx = max(1, min(64, internal.clp2(n_out)))
@@ -374,27 +413,29 @@ class _AbstractReductionKernel:
         fn, _, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         fmt = ['@P']
-        vals = [partials.ptr]
-        for a, p in zip(in_args, self.in_params):
+        vals = _launch_plan.ArgBlock()
+        vals.ptr(partials_ref, partials.ptr)
+        nin = len(self.in_params)
+        for ref, a in enumerate(in_args):
             if not isinstance(a, ndarray):
                 fmt.append(_scalar_struct_code(_get_typename(a.descr)))
-                vals.append(a._struct_value())
-        for a in out_args:
+                vals.scalar(ref, a)
+        for j, a in enumerate(out_args):
             fmt.append('P')
-            vals.append(a.data.ptr)
+            vals.ptr(nin + j, a.data.ptr)
         fmt.append(ic * 4)
-        vals.extend((n_out, n_split, 1, n_out))
+        vals.const(n_out, n_split, 1, n_out)
         for k, a in enumerate(out_args):
             fmt.append(ic)
-            vals.append(so_out[k] // a.dtype.itemsize)
-        blob = struct.pack(''.join(fmt), *vals)
+            vals.const(so_out[k] // a.dtype.itemsize)
         grid = (n_out + tx - 1) // tx
-        fn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+        _launch_plan.launch(rec, fn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
+                            struct.Struct(''.join(fmt)), vals, stream_ptr)
 
     # -- rows ---------------------------------------------------------------------------------
     def _launch_rows(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                      so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
-                     reduce_type, typedefs, device_id, stream_ptr):
+                     reduce_type, typedefs, device_id, stream_ptr, rec=None):
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
         cus = _device.get_compute_units(device_id)
@@ -480,22 +521,31 @@ class _AbstractReductionKernel:
                      cus * _tuning.get('rows_group_rows_per_lane'))
         if partial:
             rsize = self._reduce_type_size(reduce_type, mod)
-            partials = _memory.alloc(rsize * n_split * n_out)
-            vals.extend((partials.ptr, chunk))
-            blob = struct.pack(self._fast_format(rargs, ic, 'P' + ic), *vals)
-            fn.launch_packed((gx, n_split, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
+            vals.ptr(pref, partials.ptr)
+            vals.const(chunk)
+            _launch_plan.launch(
+                rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
+                struct.Struct(self._fast_format(rargs, ic, 'P' + ic)), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
-                stream_ptr)
+                stream_ptr, rec, pref)
         else:
-            blob = struct.pack(self._fast_format(rargs, ic), *vals)
-            fn.launch_packed((gx, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            _launch_plan.launch(
+                rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
+                struct.Struct(self._fast_format(rargs, ic)), vals, stream_ptr)
+
+    @staticmethod
+    def _alloc_partials(rec, nbytes):
+        """Temporary for partial results and its ref number for replays."""
+        partials = _memory.alloc(nbytes)
+        return partials, (rec.temp(nbytes) if rec is not None else -1)
 
     # -- cols ---------------------------------------------------------------------------------
     def _launch_cols(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                      so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
-                     reduce_type, typedefs, device_id, stream_ptr):
+                     reduce_type, typedefs, device_id, stream_ptr, rec=None):
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
         cus = _device.get_compute_units(device_id)
@@ -538,22 +588,24 @@ class _AbstractReductionKernel:
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
         if partial:
             rsize = self._reduce_type_size(reduce_type, mod)
-            partials = _memory.alloc(rsize * n_split * n_out)
-            vals.append(partials.ptr)
-            blob = struct.pack(self._fast_format(rargs, ic, 'P'), *vals)
-            fn.launch_packed((gx, n_split, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
+            vals.ptr(pref, partials.ptr)
+            _launch_plan.launch(
+                rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
+                struct.Struct(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
-                stream_ptr)
+                stream_ptr, rec, pref)
         else:
-            blob = struct.pack(self._fast_format(rargs, ic), *vals)
-            fn.launch_packed((gx, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            _launch_plan.launch(
+                rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
+                struct.Struct(self._fast_format(rargs, ic)), vals, stream_ptr)
 
     # -- generic ------------------------------------------------------------------------------
     def _launch_generic(self, in_args, out_args, in_shape, out_shape, n_red,
                         map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
-                        device_id, stream_ptr):
+                        device_id, stream_ptr, rec=None):
         preamble, _ = self._get_preamble_options()
         cus = _device.get_compute_units(device_id)
         n_out = internal.prod(out_shape)
@@ -597,32 +649,36 @@ class _AbstractReductionKernel:
                 out_index_32=out_ind._index_32_bits, partial_out=partial)
         fn, mod, _ = self._compile(key, emit, in_args)
         fmt = ['@']
-        vals = []
-        for a in list(in_args) + list(out_args):
+        vals = _launch_plan.ArgBlock()
+        nin = len(self.in_params)
+
+        def put(ref, a):
             if isinstance(a, ndarray):
                 fmt.append('P' + 'q' * (1 + 2 * a.ndim))
-                vals.append(a.data.ptr)
-                vals.append(a.size)
-                vals.extend(a._shape)
-                vals.extend(a._strides)
+                vals.ptr(ref, a.data.ptr)
+                vals.const(a.size, *a._shape)
+                vals.const(*a._strides)
             else:
                 fmt.append(_scalar_struct_code(_get_typename(a.descr)))
-                vals.append(a._struct_value())
+                vals.scalar(ref, a)
+        for ref, a in enumerate(in_args):
+            put(ref, a)
+        for j, a in enumerate(out_args):
+            put(nin + j, a)
         for ind in (in_ind, out_ind):
             fmt.append('q' * (1 + 2 * ind.ndim))
-            vals.append(ind.size)
-            vals.extend(ind.shape)
-            vals.extend((0,) * ind.ndim)
+            vals.const(ind.size, *ind.shape)
+            vals.const(*((0,) * ind.ndim))
         if not partial:
-            blob = struct.pack(''.join(fmt), *vals)
-            fn.launch_packed((gx, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+            _launch_plan.launch(rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
+                                struct.Struct(''.join(fmt)), vals, stream_ptr)
             return
         rsize = self._reduce_type_size(reduce_type, mod)
-        partials = _memory.alloc(rsize * n_split * n_out)
+        partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
         fmt.append('P')
-        vals.append(partials.ptr)
-        blob = struct.pack(''.join(fmt), *vals)
-        fn.launch_packed((gx, n_split, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+        vals.ptr(pref, partials.ptr)
+        _launch_plan.launch(rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
+                            struct.Struct(''.join(fmt)), vals, stream_ptr)
         # second pass through the strided output views
         frargs = [r for r in rargs if r.kind in ('out', 'raw', 'scalar')]
         fkey = ('generic_final', tuple(r.key() for r in frargs), typedefs,
@@ -637,36 +693,23 @@ class _AbstractReductionKernel:
                 out_index_32=out_ind._index_32_bits)
         ffn, _, _ = self._compile(fkey, emit_final, in_args)
         fmt = ['@']
-        vals = []
+        vals = _launch_plan.ArgBlock()
         # parameter order of emit_finalize_generic: out / raw / scalar in the
         # order they appear in `frargs`
-        objs = []
-        for a, p in zip(in_args, self.in_params):
-            if isinstance(a, ndarray):
-                if p.raw:
-                    objs.append(a)
-            else:
-                objs.append(a)
-        objs.extend(out_args)
-        for a in objs:
-            if isinstance(a, ndarray):
-                fmt.append('P' + 'q' * (1 + 2 * a.ndim))
-                vals.append(a.data.ptr)
-                vals.append(a.size)
-                vals.extend(a._shape)
-                vals.extend(a._strides)
-            else:
-                fmt.append(_scalar_struct_code(_get_typename(a.descr)))
-                vals.append(a._struct_value())
+        for ref, (a, p) in enumerate(zip(in_args, self.in_params)):
+            if not isinstance(a, ndarray) or p.raw:
+                put(ref, a)
+        for j, a in enumerate(out_args):
+            put(nin + j, a)
         fmt.append('q' * (1 + 2 * out_ind.ndim))
-        vals.append(out_ind.size)
-        vals.extend(out_ind.shape)
-        vals.extend((0,) * out_ind.ndim)
+        vals.const(out_ind.size, *out_ind.shape)
+        vals.const(*((0,) * out_ind.ndim))
         fmt.append('Pi')
-        vals.extend((partials.ptr, n_split))
-        blob = struct.pack(''.join(fmt), *vals)
+        vals.ptr(pref, partials.ptr)
+        vals.const(n_split)
         grid = max(1, min((n_out + _cg.BLOCK - 1) // _cg.BLOCK, cus * 8))
-        ffn.launch_packed((grid, 1, 1), (_cg.BLOCK, 1, 1), blob, 0, stream_ptr)
+        _launch_plan.launch(rec, ffn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
+                            struct.Struct(''.join(fmt)), vals, stream_ptr)
 
     # -- debugging aids ------------------------------------------------------------------------
     @property
@@ -716,8 +759,13 @@ class _SimpleReductionKernel(_AbstractReductionKernel):
         if hasattr(a, '__cupy_override_reduction_kernel__'):
             return a.__cupy_override_reduction_kernel__(
                 self, axis, dtype, out, keepdims)
-        arr = _convert_from_cupy_like(a, error="Argument 'a'")
         dev_id = _device.get_device_id()
+        fast_args = (a,) if out is None else (a, out)
+        done, ret, key, rec = self._fast_lookup(
+            fast_args, (axis, dtype, keepdims), dev_id)
+        if done:
+            return ret
+        arr = _convert_from_cupy_like(a, error="Argument 'a'")
         _check_peer_access(arr, dev_id)
         if out is None:
             out_args = []
@@ -726,8 +774,10 @@ class _SimpleReductionKernel(_AbstractReductionKernel):
                 raise TypeError("Argument 'out' has incorrect type")
             _check_peer_access(out, dev_id)
             out_args = [out]
-        return self._call([arr], out_args, arr._shape, axis, dtype, keepdims,
-                          True, dev_id, None, self._sort_reduce_axis)
+        ret = self._call([arr], out_args, arr._shape, axis, dtype, keepdims,
+                         True, dev_id, None, self._sort_reduce_axis, rec)
+        self._fast_remember(key, rec, fast_args, ret)
+        return ret
 
     def _get_expressions_and_types(self, in_args, out_args, dtype):
         op = self._ops.guess_routine(
@@ -830,11 +880,21 @@ class ReductionKernel(_AbstractReductionKernel):
                                  "a positional and keyword argument")
             out_args = [out]
         dev_id = _device.get_device_id()
+        key = rec = None
+        if stream is None:
+            fast_args = tuple(args[:self.nin]) + tuple(out_args)
+            done, ret, key, rec = self._fast_lookup(
+                fast_args, (axis, keepdims), dev_id)
+            if done:
+                return ret
         in_args = _preprocess_args(dev_id, args[:self.nin])
         out_args = _preprocess_args(dev_id, out_args)
         in_args, broad_shape = _broadcast(in_args, self.in_params, False)
-        return self._call(in_args, out_args, broad_shape, axis, None, keepdims,
-                          self.reduce_dims, dev_id, stream, True)
+        ret = self._call(in_args, out_args, broad_shape, axis, None, keepdims,
+                         self.reduce_dims, dev_id, stream, True, rec)
+        if rec is not None:
+            self._fast_remember(key, rec, fast_args, ret)
+        return ret
 
     def _get_expressions_and_types(self, in_args, out_args, dtype):
         in_ndarray_types = tuple(

@@ -30,6 +30,7 @@ _params = {
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
 }
 _signature = tuple(sorted(_params.items()))
+_version = 0
 
 
 def get(name):
@@ -37,13 +38,20 @@ def get(name):
 
 
 def set(**kw):
-    global _signature
+    global _signature, _version
     for k, v in kw.items():
         if k not in _params:
             raise KeyError(k)
         _params[k] = v
     _signature = tuple(sorted(_params.items()))
+    _version += 1
 
 
 def signature():
     return _signature
+
+
+def version():
+    """Counter of calls to set(): cheap stand-in for signature() in keys
+    that only live inside one process."""
+    return _version

@@ -1,0 +1,313 @@
+"""A call that repeats an earlier call's argument signature replays the recorded
+launch.  These tests compare, launch for launch and byte for byte, what the
+replay puts into the kernel's argument block with what the full path puts there
+for the same arguments.  They inspect recorded launches, so they need the
+compile-check mode (no GPU); the GPU suite checks the replayed results
+numerically (tests/test_gpu_runtime.py)."""
+import struct
+
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from cupy_amd import _dryrun
+from cupy_amd._core import _launch_plan
+
+pytestmark = pytest.mark.skipif(not _dryrun.enabled(),
+                                reason='inspects recorded launches')
+
+
+def launches_of(fn):
+    n0 = len(_dryrun.launches)
+    ret = fn()
+    return ret, _dryrun.launches[n0:]
+
+
+def words(blob, known):
+    """Argument block as a list of 8-byte words; words that look like device
+    addresses are replaced by the name of the array they point into, or by
+    'tmp' for memory the call allocated itself."""
+    out = []
+    pad = (-len(blob)) % 8
+    data = blob + b'\0' * pad
+    for (w,) in struct.iter_unpack('<Q', data):
+        if 0x7f0000000000 <= w < 0x7f8000000000:
+            out.append(known.get(w, 'tmp'))
+        else:
+            out.append(w)
+    return out
+
+
+def describe(launches, known):
+    return [(name, grid, block, shmem, words(blob, known))
+            for name, grid, block, shmem, blob in launches]
+
+
+def check_replay(kernel_tables, call, make_args, known_of):
+    """``call(*args)`` three times: the recording call, a replay with the
+    same arguments, then -- with other arrays of the same signature -- a replay
+    and, after the recorded calls have been dropped, the full path again."""
+    args1 = make_args()
+    _, first = launches_of(lambda: call(*args1))
+    assert first
+    _, again = launches_of(lambda: call(*args1))
+    k1 = known_of(args1)
+    assert describe(again, k1) == describe(first, k1)
+
+    args2 = make_args()
+    k2 = known_of(args2)
+    n_recorded = sum(len(t) for t in kernel_tables())
+    assert n_recorded >= 1
+    _, replay = launches_of(lambda: call(*args2))
+    assert sum(len(t) for t in kernel_tables()) == n_recorded      # nothing new recorded
+    for t in kernel_tables():
+        t.clear()
+    _, full = launches_of(lambda: call(*args2))
+    assert describe(replay, k2) == describe(full, k2)
+    # same structure as the first call, other addresses
+    assert [l[:4] for l in replay] == [l[:4] for l in first]
+
+
+def names(args):
+    known = {}
+    for i, a in enumerate(args):
+        if isinstance(a, cp.ndarray):
+            known[a.data.ptr] = 'arg%d' % i
+    return known
+
+
+def test_elementwise_kernel_replay_patches_pointers_and_scalars():
+    saxpy = cp.ElementwiseKernel('float32 x, float32 y, float32 a', 'float32 z',
+                                 'z = a * x + y', 'saxpy_replay')
+
+    def make():
+        n = 1 << 16
+        return (cp.ndarray((n,), np.float32), cp.ndarray((n,), np.float32), 2.5,
+                cp.ndarray((n,), np.float32))
+    check_replay(lambda: [saxpy._fast_calls], saxpy, make, names)
+    # another scalar value goes into the same slot
+    x, y, _, z = make()
+    _, a = launches_of(lambda: saxpy(x, y, 2.5, z))
+    _, b = launches_of(lambda: saxpy(x, y, -7.25, z))
+    wa, wb = words(a[0][4], names((x, y, 0, z))), words(b[0][4], names((x, y, 0, z)))
+    diff = [i for i, (p, q) in enumerate(zip(wa, wb)) if p != q]
+    assert len(diff) == 1
+    assert struct.pack('<Q', wb[diff[0]])[:4] == struct.pack('<f', -7.25)
+
+
+def test_elementwise_kernel_allocates_a_new_output_on_every_replay():
+    sq = cp.ElementwiseKernel('T x', 'T y', 'y = x * x', 'square_replay')
+    x = cp.ndarray((1000,), np.float64)
+    r1 = sq(x)
+    r2 = sq(x)
+    r3 = sq(x)
+    assert r1 is not r2 and r2 is not r3
+    assert r2.data.ptr != r3.data.ptr
+    assert r3.shape == (1000,) and r3.dtype == np.float64
+    assert len(sq._fast_calls) == 1
+
+
+def test_ufunc_replay_tiled_flat_and_generic():
+    def tiled():
+        base = cp.ndarray((512, 256), np.float32)
+        return (base.T, cp.ndarray((1, 512), np.float16), cp.ndarray((256, 512), np.float32))
+
+    def flat():
+        return (cp.ndarray((300, 7), np.int32), 3, cp.ndarray((300, 7), np.int32))
+
+    def generic():
+        big = cp.ndarray((6, 10, 14), np.float64)
+        return (big[::2, 1:9:3, ::-1], cp.ndarray((3, 3, 14), np.float64),
+                cp.ndarray((3, 3, 14), np.float64))
+
+    def known(args):
+        k = names(args)
+        for i, a in enumerate(args):
+            if isinstance(a, cp.ndarray) and a.base is not None:
+                k[a.data.ptr] = 'arg%d' % i
+        return k
+    for make, fn in ((tiled, cp.multiply), (flat, cp.add), (generic, cp.subtract)):
+        check_replay(lambda: [fn._fast_calls], fn, make, known)
+
+
+def test_ufunc_keyword_out_and_fresh_output_share_nothing():
+    a = cp.ndarray((64, 64), np.float32)
+    b = cp.ndarray((64, 64), np.float32)
+    o = cp.ndarray((64, 64), np.float32)
+    cp.maximum._fast_calls.clear()
+    assert cp.maximum(a, b, out=o) is o
+    assert cp.maximum(a, b, out=o) is o           # replay returns the given array
+    assert cp.maximum(a, b, o) is o
+    assert len(cp.maximum._fast_calls) == 1       # keyword and positional: one entry
+    r = cp.maximum(a, b)
+    r2 = cp.maximum(a, b)
+    assert r is not o and r2 is not r
+    assert len(cp.maximum._fast_calls) == 2
+
+
+def test_ufunc_replay_still_copies_overlapping_inputs():
+    buf = cp.ndarray((1025,), np.float32)
+    a, b = buf[:-1], buf[1:]
+    other = cp.ndarray((1024,), np.float32)
+    cp.add._fast_calls.clear()
+    # record with disjoint arrays of this signature ...
+    x = cp.ndarray((1025,), np.float32)[:-1]
+    y = cp.ndarray((1025,), np.float32)[1:]
+    launches_of(lambda: cp.add(x, other, y))
+    _, rep = launches_of(lambda: cp.add(x, other, y))
+    assert len(rep) == 1
+    # ... then call with an input that overlaps the output: the input must be
+    # copied first (an extra launch), exactly as on the full path
+    assert a.data.ptr % 16 == x.data.ptr % 16 and b.data.ptr % 16 == y.data.ptr % 16
+    _, ls = launches_of(lambda: cp.add(a, other, b))
+    w = words(ls[0][4], {a.data.ptr: 'a', other.data.ptr: 'other', b.data.ptr: 'b'})
+    assert w[:3] == ['tmp', 'other', 'b']          # reads a copy of `a`
+    _, ls = launches_of(lambda: cp.add(x, other, y))
+    w = words(ls[0][4], {x.data.ptr: 'x', other.data.ptr: 'other', y.data.ptr: 'y'})
+    assert w[:3] == ['x', 'other', 'y']
+    # in == out (the very same array) needs no copy
+    _, ls = launches_of(lambda: cp.add(y, other, y))
+    _, ls = launches_of(lambda: cp.add(y, other, y))
+    assert len(ls) == 1
+
+
+def test_scalar_conversion_matches_the_full_path():
+    from cupy_amd._core._scalar import CScalar
+
+    def full(v, dt):
+        s = CScalar(v)
+        s.apply_dtype(np.dtype(dt))
+        return s._struct_value()
+    cases = [(2.5, 'float32'), (1e39, 'float32'), (-1e39, 'float32'), (float('nan'), 'float32'),
+             (float('inf'), 'float32'), (3.0e38, 'float32'), (0.1, 'float64'), (0.1, 'float16'),
+             (7, 'int32'), (-1, 'int8'), (255, 'uint8'), (2 ** 40, 'int64'), (3, 'float64'),
+             (3, 'float32'), (True, 'bool'), (True, 'int32'), (2.75, 'int32'),
+             (np.float32(1.5), 'float64'), (np.int8(-3), 'int64')]
+    for v, dt in cases:
+        got = _launch_plan.scalar_value(v, np.dtype(dt))
+        want = full(v, dt)
+        code = {'float32': 'f', 'float64': 'd', 'float16': 'e', 'bool': '?', 'int8': 'b',
+                'uint8': 'B', 'int32': 'i', 'int64': 'q'}[dt]
+        assert struct.pack(code, got) == struct.pack(code, want), (v, dt, got, want)
+    for v, dt in ((300, 'uint8'), (-1, 'uint8'), (2 ** 31, 'int32')):
+        with pytest.raises(OverflowError):
+            full(v, dt)
+        with pytest.raises(OverflowError):
+            _launch_plan.scalar_value(v, np.dtype(dt))
+
+
+def test_python_int_out_of_range_still_raises_after_recording():
+    a = cp.ndarray((16,), np.uint8)
+    o = cp.ndarray((16,), np.uint8)
+    cp.add(a, 3, o)
+    cp.add(a, 4, o)
+    with pytest.raises(OverflowError):
+        cp.add(a, 300, o)
+
+
+def test_reduction_replay_with_and_without_partials():
+    def known(args):
+        return names(args)
+
+    def rows():
+        return (cp.ndarray((2048, 1024), np.float32), cp.ndarray((2048,), np.float32))
+
+    def cols_split():
+        return (cp.ndarray((4096, 512), np.float64), cp.ndarray((512,), np.float64))
+
+    def full():
+        return (cp.ndarray((1 << 22,), np.float32), cp.ndarray((), np.float32))
+
+    from cupy_amd._core import _routines_math as rm
+    sumk = rm._sum_auto_dtype
+    check_replay(lambda: [sumk._fast_calls], lambda a, o: sumk(a, 1, None, o, False), rows, known)
+    check_replay(lambda: [sumk._fast_calls], lambda a, o: sumk(a, 0, None, o, False), cols_split, known)
+    check_replay(lambda: [sumk._fast_calls], lambda a, o: sumk(a, None, None, o, False), full, known)
+    # the split reductions launch two kernels sharing one temporary
+    a, o = full()
+    _, ls = launches_of(lambda: sumk(a, None, None, o, False))
+    assert [l[0] for l in ls] == ['cupy_sum', 'cupy_sum_combine']
+    w0, w1 = words(ls[0][4], names((a, o))), words(ls[1][4], names((a, o)))
+    assert w0.count('tmp') == 1 and w1.count('tmp') == 1
+    raw0 = [w for (w,) in struct.iter_unpack('<Q', ls[0][4] + b'\0' * ((-len(ls[0][4])) % 8))
+            if 0x7f0000000000 <= w < 0x7f8000000000]
+    raw1 = [w for (w,) in struct.iter_unpack('<Q', ls[1][4] + b'\0' * ((-len(ls[1][4])) % 8))
+            if 0x7f0000000000 <= w < 0x7f8000000000]
+    tmp0 = [w for w in raw0 if w not in (a.data.ptr, o.data.ptr)]
+    tmp1 = [w for w in raw1 if w not in (a.data.ptr, o.data.ptr)]
+    assert tmp0 == tmp1            # both passes address the same temporary
+
+
+def test_reduction_axis_and_dtype_are_part_of_the_signature():
+    a = cp.ndarray((64, 32), np.float32)
+    r1 = a.sum(axis=0)
+    r2 = a.sum(axis=1)
+    r3 = a.sum(axis=0, keepdims=True)
+    r4 = a.sum(axis=0, dtype=np.float64)
+    r5 = a.sum(axis=0)
+    assert r1.shape == (32,) and r2.shape == (64,) and r3.shape == (1, 32)
+    assert r4.dtype == np.float64 and r5.dtype == np.float32 and r5.shape == (32,)
+    r6 = a.argmax(axis=1)
+    r7 = a.argmax(axis=1)
+    assert r6.dtype == np.int64 and r7.shape == (64,) and r6 is not r7
+
+
+def test_reduction_kernel_and_fuse_replay():
+    l2 = cp.ReductionKernel('T x, T y', 'T z', '(x - y) * (x - y)', 'a + b', 'z = sqrt(a)',
+                            '0', 'l2_replay')
+
+    def make():
+        return (cp.ndarray((256, 512), np.float32), cp.ndarray((256, 512), np.float32))
+    check_replay(lambda: [l2._fast_calls], lambda x, y: l2(x, y, axis=1), make,
+                 lambda args: names(args))
+
+    f = cp.fuse(lambda x, y, w: cp.sum((x - y) ** 2 * w, axis=-1))
+
+    def make3():
+        return (cp.ndarray((1024, 256), np.float16), cp.ndarray((1024, 256), np.float16),
+                cp.ndarray((256,), np.float32))
+    r = f(*make3())
+    args = make3()
+    r1, first = launches_of(lambda: f(*args))
+    r2, again = launches_of(lambda: f(*args))
+    assert r1 is not r2 and r1.shape == r2.shape == r.shape == (1024,)
+    k = names(args)
+    assert describe(first, k) == describe(again, k)
+    f.clear_cache()
+    r3, fresh = launches_of(lambda: f(*args))
+    assert describe(fresh, k) == describe(first, k)
+
+
+def test_tuning_change_invalidates_recorded_calls():
+    from cupy_amd._core import _tuning
+    k = cp.ElementwiseKernel('T x', 'T y', 'y = x + x', 'double_replay')
+    x = cp.ndarray((1 << 16,), np.float32)
+    y = cp.ndarray((1 << 16,), np.float32)
+    k(x, y)
+    _, a = launches_of(lambda: k(x, y))
+    old = _tuning.get('flat_block')
+    try:
+        _tuning.set(flat_block=256)
+        _, b = launches_of(lambda: k(x, y))
+        assert b[0][2] == (256, 1, 1) and a[0][2] == (old, 1, 1)
+    finally:
+        _tuning.set(flat_block=old)
+    _, c = launches_of(lambda: k(x, y))
+    assert c[0][2] == (old, 1, 1)
+
+
+def test_other_calls_take_the_full_path():
+    k = cp.ElementwiseKernel('T x', 'T y', 'y = x', 'copy_replay')
+    x = cp.ndarray((128,), np.float32)
+    y = cp.ndarray((128,), np.float32)
+    k(x, y, block_size=64)
+    k(x, y, stream=cp.cuda.Stream.null)
+    assert len(k._fast_calls) == 0
+    k(x, y)
+    assert len(k._fast_calls) == 1
+    # zero-size calls launch nothing and record nothing
+    e = cp.ndarray((0,), np.float32)
+    k(e, cp.ndarray((0,), np.float32))
+    assert len(k._fast_calls) == 1
+    with pytest.raises(TypeError):
+        k(x, y, x)
