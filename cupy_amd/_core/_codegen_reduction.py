@@ -240,15 +240,21 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
 
 def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
                       reduce_type, typedefs='', preamble='', group=32, vec=4, trips=1,
-                      batch=4, idx64=False, stream_hint=False):
+                      batch=4, idx64=False, stream_hint=False, exact=False):
     """Reduce-axis-contiguous kernel for short rows: a group of ``group`` lanes
     (power of two <= 64) covers a whole row in ``trips`` vector loads per lane
-    (``n_red <= group * vec * trips``).  To keep enough bytes in flight per
-    wave, each group works on ``batch`` rows at a time: all their loads are
-    issued first, then the ``batch`` independent cross-lane butterflies run
-    interleaved.  Fewer lanes per row with more trips per lane trade cross-lane
-    steps for in-lane accumulation.  Inputs that do not vary along the output
-    axis (``bcast_o``) are loaded once, before the row loop."""
+    (``n_red <= group * vec * trips``; ``exact``: equal).  To keep enough bytes
+    in flight per wave, each group works on ``batch`` rows at a time: all their
+    loads are issued first, then the ``batch`` independent cross-lane
+    butterflies run interleaved.  Fewer lanes per row with more trips per lane
+    trade cross-lane steps for in-lane accumulation.  Inputs that do not vary
+    along the output axis (``bcast_o``) are loaded once, before the row loop.
+
+    Every vector load is unconditional: a load under a branch makes the
+    compiler wait for it at the end of the branch, one load at a time.  Lanes
+    past the end of a row (or rows past the last one) load from a position that
+    is known to be valid instead, and their values are left out of the
+    accumulation by a select."""
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     nt = 'true' if stream_hint else 'false'
     ins = [a for a in args if a.kind == 'in']
@@ -260,15 +266,22 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
     src.append('  const %s _first = ((%s)blockIdx.x * %d + threadIdx.x) / %d;' % (
         idx_t, idx_t, BLOCK, group))
     src.append('  const %s _step = (%s)gridDim.x * %d;' % (idx_t, idx_t, BLOCK // group))
-    src.append('  const %s _j_vend = _n_red / %d * %d;' % (idx_t, vec, vec))
-    # trip t of this lane covers elements [_jv(t), _jv(t) + vec)
+    # trip t of this lane covers elements [_JV(t), _JV(t) + vec)
     src.append('#define _JV(t) ((%s)((t) * %d + _lane) * %d)' % (idx_t, group, vec))
+    if exact:
+        src.append('#define _JOK(t) true')
+        src.append('#define _JC(t) _JV(t)')
+    else:
+        src.append('  const %s _j_vend = _n_red / %d * %d;' % (idx_t, vec, vec))
+        src.append('#define _JOK(t) (_JV(t) < _j_vend)')
+        # position 0 always holds a whole vector (the host guarantees n_red >= vec)
+        src.append('#define _JC(t) (_JOK(t) ? _JV(t) : (%s)0)' % idx_t)
     for a in ins:
         if a.bcast_o and not a.bcast_r:
             src.append('  cupy::Vec<%s, %d> _h_%s[%d];' % (a.store_t, vec, a.name, trips))
             src.append('#pragma unroll')
-            src.append('  for (int _t = 0; _t < %d; ++_t) if (_JV(_t) < _j_vend) '
-                       '_h_%s[_t] = cupy::load_vec<%s, %d, false>(_p_%s + _JV(_t));' % (
+            src.append('  for (int _t = 0; _t < %d; ++_t) '
+                       '_h_%s[_t] = cupy::load_vec<%s, %d, false>(_p_%s + _JC(_t));' % (
                            trips, a.name, a.store_t, vec, a.name))
     src.append('  for (%s _i0 = _first; _i0 < _n_out; _i0 += _step * %d) {' % (idx_t, batch))
     for a in ins:
@@ -277,29 +290,35 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
                 a.store_t, vec, a.name, batch, trips))
     src.append('#pragma unroll')
     src.append('    for (int _r = 0; _r < %d; ++_r) {' % batch)
-    src.append('      const %s _i = _i0 + _r * _step;' % idx_t)
-    src.append('      if (_i < _n_out) {')
+    if batch > 1:
+        # rows past the end re-read row _i0; their results are dropped below
+        src.append('      const %s _i = (_i0 + _r * _step < _n_out) ? _i0 + _r * _step : _i0;'
+                   % idx_t)
+    else:
+        src.append('      const %s _i = _i0;' % idx_t)
     src.append('#pragma unroll')
-    src.append('        for (int _t = 0; _t < %d; ++_t) if (_JV(_t) < _j_vend) {' % trips)
+    src.append('      for (int _t = 0; _t < %d; ++_t) {' % trips)
     for a in ins:
         if not a.bcast_o and not a.bcast_r:
-            src.append('          _l_%s[_r][_t] = cupy::load_vec<%s, %d, %s>('
-                       '_p_%s + (ptrdiff_t)_i * _so_%s + _JV(_t));' % (
+            src.append('        _l_%s[_r][_t] = cupy::load_vec<%s, %d, %s>('
+                       '_p_%s + (ptrdiff_t)_i * _so_%s + _JC(_t));' % (
                            a.name, a.store_t, vec, nt, a.name, a.name))
-    src.append('        }')
     src.append('      }')
     src.append('    }')
     src.append('    _type_reduce _s[%d];' % batch)
     src.append('#pragma unroll')
     src.append('    for (int _r = 0; _r < %d; ++_r) {' % batch)
-    src.append('      const %s _i = _i0 + _r * _step;' % idx_t)
+    if batch > 1:
+        src.append('      const %s _i = (_i0 + _r * _step < _n_out) ? _i0 + _r * _step : _i0;'
+                   % idx_t)
+    else:
+        src.append('      const %s _i = _i0;' % idx_t)
     src.append('      _type_reduce _acc = %s;' % _identity_decl(identity))
-    src.append('      if (_i < _n_out) {')
     src.append('#pragma unroll')
-    src.append('        for (int _t = 0; _t < %d; ++_t) if (_JV(_t) < _j_vend) {' % trips)
+    src.append('      for (int _t = 0; _t < %d; ++_t) {' % trips)
     src.append('#pragma unroll')
-    src.append('          for (int _k = 0; _k < %d; ++_k) {' % vec)
-    src.append('            const IndexT _J = _JV(_t) + _k;')
+    src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
+    src.append('          const IndexT _J = _JV(_t) + _k;')
     for a in ins:
         if a.bcast_r:
             val = '_p_%s[(ptrdiff_t)_i * _so_%s]' % (a.name, a.name)
@@ -307,23 +326,28 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
             val = '_h_%s[_t].v[_k]' % a.name
         else:
             val = '_l_%s[_r][_t].v[_k]' % a.name
-        src.append('            const %s %s(%s);' % (a.var_t, a.name, val))
-    src.append('            _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
-    src.append('            _acc = REDUCE(_acc, _a);')
-    src.append('          }')
-    src.append('        }')
-    src.append('        for (%s _jt = _j_vend + _lane; _jt < _n_red; _jt += %d) {' % (idx_t, group))
-    src.append('          const IndexT _J = _jt;')
-    for a in ins:
-        if a.bcast_r:
-            val = '_p_%s[(ptrdiff_t)_i * _so_%s]' % (a.name, a.name)
-        else:
-            val = '_p_%s[(ptrdiff_t)_i * _so_%s + _jt]' % (a.name, a.name)
         src.append('          const %s %s(%s);' % (a.var_t, a.name, val))
     src.append('          _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
-    src.append('          _acc = REDUCE(_acc, _a);')
+    if exact:
+        src.append('          _acc = REDUCE(_acc, _a);')
+    else:
+        src.append('          const _type_reduce _n = REDUCE(_acc, _a);')
+        src.append('          _acc = _JOK(_t) ? _n : _acc;')
     src.append('        }')
     src.append('      }')
+    if not exact:
+        src.append('      for (%s _jt = _j_vend + _lane; _jt < _n_red; _jt += %d) {' % (
+            idx_t, group))
+        src.append('        const IndexT _J = _jt;')
+        for a in ins:
+            if a.bcast_r:
+                val = '_p_%s[(ptrdiff_t)_i * _so_%s]' % (a.name, a.name)
+            else:
+                val = '_p_%s[(ptrdiff_t)_i * _so_%s + _jt]' % (a.name, a.name)
+            src.append('        const %s %s(%s);' % (a.var_t, a.name, val))
+        src.append('        _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+        src.append('        _acc = REDUCE(_acc, _a);')
+        src.append('      }')
     src.append('      _s[_r] = _acc;')
     src.append('    }')
     if group > 1:
@@ -344,6 +368,8 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
     src.append('    }')
     src.append('  }')
     src.append('#undef _JV')
+    src.append('#undef _JOK')
+    src.append('#undef _JC')
     src.append('}')
     return '\n'.join(src) + '\n'
 

@@ -492,10 +492,11 @@ class _AbstractReductionKernel:
                 group //= 2
             batch = max(1, min(batch, budget // max(1, per_trip * trips)))
         bcast_o = [(s == 0 and n_out > 1) for s in so_in] if batched else None
+        exact = batched and n_red == group * vec * trips
         rargs = self._rargs(in_args, out_args, bcast_r=bcast_r, bcast_o=bcast_o)
         key = ('rows', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, group, vec, idx64, partial, device_id,
-               batched, trips, _tuning.signature())
+               batched, trips, exact, _tuning.signature())
 
         def emit():
             if batched:
@@ -503,7 +504,7 @@ class _AbstractReductionKernel:
                     self.name, rargs, self.identity, map_expr, reduce_expr,
                     post_map_expr, reduce_type, typedefs, preamble, group=group,
                     vec=vec, trips=trips, batch=batch, idx64=idx64,
-                    stream_hint=_tuning.get('rows_stream'))
+                    stream_hint=_tuning.get('rows_stream'), exact=exact)
             return self.name, _cg.emit_rows(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, group=group,
