@@ -165,7 +165,9 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
     params = ', '.join([_param_decl(op) for op in operands if op.kind != 'indexer']
                        + ['const %s _n' % idx_t]
                        + [_param_decl(op) for op in operands if op.kind == 'indexer'])
-    nt = 'true' if stream_hint else 'false'
+    _nt_l, _nt_s = stream_hint if isinstance(stream_hint, tuple) else (stream_hint, stream_hint)
+    ntl = 'true' if _nt_l else 'false'
+    nts = 'true' if _nt_s else 'false'
     use_i = uses_identifier(operation, 'i')
     set_ind = '_ind.set(i);' if needs_ind and uses_identifier(operation, '_ind') else ''
 
@@ -204,7 +206,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
                     body.append(
                         '      cupy::Vec<%s, %d> _l_%s_%d = cupy::load_vec<%s, %d, %s>('
                         '_p_%s + (_v0 + %d) * %d);' % (
-                            op.store_t, vec, op.name, u, op.store_t, vec, nt,
+                            op.store_t, vec, op.name, u, op.store_t, vec, ntl,
                             op.name, u * block, vec))
                 else:
                     body.append('      cupy::Vec<%s, %d> _l_%s_%d;' % (
@@ -224,7 +226,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
                 if op.is_out:
                     body.append(
                         '        cupy::store_vec<%s, %d, %s>(_p_%s + _base, _l_%s_%d);' % (
-                            op.store_t, vec, nt, op.name, op.name, u))
+                            op.store_t, vec, nts, op.name, op.name, u))
             body.append('      }')
         body.append('    } else {')
         body.append('      for (%s _v = _v0; _v < _nvec; _v += %d) {' % (idx_t, block))
@@ -239,7 +241,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
         if (not op.is_out) or op.read_out:
             body.append('%scupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>('
                         '_p_%s + _base);' % (pad, op.store_t, vec, op.name,
-                                             op.store_t, vec, nt, op.name))
+                                             op.store_t, vec, ntl, op.name))
         else:
             body.append('%scupy::Vec<%s, %d> _l_%s;' % (pad, op.store_t, vec, op.name))
     body.append('#pragma unroll')
@@ -252,7 +254,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
     for op in iter_arrays:
         if op.is_out:
             body.append('%scupy::store_vec<%s, %d, %s>(_p_%s + _base, _l_%s);' % (
-                pad, op.store_t, vec, nt, op.name, op.name))
+                pad, op.store_t, vec, nts, op.name, op.name))
     body.append('      }')
     body.append('    }')
     body.append('  }')
@@ -370,7 +372,9 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     arrays = [op for op in operands if op.kind == 'array']
     needs_ind = any(op.kind == 'indexer' for op in operands)
-    nt = 'true' if stream_hint else 'false'
+    _nt_l, _nt_s = stream_hint if isinstance(stream_hint, tuple) else (stream_hint, stream_hint)
+    ntl = 'true' if _nt_l else 'false'
+    nts = 'true' if _nt_s else 'false'
     use_i = uses_identifier(operation, 'i')
     set_ind = '_ind.set(i);' if needs_ind and uses_identifier(operation, '_ind') else ''
     assert tile_r % vec == 0 and tile_c % vec == 0
@@ -424,7 +428,7 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         src.append('        const int _lc = _v / %d;' % (tile_r // vec))
         for op in c_ops:
             src.append('        { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s);' % (
-                op.store_t, vec, op.store_t, vec, nt, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
+                op.store_t, vec, op.store_t, vec, ntl, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
             src.append('#pragma unroll')
             src.append('          for (int _k = 0; _k < %d; ++_k) '
                        '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (vec, op.name, pitch))
@@ -468,7 +472,7 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         if lay == 'R':
             if (not op.is_out) or op.read_out:
                 src.append('        cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
-                    op.store_t, vec, op.name, op.store_t, vec, nt, gaddr(op, '_r', '_c')))
+                    op.store_t, vec, op.name, op.store_t, vec, ntl, gaddr(op, '_r', '_c')))
             else:
                 src.append('        cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
         elif lay == 'R0':
@@ -482,7 +486,7 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     for op in arrays:
         if op.is_out:
             src.append('        cupy::store_vec<%s, %d, %s>(%s, _l_%s);' % (
-                op.store_t, vec, nt, gaddr(op, '_r', '_c'), op.name))
+                op.store_t, vec, nts, gaddr(op, '_r', '_c'), op.name))
     src.append('      }')
     src.append('    } else {')
 

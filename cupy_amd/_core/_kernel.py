@@ -454,7 +454,8 @@ class _ElementwisePlanner:
         idx64 = size > _INT32_MAX - (1 << 24)
         unroll = _tuning.get('flat_unroll') if vec > 1 else 1
         block = _tuning.get('flat_block')
-        stream_hint = _tuning.get('flat_stream')
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('flat_stream'), *self._traffic(args, nin, bcast))
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
         if self._uses_ind:
             operands.append(_cg.Operand('indexer', '_ind', '', ndim=1,
@@ -485,6 +486,27 @@ class _ElementwisePlanner:
                           _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu'))))
         _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
                             stream_ptr)
+
+    def _traffic(self, args, nin, bcast_names):
+        """Bytes a launch reads and writes (broadcast operands and raw arrays
+        not counted; an array passed twice counted once)."""
+        in_bytes = out_bytes = 0
+        seen = set()
+        for idx, (a, p) in enumerate(zip(args, self.params)):
+            if not isinstance(a, ndarray) or p.raw or p.name in bcast_names:
+                continue
+            if id(a) in seen:
+                continue
+            seen.add(id(a))
+            nbytes = a.dtype.itemsize
+            for ext, st in zip(a._shape, a._strides):
+                if st != 0:
+                    nbytes *= ext
+            if idx >= nin:
+                out_bytes += nbytes
+            else:
+                in_bytes += nbytes
+        return in_bytes, out_bytes
 
     def _flat_values(self, args):
         """Argument values for kernels that take plain pointers: data pointer
@@ -619,7 +641,9 @@ class _ElementwisePlanner:
             span = max(span, abs(cs[0]) * nr + abs(cs[1]) * nc)
         idx64 = span > _INT32_MAX or nr * nc > _INT32_MAX
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
-        stream_hint = _tuning.get('tiled_stream')
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('tiled_stream'),
+            *self._traffic(args, nin, [n for n, l in layouts.items() if l == 'R0']))
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
                threads)

@@ -13,9 +13,13 @@ _params = {
     'flat_block': 1024,         # threads per workgroup
     'flat_unroll': 1,           # vectors per thread per trip
     'flat_blocks_per_cu': 64,   # grid cap, in workgroups per CU
-    'flat_stream': True,        # non-temporal loads/stores
+    # Non-temporal hints of the elementwise kernels: True / False for loads and
+    # stores alike, or 'auto' = by footprint against the last-level cache
+    # (see stream_policy below)
+    'flat_stream': 'auto',
     # tiled 2-d elementwise kernel
-    'tiled_stream': True,
+    'tiled_stream': 'auto',
+    'cache_bytes': 256 << 20,   # capacity of the memory-side cache (Infinity Cache)
     # reductions
     'rows_stream': True,
     'rows_unroll': 1,
@@ -49,6 +53,29 @@ def set(**kw):
 
 def signature():
     return _signature
+
+
+def stream_policy(setting, in_bytes, out_bytes):
+    """(non-temporal loads?, non-temporal stores?) of an elementwise launch
+    that reads ``in_bytes`` and writes ``out_bytes``.
+
+    Measured on MI355X with copy (1 stream in, 1 out) and saxpy (2 in, 1 out)
+    kernels from 16 MiB to 1 GiB per array: inputs that together exceed the
+    memory-side cache are best read with the non-temporal hint and, if the
+    output fits that cache, written without it (the cache absorbs the writes
+    and the next kernel finds the result there); inputs that fit are best read
+    without the hint while the output streams past them; when neither side
+    fits, both stream."""
+    if isinstance(setting, (tuple, list)):
+        return bool(setting[0]), bool(setting[1])
+    if setting != 'auto':
+        return bool(setting), bool(setting)
+    # an eighth of slack: operand sets of exactly the cache's size (plus a
+    # small broadcast operand) still behave as fitting
+    cache = _params['cache_bytes'] * 9 // 8
+    loads_nt = in_bytes > cache
+    stores_nt = (not loads_nt) or out_bytes > cache
+    return loads_nt, stores_nt
 
 
 def version():
