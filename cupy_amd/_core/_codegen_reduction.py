@@ -182,25 +182,45 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     if vec > 1:
         src.append('    const %s _j_vend = _j_begin + (_j_end - _j_begin) / %d * %d;' % (
             idx_t, vec, vec))
-        src.append('#pragma unroll %d' % unroll)
-        src.append('    for (%s _j = _j_begin + _lane * %d; _j < _j_vend; _j += %d) {' % (
-            idx_t, vec, lanes * vec))
-        for a in ins:
-            if a.bcast_r:
-                src.append('      const %s _b_%s = _row_%s[0];' % (a.store_t, a.name, a.name))
-            else:
-                src.append('      const cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>('
-                           '_row_%s + _j);' % (a.store_t, vec, a.name, a.store_t, vec,
-                                               nt, a.name))
-        src.append('#pragma unroll')
-        src.append('      for (int _k = 0; _k < %d; ++_k) {' % vec)
-        src.append('        const IndexT _J = _j + _k;')
-        for a in ins:
-            val = ('_b_%s' % a.name) if a.bcast_r else ('_l_%s.v[_k]' % a.name)
-            src.append('        const %s %s(%s);' % (a.var_t, a.name, val))
-        src.append('        _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
-        src.append('        _acc[_k] = REDUCE(_acc[_k], _a);')
-        src.append('      }')
+        stride = lanes * vec
+
+        def loads(pad, j_expr, suffix):
+            for a in ins:
+                if a.bcast_r:
+                    src.append('%sconst %s _b_%s%s = _row_%s[0];' % (
+                        pad, a.store_t, a.name, suffix, a.name))
+                else:
+                    src.append('%sconst cupy::Vec<%s, %d> _l_%s%s = cupy::load_vec<%s, %d, %s>('
+                               '_row_%s + (%s));' % (pad, a.store_t, vec, a.name, suffix,
+                                                     a.store_t, vec, nt, a.name, j_expr))
+
+        def accumulate(pad, j_expr, suffix):
+            src.append('#pragma unroll')
+            src.append('%sfor (int _k = 0; _k < %d; ++_k) {' % (pad, vec))
+            src.append('%s  const IndexT _J = (%s) + _k;' % (pad, j_expr))
+            for a in ins:
+                val = ('_b_%s%s' % (a.name, suffix)) if a.bcast_r else (
+                    '_l_%s%s.v[_k]' % (a.name, suffix))
+                src.append('%s  const %s %s(%s);' % (pad, a.var_t, a.name, val))
+            src.append('%s  _type_reduce _a = static_cast<_type_reduce>(%s);' % (
+                pad, pre_map_expr))
+            src.append('%s  _acc[_k] = REDUCE(_acc[_k], _a);' % pad)
+            src.append('%s}' % pad)
+
+        src.append('    %s _j = _j_begin + _lane * %d;' % (idx_t, vec))
+        if unroll > 1:
+            # `unroll` vectors per lane and trip, every load issued before the
+            # first value is used
+            src.append('    for (; _j + %d < _j_vend; _j += %d) {' % (
+                (unroll - 1) * stride, unroll * stride))
+            for u in range(unroll):
+                loads('      ', '_j + %d' % (u * stride), '_%d' % u)
+            for u in range(unroll):
+                accumulate('      ', '_j + %d' % (u * stride), '_%d' % u)
+            src.append('    }')
+        src.append('    for (; _j < _j_vend; _j += %d) {' % stride)
+        loads('      ', '_j', '')
+        accumulate('      ', '_j', '')
         src.append('    }')
     else:
         src.append('    const %s _j_vend = _j_begin;' % idx_t)
@@ -403,34 +423,59 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('  if (_c < _n_out) {')
     src.append('    const bool _full = _c + %d <= _n_out;' % vec)
     src.append('    if (_full) {')
-    src.append('#pragma unroll %d' % unroll)
-    src.append('      for (%s _j = (%s)blockIdx.y * %d + _ty; _j < _n_red; _j += (%s)gridDim.y * %d) {' % (
-        idx_t, idx_t, ty, idx_t, ty))
-    for a in ins:
-        if partial_in:
-            # partial results may have any size: plain element reads
-            src.append('        const _type_reduce* _l_%s = _p_%s + (ptrdiff_t)_j * _sr_%s + _c;' % (
-                a.name, a.name, a.name))
-        elif a.bcast_o:
-            src.append('        const %s _b_%s = _p_%s[(ptrdiff_t)_j * _sr_%s];' % (
-                a.store_t, a.name, a.name, a.name))
-        else:
-            src.append('        const cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>('
-                       '_p_%s + (ptrdiff_t)_j * _sr_%s + _c);' % (
-                           a.store_t, vec, a.name, a.store_t, vec, nt, a.name, a.name))
-    src.append('        const IndexT _J = _j;')
-    src.append('#pragma unroll')
-    src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
-    if partial_in:
-        a = ins[0]
-        src.append('          _acc[_k] = REDUCE(_acc[_k], _l_%s[_k]);' % a.name)
-    else:
+    src.append('      const %s _jstep = (%s)gridDim.y * %d;' % (idx_t, idx_t, ty))
+    src.append('      %s _j = (%s)blockIdx.y * %d + _ty;' % (idx_t, idx_t, ty))
+
+    def loads(pad, j_expr, suffix):
         for a in ins:
-            val = ('_b_%s' % a.name) if a.bcast_o else ('_l_%s.v[_k]' % a.name)
-            src.append('          const %s %s(%s);' % (a.var_t, a.name, val))
-        src.append('          _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
-        src.append('          _acc[_k] = REDUCE(_acc[_k], _a);')
-    src.append('        }')
+            if partial_in:
+                # partial results may have any size: plain element reads
+                src.append('%s_type_reduce _l_%s%s[%d];' % (pad, a.name, suffix, vec))
+                src.append('#pragma unroll')
+                src.append('%sfor (int _k = 0; _k < %d; ++_k) _l_%s%s[_k] = '
+                           '_p_%s[(ptrdiff_t)(%s) * _sr_%s + _c + _k];' % (
+                               pad, vec, a.name, suffix, a.name, j_expr, a.name))
+            elif a.bcast_o:
+                src.append('%sconst %s _b_%s%s = _p_%s[(ptrdiff_t)(%s) * _sr_%s];' % (
+                    pad, a.store_t, a.name, suffix, a.name, j_expr, a.name))
+            else:
+                src.append('%sconst cupy::Vec<%s, %d> _l_%s%s = cupy::load_vec<%s, %d, %s>('
+                           '_p_%s + (ptrdiff_t)(%s) * _sr_%s + _c);' % (
+                               pad, a.store_t, vec, a.name, suffix, a.store_t, vec, nt,
+                               a.name, j_expr, a.name))
+
+    def accumulate(pad, j_expr, suffix):
+        src.append('%s{' % pad)
+        src.append('%s  const IndexT _J = %s;' % (pad, j_expr))
+        src.append('#pragma unroll')
+        src.append('%s  for (int _k = 0; _k < %d; ++_k) {' % (pad, vec))
+        if partial_in:
+            a = ins[0]
+            src.append('%s    _acc[_k] = REDUCE(_acc[_k], _l_%s%s[_k]);' % (pad, a.name, suffix))
+        else:
+            for a in ins:
+                val = ('_b_%s%s' % (a.name, suffix)) if a.bcast_o else (
+                    '_l_%s%s.v[_k]' % (a.name, suffix))
+                src.append('%s    const %s %s(%s);' % (pad, a.var_t, a.name, val))
+            src.append('%s    _type_reduce _a = static_cast<_type_reduce>(%s);' % (
+                pad, pre_map_expr))
+            src.append('%s    _acc[_k] = REDUCE(_acc[_k], _a);' % pad)
+        src.append('%s  }' % pad)
+        src.append('%s}' % pad)
+
+    if unroll > 1:
+        # `unroll` row-slices per trip: every load is issued before the first
+        # value is used, so that many requests are in flight per lane
+        src.append('      for (; _j + %d * _jstep < _n_red; _j += %d * _jstep) {' % (
+            unroll - 1, unroll))
+        for u in range(unroll):
+            loads('        ', '_j + %d * _jstep' % u, '_%d' % u)
+        for u in range(unroll):
+            accumulate('        ', '_j + %d * _jstep' % u, '_%d' % u)
+        src.append('      }')
+    src.append('      for (; _j < _n_red; _j += _jstep) {')
+    loads('        ', '_j', '')
+    accumulate('        ', '_j', '')
     src.append('      }')
     src.append('    } else {')
     src.append('      for (%s _j = (%s)blockIdx.y * %d + _ty; _j < _n_red; _j += (%s)gridDim.y * %d) {' % (

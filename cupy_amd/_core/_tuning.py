@@ -22,14 +22,14 @@ _params = {
     'cache_bytes': 256 << 20,   # capacity of the memory-side cache (Infinity Cache)
     # reductions
     'rows_stream': True,
-    'rows_unroll': 1,
+    'rows_unroll': 4,
     'rows_block_mode_bytes': 32768,   # row length from which a workgroup owns a row
     'rows_batch': 2,            # short rows handled per lane group at a time
     'rows_trips': 4,            # ... with up to this many vector loads per lane and row
     'rows_lane_bytes': 128,     # ... and at most this many bytes in flight per lane
     'rows_group_rows_per_lane': 64,   # grid cap for sub-wave groups: CUs * this workgroups
     'cols_stream': True,
-    'cols_unroll': 4,
+    'cols_unroll': 1,
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
 }
