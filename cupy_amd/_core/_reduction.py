@@ -493,10 +493,12 @@ class _AbstractReductionKernel:
             batch = max(1, min(batch, budget // max(1, per_trip * trips)))
         bcast_o = [(s == 0 and n_out > 1) for s in so_in] if batched else None
         exact = batched and n_red == group * vec * trips
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('rows_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         rargs = self._rargs(in_args, out_args, bcast_r=bcast_r, bcast_o=bcast_o)
         key = ('rows', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, group, vec, idx64, partial, device_id,
-               batched, trips, exact, _tuning.signature())
+               batched, trips, exact, stream_hint, _tuning.signature())
 
         def emit():
             if batched:
@@ -504,12 +506,12 @@ class _AbstractReductionKernel:
                     self.name, rargs, self.identity, map_expr, reduce_expr,
                     post_map_expr, reduce_type, typedefs, preamble, group=group,
                     vec=vec, trips=trips, batch=batch, idx64=idx64,
-                    stream_hint=_tuning.get('rows_stream'), exact=exact)
+                    stream_hint=stream_hint, exact=exact)
             return self.name, _cg.emit_rows(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, group=group,
                 vec=vec, idx64=idx64, partial_out=partial,
-                stream_hint=_tuning.get('rows_stream'),
+                stream_hint=stream_hint,
                 unroll=_tuning.get('rows_unroll'))
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
@@ -536,6 +538,15 @@ class _AbstractReductionKernel:
             _launch_plan.launch(
                 rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
                 struct.Struct(self._fast_format(rargs, ic)), vals, stream_ptr)
+
+    @staticmethod
+    def _read_bytes(ins, n_out, n_red, so_in, sr):
+        """Bytes the iterated inputs of a canonical (n_out, n_red) problem
+        occupy (broadcast axes not counted)."""
+        total = 0
+        for a, s_o, s_r in zip(ins, so_in, sr):
+            total += a.dtype.itemsize * (n_out if s_o else 1) * (n_red if s_r else 1)
+        return total
 
     @staticmethod
     def _alloc_partials(rec, nbytes):
@@ -574,16 +585,18 @@ class _AbstractReductionKernel:
                    + [abs(s) * n_out for s in so_out] + [n_red + n_split * ty])
         idx64 = span > _INT32_MAX - (1 << 24)
         rargs = self._rargs(in_args, out_args, bcast_o=bcast_o)
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
-               _tuning.signature())
+               stream_hint, _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
                 idx64=idx64, partial_out=partial,
-                stream_hint=_tuning.get('cols_stream'), unroll=_tuning.get('cols_unroll'))
+                stream_hint=stream_hint, unroll=_tuning.get('cols_unroll'))
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)

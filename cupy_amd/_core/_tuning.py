@@ -1,9 +1,11 @@
 """Launch-geometry and code-shape parameters of the emitters, in one place.
 
 The values are the result of measurements on MI355X (256 CUs, wave64, HBM3E):
-streaming kernels do best with one 16-byte access per operand in flight per
-thread (more unrolling lowers the achieved bandwidth), non-temporal accesses,
-and grids large enough that every CU always has several workgroups queued.
+elementwise kernels do best with one 16-byte access per operand in flight per
+thread (more unrolling lowers the achieved bandwidth), row reductions with
+four, non-temporal accesses for operand sets larger than the memory-side
+cache, and grids large enough that every CU always has several workgroups
+queued.
 ``set(**kw)`` changes a parameter for experiments; kernels are re-planned
 because ``signature()`` is part of every kernel memo key.
 """
@@ -21,7 +23,8 @@ _params = {
     'tiled_stream': 'auto',
     'cache_bytes': 256 << 20,   # capacity of the memory-side cache (Infinity Cache)
     # reductions
-    'rows_stream': True,
+    'rows_stream': True,       # non-temporal loads: True / False / 'auto' (by footprint);
+                               # measured better or equal from 16 MiB inputs upwards
     'rows_unroll': 4,
     'rows_block_mode_bytes': 32768,   # row length from which a workgroup owns a row
     'rows_batch': 2,            # short rows handled per lane group at a time
@@ -46,7 +49,7 @@ def set(**kw):
     for k, v in kw.items():
         if k not in _params:
             raise KeyError(k)
-        _params[k] = v
+        _params[k] = tuple(v) if isinstance(v, list) else v
     _signature = tuple(sorted(_params.items()))
     _version += 1
 
@@ -56,26 +59,23 @@ def signature():
 
 
 def stream_policy(setting, in_bytes, out_bytes):
-    """(non-temporal loads?, non-temporal stores?) of an elementwise launch
-    that reads ``in_bytes`` and writes ``out_bytes``.
+    """(non-temporal loads?, non-temporal stores?) of a launch that reads
+    ``in_bytes`` and writes ``out_bytes``.
 
-    Measured on MI355X with copy (1 stream in, 1 out) and saxpy (2 in, 1 out)
-    kernels from 16 MiB to 1 GiB per array: inputs that together exceed the
-    memory-side cache are best read with the non-temporal hint and, if the
-    output fits that cache, written without it (the cache absorbs the writes
-    and the next kernel finds the result there); inputs that fit are best read
-    without the hint while the output streams past them; when neither side
-    fits, both stream."""
+    'auto': a launch whose operands together exceed the memory-side cache
+    streams (both hints on); one that fits uses neither, so that a following
+    kernel finds the operands and the result in the cache.  Measured on MI355X
+    (copy-like and two-input kernels, 4 MiB to 1 GiB per array, called
+    repeatedly on the same arrays, in producer-consumer chains and in the mixed
+    benchmark sequence): mixed settings win single cases by up to 10 % but lose
+    others by as much, depending on what the neighbouring kernels leave in the
+    cache; this rule is never far from the best."""
     if isinstance(setting, (tuple, list)):
         return bool(setting[0]), bool(setting[1])
     if setting != 'auto':
         return bool(setting), bool(setting)
-    # an eighth of slack: operand sets of exactly the cache's size (plus a
-    # small broadcast operand) still behave as fitting
-    cache = _params['cache_bytes'] * 9 // 8
-    loads_nt = in_bytes > cache
-    stores_nt = (not loads_nt) or out_bytes > cache
-    return loads_nt, stores_nt
+    big = in_bytes + out_bytes > _params['cache_bytes']
+    return big, big
 
 
 def version():
