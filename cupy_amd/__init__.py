@@ -34,6 +34,7 @@ def get_default_memory_pool():
 from cupy_amd._core._reduction import (  # noqa
     ReductionKernel, create_reduction_func)
 from cupy_amd._core.fusion import fuse  # noqa
+from cupy_amd._core.raw import RawKernel, RawModule  # noqa
 from cupy_amd._core._routines_math import sum, prod, nansum  # noqa
 from cupy_amd._core._routines_statistics import (  # noqa
     amax, amin, argmax, argmin)

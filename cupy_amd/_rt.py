@@ -103,6 +103,11 @@ _PROTOTYPES = {
         _c.c_char_p, _c.c_char_p, _c.c_int, _c.POINTER(_c.c_char_p),
         _c.c_int, _c.POINTER(_c.c_char_p), _c.POINTER(_c.c_char_p),
         _c.POINTER(_vp), _c.POINTER(_c.c_size_t), _c.POINTER(_vp)]),
+    'rt_compile_named': (_c.c_int, [
+        _c.c_char_p, _c.c_char_p, _c.c_int, _c.POINTER(_c.c_char_p),
+        _c.c_int, _c.POINTER(_c.c_char_p), _c.POINTER(_c.c_char_p),
+        _c.c_int, _c.POINTER(_c.c_char_p), _c.POINTER(_vp),
+        _c.POINTER(_vp), _c.POINTER(_c.c_size_t), _c.POINTER(_vp)]),
     'rt_free_buffer': (None, [_vp]),
     'rt_module_load': (_c.c_int, [_vp, _c.POINTER(_vp)]),
     'rt_module_unload': (_c.c_int, [_vp]),

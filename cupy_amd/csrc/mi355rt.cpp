@@ -153,15 +153,19 @@ int rt_rtc_version(int* major, int* minor) {
   return 0;
 }
 
-int rt_compile(const char* source, const char* name,
-               int n_options, const char* const* options,
-               int n_headers, const char* const* headers,
-               const char* const* header_names,
-               void** code, size_t* code_len, char** log) {
+static int compile_impl(const char* source, const char* name,
+                        int n_options, const char* const* options,
+                        int n_headers, const char* const* headers,
+                        const char* const* header_names,
+                        int n_names, const char* const* name_expressions, char** lowered,
+                        void** code, size_t* code_len, char** log) {
   if (!source || !code || !code_len || !log) return fail_invalid("rt_compile: null argument");
+  if (n_names < 0 || (n_names > 0 && (!name_expressions || !lowered)))
+    return fail_invalid("rt_compile_named: bad name expression arguments");
   *code = nullptr;
   *code_len = 0;
   *log = nullptr;
+  for (int i = 0; i < n_names; ++i) lowered[i] = nullptr;
   hiprtcProgram prog = nullptr;
   hiprtcResult r = hiprtcCreateProgram(&prog, source, name ? name : "kernel.hip", n_headers,
                                        const_cast<const char**>(headers),
@@ -169,6 +173,14 @@ int rt_compile(const char* source, const char* name,
   if (r != HIPRTC_SUCCESS) {
     *log = dup_string("");
     return fail_rtc(r, "hiprtcCreateProgram");
+  }
+  for (int i = 0; i < n_names; ++i) {
+    r = hiprtcAddNameExpression(prog, name_expressions[i]);
+    if (r != HIPRTC_SUCCESS) {
+      *log = dup_string("");
+      hiprtcDestroyProgram(&prog);
+      return fail_rtc(r, "hiprtcAddNameExpression");
+    }
   }
   hiprtcResult rc = hiprtcCompileProgram(prog, n_options, const_cast<const char**>(options));
   size_t log_size = 0;
@@ -183,26 +195,54 @@ int rt_compile(const char* source, const char* name,
     hiprtcDestroyProgram(&prog);
     return fail_rtc(rc, "hiprtcCompileProgram");
   }
+  // lowered names live inside the program object: copy them before it goes
+  for (int i = 0; i < n_names; ++i) {
+    const char* low = nullptr;
+    r = hiprtcGetLoweredName(prog, name_expressions[i], &low);
+    if (r != HIPRTC_SUCCESS || !low) {
+      for (int k = 0; k < i; ++k) { std::free(lowered[k]); lowered[k] = nullptr; }
+      hiprtcDestroyProgram(&prog);
+      return fail_rtc(r != HIPRTC_SUCCESS ? r : HIPRTC_ERROR_NAME_EXPRESSION_NOT_VALID,
+                      "hiprtcGetLoweredName");
+    }
+    lowered[i] = dup_string(low);
+  }
   size_t size = 0;
   r = hiprtcGetCodeSize(prog, &size);
-  if (r != HIPRTC_SUCCESS) {
-    hiprtcDestroyProgram(&prog);
-    return fail_rtc(r, "hiprtcGetCodeSize");
+  void* buf = nullptr;
+  if (r == HIPRTC_SUCCESS) {
+    buf = std::malloc(size ? size : 1);
+    if (buf) r = hiprtcGetCode(prog, static_cast<char*>(buf));
   }
-  void* buf = std::malloc(size ? size : 1);
-  if (!buf) {
-    hiprtcDestroyProgram(&prog);
-    return fail_invalid("rt_compile: out of host memory");
-  }
-  r = hiprtcGetCode(prog, static_cast<char*>(buf));
   hiprtcDestroyProgram(&prog);
-  if (r != HIPRTC_SUCCESS) {
+  if (r != HIPRTC_SUCCESS || !buf) {
     std::free(buf);
-    return fail_rtc(r, "hiprtcGetCode");
+    for (int k = 0; k < n_names; ++k) { std::free(lowered[k]); lowered[k] = nullptr; }
+    if (r != HIPRTC_SUCCESS) return fail_rtc(r, "hiprtcGetCode");
+    return fail_invalid("rt_compile: out of host memory");
   }
   *code = buf;
   *code_len = size;
   return 0;
+}
+
+int rt_compile(const char* source, const char* name,
+               int n_options, const char* const* options,
+               int n_headers, const char* const* headers,
+               const char* const* header_names,
+               void** code, size_t* code_len, char** log) {
+  return compile_impl(source, name, n_options, options, n_headers, headers, header_names,
+                      0, nullptr, nullptr, code, code_len, log);
+}
+
+int rt_compile_named(const char* source, const char* name,
+                     int n_options, const char* const* options,
+                     int n_headers, const char* const* headers,
+                     const char* const* header_names,
+                     int n_names, const char* const* name_expressions, char** lowered_names,
+                     void** code, size_t* code_len, char** log) {
+  return compile_impl(source, name, n_options, options, n_headers, headers, header_names,
+                      n_names, name_expressions, lowered_names, code, code_len, log);
 }
 
 void rt_free_buffer(void* p) { std::free(p); }

@@ -10,6 +10,7 @@ import ctypes
 import hashlib
 import os
 import re
+import struct
 import sys
 import threading
 
@@ -113,18 +114,39 @@ def get_arch(device_id=None):
     return _device.get_device_properties(device_id)['arch'].split(':')[0]
 
 
-def compile_source(source, options=(), arch='gfx950', name='kernel.hip'):
-    """Compiles HIP source to a gfx950 code object (bytes); no caching."""
-    opts = ('--offload-arch=' + arch,) + _BASE_OPTIONS + (
+# Options of user-written (raw) kernels: no contraction override -- the source
+# is the user's, so are its floating-point semantics.
+_RAW_BASE_OPTIONS = (
+    '-std=c++17', '-O3',
+    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+)
+
+
+def compile_source(source, options=(), arch='gfx950', name='kernel.hip',
+                   base_options=_BASE_OPTIONS, name_expressions=None, with_log=False):
+    """Compiles HIP source to a gfx950 code object (bytes); no caching.  With
+    ``name_expressions`` or ``with_log`` returns ``(code, [lowered name per
+    expression], compiler log)``."""
+    opts = ('--offload-arch=' + arch,) + tuple(base_options) + (
         '-I' + _INCLUDE_DIR,) + tuple(options)
     enc = [o.encode() for o in opts]
     c_opts = (ctypes.c_char_p * len(enc))(*enc)
     code = ctypes.c_void_p()
     size = ctypes.c_size_t(0)
     log = ctypes.c_void_p()
-    status = _rt.lib.rt_compile(
-        source.encode(), name.encode(), len(enc), c_opts, 0, None, None,
-        ctypes.byref(code), ctypes.byref(size), ctypes.byref(log))
+    lowered = None
+    if name_expressions:
+        names = [n.encode() for n in name_expressions]
+        c_names = (ctypes.c_char_p * len(names))(*names)
+        lowered = (ctypes.c_void_p * len(names))()
+        status = _rt.lib.rt_compile_named(
+            source.encode(), name.encode(), len(enc), c_opts, 0, None, None,
+            len(names), c_names, lowered,
+            ctypes.byref(code), ctypes.byref(size), ctypes.byref(log))
+    else:
+        status = _rt.lib.rt_compile(
+            source.encode(), name.encode(), len(enc), c_opts, 0, None, None,
+            ctypes.byref(code), ctypes.byref(size), ctypes.byref(log))
     try:
         log_text = ctypes.string_at(log.value).decode(errors='replace') \
             if log.value else ''
@@ -136,12 +158,19 @@ def compile_source(source, options=(), arch='gfx950', name='kernel.hip'):
                     exc.dump(sys.stderr)
                 raise exc
             _rt.check(status)
-        return ctypes.string_at(code.value, size.value)
+        binary = ctypes.string_at(code.value, size.value)
+        if lowered is None:
+            return (binary, [], log_text) if with_log else binary
+        return binary, [ctypes.string_at(p).decode() for p in lowered], log_text
     finally:
         if code.value:
             _rt.lib.rt_free_buffer(code)
         if log.value:
             _rt.lib.rt_free_buffer(log)
+        if lowered is not None:
+            for p in lowered:
+                if p:
+                    _rt.lib.rt_free_buffer(p)
 
 
 def _cache_key(source, options, arch):
@@ -199,6 +228,98 @@ def compile_with_cache(source, options=()):
     mod.load(code)
     with _memo_lock:
         mod = _module_memo.setdefault(key, mod)
+    return mod
+
+
+# Cache entries of modules built with name expressions store the lowered names
+# ahead of the code object, in the reference's layout
+# (cupy/cuda/compiler.py:545-621): magic, uint32 count, count x (uint32 length,
+# UTF-8 bytes), code object; names ordered by sorted(name_expressions).
+_PAYLOAD_MAGIC = b'\x93CUPYNE\x00'
+
+
+def _encode_named_payload(lowered, code):
+    parts = [_PAYLOAD_MAGIC, struct.pack('<I', len(lowered))]
+    for n in lowered:
+        e = n.encode('utf-8')
+        parts.append(struct.pack('<I', len(e)))
+        parts.append(e)
+    parts.append(code)
+    return b''.join(parts)
+
+
+def _decode_named_payload(payload, count):
+    if not payload.startswith(_PAYLOAD_MAGIC):
+        return None
+    pos = len(_PAYLOAD_MAGIC)
+    if len(payload) < pos + 4:
+        return None
+    (stored,) = struct.unpack_from('<I', payload, pos)
+    pos += 4
+    if stored != count:
+        return None
+    names = []
+    for _ in range(stored):
+        if len(payload) < pos + 4:
+            return None
+        (size,) = struct.unpack_from('<I', payload, pos)
+        pos += 4
+        if len(payload) < pos + size:
+            return None
+        names.append(payload[pos:pos + size].decode('utf-8'))
+        pos += size
+    return names, payload[pos:]
+
+
+def compile_raw_with_cache(source, options=(), name_expressions=None, log_stream=None):
+    """Loaded module for user-written source (cupy/_core/raw.pyx:541-558
+    ``_get_raw_module``): no bundled headers are prepended, the user's options
+    follow the target option, and ``module.mapping`` maps each name expression
+    to its lowered symbol."""
+    options = tuple(options)
+    exprs = tuple(sorted(name_expressions)) if name_expressions else ()
+    dev = _device.get_device_id()
+    key = (dev, 'raw', source, options, exprs)
+    mod = _module_memo.get(key)
+    if mod is not None and log_stream is None:
+        stats['memo_hit'] += 1
+        return mod
+    arch = get_arch()
+    ckey = _cache_key(source, ('raw',) + options + exprs, arch)
+    use_disk = (os.environ.get('CUPY_CACHE_IN_MEMORY', '0') in ('', '0')
+                and log_stream is None)
+    payload = _get_disk_cache().load(ckey) if use_disk else None
+    lowered = None
+    code = None
+    if payload is not None:
+        if exprs:
+            dec = _decode_named_payload(payload, len(exprs))
+            if dec is not None:
+                lowered, code = dec
+        else:
+            code = payload
+    if code is None:
+        if exprs:
+            code, lowered, log_text = compile_source(
+                source, options, arch, base_options=_RAW_BASE_OPTIONS,
+                name_expressions=exprs)
+            payload = _encode_named_payload(lowered, code)
+        else:
+            code, _, log_text = compile_source(
+                source, options, arch, base_options=_RAW_BASE_OPTIONS, with_log=True)
+            payload = code
+        if log_stream is not None and log_text:
+            log_stream.write(log_text)
+        stats['compiled'] += 1
+        if use_disk:
+            _get_disk_cache().save(ckey, payload, None)
+    else:
+        stats['disk_hit'] += 1
+    mod = _function.Module()
+    mod.load(code)
+    mod.mapping = dict(zip(exprs, lowered)) if exprs else None
+    with _memo_lock:
+        _module_memo[key] = mod
     return mod
 
 

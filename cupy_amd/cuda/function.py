@@ -62,6 +62,7 @@ class Module:
         self.ptr = 0
         self.code = None
         self._metadata = None
+        self.mapping = None       # name expression -> lowered symbol
 
     @property
     def metadata(self):
@@ -86,6 +87,11 @@ class Module:
         p = ctypes.c_void_p()
         _rt.check(_rt.lib.rt_module_load(self.code, ctypes.byref(p)))
         self.ptr = p.value or 0
+
+    def load_file(self, filename):
+        """Loads a code object (.hsaco / .co) from a file."""
+        with open(filename, 'rb') as f:
+            self.load(f.read())
 
     def get_function(self, name):
         return Function(self, name)
@@ -173,22 +179,26 @@ class Function:
             _rt.check(status)
 
     def __call__(self, grid, block, args, shared_mem=0, stream=None):
-        """Launch with one Python object per kernel parameter."""
-        grid = tuple(grid) + (1,) * (3 - len(grid))
-        block = tuple(block) + (1,) * (3 - len(block))
-        bufs = [ctypes.create_string_buffer(b, len(b))
-                for b in map(_arg_to_bytes, args)]
+        """Launch with one Python object per kernel parameter.  Each object's
+        bytes are placed at the parameter's offset in the argument block, cut
+        or zero-padded to the parameter's size as recorded in the code object
+        (an array passed for a pointer parameter contributes its address)."""
+        grid = tuple(int(g) for g in grid) + (1,) * (3 - len(grid))
+        block = tuple(int(b) for b in block) + (1,) * (3 - len(block))
+        grid = tuple(max(1, g) for g in grid)
+        block = tuple(max(1, b) for b in block)
+        params = self.meta['args']
+        if len(args) != len(params):
+            raise TypeError('kernel %s takes %d arguments, %d given'
+                            % (self.name, len(params), len(args)))
+        blob = bytearray(self._arg_size)
+        for a, (offset, size, _kind) in zip(args, params):
+            b = bytes(_arg_to_bytes(a))
+            n = min(len(b), size)
+            blob[offset:offset + n] = b[:n]
         stream_ptr = (_stream.get_current_stream_ptr() if stream is None
                       else stream.ptr)
-        if _dryrun.enabled():
-            _dryrun.record_launch(self.name, grid, block, shared_mem,
-                                  b''.join(b.raw for b in bufs))
-            return
-        params = (ctypes.c_void_p * max(len(bufs), 1))(
-            *[ctypes.addressof(b) for b in bufs])
-        _rt.check(_rt.lib.rt_launch(
-            self.ptr, grid[0], grid[1], grid[2], block[0], block[1], block[2],
-            shared_mem, stream_ptr, params))
+        self.launch_packed(grid, block, bytes(blob), shared_mem, stream_ptr)
 
     def linear_launch(self, size, args, shared_mem=0, block_max_size=128,
                       stream=None):

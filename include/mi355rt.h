@@ -94,6 +94,17 @@ int rt_compile(const char* source, const char* name,
                int n_headers, const char* const* headers,
                const char* const* header_names,
                void** code, size_t* code_len, char** log);
+/* The same with C++ name expressions (nvrtc.pyx:232-250 addNameExpression /
+ * getLoweredName; used by cupy/_core/raw.pyx:439-499 `RawModule.get_function`
+ * for template kernels): `lowered_names[i]` receives the mangled symbol of
+ * `name_expressions[i]` as a malloc'd string (free each with rt_free_buffer). */
+int rt_compile_named(const char* source, const char* name,
+                     int n_options, const char* const* options,
+                     int n_headers, const char* const* headers,
+                     const char* const* header_names,
+                     int n_names, const char* const* name_expressions,
+                     char** lowered_names,
+                     void** code, size_t* code_len, char** log);
 void rt_free_buffer(void* p);
 
 /* ---- module / function / launch ------------------------------------------- */
