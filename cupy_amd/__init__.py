@@ -35,10 +35,13 @@ from cupy_amd._core._reduction import (  # noqa
     ReductionKernel, create_reduction_func)
 from cupy_amd._core.fusion import fuse  # noqa
 from cupy_amd._core.raw import RawKernel, RawModule  # noqa
-from cupy_amd._core._routines_math import sum, prod, nansum  # noqa
+from cupy_amd._core._routines_math import (  # noqa
+    sum, prod, nansum, nanprod, count_nonzero)
 from cupy_amd._core._routines_statistics import (  # noqa
-    amax, amin, argmax, argmin)
+    amax, amin, argmax, argmin, mean, var, std, ptp, nanmin, nanmax, nanmean,
+    nanvar, nanstd, nanargmax, nanargmin)
 from cupy_amd._core._routines_logic import all, any  # noqa
+from cupy_amd._core._scan import cumsum, cumprod, nancumsum, nancumprod  # noqa
 from cupy_amd._creation import (  # noqa
     empty, empty_like, zeros, zeros_like, ones, ones_like, full, full_like, arange)
 

@@ -102,6 +102,7 @@ def _fast_params(args, idx_t, partial_in, partial_out):
             parts.append('const %s %s' % (a.store_t, a.name))
     parts.append('const %s _n_out' % idx_t)
     parts.append('const %s _n_red' % idx_t)
+    parts.append('const long long _in_total')     # element count of the whole problem
     for a in args:
         if a.kind == 'in':
             parts.append('const %s _so_%s' % (idx_t, a.name))   # stride along i
@@ -111,6 +112,10 @@ def _fast_params(args, idx_t, partial_in, partial_out):
     if partial_out:
         parts.append('_type_reduce* __restrict__ _partials')
     return ', '.join(parts)
+
+
+_SIZE_INDEXERS = ('  const SizeOnly _in_ind((ptrdiff_t)_in_total); '
+                  'const SizeOnly _out_ind((ptrdiff_t)_n_out); (void)_in_ind; (void)_out_ind;')
 
 
 def _identity_decl(identity):
@@ -151,6 +156,7 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         BLOCK, name, params))
+    src.append(_SIZE_INDEXERS)
     if block_mode:
         src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (BLOCK // WAVE))
         src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
@@ -282,6 +288,7 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         BLOCK, name, params))
+    src.append(_SIZE_INDEXERS)
     src.append('  const int _lane = threadIdx.x %% %d;' % group)
     src.append('  const %s _first = ((%s)blockIdx.x * %d + threadIdx.x) / %d;' % (
         idx_t, idx_t, BLOCK, group))
@@ -411,6 +418,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         BLOCK, name, params))
+    src.append(_SIZE_INDEXERS)
     src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (
         waves * tx * vec))
     src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')

@@ -10,6 +10,7 @@ cupy/_core/_reduction.pyx (axis handling :147-176, ``_call`` :309-427,
 launched, split over the grid with a second combining pass when there are too
 few outputs to fill 256 CUs.
 """
+import re
 import struct
 import threading
 import warnings
@@ -96,6 +97,9 @@ _known_type_sizes = {
     'unsigned short': 2, 'int': 4, 'unsigned int': 4, 'long long': 8,
     'unsigned long long': 8, 'float16': 2, 'float': 4, 'double': 8,
 }
+
+
+_SIZE_CALL = re.compile(r'\b_(?:in|out)_ind\s*\.\s*size\s*\(\s*\)')
 
 
 class _AbstractReductionKernel:
@@ -242,8 +246,11 @@ class _AbstractReductionKernel:
         o_out = ostrides[len(in_arr_idx):]
 
         exprs = (map_expr, reduce_expr, post_map_expr)
+        # `_in_ind.size()` / `_out_ind.size()` are available everywhere; any
+        # other use of the indexers needs the kernel that has them
         needs_indexers = any(
-            uses_identifier(e, n) for e in exprs + (self._get_preamble_options()[0],)
+            uses_identifier(_SIZE_CALL.sub('', e), n)
+            for e in exprs + (self._get_preamble_options()[0],)
             for n in ('_in_ind', '_out_ind', '_i', '_j'))
         canonical = (len(rshape) <= 1 and len(oshape) <= 1 and not has_raw
                      and not needs_indexers and in_arr_idx)
@@ -362,7 +369,7 @@ class _AbstractReductionKernel:
                 fmt.append('P' + 'q' * (1 + 2 * a.ndim))
             else:
                 fmt.append(_scalar_struct_code(a.store_t))
-        fmt.append(ic * 2)
+        fmt.append(ic * 2 + 'q')
         for a in rargs:
             if a.kind == 'in':
                 fmt.append(ic * 2)
@@ -381,7 +388,7 @@ class _AbstractReductionKernel:
                 vals.scalar(ref, a)
         for j, a in enumerate(out_args):
             vals.ptr(nin + j, a.data.ptr)
-        vals.const(n_out, n_red)
+        vals.const(n_out, n_red, n_out * n_red)
         k = 0
         for a, p in zip(in_args, self.in_params):
             if isinstance(a, ndarray) and not p.raw:
@@ -394,7 +401,7 @@ class _AbstractReductionKernel:
 
     def _finalize_partials(self, partials, n_split, out_args, out_arr_idx, n_out,
                            so_out, in_args, reduce_expr, post_map_expr, reduce_type,
-                           typedefs, device_id, stream_ptr, rec, partials_ref):
+                           typedefs, device_id, stream_ptr, rec, partials_ref, in_total):
         """Second pass: combine ``partials[s][i]`` over s, then POST_MAP."""
         preamble, _ = self._get_preamble_options()
         tx = max(1, min(64, internal.clp2(n_out)))
@@ -423,8 +430,8 @@ class _AbstractReductionKernel:
         for j, a in enumerate(out_args):
             fmt.append('P')
             vals.ptr(nin + j, a.data.ptr)
-        fmt.append(ic * 4)
-        vals.const(n_out, n_split, 1, n_out)
+        fmt.append(ic * 2 + 'q' + ic * 2)
+        vals.const(n_out, n_split, in_total, 1, n_out)
         for k, a in enumerate(out_args):
             fmt.append(ic)
             vals.const(so_out[k] // a.dtype.itemsize)
@@ -533,7 +540,7 @@ class _AbstractReductionKernel:
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
-                stream_ptr, rec, pref)
+                stream_ptr, rec, pref, n_out * n_red)
         else:
             _launch_plan.launch(
                 rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
@@ -610,7 +617,7 @@ class _AbstractReductionKernel:
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
-                stream_ptr, rec, pref)
+                stream_ptr, rec, pref, n_out * n_red)
         else:
             _launch_plan.launch(
                 rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),

@@ -44,6 +44,21 @@ _nansum_keep_dtype = create_reduction_func(
      'out0 = type_out0_raw(a)', None), 0)
 
 
+_nanprod_auto_dtype = create_reduction_func(
+    'cupy_nanprod', _sumprod_types,
+    ('(in0 == in0) ? in0 : type_in0_raw(1)', 'a * b',
+     'out0 = type_out0_raw(a)', None), 1)
+
+_nanprod_keep_dtype = create_reduction_func(
+    'cupy_nanprod_with_dtype', _keep_types,
+    ('(in0 == in0) ? in0 : type_in0_raw(1)', 'a * b',
+     'out0 = type_out0_raw(a)', None), 1)
+
+_count_nonzero = create_reduction_func(
+    'cupy_count_nonzero', tuple('%s->q' % c for c in '?bBhHiIlLqQefd'),
+    ('(in0 != type_in0_raw(0)) ? 1 : 0', 'a + b', 'out0 = a', None), 0)
+
+
 def _ndarray_sum(self, axis, dtype, out, keepdims):
     if dtype is None:
         return _sum_auto_dtype(self, axis, dtype, out, keepdims)
@@ -99,3 +114,21 @@ def nansum(a, axis=None, dtype=None, out=None, keepdims=False):
         return _fusion_thread_local.call_reduction(
             func, a, axis=axis, dtype=dtype, out=out)
     return func(a, axis, dtype, out, keepdims)
+
+
+def nanprod(a, axis=None, dtype=None, out=None, keepdims=False):
+    """Product of array elements over the given axes, NaNs counted as one.
+
+    .. seealso:: :func:`numpy.nanprod`
+    """
+    if dtype is None:
+        return _nanprod_auto_dtype(a, axis, dtype, out, keepdims)
+    return _nanprod_keep_dtype(a, axis, dtype, out, keepdims)
+
+
+def count_nonzero(a, axis=None):
+    """Number of non-zero elements, as an array (no synchronisation).
+
+    .. seealso:: :func:`numpy.count_nonzero`
+    """
+    return _count_nonzero(a, axis=axis)

@@ -47,6 +47,23 @@ __device__ __forceinline__ min_max_st<T> _mm_pick(min_max_st<T> a, min_max_st<T>
   return r;
 }
 
+// NaN-ignoring variant: a number beats NaN; NaN survives only among NaNs.
+template <bool kMax, typename T>
+__device__ __forceinline__ min_max_st<T> _mm_pick_nanlast(min_max_st<T> a, min_max_st<T> b) {
+  const bool a_valid = a.index != -1;
+  const bool b_valid = b.index != -1;
+  const bool an = _mm_isnan(a.value), bn = _mm_isnan(b.value);
+  const bool cmp = kMax ? (a.value > b.value) : (a.value < b.value);
+  const bool a_better = (!an & bn) | (!an & !bn & cmp);
+  const bool tie = (a.value == b.value) | (an & bn);
+  bool take_a = a_better | (tie & (a.index <= b.index));
+  take_a = (take_a & a_valid) | !b_valid;
+  min_max_st<T> r;
+  r.value = take_a ? a.value : b.value;
+  r.index = take_a ? a.index : b.index;
+  return r;
+}
+
 // ---- argmin / argmax state ---------------------------------------------------
 // For element types of at most 32 bits (and 32-bit reduce indices) value and
 // index are packed into one signed 64-bit key: the high word is an
@@ -141,6 +158,10 @@ template <typename T> __device__ __forceinline__ min_max_st<T> my_argmax(
     const min_max_st<T>& a, const min_max_st<T>& b) { return _mm_pick<true, false>(a, b); }
 template <typename T> __device__ __forceinline__ min_max_st<T> my_argmax_float(
     const min_max_st<T>& a, const min_max_st<T>& b) { return _mm_pick<true, true>(a, b); }
+template <typename T> __device__ __forceinline__ min_max_st<T> my_nanmin(
+    const min_max_st<T>& a, const min_max_st<T>& b) { return _mm_pick_nanlast<false>(a, b); }
+template <typename T> __device__ __forceinline__ min_max_st<T> my_nanmax(
+    const min_max_st<T>& a, const min_max_st<T>& b) { return _mm_pick_nanlast<true>(a, b); }
 '''
 
 _int_sigs = ('?->?', 'b->b', 'B->B', 'h->h', 'H->H', 'i->i', 'I->I', 'l->l',
@@ -198,22 +219,273 @@ def _ndarray_argmin(self, axis, out, dtype, keepdims):
     return _argmin(self, axis=axis, out=out, dtype=dtype, keepdims=keepdims)
 
 
+_float_sigs = ('e->e', 'f->f', 'd->d')
+
+# NaNs are skipped; a slice of NaNs only gives NaN
+# (cupy/_core/_routines_statistics.pyx:307-326)
+nanmin = create_reduction_func(
+    'cupy_nanmin', _int_sigs + _float_sigs,
+    ('min_max_st<type_in0_raw>(in0)', 'my_nanmin(a, b)', 'out0 = a.value',
+     'min_max_st<type_in0_raw>'),
+    None, _min_max_preamble)
+
+nanmax = create_reduction_func(
+    'cupy_nanmax', _int_sigs + _float_sigs,
+    ('min_max_st<type_in0_raw>(in0)', 'my_nanmax(a, b)', 'out0 = a.value',
+     'min_max_st<type_in0_raw>'),
+    None, _min_max_preamble)
+
+# index -1 = "no element": NaNs never take part; a slice of NaNs only gives -1
+# (:365-391)
+_nanarg_sigs = tuple('%s->q' % c for c in '?BhHiIlLqQefd')
+
+_nanargmin_func = create_reduction_func(
+    'cupy_nanargmin', _nanarg_sigs,
+    ('min_max_st<type_in0_raw>(in0, _mm_isnan(in0) ? (IndexT)-1 : (IndexT)_J)',
+     'my_argmin(a, b)', 'out0 = a.index', 'min_max_st<type_in0_raw>'),
+    None, _min_max_preamble, sort_reduce_axis=False)
+
+_nanargmax_func = create_reduction_func(
+    'cupy_nanargmax', _nanarg_sigs,
+    ('min_max_st<type_in0_raw>(in0, _mm_isnan(in0) ? (IndexT)-1 : (IndexT)_J)',
+     'my_argmax(a, b)', 'out0 = a.index', 'min_max_st<type_in0_raw>'),
+    None, _min_max_preamble, sort_reduce_axis=False)
+
+# mean = sum / count, the count taken from the problem's size (:647-666)
+_mean_sigs = ('?->d', 'B->d', 'h->d', 'H->d', 'i->d', 'I->d', 'l->d', 'L->d',
+              'q->d', 'Q->d', ('e->e', (None, None, None, 'float')), 'f->f', 'd->d')
+
+_mean_core = create_reduction_func(
+    'cupy_mean', _mean_sigs,
+    ('in0', 'a + b',
+     'out0 = a / _type_reduce(_in_ind.size() / _out_ind.size())', None))
+
+_mean_core_empty = create_reduction_func(
+    'cupy_mean_empty', _mean_sigs,
+    ('in0', 'a + b',
+     'out0 = a / _type_reduce(_in_ind.size() / _out_ind.size())', None), 0)
+
+_nanmean_preamble = '''
+template <typename T>
+struct nanmean_st {
+  typedef long long ll;
+  T value;
+  ll count;
+  __device__ nanmean_st() : value(0), count(0) {}
+  __device__ nanmean_st(T v) : value(v != v ? T(0) : v), count(v != v ? 0 : 1) {}
+  __device__ nanmean_st(T v, ll c) : value(v), count(c) {}
+};
+template <typename T>
+__device__ nanmean_st<T> my_nanmean(const nanmean_st<T>& a, const nanmean_st<T>& b) {
+  return nanmean_st<T>(a.value + b.value, a.count + b.count);
+}
+'''
+
+_nanmean_func = create_reduction_func(
+    'cupy_nanmean',
+    (('e->e', ('nanmean_st<float>(static_cast<float>(in0))', None,
+               'out0 = a.value / float(a.count)', 'nanmean_st<float>')),
+     'f->f', 'd->d'),
+    ('nanmean_st<type_out0_raw>(in0)', 'my_nanmean(a, b)',
+     'out0 = a.value / type_out0_raw(a.count)', 'nanmean_st<type_out0_raw>'),
+    None, _nanmean_preamble)
+
+_count_non_nan = create_reduction_func(
+    'cupy_count_non_nan', ('e->q', 'f->q', 'd->q'),
+    ('(in0 == in0) ? 1 : 0', 'a + b', 'out0 = a', None), 0)
+
+
 def _ndarray_mean(self, axis, dtype, out, keepdims):
-    from cupy_amd._core import _ufuncs
+    if self.size == 0:
+        # NaN (and no error): numpy/numpy#13582
+        return _mean_core_empty(self, axis, dtype, out, keepdims)
+    return _mean_core(self, axis, dtype, out, keepdims)
+
+
+def _ndarray_ptp(self, axis, out, keepdims):
+    result = _amax(self, axis=axis, out=out, keepdims=keepdims)
+    result -= _amin(self, axis=axis, out=None, keepdims=keepdims)
+    return result
+
+
+_norm_preamble = '''
+template <typename T> __device__ T my_norm(T x) { return x * x; }
+'''
+
+_var_cores = {}
+
+
+def _var_core(out_type):
+    """ReductionKernel ``out = alpha * sum((x - mean)**2)`` with ``out_type``
+    output (``None``: the type of the given output array); built on first use
+    (cupy/_core/_routines_statistics.pyx:611-643)."""
+    from cupy_amd._core._reduction import ReductionKernel
+    ker = _var_cores.get(out_type)
+    if ker is None:
+        if out_type is None:
+            ker = ReductionKernel(
+                'S x, T mean, U alpha', 'U out', 'my_norm(x - mean)', 'a + b',
+                'out = alpha * a', '0', 'cupy_var_core_out', preamble=_norm_preamble)
+        else:
+            alpha_t = 'float64' if out_type == 'float64' else 'float32'
+            ker = ReductionKernel(
+                'S x, T mean, %s alpha' % alpha_t, '%s out' % out_type,
+                'my_norm(x - mean)', 'a + b', 'out = alpha * a', '0',
+                'cupy_var_core_' + out_type, preamble=_norm_preamble)
+        _var_cores[out_type] = ker
+    return ker
+
+
+def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
     import numpy
+    if axis is None:
+        axis = tuple(range(a.ndim))
+    if not isinstance(axis, tuple):
+        axis = (axis,)
     if dtype is None:
-        dtype = self.dtype if self.dtype.kind == 'f' else numpy.dtype('float64')
-    total = self.sum(axis=axis, dtype=dtype if numpy.dtype(dtype).kind == 'f'
-                     else None, keepdims=keepdims)
-    count = max(self.size // max(total.size, 1), 1) if self.size else 0
-    if count == 0:
-        count = float('nan')
-    res = _ufuncs.true_divide(total, total.dtype.type(count) if count == count
-                              else float('nan'))
-    if out is not None:
-        _ufuncs.elementwise_copy(res, out, casting='unsafe')
-        return out
-    return res.astype(dtype, copy=False)
+        if a.dtype.kind in 'biu':
+            dtype_mean = dtype_out = numpy.dtype('float64')
+        else:
+            dtype_mean = dtype_out = a.dtype
+    else:
+        dtype_mean = a.dtype
+        dtype_out = numpy.dtype(dtype)
+    items = 1
+    for ax in axis:
+        items *= a.shape[ax]
+    div = max(items - ddof, 0)
+    alpha = 1. / div if div != 0 else float('nan')
+    arrmean = a.mean(axis=axis, dtype=dtype_mean, out=None, keepdims=True)
+    if out is None:
+        name = dtype_out.name if dtype_out.name in ('float16', 'float32') else 'float64'
+        return _var_core(name)(a, arrmean, alpha, axis=axis, keepdims=keepdims)
+    out = _var_core(None)(a, arrmean, alpha, out, axis=axis, keepdims=keepdims)
+    return out.astype(dtype_out, copy=False)
+
+
+def _ndarray_std(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+    from cupy_amd._core import _ufuncs
+    ret = _ndarray_var(a, axis=axis, dtype=dtype, out=None, ddof=ddof, keepdims=keepdims)
+    return _ufuncs.sqrt(ret, dtype=dtype, out=out)
+
+
+_nanvar_preamble = '''
+template <typename S, typename T>
+__device__ T nanvar_impl(S x, T mean, long long alpha) {
+  return ((x != x) ? T(0) : T((x - mean) * (x - mean))) / alpha;
+}
+'''
+
+_nanvar_cores = {}
+
+
+def _nanvar(a, axis, dtype, out, ddof, keepdims):
+    """Variance ignoring NaNs (cupy/_core/_routines_statistics.pyx:699-760)."""
+    from cupy_amd._core._reduction import ReductionKernel
+    from cupy_amd._core import _routines_math
+    if not _nanvar_cores:
+        _nanvar_cores['new'] = ReductionKernel(
+            'S x, T sum, int64 _count, int64 ddof', 'S out',
+            'nanvar_impl(x, sum / _count, max(_count - ddof, 0LL))',
+            'a + b', 'out = a', '0', '_nanvar_core', preamble=_nanvar_preamble)
+        _nanvar_cores['out'] = ReductionKernel(
+            'S x, T sum, int64 _count, int64 ddof', 'U out',
+            'nanvar_impl(x, sum / _count, max(_count - ddof, 0LL))',
+            'a + b', 'out = a', '0', '_nanvar_core', preamble=_nanvar_preamble)
+    count = _count_non_nan(a, axis=axis, keepdims=True)
+    arrsum = _routines_math.nansum(a, axis=axis, dtype=dtype, out=None, keepdims=True)
+    if out is None:
+        return _nanvar_cores['new'](a, arrsum, count, ddof, axis=axis, keepdims=keepdims)
+    _nanvar_cores['out'](a, arrsum, count, ddof, out, axis=axis, keepdims=keepdims)
+    return out
+
+
+def _nanstd(a, axis, dtype, out, ddof, keepdims):
+    from cupy_amd._core import _ufuncs
+    var = _nanvar(a, axis, dtype, None, ddof, keepdims)
+    return _ufuncs.sqrt(var, dtype=dtype, out=out)
+
+
+def mean(a, axis=None, dtype=None, out=None, keepdims=False):
+    """Arithmetic mean along the given axes.
+
+    .. seealso:: :func:`numpy.mean`
+    """
+    return a.mean(axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+
+
+def var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+    """Variance along the given axes.
+
+    .. seealso:: :func:`numpy.var`
+    """
+    return a.var(axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims)
+
+
+def std(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+    """Standard deviation along the given axes.
+
+    .. seealso:: :func:`numpy.std`
+    """
+    return a.std(axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims)
+
+
+def ptp(a, axis=None, out=None, keepdims=False):
+    """Range (maximum - minimum) along the given axes.
+
+    .. seealso:: :func:`numpy.ptp`
+    """
+    return _ndarray_ptp(a, axis, out, keepdims)
+
+
+def nanmean(a, axis=None, dtype=None, out=None, keepdims=False):
+    """Mean ignoring NaNs.
+
+    .. seealso:: :func:`numpy.nanmean`
+    """
+    if a.dtype.kind in 'biu':
+        return a.mean(axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+    return _nanmean_func(a, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+
+
+def nanvar(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+    """Variance ignoring NaNs.
+
+    .. seealso:: :func:`numpy.nanvar`
+    """
+    if a.dtype.kind in 'biu':
+        return a.var(axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims)
+    return _nanvar(a, axis, dtype, out, ddof, keepdims)
+
+
+def nanstd(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+    """Standard deviation ignoring NaNs.
+
+    .. seealso:: :func:`numpy.nanstd`
+    """
+    if a.dtype.kind in 'biu':
+        return a.std(axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims)
+    return _nanstd(a, axis, dtype, out, ddof, keepdims)
+
+
+def nanargmax(a, axis=None, dtype=None, out=None, keepdims=False):
+    """Index of the maximum ignoring NaNs (-1 where a slice holds only NaNs).
+
+    .. seealso:: :func:`numpy.nanargmax`
+    """
+    if a.dtype.kind in 'biu':
+        return a.argmax(axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+    return _nanargmax_func(a, axis=axis, out=out, dtype=dtype, keepdims=keepdims)
+
+
+def nanargmin(a, axis=None, dtype=None, out=None, keepdims=False):
+    """Index of the minimum ignoring NaNs (-1 where a slice holds only NaNs).
+
+    .. seealso:: :func:`numpy.nanargmin`
+    """
+    if a.dtype.kind in 'biu':
+        return a.argmin(axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+    return _nanargmin_func(a, axis=axis, out=out, dtype=dtype, keepdims=keepdims)
 
 
 def amax(a, axis=None, out=None, keepdims=False):

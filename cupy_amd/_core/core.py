@@ -694,6 +694,28 @@ class ndarray:
         from cupy_amd._core import _routines_statistics
         return _routines_statistics._ndarray_mean(self, axis, dtype, out, keepdims)
 
+    def var(self, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+        from cupy_amd._core import _routines_statistics
+        return _routines_statistics._ndarray_var(
+            self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims)
+
+    def std(self, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+        from cupy_amd._core import _routines_statistics
+        return _routines_statistics._ndarray_std(
+            self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims)
+
+    def ptp(self, axis=None, out=None, keepdims=False):
+        from cupy_amd._core import _routines_statistics
+        return _routines_statistics._ndarray_ptp(self, axis, out, keepdims)
+
+    def cumsum(self, axis=None, dtype=None, out=None):
+        from cupy_amd._core import _scan
+        return _scan.cumsum(self, axis, dtype, out)
+
+    def cumprod(self, axis=None, dtype=None, out=None):
+        from cupy_amd._core import _scan
+        return _scan.cumprod(self, axis, dtype, out)
+
     def any(self, axis=None, out=None, keepdims=False):
         from cupy_amd._core import _routines_logic
         return _routines_logic._ndarray_any(self, axis, out, keepdims)

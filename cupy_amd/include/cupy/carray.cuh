@@ -303,6 +303,15 @@ _CUPY_DEV void store_vec(T* p, const Vec<T, N>& x) {
 
 }  // namespace cupy
 
+// Stand-in for a CIndexer in kernels that address their operands directly:
+// only the element count is available (``_in_ind.size() / _out_ind.size()`` is
+// how reduction post-maps ask for the number of reduced elements).
+struct SizeOnly {
+  ptrdiff_t size_;
+  __device__ __forceinline__ explicit SizeOnly(ptrdiff_t n) : size_(n) {}
+  __device__ __forceinline__ ptrdiff_t size() const { return size_; }
+};
+
 // ---------------------------------------------------------------------------
 // Wave64 / workgroup reduction helpers.
 // ---------------------------------------------------------------------------
@@ -316,6 +325,33 @@ _CUPY_DEV T shfl_xor(const T& v, int mask) {
   __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
   for (int k = 0; k < kWords; ++k) w[k] = __shfl_xor(w[k], mask, 64);
+  T r = v;
+  __builtin_memcpy(&r, w, sizeof(T));
+  return r;
+}
+
+// Value of lane (lane - delta) within groups of `kWidth` adjacent lanes; the
+// first `delta` lanes of a group keep their own value.
+template <int kWidth = 64, typename T>
+_CUPY_DEV T shfl_up(const T& v, int delta) {
+  constexpr int kWords = (sizeof(T) + 3) / 4;
+  int w[kWords] = {};
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) w[k] = __shfl_up(w[k], delta, kWidth);
+  T r = v;
+  __builtin_memcpy(&r, w, sizeof(T));
+  return r;
+}
+
+// Value of lane `src` of the caller's group of `kWidth` adjacent lanes.
+template <int kWidth = 64, typename T>
+_CUPY_DEV T shfl_idx(const T& v, int src) {
+  constexpr int kWords = (sizeof(T) + 3) / 4;
+  int w[kWords] = {};
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) w[k] = __shfl(w[k], src, kWidth);
   T r = v;
   __builtin_memcpy(&r, w, sizeof(T));
   return r;

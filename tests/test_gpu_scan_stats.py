@@ -1,0 +1,201 @@
+"""cumsum / cumprod and the statistics reductions (mean, var, std, ptp, the
+nan-variants) against NumPy on the same seeded inputs.  Integer results are
+bit-exact; floating-point results are compared within the reduction tolerance
+(the evaluation order differs from NumPy's)."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from helpers import assert_exact
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1,), (7,), (64,), (1000,), (4097,), (3, 5), (129, 33), (33, 129), (2, 3, 4),
+          (5, 1, 7), (40, 50, 6), (1 << 16,), (300, 1000)]
+
+
+def _rand(rng, shape, dtype):
+    dtype = np.dtype(dtype)
+    if dtype.kind == 'f':
+        return rng.uniform(-1, 1, shape).astype(dtype)
+    if dtype.kind == 'b':
+        return rng.integers(0, 2, shape).astype(dtype)
+    return rng.integers(-3 if dtype.kind == 'i' else 0, 4, shape).astype(dtype)
+
+
+@pytest.mark.parametrize('dtype', [np.int8, np.uint8, np.int32, np.int64, np.bool_])
+@pytest.mark.parametrize('shape', SHAPES)
+def test_cumsum_integers_exact(shape, dtype):
+    rng = np.random.default_rng(21)
+    h = _rand(rng, shape, dtype)
+    d = cp.asarray(h)
+    for axis in [None] + list(range(len(shape))):
+        assert_exact(d.cumsum(axis=axis).get(), h.cumsum(axis=axis))
+    assert_exact(cp.cumsum(d, axis=-1, dtype=np.int32).get(), h.cumsum(axis=-1, dtype=np.int32))
+
+
+@pytest.mark.parametrize('shape', [(7,), (1000,), (129, 33), (40, 50, 6)])
+def test_cumprod_integers_exact(shape):
+    rng = np.random.default_rng(22)
+    h = rng.choice(np.array([-1, 1, 1, 1, 2], dtype=np.int64), size=shape)
+    d = cp.asarray(h)
+    for axis in [None] + list(range(len(shape))):
+        assert_exact(d.cumprod(axis=axis).get(), h.cumprod(axis=axis))
+
+
+@pytest.mark.parametrize('dtype,rtol', [(np.float32, 1e-5), (np.float64, 1e-12), (np.float16, 2e-3)])
+@pytest.mark.parametrize('shape', SHAPES)
+def test_cumsum_floats(shape, dtype, rtol):
+    rng = np.random.default_rng(23)
+    h = _rand(rng, shape, dtype)
+    d = cp.asarray(h)
+    for axis in [None] + list(range(len(shape))):
+        got = d.cumsum(axis=axis).get()
+        want = np.cumsum(h.astype(np.float64), axis=axis)
+        bound = rtol * np.cumsum(np.abs(h).astype(np.float64), axis=axis) + 1e-300
+        assert got.dtype == dtype and got.shape == want.shape
+        assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+
+
+def test_large_one_dimensional_scans_use_every_pass():
+    rng = np.random.default_rng(24)
+    h = rng.integers(-5, 6, (1 << 23) + 12345).astype(np.int32)
+    d = cp.asarray(h)
+    assert_exact(d.cumsum().get(), h.cumsum())
+    hf = rng.uniform(0, 1, 1 << 22).astype(np.float32)
+    got = cp.asarray(hf).cumsum().get()
+    want = np.cumsum(hf.astype(np.float64))
+    assert np.all(np.abs(got - want) <= 1e-5 * want + 1e-6)
+    # long columns, few of them: chunks along the strided axis
+    hm = rng.integers(-5, 6, (70000, 24)).astype(np.int64)
+    assert_exact(cp.asarray(hm).cumsum(axis=0).get(), hm.cumsum(axis=0))
+    assert_exact(cp.asarray(hm.T.copy()).cumsum(axis=1).get(), hm.T.cumsum(axis=1))
+
+
+def test_scan_views_out_and_nan_variants():
+    rng = np.random.default_rng(25)
+    h = rng.integers(-3, 4, (64, 48)).astype(np.int64)
+    d = cp.asarray(h)
+    assert_exact(d.T.cumsum(axis=0).get(), h.T.cumsum(axis=0))           # non-contiguous input
+    assert_exact(d[::2, 1::3].cumsum(axis=1).get(), h[::2, 1::3].cumsum(axis=1))
+    out = cp.empty((64, 48), np.int64)
+    assert cp.cumsum(d, axis=1, out=out) is out
+    assert_exact(out.get(), h.cumsum(axis=1))
+    out_t = cp.empty((48, 64), np.int64).T                                # non-contiguous out
+    cp.cumsum(d, axis=0, out=out_t)
+    assert_exact(out_t.get(), h.cumsum(axis=0))
+    d2 = cp.asarray(h)
+    cp.cumsum(d2, axis=1, out=d2)                                         # in place
+    assert_exact(d2.get(), h.cumsum(axis=1))
+    with pytest.raises(ValueError):
+        cp.cumsum(d, axis=0, out=cp.empty((3, 3), np.int64))
+    with pytest.raises(np.exceptions.AxisError):
+        d.cumsum(axis=2)
+    f = rng.uniform(-1, 1, (50, 70))
+    f[rng.uniform(size=f.shape) < 0.2] = np.nan
+    df = cp.asarray(f)
+    for axis in (None, 0, 1):
+        np.testing.assert_allclose(cp.nancumsum(df, axis=axis).get(), np.nancumsum(f, axis=axis),
+                                   rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(cp.nancumprod(df, axis=axis).get(), np.nancumprod(f, axis=axis),
+                                   rtol=1e-10, atol=1e-300)
+    got = cp.cumsum(df, axis=1).get()
+    assert np.array_equal(np.isnan(got), np.isnan(np.cumsum(f, axis=1)))
+    e = cp.asarray(np.zeros((0, 5)))
+    assert e.cumsum(axis=0).shape == (0, 5) and e.cumsum().shape == (0,)
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64, np.int32, np.float16, np.bool_])
+@pytest.mark.parametrize('shape,axes', [((1000,), [None, 0]), ((129, 33), [None, 0, 1, (0, 1)]),
+                                        ((40, 50, 6), [None, 0, 1, 2, (0, 2), (1, 2)]),
+                                        ((300, 1000), [0, 1])])
+def test_mean_var_std_ptp(shape, axes, dtype):
+    rng = np.random.default_rng(26)
+    h = _rand(rng, shape, dtype)
+    d = cp.asarray(h)
+    tol = {np.float16: 4e-3, np.float32: 2e-5}.get(dtype, 1e-11)
+    for axis in axes:
+        for keepdims in (False, True):
+            got = d.mean(axis=axis, keepdims=keepdims).get()
+            want = h.mean(axis=axis, keepdims=keepdims)
+            assert got.dtype == want.dtype and got.shape == want.shape
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64),
+                                       rtol=tol, atol=tol)
+        if dtype is not np.bool_:
+            for ddof in (0, 1):
+                got = d.var(axis=axis, ddof=ddof).get()
+                want = h.var(axis=axis, ddof=ddof)
+                assert got.dtype == want.dtype and got.shape == want.shape
+                np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64),
+                                           rtol=20 * tol, atol=tol)
+                got = cp.std(d, axis=axis, ddof=ddof).get()
+                want = np.std(h, axis=axis, ddof=ddof)
+                assert got.dtype == want.dtype
+                np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64),
+                                           rtol=20 * tol, atol=tol)
+            assert_exact(d.ptp(axis=axis).get(), np.ptp(h, axis=axis))
+    got = cp.mean(d, axis=0, dtype=np.float64).get()
+    np.testing.assert_allclose(got, h.mean(axis=0, dtype=np.float64), rtol=1e-12, atol=1e-12)
+    out = cp.empty(np.mean(h, axis=0).shape, np.float64)
+    assert d.mean(axis=0, out=out) is out
+
+
+def test_mean_of_nothing_is_nan():
+    e = cp.asarray(np.zeros((0, 3), np.float32))
+    with np.errstate(all='ignore'):
+        assert np.isnan(e.mean().get())
+        assert e.mean(axis=1).shape == (0,)
+        assert np.isnan(e.mean(axis=0).get()).all()
+        assert np.isnan(e.var().get())
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64, np.float16])
+def test_nan_reductions(dtype):
+    rng = np.random.default_rng(27)
+    h = rng.uniform(-1, 1, (60, 90)).astype(dtype)
+    h[rng.uniform(size=h.shape) < 0.3] = np.nan
+    h[5, :] = np.nan
+    h[:, 7] = np.nan
+    d = cp.asarray(h)
+    tol = {np.float16: 4e-3, np.float32: 2e-5}.get(dtype, 1e-11)
+    import warnings
+    with np.errstate(all='ignore'):
+        with warnings.catch_warnings():
+            warnings.simplefilter('ignore')
+            for axis in (None, 0, 1):
+                assert_exact(cp.nanmin(d, axis=axis).get(), np.nanmin(h, axis=axis))
+                assert_exact(cp.nanmax(d, axis=axis).get(), np.nanmax(h, axis=axis))
+                got = cp.nanmean(d, axis=axis).get()
+                want = np.nanmean(h, axis=axis)
+                assert got.dtype == want.dtype
+                np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64),
+                                           rtol=tol, atol=tol)
+                for ddof in (0, 1):
+                    got = cp.nanvar(d, axis=axis, ddof=ddof).get()
+                    want = np.nanvar(h, axis=axis, ddof=ddof)
+                    assert got.dtype == want.dtype
+                    np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64),
+                                               rtol=20 * tol, atol=tol)
+                    got = cp.nanstd(d, axis=axis, ddof=ddof).get()
+                    np.testing.assert_allclose(got.astype(np.float64),
+                                               np.nanstd(h, axis=axis, ddof=ddof).astype(np.float64),
+                                               rtol=20 * tol, atol=tol)
+                got = cp.nanprod(d, axis=axis).get()
+                want = np.nanprod(h.astype(np.float64), axis=axis)
+                # float16 products of many factors below one underflow
+                np.testing.assert_allclose(got.astype(np.float64), want, rtol=50 * tol,
+                                           atol=1e-4 if dtype is np.float16 else 1e-30)
+    # arg-variants: slices of only NaNs give -1 (NumPy raises there)
+    good = np.ones(h.shape[0], bool)
+    good[5] = False
+    got = cp.nanargmax(d, axis=1).get()
+    assert got[5] == -1
+    ref = np.array([np.nanargmax(r) for r in h[good]])
+    assert np.array_equal(got[good], ref)
+    got = cp.nanargmin(d, axis=1).get()
+    assert got[5] == -1
+    assert np.array_equal(got[good], np.array([np.nanargmin(r) for r in h[good]]))
+    hi = rng.integers(0, 9, (20, 30)).astype(np.int32)
+    assert_exact(cp.nanargmax(cp.asarray(hi), axis=1).get(), np.nanargmax(hi, axis=1))
+    assert_exact(cp.count_nonzero(cp.asarray(hi), axis=0).get(), np.count_nonzero(hi, axis=0))
+    assert int(cp.count_nonzero(cp.asarray(hi)).get()) == np.count_nonzero(hi)
