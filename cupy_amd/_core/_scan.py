@@ -46,7 +46,8 @@ def _acc_type(t):
     return 'float' if t == 'float16' else t
 
 
-def _emit(in_t, out_t, op, skip_nan, vec, trips, idx64, group=64):
+def _emit(in_t, out_t, op, skip_nan, vec, trips, idx64, group=64, stream=(True, False),
+          ragged=True):
     acc_t = _acc_type(out_t)
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     op_c = '+' if op == _SUM else '*'
@@ -64,8 +65,27 @@ typedef %(idx_t)s _idx_t;
 #define SCAN_IDENTITY (_acc_t(%(ident)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
 #define GROUP %(group)d
+// RAGGED: a row may end inside a vector (its length is no multiple of VEC)
+#define RAGGED %(ragged)d
 __device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+
+// One round of loads of a group: TRIPS vectors per lane, all unconditional (a
+// vector that would start past the end of the chunk is read from the row start
+// instead, which always holds one; its values are not used).
+__device__ __forceinline__ void _rows_load(
+    cupy::Vec<_in_t, VEC> (&raw)[TRIPS], const _in_t* __restrict__ src, const _idx_t base,
+    const _idx_t j0, const _idx_t j1, const int lane) {
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    const _idx_t j = base + (t * GROUP + lane) * VEC;
+    const _idx_t jc = (j + VEC <= j1) ? j : 0;
+    if (VEC > 1) raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + jc);
+    else raw[t].v[0] = src[(j < j1) ? j : j0];
+  }
+}
 
 // mode 0: scan, no carry-in.  mode 1: write only the chunk totals.
 // mode 2: scan seeded with carry[chunk - 1] (the inclusive scan of the totals).
@@ -85,57 +105,78 @@ __device__ __forceinline__ void scan_rows_impl(
     const _in_t* src = in + (ptrdiff_t)row * n;
     _acc_t carry = SCAN_IDENTITY;
     if (kMode == 2 && chunk > 0) carry = totals[(ptrdiff_t)row * n_chunks + chunk - 1];
+    // the vectors of the first round; later rounds are requested one round
+    // ahead, before the current one is scanned
+    cupy::Vec<_in_t, VEC> raw[TRIPS];
+    _rows_load(raw, src, j0, j0, j1, lane);
     for (_idx_t base = j0; base < j1; base += GROUP * VEC * TRIPS) {
-      // every load of this lane first ...
-      cupy::Vec<_in_t, VEC> raw[TRIPS];
+      cupy::Vec<_in_t, VEC> next[TRIPS];
+      const _idx_t nbase = base + GROUP * VEC * TRIPS;
+      if (nbase < j1) _rows_load(next, src, nbase, j0, j1, lane);
+      _acc_t v[TRIPS][VEC];
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t) {
         const _idx_t j = base + (t * GROUP + lane) * VEC;
-        const _idx_t jc = (j + VEC <= j1) ? j : 0;       // the row start always holds a vector
-        if (VEC > 1) raw[t] = cupy::load_vec<_in_t, VEC, true>(src + jc);
-        else raw[t].v[0] = src[(j < j1) ? j : j0];
-      }
+        if (RAGGED && VEC > 1 && j + VEC > j1) {
+          // a row that ends inside this vector: element-wise, past-the-end = identity
 #pragma unroll
-      for (int t = 0; t < TRIPS; ++t) {
-        const _idx_t j = base + (t * GROUP + lane) * VEC;
-        _acc_t v[VEC];
-        if (VEC > 1 && j + VEC > j1) {
-          // ragged end of the chunk: element-wise, past-the-end = identity
-#pragma unroll
-          for (int k = 0; k < VEC; ++k) v[k] = (j + k < j1) ? _load_value(src[j + k]) : SCAN_IDENTITY;
+          for (int k = 0; k < VEC; ++k)
+            v[t][k] = (j + k < j1) ? _load_value(src[j + k]) : SCAN_IDENTITY;
         } else {
 #pragma unroll
-          for (int k = 0; k < VEC; ++k) v[k] = (j + k < j1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+          for (int k = 0; k < VEC; ++k)
+            v[t][k] = ((RAGGED ? j + k : j) < j1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
         }
 #pragma unroll
-        for (int k = 1; k < VEC; ++k) v[k] = SCAN_OP(v[k - 1], v[k]);
-        // inclusive scan of the lane totals across the wave
-        _acc_t incl = v[VEC - 1];
+        for (int k = 1; k < VEC; ++k) v[t][k] = SCAN_OP(v[t][k - 1], v[t][k]);
+      }
+      if (kMode == 1) {
+        // only the chunk total is wanted: a per-lane running value, combined
+        // across the lanes once, after the last round
+#pragma unroll
+        for (int t = 0; t < TRIPS; ++t) carry = SCAN_OP(carry, v[t][VEC - 1]);
+      } else {
+        // inclusive scans of the lane totals across the group, the TRIPS
+        // independent scans step by step side by side
+        _acc_t incl[TRIPS];
+#pragma unroll
+        for (int t = 0; t < TRIPS; ++t) incl[t] = v[t][VEC - 1];
 #pragma unroll
         for (int d = 1; d < GROUP; d <<= 1) {
-          const _acc_t o = cupy::shfl_up<GROUP>(incl, d);
-          if (lane >= d) incl = SCAN_OP(o, incl);
-        }
-        const _acc_t trip_total = cupy::shfl_idx<GROUP>(incl, GROUP - 1);
-        if (kMode != 1) {
-          _acc_t before = cupy::shfl_up<GROUP>(incl, 1);
-          before = (lane == 0) ? carry : SCAN_OP(carry, before);
-          _out_t* dst = out + (ptrdiff_t)row * n + j;
-          if (VEC > 1 && j + VEC <= j1) {
-            cupy::Vec<_out_t, VEC> r;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(SCAN_OP(before, v[k]));
-            cupy::store_vec<_out_t, VEC, false>(dst, r);
-          } else {
-#pragma unroll
-            for (int k = 0; k < VEC; ++k)
-              if (j + k < j1) dst[k] = static_cast<_out_t>(SCAN_OP(before, v[k]));
+          for (int t = 0; t < TRIPS; ++t) {
+            const _acc_t o = cupy::shfl_up<GROUP>(incl[t], d);
+            incl[t] = (lane >= d) ? SCAN_OP(o, incl[t]) : incl[t];
           }
         }
-        carry = SCAN_OP(carry, trip_total);
+#pragma unroll
+        for (int t = 0; t < TRIPS; ++t) {
+          const _idx_t j = base + (t * GROUP + lane) * VEC;
+          const _acc_t trip_total = cupy::shfl_idx<GROUP>(incl[t], GROUP - 1);
+          _acc_t before = cupy::shfl_up<GROUP>(incl[t], 1);
+          before = (lane == 0) ? carry : SCAN_OP(carry, before);
+          _out_t* dst = out + (ptrdiff_t)row * n + j;
+          if (VEC > 1 && (RAGGED ? j + VEC <= j1 : j < j1)) {
+            cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(SCAN_OP(before, v[t][k]));
+            cupy::store_vec<_out_t, VEC, NT_STORE>(dst, r);
+          } else if (RAGGED || VEC == 1) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k)
+              if (j + k < j1) dst[k] = static_cast<_out_t>(SCAN_OP(before, v[t][k]));
+          }
+          carry = SCAN_OP(carry, trip_total);
+        }
       }
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) raw[t] = next[t];
     }
-    if (kMode == 1 && lane == 0) totals[(ptrdiff_t)row * n_chunks + chunk] = carry;
+    if (kMode == 1) {
+#pragma unroll
+      for (int m = GROUP / 2; m > 0; m >>= 1) carry = SCAN_OP(carry, cupy::shfl_xor(carry, m));
+      if (lane == 0) totals[(ptrdiff_t)row * n_chunks + chunk] = carry;
+    }
   }
 }
 
@@ -168,7 +209,7 @@ __device__ __forceinline__ void scan_cols_impl(
       cupy::Vec<_in_t, VEC> raw[TRIPS];
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t)
-        raw[t] = cupy::load_vec<_in_t, VEC, true>(in + col + (ptrdiff_t)(j + t) * inner);
+        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + col + (ptrdiff_t)(j + t) * inner);
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t) {
         cupy::Vec<_out_t, VEC> r;
@@ -177,18 +218,18 @@ __device__ __forceinline__ void scan_cols_impl(
           run[k] = SCAN_OP(run[k], _load_value(raw[t].v[k]));
           r.v[k] = static_cast<_out_t>(run[k]);
         }
-        if (kMode != 1) cupy::store_vec<_out_t, VEC, false>(out + col + (ptrdiff_t)(j + t) * inner, r);
+        if (kMode != 1) cupy::store_vec<_out_t, VEC, NT_STORE>(out + col + (ptrdiff_t)(j + t) * inner, r);
       }
     }
     for (; j < j1; ++j) {
-      const cupy::Vec<_in_t, VEC> raw = cupy::load_vec<_in_t, VEC, true>(in + col + (ptrdiff_t)j * inner);
+      const cupy::Vec<_in_t, VEC> raw = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + col + (ptrdiff_t)j * inner);
       cupy::Vec<_out_t, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) {
         run[k] = SCAN_OP(run[k], _load_value(raw.v[k]));
         r.v[k] = static_cast<_out_t>(run[k]);
       }
-      if (kMode != 1) cupy::store_vec<_out_t, VEC, false>(out + col + (ptrdiff_t)j * inner, r);
+      if (kMode != 1) cupy::store_vec<_out_t, VEC, NT_STORE>(out + col + (ptrdiff_t)j * inner, r);
     }
     if (kMode == 1) {
 #pragma unroll
@@ -215,16 +256,19 @@ COLS_KERNEL(cupy_scan_cols, 0)
 COLS_KERNEL(cupy_scan_cols_totals, 1)
 COLS_KERNEL(cupy_scan_cols_seeded, 2)
 ''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident,
-           vec=vec, trips=trips, conv=conv, block=_BLOCK, group=group)
+           vec=vec, trips=trips, conv=conv, block=_BLOCK, group=group,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
+           ragged=1 if ragged else 0)
 
 
-def _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group=64):
+def _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group=64,
+            stream=(True, False), ragged=True):
     key = (_device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
-           trips, idx64, group)
+           trips, idx64, group, stream, ragged)
     mod = _memo.get(key)
     if mod is None:
         src = _emit(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
-                    vec, trips, idx64, group)
+                    vec, trips, idx64, group, stream, ragged)
         mod = compiler.compile_with_cache(src)
         with _lock:
             mod = _memo.setdefault(key, mod)
@@ -245,6 +289,16 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
     idx64 = outer * n * inner > 0x7fffffff - (1 << 24)
     ic = 'q' if idx64 else 'i'
     item = max(in_dtype.itemsize, out_dtype.itemsize)
+    total = outer * n * inner
+    setting = _tuning.get('scan_stream')
+    if setting == 'auto':
+        # Inputs stream.  Many rows (or column strips) are written at once, far
+        # apart in memory: such writes gain from being collected in the
+        # memory-side cache as long as the output fits it.
+        stream = (True, total * out_dtype.itemsize > _tuning.get('cache_bytes'))
+    else:
+        stream = _tuning.stream_policy(setting, total * in_dtype.itemsize,
+                                       total * out_dtype.itemsize)
     if inner == 1:
         vec = max(1, 16 // item)
         while vec > 1 and (src.data.ptr % (vec * in_dtype.itemsize)
@@ -255,20 +309,21 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         # with up to four vectors; long rows: whole waves
         trips = 4
         group = _WAVE
-        while group > 1 and (group // 2) * vec * trips >= n:
-            group //= 2
         while trips > 1 and group * vec * (trips // 2) >= n:
             trips //= 2
+        while group > 1 and (group // 2) * vec * trips >= n:
+            group //= 2
         per_group = group * vec * trips
         # enough waves to fill the device: cut rows into chunks if there are few
-        want = cus * 16
+        want = cus * _tuning.get('scan_waves_per_cu')
         n_chunks = 1
         if may_chunk and group == _WAVE and outer < want and n > 2 * per_group:
             n_chunks = min((want + outer - 1) // outer, (n + per_group - 1) // per_group)
         chunk_len = (n + n_chunks - 1) // n_chunks
         chunk_len = (chunk_len + per_group - 1) // per_group * per_group
         n_chunks = (n + chunk_len - 1) // chunk_len
-        mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group)
+        mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group, stream,
+                      ragged=n % vec != 0)
         groups = outer * n_chunks
         per_block = _BLOCK // group
         grid = max(1, min((groups + per_block - 1) // per_block, cus * 32))
@@ -295,7 +350,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
             n_chunks = min((want + threads - 1) // threads, n // 64)
         chunk_len = (n + n_chunks - 1) // n_chunks
         n_chunks = (n + chunk_len - 1) // chunk_len
-        mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64)
+        mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, 64, stream)
         work = threads * n_chunks
         grid = max(1, min((work + _BLOCK - 1) // _BLOCK, cus * 64))
         fmt = '@PPP' + ic * 5

@@ -33,6 +33,8 @@ _params = {
     'rows_group_rows_per_lane': 64,   # grid cap for sub-wave groups: CUs * this workgroups
     'cols_stream': True,
     'cols_unroll': 1,
+    'scan_stream': 'auto',      # non-temporal hints of the scan kernels
+    'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
 }
