@@ -39,20 +39,21 @@ HBM_PEAK_GBPS = 8000.0
 # WRITE_SIZE counters, scaled by what the same counters read for the plain copy
 # kernel that --calibrate adds (2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE on this
 # device); the summary of those runs is profiles/pmc_traffic_bench_suite.md.
-# Operations that share a kernel name and launch shape with another one of a
-# different size cannot be told apart in the counter output and are left out.
+# Two-pass reductions count both of their kernels.
 MEASURED_TRAFFIC_BYTES = {
-    'C1 saxpy f32 2^26': 536850563 + 268416769,
-    'C2a x.T*y f32(T)xf16 8192^2': 269876044 + 268504827,
-    'C2b tmp+1 f32 8192^2': 268438400 + 268477053,
-    'C3 sum float32 axis=1 16384^2': 1073664650 + 524252,
-    'C3 sum float64 axis=1 8192^2': 536847235 + 262126,
-    'C3 sum float32 axis=0 16384^2': 1073633294 + 2097006,
-    'C3 sum float32 axis=None 16384^2': 1073633294 + 2097006,
-    'C4 argmin i32 (2^20,128)': 536866305 + 8388344,
-    'C4 argmax i32 (2^20,128)': 536866305 + 8388344,
-    'C4 argmax f32 (2^16,4096)': 1073634573 + 524288,
-    'C5 fused sum((x-y)^2*w) f16 (2^18,256)': 268475643 + 1048503,
+    'C1 saxpy f32 2^26': 536849410 + 268422273,
+    'C2a x.T*y f32(T)xf16 8192^2': 269906693 + 268539003,
+    'C2b tmp+1 f32 8192^2': 268435456 + 268473854,
+    'C3 sum float32 axis=1 16384^2': 1073677445 + 524710,
+    'C3 sum float32 axis=0 16384^2': 1073677317 + 2097049 + 2122574 + 65533,
+    'C3 sum float32 axis=None 16384^2': 1073678341 + 65629 + 11391 + 32,
+    'C3 sum float64 axis=1 8192^2': 536851714 + 262259,
+    'C3 sum float64 axis=0 8192^2': 536851458 + 2097049 + 2122574 + 65533,
+    'C3 sum float64 axis=None 8192^2': 536852482 + 65597 + 19582 + 32,
+    'C4 argmax i32 (2^20,128)': 536871936 + 8393060,
+    'C4 argmin i32 (2^20,128)': 536870912 + 8392612,
+    'C4 argmax f32 (2^16,4096)': 1073712898 + 524998,
+    'C5 fused sum((x-y)^2*w) f16 (2^18,256)': 268461054 + 1048557,
 }
 
 
