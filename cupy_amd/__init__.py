@@ -49,23 +49,6 @@ max = amax
 min = amin
 
 
-def mean(a, axis=None, dtype=None, out=None, keepdims=False):
-    """Arithmetic mean along the given axes."""
-    return a.mean(axis=axis, dtype=dtype, out=out, keepdims=keepdims)
-
-
-def where(condition, x=None, y=None):
-    """Elementwise selection ``condition ? x : y``."""
-    if x is None or y is None:
-        raise NotImplementedError('where() with one argument is not supported')
-    return _ufuncs_module._where_ufunc(condition.astype('?', copy=False), x, y)
-
-
-def clip(a, a_min, a_max, out=None):
-    """Limits the values of an array to ``[a_min, a_max]``."""
-    return _ufuncs_module._clip(a, a_min, a_max, out=out)
-
-
 def transpose(a, axes=None):
     return a.transpose(axes)
 

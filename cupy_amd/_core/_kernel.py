@@ -1406,6 +1406,10 @@ class ufunc:
         raise NotImplementedError(f'`{self.name}.reduce` is not supported yet')
 
     def accumulate(self, array, axis=0, dtype=None, out=None):
+        if self.name == 'cupy_add':
+            return array.cumsum(axis, dtype, out)
+        if self.name == 'cupy_multiply':
+            return array.cumprod(axis, dtype, out)
         raise NotImplementedError(
             f'`{self.name}.accumulate` is not supported yet')
 

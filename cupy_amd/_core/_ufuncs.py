@@ -372,3 +372,279 @@ _clip = create_ufunc(
     'cupy_clip',
     tuple('%s%s%s->%s' % (c, c, c, c) for c in '?' + _INTS + _FLOATS),
     'out0 = in0 < in1 ? in1 : (in0 > in2 ? in2 : in0)')
+
+
+# ---------------------------------------------------------------------------------
+# The rest of NumPy's real-valued catalogue (reference: cupy/_math/arithmetic.py,
+# floating.py, rational.py, trigonometric.py, explog.py, misc.py, special.py,
+# cupy/_binary/elementwise.py, cupy/_logic/comparison.py).
+# ---------------------------------------------------------------------------------
+
+fabs = create_ufunc(
+    'cupy_fabs',
+    (('e->e', 'out0 = fabsf(in0)'), ('f->f', 'out0 = fabsf(in0)'), ('d->d', 'out0 = fabs(in0)')),
+    doc='Absolute value of floating-point elements.\n\n.. seealso:: :data:`numpy.fabs`')
+
+fmod = create_ufunc(
+    'cupy_fmod',
+    tuple(('%s%s->%s' % (c, c, c), 'out0 = in1 == 0 ? (out0_type)0 : (out0_type)(in0 % in1)')
+          for c in _INTS) + (
+        ('ee->e', 'out0 = fmodf(in0, in1)'), ('ff->f', 'out0 = fmodf(in0, in1)'),
+        ('dd->d', 'out0 = fmod(in0, in1)')),
+    doc='Remainder of C division (sign of the dividend).\n\n.. seealso:: :data:`numpy.fmod`')
+
+float_power = create_ufunc(
+    'cupy_float_power', (('dd->d', 'out0 = pow(in0, in1)'),),
+    doc='Power computed in float64 whatever the inputs.\n\n.. seealso:: :data:`numpy.float_power`')
+
+_gcd_preamble = '''
+template <typename T> __device__ __forceinline__ T _cupy_gcd(T a, T b) {
+  while (b != 0) { const T r = a % b; a = b; b = r; }
+  return a < 0 ? (T)(-a) : a;
+}
+template <typename T> __device__ __forceinline__ T _cupy_lcm(T a, T b) {
+  const T g = _cupy_gcd(a, b);
+  if (g == 0) return 0;
+  const T r = a / g * b;
+  return r < 0 ? (T)(-r) : r;
+}
+'''
+
+
+def _no_bool(name):
+    def raiser():
+        raise TypeError('%s cannot be computed with boolean arrays' % name)
+    return raiser
+
+
+gcd = create_ufunc(
+    'cupy_gcd', (('??->?', _no_bool('gcd')),) + _sig(_INTS, 2),
+    'out0 = _cupy_gcd(in0, in1)', preamble=_gcd_preamble,
+    doc='Greatest common divisor.\n\n.. seealso:: :data:`numpy.gcd`')
+lcm = create_ufunc(
+    'cupy_lcm', (('??->?', _no_bool('lcm')),) + _sig(_INTS, 2),
+    'out0 = _cupy_lcm(in0, in1)', preamble=_gcd_preamble,
+    doc='Least common multiple.\n\n.. seealso:: :data:`numpy.lcm`')
+
+heaviside = create_ufunc(
+    'cupy_heaviside', _sig(_FLOATS, 2),
+    'out0 = (in0 != in0) ? in0 : (in0 == 0 ? in1 : (out0_type)(in0 > 0 ? 1 : 0))',
+    doc='Heaviside step function.\n\n.. seealso:: :data:`numpy.heaviside`')
+
+_sinc_preamble = '''
+template <typename T> __device__ __forceinline__ T _cupy_sinc(T x) {
+  if (x == 0) return 1;
+  const T px = x * (T)3.14159265358979323846;
+  return sin(px) / px;
+}
+'''
+sinc = create_ufunc(
+    'cupy_sinc',
+    (('e->e', 'out0 = _cupy_sinc((float)in0)'), ('f->f', 'out0 = _cupy_sinc(in0)'),
+     ('d->d', 'out0 = _cupy_sinc(in0)')),
+    preamble=_sinc_preamble,
+    doc='Normalised sinc: sin(pi x) / (pi x).\n\n.. seealso:: :func:`numpy.sinc`')
+
+ldexp = create_ufunc(
+    'cupy_ldexp',
+    (('ei->e', 'out0 = ldexpf(in0, in1)'), ('fi->f', 'out0 = ldexpf(in0, in1)'),
+     ('el->e', 'out0 = ldexpf(in0, (int)(in1 > 65536 ? 65536 : (in1 < -65536 ? -65536 : in1)))'),
+     ('fl->f', 'out0 = ldexpf(in0, (int)(in1 > 65536 ? 65536 : (in1 < -65536 ? -65536 : in1)))'),
+     ('di->d', 'out0 = ldexp(in0, in1)'),
+     ('dl->d', 'out0 = ldexp(in0, (int)(in1 > 65536 ? 65536 : (in1 < -65536 ? -65536 : in1)))')),
+    doc='x1 * 2**x2.\n\n.. seealso:: :data:`numpy.ldexp`')
+
+frexp = create_ufunc(
+    'cupy_frexp',
+    (('e->ei', 'int _e; out0 = frexpf(in0, &_e); out1 = _e'),
+     ('f->fi', 'int _e; out0 = frexpf(in0, &_e); out1 = _e'),
+     ('d->di', 'int _e; out0 = frexp(in0, &_e); out1 = _e')),
+    doc='Mantissa and exponent of two.\n\n.. seealso:: :data:`numpy.frexp`')
+
+modf = create_ufunc(
+    'cupy_modf',
+    (('e->ee', 'float _i; out0 = modff(in0, &_i); out1 = _i'),
+     ('f->ff', 'float _i; out0 = modff(in0, &_i); out1 = _i'),
+     ('d->dd', 'double _i; out0 = modf(in0, &_i); out1 = _i')),
+    doc='Fractional and integral parts.\n\n.. seealso:: :data:`numpy.modf`')
+
+nextafter = create_ufunc(
+    'cupy_nextafter',
+    (('ee->e', 'out0 = _cupy_nextafter_half(in0, in1)'),
+     ('ff->f', 'out0 = nextafterf(in0, in1)'), ('dd->d', 'out0 = nextafter(in0, in1)')),
+    preamble='''
+__device__ __forceinline__ float16 _cupy_nextafter_half(float16 x, float16 y) {
+  // one step in the ordered integer image of the half's bits
+  unsigned short xb, yb;
+  __builtin_memcpy(&xb, &x, 2);
+  __builtin_memcpy(&yb, &y, 2);
+  const float xf = x, yf = y;
+  if (xf != xf || yf != yf) { unsigned short q = 0x7e00; float16 r; __builtin_memcpy(&r, &q, 2); return r; }
+  if (xf == yf) return y;
+  unsigned short rb;
+  if ((xb & 0x7fff) == 0) rb = (unsigned short)((yb & 0x8000) | 1);
+  else if ((xf < yf) == ((xb & 0x8000) == 0)) rb = (unsigned short)(xb + 1);
+  else rb = (unsigned short)(xb - 1);
+  float16 r; __builtin_memcpy(&r, &rb, 2); return r;
+}
+''',
+    doc='Next representable value towards x2.\n\n.. seealso:: :data:`numpy.nextafter`')
+
+_logaddexp_preamble = '''
+template <typename T> __device__ __forceinline__ T _cupy_logaddexp(T x, T y) {
+  if (x == y) return x + (T)0.693147180559945309417;       // also +-inf
+  const T d = x - y;
+  if (d > 0) return x + log1p(exp(-d));
+  if (d <= 0) return y + log1p(exp(d));
+  return x + y;                                            // NaN
+}
+template <typename T> __device__ __forceinline__ T _cupy_logaddexp2(T x, T y) {
+  const T k = (T)1.442695040888963407359924681;            // 1 / ln 2
+  if (x == y) return x + (T)1;
+  const T d = x - y;
+  if (d > 0) return x + log1p(exp2(-d)) * k;
+  if (d <= 0) return y + log1p(exp2(d)) * k;
+  return x + y;
+}
+'''
+logaddexp = create_ufunc(
+    'cupy_logaddexp',
+    (('ee->e', 'out0 = _cupy_logaddexp((float)in0, (float)in1)'),
+     ('ff->f', 'out0 = _cupy_logaddexp(in0, in1)'), ('dd->d', 'out0 = _cupy_logaddexp(in0, in1)')),
+    preamble=_logaddexp_preamble,
+    doc='log(exp(x1) + exp(x2)).\n\n.. seealso:: :data:`numpy.logaddexp`')
+logaddexp2 = create_ufunc(
+    'cupy_logaddexp2',
+    (('ee->e', 'out0 = _cupy_logaddexp2((float)in0, (float)in1)'),
+     ('ff->f', 'out0 = _cupy_logaddexp2(in0, in1)'), ('dd->d', 'out0 = _cupy_logaddexp2(in0, in1)')),
+    preamble=_logaddexp_preamble,
+    doc='log2(2**x1 + 2**x2).\n\n.. seealso:: :data:`numpy.logaddexp2`')
+
+deg2rad = create_ufunc(
+    'cupy_deg2rad',
+    (('e->e', 'out0 = (float)in0 * 0.017453292519943295f'),
+     ('f->f', 'out0 = in0 * 0.017453292519943295f'),
+     ('d->d', 'out0 = in0 * 0.017453292519943295')),
+    doc='Degrees to radians.\n\n.. seealso:: :data:`numpy.deg2rad`')
+rad2deg = create_ufunc(
+    'cupy_rad2deg',
+    (('e->e', 'out0 = (float)in0 * 57.29577951308232f'),
+     ('f->f', 'out0 = in0 * 57.29577951308232f'),
+     ('d->d', 'out0 = in0 * 57.29577951308232')),
+    doc='Radians to degrees.\n\n.. seealso:: :data:`numpy.rad2deg`')
+radians = deg2rad
+degrees = rad2deg
+
+bitwise_count = create_ufunc(
+    'cupy_bitwise_count',
+    tuple(('%s->B' % c, 'out0 = __popcll((unsigned long long)(in0 < 0 ? -in0 : in0))')
+          for c in 'bhilq') +
+    tuple(('%s->B' % c, 'out0 = __popcll((unsigned long long)in0)') for c in '?BHILQ'),
+    doc='Number of set bits of the absolute value.\n\n.. seealso:: :data:`numpy.bitwise_count`')
+
+i0 = create_ufunc(
+    'cupy_i0',
+    (('e->e', 'out0 = cyl_bessel_i0f((float)in0)'), ('f->f', 'out0 = cyl_bessel_i0f(in0)'),
+     ('d->d', 'out0 = cyl_bessel_i0(in0)')),
+    doc='Modified Bessel function of the first kind, order 0.\n\n.. seealso:: :func:`numpy.i0`')
+
+_is_close = create_ufunc(
+    'cupy_is_close',
+    (('eeee?->?', None), ('ffff?->?', None), ('dddd?->?', None)),
+    '''
+    bool equal_nan = in4;
+    if (isfinite(in0) && isfinite(in1)) {
+      out0 = fabs(in0 - in1) <= in3 + in2 * fabs(in1);
+    } else if (equal_nan) {
+      out0 = (in0 == in1) || (isnan(in0) && isnan(in1));
+    } else {
+      out0 = (in0 == in1);
+    }
+    ''')
+
+_nan_to_num = create_ufunc(
+    'cupy_nan_to_num_',
+    tuple(('%s%s%s%s->%s' % (c, c, c, c, c), 'out0 = in0') for c in '?' + _INTS) +
+    tuple(('%s%s%s%s->%s' % (c, c, c, c, c), None) for c in _FLOATS),
+    'out0 = isnan(in0) ? in1 : (isinf(in0) ? (in0 > 0 ? in2 : in3) : in0)')
+
+
+def isclose(a, b, rtol=1.e-5, atol=1.e-8, equal_nan=False):
+    """Elementwise ``|a - b| <= atol + rtol * |b|`` as a boolean array.
+
+    .. seealso:: :func:`numpy.isclose`
+    """
+    import numpy
+    from cupy_amd._core.core import array
+    a = array(a, copy=False)
+    b = array(b, copy=False)
+    dt = numpy.result_type(a.dtype, b.dtype)
+    if dt.kind != 'f':
+        dt = numpy.dtype('float64')
+    return _is_close(a.astype(dt, copy=False), b.astype(dt, copy=False),
+                     dt.type(rtol), dt.type(atol), bool(equal_nan))
+
+
+def allclose(a, b, rtol=1.e-5, atol=1.e-8, equal_nan=False):
+    """0-d boolean array: all elements close (no synchronisation).
+
+    .. seealso:: :func:`numpy.allclose`
+    """
+    return isclose(a, b, rtol, atol, equal_nan).all()
+
+
+def nan_to_num(x, copy=True, nan=0.0, posinf=None, neginf=None):
+    """Replaces NaN and infinities with finite numbers.
+
+    .. seealso:: :func:`numpy.nan_to_num`
+    """
+    import numpy
+    from cupy_amd._core.core import array
+    x = array(x, copy=False)
+    if x.dtype.kind != 'f':
+        return x.copy() if copy else x
+    info = numpy.finfo(x.dtype)
+    posinf = info.max if posinf is None else posinf
+    neginf = info.min if neginf is None else neginf
+    t = x.dtype.type
+    with numpy.errstate(all='ignore'):
+        args = (x, t(nan), t(posinf), t(neginf))
+    return _nan_to_num(*args, out=None if copy else x)
+
+
+def clip(a, a_min=None, a_max=None, out=None):
+    """Limits the values to ``[a_min, a_max]``.
+
+    .. seealso:: :func:`numpy.clip`
+    """
+    if a_min is None and a_max is None:
+        raise ValueError('array_clip: must set either max or min')
+    if a_min is None:
+        return minimum(a, a_max, out=out)
+    if a_max is None:
+        return maximum(a, a_min, out=out)
+    return _clip(a, a_min, a_max, out=out)
+
+
+def where(condition, x=None, y=None):
+    """Elements of ``x`` where ``condition`` holds, of ``y`` elsewhere.
+
+    .. seealso:: :func:`numpy.where`
+    """
+    if x is None or y is None:
+        raise NotImplementedError(
+            'where(condition) alone returns indices, which needs a stream '
+            'compaction that is not part of this package')
+    from cupy_amd._core.core import array
+    condition = array(condition, copy=False)
+    if condition.dtype != bool:
+        condition = condition.astype(bool)
+    return _where_ufunc(condition, x, y)
+
+
+def divmod(x1, x2, out1=None, out2=None):
+    """Quotient and remainder of floor division, as two arrays.
+
+    .. seealso:: :data:`numpy.divmod`
+    """
+    return floor_divide(x1, x2, out1), remainder(x1, x2, out2)
