@@ -378,14 +378,13 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
     src.append('      _s[_r] = _acc;')
     src.append('    }')
     if group > 1:
-        src.append('#pragma unroll')
-        src.append('    for (int _m = %d; _m > 0; _m >>= 1) {' % (group // 2))
-        src.append('#pragma unroll')
-        src.append('      for (int _r = 0; _r < %d; ++_r) {' % batch)
-        src.append('        _type_reduce _o = cupy::shfl_xor(_s[_r], _m);')
-        src.append('        _s[_r] = REDUCE(_s[_r], _o);')
-        src.append('      }')
-        src.append('    }')
+        m = 1
+        while m < group:
+            # the steps of the `batch` independent all-reduces side by side
+            src.append('#pragma unroll')
+            src.append('    for (int _r = 0; _r < %d; ++_r) '
+                       '_s[_r] = cupy::xor_combine<%d, false>(_s[_r], _ReduceOp());' % (batch, m))
+            m *= 2
     src.append('#pragma unroll')
     src.append('    for (int _r = 0; _r < %d; ++_r) {' % batch)
     src.append('      const %s _i = _i0 + _r * _step;' % idx_t)
@@ -511,11 +510,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     if tx < WAVE:
         src.append('#pragma unroll')
         src.append('  for (int _k = 0; _k < %d; ++_k) {' % vec)
-        src.append('#pragma unroll')
-        src.append('    for (int _m = %d; _m < %d; _m <<= 1) {' % (tx, WAVE))
-        src.append('      _type_reduce _o = cupy::shfl_xor(_acc[_k], _m);')
-        src.append('      _acc[_k] = REDUCE(_acc[_k], _o);')
-        src.append('    }')
+        src.append('    _acc[_k] = cupy::strided_allreduce<%d>(_acc[_k], _ReduceOp());' % tx)
         src.append('  }')
     src.append('  const int _wave = threadIdx.x / %d;' % WAVE)
     src.append('  if ((threadIdx.x %% %d) < %d) {' % (WAVE, tx))
@@ -597,11 +592,7 @@ def emit_generic(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('      }')
     src.append('    }')
     if tx < WAVE:
-        src.append('#pragma unroll')
-        src.append('    for (int _m = %d; _m < %d; _m <<= 1) {' % (tx, WAVE))
-        src.append('      _type_reduce _o = cupy::shfl_xor(_s, _m);')
-        src.append('      _s = REDUCE(_s, _o);')
-        src.append('    }')
+        src.append('    _s = cupy::strided_allreduce<%d>(_s, _ReduceOp());' % tx)
     src.append('    if ((threadIdx.x %% %d) < %d) _sm[(threadIdx.x / %d) * %d + _tx] = _s;' % (
         WAVE, tx, WAVE, tx))
     src.append('    __syncthreads();')

@@ -357,18 +357,91 @@ _CUPY_DEV T shfl_idx(const T& v, int src) {
   return r;
 }
 
-// Butterfly over groups of `kGroup` adjacent lanes (power of two <= 64): every
-// lane of a group ends up holding the group's reduction.  `op` must be
-// commutative (as well as associative): the two partners of an exchange apply
-// it with swapped operands.
+// One value moved between lanes by a data-parallel-primitive modifier
+// (`kCtrl`: quad permutation, row mirror / half mirror, row rotation), word by
+// word.  These run in the vector ALU; a general shuffle goes through the LDS
+// crossbar.
+template <int kCtrl, typename T>
+_CUPY_DEV T _dpp_move(const T& v) {
+  constexpr int kWords = (sizeof(T) + 3) / 4;
+  int w[kWords] = {};
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) w[k] = __builtin_amdgcn_update_dpp(w[k], w[k], kCtrl, 0xf, 0xf, false);
+  T r = v;
+  __builtin_memcpy(&r, w, sizeof(T));
+  return r;
+}
+
+// Exchange of 16-lane rows (kMask == 16) or wave halves (kMask == 32): `lo`
+// receives the value of the lower partner of every pair, `hi` that of the
+// upper one, in both partners alike.
+template <int kMask, typename T>
+_CUPY_DEV void _swap_halves(const T& v, T& lo, T& hi) {
+  constexpr int kWords = (sizeof(T) + 3) / 4;
+  unsigned w[kWords] = {}, a[kWords], b[kWords];
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) {
+    if (kMask == 16) {
+      auto r = __builtin_amdgcn_permlane16_swap(w[k], w[k], false, false);
+      a[k] = r[0]; b[k] = r[1];
+    } else {
+      auto r = __builtin_amdgcn_permlane32_swap(w[k], w[k], false, false);
+      a[k] = r[0]; b[k] = r[1];
+    }
+  }
+  lo = v; hi = v;
+  __builtin_memcpy(&lo, a, sizeof(T));
+  __builtin_memcpy(&hi, b, sizeof(T));
+}
+
+// One step of an all-reduce over lanes: combines the caller's value with that
+// of a partner lane chosen so that the steps for masks 1, 2, 4, ... together
+// cover the same lanes as exchanges with (lane ^ mask) would.
+//   kKeepLow == false: the group is reduced down to mask 1 (row reductions):
+//     masks 1 and 2 permute within quads, 4 and 8 mirror half rows / rows.
+//   kKeepLow == true: lanes that differ in their low bits must stay apart
+//     (column reductions, masks tx .. 32): masks below 16 rotate within rows.
+// Masks 16 and 32 swap rows / wave halves and apply `op` to the same pair of
+// operands, in the same order, in both partners.  `op` must be commutative
+// and associative.
+template <int kMask, bool kKeepLow, typename T, typename Op>
+_CUPY_DEV T xor_combine(const T& v, Op op) {
+  if (kMask >= 16) {
+    T lo, hi;
+    _swap_halves<kMask>(v, lo, hi);
+    return op(lo, hi);
+  }
+  if (kKeepLow) return op(v, _dpp_move<0x120 + kMask>(v));          // row_ror:kMask
+  if (kMask == 1) return op(v, _dpp_move<0xB1>(v));                  // quad_perm [1,0,3,2]
+  if (kMask == 2) return op(v, _dpp_move<0x4E>(v));                  // quad_perm [2,3,0,1]
+  if (kMask == 4) return op(v, _dpp_move<0x141>(v));                 // row_half_mirror
+  return op(v, _dpp_move<0x140>(v));                                 // row_mirror
+}
+
+template <int kMask, int kTop, bool kKeepLow> struct _AllReduce {
+  template <typename T, typename Op>
+  static _CUPY_DEV T run(T v, Op op) {
+    return _AllReduce<kMask * 2, kTop, kKeepLow>::run(xor_combine<kMask, kKeepLow>(v, op), op);
+  }
+};
+template <int kTop, bool kKeepLow> struct _AllReduce<kTop, kTop, kKeepLow> {
+  template <typename T, typename Op>
+  static _CUPY_DEV T run(T v, Op) { return v; }
+};
+
+// All-reduce over groups of `kGroup` adjacent lanes (power of two <= 64):
+// every lane of a group ends up holding the group's reduction.
 template <int kGroup, typename T, typename Op>
 _CUPY_DEV T group_allreduce(T v, Op op) {
-#pragma unroll
-  for (int m = kGroup >> 1; m > 0; m >>= 1) {
-    T other = shfl_xor(v, m);
-    v = op(v, other);
-  }
-  return v;
+  return _AllReduce<1, kGroup, false>::run(v, op);
+}
+
+// All-reduce over the lanes that share (lane % kStride): masks kStride .. 32.
+template <int kStride, typename T, typename Op>
+_CUPY_DEV T strided_allreduce(T v, Op op) {
+  return _AllReduce<kStride, 64, true>::run(v, op);
 }
 
 }  // namespace cupy
