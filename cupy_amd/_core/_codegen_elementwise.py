@@ -418,6 +418,26 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     src.append('    const %s _c0 = ((_tile / _ntr + _tr) %% _ntc) * %d;' % (idx_t, tile_c))
     src.append('    const bool _interior = (_r0 + %d <= _nr) && (_c0 + %d <= _nc);' % (
         tile_r, tile_c))
+    # Row-major inputs of an interior tile are requested first of all, for every
+    # trip of the consume loop at once: they are in flight while the transposed
+    # operands are staged, and none of them waits behind a store.
+    n_it = n_work // threads
+    pre_ops = [op for op in arrays
+               if layouts[op.name] == 'R' and ((not op.is_out) or op.read_out)]
+    for op in pre_ops:
+        src.append('    cupy::Vec<%s, %d> _pre_%s[%d];' % (op.store_t, vec, op.name, n_it))
+    if pre_ops:
+        src.append('    if (_interior) {')
+        src.append('#pragma unroll')
+        src.append('      for (int _it = 0; _it < %d; ++_it) {' % n_it)
+        src.append('        const int _w = threadIdx.x + _it * %d;' % threads)
+        src.append('        const %s _r = _r0 + _w / %d;' % (idx_t, tile_c // vec))
+        src.append('        const %s _c = _c0 + (_w %% %d) * %d;' % (idx_t, tile_c // vec, vec))
+        for op in pre_ops:
+            src.append('        _pre_%s[_it] = cupy::load_vec<%s, %d, %s>(%s);' % (
+                op.name, op.store_t, vec, ntl, gaddr(op, '_r', '_c')))
+        src.append('      }')
+        src.append('    }')
     if c_ops:
         # ---- stage transposed operands: rows are the fast direction -------------------
         src.append('    if (_interior) {')
@@ -471,8 +491,8 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         lay = layouts[op.name]
         if lay == 'R':
             if (not op.is_out) or op.read_out:
-                src.append('        cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
-                    op.store_t, vec, op.name, op.store_t, vec, ntl, gaddr(op, '_r', '_c')))
+                src.append('        cupy::Vec<%s, %d> _l_%s = _pre_%s[_it];' % (
+                    op.store_t, vec, op.name, op.name))
             else:
                 src.append('        cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
         elif lay == 'R0':

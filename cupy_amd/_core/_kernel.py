@@ -454,6 +454,10 @@ class _ElementwisePlanner:
         idx64 = size > _INT32_MAX - (1 << 24)
         unroll = _tuning.get('flat_unroll') if vec > 1 else 1
         block = _tuning.get('flat_block')
+        if len(itemsizes) <= 2 and block > 512:
+            # one stream in, one out: measured 2 % faster with smaller
+            # workgroups (the grid cap below keeps threads per CU the same)
+            block = 512
         stream_hint = _tuning.stream_policy(
             _tuning.get('flat_stream'), *self._traffic(args, nin, bcast))
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
@@ -483,7 +487,8 @@ class _ElementwisePlanner:
         nvec = size // vec
         per_block = block * unroll
         grid = max(1, min((max(nvec, size - nvec * vec) + per_block - 1) // per_block,
-                          _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu'))))
+                          _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu'))
+                          * (_tuning.get('flat_block') // block)))
         _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
                             stream_ptr)
 

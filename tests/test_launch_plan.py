@@ -280,19 +280,20 @@ def test_reduction_kernel_and_fuse_replay():
 
 def test_tuning_change_invalidates_recorded_calls():
     from cupy_amd._core import _tuning
-    k = cp.ElementwiseKernel('T x', 'T y', 'y = x + x', 'double_replay')
+    k = cp.ElementwiseKernel('T x, T w', 'T y', 'y = x + w', 'add_replay')
     x = cp.ndarray((1 << 16,), np.float32)
+    w = cp.ndarray((1 << 16,), np.float32)
     y = cp.ndarray((1 << 16,), np.float32)
-    k(x, y)
-    _, a = launches_of(lambda: k(x, y))
+    k(x, w, y)
+    _, a = launches_of(lambda: k(x, w, y))
     old = _tuning.get('flat_block')
     try:
         _tuning.set(flat_block=256)
-        _, b = launches_of(lambda: k(x, y))
+        _, b = launches_of(lambda: k(x, w, y))
         assert b[0][2] == (256, 1, 1) and a[0][2] == (old, 1, 1)
     finally:
         _tuning.set(flat_block=old)
-    _, c = launches_of(lambda: k(x, y))
+    _, c = launches_of(lambda: k(x, w, y))
     assert c[0][2] == (old, 1, 1)
 
 
