@@ -4,6 +4,7 @@ run-time compiler and kernel launch.  The sub-package keeps the reference's
 from cupy_amd.cuda import device  # noqa
 from cupy_amd.cuda import stream  # noqa
 from cupy_amd.cuda import memory  # noqa
+from cupy_amd.cuda import memory_hook  # noqa
 from cupy_amd.cuda import function  # noqa
 from cupy_amd.cuda import compiler  # noqa
 from cupy_amd.cuda import runtime  # noqa

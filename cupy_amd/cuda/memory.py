@@ -16,6 +16,7 @@ from cupy_amd import _dryrun
 from cupy_amd import _rt
 from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import stream as _stream
+from cupy_amd.cuda import memory_hook as _memory_hook
 
 _allocation_unit_size = 512
 
@@ -104,6 +105,19 @@ class PooledMemory(BaseMemory):
         if not ptr:
             return
         pool = self._pool()
+        hooks = _memory_hook.get_memory_hooks() if _memory_hook._has_memory_hooks() else None
+        if hooks:
+            kw = dict(device_id=self.device_id, mem_size=self.size, mem_ptr=ptr,
+                      pmem_id=id(self))
+            for hook in list(hooks.values()):
+                hook.free_preprocess(**kw)
+            try:
+                if pool is not None:
+                    pool._free(ptr, self.size)
+            finally:
+                for hook in list(hooks.values()):
+                    hook.free_postprocess(**kw)
+            return
         if pool is not None:
             pool._free(ptr, self.size)
 
@@ -258,29 +272,44 @@ class SingleDeviceMemoryPool:
         self._handle = ctypes.c_void_p()
         self._live = {}      # address -> MemoryPointer from a Python allocator
         self._callbacks = None
-        if allocator is None and _dryrun.enabled():
+        # Fresh memory always comes through this Python callback (a pool hit
+        # never gets here, and a device allocation costs far more than the
+        # call): that is where a custom allocator plugs in and where the
+        # alloc_* memory hooks are run.
+        if allocator is None:
             allocator = _malloc
-        if allocator is None or allocator is _malloc and not _dryrun.enabled():
-            _rt.check(_rt.lib.rt_pool_create(ctypes.byref(self._handle)))
-        else:
-            live = self._live
+        live = self._live
+        device_id = self._device_id
 
-            def alloc_cb(ctx, size, out):
+        def alloc_cb(ctx, size, out):
+            hooks = (_memory_hook.get_memory_hooks()
+                     if _memory_hook._has_memory_hooks() else None)
+            memptr = None
+            try:
+                if hooks:
+                    for hook in list(hooks.values()):
+                        hook.alloc_preprocess(device_id=device_id, mem_size=size)
                 try:
                     memptr = allocator(size)
-                except Exception:
-                    return 1
-                live[memptr.ptr] = memptr
-                out[0] = memptr.ptr
-                return 0
+                finally:
+                    if hooks:
+                        for hook in list(hooks.values()):
+                            hook.alloc_postprocess(
+                                device_id=device_id, mem_size=size,
+                                mem_ptr=memptr.ptr if memptr is not None else 0)
+            except Exception:
+                return 1
+            live[memptr.ptr] = memptr
+            out[0] = memptr.ptr
+            return 0
 
-            def free_cb(ctx, address, size):
-                live.pop(address, None)
+        def free_cb(ctx, address, size):
+            live.pop(address, None)
 
-            self._callbacks = (_rt.POOL_ALLOC_FN(alloc_cb), _rt.POOL_FREE_FN(free_cb))
-            _rt.check(_rt.lib.rt_pool_create_with_allocator(
-                ctypes.byref(self._handle), self._callbacks[0],
-                self._callbacks[1], None))
+        self._callbacks = (_rt.POOL_ALLOC_FN(alloc_cb), _rt.POOL_FREE_FN(free_cb))
+        _rt.check(_rt.lib.rt_pool_create_with_allocator(
+            ctypes.byref(self._handle), self._callbacks[0],
+            self._callbacks[1], None))
         limit = _parse_limit_string()
         if limit['size'] is not None or limit['fraction'] is not None:
             self.set_limit(**limit)
@@ -295,6 +324,26 @@ class SingleDeviceMemoryPool:
 
     # -- allocation -------------------------------------------------------------
     def malloc(self, size):
+        if _memory_hook._has_memory_hooks():
+            hooks = _memory_hook.get_memory_hooks()
+            if hooks:
+                rounded = _round_size(size)
+                memptr = None
+                for hook in list(hooks.values()):
+                    hook.malloc_preprocess(device_id=self._device_id, size=size,
+                                           mem_size=rounded)
+                try:
+                    memptr = self._malloc(size)
+                finally:
+                    for hook in list(hooks.values()):
+                        hook.malloc_postprocess(
+                            device_id=self._device_id, size=size, mem_size=rounded,
+                            mem_ptr=memptr.ptr if memptr is not None else 0,
+                            pmem_id=id(memptr.mem) if memptr is not None else 0)
+                return memptr
+        return self._malloc(size)
+
+    def _malloc(self, size):
         if size == 0:
             return MemoryPointer(Memory(0), 0)
         rounded = _round_size(size)
