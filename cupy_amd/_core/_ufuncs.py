@@ -7,6 +7,7 @@ cupy/_core/_ufuncs.py:7-13 (elementwise_copy) and cupy/_math/misc.py:197-206
 (square); the rest of the catalogue follows NumPy's ``ufunc.types``.  Complex
 loops are left out: the emitters have no complex type.
 """
+from cupy_amd._core import _fusion_thread_local
 from cupy_amd._core._kernel import create_ufunc
 
 _INTS = 'bBhHiIlLqQ'
@@ -619,6 +620,8 @@ def clip(a, a_min=None, a_max=None, out=None):
     """
     if a_min is None and a_max is None:
         raise ValueError('array_clip: must set either max or min')
+    if _fusion_thread_local.is_fusing() and a_min is not None and a_max is not None:
+        return _fusion_thread_local.call_ufunc(_clip, a, a_min, a_max, out=out)
     if a_min is None:
         return minimum(a, a_max, out=out)
     if a_max is None:
@@ -635,6 +638,8 @@ def where(condition, x=None, y=None):
         raise NotImplementedError(
             'where(condition) alone returns indices, which needs a stream '
             'compaction that is not part of this package')
+    if _fusion_thread_local.is_fusing():
+        return _fusion_thread_local.call_ufunc(_where_ufunc, condition, x, y)
     from cupy_amd._core.core import array
     condition = array(condition, copy=False)
     if condition.dtype != bool:

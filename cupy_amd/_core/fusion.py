@@ -384,7 +384,8 @@ class _FusionHistory:
         return fop
 
     def set_reduce_op(self, raw, arg, kwargs):
-        assert self.reduce_op is None
+        if self.reduce_op is not None:
+            raise NotImplementedError('Multiple reduction is not implemented yet')
         for op in raw._ops.ops:
             input_type, = op.in_types
             output_type, = op.out_types

@@ -189,3 +189,23 @@ def test_nested_fused_functions():
     x = shaped_random((64,), 'float32', 20)
     y = shaped_random((64,), 'float32', 21)
     assert_exact(outer(cp.asarray(x), cp.asarray(y)).get(), x * y + x)
+
+
+def test_fused_where_and_clip_follow_numpy():
+    rng = np.random.default_rng(41)
+    a = rng.standard_normal((70, 33)).astype(np.float32)
+    b = rng.standard_normal((70, 33)).astype(np.float32)
+
+    @cp.fuse()
+    def f(x, y):
+        return cp.where(x > y, x, y) + cp.clip(x, 0, 1)
+    got = f(cp.asarray(a), cp.asarray(b)).get()
+    want = np.where(a > b, a, b) + np.clip(a, 0, 1)
+    assert got.dtype == want.dtype
+    assert np.array_equal(got, want)
+
+    @cp.fuse()
+    def g(x):
+        return cp.sum(x) + cp.amax(x)
+    with pytest.raises(NotImplementedError):
+        g(cp.asarray(a))
