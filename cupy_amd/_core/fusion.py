@@ -679,9 +679,21 @@ class Fusion:
             _thread_local.is_old_fusing = True
             try:
                 self._memo[key] = history.get_fusion(self.func, args, self.name)
+            except Exception:
+                # Not expressible as ONE elementwise or map-reduce kernel
+                # (several reductions, arrays combined with a reduced value,
+                # ...).  The reference hands such functions to its second
+                # tracer (cupy/_core/fusion.pyx:860-871), whose multi-pass
+                # kernels need a grid-wide barrier.  Here the function runs as
+                # written: every step launches its own generated kernel on the
+                # current stream, temporaries come from the pool.  Errors of
+                # the function itself surface from that run.
+                self._memo[key] = None
             finally:
                 _thread_local.history = None
                 _thread_local.is_old_fusing = False
+        if self._memo[key] is None:
+            return self.func(*args)
         kernel, kwargs = self._memo[key]
         call_args = []
         for a in args:

@@ -161,20 +161,22 @@ def test_fused_min_max_prod():
     four_way(lambda xp: lambda a: xp.prod(a * 0.5 + 1, axis=1), [x], exact=False, rtol=1e-4)
 
 
-def test_reduction_restrictions():
+def test_functions_the_single_kernel_cannot_express_still_compute():
+    # two chained reductions, and a reduced value broadcast back over the
+    # input: neither is one map-reduce kernel; both run as kernel sequences
+    h = shaped_random((5, 7), 'float32', 19)
+
     @cp.fuse()
     def two(a):
         return cp.sum(cp.sum(a, axis=0))
 
-    with pytest.raises(NotImplementedError):
-        two(cp.zeros((3, 3), np.float32))
+    np.testing.assert_allclose(two(cp.asarray(h)).get(), h.sum(axis=0).sum(), rtol=1e-5)
 
     @cp.fuse()
     def mixed(a):
         return cp.sum(a, axis=0) + a
 
-    with pytest.raises(Exception, match='Shape mismatch'):
-        mixed(cp.zeros((3, 3), np.float32))
+    np.testing.assert_allclose(mixed(cp.asarray(h)).get(), h.sum(axis=0) + h, rtol=1e-5)
 
 
 def test_nested_fused_functions():
@@ -204,8 +206,29 @@ def test_fused_where_and_clip_follow_numpy():
     assert got.dtype == want.dtype
     assert np.array_equal(got, want)
 
+
+
+def test_functions_beyond_one_kernel_run_as_a_kernel_sequence():
+    rng = np.random.default_rng(42)
+    a = rng.standard_normal((70, 33)).astype(np.float32)
+    b = rng.standard_normal((70, 33)).astype(np.float32)
+
     @cp.fuse()
-    def g(x):
-        return cp.sum(x) + cp.amax(x)
-    with pytest.raises(NotImplementedError):
-        g(cp.asarray(a))
+    def two_reductions(x):
+        return cp.sum(x, axis=1) + cp.amax(x, axis=1)
+
+    @cp.fuse()
+    def normalise(x, y):
+        return (x - cp.sum(x, axis=0)) * y          # a reduced value meets an array
+
+    for _ in range(2):                                # second call: remembered as a sequence
+        got = two_reductions(cp.asarray(a)).get()
+        np.testing.assert_allclose(got, a.sum(axis=1) + a.max(axis=1), rtol=1e-5, atol=1e-5)
+        got = normalise(cp.asarray(a), cp.asarray(b)).get()
+        np.testing.assert_allclose(got, (a - a.sum(axis=0)) * b, rtol=1e-5, atol=1e-5)
+
+    @cp.fuse()
+    def broken(x):
+        return x + undefined_name                     # noqa: F821
+    with pytest.raises(NameError):
+        broken(cp.asarray(a))
