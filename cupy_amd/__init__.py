@@ -18,7 +18,7 @@ __version__ = '0.1.0'
 # dtypes and constants re-exported from NumPy
 from numpy import (  # noqa
     bool_, int8, int16, int32, int64, uint8, uint16, uint32, uint64,
-    float16, float32, float64, dtype, newaxis, inf, nan, pi, e)
+    float16, float32, float64, complex64, complex128, dtype, newaxis, inf, nan, pi, e)
 from numpy import result_type, can_cast, promote_types  # noqa
 from numpy.exceptions import AxisError, ComplexWarning  # noqa
 

@@ -8,7 +8,7 @@ from numpy.exceptions import ComplexWarning
 _dtype_memo = {}
 
 # dtypes the generated kernels can address
-SUPPORTED_CHARS = '?bhilqBHILQefd'
+SUPPORTED_CHARS = '?bhilqBHILQefdFD'
 
 
 def get_dtype(t):

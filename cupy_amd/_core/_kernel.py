@@ -475,7 +475,7 @@ class _ElementwisePlanner:
                 idx64=idx64, bcast=tuple(bcast), stream_hint=stream_hint, block=block)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             fmt = self._arg_format(operands, 'q' if idx64 else 'i', flat=True)
-            entry = (fn, struct.Struct(fmt), code)
+            entry = (fn, _make_packer(fmt), code)
             with self._lock:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
@@ -671,7 +671,7 @@ class _ElementwisePlanner:
                 elif o.kind == 'scalar':
                     fmt.append(_scalar_struct_code(o.store_t))
             fmt.append(ic * (2 + 2 * len(arrays)))
-            entry = (fn, struct.Struct(''.join(fmt)), code)
+            entry = (fn, _make_packer(fmt), code)
             with self._lock:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
@@ -724,7 +724,7 @@ class _ElementwisePlanner:
                     fmt.append(_scalar_struct_code(o.store_t))
                 else:
                     fmt.append('q' * (1 + 2 * o.ndim))
-            entry = (fn, struct.Struct(''.join(fmt)), code)
+            entry = (fn, _make_packer(fmt), code)
             with self._lock:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
@@ -758,6 +758,7 @@ _SCALAR_CODES = {
     'bool': '?', 'signed char': 'b', 'unsigned char': 'B', 'short': 'h',
     'unsigned short': 'H', 'int': 'i', 'unsigned int': 'I', 'long long': 'q',
     'unsigned long long': 'Q', 'float16': '2s', 'float': '4s', 'double': '8s',
+    'complex<float>': 'F', 'complex<double>': 'D',
 }
 
 
@@ -772,6 +773,50 @@ def _scalar_struct_code(ctype):
     if code == '8s':
         return 'd'
     return code
+
+
+class _ComplexPacker:
+    """``struct.Struct`` stand-in for argument blocks that hold complex
+    scalars: each takes one value on the way in and is laid out as two floats
+    at the alignment of the kernel's ``complex<T>`` (twice the part's size)."""
+    __slots__ = ('_struct', '_slots', 'size')
+
+    def __init__(self, fmt):
+        out = []
+        slots = []
+        n_values = 0
+        for ch in fmt:
+            if ch in 'FD':
+                part = 'f' if ch == 'F' else 'd'
+                align = 8 if ch == 'F' else 16
+                here = struct.calcsize(''.join(out))
+                out.append('x' * (-here % align) + part * 2)
+                slots.append(n_values)
+                n_values += 1
+            else:
+                out.append(ch)
+                if ch == '?' or (ch.isalpha() and ch != 'x'):
+                    n_values += 1
+        self._struct = struct.Struct(''.join(out))
+        self._slots = tuple(reversed(slots))
+        self.size = self._struct.size
+
+    def pack(self, *vals):
+        vals = list(vals)
+        for i in self._slots:
+            v = complex(vals[i])
+            vals[i:i + 1] = (v.real, v.imag)
+        return self._struct.pack(*vals)
+
+
+def _make_packer(fmt):
+    """Packer of an argument block from a struct format (string or list of
+    pieces) in which 'F' / 'D' stand for complex64 / complex128 scalars."""
+    if not isinstance(fmt, str):
+        fmt = ''.join(fmt)
+    if 'F' in fmt or 'D' in fmt:
+        return _ComplexPacker(fmt)
+    return struct.Struct(fmt)
 
 
 # ---------------------------------------------------------------------------------
@@ -966,7 +1011,14 @@ def fix_cast_expr(src_type, dst_type, expr):
     if src_kind == dst_kind:
         return expr
     if src_kind == 'b':
+        if dst_kind == 'c':
+            return 'static_cast<%s>((%s) ? 1 : 0)' % (_get_typename(dst_type), expr)
         return '((%s) ? 1 : 0)' % expr
+    if src_kind == 'c':
+        # to bool: NumPy's truth value; to a real type: the real part
+        return 'static_cast<%s>(%s)' % (_get_typename(dst_type), expr)
+    if dst_kind == 'c':
+        return 'static_cast<%s>(%s)' % (_get_typename(dst_type), expr)
     return expr
 
 
@@ -1428,7 +1480,7 @@ def _make_cast(src_dtype, dst_dtype):
     None when a plain C++ conversion does."""
     src = get_dtype(src_dtype)
     dst = get_dtype(dst_dtype)
-    if src.kind == dst.kind or src.kind != 'b':
+    if src.kind == dst.kind or (src.kind != 'b' and 'c' not in (src.kind, dst.kind)):
         return None
     return lambda e: fix_cast_expr(src, dst, e)
 

@@ -128,7 +128,7 @@ def call_signature(args, dev_id):
             if d.device_id != dev_id:
                 return None
             sig.append((a.dtype, a._shape, a._strides, d.ptr & 15))
-        elif t is float or t is bool:
+        elif t is float or t is bool or t is complex:
             sig.append(t)
         elif t is int:
             if not (_INT64_MIN <= a <= _INT64_MAX):

@@ -29,7 +29,7 @@ from cupy_amd._core._dtype import get_dtype
 from cupy_amd._core._kernel import (
     _get_param_info, _decide_params_type, _preprocess_args, _broadcast,
     _get_out_args_from_optionals, _get_out_args_with_params,
-    _check_peer_access, _scalar_struct_code, _max_vector_width, _aligned)
+    _check_peer_access, _scalar_struct_code, _make_packer, _max_vector_width, _aligned)
 from cupy_amd._core._scalar import CScalar, get_typename as _get_typename
 from cupy_amd._core.core import ndarray, _convert_from_cupy_like
 from cupy_amd.cuda import compiler
@@ -437,7 +437,7 @@ class _AbstractReductionKernel:
             vals.const(so_out[k] // a.dtype.itemsize)
         grid = (n_out + tx - 1) // tx
         _launch_plan.launch(rec, fn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
-                            struct.Struct(''.join(fmt)), vals, stream_ptr)
+                            _make_packer(fmt), vals, stream_ptr)
 
     # -- rows ---------------------------------------------------------------------------------
     def _launch_rows(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
@@ -536,7 +536,7 @@ class _AbstractReductionKernel:
             vals.const(chunk)
             _launch_plan.launch(
                 rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
-                struct.Struct(self._fast_format(rargs, ic, 'P' + ic)), vals, stream_ptr)
+                _make_packer(self._fast_format(rargs, ic, 'P' + ic)), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
@@ -544,7 +544,7 @@ class _AbstractReductionKernel:
         else:
             _launch_plan.launch(
                 rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
-                struct.Struct(self._fast_format(rargs, ic)), vals, stream_ptr)
+                _make_packer(self._fast_format(rargs, ic)), vals, stream_ptr)
 
     @staticmethod
     def _read_bytes(ins, n_out, n_red, so_in, sr):
@@ -613,7 +613,7 @@ class _AbstractReductionKernel:
             vals.ptr(pref, partials.ptr)
             _launch_plan.launch(
                 rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
-                struct.Struct(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
+                _make_packer(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
@@ -621,7 +621,7 @@ class _AbstractReductionKernel:
         else:
             _launch_plan.launch(
                 rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
-                struct.Struct(self._fast_format(rargs, ic)), vals, stream_ptr)
+                _make_packer(self._fast_format(rargs, ic)), vals, stream_ptr)
 
     # -- generic ------------------------------------------------------------------------------
     def _launch_generic(self, in_args, out_args, in_shape, out_shape, n_red,
@@ -692,14 +692,14 @@ class _AbstractReductionKernel:
             vals.const(*((0,) * ind.ndim))
         if not partial:
             _launch_plan.launch(rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
-                                struct.Struct(''.join(fmt)), vals, stream_ptr)
+                                _make_packer(fmt), vals, stream_ptr)
             return
         rsize = self._reduce_type_size(reduce_type, mod)
         partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
         fmt.append('P')
         vals.ptr(pref, partials.ptr)
         _launch_plan.launch(rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
-                            struct.Struct(''.join(fmt)), vals, stream_ptr)
+                            _make_packer(fmt), vals, stream_ptr)
         # second pass through the strided output views
         frargs = [r for r in rargs if r.kind in ('out', 'raw', 'scalar')]
         fkey = ('generic_final', tuple(r.key() for r in frargs), typedefs,
@@ -730,7 +730,7 @@ class _AbstractReductionKernel:
         vals.const(n_split)
         grid = max(1, min((n_out + _cg.BLOCK - 1) // _cg.BLOCK, cus * 8))
         _launch_plan.launch(rec, ffn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
-                            struct.Struct(''.join(fmt)), vals, stream_ptr)
+                            _make_packer(fmt), vals, stream_ptr)
 
     # -- debugging aids ------------------------------------------------------------------------
     @property

@@ -9,13 +9,13 @@ _sumprod_types = (
     '?->l', 'b->l', 'B->L', 'h->l', 'H->L', 'i->l', 'I->L', 'l->l', 'L->L',
     'q->q', 'Q->Q',
     ('e->e', (None, None, None, 'float')),
-    'f->f', 'd->d')
+    'f->f', 'd->d', 'F->F', 'D->D')
 
 _keep_types = (
     '?->?', 'b->b', 'B->B', 'h->h', 'H->H', 'i->i', 'I->I', 'l->l', 'L->L',
     'q->q', 'Q->Q',
     ('e->e', (None, None, None, 'float')),
-    'f->f', 'd->d')
+    'f->f', 'd->d', 'F->F', 'D->D')
 
 _sum_auto_dtype = create_reduction_func(
     'cupy_sum', _sumprod_types,
@@ -55,7 +55,7 @@ _nanprod_keep_dtype = create_reduction_func(
      'out0 = type_out0_raw(a)', None), 1)
 
 _count_nonzero = create_reduction_func(
-    'cupy_count_nonzero', tuple('%s->q' % c for c in '?bBhHiIlLqQefd'),
+    'cupy_count_nonzero', tuple('%s->q' % c for c in '?bBhHiIlLqQefdFD'),
     ('(in0 != type_in0_raw(0)) ? 1 : 0', 'a + b', 'out0 = a', None), 0)
 
 

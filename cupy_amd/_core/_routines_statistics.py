@@ -253,7 +253,8 @@ _nanargmax_func = create_reduction_func(
 
 # mean = sum / count, the count taken from the problem's size (:647-666)
 _mean_sigs = ('?->d', 'B->d', 'h->d', 'H->d', 'i->d', 'I->d', 'l->d', 'L->d',
-              'q->d', 'Q->d', ('e->e', (None, None, None, 'float')), 'f->f', 'd->d')
+              'q->d', 'Q->d', ('e->e', (None, None, None, 'float')), 'f->f', 'd->d',
+              'F->F', 'D->D')
 
 _mean_core = create_reduction_func(
     'cupy_mean', _mean_sigs,

@@ -11,6 +11,8 @@ import numpy
 from cupy_amd._core._dtype import get_dtype
 
 _typenames = {
+    numpy.dtype('complex128'): 'complex<double>',
+    numpy.dtype('complex64'): 'complex<float>',
     numpy.dtype('float64'): 'double',
     numpy.dtype('float32'): 'float',
     numpy.dtype('float16'): 'float16',
@@ -171,4 +173,9 @@ def get_scalar_literal(obj, dtype):
                 return 'CUDART_INF_F' if v > 0 else '-CUDART_INF_F'
             return repr(v) + 'f'
         return repr(v)
+    if kind == 'c':
+        v = complex(obj)
+        part = numpy.dtype('float32' if dtype.itemsize == 8 else 'float64')
+        return '%s(%s, %s)' % (get_typename(dtype), get_scalar_literal(v.real, part),
+                               get_scalar_literal(v.imag, part))
     raise TypeError(f'Unsupported dtype: {dtype}')

@@ -391,10 +391,10 @@ def scan_core(a, axis, op, dtype=None, out=None, skip_nan=False):
         dtype = numpy.dtype(dtype)
     else:
         dtype = out.dtype
-    if dtype.kind not in 'biuf':
+    if dtype.kind not in 'biufc':
         raise TypeError('scan does not support dtype %s' % dtype)
     src = a
-    if not src._c_contiguous or src.dtype.kind not in 'biuf':
+    if not src._c_contiguous or src.dtype.kind not in 'biufc':
         src = src.astype(dtype, order='C')
     if axis is None:
         shape = (a.size,)
@@ -414,7 +414,7 @@ def scan_core(a, axis, op, dtype=None, out=None, skip_nan=False):
         if may_share_bounds(a, out):
             src = a.copy()
     stream_ptr = _stream.get_current_stream_ptr()
-    _scan_contiguous(src, result, outer, n, inner, op, skip_nan and src.dtype.kind == 'f',
+    _scan_contiguous(src, result, outer, n, inner, op, skip_nan and src.dtype.kind in 'fc',
                      stream_ptr)
     if out is not None and not direct:
         _ufuncs.elementwise_copy(result, out)

@@ -4,14 +4,16 @@ NumPy's promotion) and the HIP routine of each loop.
 The arithmetic tables correspond to the reference's
 cupy/_core/_routines_math.pyx:878-1060 (add, subtract, multiply, power, ...),
 cupy/_core/_ufuncs.py:7-13 (elementwise_copy) and cupy/_math/misc.py:197-206
-(square); the rest of the catalogue follows NumPy's ``ufunc.types``.  Complex
-loops are left out: the emitters have no complex type.
+(square); the rest of the catalogue follows NumPy's ``ufunc.types``.  Complex loops
+('F', 'D') compute with ``complex<float>`` / ``complex<double>`` of
+cupy/complex.cuh.
 """
 from cupy_amd._core import _fusion_thread_local
 from cupy_amd._core._kernel import create_ufunc
 
 _INTS = 'bBhHiIlLqQ'
 _FLOATS = 'efd'
+_COMPLEX = 'FD'
 
 
 def _sig(chars, nin, out=None):
@@ -20,7 +22,7 @@ def _sig(chars, nin, out=None):
 
 elementwise_copy = create_ufunc(
     'cupy_copy',
-    _sig('?' + _INTS + _FLOATS, 1),
+    _sig('?' + _INTS + _FLOATS + _COMPLEX, 1),
     'out0 = in0',
     default_casting='unsafe')
 
@@ -30,7 +32,7 @@ def _create_arithmetic(name, op, boolop, doc):
         boolop = 'out0 = in0 %s in1' % boolop
     return create_ufunc(
         'cupy_' + name,
-        (('??->?', boolop),) + _sig(_INTS + _FLOATS, 2),
+        (('??->?', boolop),) + _sig(_INTS + _FLOATS + _COMPLEX, 2),
         'out0 = in0 %s in1' % op,
         doc=doc)
 
@@ -63,7 +65,7 @@ multiply = _create_arithmetic(
 
 true_divide = create_ufunc(
     'cupy_true_divide',
-    _sig(_INTS, 2, 'd') + _sig(_FLOATS, 2),
+    _sig(_INTS, 2, 'd') + _sig(_FLOATS + _COMPLEX, 2),
     'out0 = (out0_type)in0 / (out0_type)in1',
     doc='Elementwise true division.\n\n.. seealso:: :data:`numpy.true_divide`')
 divide = true_divide
@@ -136,26 +138,28 @@ power = create_ufunc(
     ('??->b',) + _sig(_INTS, 2) + (
         ('ee->e', 'out0 = powf(in0, in1)'),
         ('ff->f', 'out0 = powf(in0, in1)'),
-        ('dd->d', 'out0 = pow(in0, in1)')),
+        ('dd->d', 'out0 = pow(in0, in1)'),
+        ('FF->F', 'out0 = pow(in0, in1)'),
+        ('DD->D', 'out0 = pow(in0, in1)')),
     'out0 = integral_power(in0, in1)',
     preamble=_power_preamble,
     doc='Computes ``x1 ** x2`` elementwise.\n\n.. seealso:: :data:`numpy.power`')
 
 negative = create_ufunc(
     'cupy_negative',
-    (('?->?', _negative_boolean_error),) + _sig(_INTS + _FLOATS, 1),
+    (('?->?', _negative_boolean_error),) + _sig(_INTS + _FLOATS + _COMPLEX, 1),
     'out0 = -in0',
     doc='Takes numerical negative elementwise.\n\n.. seealso:: :data:`numpy.negative`')
 
 positive = create_ufunc(
     'cupy_positive',
-    (('?->?', _positive_boolean_error),) + _sig(_INTS + _FLOATS, 1),
+    (('?->?', _positive_boolean_error),) + _sig(_INTS + _FLOATS + _COMPLEX, 1),
     'out0 = +in0',
     doc='Takes numerical positive elementwise.\n\n.. seealso:: :data:`numpy.positive`')
 
 square = create_ufunc(
     'cupy_square',
-    _sig(_INTS + _FLOATS, 1),
+    _sig(_INTS + _FLOATS + _COMPLEX, 1),
     'out0 = in0 * in0',
     doc='Elementwise square of the input.\n\n.. seealso:: :data:`numpy.square`')
 
@@ -167,7 +171,9 @@ absolute = create_ufunc(
      'q->q', ('Q->Q', 'out0 = in0'),
      ('e->e', 'out0 = fabsf(in0)'),
      ('f->f', 'out0 = fabsf(in0)'),
-     ('d->d', 'out0 = fabs(in0)')),
+     ('d->d', 'out0 = fabs(in0)'),
+     ('F->f', 'out0 = abs(in0)'),
+     ('D->d', 'out0 = abs(in0)')),
     'out0 = in0 > 0 ? in0 : -in0',
     doc='Elementwise absolute value.\n\n.. seealso:: :data:`numpy.absolute`')
 abs = absolute
@@ -179,49 +185,67 @@ sign = create_ufunc(
      'q->q', ('Q->Q', 'out0 = in0 > 0'),
      ('e->e', 'out0 = isnan(in0) ? in0 : (out0_type)((in0 > 0) - (in0 < 0))'),
      ('f->f', 'out0 = isnan(in0) ? in0 : (out0_type)((in0 > 0) - (in0 < 0))'),
-     ('d->d', 'out0 = isnan(in0) ? in0 : (out0_type)((in0 > 0) - (in0 < 0))')),
+     ('d->d', 'out0 = isnan(in0) ? in0 : (out0_type)((in0 > 0) - (in0 < 0))'),
+     ('F->F', 'out0 = _cupy_csign(in0)'),
+     ('D->D', 'out0 = _cupy_csign(in0)')),
     'out0 = (in0 > 0) - (in0 < 0)',
+    preamble='''
+// z / |z|; 0 for 0, NaN for what has no direction (NumPy >= 2)
+template <typename T> __device__ __forceinline__ complex<T> _cupy_csign(const complex<T>& z) {
+  const T a = abs(z);
+  if (a == 0) return complex<T>(0, 0);
+  if (isnan(a)) return complex<T>(CUDART_NAN, CUDART_NAN);
+  if (isinf(a)) {
+    if (isinf(z.re) && isinf(z.im)) return complex<T>(CUDART_NAN, CUDART_NAN);
+    if (isinf(z.re)) return complex<T>(z.re > 0 ? 1 : -1, 0);
+    return complex<T>(0, z.im > 0 ? 1 : -1);
+  }
+  return complex<T>(z.re / a, z.im / a);
+}
+''',
     doc='Elementwise sign.\n\n.. seealso:: :data:`numpy.sign`')
 
 reciprocal = create_ufunc(
     'cupy_reciprocal',
     _sig(_INTS, 1) + (
         ('e->e', 'out0 = 1 / in0'), ('f->f', 'out0 = 1 / in0'),
-        ('d->d', 'out0 = 1 / in0')),
+        ('d->d', 'out0 = 1 / in0'),
+        ('F->F', 'out0 = in0_type(1) / in0'),
+        ('D->D', 'out0 = in0_type(1) / in0')),
     'out0 = in0 == 0 ? 0 : (1 / in0)',
     doc='Elementwise reciprocal.\n\n.. seealso:: :data:`numpy.reciprocal`')
 
 
-def _float_unary(name, f32, f64, doc):
-    return create_ufunc(
-        'cupy_' + name,
-        (('e->e', 'out0 = %s(in0)' % f32),
-         ('f->f', 'out0 = %s(in0)' % f32),
-         ('d->d', 'out0 = %s(in0)' % f64)),
-        doc=doc)
+def _float_unary(name, f32, f64, doc, cplx=None):
+    loops = (('e->e', 'out0 = %s(in0)' % f32),
+             ('f->f', 'out0 = %s(in0)' % f32),
+             ('d->d', 'out0 = %s(in0)' % f64))
+    if cplx:
+        loops += (('F->F', 'out0 = %s(in0)' % cplx), ('D->D', 'out0 = %s(in0)' % cplx))
+    return create_ufunc('cupy_' + name, loops, doc=doc)
 
 
-sqrt = _float_unary('sqrt', 'sqrtf', 'sqrt', 'Elementwise square root.')
+sqrt = _float_unary('sqrt', 'sqrtf', 'sqrt', 'Elementwise square root.', 'sqrt')
 cbrt = _float_unary('cbrt', 'cbrtf', 'cbrt', 'Elementwise cube root.')
-exp = _float_unary('exp', 'expf', 'exp', 'Elementwise exponential.')
+exp = _float_unary('exp', 'expf', 'exp', 'Elementwise exponential.', 'exp')
 exp2 = _float_unary('exp2', 'exp2f', 'exp2', 'Elementwise 2**x.')
 expm1 = _float_unary('expm1', 'expm1f', 'expm1', 'Elementwise exp(x) - 1.')
-log = _float_unary('log', 'logf', 'log', 'Elementwise natural logarithm.')
-log2 = _float_unary('log2', 'log2f', 'log2', 'Elementwise base-2 logarithm.')
-log10 = _float_unary('log10', 'log10f', 'log10', 'Elementwise base-10 logarithm.')
+log = _float_unary('log', 'logf', 'log', 'Elementwise natural logarithm.', 'log')
+log2 = _float_unary('log2', 'log2f', 'log2', 'Elementwise base-2 logarithm.', 'log2')
+log10 = _float_unary('log10', 'log10f', 'log10', 'Elementwise base-10 logarithm.', 'log10')
 log1p = _float_unary('log1p', 'log1pf', 'log1p', 'Elementwise log(1 + x).')
-sin = _float_unary('sin', 'sinf', 'sin', 'Elementwise sine.')
-cos = _float_unary('cos', 'cosf', 'cos', 'Elementwise cosine.')
-tan = _float_unary('tan', 'tanf', 'tan', 'Elementwise tangent.')
-arcsin = _float_unary('arcsin', 'asinf', 'asin', 'Elementwise inverse sine.')
-arccos = _float_unary('arccos', 'acosf', 'acos', 'Elementwise inverse cosine.')
-arctan = _float_unary('arctan', 'atanf', 'atan', 'Elementwise inverse tangent.')
-sinh = _float_unary('sinh', 'sinhf', 'sinh', 'Elementwise hyperbolic sine.')
-cosh = _float_unary('cosh', 'coshf', 'cosh', 'Elementwise hyperbolic cosine.')
-tanh = _float_unary('tanh', 'tanhf', 'tanh', 'Elementwise hyperbolic tangent.')
-arcsinh = _float_unary('arcsinh', 'asinhf', 'asinh', 'Elementwise inverse sinh.')
-arccosh = _float_unary('arccosh', 'acoshf', 'acosh', 'Elementwise inverse cosh.')
-arctanh = _float_unary('arctanh', 'atanhf', 'atanh', 'Elementwise inverse tanh.')
+sin = _float_unary('sin', 'sinf', 'sin', 'Elementwise sine.', 'sin')
+cos = _float_unary('cos', 'cosf', 'cos', 'Elementwise cosine.', 'cos')
+tan = _float_unary('tan', 'tanf', 'tan', 'Elementwise tangent.', 'tan')
+arcsin = _float_unary('arcsin', 'asinf', 'asin', 'Elementwise inverse sine.', 'asin')
+arccos = _float_unary('arccos', 'acosf', 'acos', 'Elementwise inverse cosine.', 'acos')
+arctan = _float_unary('arctan', 'atanf', 'atan', 'Elementwise inverse tangent.', 'atan')
+sinh = _float_unary('sinh', 'sinhf', 'sinh', 'Elementwise hyperbolic sine.', 'sinh')
+cosh = _float_unary('cosh', 'coshf', 'cosh', 'Elementwise hyperbolic cosine.', 'cosh')
+tanh = _float_unary('tanh', 'tanhf', 'tanh', 'Elementwise hyperbolic tangent.', 'tanh')
+arcsinh = _float_unary('arcsinh', 'asinhf', 'asinh', 'Elementwise inverse sinh.', 'asinh')
+arccosh = _float_unary('arccosh', 'acoshf', 'acosh', 'Elementwise inverse cosh.', 'acosh')
+arctanh = _float_unary('arctanh', 'atanhf', 'atanh', 'Elementwise inverse tanh.', 'atanh')
 
 
 def _rounding(name, f32, f64, doc):
@@ -266,7 +290,9 @@ maximum = create_ufunc(
     ('??->?',) + _sig(_INTS, 2) + (
         ('ee->e', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 > in1 ? in0 : in1)'),
         ('ff->f', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 > in1 ? in0 : in1)'),
-        ('dd->d', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 > in1 ? in0 : in1)')),
+        ('dd->d', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 > in1 ? in0 : in1)'),
+        ('FF->F', 'out0 = (in0 >= in1 || isnan(in0)) ? in0 : in1'),
+        ('DD->D', 'out0 = (in0 >= in1 || isnan(in0)) ? in0 : in1')),
     'out0 = in0 > in1 ? in0 : in1',
     doc='Elementwise maximum; NaNs propagate.\n\n.. seealso:: :data:`numpy.maximum`')
 
@@ -275,7 +301,9 @@ minimum = create_ufunc(
     ('??->?',) + _sig(_INTS, 2) + (
         ('ee->e', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 < in1 ? in0 : in1)'),
         ('ff->f', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 < in1 ? in0 : in1)'),
-        ('dd->d', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 < in1 ? in0 : in1)')),
+        ('dd->d', 'out0 = (isnan(in0) | isnan(in1)) ? (isnan(in0) ? in0 : in1) : (in0 < in1 ? in0 : in1)'),
+        ('FF->F', 'out0 = (in0 <= in1 || isnan(in0)) ? in0 : in1'),
+        ('DD->D', 'out0 = (in0 <= in1 || isnan(in0)) ? in0 : in1')),
     'out0 = in0 < in1 ? in0 : in1',
     doc='Elementwise minimum; NaNs propagate.\n\n.. seealso:: :data:`numpy.minimum`')
 
@@ -284,7 +312,9 @@ fmax = create_ufunc(
     ('??->?',) + _sig(_INTS, 2) + (
         ('ee->e', 'out0 = fmaxf(in0, in1)'),
         ('ff->f', 'out0 = fmaxf(in0, in1)'),
-        ('dd->d', 'out0 = fmax(in0, in1)')),
+        ('dd->d', 'out0 = fmax(in0, in1)'),
+        ('FF->F', 'out0 = (in0 >= in1 || isnan(in1)) ? in0 : in1'),
+        ('DD->D', 'out0 = (in0 >= in1 || isnan(in1)) ? in0 : in1')),
     'out0 = in0 > in1 ? in0 : in1',
     doc='Elementwise maximum ignoring NaNs.')
 
@@ -293,7 +323,9 @@ fmin = create_ufunc(
     ('??->?',) + _sig(_INTS, 2) + (
         ('ee->e', 'out0 = fminf(in0, in1)'),
         ('ff->f', 'out0 = fminf(in0, in1)'),
-        ('dd->d', 'out0 = fmin(in0, in1)')),
+        ('dd->d', 'out0 = fmin(in0, in1)'),
+        ('FF->F', 'out0 = (in0 <= in1 || isnan(in1)) ? in0 : in1'),
+        ('DD->D', 'out0 = (in0 <= in1 || isnan(in1)) ? in0 : in1')),
     'out0 = in0 < in1 ? in0 : in1',
     doc='Elementwise minimum ignoring NaNs.')
 
@@ -301,7 +333,7 @@ fmin = create_ufunc(
 def _comparison(name, op, doc):
     return create_ufunc(
         'cupy_' + name,
-        _sig('?' + _INTS + _FLOATS, 2, '?'),
+        _sig('?' + _INTS + _FLOATS + _COMPLEX, 2, '?'),
         'out0 = in0 %s in1' % op,
         doc=doc)
 
@@ -314,16 +346,16 @@ equal = _comparison('equal', '==', 'Tests elementwise ``x1 == x2``.')
 not_equal = _comparison('not_equal', '!=', 'Tests elementwise ``x1 != x2``.')
 
 logical_and = create_ufunc(
-    'cupy_logical_and', _sig('?' + _INTS + _FLOATS, 2, '?'),
+    'cupy_logical_and', _sig('?' + _INTS + _FLOATS + _COMPLEX, 2, '?'),
     'out0 = in0 && in1', doc='Elementwise logical AND.')
 logical_or = create_ufunc(
-    'cupy_logical_or', _sig('?' + _INTS + _FLOATS, 2, '?'),
+    'cupy_logical_or', _sig('?' + _INTS + _FLOATS + _COMPLEX, 2, '?'),
     'out0 = in0 || in1', doc='Elementwise logical OR.')
 logical_xor = create_ufunc(
-    'cupy_logical_xor', _sig('?' + _INTS + _FLOATS, 2, '?'),
+    'cupy_logical_xor', _sig('?' + _INTS + _FLOATS + _COMPLEX, 2, '?'),
     'out0 = !in0 != !in1', doc='Elementwise logical XOR.')
 logical_not = create_ufunc(
-    'cupy_logical_not', _sig('?' + _INTS + _FLOATS, 1, '?'),
+    'cupy_logical_not', _sig('?' + _INTS + _FLOATS + _COMPLEX, 1, '?'),
     'out0 = !in0', doc='Elementwise logical NOT.')
 
 bitwise_and = create_ufunc(
@@ -350,15 +382,15 @@ right_shift = create_ufunc(
 
 isnan = create_ufunc(
     'cupy_isnan',
-    tuple(('%s->?' % c, 'out0 = false') for c in '?' + _INTS) + _sig(_FLOATS, 1, '?'),
+    tuple(('%s->?' % c, 'out0 = false') for c in '?' + _INTS) + _sig(_FLOATS + _COMPLEX, 1, '?'),
     'out0 = isnan(in0)', doc='Tests elementwise for NaN.')
 isinf = create_ufunc(
     'cupy_isinf',
-    tuple(('%s->?' % c, 'out0 = false') for c in '?' + _INTS) + _sig(_FLOATS, 1, '?'),
+    tuple(('%s->?' % c, 'out0 = false') for c in '?' + _INTS) + _sig(_FLOATS + _COMPLEX, 1, '?'),
     'out0 = isinf(in0)', doc='Tests elementwise for +/- infinity.')
 isfinite = create_ufunc(
     'cupy_isfinite',
-    tuple(('%s->?' % c, 'out0 = true') for c in '?' + _INTS) + _sig(_FLOATS, 1, '?'),
+    tuple(('%s->?' % c, 'out0 = true') for c in '?' + _INTS) + _sig(_FLOATS + _COMPLEX, 1, '?'),
     'out0 = isfinite(in0)', doc='Tests elementwise for finiteness.')
 signbit = create_ufunc(
     'cupy_signbit', _sig(_FLOATS, 1, '?'),
@@ -366,12 +398,12 @@ signbit = create_ufunc(
 
 _where_ufunc = create_ufunc(
     'cupy_where',
-    tuple('?%s%s->%s' % (c, c, c) for c in '?' + _INTS + _FLOATS),
+    tuple('?%s%s->%s' % (c, c, c) for c in '?' + _INTS + _FLOATS + _COMPLEX),
     'out0 = in0 ? in1 : in2')
 
 _clip = create_ufunc(
     'cupy_clip',
-    tuple('%s%s%s->%s' % (c, c, c, c) for c in '?' + _INTS + _FLOATS),
+    tuple('%s%s%s->%s' % (c, c, c, c) for c in '?' + _INTS + _FLOATS + _COMPLEX),
     'out0 = in0 < in1 ? in1 : (in0 > in2 ? in2 : in0)')
 
 
@@ -653,3 +685,119 @@ def divmod(x1, x2, out1=None, out2=None):
     .. seealso:: :data:`numpy.divmod`
     """
     return floor_divide(x1, x2, out1), remainder(x1, x2, out2)
+
+
+# ---------------------------------------------------------------------------------
+# Complex-number helpers (reference: cupy/_core/_routines_math.pyx:908-949,
+# cupy/_math/misc.py real/imag/angle).
+# ---------------------------------------------------------------------------------
+
+conjugate = create_ufunc(
+    'cupy_conjugate',
+    _sig(_INTS + _FLOATS, 1) + (
+        ('F->F', 'out0 = conj(in0)'), ('D->D', 'out0 = conj(in0)')),
+    'out0 = in0',
+    doc='Complex conjugate, elementwise.\n\n.. seealso:: :data:`numpy.conjugate`')
+conj = conjugate
+
+_real_ufunc = create_ufunc(
+    'cupy_real',
+    _sig('?' + _INTS + _FLOATS, 1) + (
+        ('F->f', 'out0 = in0.real()'), ('D->d', 'out0 = in0.real()')),
+    'out0 = in0')
+_imag_ufunc = create_ufunc(
+    'cupy_imag',
+    _sig('?' + _INTS + _FLOATS, 1) + (
+        ('F->f', 'out0 = in0.imag()'), ('D->d', 'out0 = in0.imag()')),
+    'out0 = 0')
+
+_angle_ufunc = create_ufunc(
+    'cupy_angle',
+    tuple(('%s->d' % c, 'out0 = in0 >= 0 ? 0.0 : M_PI') for c in '?' + _INTS) + (
+        ('e->e', 'out0 = atan2f(0.0f, in0)'),
+        ('f->f', 'out0 = atan2f(0.0f, in0)'),
+        ('d->d', 'out0 = atan2(0.0, in0)'),
+        ('F->f', 'out0 = arg(in0)'),
+        ('D->d', 'out0 = arg(in0)')))
+_angle_deg_ufunc = create_ufunc(
+    'cupy_angle_deg',
+    tuple(('%s->d' % c, 'out0 = in0 >= 0 ? 0.0 : 180.0') for c in '?' + _INTS) + (
+        ('e->e', 'out0 = atan2f(0.0f, in0) * (float)(180.0 / M_PI)'),
+        ('f->f', 'out0 = atan2f(0.0f, in0) * (float)(180.0 / M_PI)'),
+        ('d->d', 'out0 = atan2(0.0, in0) * (180.0 / M_PI)'),
+        ('F->f', 'out0 = arg(in0) * (float)(180.0 / M_PI)'),
+        ('D->d', 'out0 = arg(in0) * (180.0 / M_PI)')))
+
+
+def angle(z, deg=False):
+    """Angle of the complex argument, in radians or degrees.
+
+    .. seealso:: :func:`numpy.angle`
+    """
+    if deg:
+        return _angle_deg_ufunc(z)
+    return _angle_ufunc(z)
+
+
+def real(val):
+    """Real part of the elements (a view for complex arrays).
+
+    .. seealso:: :func:`numpy.real`
+    """
+    from cupy_amd._core.core import array
+    return array(val, copy=False).real
+
+
+def imag(val):
+    """Imaginary part of the elements (a view for complex arrays).
+
+    .. seealso:: :func:`numpy.imag`
+    """
+    from cupy_amd._core.core import array
+    return array(val, copy=False).imag
+
+
+def iscomplexobj(x):
+    """True if the argument's type is complex.
+
+    .. seealso:: :func:`numpy.iscomplexobj`
+    """
+    import numpy
+    dtype = getattr(x, 'dtype', None)
+    if dtype is None:
+        return numpy.iscomplexobj(x)
+    return numpy.dtype(dtype).kind == 'c'
+
+
+def isrealobj(x):
+    """True if the argument's type is not complex.
+
+    .. seealso:: :func:`numpy.isrealobj`
+    """
+    return not iscomplexobj(x)
+
+
+def iscomplex(x):
+    """Tests elementwise for a non-zero imaginary part.
+
+    .. seealso:: :func:`numpy.iscomplex`
+    """
+    from cupy_amd._core.core import array
+    x = array(x, copy=False)
+    if x.dtype.kind == 'c':
+        return x.imag != 0
+    from cupy_amd import zeros
+    return zeros(x.shape, bool)
+
+
+def isreal(x):
+    """Tests elementwise for a zero imaginary part.
+
+    .. seealso:: :func:`numpy.isreal`
+    """
+    from cupy_amd._core.core import array
+    x = array(x, copy=False)
+    if x.dtype.kind == 'c':
+        return x.imag == 0
+    from cupy_amd import ones
+    return ones(x.shape, bool)

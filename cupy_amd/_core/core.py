@@ -716,6 +716,53 @@ class ndarray:
         from cupy_amd._core import _scan
         return _scan.cumprod(self, axis, dtype, out)
 
+    # -- complex numbers (reference: cupy/_core/core.pyx real/imag/conj) ----------------
+    def _complex_part(self, second):
+        part = numpy.dtype('float32' if self.dtype.itemsize == 8 else 'float64')
+        v = self._view(self._shape, self._strides, part)
+        if second:
+            v.data = self.data + part.itemsize
+        return v
+
+    @property
+    def real(self):
+        """Real part: a view of the same memory for complex arrays, the array
+        itself otherwise."""
+        if self.dtype.kind == 'c':
+            return self._complex_part(False)
+        return self
+
+    @real.setter
+    def real(self, value):
+        from cupy_amd._core._ufuncs import elementwise_copy
+        elementwise_copy(value, self.real, casting='unsafe')
+
+    @property
+    def imag(self):
+        """Imaginary part: a view of the same memory for complex arrays, a new
+        array of zeros otherwise."""
+        if self.dtype.kind == 'c':
+            return self._complex_part(True)
+        out = ndarray._new_contiguous(self._shape, self.dtype)
+        out.fill(0)
+        return out
+
+    @imag.setter
+    def imag(self, value):
+        if self.dtype.kind != 'c':
+            raise TypeError('cupy.ndarray does not have imaginary part to set')
+        from cupy_amd._core._ufuncs import elementwise_copy
+        elementwise_copy(value, self.imag, casting='unsafe')
+
+    def conj(self):
+        """Complex conjugate; the array itself when it is not complex."""
+        if self.dtype.kind != 'c':
+            return self
+        from cupy_amd._core._ufuncs import conjugate
+        return conjugate(self)
+
+    conjugate = conj
+
     def any(self, axis=None, out=None, keepdims=False):
         from cupy_amd._core import _routines_logic
         return _routines_logic._ndarray_any(self, axis, out, keepdims)

@@ -71,7 +71,9 @@ class Memory(BaseMemory):
 
     def __del__(self):
         ptr, self.ptr = getattr(self, 'ptr', 0), 0
-        if ptr and type(self) is Memory and not _dryrun.enabled():
+        if not ptr or _dryrun is None or _rt is None:     # interpreter shutdown
+            return
+        if type(self) is Memory and not _dryrun.enabled():
             try:
                 _rt.lib.rt_free(ptr)
             except Exception:

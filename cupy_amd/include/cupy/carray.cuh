@@ -87,6 +87,8 @@ _CUPY_DEV bool isfinite(float16 x) { return x.isfinite(); }
 _CUPY_DEV int signbit(float16 x) { return x.signbit(); }
 _CUPY_DEV float16 copysign(float16 x, float16 y) { return float16::copysign(x, y); }
 
+#include <cupy/complex.cuh>
+
 // ---------------------------------------------------------------------------
 // CArray: strided N-d view passed by value to a kernel.
 //   data pointer, element count, shape[ndim], strides[ndim] (strides in bytes)

@@ -1,0 +1,240 @@
+"""complex64 / complex128 on the GPU against NumPy on the same seeded inputs.
+
+Bars: arithmetic whose NumPy loop is a fixed sequence of IEEE operations (add,
+subtract, multiply, Smith's division, square, conjugate, comparisons, casts) is
+bit-exact; absolute value within 2 ulp; the elementary functions, computed here
+by their textbook formulas and there by the C library's, within
+32 eps * (1 + |result|) in the complex plane; sums within the reduction
+tolerance of the real types."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from helpers import assert_exact, assert_ulp
+
+pytestmark = pytest.mark.gpu
+
+CTYPES = ['complex64', 'complex128']
+
+
+def crandom(shape, dtype, seed, scale=1.0):
+    rng = np.random.default_rng(seed)
+    z = rng.standard_normal(shape) + 1j * rng.standard_normal(shape)
+    return (z * scale).astype(dtype)
+
+
+def assert_cclose(got, want, eps_factor=32):
+    got, want = np.asarray(got), np.asarray(want)
+    assert got.dtype == want.dtype and got.shape == want.shape, (got.dtype, want.dtype)
+    eps = np.finfo(want.real.dtype).eps
+    err = np.abs(got.astype(np.complex128) - want.astype(np.complex128))
+    bound = eps_factor * eps * (1 + np.abs(want.astype(np.complex128)))
+    bad = ~(err <= bound)
+    assert not bad.any(), (got[bad][:4], want[bad][:4])
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_arithmetic_is_bit_exact(dtype):
+    a = crandom((97, 53), dtype, 1)
+    b = crandom((97, 53), dtype, 2)
+    da, db = cp.asarray(a), cp.asarray(b)
+    assert_exact((da + db).get(), a + b)
+    assert_exact((da - db).get(), a - b)
+    assert_exact((da * db).get(), a * b)
+    assert_exact((da / db).get(), a / b)
+    assert_exact((-da).get(), -a)
+    assert_exact(cp.square(da).get(), np.square(a))
+    assert_exact(cp.conjugate(da).get(), np.conjugate(a))
+    assert_exact(da.conj().get(), a.conj())
+    assert_exact(cp.reciprocal(da).get(), np.reciprocal(a))
+    assert_ulp(abs(da).get(), abs(a), 2)
+    # broadcasting and non-contiguous operands
+    assert_exact((da[::2, 1::3] * db.T[1::3, ::2].T).get(), a[::2, 1::3] * b.T[1::3, ::2].T)
+    assert_exact((da + db[0]).get(), a + b[0])
+    assert_exact((da * db[:, :1]).get(), a * b[:, :1])
+    assert_exact(cp.ascontiguousarray(da.T).get(), np.ascontiguousarray(a.T))
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_scalars_and_mixed_types(dtype):
+    a = crandom((1000,), dtype, 3)
+    f = np.random.default_rng(4).standard_normal(1000).astype(np.float32)
+    h = f.astype(np.float16)
+    i = np.arange(1000, dtype=np.int32) - 500
+    da = cp.asarray(a)
+    for s in (2, 2.5, 1 - 2j, np.float32(3), np.complex64(1 + 1j), np.complex128(2 - 1j)):
+        assert_exact((da * s).get(), a * s)
+        assert_exact((s + da).get(), s + a)
+        assert_exact((da * s).get(), a * s)          # replayed launch
+    for other in (f, h, i):
+        assert_exact((da * cp.asarray(other)).get(), a * other)
+        assert_exact((cp.asarray(other) - da).get(), other - a)
+    assert_exact((cp.asarray(f) * 1j).get(), f * 1j)
+    assert_exact((cp.asarray(i) + 1j).get(), i + 1j)
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_division_special_cases(dtype):
+    t = np.dtype(dtype).type
+    num = np.array([1 + 1j, 1 + 1j, 0j, 1e30 + 1e30j, 1e-30 + 1e-30j, 3 - 4j, np.inf + 1j], dtype)
+    den = np.array([0j, 1e-30 + 1e30j, 0j, 1e30 + 1e-30j, 1e30 - 1e30j, 0 + 2j, 2 + 0j], dtype)
+    with np.errstate(all='ignore'):
+        want = num / den
+    assert_exact((cp.asarray(num) / cp.asarray(den)).get(), want)
+    assert t is not None
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+@pytest.mark.parametrize('name', [
+    'sqrt', 'exp', 'log', 'log2', 'log10', 'sin', 'cos', 'tan', 'sinh', 'cosh', 'tanh',
+    'arcsin', 'arccos', 'arctan', 'arcsinh', 'arccosh', 'arctanh'])
+def test_elementary_functions(name, dtype):
+    a = crandom((4000,), dtype, 5, scale=1.5)
+    with np.errstate(all='ignore'):
+        want = getattr(np, name)(a)
+    assert_cclose(getattr(cp, name)(cp.asarray(a)).get(), want)
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_power_sign_and_angle(dtype):
+    a = crandom((3000,), dtype, 6)
+    b = crandom((3000,), dtype, 7)
+    da, db = cp.asarray(a), cp.asarray(b)
+    assert_cclose(cp.power(da, db).get(), np.power(a, b), 64)
+    assert_cclose((da ** 2).get(), a ** 2)
+    assert_cclose((da ** 0.5).get(), a ** 0.5)
+    assert_cclose(cp.sign(da).get(), np.sign(a), 4)
+    z = np.array([0j, np.nan + 1j, np.inf + 1j, 1 - np.inf * 1j], dtype)
+    with np.errstate(all='ignore'):
+        assert_exact(cp.sign(cp.asarray(z)).get(), np.sign(z))
+    real_t = a.real.dtype
+    eps = np.finfo(real_t).eps
+    np.testing.assert_allclose(cp.angle(da).get(), np.angle(a), rtol=4 * eps, atol=4 * eps)
+    np.testing.assert_allclose(cp.angle(da, deg=True).get(), np.angle(a, deg=True),
+                               rtol=4 * eps, atol=400 * eps)
+    assert cp.angle(da).dtype == real_t
+    r = np.array([-2.0, 0.0, 3.0, np.nan], np.float32)
+    assert_exact(cp.angle(cp.asarray(r)).get(), np.angle(r))
+    k = np.array([-2, 0, 3], np.int32)
+    assert_exact(cp.angle(cp.asarray(k)).get(), np.angle(k))
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_comparisons_and_predicates(dtype):
+    rng = np.random.default_rng(8)
+    a = (rng.integers(-2, 3, 500) + 1j * rng.integers(-2, 3, 500)).astype(dtype)
+    b = (rng.integers(-2, 3, 500) + 1j * rng.integers(-2, 3, 500)).astype(dtype)
+    a[::7] = np.nan + 1j
+    b[::11] = complex(1, np.nan)
+    a[3] = np.inf
+    da, db = cp.asarray(a), cp.asarray(b)
+    for name in ('equal', 'not_equal', 'less', 'less_equal', 'greater', 'greater_equal',
+                 'logical_and', 'logical_or', 'logical_xor', 'maximum', 'minimum',
+                 'fmax', 'fmin'):
+        assert_exact(getattr(cp, name)(da, db).get(), getattr(np, name)(a, b))
+    for name in ('isnan', 'isinf', 'isfinite', 'logical_not'):
+        assert_exact(getattr(cp, name)(da).get(), getattr(np, name)(a))
+    c = rng.integers(0, 2, 500).astype(bool)
+    assert_exact(cp.where(cp.asarray(c), da, db).get(), np.where(c, a, b))
+
+
+def test_casts_follow_numpy():
+    a = crandom((300,), 'complex128', 9, scale=50)
+    a[::5] = 0
+    d = cp.asarray(a)
+    assert_exact(d.astype(np.complex64).get(), a.astype(np.complex64))
+    with pytest.warns(np.exceptions.ComplexWarning):
+        got = d.astype(np.float32).get()
+    with pytest.warns(np.exceptions.ComplexWarning):
+        assert_exact(got, a.astype(np.float32))
+    assert_exact(d.astype(bool).get(), a.astype(bool))
+    f = np.random.default_rng(10).standard_normal(300).astype(np.float16)
+    assert_exact(cp.asarray(f).astype(np.complex64).get(), f.astype(np.complex64))
+    i = np.arange(-150, 150, dtype=np.int64)
+    assert_exact(cp.asarray(i).astype(np.complex128).get(), i.astype(np.complex128))
+    b = np.array([True, False, True])
+    assert_exact(cp.asarray(b).astype(np.complex64).get(), b.astype(np.complex64))
+    with pytest.raises(TypeError):
+        cp.add(d, d, out=cp.zeros(300, np.float64))
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_real_and_imag_are_views(dtype):
+    a = crandom((40, 30), dtype, 11)
+    d = cp.asarray(a)
+    assert_exact(d.real.get(), a.real)
+    assert_exact(d.imag.get(), a.imag)
+    assert_exact(d.T[::2].imag.get(), a.T[::2].imag)
+    assert_exact((d.real * d.imag).get(), a.real * a.imag)
+    assert_exact(cp.real(d).get(), np.real(a))
+    assert_exact(cp.imag(d).get(), np.imag(a))
+    new = np.random.default_rng(12).standard_normal((40, 30)).astype(a.real.dtype)
+    d.real = cp.asarray(new)
+    d.imag = 2.5
+    a = a.copy()
+    a.real = new
+    a.imag = 2.5
+    assert_exact(d.get(), a)
+    assert_exact(cp.iscomplex(d).get(), np.iscomplex(a))
+    assert cp.iscomplexobj(d) and not cp.isrealobj(d)
+    r = cp.asarray(new)
+    assert_exact(r.imag.get(), new.imag)
+    assert not cp.iscomplexobj(r)
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_reductions_and_scans(dtype):
+    a = crandom((301, 203), dtype, 13)
+    d = cp.asarray(a)
+    rtol = 1e-5 if dtype == 'complex64' else 1e-12
+    for axis in (None, 0, 1):
+        bound = rtol * np.abs(a).sum(axis=axis)
+        assert (np.abs(d.sum(axis=axis).get() - a.sum(axis=axis)) <= bound).all()
+        assert (np.abs(d.mean(axis=axis).get() - a.mean(axis=axis)) <= bound).all()
+        assert d.sum(axis=axis).dtype == a.dtype
+        want = np.cumsum(a, axis=axis)
+        got = cp.cumsum(d, axis=axis).get()
+        assert got.shape == want.shape and got.dtype == want.dtype
+        assert (np.abs(got - want) <= rtol * np.cumsum(np.abs(a), axis=axis)).all()
+    small = crandom((6, 5), dtype, 14)
+    np.testing.assert_allclose(cp.asarray(small).prod(axis=1).get(), small.prod(axis=1),
+                               rtol=100 * rtol)
+    np.testing.assert_allclose(cp.cumprod(cp.asarray(small), axis=0).get(),
+                               np.cumprod(small, axis=0), rtol=100 * rtol)
+    z = a.copy()
+    z[::3, ::2] = complex(np.nan, 1)
+    z[1::3, 1::2] = 0
+    dz = cp.asarray(z)
+    np.testing.assert_allclose(cp.nansum(dz, axis=0).get(), np.nansum(z, axis=0),
+                               rtol=1000 * rtol, atol=1000 * rtol)
+    assert_exact(cp.count_nonzero(dz, axis=1).get(), np.count_nonzero(z, axis=1))
+    # big enough for the multi-block paths
+    big = crandom((3, 200000), dtype, 15)
+    db = cp.asarray(big)
+    for axis in (None, 0, 1):
+        bound = rtol * np.abs(big).sum(axis=axis)
+        assert (np.abs(db.sum(axis=axis).get() - big.sum(axis=axis)) <= bound).all()
+    got = cp.cumsum(db, axis=1).get()
+    assert (np.abs(got - np.cumsum(big, axis=1)) <= rtol * np.cumsum(np.abs(big), axis=1)).all()
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_user_kernels_with_complex_parameters(dtype):
+    a = crandom((513,), dtype, 16)
+    d = cp.asarray(a)
+    k = cp.ElementwiseKernel('T x, T s, float32 t', 'T y', 'y = x * s + conj(x) * (T)t',
+                             'cplx_axpy')
+    s = 2 - 3j
+    want = a * a.dtype.type(s) + np.conj(a) * a.dtype.type(0.5)
+    assert_exact(k(d, s, 0.5).get(), want)
+    assert_exact(k(d, 1j, 0.25).get(), a * a.dtype.type(1j) + np.conj(a) * a.dtype.type(0.25))
+    r = cp.ReductionKernel('T x', 'T y', 'x * conj(x)', 'a + b', 'y = a', '0', 'cplx_norm2')
+    m = crandom((37, 41), dtype, 17)
+    got = r(cp.asarray(m), axis=1).get()
+    rtol = 1e-5 if dtype == 'complex64' else 1e-12
+    np.testing.assert_allclose(got, (m * m.conj()).sum(axis=1), rtol=rtol, atol=rtol)
+
+    @cp.fuse()
+    def f(x, y):
+        return x * y + cp.conj(x)
+    assert_exact(f(d, d).get(), a * a + np.conj(a))
