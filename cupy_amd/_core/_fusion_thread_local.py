@@ -17,6 +17,15 @@ def call_ufunc(fusion_op, *args, **kwargs):
     return thread_local.history.call_ufunc(fusion_op, *args, **kwargs)
 
 
+def records_keepdims():
+    """True while a function is recorded for a kernel sequence: reductions
+    may then keep the reduced axes (the single-kernel tracer cannot)."""
+    return getattr(getattr(thread_local, 'history', None), 'split', False)
+
+
 def call_reduction(fusion_op, *args, **kwargs):
+    history = thread_local.history
+    if getattr(history, 'split', False):
+        return history.call_reduction(fusion_op, *args, **kwargs)
     from cupy_amd._core import fusion
     return fusion._call_reduction(fusion_op, *args, **kwargs)

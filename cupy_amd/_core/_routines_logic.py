@@ -24,18 +24,18 @@ def _ndarray_any(self, axis, out, keepdims):
 def all(a, axis=None, out=None, keepdims=False):
     """Tests whether all elements along the given axes are true."""
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.all does not support `keepdims` in fusion yet.')
-        return _fusion_thread_local.call_reduction(_all, a, axis=axis, out=out)
+        return _fusion_thread_local.call_reduction(_all, a, axis=axis, out=out, keepdims=keepdims)
     return a.all(axis=axis, out=out, keepdims=keepdims)
 
 
 def any(a, axis=None, out=None, keepdims=False):
     """Tests whether any element along the given axes is true."""
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.any does not support `keepdims` in fusion yet.')
-        return _fusion_thread_local.call_reduction(_any, a, axis=axis, out=out)
+        return _fusion_thread_local.call_reduction(_any, a, axis=axis, out=out, keepdims=keepdims)
     return a.any(axis=axis, out=out, keepdims=keepdims)

@@ -77,12 +77,12 @@ def sum(a, axis=None, dtype=None, out=None, keepdims=False):
     .. seealso:: :func:`numpy.sum`
     """
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.sum does not support `keepdims` in fusion yet.')
         func = _sum_auto_dtype if dtype is None else _sum_keep_dtype
         return _fusion_thread_local.call_reduction(
-            func, a, axis=axis, dtype=dtype, out=out)
+            func, a, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
     return a.sum(axis, dtype, out, keepdims)
 
 
@@ -92,12 +92,12 @@ def prod(a, axis=None, dtype=None, out=None, keepdims=False):
     .. seealso:: :func:`numpy.prod`
     """
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.prod does not support `keepdims` in fusion yet.')
         func = _prod_auto_dtype if dtype is None else _prod_keep_dtype
         return _fusion_thread_local.call_reduction(
-            func, a, axis=axis, dtype=dtype, out=out)
+            func, a, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
     return a.prod(axis, dtype, out, keepdims)
 
 
@@ -108,11 +108,11 @@ def nansum(a, axis=None, dtype=None, out=None, keepdims=False):
     """
     func = _nansum_auto_dtype if dtype is None else _nansum_keep_dtype
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.nansum does not support `keepdims` in fusion yet.')
         return _fusion_thread_local.call_reduction(
-            func, a, axis=axis, dtype=dtype, out=out)
+            func, a, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
     return func(a, axis, dtype, out, keepdims)
 
 

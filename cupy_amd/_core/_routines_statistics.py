@@ -495,10 +495,10 @@ def amax(a, axis=None, out=None, keepdims=False):
     .. seealso:: :func:`numpy.amax`
     """
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.amax does not support `keepdims` in fusion yet.')
-        return _fusion_thread_local.call_reduction(_amax, a, axis=axis, out=out)
+        return _fusion_thread_local.call_reduction(_amax, a, axis=axis, out=out, keepdims=keepdims)
     return a.max(axis=axis, out=out, keepdims=keepdims)
 
 
@@ -508,10 +508,10 @@ def amin(a, axis=None, out=None, keepdims=False):
     .. seealso:: :func:`numpy.amin`
     """
     if _fusion_thread_local.is_fusing():
-        if keepdims:
+        if keepdims and not _fusion_thread_local.records_keepdims():
             raise NotImplementedError(
                 'cupy.amin does not support `keepdims` in fusion yet.')
-        return _fusion_thread_local.call_reduction(_amin, a, axis=axis, out=out)
+        return _fusion_thread_local.call_reduction(_amin, a, axis=axis, out=out, keepdims=keepdims)
     return a.min(axis=axis, out=out, keepdims=keepdims)
 
 

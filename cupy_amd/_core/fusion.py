@@ -616,8 +616,10 @@ class Fusion:
     """Callable returned by :func:`fuse`; behaves like an ElementwiseKernel or
     ReductionKernel specialised per argument types."""
 
-    def __init__(self, func, name=None):
+    def __init__(self, func, name=None, split=True):
         self.func = func
+        self._may_split = split
+        self._plans = {}
         name = name or getattr(func, '__name__', 'fused')
         # '<lambda>' and the like are not C identifiers
         name = re.sub(r'[^a-zA-Z0-9_]', '_', name)
@@ -684,16 +686,18 @@ class Fusion:
                 # (several reductions, arrays combined with a reduced value,
                 # ...).  The reference hands such functions to its second
                 # tracer (cupy/_core/fusion.pyx:860-871), whose multi-pass
-                # kernels need a grid-wide barrier.  Here the function runs as
-                # written: every step launches its own generated kernel on the
-                # current stream, temporaries come from the pool.  Errors of
-                # the function itself surface from that run.
+                # kernels need a grid-wide barrier.  Here the function is cut
+                # into a sequence of fused kernels (_fusion_split), or, if it
+                # cannot be recorded either, runs as written: every step
+                # launches its own generated kernel on the current stream,
+                # temporaries come from the pool.  Errors of the function
+                # itself surface from that run.
                 self._memo[key] = None
             finally:
                 _thread_local.history = None
                 _thread_local.is_old_fusing = False
         if self._memo[key] is None:
-            return self.func(*args)
+            return self._call_sequence(args, key, sig)
         kernel, kwargs = self._memo[key]
         call_args = []
         for a in args:
@@ -710,9 +714,34 @@ class Fusion:
             self._fast[sig] = (kernel, kwargs)
         return kernel(*call_args, **kwargs)
 
+    def _call_sequence(self, args, key, sig):
+        """The function as a sequence of fused kernels, planned once per
+        argument types and shapes; as written if it cannot be recorded."""
+        if not self._may_split:
+            return self.func(*args)
+        plan_key = (key, tuple(a.shape for a in args if isinstance(a, ndarray)))
+        plan = self._plans.get(plan_key)
+        if plan is None:
+            from cupy_amd._core import _fusion_split
+            try:
+                plan = _fusion_split.trace(self.func, args, self.name)
+            except Exception:
+                plan = False
+            if len(self._plans) >= 64:
+                self._plans.clear()
+            self._plans[plan_key] = plan
+        if plan is False:
+            return self.func(*args)
+        if sig is not None:
+            if len(self._fast) >= 256:
+                self._fast.clear()
+            self._fast[sig] = (plan.run, {})
+        return plan.run(*args)
+
     def clear_cache(self):
         self._memo = {}
         self._fast = {}
+        self._plans = {}
 
 
 def fuse(*args, **kwargs):

@@ -232,3 +232,55 @@ def test_functions_beyond_one_kernel_run_as_a_kernel_sequence():
         return x + undefined_name                     # noqa: F821
     with pytest.raises(NameError):
         broken(cp.asarray(a))
+
+
+def test_kernel_sequences_match_numpy():
+    rng = np.random.default_rng(43)
+    a = rng.standard_normal((301, 77)).astype(np.float32)
+    b = rng.standard_normal((301, 77)).astype(np.float32)
+
+    def softmax(xp):
+        def f(x):
+            e = xp.exp(x - xp.amax(x, axis=1, keepdims=True))
+            return e / xp.sum(e, axis=1, keepdims=True)
+        return f
+
+    def ratio(xp):
+        def f(x, y, s):
+            return xp.sum((x - y) ** 2, axis=1) / xp.sum(x * x * s, axis=1)
+        return f
+
+    def var0(xp):
+        def f(x):
+            m = x.sum(axis=0) / x.shape[0]
+            return ((x - m) ** 2).sum(axis=0) / x.shape[0]
+        return f
+
+    def centred(xp):
+        def f(x, y):
+            return (x - xp.sum(x) / x.size) * y, xp.amin(y, axis=0)
+        return f
+
+    for make, args in ((softmax, (a,)), (ratio, (a, b, 2.0)), (var0, (a,)), (centred, (a, b))):
+        want = make(np)(*args)
+        fused = cp.fuse(make(cp))
+        dev = [cp.asarray(v) if isinstance(v, np.ndarray) else v for v in args]
+        for _ in range(2):                                   # plan, then remembered plan
+            got = fused(*dev)
+            assert fused._plans and all(fused._plans.values())
+            if not isinstance(want, tuple):
+                got, ref = (got,), (want,)
+            else:
+                ref = want
+            for g, w in zip(got, ref):
+                assert g.dtype == w.dtype and g.shape == w.shape
+                np.testing.assert_allclose(g.get(), w, rtol=2e-5, atol=2e-5)
+
+    # float16 intermediates round like the eager evaluation
+    h = rng.standard_normal((64, 40)).astype(np.float16)
+
+    @cp.fuse()
+    def spread(x):
+        return (x - cp.amax(x, axis=1, keepdims=True)) * (x - cp.amin(x, axis=1, keepdims=True))
+    want = (h - h.max(axis=1, keepdims=True)) * (h - h.min(axis=1, keepdims=True))
+    assert_exact(spread(cp.asarray(h)).get(), want)
