@@ -29,8 +29,8 @@ struct alignas(2 * sizeof(T)) complex {
     re -= z.re; im -= z.im; return *this;
   }
   __device__ __forceinline__ complex& operator*=(const complex& z) {
-    const T r = re * z.re - im * z.im;
-    im = re * z.im + im * z.re;
+    const T r = fma(re, z.re, -(im * z.im));
+    im = fma(re, z.im, im * z.re);
     re = r;
     return *this;
   }
@@ -50,9 +50,13 @@ template <typename T>
 __device__ __forceinline__ complex<T> operator-(const complex<T>& a, const complex<T>& b) {
   return complex<T>(a.re - b.re, a.im - b.im);
 }
+// One product rounded, the other fused into the sum: what NumPy's vectorised
+// complex multiply computes on hosts with fused multiply-add (multiply, then
+// multiply-add/subtract), and one rounding closer to the exact result than
+// the four-product formula.
 template <typename T>
 __device__ __forceinline__ complex<T> operator*(const complex<T>& a, const complex<T>& b) {
-  return complex<T>(a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re);
+  return complex<T>(fma(a.re, b.re, -(a.im * b.im)), fma(a.re, b.im, a.im * b.re));
 }
 // Smith's algorithm, the way NumPy divides: scale by the larger component of
 // the divisor so that intermediate products neither overflow nor underflow.
@@ -136,15 +140,38 @@ template <typename T>
 __device__ __forceinline__ complex<T> polar(T rho, T theta) {
   return complex<T>(rho * cos(theta), rho * sin(theta));
 }
+// exp(x) * (c, s) where exp(x) alone may overflow although the products do
+// not: above the threshold the exponential is taken in two factors.
+template <typename T>
+__device__ __forceinline__ complex<T> _exp_times(T x, T c, T s) {
+  const T big = sizeof(T) == 4 ? T(88) : T(709);
+  if (x > big) {
+    const T e1 = exp(x - big / 2);
+    const T e2 = exp(big / 2);
+    return complex<T>(e1 * c * e2, e1 * s * e2);
+  }
+  const T e = exp(x);
+  return complex<T>(e * c, e * s);
+}
 template <typename T>
 __device__ __forceinline__ complex<T> exp(const complex<T>& z) {
-  const T e = exp(z.re);
-  if (z.im == 0) return complex<T>(e, z.im);          // keeps inf + 0j from turning into NaN
-  return complex<T>(e * cos(z.im), e * sin(z.im));
+  if (z.im == 0) return complex<T>(exp(z.re), z.im);    // keeps inf + 0j from turning into NaN
+  return _exp_times(z.re, cos(z.im), sin(z.im));
 }
 template <typename T>
 __device__ __forceinline__ complex<T> log(const complex<T>& z) {
-  return complex<T>(log(hypot(z.re, z.im)), atan2(z.im, z.re));
+  const T ax = z.re < 0 ? -z.re : z.re;
+  const T ay = z.im < 0 ? -z.im : z.im;
+  const T m = ax > ay ? ax : ay;
+  const T n = ax > ay ? ay : ax;
+  T re;
+  if (m > T(0.5) && m < T(2)) {
+    // |z| near 1: log|z| = log1p(|z|^2 - 1) / 2 without forming |z|
+    re = log1p((m - 1) * (m + 1) + n * n) / 2;
+  } else {
+    re = log(hypot(z.re, z.im));
+  }
+  return complex<T>(re, atan2(z.im, z.re));
 }
 template <typename T>
 __device__ __forceinline__ complex<T> log10(const complex<T>& z) {
@@ -164,7 +191,9 @@ __device__ __forceinline__ complex<T> sqrt(const complex<T>& z) {
     return complex<T>(r, z.im / (2 * r));
   }
   const T i = sqrt((m - z.re) / 2);
-  return complex<T>((z.im < 0 ? -z.im : z.im) / (2 * i), z.im < 0 ? -i : i);
+  // below the cut (negative real axis approached with im = -0) the root is -i|..|
+  const bool below = __builtin_signbit(z.im);
+  return complex<T>((below ? -z.im : z.im) / (2 * i), below ? -i : i);
 }
 template <typename T>
 __device__ __forceinline__ complex<T> pow(const complex<T>& a, const complex<T>& b) {
@@ -174,29 +203,55 @@ __device__ __forceinline__ complex<T> pow(const complex<T>& a, const complex<T>&
 }
 template <typename T>
 __device__ __forceinline__ complex<T> pow(const complex<T>& a, T b) { return pow(a, complex<T>(b)); }
+// (cosh x, sinh x) scaled so that neither overflows before it is multiplied by
+// a sine or cosine: for large |x| both are exp(|x|) / 2.
 template <typename T>
 __device__ __forceinline__ complex<T> sinh(const complex<T>& z) {
+  const T ax = z.re < 0 ? -z.re : z.re;
+  if (ax > (sizeof(T) == 4 ? T(80) : T(700))) {
+    const complex<T> h = _exp_times(ax, cos(z.im) / 2, sin(z.im) / 2);
+    return complex<T>(z.re < 0 ? -h.re : h.re, h.im);
+  }
   return complex<T>(sinh(z.re) * cos(z.im), cosh(z.re) * sin(z.im));
 }
 template <typename T>
 __device__ __forceinline__ complex<T> cosh(const complex<T>& z) {
+  const T ax = z.re < 0 ? -z.re : z.re;
+  if (ax > (sizeof(T) == 4 ? T(80) : T(700))) {
+    const complex<T> h = _exp_times(ax, cos(z.im) / 2, sin(z.im) / 2);
+    return complex<T>(h.re, z.re < 0 ? -h.im : h.im);
+  }
   return complex<T>(cosh(z.re) * cos(z.im), sinh(z.re) * sin(z.im));
 }
 template <typename T>
 __device__ __forceinline__ complex<T> tanh(const complex<T>& z) {
-  // tanh(x + iy) = (sinh 2x + i sin 2y) / (cosh 2x + cos 2y)
-  const T tx = 2 * z.re, ty = 2 * z.im;
-  if (tx > 40 || tx < -40) return complex<T>(tx > 0 ? 1 : -1, 0);     // cosh would overflow
-  const T d = cosh(tx) + cos(ty);
-  return complex<T>(sinh(tx) / d, sin(ty) / d);
+  // Kahan's form: with t = tan y, b = 1 + t^2, s = sinh x, r = sqrt(1 + s^2),
+  //   tanh(x + iy) = (b r s + i t) / (1 + b s^2),
+  // which has no cancellation near the poles (x = 0, y = pi/2 + k pi).
+  const T ax = z.re < 0 ? -z.re : z.re;
+  if (ax > (sizeof(T) == 4 ? T(11) : T(22))) {
+    // |tanh| is 1 to working precision; the imaginary part underflows to a
+    // zero with the sign of sin(2y)
+    const T e = exp(-2 * ax);
+    return complex<T>(z.re > 0 ? T(1) : T(-1), 4 * sin(z.im) * cos(z.im) * e);
+  }
+  const T t = tan(z.im);
+  const T b = 1 + t * t;
+  const T sh = sinh(z.re);
+  const T r = sqrt(1 + sh * sh);
+  const T d = 1 + b * sh * sh;
+  return complex<T>(b * r * sh / d, t / d);
 }
 template <typename T>
 __device__ __forceinline__ complex<T> sin(const complex<T>& z) {
-  return complex<T>(sin(z.re) * cosh(z.im), cos(z.re) * sinh(z.im));
+  // sin z = -i sinh(i z)
+  const complex<T> t = sinh(complex<T>(-z.im, z.re));
+  return complex<T>(t.im, -t.re);
 }
 template <typename T>
 __device__ __forceinline__ complex<T> cos(const complex<T>& z) {
-  return complex<T>(cos(z.re) * cosh(z.im), -sin(z.re) * sinh(z.im));
+  // cos z = cosh(i z)
+  return cosh(complex<T>(-z.im, z.re));
 }
 template <typename T>
 __device__ __forceinline__ complex<T> tan(const complex<T>& z) {
@@ -206,9 +261,28 @@ __device__ __forceinline__ complex<T> tan(const complex<T>& z) {
 }
 template <typename T>
 __device__ __forceinline__ complex<T> asinh(const complex<T>& z) {
-  // log(z + sqrt(z*z + 1))
-  const complex<T> s = sqrt(complex<T>(z.re * z.re - z.im * z.im + 1, 2 * z.re * z.im));
-  return log(complex<T>(z.re + s.re, z.im + s.im));
+  // asinh is odd: work in the half plane Re z >= 0, where w = z + sqrt(1 + z^2)
+  // adds parts of equal sign.  log w is taken as log1p(w - 1), with
+  // w - 1 = z + z^2 / (sqrt(1 + z^2) + 1) formed without cancellation, so small
+  // arguments keep their relative accuracy.
+  const bool neg = z.re < 0 || (z.re == 0 && __builtin_signbit(z.re));
+  const T x = neg ? -z.re : z.re;
+  const T y = neg ? -z.im : z.im;
+  const T ay = y < 0 ? -y : y;
+  complex<T> r;
+  if (x > (sizeof(T) == 4 ? T(1e18) : T(1e150)) || ay > (sizeof(T) == 4 ? T(1e18) : T(1e150))) {
+    // z^2 would overflow: asinh z = log(2 z)
+    const complex<T> l = log(complex<T>(x, y));
+    r = complex<T>(l.re + T(0.69314718055994530942), l.im);
+  } else {
+    const complex<T> u(x * x - y * y, 2 * x * y);
+    const complex<T> s = sqrt(complex<T>(1 + u.re, u.im));
+    const complex<T> q = u / complex<T>(s.re + 1, s.im);
+    const T dr = x + q.re;
+    const T di = y + q.im;
+    r = complex<T>(log1p(dr * (2 + dr) + di * di) / 2, atan2(di, 1 + dr));
+  }
+  return neg ? complex<T>(-r.re, -r.im) : r;
 }
 template <typename T>
 __device__ __forceinline__ complex<T> acosh(const complex<T>& z) {
@@ -218,10 +292,24 @@ __device__ __forceinline__ complex<T> acosh(const complex<T>& z) {
 }
 template <typename T>
 __device__ __forceinline__ complex<T> atanh(const complex<T>& z) {
-  // (log(1 + z) - log(1 - z)) / 2
-  const complex<T> a = log(complex<T>(1 + z.re, z.im));
-  const complex<T> b = log(complex<T>(1 - z.re, -z.im));
-  return complex<T>((a.re - b.re) / 2, (a.im - b.im) / 2);
+  // atanh is odd: with x >= 0,
+  //   Re = log1p(4x / ((1-x)^2 + y^2)) / 4, Im = atan2(2y, (1-x)(1+x) - y^2) / 2
+  // (the argument of log1p is then >= 0, away from its singularity at -1)
+  const bool neg = z.re < 0 || (z.re == 0 && __builtin_signbit(z.re));
+  const T x = neg ? -z.re : z.re;
+  const T y = neg ? -z.im : z.im;
+  const T ay = y < 0 ? -y : y;
+  complex<T> r;
+  if (x > (sizeof(T) == 4 ? T(1e18) : T(1e150)) || ay > (sizeof(T) == 4 ? T(1e18) : T(1e150))) {
+    // far from the origin atanh z -> 1/z +- i pi/2
+    const complex<T> inv = complex<T>(1) / complex<T>(x, y);
+    r = complex<T>(inv.re, y < 0 || (y == 0 && __builtin_signbit(y))
+                               ? T(-1.57079632679489661923) : T(1.57079632679489661923));
+  } else {
+    r = complex<T>(log1p(4 * x / ((1 - x) * (1 - x) + y * y)) / 4,
+                   atan2(2 * y, (1 - x) * (1 + x) - y * y) / 2);
+  }
+  return neg ? complex<T>(-r.re, -r.im) : r;
 }
 template <typename T>
 __device__ __forceinline__ complex<T> asin(const complex<T>& z) {

