@@ -228,12 +228,12 @@ def _float_unary(name, f32, f64, doc, cplx=None):
 sqrt = _float_unary('sqrt', 'sqrtf', 'sqrt', 'Elementwise square root.', 'sqrt')
 cbrt = _float_unary('cbrt', 'cbrtf', 'cbrt', 'Elementwise cube root.')
 exp = _float_unary('exp', 'expf', 'exp', 'Elementwise exponential.', 'exp')
-exp2 = _float_unary('exp2', 'exp2f', 'exp2', 'Elementwise 2**x.')
-expm1 = _float_unary('expm1', 'expm1f', 'expm1', 'Elementwise exp(x) - 1.')
+exp2 = _float_unary('exp2', 'exp2f', 'exp2', 'Elementwise 2**x.', 'exp2')
+expm1 = _float_unary('expm1', 'expm1f', 'expm1', 'Elementwise exp(x) - 1.', 'expm1')
 log = _float_unary('log', 'logf', 'log', 'Elementwise natural logarithm.', 'log')
 log2 = _float_unary('log2', 'log2f', 'log2', 'Elementwise base-2 logarithm.', 'log2')
 log10 = _float_unary('log10', 'log10f', 'log10', 'Elementwise base-10 logarithm.', 'log10')
-log1p = _float_unary('log1p', 'log1pf', 'log1p', 'Elementwise log(1 + x).')
+log1p = _float_unary('log1p', 'log1pf', 'log1p', 'Elementwise log(1 + x).', 'log1p')
 sin = _float_unary('sin', 'sinf', 'sin', 'Elementwise sine.', 'sin')
 cos = _float_unary('cos', 'cosf', 'cos', 'Elementwise cosine.', 'cos')
 tan = _float_unary('tan', 'tanf', 'tan', 'Elementwise tangent.', 'tan')
@@ -262,7 +262,7 @@ def _rounding(name, f32, f64, doc):
 floor = _rounding('floor', 'floorf', 'floor', 'Elementwise floor.')
 ceil = _rounding('ceil', 'ceilf', 'ceil', 'Elementwise ceiling.')
 trunc = _rounding('trunc', 'truncf', 'trunc', 'Elementwise truncation.')
-rint = _float_unary('rint', 'rintf', 'rint', 'Elementwise round half to even.')
+rint = _float_unary('rint', 'rintf', 'rint', 'Elementwise round half to even.', 'rint')
 
 arctan2 = create_ufunc(
     'cupy_arctan2',
@@ -331,9 +331,14 @@ fmin = create_ufunc(
 
 
 def _comparison(name, op, doc):
+    # int64 against uint64 compares the values, not their common C type: a
+    # negative number is below every unsigned one
+    signed_first = 'out0 = in0 < 0 ? (-1 %s 0) : ((unsigned long long)in0 %s in1)' % (op, op)
+    unsigned_first = 'out0 = in1 < 0 ? (0 %s -1) : (in0 %s (unsigned long long)in1)' % (op, op)
     return create_ufunc(
         'cupy_' + name,
-        _sig('?' + _INTS + _FLOATS + _COMPLEX, 2, '?'),
+        _sig('?' + _INTS, 2, '?') + (('qQ->?', signed_first), ('Qq->?', unsigned_first))
+        + _sig(_FLOATS + _COMPLEX, 2, '?'),
         'out0 = in0 %s in1' % op,
         doc=doc)
 
@@ -427,7 +432,7 @@ fmod = create_ufunc(
     doc='Remainder of C division (sign of the dividend).\n\n.. seealso:: :data:`numpy.fmod`')
 
 float_power = create_ufunc(
-    'cupy_float_power', (('dd->d', 'out0 = pow(in0, in1)'),),
+    'cupy_float_power', (('dd->d', 'out0 = pow(in0, in1)'), ('DD->D', 'out0 = pow(in0, in1)')),
     doc='Power computed in float64 whatever the inputs.\n\n.. seealso:: :data:`numpy.float_power`')
 
 _gcd_preamble = '''
@@ -570,9 +575,9 @@ degrees = rad2deg
 
 bitwise_count = create_ufunc(
     'cupy_bitwise_count',
-    tuple(('%s->B' % c, 'out0 = __popcll((unsigned long long)(in0 < 0 ? -in0 : in0))')
-          for c in 'bhilq') +
-    tuple(('%s->B' % c, 'out0 = __popcll((unsigned long long)in0)') for c in '?BHILQ'),
+    tuple(('%s->B' % c,
+           'out0 = __popcll((unsigned long long)(in0 < 0 ? -in0 : in0))' if c.islower()
+           else 'out0 = __popcll((unsigned long long)in0)') for c in _INTS),
     doc='Number of set bits of the absolute value.\n\n.. seealso:: :data:`numpy.bitwise_count`')
 
 i0 = create_ufunc(
@@ -699,6 +704,12 @@ conjugate = create_ufunc(
     'out0 = in0',
     doc='Complex conjugate, elementwise.\n\n.. seealso:: :data:`numpy.conjugate`')
 conj = conjugate
+
+# names of the array API standard, as in NumPy 2
+acos, acosh, asin, asinh, atan, atanh, atan2 = (
+    arccos, arccosh, arcsin, arcsinh, arctan, arctanh, arctan2)
+bitwise_invert, bitwise_left_shift, bitwise_right_shift = invert, left_shift, right_shift
+pow = power
 
 _real_ufunc = create_ufunc(
     'cupy_real',

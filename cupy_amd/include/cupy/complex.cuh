@@ -173,6 +173,33 @@ __device__ __forceinline__ complex<T> log(const complex<T>& z) {
   }
   return complex<T>(re, atan2(z.im, z.re));
 }
+// log(1 + z) without forming 1 + z: |1 + z|^2 - 1 = x (2 + x) + y^2
+template <typename T>
+__device__ __forceinline__ complex<T> log1p(const complex<T>& z) {
+  const T ax = z.re < 0 ? -z.re : z.re;
+  const T ay = z.im < 0 ? -z.im : z.im;
+  if (ax > T(0.5) || ay > T(0.5)) return log(complex<T>(1 + z.re, z.im));
+  return complex<T>(log1p(z.re * (2 + z.re) + z.im * z.im) / 2, atan2(z.im, 1 + z.re));
+}
+// exp(z) - 1 = expm1(x) cos y - 2 sin^2(y / 2) + i exp(x) sin y
+template <typename T>
+__device__ __forceinline__ complex<T> expm1(const complex<T>& z) {
+  const T ax = z.re < 0 ? -z.re : z.re;
+  if (ax > T(1)) {
+    const complex<T> e = exp(z);
+    return complex<T>(e.re - 1, e.im);
+  }
+  const T sh = sin(z.im / 2);
+  return complex<T>(expm1(z.re) * cos(z.im) - 2 * sh * sh, exp(z.re) * sin(z.im));
+}
+template <typename T>
+__device__ __forceinline__ complex<T> exp2(const complex<T>& z) {
+  return exp(complex<T>(z.re * T(0.69314718055994530942), z.im * T(0.69314718055994530942)));
+}
+template <typename T>
+__device__ __forceinline__ complex<T> rint(const complex<T>& z) {
+  return complex<T>(rint(z.re), rint(z.im));
+}
 template <typename T>
 __device__ __forceinline__ complex<T> log10(const complex<T>& z) {
   return log(z) * T(0.43429448190325182765);

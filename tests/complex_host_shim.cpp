@@ -15,6 +15,7 @@ using namespace std;
 UN(sqrt, sqrt) UN(exp, exp) UN(log, log) UN(log2, log2) UN(log10, log10) UN(sin, sin) UN(cos, cos) UN(tan, tan)
 UN(sinh, sinh) UN(cosh, cosh) UN(tanh, tanh) UN(arcsin, asin) UN(arccos, acos) UN(arctan, atan)
 UN(arcsinh, asinh) UN(arccosh, acosh) UN(arctanh, atanh)
+UN(log1p, log1p) UN(expm1, expm1) UN(exp2, exp2)
 #define BIN(name, expr) \
   extern "C" void c64_##name(const float* a_, const float* b_, float* out, int n) { \
     for (int i = 0; i < n; ++i) { complex<float> a(a_[2*i], a_[2*i+1]), b(b_[2*i], b_[2*i+1]); complex<float> r = expr; out[2*i] = r.re; out[2*i+1] = r.im; } } \

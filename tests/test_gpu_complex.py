@@ -96,7 +96,8 @@ def test_division_special_cases(dtype):
 @pytest.mark.parametrize('dtype', CTYPES)
 @pytest.mark.parametrize('name', [
     'sqrt', 'exp', 'log', 'log2', 'log10', 'sin', 'cos', 'tan', 'sinh', 'cosh', 'tanh',
-    'arcsin', 'arccos', 'arctan', 'arcsinh', 'arccosh', 'arctanh'])
+    'arcsin', 'arccos', 'arctan', 'arcsinh', 'arccosh', 'arctanh', 'log1p', 'expm1', 'exp2',
+    'rint'])
 def test_elementary_functions(name, dtype):
     a = crandom((4000,), dtype, 5, scale=1.5)
     with np.errstate(all='ignore'):
@@ -112,6 +113,9 @@ def test_power_sign_and_angle(dtype):
     assert_cclose(cp.power(da, db).get(), np.power(a, b), 64)
     assert_cclose((da ** 2).get(), a ** 2)
     assert_cclose((da ** 0.5).get(), a ** 0.5)
+    got = cp.float_power(da, db)
+    assert got.dtype == np.complex128
+    assert_cclose(got.get(), np.float_power(a, b), 64)
     assert_cclose(cp.sign(da).get(), np.sign(a), 4)
     z = np.array([0j, np.nan + 1j, np.inf + 1j, 1 - np.inf * 1j], dtype)
     with np.errstate(all='ignore'):

@@ -137,3 +137,15 @@ def test_accumulate_follows_cumsum_and_cumprod():
                  np.multiply.accumulate(small, axis=1))
     with pytest.raises(NotImplementedError):
         cp.maximum.accumulate(d)
+
+
+def test_int64_against_uint64_compares_values():
+    a = np.array([-1, 0, 1, -2**63, 2**63 - 1, 5, 7], np.int64)
+    b = np.array([2**64 - 1, 0, 1, 2**63, 2**63 - 1, 2**63 + 5, 6], np.uint64)
+    da, db = cp.asarray(a), cp.asarray(b)
+    for name in ('equal', 'not_equal', 'less', 'less_equal', 'greater', 'greater_equal'):
+        assert_exact(getattr(cp, name)(da, db).get(), getattr(np, name)(a, b))
+        assert_exact(getattr(cp, name)(db, da).get(), getattr(np, name)(b, a))
+    # the array API names are the same objects
+    assert cp.acos is cp.arccos and cp.atan2 is cp.arctan2 and cp.pow is cp.power
+    assert cp.bitwise_invert is cp.invert and cp.bitwise_left_shift is cp.left_shift
