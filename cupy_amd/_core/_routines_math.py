@@ -121,9 +121,14 @@ def nanprod(a, axis=None, dtype=None, out=None, keepdims=False):
 
     .. seealso:: :func:`numpy.nanprod`
     """
-    if dtype is None:
-        return _nanprod_auto_dtype(a, axis, dtype, out, keepdims)
-    return _nanprod_keep_dtype(a, axis, dtype, out, keepdims)
+    func = _nanprod_auto_dtype if dtype is None else _nanprod_keep_dtype
+    if _fusion_thread_local.is_fusing():
+        if keepdims and not _fusion_thread_local.records_keepdims():
+            raise NotImplementedError(
+                'cupy.nanprod does not support `keepdims` in fusion yet.')
+        return _fusion_thread_local.call_reduction(
+            func, a, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+    return func(a, axis, dtype, out, keepdims)
 
 
 def count_nonzero(a, axis=None):

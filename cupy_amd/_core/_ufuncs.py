@@ -745,6 +745,8 @@ def angle(z, deg=False):
 
     .. seealso:: :func:`numpy.angle`
     """
+    if _fusion_thread_local.is_fusing():
+        return _fusion_thread_local.call_ufunc(_angle_deg_ufunc if deg else _angle_ufunc, z)
     if deg:
         return _angle_deg_ufunc(z)
     return _angle_ufunc(z)
@@ -755,6 +757,8 @@ def real(val):
 
     .. seealso:: :func:`numpy.real`
     """
+    if _fusion_thread_local.is_fusing():
+        return _fusion_thread_local.call_ufunc(_real_ufunc, val)
     from cupy_amd._core.core import array
     return array(val, copy=False).real
 
@@ -764,6 +768,8 @@ def imag(val):
 
     .. seealso:: :func:`numpy.imag`
     """
+    if _fusion_thread_local.is_fusing():
+        return _fusion_thread_local.call_ufunc(_imag_ufunc, val)
     from cupy_amd._core.core import array
     return array(val, copy=False).imag
 
@@ -812,3 +818,77 @@ def isreal(x):
         return x.imag == 0
     from cupy_amd import ones
     return ones(x.shape, bool)
+
+
+# ---------------------------------------------------------------------------------
+# Rounding to decimals (reference: cupy/_math/rounding.py:11-40 and the
+# `_round_ufunc` of cupy/_core/_routines_math.pyx); the order of operations is
+# NumPy's: scale by the power of ten in the array's own type, round half to
+# even, scale back.  Integers go through double, as in NumPy.
+# ---------------------------------------------------------------------------------
+
+_round_preamble = '''
+template <typename T> __device__ __forceinline__ T _cupy_round_real(T v, long long d) {
+  if (d == 0) return T(rint(v));
+  if (d > 0) { const T x = T(pow(10.0, (double)d)); return T(rint(v * x)) / x; }
+  const T x = T(pow(10.0, (double)(-d)));
+  return T(rint(v / x)) * x;
+}
+__device__ __forceinline__ float16 _cupy_round_half(float16 v, long long d) {
+  if (d == 0) return float16(rintf(float(v)));
+  const float16 x = float16(pow(10.0, (double)(d > 0 ? d : -d)));
+  if (d > 0) return float16(rintf(float(float16(float(v) * float(x))))) / x;
+  return float16(rintf(float(float16(float(v) / float(x))))) * x;
+}
+template <typename T> __device__ __forceinline__ T _cupy_round_int(T v, long long d) {
+  if (d >= 0) return v;
+  const double x = pow(10.0, (double)(-d));
+  return (T)(rint((double)v / x) * x);
+}
+template <typename T> __device__ __forceinline__ complex<T> _cupy_round_complex(
+    const complex<T>& v, long long d) {
+  return complex<T>(_cupy_round_real(v.re, d), _cupy_round_real(v.im, d));
+}
+'''
+
+_round_ufunc = create_ufunc(
+    'cupy_round',
+    (('?q->e', 'out0 = _cupy_round_half(float16(in0 ? 1.0f : 0.0f), in1)'),)
+    + tuple(('%sq->%s' % (c, c), 'out0 = _cupy_round_int(in0, in1)') for c in _INTS)
+    + (('eq->e', 'out0 = _cupy_round_half(in0, in1)'),
+       ('fq->f', 'out0 = _cupy_round_real(in0, in1)'),
+       ('dq->d', 'out0 = _cupy_round_real(in0, in1)'),
+       ('Fq->F', 'out0 = _cupy_round_complex(in0, in1)'),
+       ('Dq->D', 'out0 = _cupy_round_complex(in0, in1)')),
+    preamble=_round_preamble)
+
+
+def around(a, decimals=0, out=None):
+    """Rounds to the given number of decimals (half to even).
+
+    .. seealso:: :func:`numpy.around`
+    """
+    import operator
+    decimals = operator.index(decimals)
+    if _fusion_thread_local.is_fusing():
+        return _fusion_thread_local.call_ufunc(_round_ufunc, a, decimals, out=out)
+    from cupy_amd._core.core import array
+    import numpy
+    return _round_ufunc(array(a, copy=False), numpy.int64(decimals), out=out)
+
+
+round = around
+
+
+def round_(a, decimals=0, out=None):
+    import warnings
+    warnings.warn('Please use `round` instead.', DeprecationWarning)
+    return around(a, decimals, out=out)
+
+
+fix = create_ufunc(
+    'cupy_fix',
+    tuple(('%s->%s' % (c, c), 'out0 = in0') for c in '?' + _INTS) + (
+        ('e->e', 'out0 = truncf(in0)'), ('f->f', 'out0 = truncf(in0)'),
+        ('d->d', 'out0 = trunc(in0)')),
+    doc='Rounds towards zero.\n\n.. seealso:: :func:`numpy.fix`')

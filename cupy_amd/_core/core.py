@@ -763,6 +763,10 @@ class ndarray:
 
     conjugate = conj
 
+    def round(self, decimals=0, out=None):
+        from cupy_amd._core._ufuncs import around
+        return around(self, decimals, out)
+
     def any(self, axis=None, out=None, keepdims=False):
         from cupy_amd._core import _routines_logic
         return _routines_logic._ndarray_any(self, axis, out, keepdims)

@@ -149,3 +149,32 @@ def test_int64_against_uint64_compares_values():
     # the array API names are the same objects
     assert cp.acos is cp.arccos and cp.atan2 is cp.arctan2 and cp.pow is cp.power
     assert cp.bitwise_invert is cp.invert and cp.bitwise_left_shift is cp.left_shift
+
+
+def test_around_follows_numpy():
+    rng = np.random.default_rng(77)
+    for dtype in ('float16', 'float32', 'float64'):
+        x = (rng.standard_normal(2000) * 100).astype(dtype)
+        x[:8] = [0.5, 1.5, 2.5, -0.5, -1.5, 0.125, 0.375, 2.675]
+        d = cp.asarray(x)
+        for decimals in (0, 1, 2, -1):
+            assert_exact(cp.around(d, decimals).get(), np.around(x, decimals))
+        assert_exact(d.round(1).get(), x.round(1))
+        assert_exact(cp.fix(d).get(), np.fix(x))
+    i = rng.integers(-1000, 1000, 500).astype(np.int32)
+    i[:6] = [15, 25, 35, -15, -25, 5]
+    di = cp.asarray(i)
+    for decimals in (0, 2, -1, -2):
+        assert_exact(cp.around(di, decimals).get(), np.around(i, decimals))
+    z = (rng.standard_normal(300) + 1j * rng.standard_normal(300)).astype(np.complex64) * 10
+    assert_exact(cp.around(cp.asarray(z), 1).get(), np.around(z, 1))
+    out = cp.zeros(2000, np.float64)
+    r = cp.around(cp.asarray(x), 2, out=out)
+    assert r is out
+    assert_exact(out.get(), np.around(x, 2))
+
+    @cp.fuse()
+    def f(a):
+        return cp.around(a * 3, 1) + cp.real(a)
+    x32 = x.astype(np.float32)
+    assert_exact(f(cp.asarray(x32)).get(), np.around(x32 * 3, 1) + np.real(x32))
