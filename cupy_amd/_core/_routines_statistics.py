@@ -311,6 +311,8 @@ def _ndarray_ptp(self, axis, out, keepdims):
 
 _norm_preamble = '''
 template <typename T> __device__ T my_norm(T x) { return x * x; }
+__device__ float my_norm(const complex<float>& x) { return norm(x); }
+__device__ double my_norm(const complex<double>& x) { return norm(x); }
 '''
 
 _var_cores = {}
@@ -348,6 +350,9 @@ def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
             dtype_mean = dtype_out = numpy.dtype('float64')
         else:
             dtype_mean = dtype_out = a.dtype
+            if a.dtype.kind == 'c':
+                # |x - mean|**2 is real
+                dtype_out = numpy.dtype(a.dtype.char.lower())
     else:
         dtype_mean = a.dtype
         dtype_out = numpy.dtype(dtype)

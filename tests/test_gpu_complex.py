@@ -252,3 +252,18 @@ def test_user_kernels_with_complex_parameters(dtype):
     def f(x, y):
         return x * y + cp.conj(x)
     assert_cclose(f(d, d).get(), a * a + np.conj(a), 8)
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+def test_variance_of_complex_is_real(dtype):
+    a = crandom((61, 47), dtype, 21)
+    d = cp.asarray(a)
+    rtol = 1e-5 if dtype == 'complex64' else 1e-12
+    for axis in (None, 0, 1):
+        for ddof in (0, 1):
+            got = d.var(axis=axis, ddof=ddof)
+            want = a.var(axis=axis, ddof=ddof)
+            assert got.dtype == want.dtype and got.shape == want.shape
+            np.testing.assert_allclose(got.get(), want, rtol=20 * rtol)
+            np.testing.assert_allclose(d.std(axis=axis, ddof=ddof).get(),
+                                       a.std(axis=axis, ddof=ddof), rtol=20 * rtol)
