@@ -684,12 +684,17 @@ def where(condition, x=None, y=None):
     return _where_ufunc(condition, x, y)
 
 
-def divmod(x1, x2, out1=None, out2=None):
-    """Quotient and remainder of floor division, as two arrays.
-
-    .. seealso:: :data:`numpy.divmod`
-    """
-    return floor_divide(x1, x2, out1), remainder(x1, x2, out2)
+divmod = create_ufunc(
+    'cupy_divmod',
+    tuple('%s%s->%s%s' % (c, c, c, c) for c in _INTS) + (
+        ('ee->ee', 'out0 = _cupy_fdiv<float>(in0, in1); out1 = _cupy_fmod_py<float>(in0, in1)'),
+        ('ff->ff', 'out0 = _cupy_fdiv<float>(in0, in1); out1 = _cupy_fmod_py<float>(in0, in1)'),
+        ('dd->dd', 'out0 = _cupy_fdiv<double>(in0, in1); out1 = _cupy_fmod_py<double>(in0, in1)')),
+    'out0 = _floor_divide(in0, in1); '
+    'out1 = in1 == 0 ? (out1_type)0 : (out1_type)(in0 - out0 * in1)',
+    preamble=_float_floor_divide,
+    doc='Quotient and remainder of floor division, as two arrays.\n\n'
+        '.. seealso:: :data:`numpy.divmod`')
 
 
 # ---------------------------------------------------------------------------------

@@ -18,7 +18,7 @@ _SAME_TYPES = (
     'abs absolute acos acosh add arccos arccosh arcsin arcsinh arctan arctan2 arctanh asin '
     'asinh atan atan2 atanh bitwise_and bitwise_count bitwise_invert bitwise_left_shift '
     'bitwise_not bitwise_or bitwise_right_shift bitwise_xor cbrt ceil conj conjugate copysign '
-    'cos cosh deg2rad degrees equal exp exp2 expm1 fabs float_power floor floor_divide fmax '
+    'cos cosh deg2rad degrees divmod equal exp exp2 expm1 fabs float_power floor floor_divide fmax '
     'fmin fmod frexp greater greater_equal heaviside hypot invert isfinite isinf isnan ldexp '
     'left_shift less less_equal log log10 log1p log2 logaddexp logaddexp2 logical_and '
     'logical_not logical_or logical_xor maximum minimum mod modf multiply nextafter not_equal '
