@@ -99,3 +99,68 @@ def test_single_kernel_functions_do_not_take_this_route():
     x, y = arrays((10, 20), (10, 20))
     _, names = kernels_of(f, x, y)
     assert names == ['f'] and not f._plans
+
+
+CASES = {
+    # name: (function of (xp, captured), number of arrays, extra args, kernels, result shapes)
+    'tuple_axis': (lambda xp, c: lambda a: a - xp.sum(a, axis=(0, 2), keepdims=True) / 24,
+                   1, (), 2, [(6, 5, 4)]),
+    'negative_axis': (lambda xp, c: lambda a: xp.sum(a, axis=-1) * xp.amax(a, axis=-1),
+                      1, (), 3, [(6, 5)]),
+    'captured_array': (lambda xp, c: lambda a: (a + c) / xp.sum(a + c, axis=2, keepdims=True),
+                       1, (), 2, [(6, 5, 4)]),
+    'scalar_argument': (lambda xp, c: lambda a, s: a * s - xp.sum(a * s),
+                        1, (2.5,), 2, [(6, 5, 4)]),
+    'returns_an_argument': (lambda xp, c: lambda a: (a, a - xp.amin(a)),
+                            1, (), 2, [(6, 5, 4), (6, 5, 4)]),
+    'none_argument': (lambda xp, c: lambda a, b: a - xp.sum(a) if b is None else a + b,
+                      1, (None,), 2, [(6, 5, 4)]),
+    'zero_dimensional': (lambda xp, c: lambda a: xp.sum(a) / xp.amax(a),
+                         1, (), 3, [()]),
+    'astype': (lambda xp, c: lambda a: (a - xp.sum(a, axis=0)).astype(np.float64),
+               1, (), 2, [(6, 5, 4)]),
+    'methods': (lambda xp, c: lambda a: a.max(axis=1) - a.min(axis=1) + a.sum(axis=1),
+                1, (), 4, [(6, 4)]),
+    'logic': (lambda xp, c: lambda a: xp.where(xp.all(a > 0, axis=0), xp.sum(a, axis=0), 0),
+              1, (), 3, [(5, 4)]),
+    'two_arrays': (lambda xp, c: lambda a, b: (a - b) / xp.sum(a * b, axis=1, keepdims=True),
+                   2, (), 2, [(6, 5, 4)]),
+}
+
+
+@pytest.mark.parametrize('name', sorted(CASES))
+def test_recorded_shapes_and_kernel_counts(name):
+    make, n_arrays, extra, n_kernels, shapes = CASES[name]
+    captured = cp.asarray(np.ones(4, np.float32))
+    f = cp.fuse(make(cp, captured))
+    args = arrays(*[(6, 5, 4)] * n_arrays) + list(extra)
+    out, names = kernels_of(f, *args)
+    outs = out if isinstance(out, tuple) else (out,)
+    assert [o.shape for o in outs] == shapes
+    assert len(names) == n_kernels and all('_part' in n for n in names)
+    host = [np.ones((6, 5, 4), np.float32)] * n_arrays + list(extra)
+    want = make(np, np.ones(4, np.float32))(*host)
+    wants = want if isinstance(want, tuple) else (want,)
+    assert [o.dtype for o in outs] == [np.asarray(w).dtype for w in wants]
+
+
+def test_errors_of_the_function_surface():
+    x, = arrays((6, 5, 4))
+    with pytest.raises(ValueError):
+        cp.fuse(lambda a: a - cp.sum(a, axis=(0, 0)))(x)
+    with pytest.raises(cp.AxisError):
+        cp.fuse(lambda a: a - cp.sum(a, axis=5))(x)
+
+
+def test_nested_fused_functions_are_inlined_in_the_pieces():
+    @cp.fuse()
+    def inner(a, b):
+        return a * b + 1
+
+    @cp.fuse()
+    def outer(a, b):
+        return inner(a, b) - cp.sum(inner(a, b), axis=0)
+
+    x, y = arrays((6, 5), (6, 5))
+    out, names = kernels_of(outer, x, y)
+    assert out.shape == (6, 5) and names[0] == 'outer_part0' and names[-1] == 'outer_part1'

@@ -248,6 +248,14 @@ def test_user_kernels_with_complex_parameters(dtype):
     rtol = 1e-5 if dtype == 'complex64' else 1e-12
     np.testing.assert_allclose(got, (m * m.conj()).sum(axis=1), rtol=rtol, atol=rtol)
 
+    scaled = cp.ReductionKernel('T x, T s, float32 t', 'T y', 'x * s + (T)t', 'a + b', 'y = a',
+                                '0', 'cplx_scaled_sum')
+    for axis in (0, 1, None):
+        for s, t in ((2 - 3j, 0.5), (1j, 0.25)):          # second pair: replayed launch
+            want = (m * m.dtype.type(s) + m.dtype.type(t)).sum(axis=axis)
+            np.testing.assert_allclose(scaled(cp.asarray(m), s, t, axis=axis).get(), want,
+                                       rtol=20 * rtol, atol=20 * rtol)
+
     @cp.fuse()
     def f(x, y):
         return x * y + cp.conj(x)

@@ -284,3 +284,21 @@ def test_kernel_sequences_match_numpy():
         return (x - cp.amax(x, axis=1, keepdims=True)) * (x - cp.amin(x, axis=1, keepdims=True))
     want = (h - h.max(axis=1, keepdims=True)) * (h - h.min(axis=1, keepdims=True))
     assert_exact(spread(cp.asarray(h)).get(), want)
+
+
+def test_kernel_sequence_cases_match_numpy():
+    from test_fusion_split import CASES
+    rng = np.random.default_rng(44)
+    captured = rng.uniform(0.5, 1.5, 4).astype(np.float32)
+    for name in sorted(CASES):
+        make, n_arrays, extra, _, shapes = CASES[name]
+        host = [rng.uniform(0.5, 1.5, (6, 5, 4)).astype(np.float32) for _ in range(n_arrays)]
+        want = make(np, captured)(*host, *extra)
+        fused = cp.fuse(make(cp, cp.asarray(captured)))
+        got = fused(*[cp.asarray(h) for h in host], *extra)
+        assert all(fused._plans.values()), name
+        gots = got if isinstance(got, tuple) else (got,)
+        wants = want if isinstance(want, tuple) else (want,)
+        for g, w in zip(gots, wants):
+            assert g.shape == np.shape(w) and g.dtype == np.asarray(w).dtype, name
+            np.testing.assert_allclose(g.get(), w, rtol=1e-5, atol=1e-5, err_msg=name)
