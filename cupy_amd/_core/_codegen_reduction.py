@@ -423,7 +423,9 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
     src.append('  const int _tx = threadIdx.x %% %d;' % tx)
     src.append('  const int _ty = threadIdx.x / %d;' % tx)
-    src.append('  const %s _c = ((%s)blockIdx.x * %d + _tx) * %d;' % (idx_t, idx_t, tx, vec))
+    # column blocks beyond the capacity of grid.x continue along grid.z
+    src.append('  const %s _c = ((((%s)blockIdx.z * gridDim.x + blockIdx.x) * %d) + _tx) * %d;' % (
+        idx_t, idx_t, tx, vec))
     src.append('  _type_reduce _acc[%d];' % vec)
     src.append('#pragma unroll')
     src.append('  for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (vec, _identity_decl(identity)))

@@ -325,6 +325,12 @@ def _grid_limit(dev_id, blocks_per_cu):
     return g
 
 
+def _max_blocks(block):
+    """Most workgroups of ``block`` work-items one grid dimension may hold: a
+    dispatch carries its size in work-items in 32 bits per dimension."""
+    return min(0x7fffffff, 0xffffffff // block)
+
+
 class _ElementwisePlanner:
     """Builds, memoises and launches the kernels of one elementwise operation
     (an ElementwiseKernel, or one loop of a ufunc)."""
@@ -682,7 +688,7 @@ class _ElementwisePlanner:
             item = a.dtype.itemsize
             block_args.const(cs[0] // item, cs[1] // item)
         ntiles = ((nr + tile_r - 1) // tile_r) * ((nc + tile_c - 1) // tile_c)
-        grid = max(1, min(ntiles, 0x7fffffff))
+        grid = max(1, min(ntiles, _max_blocks(threads)))
         _launch_plan.launch(rec, fn, (grid, 1, 1), (threads, 1, 1), packer, block_args,
                             stream_ptr)
         return True

@@ -29,7 +29,7 @@ from cupy_amd._core._dtype import get_dtype
 from cupy_amd._core._kernel import (
     _get_param_info, _decide_params_type, _preprocess_args, _broadcast,
     _get_out_args_from_optionals, _get_out_args_with_params,
-    _check_peer_access, _scalar_struct_code, _make_packer, _max_vector_width, _aligned)
+    _check_peer_access, _scalar_struct_code, _make_packer, _max_blocks, _max_vector_width, _aligned)
 from cupy_amd._core._scalar import CScalar, get_typename as _get_typename
 from cupy_amd._core.core import ndarray, _convert_from_cupy_like
 from cupy_amd.cuda import compiler
@@ -436,7 +436,9 @@ class _AbstractReductionKernel:
             fmt.append(ic)
             vals.const(so_out[k] // a.dtype.itemsize)
         grid = (n_out + tx - 1) // tx
-        _launch_plan.launch(rec, fn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
+        gz = (grid + _max_blocks(_cg.BLOCK) - 1) // _max_blocks(_cg.BLOCK)
+        grid = (grid + gz - 1) // gz
+        _launch_plan.launch(rec, fn, (grid, 1, gz), (_cg.BLOCK, 1, 1),
                             _make_packer(fmt), vals, stream_ptr)
 
     # -- rows ---------------------------------------------------------------------------------
@@ -524,7 +526,7 @@ class _AbstractReductionKernel:
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
         if group == _cg.BLOCK:
-            gx = min(n_out, 0x7fffffff)
+            gx = min(n_out, _max_blocks(_cg.BLOCK))
         else:
             rows_per_block = _cg.BLOCK // group * (batch if batched else 1)
             gx = min((n_out + rows_per_block - 1) // rows_per_block,
@@ -584,7 +586,11 @@ class _AbstractReductionKernel:
         tx = max(1, min(64, internal.clp2((n_out + vec - 1) // vec)))
         ty = _cg.BLOCK // tx
         gx = (n_out + tx * vec - 1) // (tx * vec)
-        want = (cus * _tuning.get('target_blocks_per_cu') + gx - 1) // gx
+        # the kernel does not loop over column blocks: beyond what grid.x may
+        # hold they continue along grid.z
+        gz = (gx + _max_blocks(_cg.BLOCK) - 1) // _max_blocks(_cg.BLOCK)
+        gx = (gx + gz - 1) // gz
+        want = (cus * _tuning.get('target_blocks_per_cu') + gx * gz - 1) // (gx * gz)
         most = max(1, n_red // (ty * 8))
         n_split = max(1, min(want, most, 65535))
         partial = n_split > 1
@@ -612,7 +618,7 @@ class _AbstractReductionKernel:
             partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
             vals.ptr(pref, partials.ptr)
             _launch_plan.launch(
-                rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
+                rec, fn, (gx, n_split, gz), (_cg.BLOCK, 1, 1),
                 _make_packer(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
@@ -620,7 +626,7 @@ class _AbstractReductionKernel:
                 stream_ptr, rec, pref, n_out * n_red)
         else:
             _launch_plan.launch(
-                rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
+                rec, fn, (gx, 1, gz), (_cg.BLOCK, 1, 1),
                 _make_packer(self._fast_format(rargs, ic)), vals, stream_ptr)
 
     # -- generic ------------------------------------------------------------------------------
@@ -650,7 +656,7 @@ class _AbstractReductionKernel:
         tx = max(min(contiguous, 64), _cg.BLOCK // max(1, n_red))
         tx = max(1, min(64, internal.flp2(tx), internal.clp2(n_out)))
         ty = _cg.BLOCK // tx
-        gx = min((n_out + tx - 1) // tx, 0x7fffffff)
+        gx = min((n_out + tx - 1) // tx, _max_blocks(_cg.BLOCK))
         want = (cus * _tuning.get('target_blocks_per_cu') + gx - 1) // gx
         most = max(1, n_red // (ty * 8))
         n_split = max(1, min(want, most, 65535))

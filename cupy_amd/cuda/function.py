@@ -162,6 +162,11 @@ class Function:
             stream_ptr = _stream.get_current_stream_ptr()
         gx, gy, gz = grid
         bx, by, bz = block
+        if gx * bx > 0xffffffff or gy * by > 0xffffffff or gz * bz > 0xffffffff:
+            # a dispatch holds its size in work-items in 32 bits per dimension
+            raise ValueError(
+                'kernel %s: grid %r x block %r exceeds 2**32 - 1 work-items in one dimension'
+                % (self.name, grid, block))
         n = len(arg_block)
         if n > self._arg_size or n < self._arg_min:
             raise ValueError(

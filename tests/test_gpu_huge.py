@@ -1,0 +1,172 @@
+"""Arrays beyond 2**31 elements or 2**31 bytes: the kernels then compute
+offsets (and, for arg-reductions, indices) in 64 bits.  The reference holds
+such cases as slow tests (tests/cupy_tests/sorting_tests/test_search.py:88-92,
+168-173 index beyond 2**32; math_tests/test_sumprod.py:68-74 broadcast sum of
+2**31 elements; :845-856 scan of 2**32 elements).
+
+Inputs are generated on the device from the element index and results are
+checked on the device against closed forms of the same index, so nothing large
+crosses to the host."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+
+pytestmark = pytest.mark.gpu
+
+_fill_mod100_i8 = cp.ElementwiseKernel('', 'int8 y', 'y = i % 100', 'fill_mod100_i8')
+_fill_mod50_i8 = cp.ElementwiseKernel('', 'int8 y', 'y = i % 50', 'fill_mod50_i8')
+_fill_mod1000_f32 = cp.ElementwiseKernel('', 'float32 y', 'y = i % 1000', 'fill_mod1000_f32')
+_fill_half_f64 = cp.ElementwiseKernel('', 'float64 y', 'y = i * 0.5', 'fill_half_f64')
+
+
+@pytest.fixture(autouse=True)
+def release_memory():
+    yield
+    cp.get_default_memory_pool().free_all_blocks()
+
+
+def sum_mod(n, m):
+    """sum(i % m for i in range(n))"""
+    full, rest = divmod(n, m)
+    return full * (m * (m - 1) // 2) + rest * (rest - 1) // 2
+
+
+def sum_mod100(n):
+    return sum_mod(n, 100)
+
+
+def test_elementwise_and_full_reductions_beyond_2_to_32_elements():
+    n = 2 ** 32 + 5
+    a = _fill_mod50_i8(size=n)                        # loop index in 64 bits
+    assert a.shape == (n,)
+    for pos in (0, 49, 50, 2 ** 31 - 1, 2 ** 31, 2 ** 32 - 1, 2 ** 32, n - 1):
+        assert int(a[pos].get()) == pos % 50, pos
+    assert int(a.sum().get()) == sum_mod(n, 50)       # two-pass reduction, 64-bit offsets
+    b = a + a                                         # flat vector kernel
+    assert int(b.sum().get()) == 2 * sum_mod(n, 50)
+    for pos in (2 ** 31 + 7, 2 ** 32 + 3, n - 1):
+        assert int(b[pos].get()) == 2 * (pos % 50), pos
+    del b
+    # index beyond 2**32 out of an arg-reduction; ties resolve to the first
+    assert int(a.argmax().get()) == 49
+    assert int(a.argmin().get()) == 0
+    a.fill(0)
+    a[n - 1] = 1
+    assert int(a.argmax().get()) == n - 1
+    a[2 ** 32 + 1] = 1
+    assert int(a.argmax().get()) == 2 ** 32 + 1
+    a[n - 1] = -1
+    assert int(a.argmin().get()) == n - 1
+
+
+def test_scan_of_2_to_32_elements():
+    n = 2 ** 32
+    a = cp.ones(n, 'b')
+    r = cp.cumprod(a, dtype='b')
+    assert r.shape == (n,) and r.dtype == np.int8
+    assert bool((r == 1).all().get())
+    del r
+    a[2 ** 31 + 11] = 0                               # everything after it becomes 0
+    r = cp.cumprod(a, dtype='b')
+    assert int(r.sum().get()) == 2 ** 31 + 11
+    assert int(r[2 ** 31 + 10].get()) == 1 and int(r[2 ** 31 + 11].get()) == 0
+    assert int(r[n - 1].get()) == 0
+
+
+def test_more_than_2_to_31_bytes_with_fewer_elements():
+    n = 2 ** 28 + 3
+    x = _fill_half_f64(size=n)
+    y = x * 2.0
+    check = cp.ElementwiseKernel('float64 y', 'bool ok', 'ok = y == (double)i', 'is_index_f64')
+    assert bool(check(y).all().get())
+    assert float(y[n - 1].get()) == n - 1
+
+
+def test_transposed_operand_beyond_2_to_31_bytes():
+    rows, cols = 40000, 20000                         # 3.2 GB of float32
+    x = _fill_mod1000_f32(size=rows * cols).reshape(rows, cols)
+    t = x.T * 2.0                                     # tiled kernel, 64-bit offsets
+    assert t.shape == (cols, rows) and t._c_contiguous
+    check = cp.ElementwiseKernel(
+        'float32 t', 'bool ok',
+        'const long long c = i / 40000, r = i % 40000;'
+        'ok = t == 2.0f * (float)((r * 20000 + c) % 1000)', 'is_transposed_mod1000')
+    assert bool(check(t).all().get())
+    host = t[cols - 3:, rows - 5:].get()
+    r, c = np.meshgrid(np.arange(rows - 5, rows), np.arange(cols - 3, cols))
+    assert np.array_equal(host, (2.0 * ((r * cols + c) % 1000)).astype(np.float32))
+
+
+def test_axis_reductions_and_scans_with_rows_beyond_2_to_30():
+    m = 2 ** 30 + 1
+    a = _fill_mod100_i8(size=3 * m).reshape(3, m)
+    rows = a.sum(axis=1).get()
+    want = [sum_mod100((k + 1) * m) - sum_mod100(k * m) for k in range(3)]
+    assert rows.tolist() == want
+    colsum = a.sum(axis=0)
+    assert colsum.shape == (m,) and colsum.dtype == np.int64
+    check = cp.ElementwiseKernel(
+        'int64 s', 'bool ok',
+        'const long long m = 1073741825LL;'
+        'ok = s == (i % 100) + ((m + i) % 100) + ((2 * m + i) % 100)', 'is_colsum_mod100')
+    assert bool(check(colsum).all().get())
+    del colsum
+    running = cp.cumsum(a, axis=0, dtype=np.int16)
+    check3 = cp.ElementwiseKernel(
+        'int16 s', 'bool ok',
+        'const long long m = 1073741825LL; const long long k = i / m, j = i % m;'
+        'long long w = 0; for (long long q = 0; q <= k; ++q) w += (q * m + j) % 100;'
+        'ok = s == w', 'is_running_colsum_mod100')
+    assert bool(check3(running).all().get())
+    del running
+    # argmax over rows whose element offsets need 64 bits although the index
+    # within a row does not
+    b = a.reshape(-1)[:3000000 * 1027].reshape(3000000, 1027)
+    idx = b.argmax(axis=1)
+    check2 = cp.ElementwiseKernel(
+        'int64 k', 'bool ok', 'ok = k == (99 - ((long long)i * 1027) % 100) % 100', 'is_first_99')
+    assert bool(check2(idx).all().get())
+
+
+def test_broadcast_input_of_2_to_31_elements():
+    base = _fill_mod100_i8(size=2048 * 1024).reshape(2048, 1, 1024)
+    a = cp.broadcast_to(base, (2048, 1024, 1024))
+    got = a.sum(axis=2)
+    assert got.shape == (2048, 1024) and got.dtype == np.int64
+    want = base.sum(axis=2)                           # (2048, 1), the same for every copy
+    assert bool((got == want).all().get())
+    assert np.array_equal(want.get()[:3, 0],
+                          [sum_mod100((k + 1) * 1024) - sum_mod100(k * 1024) for k in range(3)])
+
+
+def test_strided_view_into_more_than_2_to_31_bytes():
+    n = 1300
+    base = _fill_mod100_i8(size=n * n * n).reshape(n, n, n)
+    other = _fill_mod100_i8(size=n * (n // 2) * n).reshape(n, n // 2, n)
+    r = base[:, ::2, :] + other
+    assert r.shape == (n, n // 2, n)
+    for k in (0, n // 2, n - 1):
+        i0, i1, i2 = np.meshgrid([k], np.arange(0, n, 2), np.arange(n), indexing='ij')
+        lhs = (i0 * n * n + i1 * n + i2) % 100
+        j0, j1, j2 = np.meshgrid([k], np.arange(n // 2), np.arange(n), indexing='ij')
+        rhs = (j0 * (n // 2) * n + j1 * n + j2) % 100
+        assert np.array_equal(r[k].get(), (lhs + rhs)[0].astype(np.int8)), k
+
+
+def test_many_short_rows():
+    n_rows, width = 2 ** 25, 64                      # 2 GiB of int8, 33.5 million results
+    a = _fill_mod100_i8(size=n_rows * width).reshape(n_rows, width)
+    rows = a.sum(axis=1)
+    assert rows.shape == (n_rows,) and rows.dtype == np.int64
+    assert int(rows.sum().get()) == sum_mod100(n_rows * width)
+    for k in (0, 1, 2 ** 24 + 3, n_rows - 1):
+        assert int(rows[k].get()) == sum_mod100((k + 1) * width) - sum_mod100(k * width), k
+    first = a.argmax(axis=1)
+    check = cp.ElementwiseKernel(
+        'int64 k', 'bool ok',
+        # the row starts at (64 i) % 100; the largest value is 99 if the row
+        # reaches it, the last element of the row otherwise
+        'const long long s = ((long long)i * 64) % 100;'
+        'ok = k == (s + 63 >= 99 ? 99 - s : 63)', 'is_row_argmax_mod100')
+    assert bool(check(first).all().get())

@@ -1,0 +1,60 @@
+"""Launch geometry for arrays beyond 2**31 elements, without a GPU: in the
+compile-check mode allocations are addresses only, so the host path can be
+driven with shapes of any size.  A dispatch holds its size in work-items in 32
+bits per dimension; launches beyond that are rejected by Function.launch_packed,
+so every case below would raise if a grid were too large.  The same shapes run
+on the device in tests/test_gpu_huge.py."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from cupy_amd import _dryrun
+
+pytestmark = pytest.mark.skipif(not _dryrun.enabled(),
+                                reason='drives the host path with fake allocations')
+
+
+def launches_of(fn):
+    n0 = len(_dryrun.launches)
+    out = fn()
+    return out, _dryrun.launches[n0:]
+
+
+CASES = {
+    'flat': lambda: cp.empty((2 ** 32 + 1,), np.int8) + cp.empty((2 ** 32 + 1,), np.int8),
+    'full_sum': lambda: cp.empty((2 ** 32 + 1,), np.int8).sum(),
+    'argmax': lambda: cp.empty((2 ** 32 + 1,), np.int8).argmax(),
+    'rows_few': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=1),
+    'rows_many': lambda: cp.empty((2 ** 25, 64), np.int8).sum(axis=1),
+    'rows_very_many': lambda: cp.empty((2 ** 29, 4), np.int8).sum(axis=1),
+    'cols_wide': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=0),
+    'cols_split': lambda: cp.empty((2 ** 16, 2 ** 16), np.int8).sum(axis=0),
+    'tiled': lambda: cp.empty((2 ** 17, 2 ** 16), np.int8).T * np.int8(2),
+    'generic': lambda: cp.empty((70, 2 ** 13, 2 ** 13), np.int8)[::2, :, ::2].sum(axis=1),
+    'scan_rows': lambda: cp.cumsum(cp.empty((2 ** 32 + 1,), np.int8), dtype='b'),
+    'scan_cols': lambda: cp.cumsum(cp.empty((3, 2 ** 30 + 1), np.int8), axis=0, dtype='b'),
+}
+
+
+@pytest.mark.parametrize('name', sorted(CASES))
+def test_dispatch_fits_32_bit_work_item_counts(name):
+    _, launches = launches_of(CASES[name])
+    assert launches
+    for kernel, grid, block, _, _ in launches:
+        for g, b in zip(grid, block):
+            assert 1 <= g * b <= 0xffffffff, (kernel, grid, block)
+        assert grid[1] <= 65535 and grid[2] <= 65535, (kernel, grid)
+
+
+def test_an_oversized_dispatch_is_rejected_not_truncated():
+    k = cp.RawKernel('extern "C" __global__ void nop(int* p) {}', 'nop')
+    x = cp.empty((4,), np.int32)
+    with pytest.raises(ValueError, match='work-items'):
+        k((2 ** 24,), (256,), (x,))
+
+
+def test_column_blocks_beyond_grid_x_continue_along_grid_z():
+    out, launches = launches_of(CASES['cols_wide'])
+    (kernel, grid, block, _, _), = launches
+    assert grid[2] == 2 and grid[0] * grid[2] * 64 >= 2 ** 30 + 1
+    assert out.shape == (2 ** 30 + 1,)
