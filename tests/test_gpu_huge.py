@@ -170,3 +170,51 @@ def test_many_short_rows():
         'const long long s = ((long long)i * 64) % 100;'
         'ok = k == (s + 63 >= 99 ? 99 - s : 63)', 'is_row_argmax_mod100')
     assert bool(check(first).all().get())
+
+
+def test_very_many_tiny_rows():
+    n_rows = 2 ** 29                                  # 2 GiB in, 4 GiB of int64 out
+    a = _fill_mod100_i8(size=n_rows * 4).reshape(n_rows, 4)
+    rows = a.sum(axis=1)
+    check = cp.ElementwiseKernel(
+        'int64 s', 'bool ok',
+        'const long long b = (long long)i * 4;'
+        'ok = s == b % 100 + (b + 1) % 100 + (b + 2) % 100 + (b + 3) % 100', 'is_rowsum4_mod100')
+    assert bool(check(rows).all().get())
+
+
+def test_three_dimensional_view_that_does_not_merge():
+    na, nb, nc = 70, 8192, 8192                       # 4.7e9 elements underneath
+    base = _fill_mod100_i8(size=na * nb * nc).reshape(na, nb, nc)
+    view = base[::2, ::2, ::2]                        # no two axes merge
+    assert view.shape == (35, 4096, 4096)
+    value = '(2 * a * 8192LL * 8192 + 2 * b * 8192 + 2 * c) % 100'
+    # elementwise through the indexer kernel, offsets in 64 bits
+    r = view + np.int8(1)
+    assert r._c_contiguous and r.shape == view.shape
+    check = cp.ElementwiseKernel(
+        'int8 v', 'bool ok',
+        'const long long c = i % 4096, b = (i / 4096) % 4096, a = i / (4096LL * 4096);'
+        'ok = v == VALUE + 1'.replace('VALUE', value), 'is_view_plus_one')
+    assert bool(check(r).all().get())
+    del r
+    # reduction over the middle axis of the same view
+    s = view.sum(axis=1)
+    assert s.shape == (35, 4096) and s.dtype == np.int64
+    check2 = cp.ElementwiseKernel(
+        'int64 s', 'bool ok',
+        'const long long c = i % 4096, a = i / 4096; long long w = 0;'
+        'for (long long b = 0; b < 4096; ++b) w += VALUE;'
+        'ok = s == w'.replace('VALUE', value), 'is_view_middle_sum')
+    assert bool(check2(s).all().get())
+    # and an arg-reduction over its leading axis
+    k = view.argmax(axis=0)
+    assert k.shape == (4096, 4096) and k.dtype == np.int64
+    check3 = cp.ElementwiseKernel(
+        'int64 k', 'bool ok',
+        'const long long c = i % 4096, b = i / 4096; long long best = -1, at = -1;'
+        'for (long long a = 0; a < 35; ++a) {'
+        '  const long long v = VALUE;'
+        '  if (v > best) { best = v; at = a; } }'
+        'ok = k == at'.replace('VALUE', value), 'is_view_leading_argmax')
+    assert bool(check3(k).all().get())
