@@ -176,3 +176,53 @@ def test_compile_error_surfaces_as_exception():
     with pytest.raises(cp.cuda.CompileException) as info:
         k(cp.zeros((4,), np.float32))
     assert 'undefined_function' in str(info.value)
+
+
+def test_threads_with_their_own_streams():
+    """Eight threads, each on its own stream, compile the same cold kernels at
+    the same moment, then run elementwise, reduction, fused and scan calls on
+    private data while allocating from the shared pool (the scenario of the
+    reference's tests/cupy_tests/core_tests/test_multithreading.py:56-155)."""
+    import threading
+    n_threads = 8
+    barrier = threading.Barrier(n_threads)
+    kernel = cp.ElementwiseKernel('T x, T y, T a', 'T z', 'z = a * x + y + 7', 'threads_cold_axpy')
+    fused = cp.fuse(lambda x, y: cp.sum((x - y) * (x - y), axis=1))
+    errors = []
+    results = [None] * n_threads
+
+    def worker(k):
+        try:
+            rng = np.random.default_rng(100 + k)
+            stream = cp.cuda.Stream()
+            with stream:
+                barrier.wait()
+                for it in range(12):
+                    rows = 50 + 7 * k + it
+                    x = rng.standard_normal((rows, 257)).astype(np.float32)
+                    y = rng.standard_normal((rows, 257)).astype(np.float32)
+                    dx, dy = cp.asarray(x), cp.asarray(y)
+                    z = kernel(dx, dy, np.float32(k + 1))
+                    s = (dx * dy).sum(axis=0)
+                    f = fused(dx, dy)
+                    c = cp.cumsum(dx, axis=1)
+                    idx = dx.argmax(axis=1)
+                    stream.synchronize()
+                    assert np.array_equal(z.get(), np.float32(k + 1) * x + y + np.float32(7))
+                    np.testing.assert_allclose(s.get(), (x * y).sum(axis=0), rtol=1e-4, atol=1e-4)
+                    np.testing.assert_allclose(f.get(), ((x - y) ** 2).sum(axis=1), rtol=1e-4)
+                    np.testing.assert_allclose(c.get(), np.cumsum(x, axis=1), rtol=1e-4, atol=1e-4)
+                    assert np.array_equal(idx.get(), x.argmax(axis=1))
+            results[k] = True
+        except Exception as e:          # noqa: BLE001 - reported by the main thread
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(n_threads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert all(results)
+    # one compiled kernel per input type tuple, however many threads raced for it
+    assert len(kernel._cached_codes) == 1
