@@ -186,6 +186,103 @@ def build_cases(cp, scale=1):
     return cases
 
 
+def build_next_cases(cp):
+    """Operations of the components built after the five configurations (scans,
+    statistics, complex types, multi-kernel fused functions), at shapes of the
+    same size class.  ``bytes`` is the algorithmic traffic: every input element
+    read once, every output element written once -- also where the operation as
+    defined takes several passes (variance, softmax), so that the fraction of
+    peak shows the cost of those passes."""
+    cases = []
+
+    def add(name, nbytes, gpu, cpu, check, kernel):
+        cases.append(dict(name=name, config='next', bytes=int(nbytes), gpu=gpu, cpu=cpu,
+                          check=check, kernel=kernel))
+
+    def close(got, want, rtol, scale=None):
+        got = got.get().astype(np.float64 if got.dtype.kind != 'c' else np.complex128)
+        err = np.abs(got - want)
+        bound = rtol * (np.abs(want) if scale is None else scale) + 1e-30
+        return bool(np.all(err <= bound))
+
+    rng = np.random.default_rng(11)
+    # ---- scans ------------------------------------------------------------------------
+    for shape, axis in (((1 << 20, 64), 1), ((8192, 8192), 1), ((64, 1 << 20), 0),
+                        ((1 << 26,), 0)):
+        a = rng.standard_normal(shape, dtype=np.float32)
+        da = cp.asarray(a)
+        out = cp.empty(shape, np.float32)
+        label = 'cumsum f32 %s axis=%d' % ('x'.join(str(s) for s in shape), axis)
+
+        def check(a=a, out=out, axis=axis):
+            return close(out, np.cumsum(a, axis=axis, dtype=np.float64), 1e-5,
+                         np.cumsum(np.abs(a), axis=axis, dtype=np.float64))
+        add(label, 2 * a.nbytes, lambda da=da, axis=axis, out=out: cp.cumsum(da, axis=axis, out=out),
+            lambda a=a, axis=axis: np.cumsum(a, axis=axis), check, 'cupy_scan')
+    # ---- statistics -------------------------------------------------------------------
+    m = rng.standard_normal((16384, 8192), dtype=np.float32)
+    dm = cp.asarray(m)
+    o_mean = cp.empty((16384,), np.float32)
+    add('mean f32 16384x8192 axis=1', m.nbytes + 16384 * 4,
+        lambda: dm.mean(axis=1, out=o_mean), lambda: m.mean(axis=1),
+        lambda: close(o_mean, m.mean(axis=1, dtype=np.float64), 1e-5,
+                      np.abs(m).mean(axis=1, dtype=np.float64)), 'cupy_mean')
+    res_var = [None]
+
+    def gpu_var():
+        res_var[0] = dm.var(axis=0)
+    add('var f32 16384x8192 axis=0 (two passes by definition)', m.nbytes + 8192 * 4,
+        gpu_var, lambda: m.var(axis=0),
+        lambda: close(res_var[0], m.var(axis=0, dtype=np.float64), 1e-4), 'cupy_var_core')
+    mn = m.copy()
+    mn[::7, ::5] = np.nan
+    dmn = cp.asarray(mn)
+    o_nanmax = cp.empty((16384,), np.float32)
+    add('nanmax f32 16384x8192 axis=1', m.nbytes + 16384 * 4,
+        lambda: cp.nanmax(dmn, axis=1, out=o_nanmax), lambda: np.nanmax(mn, axis=1),
+        lambda: bool(np.array_equal(o_nanmax.get(), np.nanmax(mn, axis=1))), 'cupy_nanmax')
+    # ---- complex ----------------------------------------------------------------------
+    n = 1 << 25
+    z1 = (rng.standard_normal(n) + 1j * rng.standard_normal(n)).astype(np.complex64)
+    z2 = (rng.standard_normal(n) + 1j * rng.standard_normal(n)).astype(np.complex64)
+    dz1, dz2 = cp.asarray(z1), cp.asarray(z2)
+    oz = cp.empty((n,), np.complex64)
+    add('multiply complex64 2^25', 3 * z1.nbytes, lambda: cp.multiply(dz1, dz2, oz),
+        lambda: np.multiply(z1, z2),
+        lambda: close(oz, z1.astype(np.complex128) * z2.astype(np.complex128), 5e-7), 'cupy_multiply')
+    oa = cp.empty((n,), np.float32)
+    add('absolute complex64 2^25', z1.nbytes + n * 4, lambda: cp.absolute(dz1, oa),
+        lambda: np.absolute(z1),
+        lambda: close(oa, np.abs(z1.astype(np.complex128)), 3e-7), 'cupy_absolute')
+    w1 = (rng.standard_normal(n // 2) + 1j * rng.standard_normal(n // 2))
+    dw1 = cp.asarray(w1)
+    osum = cp.empty((), np.complex128)
+    add('sum complex128 2^24', w1.nbytes + 16, lambda: dw1.sum(out=osum), lambda: w1.sum(),
+        lambda: close(osum, np.asarray(w1.sum()), 1e-12, np.abs(w1).sum()), 'cupy_sum')
+    # ---- multi-kernel fused function ----------------------------------------------------
+    s = rng.standard_normal((16384, 4096), dtype=np.float32)
+    ds = cp.asarray(s)
+
+    @cp.fuse(kernel_name='softmax_rows')
+    def softmax(x):
+        e = cp.exp(x - cp.amax(x, axis=1, keepdims=True))
+        return e / cp.sum(e, axis=1, keepdims=True)
+    res_sm = [None]
+
+    def gpu_softmax():
+        res_sm[0] = softmax(ds)
+
+    def cpu_softmax():
+        e = np.exp(s - s.max(axis=1, keepdims=True))
+        return e / e.sum(axis=1, keepdims=True)
+    add('fused softmax f32 16384x4096 (3 kernels, x read 3 times)', 2 * s.nbytes, gpu_softmax,
+        cpu_softmax, lambda: close(res_sm[0], cpu_softmax().astype(np.float64), 1e-5), 'softmax_rows')
+    ex = cp.empty((16384, 4096), np.float32)
+    add('exp f32 2^26', 2 * s.nbytes, lambda: cp.exp(ds, ex), lambda: np.exp(s),
+        lambda: close(ex, np.exp(s.astype(np.float64)), 3e-7), 'cupy_exp')
+    return cases
+
+
 def time_case_events(cp, fn, repeats, inner):
     """Median over ``repeats`` of the time per call, each sample being
     ``inner`` back-to-back calls bracketed by two events on the launch stream."""
@@ -260,6 +357,10 @@ def main():
     ap.add_argument('--no-detail', action='store_true',
                     help='skip per-operation event timing and launch latency')
     ap.add_argument('--only', default='', help='run only cases whose name contains this')
+    ap.add_argument('--suite', default='configs', choices=('configs', 'next'),
+                    help="'configs': the five benchmark configurations (the headline figure); "
+                         "'next': scans, statistics, complex types and multi-kernel fused "
+                         "functions at shapes of the same size class")
     ap.add_argument('--calibrate', action='store_true',
                     help='add a plain copy kernel of known size (256 MiB in, 256 MiB out) to '
                          'every step, as the yardstick for hardware traffic counters')
@@ -275,7 +376,7 @@ def main():
     props = cp.cuda.device.get_device_properties(0)
     log('device:', props['arch'], props['compute_units'], 'CUs')
     t0 = time.perf_counter()
-    cases = build_cases(cp, args.scale)
+    cases = build_cases(cp, args.scale) if args.suite == 'configs' else build_next_cases(cp)
     if args.only:
         cases = [c for c in cases if args.only in c['name']]
     log('inputs ready in %.1f s' % (time.perf_counter() - t0))
@@ -334,7 +435,8 @@ def main():
         roof = {'bound': 'hbm', 'kernel': dom['kernel'], 'operation': dom['name'],
                 'achieved': dom['gbps'], 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
                 'frac': dom['frac'],
-                'traffic': MEASURED_TRAFFIC_BYTES.get(dom['name']) if args.scale == 1 else None,
+                'traffic': MEASURED_TRAFFIC_BYTES.get(dom['name'])
+                if args.scale == 1 and args.suite == 'configs' else None,
                 'launch_us': dom['us'], 'algorithmic_bytes': dom['bytes']}
     else:
         roof = {'bound': 'hbm', 'achieved': round(value, 1), 'peak': HBM_PEAK_GBPS,
@@ -358,9 +460,10 @@ def main():
             model = 'unknown'
         cpu = {'value': round(total_bytes / best / 1e9, 2), 'unit': 'GB/s', 'cores': 1,
                'kind': 'port',
-               'sample': 'one full pass of the same 13 operations with NumPy %s on the host '
+               'sample': 'one full pass of the same %d operations with NumPy %s on the host '
                          '(best of 3 after a warm pass, outputs preallocated where NumPy allows); '
-                         '%d host cores visible, CPU: %s' % (np.__version__, os.cpu_count(), model),
+                         '%d host cores visible, CPU: %s' % (
+                             len(cases), np.__version__, os.cpu_count(), model),
                'seconds_per_pass': round(best, 3)}
 
     result = {
@@ -377,7 +480,10 @@ def main():
         'dtype': 'f32/f64/f16/i32 (the element types of the five configurations)',
         'data': 'synthetic (seeded NumPy RNG, uploaded once)',
         'config': {'workload': 'C1-C5 of BASELINE.json at full shapes, 13 operations per step'
-                   if args.scale == 1 and not args.only else
+                   if args.scale == 1 and not args.only and args.suite == 'configs' else
+                   'NOT the benchmark figure: scans, statistics, complex types and multi-kernel '
+                   'fused functions, %d operations per step' % len(cases)
+                   if args.suite == 'next' and not args.only else
                    'REDUCED run (scale=%d only=%r): not the benchmark figure' % (args.scale, args.only),
                    'bytes_per_step': total_bytes, 'operations': len(cases)},
         'frac_of_hbm_peak': round(value / HBM_PEAK_GBPS, 4),

@@ -434,9 +434,19 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('    if (_full) {')
     src.append('      const %s _jstep = (%s)gridDim.y * %d;' % (idx_t, idx_t, ty))
     src.append('      %s _j = (%s)blockIdx.y * %d + _ty;' % (idx_t, idx_t, ty))
+    # operands that do not vary along the reduce axis are read once
+    for a in ins:
+        if a.bcast_r and not partial_in:
+            if a.bcast_o:
+                src.append('      const %s _r_%s = _p_%s[0];' % (a.store_t, a.name, a.name))
+            else:
+                src.append('      const cupy::Vec<%s, %d> _r_%s = cupy::load_vec<%s, %d, false>('
+                           '_p_%s + _c);' % (a.store_t, vec, a.name, a.store_t, vec, a.name))
 
     def loads(pad, j_expr, suffix):
         for a in ins:
+            if a.bcast_r and not partial_in:
+                continue
             if partial_in:
                 # partial results may have any size: plain element reads
                 src.append('%s_type_reduce _l_%s%s[%d];' % (pad, a.name, suffix, vec))
@@ -463,8 +473,11 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
             src.append('%s    _acc[_k] = REDUCE(_acc[_k], _l_%s%s[_k]);' % (pad, a.name, suffix))
         else:
             for a in ins:
-                val = ('_b_%s%s' % (a.name, suffix)) if a.bcast_o else (
-                    '_l_%s%s.v[_k]' % (a.name, suffix))
+                if a.bcast_r:
+                    val = ('_r_%s' % a.name) if a.bcast_o else ('_r_%s.v[_k]' % a.name)
+                else:
+                    val = ('_b_%s%s' % (a.name, suffix)) if a.bcast_o else (
+                        '_l_%s%s.v[_k]' % (a.name, suffix))
                 src.append('%s    const %s %s(%s);' % (pad, a.var_t, a.name, val))
             src.append('%s    _type_reduce _a = static_cast<_type_reduce>(%s);' % (
                 pad, pre_map_expr))
@@ -490,7 +503,10 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('      for (%s _j = (%s)blockIdx.y * %d + _ty; _j < _n_red; _j += (%s)gridDim.y * %d) {' % (
         idx_t, idx_t, ty, idx_t, ty))
     src.append('        const IndexT _J = _j;')
-    src.append('        for (int _k = 0; _k < %d && _c + _k < _n_out; ++_k) {' % vec)
+    # a constant trip count with the bound tested inside: the accumulators are
+    # then indexed by constants only and stay in registers whatever their type
+    src.append('#pragma unroll')
+    src.append('        for (int _k = 0; _k < %d; ++_k) if (_c + _k < _n_out) {' % vec)
     if partial_in:
         a = ins[0]
         src.append('          _acc[_k] = REDUCE(_acc[_k], _p_%s[(ptrdiff_t)_j * _sr_%s + _c + _k]);' % (

@@ -597,7 +597,7 @@ class _AbstractReductionKernel:
         span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
                    + [abs(s) * n_out for s in so_out] + [n_red + n_split * ty])
         idx64 = span > _INT32_MAX - (1 << 24)
-        rargs = self._rargs(in_args, out_args, bcast_o=bcast_o)
+        rargs = self._rargs(in_args, out_args, bcast_r=[s == 0 for s in sr], bcast_o=bcast_o)
         stream_hint = _tuning.stream_policy(
             _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,

@@ -8,6 +8,7 @@ and among equals (or among NaNs) the smaller index wins -- which is NumPy's
 first-occurrence rule.
 """
 from cupy_amd._core import _fusion_thread_local
+from cupy_amd._core import internal
 from cupy_amd._core._reduction import create_reduction_func
 
 _min_max_preamble = '''
@@ -339,7 +340,78 @@ def _var_core(out_type):
     return ker
 
 
+_var_onepass_preamble = '''
+// Sums of d and d*d for d = x - k, k a pivot near the data (shifted-data
+// algorithm, Chan, Golub, LeVeque 1983): with sum(d*d) - sum(d)^2 / n the
+// variance comes out of ONE pass.  The cancellation in that difference grows
+// with (distance of the pivot from the mean / standard deviation)^2, which the
+// choice of the pivot keeps near one.
+template <typename T>
+struct var_st {
+  T s1, s2;
+  __device__ __forceinline__ var_st() : s1(0), s2(0) {}
+  __device__ __forceinline__ explicit var_st(T d) : s1(d), s2(d * d) {}
+};
+template <typename T>
+__device__ __forceinline__ var_st<T> operator+(const var_st<T>& a, const var_st<T>& b) {
+  var_st<T> r;
+  r.s1 = a.s1 + b.s1;
+  r.s2 = a.s2 + b.s2;
+  return r;
+}
+template <typename T>
+__device__ __forceinline__ T var_finish(const var_st<T>& a, T inv_n, T alpha) {
+  const T m2 = a.s2 - a.s1 * a.s1 * inv_n;
+  return alpha * (m2 < 0 ? T(0) : m2);          // NaN stays NaN
+}
+'''
+
+_var_onepass_cores = {}
+_median3 = None
+
+
+def _var_onepass(out_name):
+    """ReductionKernel of the one-pass variance, accumulating in double for a
+    float64 result and in float otherwise (as the sums of those types do)."""
+    from cupy_amd._core._reduction import ReductionKernel
+    ker = _var_onepass_cores.get(out_name)
+    if ker is None:
+        work, scalar_t = ('double', 'float64') if out_name == 'float64' else ('float', 'float32')
+        ker = ReductionKernel(
+            'S x, S k, %s inv_n, %s alpha' % (scalar_t, scalar_t), '%s out' % out_name,
+            'var_st<%s>(static_cast<%s>(x) - static_cast<%s>(k))' % (work, work, work),
+            'a + b', 'out = var_finish<%s>(a, inv_n, alpha)' % work, 'var_st<%s>()' % work,
+            'cupy_var_' + out_name, reduce_type='var_st<%s>' % work,
+            preamble=_var_onepass_preamble)
+        _var_onepass_cores[out_name] = ker
+    return ker
+
+
+def _var_pivot(a, axis):
+    """Per output, the median of the first, middle and last element along the
+    reduced axes (shape of ``a`` with the reduced axes of length one): a value
+    near the data unless two of the three probes are outliers."""
+    global _median3
+    if _median3 is None:
+        from cupy_amd._core._kernel import ElementwiseKernel
+        _median3 = ElementwiseKernel(
+            'T a, T b, T c', 'T k',
+            'const T lo = a < b ? a : b; const T hi = a < b ? b : a;'
+            'k = (a != a || b != b) ? (a != a ? a : b) : (c < lo ? lo : (c > hi ? hi : c))',
+            'cupy_var_pivot')
+    probes = []
+    for pick in (lambda n: 0, lambda n: n // 2, lambda n: n - 1):
+        key = tuple(slice(pick(n), pick(n) + 1) if ax in axis else slice(None)
+                    for ax, n in enumerate(a.shape))
+        probes.append(a[key])
+    return _median3(*probes)
+
+
 def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
+    """Variance.  Real inputs take one pass over the data around a pivot read
+    from the data itself (the reference reads them twice: the mean first, then
+    the squared deviations, cupy/_core/_routines_statistics.pyx:553-598);
+    complex inputs keep that two-pass form."""
     import numpy
     if axis is None:
         axis = tuple(range(a.ndim))
@@ -361,6 +433,12 @@ def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
         items *= a.shape[ax]
     div = max(items - ddof, 0)
     alpha = 1. / div if div != 0 else float('nan')
+    if (a.dtype.kind in 'biuf' and dtype_out.kind == 'f' and dtype_out.itemsize <= 8
+            and items > 0 and (out is None or out.dtype == dtype_out)):
+        axis = tuple(internal._normalize_axis_index(ax, a.ndim) for ax in axis)
+        pivot = _var_pivot(a, axis)
+        args = (a, pivot, 1. / items, alpha) + (() if out is None else (out,))
+        return _var_onepass(dtype_out.name)(*args, axis=axis, keepdims=keepdims)
     arrmean = a.mean(axis=axis, dtype=dtype_mean, out=None, keepdims=True)
     if out is None:
         name = dtype_out.name if dtype_out.name in ('float16', 'float32') else 'float64'

@@ -199,3 +199,61 @@ def test_nan_reductions(dtype):
     assert_exact(cp.nanargmax(cp.asarray(hi), axis=1).get(), np.nanargmax(hi, axis=1))
     assert_exact(cp.count_nonzero(cp.asarray(hi), axis=0).get(), np.count_nonzero(hi, axis=0))
     assert int(cp.count_nonzero(cp.asarray(hi)).get()) == np.count_nonzero(hi)
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'float64'])
+def test_one_pass_variance_is_stable_and_matches_numpy(dtype):
+    """The variance is computed in one pass over the data, as sums of (x - k)
+    and (x - k)**2 around a pivot k taken from the data.  Data with a mean far
+    above its spread is where a plain sum-of-squares formula cancels
+    catastrophically; with the pivot it must not."""
+    rng = np.random.default_rng(91)
+    rtol = 2e-5 if dtype == 'float32' else 1e-11
+    for offset in (0.0, 1.0e3, 1.0e4, -3.0e5):
+        h = (rng.standard_normal((513, 1031)) + offset).astype(dtype)
+        d = cp.asarray(h)
+        for axis in (None, 0, 1):
+            for ddof in (0, 1):
+                want = h.astype(np.float64).var(axis=axis, ddof=ddof)
+                got = d.var(axis=axis, ddof=ddof)
+                assert got.dtype == np.dtype(dtype)
+                np.testing.assert_allclose(got.get(), want, rtol=rtol)
+    # an outlier where a probe of the pivot looks: the median of three probes
+    # ignores it
+    h = rng.standard_normal((513, 1031)).astype(dtype)
+    h[0, :] = 1.0e6
+    h[:, 1030] = -1.0e6
+    d = cp.asarray(h)
+    for axis in (0, 1):
+        np.testing.assert_allclose(d.var(axis=axis).get(), h.astype(np.float64).var(axis=axis),
+                                   rtol=rtol)
+    # NaN and infinity propagate as in NumPy
+    h = rng.standard_normal((40, 50)).astype(dtype)
+    h[3, 4] = np.nan
+    h[5, 6] = np.inf
+    with np.errstate(all='ignore'):
+        want = h.var(axis=0)
+    got = cp.asarray(h).var(axis=0).get()
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_allclose(got[~np.isnan(want)], want[~np.isnan(want)], rtol=20 * rtol)
+    # long reductions split over many blocks, and integers (computed in double)
+    h = (rng.standard_normal((3, 400001)) * 3 + 100).astype(dtype)
+    np.testing.assert_allclose(cp.asarray(h).var(axis=1).get(),
+                               h.astype(np.float64).var(axis=1), rtol=20 * rtol)
+    np.testing.assert_allclose(cp.asarray(h).var().get(), h.astype(np.float64).var(),
+                               rtol=20 * rtol)
+    i = rng.integers(-1000, 1000, (257, 129)).astype(np.int32)
+    got = cp.asarray(i).var(axis=0, ddof=1)
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(got.get(), i.var(axis=0, ddof=1), rtol=1e-12)
+    # constant data: exactly zero
+    c = np.full((100, 100), 7.25, dtype)
+    assert np.array_equal(cp.asarray(c).var(axis=0).get(), np.zeros(100, dtype))
+    # out= and std
+    out = cp.empty((1031,), dtype)
+    h = rng.standard_normal((513, 1031)).astype(dtype)
+    r = cp.asarray(h).var(axis=0, out=out)
+    assert r is out
+    np.testing.assert_allclose(out.get(), h.var(axis=0), rtol=20 * rtol)
+    np.testing.assert_allclose(cp.asarray(h).std(axis=1, ddof=1).get(), h.std(axis=1, ddof=1),
+                               rtol=20 * rtol)
