@@ -424,9 +424,15 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     n_it = n_work // threads
     pre_ops = [op for op in arrays
                if layouts[op.name] == 'R' and ((not op.is_out) or op.read_out)]
+    row_ops = [op for op in arrays
+               if layouts[op.name] == 'R0' and ((not op.is_out) or op.read_out)]
     for op in pre_ops:
         src.append('    cupy::Vec<%s, %d> _pre_%s[%d];' % (op.store_t, vec, op.name, n_it))
-    if pre_ops:
+    # per-row values travel with them: a load left to the consume loop would
+    # only be issued after the wait for the vectors
+    for op in row_ops:
+        src.append('    %s _prer_%s[%d];' % (op.store_t, op.name, n_it))
+    if pre_ops or row_ops:
         src.append('    if (_interior) {')
         src.append('#pragma unroll')
         src.append('      for (int _it = 0; _it < %d; ++_it) {' % n_it)
@@ -436,6 +442,8 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         for op in pre_ops:
             src.append('        _pre_%s[_it] = cupy::load_vec<%s, %d, %s>(%s);' % (
                 op.name, op.store_t, vec, ntl, gaddr(op, '_r', '_c')))
+        for op in row_ops:
+            src.append('        _prer_%s[_it] = *%s;' % (op.name, gaddr(op, '_r', '0')))
         src.append('      }')
         src.append('    }')
     if c_ops:
@@ -496,7 +504,11 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
             else:
                 src.append('        cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
         elif lay == 'R0':
-            src.append('        const %s _b_%s = *%s;' % (op.store_t, op.name, gaddr(op, '_r', '0')))
+            if (not op.is_out) or op.read_out:
+                src.append('        const %s _b_%s = _prer_%s[_it];' % (op.store_t, op.name, op.name))
+            else:
+                src.append('        const %s _b_%s = *%s;' % (
+                    op.store_t, op.name, gaddr(op, '_r', '0')))
     src.append('#pragma unroll')
     src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
     if use_i or set_ind:

@@ -645,6 +645,17 @@ class _ElementwisePlanner:
         else:
             tile_r = tile_c = 64
             threads = 256
+        if n_transposed == 0:
+            # Nothing is staged: every operand runs along the columns, so the
+            # tile is made as wide as divides the row length (up to one vector
+            # per thread) and a few rows high -- long contiguous runs, like the
+            # flat kernel, with the per-row operands read once per row.
+            wide = threads * vec
+            while wide > tile_c and nc % wide:
+                wide //= 2
+            if wide > tile_c:
+                tile_r = tile_r * tile_c // wide
+                tile_c = wide
         if lds_item * tile_r * (tile_c + 1) > 150 * 1024:
             return None       # too many staged operands for the LDS
         span = 0
