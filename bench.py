@@ -275,7 +275,7 @@ def build_next_cases(cp):
     def cpu_softmax():
         e = np.exp(s - s.max(axis=1, keepdims=True))
         return e / e.sum(axis=1, keepdims=True)
-    add('fused softmax f32 16384x4096 (3 kernels, x read 3 times)', 2 * s.nbytes, gpu_softmax,
+    add('fused softmax f32 16384x4096 (one kernel, rows in registers)', 2 * s.nbytes, gpu_softmax,
         cpu_softmax, lambda: close(res_sm[0], cpu_softmax().astype(np.float64), 1e-5), 'softmax_rows')
     ex = cp.empty((16384, 4096), np.float32)
     add('exp f32 2^26', 2 * s.nbytes, lambda: cp.exp(ds, ex), lambda: np.exp(s),

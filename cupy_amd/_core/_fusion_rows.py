@@ -1,0 +1,444 @@
+"""One kernel for fused functions whose reductions all run along the last axis.
+
+Row-wise normalisations -- softmax, standardisation, a norm followed by a
+division -- reduce every row of a matrix and combine the results with the row
+again.  Cut at the reductions (``_fusion_split``) they become a sequence of
+kernels that each read the matrix once more.  When a row is short enough to be
+held in the registers of one workgroup, the whole function fits in ONE kernel:
+a group of lanes loads a row, runs the reductions one after the other on the
+registers (wave all-reduce, LDS across waves), evaluates the elementwise results
+from the same registers and stores them.  The matrix is read once and written
+once.  The reference has no counterpart on this platform: its general tracer
+needs a grid-wide barrier (cupy/_core/_fusion_kernel.pyx:99-115).
+
+The pieces of the function (one map-reduce function per reduction, one
+elementwise function per result) are traced by the single-kernel tracer of
+``fusion.py`` in "describe" mode; this module only composes the device
+functions it produced.
+"""
+import numpy
+
+from cupy_amd._core import _codegen_reduction as _cg
+from cupy_amd._core import _launch_plan
+from cupy_amd._core import _tuning
+from cupy_amd._core import internal
+from cupy_amd._core._kernel import _make_packer, _scalar_struct_code, _aligned
+from cupy_amd._core._scalar import CScalar, get_typename
+from cupy_amd._core.core import ndarray
+from cupy_amd.cuda import compiler
+from cupy_amd.cuda import device as _device
+from cupy_amd.cuda import stream as _stream
+
+BLOCK = 256
+WAVE = 64
+# registers (32-bit words) per lane that rows held in registers may take
+_ROW_WORDS_PER_LANE = 64
+
+
+class _Unsupported(Exception):
+    pass
+
+
+def _kind_of_leaf(shape, full):
+    """How an argument of ``shape`` meets the rows of a ``full``-shaped array."""
+    if shape is None or internal.prod(shape) == 1 and len(shape) <= len(full) \
+            and all(s == 1 for s in shape):
+        return 'uni'
+    if tuple(shape) == tuple(full):
+        return 'full'
+    if len(full) >= 2 and tuple(shape) == tuple(full[:-1]) + (1,):
+        return 'rowk'
+    if len(shape) <= len(full) and shape[-1] == full[-1] and all(s == 1 for s in shape[:-1]):
+        return 'col'
+    raise _Unsupported('argument of shape %r against rows of %r' % (shape, full))
+
+
+def _classify(nodes, full):
+    """Kind of every recorded value: 'full' (one per element), 'col' (one per
+    column), 'row' / 'rowk' (one per row, without / with the reduced axis kept),
+    'uni' (one for all)."""
+    kinds = {}
+    last = len(full) - 1
+    for n in nodes:
+        if n.kind == 'leaf':
+            k = _kind_of_leaf(n.shape, full)
+        elif n.kind == 'reduce':
+            src = n.args[0]
+            if kinds.get(src.order) != 'full' or n.kwargs['axes'] != (last,):
+                raise _Unsupported('a reduction that is not along the last axis of a row')
+            k = 'row'
+        elif n.kind == 'keepdims':
+            k = 'rowk'
+        else:
+            ks = set(kinds[a.order] for a in n.args if hasattr(a, 'order'))
+            ks.discard('uni')
+            if not ks:
+                k = 'uni'
+            elif 'row' in ks:
+                # without the reduced axis NumPy would line such a value up with
+                # the columns; only values of the same family may meet it
+                if ks != {'row'} and len(full) > 1:
+                    raise _Unsupported('a reduced value without keepdims meets an array')
+                k = 'row' if ks == {'row'} else 'full'
+            elif 'full' in ks or ks == {'rowk', 'col'}:
+                k = 'full'
+            else:
+                k, = ks
+        expect = {'full': tuple(full), 'row': tuple(full[:-1]),
+                  'rowk': tuple(full[:-1]) + (1,)}.get(k)
+        if n.kind != 'leaf' and expect is not None and n.shape is not None \
+                and tuple(n.shape) != expect:
+            raise _Unsupported('shape %r of a %s value' % (n.shape, k))
+        kinds[n.order] = k
+    return kinds
+
+
+class RowPlan:
+    """The fused function as one launch."""
+
+    def __init__(self, fn, packer, grid, n_rows, in_slots, out_specs, returns, single):
+        self.fn = fn
+        self.packer = packer
+        self.grid = grid
+        self.n_rows = n_rows
+        # per kernel argument ('arg', position, x) or ('const', array, x); x is the
+        # alignment in bytes required of an array's data, or the dtype of a scalar
+        self.in_slots = tuple(in_slots)
+        self.out_specs = tuple(out_specs)    # (shape, dtype) per output pointer
+        self.returns = tuple(returns)        # ('out', k) | ('arg', position) | ('const', value)
+        self.single = single
+        self.fallback = None
+        self.steps = (('kernel', self),)
+
+    def run(self, *args):
+        vals = []
+        for what, ref, descr in self.in_slots:
+            v = args[ref] if what == 'arg' else ref
+            if type(descr) is int:
+                # an array: contiguous and aligned as the kernel's vector
+                # accesses assume, or the call goes the general way
+                ptr = v.data.ptr
+                if not v._c_contiguous or ptr % descr:
+                    return self.fallback.run(*args)
+                vals.append(ptr)
+            else:
+                vals.append(_launch_plan.scalar_value(v, descr))
+        outs = [ndarray._new_contiguous(shape, dtype) for shape, dtype in self.out_specs]
+        vals.extend(o.data.ptr for o in outs)
+        vals.append(self.n_rows)
+        self.fn.launch_packed(self.grid, (BLOCK, 1, 1), self.packer.pack(*vals), 0,
+                              _stream.get_current_stream_ptr())
+        res = []
+        for what, ref in self.returns:
+            res.append(outs[ref] if what == 'out' else args[ref] if what == 'arg' else ref)
+        return res[0] if self.single else tuple(res)
+
+
+def build(nodes, pieces, returns, single, args, name):
+    """RowPlan for the recorded function, or None when it does not have the
+    row-wise form (the caller then launches the pieces one by one).
+
+    ``pieces``: the ``_Piece`` objects of ``_fusion_split`` in evaluation order;
+    ``returns``: node order numbers or ('const', value)."""
+    try:
+        return _build(nodes, pieces, returns, single, args, name)
+    except _Unsupported:
+        return None
+
+
+def _build(nodes, pieces, returns, single, args, name):
+    from cupy_amd._core import fusion
+    reduces = [n for n in nodes if n.kind == 'reduce']
+    if not reduces:
+        raise _Unsupported('no reduction')
+    full = tuple(reduces[0].args[0].shape)
+    if len(full) < 1 or internal.prod(full) == 0:
+        raise _Unsupported('empty')
+    n_cols = full[-1]
+    n_rows = internal.prod(full[:-1])
+    kinds = _classify(nodes, full)
+    by_order = {n.order: n for n in nodes}
+
+    # ---- the values every piece starts from --------------------------------------------
+    leaf_value = {}
+    for n in nodes:
+        if n.kind == 'leaf':
+            leaf_value[n.order] = args[n.fn] if isinstance(n.fn, int) else n.fn
+    for n in nodes:
+        if n.kind == 'leaf' and kinds[n.order] != 'uni':
+            a = leaf_value[n.order]
+            if not isinstance(a, ndarray) or not a._c_contiguous:
+                raise _Unsupported('operand that is not C-contiguous')
+    full_leaves = [n for n in nodes if n.kind == 'leaf' and kinds[n.order] == 'full']
+    col_leaves = [n for n in nodes if n.kind == 'leaf' and kinds[n.order] == 'col']
+    if not full_leaves:
+        raise _Unsupported('no full-size operand')
+
+    # ---- geometry ----------------------------------------------------------------------
+    items = [leaf_value[n.order].dtype.itemsize for n in full_leaves + col_leaves]
+    vec = max(1, 16 // max(items))
+    while vec > 1:
+        ok = n_cols % vec == 0
+        for n in full_leaves + col_leaves:
+            a = leaf_value[n.order]
+            ok = ok and _aligned(a.data.ptr, min(16, vec * a.dtype.itemsize))
+        if ok:
+            break
+        vec //= 2
+    def words_for(group):
+        per_lane = (n_cols + group * vec - 1) // (group * vec)
+        return sum(per_lane * vec * max(1, it // 4) for it in items)
+    # a wave per row while the row fits its registers: no barrier, and every
+    # lane keeps many loads in flight; a workgroup per row beyond that
+    group = WAVE if words_for(WAVE) <= _tuning.get('fused_rows_wave_words') else BLOCK
+    per_lane = (n_cols + group * vec - 1) // (group * vec)          # vectors per lane and operand
+    words = words_for(group)
+    if words > _ROW_WORDS_PER_LANE or n_cols < 16:
+        raise _Unsupported('row of %d elements does not fit the registers of a group' % n_cols)
+
+    # ---- trace every piece into device functions -----------------------------------------
+    dtype_of = {}
+    for n in nodes:
+        if n.kind == 'leaf':
+            v = leaf_value[n.order]
+            dtype_of[n.order] = v.dtype if isinstance(v, (ndarray, numpy.generic)) else None
+
+    def stand_in(n):
+        if n.kind == 'leaf':
+            return leaf_value[n.order]
+        source = n.args[0] if n.kind == 'keepdims' else n
+        return ndarray._new_contiguous((1,) * len(n.shape), dtype_of[source.order])
+
+    described = []
+    for p in pieces:
+        desc = fusion.describe(p.func, [stand_in(l) for l in p.leaves], name)
+        if desc['kind'] == 'reduce':
+            (target,) = p.targets
+            dtype_of[target.order] = desc['out_params'][0].dtype
+        else:
+            for t, v in zip(p.targets, desc['out_params']):
+                dtype_of[t.order] = v.dtype
+        described.append(desc)
+    for n in nodes:
+        if n.kind == 'keepdims':
+            dtype_of[n.order] = dtype_of[n.args[0].order]
+
+    # ---- kernel parameters ---------------------------------------------------------------
+    params = []
+    fmt = ['@']
+    in_slots = []
+    cname = {}
+
+    def slot_of(n):
+        return ('arg', n.fn, ) if isinstance(n.fn, int) else ('const', n.fn)
+
+    for n in nodes:
+        if n.kind != 'leaf':
+            continue
+        v = leaf_value[n.order]
+        what, ref = slot_of(n)
+        if isinstance(v, ndarray):
+            t = get_typename(v.dtype)
+            params.append('const %s* __restrict__ _p%d' % (t, n.order))
+            fmt.append('P')
+            vector = kinds[n.order] in ('full', 'col')
+            in_slots.append((what, ref, min(16, vec * v.dtype.itemsize) if vector
+                             else v.dtype.itemsize))
+        else:
+            s = CScalar(v)
+            t = get_typename(s.descr)
+            params.append('const %s _s%d' % (t, n.order))
+            fmt.append(_scalar_struct_code(t))
+            in_slots.append((what, ref, s.descr))
+            cname[n.order] = '_s%d' % n.order
+    out_nodes = []
+    out_returns = []
+    for r in returns:
+        if isinstance(r, tuple):
+            out_returns.append(r)
+            continue
+        n = by_order[r]
+        if n.kind == 'leaf':
+            out_returns.append(slot_of(n) if isinstance(n.fn, int) else ('const', n.fn))
+            continue
+        if not any(n is m for m in out_nodes):
+            out_nodes.append(n)
+        out_returns.append(('out', [m.order for m in out_nodes].index(n.order)))
+    out_specs = []
+    for n in out_nodes:
+        if kinds[n.order] not in ('full', 'row', 'rowk'):
+            raise _Unsupported('result that is neither per element nor per row')
+        t = get_typename(dtype_of[n.order])
+        params.append('%s* __restrict__ _o%d' % (t, n.order))
+        fmt.append('P')
+        out_specs.append((tuple(n.shape), dtype_of[n.order]))
+
+    # ---- source --------------------------------------------------------------------------
+    in_bytes = sum(leaf_value[n.order].nbytes for n in full_leaves)
+    out_bytes = sum(internal.prod(s) * numpy.dtype(d).itemsize for s, d in out_specs)
+    nt_l, nt_s = _tuning.stream_policy('auto', in_bytes, out_bytes)
+    ntl = 'true' if nt_l else 'false'
+    nts = 'true' if nt_s else 'false'
+    idx_t = 'int' if n_rows * n_cols <= 0x7fffffff - (1 << 24) else 'ptrdiff_t'
+    shared = []
+    for d in described:
+        for pre in d['preambles']:
+            if pre and pre not in shared:
+                shared.append(pre)
+    src = ['#include <cupy/carray.cuh>', 'typedef int IndexT;']
+    src.extend(shared)
+    src.append('#define NCOLS %d' % n_cols)
+    src.append('#define GROUP %d' % group)
+    src.append('#define VEC %d' % vec)
+    src.append('#define PER_LANE %d' % per_lane)
+    for k, (p, d) in enumerate(zip(pieces, described)):
+        src.append('namespace piece%d {' % k)
+        if d['kind'] == 'reduce':
+            src.append(d['defs'])
+            src.append('typedef %s reduce_t;' % d['reduce_ctype'])
+            src.append('struct Op { __device__ __forceinline__ reduce_t operator()('
+                       'const reduce_t& a, const reduce_t& b) const { return (%s); } };'
+                       % d['reduce_expr'])
+        else:
+            sig = ['%s v%d' % (get_typename(v.dtype), v.index) for v in d['in_params']]
+            sig += ['%s& v%d' % (get_typename(v.dtype), v.index) for v in d['out_params']]
+            src.append('__device__ __forceinline__ void elementwise(%s) {\n%s\n}' % (
+                ', '.join(sig), d['operation']))
+        src.append('}  // namespace piece%d' % k)
+    params.append('const %s _n_rows' % idx_t)
+    fmt.append('q' if idx_t == 'ptrdiff_t' else 'i')
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, ', '.join(params)))
+    if group == BLOCK:
+        for k, d in enumerate(described):
+            if d['kind'] == 'reduce':
+                src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw%d[%d * sizeof('
+                           'piece%d::reduce_t)];' % (k, BLOCK // WAVE, k))
+                src.append('  piece%d::reduce_t* _sm%d = reinterpret_cast<piece%d::reduce_t*>('
+                           '_sm_raw%d);' % (k, k, k, k))
+    src.append('  const int _lane = threadIdx.x % GROUP;')
+    # values that do not depend on the row: one per column, one for all
+    for n in col_leaves:
+        t = get_typename(leaf_value[n.order].dtype)
+        src.append('  cupy::Vec<%s, VEC> _c%d[PER_LANE];' % (t, n.order))
+        src.append('#pragma unroll')
+        src.append('  for (int _e = 0; _e < PER_LANE; ++_e) {')
+        src.append('    const int _col = (_e * GROUP + _lane) * VEC;')
+        src.append('    _c%d[_e] = cupy::load_vec<%s, VEC, false>(_p%d + (_col < NCOLS ? _col : 0));'
+                   % (n.order, t, n.order))
+        src.append('  }')
+    for n in nodes:
+        if n.kind == 'leaf' and kinds[n.order] == 'uni' and n.order not in cname:
+            t = get_typename(leaf_value[n.order].dtype)
+            src.append('  const %s _u%d = _p%d[0];' % (t, n.order, n.order))
+            cname[n.order] = '_u%d' % n.order
+    src.append('  const %s _rows_per_block = %d / GROUP;' % (idx_t, BLOCK))
+    src.append('  for (%s _row = (%s)blockIdx.x * _rows_per_block + threadIdx.x / GROUP; '
+               '_row < _n_rows; _row += (%s)gridDim.x * _rows_per_block) {' % (idx_t, idx_t, idx_t))
+    # the row, in registers; every load is issued before any value is used
+    for n in full_leaves:
+        t = get_typename(leaf_value[n.order].dtype)
+        src.append('    cupy::Vec<%s, VEC> _f%d[PER_LANE];' % (t, n.order))
+    src.append('#pragma unroll')
+    src.append('    for (int _e = 0; _e < PER_LANE; ++_e) {')
+    src.append('      const int _col = (_e * GROUP + _lane) * VEC;')
+    src.append('      const int _cc = _col < NCOLS ? _col : 0;')
+    for n in full_leaves:
+        t = get_typename(leaf_value[n.order].dtype)
+        src.append('      _f%d[_e] = cupy::load_vec<%s, VEC, %s>(_p%d + (ptrdiff_t)_row * NCOLS + _cc);'
+                   % (n.order, t, ntl, n.order))
+    src.append('    }')
+    for n in nodes:
+        if n.kind == 'leaf' and kinds[n.order] == 'rowk':
+            t = get_typename(leaf_value[n.order].dtype)
+            src.append('    const %s _r%d = _p%d[_row];' % (t, n.order, n.order))
+            cname[n.order] = '_r%d' % n.order
+
+    def operand(n):
+        """Expression of a value inside the element loop (_e, _k) or, for
+        values per row, anywhere in the row loop."""
+        k = kinds[n.order]
+        if n.order in cname:
+            return cname[n.order]
+        if n.kind == 'keepdims':
+            return operand(n.args[0])
+        if k == 'full' and n.kind == 'leaf':
+            return '_f%d[_e].v[_k]' % n.order
+        if k == 'col' and n.kind == 'leaf':
+            return '_c%d[_e].v[_k]' % n.order
+        raise _Unsupported('value %d (%s, %s) is not available here' % (n.order, n.kind, k))
+
+    for k, (p, d) in enumerate(zip(pieces, described)):
+        call_args = [operand(l) for l in p.leaves]
+        if d['kind'] == 'reduce':
+            (target,) = p.targets
+            ident = _cg._identity_decl(d['identity']).replace('_type_reduce', 'piece%d::reduce_t' % k)
+            src.append('    piece%d::reduce_t _a%d = %s;' % (k, k, ident))
+            src.append('#pragma unroll')
+            src.append('    for (int _e = 0; _e < PER_LANE; ++_e) {')
+            src.append('      const int _col = (_e * GROUP + _lane) * VEC;')
+            src.append('#pragma unroll')
+            src.append('      for (int _k = 0; _k < VEC; ++_k) if (_col + _k < NCOLS) {')
+            src.append('        _a%d = piece%d::Op()(_a%d, piece%d::_pre_map(%s));' % (
+                k, k, k, k, ', '.join(call_args)))
+            src.append('      }')
+            src.append('    }')
+            if group == WAVE:
+                src.append('    _a%d = cupy::group_allreduce<64>(_a%d, piece%d::Op());' % (k, k, k))
+            else:
+                src.append('    _a%d = cupy::group_allreduce<64>(_a%d, piece%d::Op());' % (k, k, k))
+                src.append('    if ((threadIdx.x & 63) == 0) _sm%d[threadIdx.x >> 6] = _a%d;' % (k, k))
+                src.append('    __syncthreads();')
+                src.append('    _a%d = _sm%d[0];' % (k, k))
+                src.append('    for (int _w = 1; _w < %d; ++_w) _a%d = piece%d::Op()(_a%d, _sm%d[_w]);'
+                           % (BLOCK // WAVE, k, k, k, k))
+                src.append('    __syncthreads();')
+            t = get_typename(dtype_of[target.order])
+            src.append('    %s _t%d;' % (t, target.order))
+            src.append('    piece%d::_post_map(piece%d::_postmap_cast(_a%d), _t%d);' % (
+                k, k, k, target.order))
+            cname[target.order] = '_t%d' % target.order
+        else:
+            target_kinds = set(kinds[t.order] for t in p.targets)
+            if target_kinds <= {'row', 'rowk'}:
+                if any(kinds[l.order] in ('full', 'col') for l in p.leaves):
+                    raise _Unsupported('a value per row computed from values per element')
+                for t in p.targets:
+                    src.append('    %s _t%d;' % (get_typename(dtype_of[t.order]), t.order))
+                    cname[t.order] = '_t%d' % t.order
+                src.append('    piece%d::elementwise(%s);' % (
+                    k, ', '.join(call_args + [cname[t.order] for t in p.targets])))
+            elif target_kinds == {'full'}:
+                src.append('#pragma unroll')
+                src.append('    for (int _e = 0; _e < PER_LANE; ++_e) {')
+                src.append('      const int _col = (_e * GROUP + _lane) * VEC;')
+                for t in p.targets:
+                    src.append('      cupy::Vec<%s, VEC> _v%d;' % (
+                        get_typename(dtype_of[t.order]), t.order))
+                src.append('#pragma unroll')
+                src.append('      for (int _k = 0; _k < VEC; ++_k) {')
+                src.append('        piece%d::elementwise(%s);' % (
+                    k, ', '.join(call_args + ['_v%d.v[_k]' % t.order for t in p.targets])))
+                src.append('      }')
+                for t in p.targets:
+                    if not any(t is m for m in out_nodes):
+                        raise _Unsupported('elementwise value that is not a result')
+                    src.append('      if (_col < NCOLS) cupy::store_vec<%s, VEC, %s>('
+                               '_o%d + (ptrdiff_t)_row * NCOLS + _col, _v%d);' % (
+                                   get_typename(dtype_of[t.order]), nts, t.order, t.order))
+                src.append('    }')
+            else:
+                raise _Unsupported('results of mixed kinds in one piece')
+    # results held per row
+    for n in out_nodes:
+        if kinds[n.order] in ('row', 'rowk'):
+            src.append('    if (_lane == 0) _o%d[_row] = %s;' % (n.order, operand(n)))
+    src.append('  }')
+    src.append('}')
+    code = '\n'.join(src) + '\n'
+    fn = compiler.compile_with_cache(code, ('-DCUPY_FUSED_ROWS',)).get_function(name)
+    rows_per_block = BLOCK // group
+    cus = _device.get_compute_units(_device.get_device_id())
+    grid = max(1, min((n_rows + rows_per_block - 1) // rows_per_block, cus * 16))
+    return RowPlan(fn, _make_packer(fmt), (grid, 1, 1), n_rows, in_slots, out_specs,
+                   out_returns, single)

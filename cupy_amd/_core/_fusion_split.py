@@ -220,7 +220,8 @@ class _Tracer:
         if len(set(axes)) != len(axes):
             raise ValueError('duplicate value in \'axis\'')
         shape = tuple(s for i, s in enumerate(src.shape) if i not in axes)
-        node = self._node('reduce', func, (src,), {'axis': axis, 'dtype': dtype}, shape)
+        node = self._node('reduce', func, (src,),
+                          {'axis': axis, 'dtype': dtype, 'axes': axes}, shape)
         if keepdims:
             kept = tuple(1 if i in axes else s for i, s in enumerate(src.shape))
             node = self._node('keepdims', None, (node,), {'axes': axes}, kept)
@@ -229,7 +230,7 @@ class _Tracer:
 
 class _Piece:
     """One kernel of the plan: ``targets`` computed from ``leaves``."""
-    __slots__ = ('fused', 'leaves', 'targets')
+    __slots__ = ('fused', 'func', 'leaves', 'targets')
 
     def __init__(self, targets, leaves, stored, name):
         from cupy_amd._core import fusion
@@ -258,6 +259,7 @@ class _Piece:
             return outs[0] if len(outs) == 1 else outs
 
         piece.__name__ = name
+        self.func = piece
         self.fused = fusion.Fusion(piece, name, split=False)
 
 
@@ -383,4 +385,15 @@ def trace(func, args, name):
         n_kernels += 1
     const_leaves = [(n.order, n.fn) for n in nodes
                     if n.kind == 'leaf' and isinstance(n.fn, ndarray)]
-    return Plan(steps, len(nodes), arg_leaves, const_leaves, returns, single)
+    # all reductions along the rows of one matrix, rows short enough for the
+    # registers of a workgroup: one kernel that reads the matrix once
+    from cupy_amd._core import _fusion_rows
+    pieces = [st[1] for st in steps if st[0] == 'kernel']
+    sequence = Plan(steps, len(nodes), arg_leaves, const_leaves, returns, single)
+    row_plan = _fusion_rows.build(nodes, pieces, returns, single, args, name)
+    if row_plan is not None:
+        # for calls whose arrays are laid out differently from those the
+        # kernel was built for
+        row_plan.fallback = sequence
+        return row_plan
+    return sequence

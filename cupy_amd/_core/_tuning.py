@@ -35,6 +35,8 @@ _params = {
     'cols_unroll': 1,
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
+    # fused row-wise functions: words per lane up to which a wave takes a whole row
+    'fused_rows_wave_words': 64,
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
 }

@@ -507,8 +507,13 @@ class _FusionHistory:
             python_var = _FusionVarScalar(cuda_var, -1, False, is_weak)
         return cuda_var, python_var
 
-    def get_fusion(self, func, args, name):
-        """Runs ``func`` on proxies and returns (kernel, kwargs for its call)."""
+    def get_fusion(self, func, args, name, describe_only=False):
+        """Runs ``func`` on proxies and returns (kernel, kwargs for its call).
+        With ``describe_only`` no kernel object is made: the return value is a
+        dict of the generated pieces (parameter variables, the body of an
+        elementwise function, or the device functions, combine expression,
+        accumulator type and identity of a map-reduce function) for emitters
+        that compose several traced functions into one kernel."""
         self.ndim = max(a.ndim for a in args if isinstance(a, ndarray))
         in_params = []
         function_args = []
@@ -549,6 +554,10 @@ class _FusionHistory:
         if self.reduce_op is None:
             operation += ' '.join('{} = {};'.format(t, s)
                                   for s, t in zip(out_cvars, out_params))
+            if describe_only:
+                return dict(kind='elementwise', in_params=in_params, out_params=out_params,
+                            operation=operation, preambles=list(self.preamble_set),
+                            return_tuple=return_tuple)
             kernel = _kernel.ElementwiseKernel(
                 in_params_code, out_params_code, operation, preamble=preamble,
                 return_tuple=return_tuple, no_return=no_return, name=name)
@@ -568,6 +577,8 @@ class _FusionHistory:
                                  for s, t in zip(out_cvars, out_params))
 
         ret = self.premap_ret
+        shared_preambles = list(self.preamble_set)
+        defs_start = len(preamble)
         # the reduction's own element map (identity for sum/prod/min/max)
         preamble += 'typedef %s type_in0_raw;\n' % premap_ctype
         preamble += 'typedef %s type_out0_raw;\n' % postmap_ctype
@@ -601,6 +612,14 @@ __device__ __forceinline__ void _post_map(%s in, %s) {
                       for v in out_params),
             in_ctype, self.postmap_param.index, postmap_code)
 
+        if describe_only:
+            return dict(kind='reduce', in_params=in_params, out_params=out_params,
+                        preambles=shared_preambles, defs=preamble[defs_start:],
+                        reduce_expr=reduce_expr,
+                        reduce_ctype=(reduce_ctype if reduce_ctype != 'type_out0_raw'
+                                      else postmap_ctype),
+                        identity=self.reduce_identity, kwargs=self.reduce_kwargs,
+                        return_tuple=return_tuple)
         kernel = _reduction.ReductionKernel(
             in_params_code, out_params_code,
             '_pre_map({})'.format(', '.join(repr(p) for p in in_params)),
@@ -742,6 +761,21 @@ class Fusion:
         self._memo = {}
         self._fast = {}
         self._plans = {}
+
+
+def describe(func, args, name):
+    """Traces ``func`` on stand-ins of ``args`` with the single-kernel tracer
+    and returns the generated pieces instead of a kernel (see
+    ``_FusionHistory.get_fusion``)."""
+    history = _FusionHistory()
+    saved = (getattr(_thread_local, 'history', None),
+             getattr(_thread_local, 'is_old_fusing', False))
+    _thread_local.history = history
+    _thread_local.is_old_fusing = True
+    try:
+        return history.get_fusion(func, args, name, describe_only=True)
+    finally:
+        _thread_local.history, _thread_local.is_old_fusing = saved
 
 
 def fuse(*args, **kwargs):

@@ -22,38 +22,67 @@ def arrays(*shapes, dtype=np.float32):
     return [cp.asarray(np.ones(s, dtype)) for s in shapes]
 
 
-def test_softmax_is_three_kernels_with_no_full_size_temporary():
-    @cp.fuse()
-    def softmax(x):
-        e = cp.exp(x - cp.amax(x, axis=1, keepdims=True))
-        return e / cp.sum(e, axis=1, keepdims=True)
+def _softmax(x):
+    e = cp.exp(x - cp.amax(x, axis=1, keepdims=True))
+    return e / cp.sum(e, axis=1, keepdims=True)
 
-    x, = arrays((70, 33))
-    pool = cp.get_default_memory_pool()
+
+def test_softmax_over_long_rows_is_three_kernels_with_no_full_size_temporary():
+    softmax = cp.fuse(kernel_name='softmax')(_softmax)
+    x, = arrays((4, 100000))                  # a row does not fit the registers of a workgroup
     out, names = kernels_of(softmax, x)
-    assert names == ['softmax_part0', 'softmax_part1', 'softmax_part2']
-    assert out.shape == (70, 33) and out.dtype == np.float32
-    # the eager evaluation of the same function launches five kernels
-    _, eager = kernels_of(softmax.func, x)
-    assert len(eager) == 5
+    # (few long rows: each map-reduce kernel is followed by its combine kernel)
+    assert [n for n in names if not n.endswith('_combine')] == [
+        'softmax_part0', 'softmax_part1', 'softmax_part2']
+    assert out.shape == (4, 100000) and out.dtype == np.float32
+    # the eager evaluation of the same function launches five kernels (and two
+    # full-size temporaries)
+    _, eager = kernels_of(_softmax, x)
+    assert len([n for n in eager if not n.endswith('_combine')]) == 5
     # second call: the plan is remembered, same three launches
     _, again = kernels_of(softmax, x)
     assert again == names
-    assert pool is not None
+
+
+@pytest.mark.parametrize('shape', [(70, 33), (64, 4096), (3, 5, 1000), (1000,)])
+def test_reductions_along_short_rows_become_one_kernel(shape):
+    def standardise(x, eps):
+        m = cp.sum(x, axis=-1, keepdims=True) / x.shape[-1]
+        d = x - m
+        v = cp.sum(d * d, axis=-1, keepdims=True) / x.shape[-1]
+        return d / cp.sqrt(v + eps), m
+
+    f = cp.fuse(kernel_name='standardise')(standardise)
+    x, = arrays(shape)
+    (out, mean), names = kernels_of(f, x, 1e-5)
+    assert names == ['standardise']            # the matrix is read once
+    assert out.shape == shape and mean.shape == shape[:-1] + (1,)
+    assert out.dtype == mean.dtype == np.float32
+    # a view that is not contiguous goes through the kernel sequence instead
+    if len(shape) == 2:
+        wide, = arrays((shape[0], 2 * shape[1]))
+        (out2, _), names2 = kernels_of(f, wide[:, ::2], 1e-5)
+        assert out2.shape == shape and all('_part' in n for n in names2)
 
 
 def test_elementwise_work_feeding_two_reductions_is_fused_into_each():
-    @cp.fuse()
     def ratio(x, y, s):
-        return cp.sum((x - y) ** 2, axis=1) / cp.sum(x * x * s, axis=1), x + y
+        return cp.sum((x - y) ** 2, axis=0) / cp.sum(x * x * s, axis=0), x + y
 
+    f = cp.fuse(kernel_name='ratio')(ratio)
     x, y = arrays((40, 50), (40, 50))
-    (r, t), names = kernels_of(ratio, x, y, 2.0)
-    assert r.shape == (40,) and t.shape == (40, 50)
+    (r, t), names = kernels_of(f, x, y, 2.0)
+    assert r.shape == (50,) and t.shape == (40, 50)
     # two map-reduce kernels, then one elementwise kernel per result shape
     assert names == ['ratio_part0', 'ratio_part1', 'ratio_part2', 'ratio_part3']
-    _, eager = kernels_of(ratio.func, x, y, 2.0)
+    _, eager = kernels_of(ratio, x, y, 2.0)
     assert len(eager) > len(names)
+    # the same along the rows: everything in one kernel, both results written by it
+    def ratio_rows(x, y, s):
+        return cp.sum((x - y) ** 2, axis=1) / cp.sum(x * x * s, axis=1), x + y
+    g = cp.fuse(kernel_name='ratio_rows')(ratio_rows)
+    (r, t), names = kernels_of(g, x, y, 2.0)
+    assert names == ['ratio_rows'] and r.shape == (40,) and t.shape == (40, 50)
 
 
 def test_shapes_are_available_while_recording_and_key_the_plan():
