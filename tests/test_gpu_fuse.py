@@ -363,3 +363,30 @@ def test_row_wise_functions_in_one_kernel_match_numpy(shape):
         shifted = flat[1:].reshape(shape)           # same shape, data 2 bytes off alignment
         got = centre(shifted, cp.asarray(w))
         np.testing.assert_allclose(got.get(), want, rtol=1e-3, atol=1e-3)
+
+
+def test_row_kernel_follows_scalars_types_and_captured_arrays():
+    rng = np.random.default_rng(46)
+    shift = cp.asarray(rng.standard_normal(96).astype(np.float32))      # captured by the function
+
+    @cp.fuse()
+    def f(x, y, eps, k):
+        m = cp.sum(x * y, axis=1, keepdims=True) / k
+        above = (x + shift) > m
+        return cp.where(above, x, m) * eps, above, cp.sum(above, axis=1)
+
+    hshift = shift.get()
+    for trial, (eps, k) in enumerate(((0.5, 96), (2.0, 7), (np.float32(3), np.int64(5)))):
+        hx = rng.integers(-5, 5, (50, 96)).astype(np.int32)
+        hy = rng.standard_normal((50, 96)).astype(np.float16)
+        got = f(cp.asarray(hx), cp.asarray(hy), eps, k)
+        m = np.sum(hx * hy, axis=1, keepdims=True) / k
+        above = (hx + hshift) > m
+        want = (np.where(above, hx, m) * eps, above, np.sum(above, axis=1))
+        for g, w in zip(got, want):
+            assert g.dtype == w.dtype and g.shape == w.shape, (trial, g.dtype, w.dtype)
+            if w.dtype.kind == 'f':
+                np.testing.assert_allclose(g.get(), w, rtol=2e-3, atol=2e-3)
+            else:
+                # a comparison may flip where x + shift and the mean agree to rounding
+                assert (g.get() != w).mean() < 0.01
