@@ -261,6 +261,160 @@ COLS_KERNEL(cupy_scan_cols_seeded, 2)
            ragged=1 if ragged else 0)
 
 
+def _emit_lanes(in_t, out_t, op, skip_nan, vec, trips, idx64, lstride, stream):
+    """Scan along the middle axis of (outer, n, inner) when ``inner`` is a few
+    vectors wide: a row of ``inner = lstride * vec`` elements sits in
+    ``lstride`` adjacent lanes, a wave holds ``64 / lstride`` consecutive rows
+    per load -- contiguous in memory, so accesses stay coalesced however narrow
+    the array is -- and the scan runs across the lanes in steps of ``lstride``
+    (Kogge-Stone over rows; the ``vec`` columns of a lane never mix)."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define LSTRIDE %(lstride)d
+#define INNER (LSTRIDE * VEC)
+#define TRIP_ROWS (64 / LSTRIDE)
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+
+// mode 0: scan, no carry-in.  mode 1: write only the chunk totals (one per
+// column).  mode 2: scan seeded with the inclusive scan of the totals.
+template <int kMode>
+__device__ __forceinline__ void scan_lanes_impl(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, _acc_t* __restrict__ totals,
+    const _idx_t n_outer, const _idx_t n, const _idx_t n_chunks, const _idx_t chunk_rows) {
+  const int lane = threadIdx.x %% 64;
+  const int lrow = lane / LSTRIDE;
+  const int lcol = (lane %% LSTRIDE) * VEC;
+  const _idx_t n_work = n_outer * n_chunks;
+  const _idx_t wave_step = (_idx_t)gridDim.x * (%(block)d / 64);
+  for (_idx_t w = (_idx_t)blockIdx.x * (%(block)d / 64) + threadIdx.x / 64; w < n_work;
+       w += wave_step) {
+    const _idx_t o = w / n_chunks;
+    const _idx_t chunk = w - o * n_chunks;
+    const _idx_t r0 = chunk * chunk_rows;
+    const _idx_t r1 = (r0 + chunk_rows < n) ? (r0 + chunk_rows) : n;
+    const _in_t* src = in + (ptrdiff_t)o * n * INNER + lcol;
+    _out_t* dst = out + (ptrdiff_t)o * n * INNER + lcol;
+    _acc_t carry[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) carry[k] = SCAN_IDENTITY;
+    if (kMode == 2 && chunk > 0) {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        carry[k] = totals[((ptrdiff_t)o * n_chunks + chunk - 1) * INNER + lcol + k];
+    }
+    for (_idx_t rb = r0; rb < r1; rb += TRIP_ROWS * TRIPS) {
+      // every load of the round is requested before the first value is used; a
+      // row past the end of the chunk is read from the chunk's first row instead
+      cupy::Vec<_in_t, VEC> raw[TRIPS];
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const _idx_t r = rb + t * TRIP_ROWS + lrow;
+        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + (ptrdiff_t)(r < r1 ? r : r0) * INNER);
+      }
+      _acc_t v[TRIPS][VEC];
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const _idx_t r = rb + t * TRIP_ROWS + lrow;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          v[t][k] = (r < r1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+      }
+      if (kMode == 1) {
+        // only the column totals of the chunk are wanted: every lane adds up
+        // its own rows; the lanes are combined once, after the last round
+#pragma unroll
+        for (int t = 0; t < TRIPS; ++t) {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) carry[k] = SCAN_OP(carry[k], v[t][k]);
+        }
+        continue;
+      }
+      // inclusive scan over the rows of each trip: lanes LSTRIDE apart hold the
+      // same columns of neighbouring rows
+#pragma unroll
+      for (int d = LSTRIDE; d < 64; d <<= 1) {
+#pragma unroll
+        for (int t = 0; t < TRIPS; ++t) {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) {
+            const _acc_t up = cupy::shfl_up<64>(v[t][k], d);
+            v[t][k] = (lane >= d) ? SCAN_OP(up, v[t][k]) : v[t][k];
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const _idx_t r = rb + t * TRIP_ROWS + lrow;
+        cupy::Vec<_out_t, VEC> res;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          // the trip's total of this column sits in the last row of the wave
+          const _acc_t total = cupy::shfl_idx<64>(v[t][k], 64 - LSTRIDE + lane %% LSTRIDE);
+          res.v[k] = static_cast<_out_t>(SCAN_OP(carry[k], v[t][k]));
+          carry[k] = SCAN_OP(carry[k], total);
+        }
+        if (kMode != 1 && r < r1)
+          cupy::store_vec<_out_t, VEC, NT_STORE>(dst + (ptrdiff_t)r * INNER, res);
+      }
+    }
+    if (kMode == 1) {
+#pragma unroll
+      for (int m = LSTRIDE; m < 64; m <<= 1) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) carry[k] = SCAN_OP(carry[k], cupy::shfl_xor(carry[k], m));
+      }
+      if (lrow == 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          totals[((ptrdiff_t)o * n_chunks + chunk) * INNER + lcol + k] = carry[k];
+      }
+    }
+  }
+}
+
+#define LANES_KERNEL(NAME, MODE) \\
+extern "C" __global__ void __launch_bounds__(%(block)d) NAME( \\
+    const _in_t* in, _out_t* out, _acc_t* totals, const _idx_t n_outer, const _idx_t n, \\
+    const _idx_t n_chunks, const _idx_t chunk_rows) { \\
+  scan_lanes_impl<MODE>(in, out, totals, n_outer, n, n_chunks, chunk_rows); }
+LANES_KERNEL(cupy_scan_lanes, 0)
+LANES_KERNEL(cupy_scan_lanes_totals, 1)
+LANES_KERNEL(cupy_scan_lanes_seeded, 2)
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           lstride=lstride, ntl='true' if stream[0] else 'false',
+           nts='true' if stream[1] else 'false')
+
+
+def _module_lanes(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, lstride, stream):
+    key = ('lanes', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
+           trips, idx64, lstride, stream)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_lanes(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                          vec, trips, idx64, lstride, stream)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
 def _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group=64,
             stream=(True, False), ragged=True):
     key = (_device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
@@ -277,6 +431,22 @@ def _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group=64,
 
 def _acc_dtype(out_dtype):
     return numpy.dtype('float32') if out_dtype == numpy.float16 else out_dtype
+
+
+def _lanes_geometry(src, dst, inner, item):
+    """(vec, lanes per row) for the lane-interleaved kernel, or None when the
+    inner extent is not a small power-of-two number of vectors."""
+    if inner < 2:
+        return None
+    vec = max(1, 16 // item)
+    while vec >= 1:
+        if (inner % vec == 0 and src.data.ptr % (vec * src.dtype.itemsize) == 0
+                and dst.data.ptr % (vec * dst.dtype.itemsize) == 0):
+            lstride = inner // vec
+            if lstride <= 16 and lstride & (lstride - 1) == 0:
+                return vec, lstride
+        vec //= 2
+    return None
 
 
 def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_chunk=True):
@@ -336,6 +506,34 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                 (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
         prefix = 'cupy_scan_rows'
         totals_shape = (outer, n_chunks, 1)
+        middle_round = _WAVE * 4 * 4          # elements one wave takes per round
+    elif _lanes_geometry(src, dst, inner, item) is not None:
+        vec, lstride = _lanes_geometry(src, dst, inner, item)
+        trips = 4
+        trip_rows = _WAVE // lstride
+        per_wave = trip_rows * trips
+        want = cus * _tuning.get('scan_waves_per_cu')
+        n_chunks = 1
+        if may_chunk and outer < want and n > 2 * per_wave:
+            n_chunks = min((want + outer - 1) // outer, (n + per_wave - 1) // per_wave)
+        chunk_len = (n + n_chunks - 1) // n_chunks
+        chunk_len = (chunk_len + per_wave - 1) // per_wave * per_wave
+        n_chunks = (n + chunk_len - 1) // chunk_len
+        mod = _module_lanes(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, lstride,
+                            stream)
+        waves = outer * n_chunks
+        per_block = _BLOCK // _WAVE
+        grid = max(1, min((waves + per_block - 1) // per_block, cus * 32))
+        fmt = '@PPP' + ic * 4
+
+        def launch(name, totals_ptr):
+            blob = struct.pack(fmt, src.data.ptr, dst.data.ptr, totals_ptr, outer, n,
+                               n_chunks, chunk_len)
+            mod.get_function(name).launch_packed(
+                (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+        prefix = 'cupy_scan_lanes'
+        totals_shape = (outer, n_chunks, inner)
+        middle_round = per_wave
     else:
         vec = max(1, 16 // item)
         while vec > 1 and (src.data.ptr % (vec * in_dtype.itemsize)
@@ -362,15 +560,16 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                 (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
         prefix = 'cupy_scan_cols'
         totals_shape = (outer, n_chunks, inner)
+        middle_round = 16                     # rows a lane takes per round
     if n_chunks == 1:
         launch(prefix, 0)
         return
     totals = ndarray._new_contiguous(totals_shape, _acc_dtype(out_dtype))
     launch(prefix + '_totals', totals.data.ptr)
-    # the totals are few: one more level of chunks would cost more launches
-    # than it saves
+    # The scan of the totals is one dependent chain per row (or column): when
+    # it would take many rounds it is cut into chunks in its turn.
     _scan_contiguous(totals, totals, totals_shape[0], n_chunks, totals_shape[2], op, False,
-                     stream_ptr, may_chunk=totals.size > (1 << 20))
+                     stream_ptr, may_chunk=n_chunks > 8 * middle_round)
     launch(prefix + '_seeded', totals.data.ptr)
 
 

@@ -257,3 +257,48 @@ def test_one_pass_variance_is_stable_and_matches_numpy(dtype):
     np.testing.assert_allclose(out.get(), h.var(axis=0), rtol=20 * rtol)
     np.testing.assert_allclose(cp.asarray(h).std(axis=1, ddof=1).get(), h.std(axis=1, ddof=1),
                                rtol=20 * rtol)
+
+
+@pytest.mark.parametrize('shape,axis', [((1000, 8), 0), ((7, 1000, 2), 1), ((5000, 64), 0),
+                                        ((100001, 16), 0), ((3, 70000, 4), 1), ((50, 32), 0),
+                                        ((2, 3, 999, 8), 2)])
+@pytest.mark.parametrize('dtype', ['float32', 'float64', 'int32', 'float16'])
+def test_scans_along_an_axis_with_a_narrow_tail(shape, axis, dtype):
+    """The axes after the scanned one span a few vectors only: rows sit in
+    adjacent lanes and the scan runs across lanes (contiguous accesses), in one
+    launch or split into chunks with carried totals."""
+    rng = np.random.default_rng(93)
+    if dtype == 'int32':
+        h = rng.integers(-9, 10, shape).astype(dtype)
+    else:
+        h = rng.standard_normal(shape).astype(dtype)
+    d = cp.asarray(h)
+    got = cp.cumsum(d, axis=axis)
+    want = np.cumsum(h, axis=axis)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    if dtype == 'int32':
+        assert np.array_equal(got.get(), want)
+    else:
+        tol = {'float16': 2e-2, 'float32': 1e-5, 'float64': 1e-12}[dtype]
+        scale = np.cumsum(np.abs(h.astype(np.float64)), axis=axis)
+        assert (np.abs(got.get().astype(np.float64) - np.cumsum(h.astype(np.float64), axis=axis))
+                <= tol * scale + tol).all()
+    if dtype in ('float32', 'int32') and h.shape[axis] <= 1000:
+        small = np.sign(h).astype(dtype)
+        small[small == 0] = 1
+        assert np.array_equal(cp.cumprod(cp.asarray(small), axis=axis).get(),
+                              np.cumprod(small, axis=axis))
+    if dtype == 'float32':
+        hn = h.copy()
+        hn[..., ::3] = np.nan
+        got = cp.nancumsum(cp.asarray(hn), axis=axis).get()
+        want = np.nancumsum(hn.astype(np.float64), axis=axis)
+        assert (np.abs(got - want) <= 1e-5 * np.cumsum(np.abs(np.nan_to_num(hn)), axis=axis) + 1e-5).all()
+    # a view whose data is not aligned to the vector width takes another geometry
+    flat = cp.asarray(np.concatenate([np.zeros(1, dtype), h.ravel()]))
+    view = flat[1:].reshape(shape)
+    got = cp.cumsum(view, axis=axis).get().astype(np.float64)
+    want = np.cumsum(h.astype(np.float64), axis=axis)
+    tol = {'float16': 2e-2, 'float32': 1e-5, 'float64': 1e-12, 'int32': 0}[dtype]
+    scale = np.cumsum(np.abs(h.astype(np.float64)), axis=axis)
+    assert (np.abs(got - want) <= tol * scale + tol).all()
