@@ -402,12 +402,17 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
 
 def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
-              partial_in=False, partial_out=False, stream_hint=False, unroll=4):
+              partial_in=False, partial_out=False, stream_hint=False, unroll=4,
+              solo=False):
     """Output-axis-contiguous kernel.  Thread layout: ``tx`` threads across
     the output axis (each owning ``vec`` adjacent outputs) times 256/tx slices
     of the reduce axis; gridDim.y further slices.  ``partial_in``: the single
     input holds ``_type_reduce`` values that are combined as they are."""
-    assert tx in (1, 2, 4, 8, 16, 32, 64)
+    # ``solo``: every thread owns its columns for the whole reduce axis (a
+    # handful of rows): nothing to combine across lanes or waves
+    if solo:
+        tx = BLOCK
+    assert tx in (1, 2, 4, 8, 16, 32, 64) or solo
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     nt = 'true' if stream_hint else 'false'
     ins = [a for a in args if a.kind == 'in']
@@ -418,9 +423,10 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         BLOCK, name, params))
     src.append(_SIZE_INDEXERS)
-    src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (
-        waves * tx * vec))
-    src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
+    if not solo:
+        src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (
+            waves * tx * vec))
+        src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
     src.append('  const int _tx = threadIdx.x %% %d;' % tx)
     src.append('  const int _ty = threadIdx.x / %d;' % tx)
     # column blocks beyond the capacity of grid.x continue along grid.z
@@ -524,6 +530,17 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('      }')
     src.append('    }')
     src.append('  }')
+    if solo:
+        src.append('  if (_c < _n_out) {')
+        src.append('#pragma unroll')
+        src.append('    for (int _k = 0; _k < %d; ++_k) if (_c + _k < _n_out) {' % vec)
+        src.append('      _type_reduce _s = _acc[_k];')
+        src.append('      const %s _i = _c + _k;' % idx_t)
+        src.extend(_finish(args, partial_out, '      '))
+        src.append('    }')
+        src.append('  }')
+        src.append('}')
+        return '\n'.join(src) + '\n'
     # combine the row-slices held by the lanes of one wave, then the waves
     if tx < WAVE:
         src.append('#pragma unroll')

@@ -404,7 +404,10 @@ class _AbstractReductionKernel:
                            typedefs, device_id, stream_ptr, rec, partials_ref, in_total):
         """Second pass: combine ``partials[s][i]`` over s, then POST_MAP."""
         preamble, _ = self._get_preamble_options()
-        tx = max(1, min(64, internal.clp2(n_out)))
+        # lanes across the outputs, the rest of the workgroup down the partials:
+        # with many partials per output few lanes go across, so that no lane
+        # walks a long dependent chain of (cache-resident) loads
+        tx = max(1, min(64, internal.clp2(n_out), internal.flp2(max(1, 4096 // n_split))))
         rargs = [_cg.RArg('in', '_partial_in', '_type_reduce')]
         rargs += [r for r in self._rargs(in_args, out_args) if r.kind in ('scalar', 'out')]
         idx64 = n_split * n_out > _INT32_MAX
@@ -495,7 +498,8 @@ class _AbstractReductionKernel:
             per_trip = sum(vec * a.dtype.itemsize for a, s_o in zip(ins, so_in)
                            if not (s_o == 0 and n_out > 1))
             budget = _tuning.get('rows_lane_bytes')
-            while (trips * 2 <= _tuning.get('rows_trips') and group >= 2
+            min_group = max(1, _tuning.get('rows_min_group_bytes') // (vec * max_item))
+            while (trips * 2 <= _tuning.get('rows_trips') and group >= 2 * min_group
                    and per_trip * trips * 2 <= budget):
                 trips *= 2
                 group //= 2
@@ -584,6 +588,10 @@ class _AbstractReductionKernel:
                 break
             vec //= 2
         tx = max(1, min(64, internal.clp2((n_out + vec - 1) // vec)))
+        # a handful of rows and plenty of columns: a thread per column vector
+        solo = n_red <= 8 and n_out >= cus * _cg.BLOCK * vec
+        if solo:
+            tx = _cg.BLOCK
         ty = _cg.BLOCK // tx
         gx = (n_out + tx * vec - 1) // (tx * vec)
         # the kernel does not loop over column blocks: beyond what grid.x may
@@ -602,14 +610,14 @@ class _AbstractReductionKernel:
             _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
-               stream_hint, _tuning.signature())
+               stream_hint, solo, _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
                 idx64=idx64, partial_out=partial,
-                stream_hint=stream_hint, unroll=_tuning.get('cols_unroll'))
+                stream_hint=stream_hint, unroll=_tuning.get('cols_unroll'), solo=solo)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)

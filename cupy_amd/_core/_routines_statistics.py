@@ -168,25 +168,59 @@ template <typename T> __device__ __forceinline__ min_max_st<T> my_nanmax(
 _int_sigs = ('?->?', 'b->b', 'B->B', 'h->h', 'H->H', 'i->i', 'I->I', 'l->l',
              'L->L', 'q->q', 'Q->Q')
 
+# min / max keep a bare value (arg-reductions need the index beside it): the
+# state starts from the type's extreme, which any element replaces, so that
+# lanes without elements drop out of the combine.  NaN wins for floats.
+_extremum_preamble = '''
+template <typename T> struct _mm_is_float { static const bool value = false; };
+template <> struct _mm_is_float<float> { static const bool value = true; };
+template <> struct _mm_is_float<double> { static const bool value = true; };
+template <> struct _mm_is_float<float16> { static const bool value = true; };
+template <typename T> __device__ __forceinline__ T _mm_extreme(bool lowest) {
+  if (_mm_is_float<T>::value) return lowest ? T(-CUDART_INF_F) : T(CUDART_INF_F);
+  if (cupy::is_same<T, bool>::value) return T(!lowest);
+  if (T(-1) < T(0)) {
+    const unsigned long long top = 1ull << (8 * sizeof(T) - 1);
+    return static_cast<T>(lowest ? top : ~top);
+  }
+  return lowest ? T(0) : static_cast<T>(~0ull);
+}
+template <typename T, bool kMax>
+struct mm_val {
+  T v;
+  __device__ __forceinline__ mm_val() : v(_mm_extreme<T>(kMax)) {}
+  __device__ __forceinline__ explicit mm_val(T x) : v(x) {}
+};
+template <bool kNan, typename T, bool kMax>
+__device__ __forceinline__ mm_val<T, kMax> mm_pick(const mm_val<T, kMax>& a,
+                                                   const mm_val<T, kMax>& b) {
+  bool take_b = kMax ? (b.v > a.v) : (b.v < a.v);
+  if (kNan) take_b = (take_b | (b.v != b.v)) & !(a.v != a.v);
+  mm_val<T, kMax> r;
+  r.v = take_b ? b.v : a.v;
+  return r;
+}
+'''
+
 _amin = create_reduction_func(
     'cupy_min',
     _int_sigs + (
-        ('e->e', (None, 'my_min_float(a, b)', None, None)),
-        ('f->f', (None, 'my_min_float(a, b)', None, None)),
-        ('d->d', (None, 'my_min_float(a, b)', None, None))),
-    ('min_max_st<type_in0_raw>(in0)', 'my_min(a, b)', 'out0 = a.value',
-     'min_max_st<type_in0_raw>'),
-    None, _min_max_preamble)
+        ('e->e', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('f->f', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('d->d', (None, 'mm_pick<true>(a, b)', None, None))),
+    ('mm_val<type_in0_raw, false>(in0)', 'mm_pick<false>(a, b)', 'out0 = a.v',
+     'mm_val<type_in0_raw, false>'),
+    None, _extremum_preamble)
 
 _amax = create_reduction_func(
     'cupy_max',
     _int_sigs + (
-        ('e->e', (None, 'my_max_float(a, b)', None, None)),
-        ('f->f', (None, 'my_max_float(a, b)', None, None)),
-        ('d->d', (None, 'my_max_float(a, b)', None, None))),
-    ('min_max_st<type_in0_raw>(in0)', 'my_max(a, b)', 'out0 = a.value',
-     'min_max_st<type_in0_raw>'),
-    None, _min_max_preamble)
+        ('e->e', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('f->f', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('d->d', (None, 'mm_pick<true>(a, b)', None, None))),
+    ('mm_val<type_in0_raw, true>(in0)', 'mm_pick<false>(a, b)', 'out0 = a.v',
+     'mm_val<type_in0_raw, true>'),
+    None, _extremum_preamble)
 
 _arg_sigs = tuple('{}->{}'.format(d, r) for r in 'qlihb' for d in '?bBhHiIlLqQ') + (
     'e->q', 'f->q', 'd->q')

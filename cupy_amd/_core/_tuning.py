@@ -29,6 +29,7 @@ _params = {
     'rows_block_mode_bytes': 32768,   # row length from which a workgroup owns a row
     'rows_batch': 2,            # short rows handled per lane group at a time
     'rows_trips': 4,            # ... with up to this many vector loads per lane and row
+    'rows_min_group_bytes': 128,  # ... while the lanes of a row still cover this much per load
     'rows_lane_bytes': 128,     # ... and at most this many bytes in flight per lane
     'rows_group_rows_per_lane': 64,   # grid cap for sub-wave groups: CUs * this workgroups
     'cols_stream': True,

@@ -129,6 +129,18 @@ def test_axis_reductions_and_scans_with_rows_beyond_2_to_30():
     assert bool(check2(idx).all().get())
 
 
+def test_column_reduction_whose_blocks_continue_along_grid_z():
+    m = 2 ** 30 + 1                                   # more column blocks than grid.x holds
+    a = _fill_mod100_i8(size=9 * m).reshape(9, m)
+    colsum = a.sum(axis=0)
+    check = cp.ElementwiseKernel(
+        'int64 s', 'bool ok',
+        'const long long m = 1073741825LL; long long w = 0;'
+        'for (long long k = 0; k < 9; ++k) w += (k * m + i) % 100;'
+        'ok = s == w', 'is_colsum9_mod100')
+    assert bool(check(colsum).all().get())
+
+
 def test_broadcast_input_of_2_to_31_elements():
     base = _fill_mod100_i8(size=2048 * 1024).reshape(2048, 1, 1024)
     a = cp.broadcast_to(base, (2048, 1024, 1024))

@@ -27,7 +27,8 @@ CASES = {
     'rows_few': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=1),
     'rows_many': lambda: cp.empty((2 ** 25, 64), np.int8).sum(axis=1),
     'rows_very_many': lambda: cp.empty((2 ** 29, 4), np.int8).sum(axis=1),
-    'cols_wide': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=0),
+    'cols_wide': lambda: cp.empty((9, 2 ** 30 + 1), np.int8).sum(axis=0),
+    'cols_wide_few_rows': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=0),
     'cols_split': lambda: cp.empty((2 ** 16, 2 ** 16), np.int8).sum(axis=0),
     'tiled': lambda: cp.empty((2 ** 17, 2 ** 16), np.int8).T * np.int8(2),
     'generic': lambda: cp.empty((70, 2 ** 13, 2 ** 13), np.int8)[::2, :, ::2].sum(axis=1),
