@@ -19,12 +19,16 @@ module has three kernels, chosen by the host from the canonical 2-d form
              matrix).  Threads own ``V`` adjacent output columns and walk down
              the reduce axis, TY row-slices per workgroup and grid.y slices per
              launch; slices are combined through cross-lane exchanges, LDS and,
-             across workgroups, a partial-result buffer.
+             across workgroups, a partial-result buffer.  The same kernel
+             takes a batch of such problems (reduction over a middle axis:
+             ``in[b, j, c]`` to ``out[b, c]``).
 ``generic``  any strides: CIndexer addressing, same thread layout as ``cols``.
 
 Partial results are combined by a second ``cols`` launch that reads
 ``_type_reduce`` values (``partial_in``) -- deterministic, no atomics.
 """
+import re
+
 BLOCK = 256
 WAVE = 64
 
@@ -403,15 +407,26 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
 def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
               partial_in=False, partial_out=False, stream_hint=False, unroll=4,
-              solo=False):
+              solo=False, batched=False, clamp_tail=False):
     """Output-axis-contiguous kernel.  Thread layout: ``tx`` threads across
     the output axis (each owning ``vec`` adjacent outputs) times 256/tx slices
     of the reduce axis; gridDim.y further slices.  ``partial_in``: the single
     input holds ``_type_reduce`` values that are combined as they are."""
     # ``solo``: every thread owns its columns for the whole reduce axis (a
     # handful of rows): nothing to combine across lanes or waves
+    # ``batched``: the outputs form ``_n_out / _n_inner`` rows of ``_n_inner``
+    # adjacent columns (stored one row after the other); row b of input x
+    # starts ``_sb_x`` elements after row b - 1 and is reduced like the whole
+    # problem of the plain kernel.  Column blocks do not straddle rows: block
+    # ``_blk`` works on row ``_blk / _nbc``.
+    # ``clamp_tail``: the thread whose vector would reach past the last column
+    # loads the last full vector instead (overlapping its neighbour's) and
+    # moves its own columns to the front of its accumulators at the end; no
+    # lane then walks the reduce axis element by element.  Needs loads that
+    # may start at any element.
     if solo:
         tx = BLOCK
+    clamp_tail = clamp_tail and vec > 1 and not partial_in
     assert tx in (1, 2, 4, 8, 16, 32, 64) or solo
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     nt = 'true' if stream_hint else 'false'
@@ -419,6 +434,12 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     ty = BLOCK // tx
     waves = BLOCK // WAVE
     params = _fast_params(args, idx_t, partial_in, partial_out)
+    if batched:
+        assert not partial_in and not any(a.bcast_o for a in ins)
+        for a in ins:
+            params = re.sub(r'\b_p_%s\b' % a.name, '_q_%s' % a.name, params)
+        params += ', const %s _n_inner, const %s _nbc' % (idx_t, idx_t)
+        params += ''.join(', const %s _sb_%s' % (idx_t, a.name) for a in ins)
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         BLOCK, name, params))
@@ -430,13 +451,33 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('  const int _tx = threadIdx.x %% %d;' % tx)
     src.append('  const int _ty = threadIdx.x / %d;' % tx)
     # column blocks beyond the capacity of grid.x continue along grid.z
-    src.append('  const %s _c = ((((%s)blockIdx.z * gridDim.x + blockIdx.x) * %d) + _tx) * %d;' % (
-        idx_t, idx_t, tx, vec))
+    src.append('  const %s _blk = (%s)blockIdx.z * gridDim.x + blockIdx.x;' % (idx_t, idx_t))
+    if batched:
+        src.append('  const %s _b = _blk / _nbc;' % idx_t)
+        src.append('  const %s _c = ((_blk - _b * _nbc) * %d + _tx) * %d;' % (idx_t, tx, vec))
+        # blocks past the last row (grid rounded up along z) have no columns
+        src.append('  const %s _ncol = ((ptrdiff_t)_b * _n_inner < _n_out) ? _n_inner : 0;' % idx_t)
+        src.append('  const %s _i0 = _b * _n_inner;' % idx_t)
+        for a in ins:
+            src.append('  const %s* __restrict__ _p_%s = _q_%s + (ptrdiff_t)_b * _sb_%s;' % (
+                a.store_t, a.name, a.name, a.name))
+    else:
+        src.append('  const %s _c = (_blk * %d + _tx) * %d;' % (idx_t, tx, vec))
+        src.append('  const %s _ncol = _n_out;' % idx_t)
+        src.append('  const %s _i0 = 0;' % idx_t)
     src.append('  _type_reduce _acc[%d];' % vec)
     src.append('#pragma unroll')
     src.append('  for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (vec, _identity_decl(identity)))
-    src.append('  if (_c < _n_out) {')
-    src.append('    const bool _full = _c + %d <= _n_out;' % vec)
+    if clamp_tail:
+        src.append('  const %s _cl = (_c + %d <= _ncol) ? _c : (_ncol - %d);' % (idx_t, vec, vec))
+        src.append('  const int _shift = (int)(_c - _cl);')
+    else:
+        src.append('  const %s _cl = _c;' % idx_t)
+    src.append('  if (_c < _ncol) {')
+    if clamp_tail:
+        src.append('    const bool _full = _ncol >= %d;' % vec)
+    else:
+        src.append('    const bool _full = _c + %d <= _ncol;' % vec)
     src.append('    if (_full) {')
     src.append('      const %s _jstep = (%s)gridDim.y * %d;' % (idx_t, idx_t, ty))
     src.append('      %s _j = (%s)blockIdx.y * %d + _ty;' % (idx_t, idx_t, ty))
@@ -447,7 +488,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
                 src.append('      const %s _r_%s = _p_%s[0];' % (a.store_t, a.name, a.name))
             else:
                 src.append('      const cupy::Vec<%s, %d> _r_%s = cupy::load_vec<%s, %d, false>('
-                           '_p_%s + _c);' % (a.store_t, vec, a.name, a.store_t, vec, a.name))
+                           '_p_%s + _cl);' % (a.store_t, vec, a.name, a.store_t, vec, a.name))
 
     def loads(pad, j_expr, suffix):
         for a in ins:
@@ -465,7 +506,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
                     pad, a.store_t, a.name, suffix, a.name, j_expr, a.name))
             else:
                 src.append('%sconst cupy::Vec<%s, %d> _l_%s%s = cupy::load_vec<%s, %d, %s>('
-                           '_p_%s + (ptrdiff_t)(%s) * _sr_%s + _c);' % (
+                           '_p_%s + (ptrdiff_t)(%s) * _sr_%s + _cl);' % (
                                pad, a.store_t, vec, a.name, suffix, a.store_t, vec, nt,
                                a.name, j_expr, a.name))
 
@@ -512,7 +553,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     # a constant trip count with the bound tested inside: the accumulators are
     # then indexed by constants only and stay in registers whatever their type
     src.append('#pragma unroll')
-    src.append('        for (int _k = 0; _k < %d; ++_k) if (_c + _k < _n_out) {' % vec)
+    src.append('        for (int _k = 0; _k < %d; ++_k) if (_c + _k < _ncol) {' % vec)
     if partial_in:
         a = ins[0]
         src.append('          _acc[_k] = REDUCE(_acc[_k], _p_%s[(ptrdiff_t)_j * _sr_%s + _c + _k]);' % (
@@ -530,12 +571,21 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('      }')
     src.append('    }')
     src.append('  }')
-    if solo:
-        src.append('  if (_c < _n_out) {')
+    if clamp_tail:
+        src.append('  if (_c < _ncol && _ncol >= %d && _shift) {' % vec)
         src.append('#pragma unroll')
-        src.append('    for (int _k = 0; _k < %d; ++_k) if (_c + _k < _n_out) {' % vec)
+        src.append('    for (int _s = 1; _s < %d; ++_s) if (_shift == _s) {' % vec)
+        src.append('#pragma unroll')
+        src.append('      for (int _k = 0; _k < %d; ++_k) if (_k + _s < %d) _acc[_k] = _acc[_k + _s];' % (
+            vec, vec))
+        src.append('    }')
+        src.append('  }')
+    if solo:
+        src.append('  if (_c < _ncol) {')
+        src.append('#pragma unroll')
+        src.append('    for (int _k = 0; _k < %d; ++_k) if (_c + _k < _ncol) {' % vec)
         src.append('      _type_reduce _s = _acc[_k];')
-        src.append('      const %s _i = _c + _k;' % idx_t)
+        src.append('      const %s _i = _i0 + _c + _k;' % idx_t)
         src.extend(_finish(args, partial_out, '      '))
         src.append('    }')
         src.append('  }')
@@ -554,12 +604,12 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         vec, tx, vec))
     src.append('  }')
     src.append('  __syncthreads();')
-    src.append('  if (threadIdx.x < %d && _c < _n_out) {' % tx)
-    src.append('    for (int _k = 0; _k < %d && _c + _k < _n_out; ++_k) {' % vec)
+    src.append('  if (threadIdx.x < %d && _c < _ncol) {' % tx)
+    src.append('    for (int _k = 0; _k < %d && _c + _k < _ncol; ++_k) {' % vec)
     src.append('      _type_reduce _s = _sm[_tx * %d + _k];' % vec)
     src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[(_w * %d + _tx) * %d + _k]);' % (
         waves, tx, vec))
-    src.append('      const %s _i = _c + _k;' % idx_t)
+    src.append('      const %s _i = _i0 + _c + _k;' % idx_t)
     src.extend(_finish(args, partial_out, '      '))
     src.append('    }')
     src.append('  }')

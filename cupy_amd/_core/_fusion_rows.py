@@ -118,7 +118,7 @@ class RowPlan:
                 # an array: contiguous and aligned as the kernel's vector
                 # accesses assume, or the call goes the general way
                 ptr = v.data.ptr
-                if not v._c_contiguous or ptr % descr:
+                if not v._c_contiguous or not _aligned(ptr, descr):
                     return self.fallback.run(*args)
                 vals.append(ptr)
             else:

@@ -309,8 +309,11 @@ def _max_vector_width(itemsizes):
     return max(v, 1)
 
 
-def _aligned(ptr, nbytes):
-    return ptr % nbytes == 0
+def _aligned(value, nbytes):
+    """Whether vector accesses of ``nbytes`` may start at the address (or be
+    spaced by the byte stride) ``value``.  The device takes such accesses at
+    the alignment of one element, which every array has."""
+    return value % nbytes == 0 or _tuning.get('unaligned_vectors')
 
 
 _grid_limit_memo = {}
@@ -446,6 +449,10 @@ class _ElementwisePlanner:
         if not itemsizes:
             itemsizes = [arrays[0].dtype.itemsize]
         vec = _max_vector_width(itemsizes)
+        mixed = False
+        if _tuning.get('flat_vec_by') == 'wide' and max(itemsizes) != min(itemsizes):
+            vec = max(1, 16 // max(itemsizes))
+            mixed = True
         # every iterated array must sit on a boundary of its vector
         ai = 0
         for a, p in zip(args, params):
@@ -459,6 +466,8 @@ class _ElementwisePlanner:
             vec = 1
         idx64 = size > _INT32_MAX - (1 << 24)
         unroll = _tuning.get('flat_unroll') if vec > 1 else 1
+        if mixed and vec > 1:
+            unroll = _tuning.get('flat_mixed_unroll') if len(itemsizes) <= 2 else 1
         block = _tuning.get('flat_block')
         if len(itemsizes) <= 2 and block > 512:
             # one stream in, one out: measured 2 % faster with smaller
@@ -630,9 +639,9 @@ class _ElementwisePlanner:
                 if not _aligned(a.data.ptr, nb):
                     ok = False
                 elif layouts[nm] == 'R':
-                    if cs[0] % nb:
+                    if not _aligned(cs[0], nb):
                         ok = False
-                elif cs[1] % nb:
+                elif not _aligned(cs[1], nb):
                     ok = False
             if ok:
                 break

@@ -279,6 +279,25 @@ class _AbstractReductionKernel:
                 return self._launch_rows(*plan_args)
             if cols_ok:
                 return self._launch_cols(*plan_args)
+        # reduction over a middle axis: in[b, j, c] -> out[b, c] with c adjacent
+        # in memory everywhere and the outputs stored row after row
+        if (len(rshape) <= 1 and len(oshape) == 2 and not has_raw and not needs_indexers
+                and in_arr_idx):
+            ins = [in_args[i] for i in in_arr_idx]
+            outs = [out_args[i] for i in out_arr_idx]
+            n_batch, n_inner = oshape
+            sr = [(rs[0] if rs else 0) for rs in rstrides]
+            if (all(os_[1] == a.dtype.itemsize and os_[0] % a.dtype.itemsize == 0
+                    for os_, a in zip(o_in, ins))
+                    and all(tuple(os_) == (n_inner * a.dtype.itemsize, a.dtype.itemsize)
+                            for os_, a in zip(o_out, outs))
+                    and all(s % a.dtype.itemsize == 0 for s, a in zip(sr, ins))):
+                return self._launch_cols(
+                    in_args, out_args, in_arr_idx, out_arr_idx, n_batch * n_inner,
+                    rshape[0] if rshape else 1, [a.dtype.itemsize for a in ins], sr,
+                    [a.dtype.itemsize for a in outs], map_expr, reduce_expr,
+                    post_map_expr, reduce_type, typedefs, device_id, stream_ptr, rec,
+                    batch=(n_batch, n_inner, [os_[0] for os_ in o_in]))
         # generic: views with the reduced axes in front, merged where possible
         g_in = list(in_args)
         for k, i in enumerate(in_arr_idx):
@@ -458,7 +477,7 @@ class _AbstractReductionKernel:
                 if s_r == 0:
                     continue
                 nb = min(16, vec * a.dtype.itemsize)
-                if not _aligned(a.data.ptr, nb) or (n_out > 1 and s_o % nb):
+                if not _aligned(a.data.ptr, nb) or (n_out > 1 and not _aligned(s_o, nb)):
                     ok = False
             if ok and n_red >= vec:
                 break
@@ -570,30 +589,39 @@ class _AbstractReductionKernel:
     # -- cols ---------------------------------------------------------------------------------
     def _launch_cols(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                      so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
-                     reduce_type, typedefs, device_id, stream_ptr, rec=None):
+                     reduce_type, typedefs, device_id, stream_ptr, rec=None, batch=None):
+        """``batch`` = (rows of outputs, columns per row, byte stride of every
+        input from row to row) for the reduction over a middle axis; ``n_out``
+        is then the total number of outputs."""
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
         cus = _device.get_compute_units(device_id)
         vec = _max_vector_width([a.dtype.itemsize for a in ins])
         bcast_o = [(s == 0 and n_out > 1) for s in so_in]
+        n_batch, n_cols, sb = batch if batch else (1, n_out, None)
         while vec > 1:
-            ok = n_out >= vec
+            ok = n_cols >= vec
             for a, s_o, s_r in zip(ins, so_in, sr):
                 if s_o == 0 and n_out > 1:
                     continue
                 nb = min(16, vec * a.dtype.itemsize)
-                if not _aligned(a.data.ptr, nb) or (n_red > 1 and s_r % nb):
+                if not _aligned(a.data.ptr, nb) or (n_red > 1 and not _aligned(s_r, nb)):
                     ok = False
+            if batch and not all(_aligned(s, min(16, vec * a.dtype.itemsize))
+                                 for s, a in zip(sb, ins)):
+                ok = False
             if ok:
                 break
             vec //= 2
-        tx = max(1, min(64, internal.clp2((n_out + vec - 1) // vec)))
+        tx = max(1, min(64, internal.clp2((n_cols + vec - 1) // vec)))
         # a handful of rows and plenty of columns: a thread per column vector
-        solo = n_red <= 8 and n_out >= cus * _cg.BLOCK * vec
+        solo = (n_red <= 8 and n_out >= cus * _cg.BLOCK * vec
+                and n_cols >= _cg.BLOCK * vec)
         if solo:
             tx = _cg.BLOCK
         ty = _cg.BLOCK // tx
-        gx = (n_out + tx * vec - 1) // (tx * vec)
+        nbc = (n_cols + tx * vec - 1) // (tx * vec)
+        gx = nbc * n_batch
         # the kernel does not loop over column blocks: beyond what grid.x may
         # hold they continue along grid.z
         gz = (gx + _max_blocks(_cg.BLOCK) - 1) // _max_blocks(_cg.BLOCK)
@@ -604,38 +632,58 @@ class _AbstractReductionKernel:
         partial = n_split > 1
         span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
                    + [abs(s) * n_out for s in so_out] + [n_red + n_split * ty])
+        if batch:
+            span = max([span, gx * gz * tx * vec] + [
+                abs(s_b) * n_batch + abs(s_r) * n_red + s_o * n_cols
+                for s_b, s_r, s_o in zip(sb, sr, so_in)])
         idx64 = span > _INT32_MAX - (1 << 24)
         rargs = self._rargs(in_args, out_args, bcast_r=[s == 0 for s in sr], bcast_o=bcast_o)
+        clamp = bool(n_cols % vec and n_cols >= vec and _tuning.get('unaligned_vectors'))
+        if solo:
+            unroll = 1
+        elif partial and all(s % 128 == 0 for s in sr):
+            unroll = _tuning.get('cols_unroll')
+        else:
+            unroll = _tuning.get('cols_unroll_near')
         stream_hint = _tuning.stream_policy(
             _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
-               stream_hint, solo, _tuning.signature())
+               stream_hint, solo, bool(batch), clamp, unroll, _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
                 self.name, rargs, self.identity, map_expr, reduce_expr,
                 post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
                 idx64=idx64, partial_out=partial,
-                stream_hint=stream_hint, unroll=_tuning.get('cols_unroll'), solo=solo)
+                stream_hint=stream_hint, unroll=unroll, solo=solo,
+                batched=bool(batch), clamp_tail=clamp)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
+        tail = ''
+        if batch:
+            tail = ic * (2 + len(ins))
+            batch_vals = [n_cols, nbc] + [s // a.dtype.itemsize for s, a in zip(sb, ins)]
         if partial:
             rsize = self._reduce_type_size(reduce_type, mod)
             partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
             vals.ptr(pref, partials.ptr)
+            if batch:
+                vals.const(*batch_vals)
             _launch_plan.launch(
                 rec, fn, (gx, n_split, gz), (_cg.BLOCK, 1, 1),
-                _make_packer(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
+                _make_packer(self._fast_format(rargs, ic, 'P' + tail)), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
                 stream_ptr, rec, pref, n_out * n_red)
         else:
+            if batch:
+                vals.const(*batch_vals)
             _launch_plan.launch(
                 rec, fn, (gx, 1, gz), (_cg.BLOCK, 1, 1),
-                _make_packer(self._fast_format(rargs, ic)), vals, stream_ptr)
+                _make_packer(self._fast_format(rargs, ic, tail)), vals, stream_ptr)
 
     # -- generic ------------------------------------------------------------------------------
     def _launch_generic(self, in_args, out_args, in_shape, out_shape, n_red,

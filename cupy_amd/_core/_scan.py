@@ -28,6 +28,7 @@ import numpy
 
 from cupy_amd._core import _tuning
 from cupy_amd._core import internal
+from cupy_amd._core._kernel import _aligned
 from cupy_amd._core._scalar import get_typename as _get_typename
 from cupy_amd._core.core import ndarray
 from cupy_amd.cuda import compiler
@@ -440,8 +441,8 @@ def _lanes_geometry(src, dst, inner, item):
         return None
     vec = max(1, 16 // item)
     while vec >= 1:
-        if (inner % vec == 0 and src.data.ptr % (vec * src.dtype.itemsize) == 0
-                and dst.data.ptr % (vec * dst.dtype.itemsize) == 0):
+        if (inner % vec == 0 and _aligned(src.data.ptr, vec * src.dtype.itemsize)
+                and _aligned(dst.data.ptr, vec * dst.dtype.itemsize)):
             lstride = inner // vec
             if lstride <= 16 and lstride & (lstride - 1) == 0:
                 return vec, lstride
@@ -471,8 +472,8 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                                        total * out_dtype.itemsize)
     if inner == 1:
         vec = max(1, 16 // item)
-        while vec > 1 and (src.data.ptr % (vec * in_dtype.itemsize)
-                           or dst.data.ptr % (vec * out_dtype.itemsize)
+        while vec > 1 and (not _aligned(src.data.ptr, vec * in_dtype.itemsize)
+                           or not _aligned(dst.data.ptr, vec * out_dtype.itemsize)
                            or (outer > 1 and n % vec) or n < vec):
             vec //= 2
         # short rows: a group of lanes smaller than a wave per row, each lane
@@ -536,8 +537,8 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         middle_round = per_wave
     else:
         vec = max(1, 16 // item)
-        while vec > 1 and (src.data.ptr % (vec * in_dtype.itemsize)
-                           or dst.data.ptr % (vec * out_dtype.itemsize)
+        while vec > 1 and (not _aligned(src.data.ptr, vec * in_dtype.itemsize)
+                           or not _aligned(dst.data.ptr, vec * out_dtype.itemsize)
                            or inner % vec):
             vec //= 2
         trips = 4

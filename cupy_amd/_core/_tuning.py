@@ -15,6 +15,19 @@ _params = {
     'flat_block': 1024,         # threads per workgroup
     'flat_unroll': 1,           # vectors per thread per trip
     'flat_blocks_per_cu': 64,   # grid cap, in workgroups per CU
+    # Operands of different widths: the widest moves 16 bytes per access
+    # ('wide'; the narrower ones then move less, but consecutive lanes stay on
+    # consecutive addresses in every operand) or the narrowest does ('narrow';
+    # a lane of the wide operand then covers 32-128 bytes and each access of a
+    # wave is spread over four times its size).  Measured on 2^26 elements,
+    # narrow -> wide: float32 > 0 -> bool 54 -> 79 % of peak, int8 -> int64
+    # 17 -> 77 %, where(mask, float32, float32) 38 -> 83 %, isnan(float64)
+    # 52 -> 82 %, float32 * float16 70 -> 79 %.
+    'flat_vec_by': 'wide',
+    # ... with this many vectors per thread and trip when one array is read and
+    # one written (2: +2 to +20 points over 1 there; with three or more arrays
+    # 1 is better by 2 to 6 points)
+    'flat_mixed_unroll': 2,
     # Non-temporal hints of the elementwise kernels: True / False for loads and
     # stores alike, or 'auto' = by footprint against the last-level cache
     # (see stream_policy below)
@@ -33,11 +46,24 @@ _params = {
     'rows_lane_bytes': 128,     # ... and at most this many bytes in flight per lane
     'rows_group_rows_per_lane': 64,   # grid cap for sub-wave groups: CUs * this workgroups
     'cols_stream': True,
+    # Row-slices a thread of the column kernel loads before it uses the first:
+    # 1 when the reduce axis is split across workgroups and the rows start on
+    # cache-line boundaries (the slices of one thread are then far apart:
+    # 16384 x 4096 float32, axis 0: 45.8 us with 1, 50.2 us with 4), otherwise
+    # `cols_unroll_near` (64 x 64 x 16384, axis 1: 56.0 -> 47.8 us; 257 x 511 x
+    # 509: 78.5 -> 60.6 us)
     'cols_unroll': 1,
+    'cols_unroll_near': 4,
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
     # fused row-wise functions: words per lane up to which a wave takes a whole row
     'fused_rows_wave_words': 64,
+    # Vector accesses need only the alignment of one element: an access of 16
+    # bytes at an address that is a multiple of 4 measures within 4 % of an
+    # aligned one (reads of 2^28 bytes: 82 % of peak against 86 %), one at an odd
+    # byte address reaches 58 % where element-wide accesses stay below 30 %.
+    # False restricts vectors to operands aligned to the whole vector.
+    'unaligned_vectors': True,
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
 }

@@ -252,7 +252,8 @@ _CUPY_DEV double _floor_divide(double x, double y) { return floor(x / y); }
 // ---------------------------------------------------------------------------
 // Vector access: N consecutive elements moved with the widest instructions the
 // alignment allows (up to 16 bytes each, i.e. global_load/store_dwordx4).
-// The pointer must be aligned to min(16, N * sizeof(T)).
+// The pointer needs the alignment of one element only: the device takes wide
+// accesses at any address, at full speed when it is a multiple of 4.
 // ---------------------------------------------------------------------------
 namespace cupy {
 
@@ -278,8 +279,9 @@ _CUPY_DEV Vec<T, N> load_vec(const T* p) {
   constexpr int kTotal = sizeof(T) * N;
   constexpr int kChunk = kTotal > 16 ? 16 : kTotal;
   typedef typename _RawChunk<kChunk>::type raw_t;
+  typedef raw_t __attribute__((aligned(alignof(T)))) raw_at_t;
   Vec<T, N> out;
-  const raw_t* src = reinterpret_cast<const raw_t*>(p);
+  const raw_at_t* src = reinterpret_cast<const raw_at_t*>(p);
 #pragma unroll
   for (int c = 0; c < kTotal / kChunk; ++c) {
     raw_t r = kStream ? __builtin_nontemporal_load(src + c) : src[c];
@@ -293,7 +295,8 @@ _CUPY_DEV void store_vec(T* p, const Vec<T, N>& x) {
   constexpr int kTotal = sizeof(T) * N;
   constexpr int kChunk = kTotal > 16 ? 16 : kTotal;
   typedef typename _RawChunk<kChunk>::type raw_t;
-  raw_t* dst = reinterpret_cast<raw_t*>(p);
+  typedef raw_t __attribute__((aligned(alignof(T)))) raw_at_t;
+  raw_at_t* dst = reinterpret_cast<raw_at_t*>(p);
 #pragma unroll
   for (int c = 0; c < kTotal / kChunk; ++c) {
     raw_t r;

@@ -132,7 +132,12 @@ def test_axis_reductions_and_scans_with_rows_beyond_2_to_30():
 def test_column_reduction_whose_blocks_continue_along_grid_z():
     m = 2 ** 30 + 1                                   # more column blocks than grid.x holds
     a = _fill_mod100_i8(size=9 * m).reshape(9, m)
-    colsum = a.sum(axis=0)
+    from cupy_amd._core import _tuning
+    _tuning.set(unaligned_vectors=False)              # rows of odd length: a thread per column
+    try:
+        colsum = a.sum(axis=0)
+    finally:
+        _tuning.set(unaligned_vectors=True)
     check = cp.ElementwiseKernel(
         'int64 s', 'bool ok',
         'const long long m = 1073741825LL; long long w = 0;'

@@ -308,3 +308,51 @@ def test_large_full_reduction_is_split_and_deterministic():
     i = shaped_random((3_000_001,), 'int32', 24, scale=2 ** 30)
     assert_exact(cp.asarray(i).sum().get(), np.asarray(i.sum()))
     assert int(cp.asarray(i).argmax().get()) == int(i.argmax())
+
+
+MIDDLE = [((3, 5, 7), 'int32'), ((33, 65, 311), 'float32'), ((7, 3, 70001), 'int8'),
+          ((300, 17, 9), 'float64'), ((2, 2000, 130), 'float16'), ((64, 8, 1031), 'float32'),
+          ((5, 1, 1000), 'int16'), ((1, 40, 5000), 'float32'), ((9, 4000, 3), 'int64')]
+
+
+@pytest.mark.parametrize('shape,dtype', MIDDLE)
+def test_reduction_over_a_middle_axis(shape, dtype):
+    x = shaped_random(shape, dtype, 21)
+    dx = cp.asarray(x)
+    if np.dtype(dtype).kind == 'f':
+        got = dx.sum(axis=1).get()
+        want = x.astype(np.float64).sum(axis=1)
+        tol = {'float16': 2e-3, 'float32': 1e-5, 'float64': 1e-12}[dtype]
+        scale = np.abs(x.astype(np.float64)).sum(axis=1)
+        assert got.dtype == x.sum(axis=1).dtype
+        assert np.all(np.abs(got - want) <= tol * np.maximum(scale, 1))
+    else:
+        assert_exact(dx.sum(axis=1).get(), x.sum(axis=1))
+    assert_exact(dx.max(axis=1).get(), x.max(axis=1))
+    assert_exact(dx.argmax(axis=1).get(), x.argmax(axis=1))
+    assert_exact(dx.argmin(axis=1, keepdims=True).get(), x.argmin(axis=1, keepdims=True))
+    assert_exact(dx.min(axis=1, keepdims=True).get(), x.min(axis=1, keepdims=True))
+    # a window whose rows and batches are spaced wider than their length
+    if shape[0] > 1 and shape[2] > 4:
+        w, dw = x[1:, :, 1:-2], dx[1:, :, 1:-2]
+        assert_exact(dw.max(axis=1).get(), w.max(axis=1))
+        assert_exact(dw.argmax(axis=1).get(), w.argmax(axis=1))
+        out = cp.zeros(w.max(axis=1).shape, dtype)
+        r = dw.min(axis=1, out=out)
+        assert r is out
+        assert_exact(out.get(), w.min(axis=1))
+
+
+def test_middle_axis_of_four_dimensions_and_broadcast_batches():
+    x = shaped_random((4, 6, 50, 33), 'int32', 22)
+    dx = cp.asarray(x)
+    assert_exact(dx.sum(axis=2).get(), x.sum(axis=2))             # (4*6, 50, 33)
+    assert_exact(dx.sum(axis=1).get(), x.sum(axis=1))             # (4, 6, 50*33)
+    assert_exact(dx.sum(axis=(1, 2)).get(), x.sum(axis=(1, 2)))
+    b = np.broadcast_to(x[:1], (5, 6, 50, 33))
+    db = cp.broadcast_to(dx[:1], (5, 6, 50, 33))
+    assert_exact(db.sum(axis=2).get(), b.sum(axis=2))
+    assert_exact(db.argmax(axis=1).get(), b.argmax(axis=1))
+    k = cp.ReductionKernel('T x, T y', 'T z', 'x * y', 'a + b', 'z = a', '0', 'dot_middle')
+    y = shaped_random((4, 6, 50, 33), 'int32', 23)
+    assert_exact(k(dx, cp.asarray(y), axis=2).get(), (x * y).sum(axis=2, dtype=np.int32))
