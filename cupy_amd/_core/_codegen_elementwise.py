@@ -350,9 +350,15 @@ def emit_generic(name, operands, operation, typedefs='', preamble='',
 
 def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
                  loop_prep='', after_loop='', layouts=None, vec=4, tile_r=64,
-                 tile_c=64, threads=256, idx64=False, stream_hint=True):
+                 tile_c=64, threads=256, idx64=False, stream_hint=True, batched=False):
     """Kernel for a 2-d index space (rows r, columns c) where every array
     operand is contiguous along one of the axes.
+
+    ``batched``: ``_nbt`` such index spaces, numbered b = b0 * ``_nb1`` + b1;
+    array x starts ``b0 * _sb0_x + b1 * _sb1_x`` elements further on in space b
+    (the two slowest axes of a 3-d or 4-d problem whose arrays are permuted
+    differently).  These parameters follow the strides.  The element index
+    ``i`` is not available then.
 
     ``layouts[name]`` is
       'R'   unit stride along columns, any stride (also 0) along rows;
@@ -388,6 +394,12 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     for op in arrays:
         parts += ['const %s _sr_%s' % (idx_t, op.name),
                   'const %s _sc_%s' % (idx_t, op.name)]
+    if batched:
+        assert not (use_i or set_ind) and not needs_ind
+        parts += ['const %s _nbt' % idx_t, 'const %s _nb1' % idx_t]
+        for op in arrays:
+            parts += ['const %s _sb0_%s' % (idx_t, op.name),
+                      'const %s _sb1_%s' % (idx_t, op.name)]
     parts += [_param_decl(op) for op in operands if op.kind == 'indexer']
     params = ', '.join(parts)
 
@@ -396,8 +408,8 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         assert not op.is_out, 'transposed outputs are not handled by tiled2d'
 
     def gaddr(op, r, c):
-        return '(_p_%s + (ptrdiff_t)(%s) * _sr_%s + (ptrdiff_t)(%s) * _sc_%s)' % (
-            op.name, r, op.name, c, op.name)
+        return '(_p_%s + %s(ptrdiff_t)(%s) * _sr_%s + (ptrdiff_t)(%s) * _sc_%s)' % (
+            op.name, ('_o_%s + ' % op.name) if batched else '', r, op.name, c, op.name)
 
     src = [_header(typedefs, preamble)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
@@ -407,7 +419,18 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         src.append('  __shared__ %s _t_%s[%d];' % (op.store_t, op.name, tile_r * pitch))
     src.append('  const %s _ntr = (_nr + %d) / %d;' % (idx_t, tile_r - 1, tile_r))
     src.append('  const %s _ntc = (_nc + %d) / %d;' % (idx_t, tile_c - 1, tile_c))
-    src.append('  for (%s _tile = blockIdx.x; _tile < _ntr * _ntc; _tile += gridDim.x) {' % idx_t)
+    if batched:
+        src.append('  const %s _nt2 = _ntr * _ntc;' % idx_t)
+        src.append('  for (%s _tile_b = blockIdx.x; _tile_b < _nt2 * _nbt; _tile_b += gridDim.x) {' % idx_t)
+        src.append('    const %s _bt = _tile_b / _nt2;' % idx_t)
+        src.append('    const %s _tile = _tile_b - _bt * _nt2;' % idx_t)
+        src.append('    const %s _b0 = _bt / _nb1;' % idx_t)
+        src.append('    const %s _b1 = _bt - _b0 * _nb1;' % idx_t)
+        for op in arrays:
+            src.append('    const ptrdiff_t _o_%s = (ptrdiff_t)_b0 * _sb0_%s + (ptrdiff_t)_b1 * _sb1_%s;' % (
+                op.name, op.name, op.name))
+    else:
+        src.append('  for (%s _tile = blockIdx.x; _tile < _ntr * _ntc; _tile += gridDim.x) {' % idx_t)
     # Diagonal tile order: consecutive workgroups differ in both the row block
     # and the column block.  With power-of-two pitches, walking along one axis
     # only would keep the low address bits of either the transposed reads or the

@@ -416,6 +416,15 @@ class _ElementwisePlanner:
                     mode = 'flat'
             elif nd == 2 and not self._uses_ind:
                 mode = self._classify_2d(arrays, cstrides, args, nin)
+            elif nd in (3, 4) and not self._uses_ind and not self._uses_i:
+                plan = self._plan_batched(arrays, cshape, cstrides, args, nin)
+                if plan is not None:
+                    done = self._launch_tiled(
+                        dev_id, args, nin, arrays, plan[0], plan[1], var_types, typedefs,
+                        casts, force_read_out, stream_ptr, kernel_name, False, rec,
+                        batch=plan[2])
+                    if done is not None:
+                        return
         if mode == 'flat':
             return self._launch_flat(
                 dev_id, args, nin, arrays, cstrides, size, var_types, typedefs,
@@ -602,9 +611,52 @@ class _ElementwisePlanner:
                 return 'tiled_t'
         return 'generic'
 
+    def _plan_batched(self, arrays, cshape, cstrides, args, nin):
+        """Splits the axes of a 3-d or 4-d problem into batch axes and the two
+        axes of the tiled kernel: columns = the axis every output (and every
+        array that is not transposed) runs along with unit stride, rows = the
+        axis the transposed inputs run along, or the innermost other axis.
+        Returns ((nr, nc), [(sr, sc) per array], (batch shape, [batch strides
+        per array])) or None."""
+        nd = len(cshape)
+        outs = args[nin:]
+        is_out = [any(a is o for o in outs) for a in arrays]
+        col = None
+        for ax in range(nd - 1, -1, -1):
+            if all(cs[ax] == a.dtype.itemsize
+                   for a, cs, o in zip(arrays, cstrides, is_out) if o):
+                col = ax
+                break
+        if col is None or not any(is_out):
+            return None
+        row = None
+        for a, cs, o in zip(arrays, cstrides, is_out):
+            item = a.dtype.itemsize
+            if any(s % item for s in cs):
+                return None
+            if cs[col] == item or cs[col] == 0:
+                continue
+            if o:
+                return None
+            unit = [ax for ax in range(nd) if ax != col and cs[ax] == item]
+            if not unit or (row is not None and row not in unit):
+                return None
+            row = unit[0] if row is None else row
+        if row is None:
+            row = max(ax for ax in range(nd) if ax != col)
+        rest = [ax for ax in range(nd) if ax not in (row, col)]
+        shape2 = (cshape[row], cshape[col])
+        strides2 = [(cs[row], cs[col]) for cs in cstrides]
+        bshape = tuple(cshape[ax] for ax in rest)
+        bstrides = [tuple(cs[ax] for ax in rest) for cs in cstrides]
+        if len(rest) == 1:
+            bshape = bshape + (1,)
+            bstrides = [bs + (0,) for bs in bstrides]
+        return shape2, strides2, (bshape, bstrides)
+
     def _launch_tiled(self, dev_id, args, nin, arrays, cshape, cstrides, var_types,
                       typedefs, casts, force_read_out, stream_ptr, kernel_name, swap,
-                      rec):
+                      rec, batch=None):
         params = self.params
         if swap:
             cshape = (cshape[1], cshape[0])
@@ -670,6 +722,16 @@ class _ElementwisePlanner:
         span = 0
         for a, cs in zip(arrays, cstrides):
             span = max(span, abs(cs[0]) * nr + abs(cs[1]) * nc)
+        nbt = 1
+        if batch:
+            bshape, bstrides = batch
+            nbt = bshape[0] * bshape[1]
+            for k, bs in enumerate(bstrides):
+                cs = cstrides[k]
+                span = max(span, abs(cs[0]) * nr + abs(cs[1]) * nc
+                           + abs(bs[0]) * bshape[0] + abs(bs[1]) * bshape[1])
+            # the tile counter runs over whole tiles, edge tiles included
+            span = max(span, nbt * (nr + tile_r) * (nc + tile_c))
         idx64 = span > _INT32_MAX or nr * nc > _INT32_MAX
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
         stream_hint = _tuning.stream_policy(
@@ -677,7 +739,7 @@ class _ElementwisePlanner:
             *self._traffic(args, nin, [n for n, l in layouts.items() if l == 'R0']))
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
-               threads)
+               threads, bool(batch))
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
@@ -685,7 +747,7 @@ class _ElementwisePlanner:
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
                 tile_r=tile_r, tile_c=tile_c, threads=threads, idx64=idx64,
-                stream_hint=stream_hint)
+                stream_hint=stream_hint, batched=bool(batch))
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']
@@ -697,6 +759,8 @@ class _ElementwisePlanner:
                 elif o.kind == 'scalar':
                     fmt.append(_scalar_struct_code(o.store_t))
             fmt.append(ic * (2 + 2 * len(arrays)))
+            if batch:
+                fmt.append(ic * (2 + 2 * len(arrays)))
             entry = (fn, _make_packer(fmt), code)
             with self._lock:
                 entry = self._memo.setdefault(key, entry)
@@ -707,7 +771,12 @@ class _ElementwisePlanner:
         for a, cs in zip(arrays, cstrides):
             item = a.dtype.itemsize
             block_args.const(cs[0] // item, cs[1] // item)
-        ntiles = ((nr + tile_r - 1) // tile_r) * ((nc + tile_c - 1) // tile_c)
+        if batch:
+            block_args.const(nbt, bshape[1])
+            for a, bs in zip(arrays, bstrides):
+                item = a.dtype.itemsize
+                block_args.const(bs[0] // item, bs[1] // item)
+        ntiles = ((nr + tile_r - 1) // tile_r) * ((nc + tile_c - 1) // tile_c) * nbt
         grid = max(1, min(ntiles, _max_blocks(threads)))
         _launch_plan.launch(rec, fn, (grid, 1, 1), (threads, 1, 1), packer, block_args,
                             stream_ptr)

@@ -471,3 +471,53 @@ def test_cuda_array_interface_round_trip():
     assert np.allclose(cp.asarray(f).sum(axis=0).get(), a[:, ::2].sum(axis=0), rtol=1e-5)
     assert d.__cuda_array_interface__['strides'] is None
     assert d.T.__cuda_array_interface__['strides'] == d.T.strides
+
+
+# -- permuted operands of three and four dimensions -------------------------------------
+
+import itertools
+
+
+@pytest.mark.parametrize('shape', [(5, 70, 130), (33, 65, 31), (2, 129, 257), (64, 3, 200)])
+@pytest.mark.parametrize('dtype', ['float32', 'int8', 'float64'])
+def test_every_permutation_of_three_axes(shape, dtype):
+    x = shaped_random(shape, dtype, 31)
+    dx = cp.asarray(x)
+    for perm in itertools.permutations(range(3)):
+        t, dt = x.transpose(perm), dx.transpose(perm)
+        assert_exact(cp.ascontiguousarray(dt).get(), np.ascontiguousarray(t))
+        y = shaped_random(t.shape, dtype, 32)
+        assert_exact((dt + cp.asarray(y)).get(), t + y)
+        # both operands permuted, differently
+        u = shaped_random(shape[::-1], dtype, 33)
+        du = cp.asarray(u)
+        if u.T.shape == t.shape:
+            assert_exact((dt * du.T).get(), t * u.T)
+
+
+@pytest.mark.parametrize('perm', [(0, 2, 1, 3), (0, 1, 3, 2), (2, 0, 1, 3), (3, 1, 2, 0),
+                                  (1, 0, 3, 2), (0, 3, 1, 2), (3, 2, 1, 0)])
+def test_permutations_of_four_axes(perm):
+    shape = (3, 17, 66, 35)
+    x = shaped_random(shape, 'float32', 34)
+    dx = cp.asarray(x)
+    t, dt = x.transpose(perm), dx.transpose(perm)
+    assert_exact(cp.ascontiguousarray(dt).get(), np.ascontiguousarray(t))
+    row = shaped_random((t.shape[-1],), 'float32', 35)
+    assert_exact((dt * cp.asarray(row)).get(), t * row)
+    col = shaped_random(t.shape[:2] + (1, 1), 'float32', 36)
+    assert_exact((dt - cp.asarray(col)).get(), t - col)
+    out = cp.zeros(t.shape, 'float32')
+    cp.negative(dt, out=out)
+    assert_exact(out.get(), -t)
+
+
+def test_permuted_windows_and_mixed_types():
+    x = shaped_random((20, 70, 90), 'float16', 37)
+    y = shaped_random((90, 20, 70), 'float32', 38)
+    dx, dy = cp.asarray(x), cp.asarray(y)
+    a, da = x[1:, 2:-3, 5:], dx[1:, 2:-3, 5:]
+    b, db = y.transpose(1, 2, 0)[1:, 2:-3, 5:], dy.transpose(1, 2, 0)[1:, 2:-3, 5:]
+    assert_exact((da + db).get(), a + b)
+    assert_exact((da.transpose(1, 0, 2) > db.transpose(1, 0, 2)).get(),
+                 a.transpose(1, 0, 2) > b.transpose(1, 0, 2))
