@@ -6,7 +6,7 @@ A reduction is stated as in the reference (cupy/_core/_reduction.pyx:44-126):
 ``identity``, and ``_J`` = position of the element along the reduced axes.
 Where the reference has one template (strided per-thread accumulation followed
 by an LDS tree with a barrier per level, one launch geometry formula), this
-module has three kernels, chosen by the host from the canonical 2-d form
+module has four kernels, chosen by the host from the canonical 2-d form
 ``in[i, j]`` (i = output index, j = reduce index) of the problem:
 
 ``rows``     the reduce axis is contiguous in memory.  A group of G lanes
@@ -22,6 +22,9 @@ module has three kernels, chosen by the host from the canonical 2-d form
              across workgroups, a partial-result buffer.  The same kernel
              takes a batch of such problems (reduction over a middle axis:
              ``in[b, j, c]`` to ``out[b, c]``).
+``rows_flat`` short rows of odd length stored without gaps: a workgroup
+             copies a run of whole rows into the LDS with full vector loads
+             and lane groups reduce the rows from there.
 ``generic``  any strides: CIndexer addressing, same thread layout as ``cols``.
 
 Partial results are combined by a second ``cols`` launch that reads
@@ -400,6 +403,95 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
     src.append('#undef _JV')
     src.append('#undef _JOK')
     src.append('#undef _JC')
+    src.append('}')
+    return '\n'.join(src) + '\n'
+
+
+def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
+                   reduce_type, typedefs='', preamble='', width=3, group=1, rows=256,
+                   stream_hint=False):
+    """Reduce-axis-contiguous kernel for short rows of ``width`` elements (a
+    compile-time constant) that follow one another without gaps and whose
+    length in bytes is not a multiple of a vector: a lane group per row would
+    either leave lanes idle or load element by element.  A workgroup instead
+    copies ``rows`` consecutive rows -- one contiguous run of memory -- into
+    the LDS with full 16-byte loads on consecutive lanes, and then ``group``
+    lanes per row (a power of two) read the row back from the LDS and reduce
+    it.  Row r starts its walk ``r * group`` elements into the row (and wraps
+    around), so that the lanes of a wave are spread over the LDS banks for
+    even widths too.
+
+    Every input must have element strides (width, 1).  Same parameters as the
+    rows kernel."""
+    ins = [a for a in args if a.kind == 'in']
+    assert ins and group in (1, 2, 4, 8, 16, 32, 64) and rows % (BLOCK // group) == 0
+    nt = 'true' if stream_hint else 'false'
+    params = _fast_params(args, 'ptrdiff_t', False, False)
+    per_pass = BLOCK // group
+    src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        BLOCK, name, params))
+    src.append(_SIZE_INDEXERS)
+    src.append('  const ptrdiff_t _row0 = (ptrdiff_t)blockIdx.x * %d;' % rows)
+    src.append('  const int _nrows = (_n_out - _row0 < %d) ? (int)(_n_out - _row0) : %d;' % (rows, rows))
+    src.append('  const int _count = _nrows * %d;' % width)
+    vecs = {}
+    for a in ins:
+        # element size of the stored type is not known here: 16 bytes per lane
+        src.append('  constexpr int _V_%s = 16 / sizeof(%s) > 0 ? 16 / sizeof(%s) : 1;' % (
+            a.name, a.store_t, a.store_t))
+        src.append('  constexpr int _T_%s = (%d + %d * _V_%s - 1) / (%d * _V_%s);' % (
+            a.name, rows * width, BLOCK, a.name, BLOCK, a.name))
+        src.append('  __shared__ __attribute__((aligned(16))) char _slab_raw_%s[(%d + _V_%s) * sizeof(%s)];' % (
+            a.name, rows * width, a.name, a.store_t))
+        src.append('  %s* _slab_%s = reinterpret_cast<%s*>(_slab_raw_%s);' % (
+            a.store_t, a.name, a.store_t, a.name))
+        src.append('  const %s* _src_%s = _p_%s + _row0 * %d;' % (a.store_t, a.name, a.name, width))
+        src.append('  cupy::Vec<%s, _V_%s> _st_%s[_T_%s];' % (a.store_t, a.name, a.name, a.name))
+    # every load is issued before the first store into the LDS
+    for a in ins:
+        src.append('#pragma unroll')
+        src.append('  for (int _t = 0; _t < _T_%s; ++_t) {' % a.name)
+        src.append('    const int _q = (_t * %d + threadIdx.x) * _V_%s;' % (BLOCK, a.name))
+        src.append('    if (_q + _V_%s <= _count) _st_%s[_t] = cupy::load_vec<%s, _V_%s, %s>(_src_%s + _q);' % (
+            a.name, a.name, a.store_t, a.name, nt, a.name))
+        src.append('  }')
+    for a in ins:
+        src.append('#pragma unroll')
+        src.append('  for (int _t = 0; _t < _T_%s; ++_t) {' % a.name)
+        src.append('    const int _q = (_t * %d + threadIdx.x) * _V_%s;' % (BLOCK, a.name))
+        src.append('    if (_q + _V_%s <= _count) {' % a.name)
+        src.append('      *reinterpret_cast<cupy::Vec<%s, _V_%s>*>(_slab_%s + _q) = _st_%s[_t];' % (
+            a.store_t, a.name, a.name, a.name))
+        src.append('    } else {')
+        src.append('      for (int _k = 0; _k < _V_%s; ++_k) if (_q + _k < _count) _slab_%s[_q + _k] = _src_%s[_q + _k];' % (
+            a.name, a.name, a.name))
+        src.append('    }')
+        src.append('  }')
+    src.append('  __syncthreads();')
+    src.append('  const int _g = threadIdx.x %% %d;' % group)
+    src.append('  for (int _r = threadIdx.x / %d; _r < _nrows; _r += %d) {' % (group, per_pass))
+    src.append('    _type_reduce _s = %s;' % _identity_decl(identity))
+    src.append('    const int _rot = (_r * %d) %% %d;' % (group, width))
+    if width // group <= 32:
+        src.append('#pragma unroll')
+    src.append('    for (int _jq = _g; _jq < %d; _jq += %d) {' % (width, group))
+    src.append('      const int _j = (_jq + _rot >= %d) ? (_jq + _rot - %d) : (_jq + _rot);' % (width, width))
+    src.append('      const IndexT _J = _j;')
+    for a in ins:
+        src.append('      const %s %s(_slab_%s[_r * %d + _j]);' % (a.var_t, a.name, a.name, width))
+    src.append('      _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+    src.append('      _s = REDUCE(_s, _a);')
+    src.append('    }')
+    if group > 1:
+        src.append('    _s = cupy::group_allreduce<%d>(_s, _ReduceOp());' % group)
+        src.append('    if (_g == 0) {')
+    else:
+        src.append('    {')
+    src.append('      const ptrdiff_t _i = _row0 + _r;')
+    src.extend(_finish(args, False, '      '))
+    src.append('    }')
+    src.append('  }')
     src.append('}')
     return '\n'.join(src) + '\n'
 

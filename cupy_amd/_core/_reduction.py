@@ -463,12 +463,77 @@ class _AbstractReductionKernel:
         _launch_plan.launch(rec, fn, (grid, 1, gz), (_cg.BLOCK, 1, 1),
                             _make_packer(fmt), vals, stream_ptr)
 
+    # -- short rows through the LDS -----------------------------------------------------------
+    def _rows_flat_geometry(self, ins, n_out, n_red, so_in, sr):
+        """(lanes per row, rows per workgroup) for the kernel that stages whole
+        rows in the LDS, or None when the rows are not short, not stored back
+        to back, or served as well by a lane group per row."""
+        mode = _tuning.get('rows_flat')
+        if not mode or n_red < 3 or n_out < 4096:
+            return None
+        items = [a.dtype.itemsize for a in ins]
+        if n_red * max(items) > _tuning.get('rows_flat_max_bytes'):
+            return None
+        for a, s_o, s_r in zip(ins, so_in, sr):
+            if s_r != a.dtype.itemsize or s_o != n_red * a.dtype.itemsize:
+                return None
+        if mode == 'auto':
+            # a lane group per row does as well when a row is a whole number
+            # of vectors that fills a power-of-two group of lanes, or three
+            # quarters of one from 384 bytes per row
+            vec = _max_vector_width(items)
+            lanes = (n_red + vec - 1) // vec
+            full = internal.clp2(lanes)
+            if n_red % vec == 0 and (lanes == full or (
+                    lanes * 4 >= full * 3 and n_red * min(items) >= 384)):
+                return None
+        group = min(64, internal.clp2((n_red + 23) // 24))
+        per_pass = _cg.BLOCK // group
+        pass_bytes = per_pass * n_red * sum(items)
+        if pass_bytes > 48 * 1024:
+            return None
+        k = max(1, min(8, (24 * 1024) // pass_bytes))
+        rows = per_pass * k
+        if (n_out + rows - 1) // rows > _max_blocks(_cg.BLOCK):
+            return None
+        return group, rows
+
+    def _launch_rows_flat(self, geometry, in_args, out_args, in_arr_idx, out_arr_idx,
+                          n_out, n_red, so_in, sr, so_out, map_expr, reduce_expr,
+                          post_map_expr, reduce_type, typedefs, device_id, stream_ptr,
+                          rec=None):
+        preamble, _ = self._get_preamble_options()
+        ins = [in_args[i] for i in in_arr_idx]
+        group, rows = geometry
+        rargs = self._rargs(in_args, out_args)
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('rows_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
+        key = ('rows_flat', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
+               post_map_expr, reduce_type, n_red, group, rows, device_id, stream_hint)
+
+        def emit():
+            return self.name, _cg.emit_rows_flat(
+                self.name, rargs, self.identity, map_expr, reduce_expr, post_map_expr,
+                reduce_type, typedefs, preamble, width=n_red, group=group, rows=rows,
+                stream_hint=stream_hint)
+        fn, _, _ = self._compile(key, emit, in_args)
+        vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
+        _launch_plan.launch(
+            rec, fn, ((n_out + rows - 1) // rows, 1, 1), (_cg.BLOCK, 1, 1),
+            _make_packer(self._fast_format(rargs, 'q')), vals, stream_ptr)
+
     # -- rows ---------------------------------------------------------------------------------
     def _launch_rows(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                      so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
                      reduce_type, typedefs, device_id, stream_ptr, rec=None):
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
+        flat = self._rows_flat_geometry(ins, n_out, n_red, so_in, sr)
+        if flat is not None:
+            return self._launch_rows_flat(
+                flat, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red, so_in,
+                sr, so_out, map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                device_id, stream_ptr, rec)
         cus = _device.get_compute_units(device_id)
         vec = _max_vector_width([a.dtype.itemsize for a in ins])
         while vec > 1:

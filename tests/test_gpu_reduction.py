@@ -356,3 +356,47 @@ def test_middle_axis_of_four_dimensions_and_broadcast_batches():
     k = cp.ReductionKernel('T x, T y', 'T z', 'x * y', 'a + b', 'z = a', '0', 'dot_middle')
     y = shaped_random((4, 6, 50, 33), 'int32', 23)
     assert_exact(k(dx, cp.asarray(y), axis=2).get(), (x * y).sum(axis=2, dtype=np.int32))
+
+
+@pytest.mark.parametrize('width', [3, 5, 7, 10, 17, 24, 33, 48, 67, 100, 129, 255])
+@pytest.mark.parametrize('dtype', ['int8', 'float16', 'float32', 'float64'])
+def test_short_rows_stored_back_to_back(width, dtype):
+    for n_rows in (4096, 5000, 70001):
+        x = shaped_random((n_rows, width), dtype, 41)
+        dx = cp.asarray(x)
+        if np.dtype(dtype).kind == 'f':
+            got = dx.sum(axis=1).get()
+            want = x.astype(np.float64).sum(axis=1)
+            tol = {'float16': 2e-3, 'float32': 1e-5, 'float64': 1e-12}[dtype]
+            scale = np.abs(x.astype(np.float64)).sum(axis=1)
+            assert got.dtype == np.dtype(dtype)
+            assert np.all(np.abs(got - want) <= tol * np.maximum(scale, 1))
+        else:
+            assert_exact(dx.sum(axis=1).get(), x.sum(axis=1))
+        assert_exact(dx.max(axis=1).get(), x.max(axis=1))
+        assert_exact(dx.argmin(axis=1).get(), x.argmin(axis=1))
+        assert_exact(dx.argmax(axis=1).get(), x.argmax(axis=1))
+    # rows that start anywhere, and a strided output
+    lo, hi = width + 1, width + 1 + (n_rows - 2) * width
+    v, dv = x.reshape(-1)[lo:hi].reshape(-1, width), dx.reshape(-1)[lo:hi].reshape(-1, width)
+    assert_exact(dv.min(axis=1).get(), v.min(axis=1))
+    out = cp.zeros((v.shape[0], 2), dx.dtype)
+    dv.max(axis=1, out=out[:, 1])
+    assert_exact(out.get()[:, 1], v.max(axis=1))
+    assert not out.get()[:, 0].any()
+
+
+def test_short_rows_with_two_inputs_and_mixed_types():
+    k = cp.ReductionKernel('T x, S y', 'float32 z', '(float)x * (float)y', 'a + b', 'z = a', '0',
+                           'dot_short_rows')
+    x = shaped_random((9000, 11), 'float32', 42)
+    y = shaped_random((9000, 11), 'int8', 43)
+    got = k(cp.asarray(x), cp.asarray(y), axis=1).get()
+    want = (x.astype(np.float64) * y).sum(axis=1)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-3)
+    nan = x.copy()
+    nan[::7, 3] = np.nan
+    assert_exact(cp.asarray(nan).argmax(axis=1).get(), nan.argmax(axis=1))
+    assert_exact(cp.asarray(nan).max(axis=1).get(), nan.max(axis=1))
+    np.testing.assert_allclose(cp.nansum(cp.asarray(nan), axis=1).get(), np.nansum(nan, axis=1),
+                               rtol=1e-5, atol=1e-4)
