@@ -25,6 +25,12 @@ template <typename T> __device__ __forceinline__ bool _mm_isnan(T) { return fals
 template <> __device__ __forceinline__ bool _mm_isnan<float>(float x) { return x != x; }
 template <> __device__ __forceinline__ bool _mm_isnan<double>(double x) { return x != x; }
 template <> __device__ __forceinline__ bool _mm_isnan<float16>(float16 x) { return x.isnan(); }
+template <> __device__ __forceinline__ bool _mm_isnan<complex<float> >(complex<float> x) {
+  return (x.re != x.re) | (x.im != x.im);
+}
+template <> __device__ __forceinline__ bool _mm_isnan<complex<double> >(complex<double> x) {
+  return (x.re != x.re) | (x.im != x.im);
+}
 
 // kMax: larger values win, otherwise smaller ones; kNan: NaN wins over numbers.
 // `index == -1` marks "no element yet".  Written with selects on the members
@@ -176,19 +182,28 @@ template <typename T> struct _mm_is_float { static const bool value = false; };
 template <> struct _mm_is_float<float> { static const bool value = true; };
 template <> struct _mm_is_float<double> { static const bool value = true; };
 template <> struct _mm_is_float<float16> { static const bool value = true; };
-template <typename T> __device__ __forceinline__ T _mm_extreme(bool lowest) {
-  if (_mm_is_float<T>::value) return lowest ? T(-CUDART_INF_F) : T(CUDART_INF_F);
-  if (cupy::is_same<T, bool>::value) return T(!lowest);
-  if (T(-1) < T(0)) {
-    const unsigned long long top = 1ull << (8 * sizeof(T) - 1);
-    return static_cast<T>(lowest ? top : ~top);
+template <typename T> struct _mm_limits {
+  static __device__ __forceinline__ T get(bool lowest) {
+    if (_mm_is_float<T>::value) return lowest ? T(-CUDART_INF_F) : T(CUDART_INF_F);
+    if (cupy::is_same<T, bool>::value) return T(!lowest);
+    if (T(-1) < T(0)) {
+      const unsigned long long top = 1ull << (8 * sizeof(T) - 1);
+      return static_cast<T>(lowest ? top : ~top);
+    }
+    return lowest ? T(0) : static_cast<T>(~0ull);
   }
-  return lowest ? T(0) : static_cast<T>(~0ull);
-}
+};
+// complex numbers are ordered by real part, then by imaginary part
+template <typename U> struct _mm_limits<complex<U> > {
+  static __device__ __forceinline__ complex<U> get(bool lowest) {
+    const U inf = lowest ? U(-CUDART_INF_F) : U(CUDART_INF_F);
+    return complex<U>(inf, inf);
+  }
+};
 template <typename T, bool kMax>
 struct mm_val {
   T v;
-  __device__ __forceinline__ mm_val() : v(_mm_extreme<T>(kMax)) {}
+  __device__ __forceinline__ mm_val() : v(_mm_limits<T>::get(kMax)) {}
   __device__ __forceinline__ explicit mm_val(T x) : v(x) {}
 };
 template <bool kNan, typename T, bool kMax>
@@ -207,7 +222,9 @@ _amin = create_reduction_func(
     _int_sigs + (
         ('e->e', (None, 'mm_pick<true>(a, b)', None, None)),
         ('f->f', (None, 'mm_pick<true>(a, b)', None, None)),
-        ('d->d', (None, 'mm_pick<true>(a, b)', None, None))),
+        ('d->d', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('F->F', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('D->D', (None, 'mm_pick<true>(a, b)', None, None))),
     ('mm_val<type_in0_raw, false>(in0)', 'mm_pick<false>(a, b)', 'out0 = a.v',
      'mm_val<type_in0_raw, false>'),
     None, _extremum_preamble)
@@ -217,13 +234,15 @@ _amax = create_reduction_func(
     _int_sigs + (
         ('e->e', (None, 'mm_pick<true>(a, b)', None, None)),
         ('f->f', (None, 'mm_pick<true>(a, b)', None, None)),
-        ('d->d', (None, 'mm_pick<true>(a, b)', None, None))),
+        ('d->d', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('F->F', (None, 'mm_pick<true>(a, b)', None, None)),
+        ('D->D', (None, 'mm_pick<true>(a, b)', None, None))),
     ('mm_val<type_in0_raw, true>(in0)', 'mm_pick<false>(a, b)', 'out0 = a.v',
      'mm_val<type_in0_raw, true>'),
     None, _extremum_preamble)
 
 _arg_sigs = tuple('{}->{}'.format(d, r) for r in 'qlihb' for d in '?bBhHiIlLqQ') + (
-    'e->q', 'f->q', 'd->q')
+    'e->q', 'f->q', 'd->q', 'F->q', 'D->q')
 
 _argmin = create_reduction_func(
     'cupy_argmin', _arg_sigs,
@@ -254,7 +273,7 @@ def _ndarray_argmin(self, axis, out, dtype, keepdims):
     return _argmin(self, axis=axis, out=out, dtype=dtype, keepdims=keepdims)
 
 
-_float_sigs = ('e->e', 'f->f', 'd->d')
+_float_sigs = ('e->e', 'f->f', 'd->d', 'F->F', 'D->D')
 
 # NaNs are skipped; a slice of NaNs only gives NaN
 # (cupy/_core/_routines_statistics.pyx:307-326)
@@ -272,7 +291,7 @@ nanmax = create_reduction_func(
 
 # index -1 = "no element": NaNs never take part; a slice of NaNs only gives -1
 # (:365-391)
-_nanarg_sigs = tuple('%s->q' % c for c in '?BhHiIlLqQefd')
+_nanarg_sigs = tuple('%s->q' % c for c in '?BhHiIlLqQefdFD')
 
 _nanargmin_func = create_reduction_func(
     'cupy_nanargmin', _nanarg_sigs,

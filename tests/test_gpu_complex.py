@@ -275,3 +275,34 @@ def test_variance_of_complex_is_real(dtype):
             np.testing.assert_allclose(got.get(), want, rtol=20 * rtol)
             np.testing.assert_allclose(d.std(axis=axis, ddof=ddof).get(),
                                        a.std(axis=axis, ddof=ddof), rtol=20 * rtol)
+
+
+@pytest.mark.parametrize('dtype', ['complex64', 'complex128'])
+def test_extrema_order_by_real_then_imaginary_part(dtype):
+    rng = np.random.default_rng(51)
+    # few distinct real parts, so that the imaginary parts decide often
+    x = (rng.integers(-3, 4, (300, 71)) + 1j * rng.integers(-50, 50, (300, 71))).astype(dtype)
+    dx = cp.asarray(x)
+    for axis in (None, 0, 1):
+        assert_exact(dx.max(axis=axis).get(), x.max(axis=axis))
+        assert_exact(dx.min(axis=axis).get(), x.min(axis=axis))
+        assert_exact(dx.argmax(axis=axis).get(), x.argmax(axis=axis))
+        assert_exact(dx.argmin(axis=axis).get(), x.argmin(axis=axis))
+    flat = x.reshape(-1)[:70001 // 4]
+    assert_exact(cp.asarray(flat).argmax().get(), flat.argmax())
+    y = x.copy()
+    y[5, 7] = complex(np.nan, 1)
+    y[9, 3] = complex(2, np.nan)
+    y[200, 70] = complex(np.nan, np.nan)
+    dy = cp.asarray(y)
+    for axis in (None, 0, 1):
+        got, want = dy.max(axis=axis).get(), y.max(axis=axis)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+        assert_exact(dy.argmax(axis=axis).get(), y.argmax(axis=axis))
+        assert_exact(dy.argmin(axis=axis).get(), y.argmin(axis=axis))
+        with np.errstate(all='ignore'):
+            assert_exact(cp.nanmax(dy, axis=axis).get(), np.nanmax(y, axis=axis))
+            assert_exact(cp.nanmin(dy, axis=axis).get(), np.nanmin(y, axis=axis))
+            assert_exact(cp.nanargmax(dy, axis=axis).get(), np.nanargmax(y, axis=axis))
+            assert_exact(cp.nanargmin(dy, axis=axis).get(), np.nanargmin(y, axis=axis))
