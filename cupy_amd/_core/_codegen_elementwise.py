@@ -150,20 +150,33 @@ def _element_code(operands, operation, load_expr, store_stmt, indent):
 
 def emit_flat(name, operands, operation, typedefs='', preamble='',
               loop_prep='', after_loop='', vec=4, unroll=1, idx64=False,
-              bcast=(), stream_hint=True, block=BLOCK):
+              bcast=(), stream_hint=True, block=BLOCK, partial=None):
     """Kernel for operands that are all contiguous.
 
     ``bcast`` names array operands that hold a single element broadcast over
     the whole index space.  Trailing parameters of the kernel: the array
     pointers / scalars / raw arrays in operand order, then ``_n`` (element
     count) and, when the body uses it, ``_ind``.
+
+    ``partial`` maps names of input arrays to 'row' or 'col' when the index
+    space is a matrix of ``_nc`` columns stored row after row: a 'row' operand
+    holds a value per row, a 'col' operand a value per column, ``_sb_<name>``
+    elements apart ('col1': one element apart).  The other arrays are still walked with whole vectors;
+    row and column of an element come from one division per vector.
+    ``_nc`` and the ``_sb_`` strides follow ``_n``.
     """
+    partial = partial or {}
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     arrays = [op for op in operands if op.kind == 'array']
-    iter_arrays = [op for op in arrays if op.name not in bcast]
+    iter_arrays = [op for op in arrays if op.name not in bcast and op.name not in partial]
+    part_ops = [op for op in arrays if op.name in partial]
+    for op in part_ops:
+        assert not op.is_out
     needs_ind = any(op.kind == 'indexer' for op in operands)
     params = ', '.join([_param_decl(op) for op in operands if op.kind != 'indexer']
                        + ['const %s _n' % idx_t]
+                       + (['const %s _nc' % idx_t] if partial else [])
+                       + ['const %s _sb_%s' % (idx_t, op.name) for op in part_ops]
                        + [_param_decl(op) for op in operands if op.kind == 'indexer'])
     _nt_l, _nt_s = stream_hint if isinstance(stream_hint, tuple) else (stream_hint, stream_hint)
     ntl = 'true' if _nt_l else 'false'
@@ -179,10 +192,57 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
                     op.store_t, op.name, op.name))
         return '\n'.join(out)
 
+    def part_expr(op):
+        return '_p_%s[(ptrdiff_t)%s * _sb_%s]' % (
+            op.name, '_rk' if partial[op.name] == 'row' else '_ck', op.name)
+
+    row_ops = [op for op in part_ops if partial[op.name] == 'row']
+    col_ops = [op for op in part_ops if partial[op.name] != 'row']
+
+    def rc_init(pad, start, whole_vector=True):
+        """Row and column of element ``start``; for a whole vector also the
+        values of the per-row operands (reloaded when the vector runs into the
+        next row) and a vector of the per-column operands (one load when the
+        vector lies within a row and the operand is stored densely)."""
+        if not partial:
+            return []
+        out = ['%s%s _rk = (%s) / _nc;' % (pad, idx_t, start),
+               '%s%s _ck = (%s) - _rk * _nc;' % (pad, idx_t, start)]
+        if not whole_vector:
+            return out
+        for op in row_ops:
+            out.append('%s%s _pr_%s = %s;' % (pad, op.store_t, op.name, part_expr(op)))
+        for op in col_ops:
+            out.append('%scupy::Vec<%s, %d> _pc_%s;' % (pad, op.store_t, vec, op.name))
+            gather = ('{ %s _cc = _ck;\n%s#pragma unroll\n%s  for (int _k = 0; _k < %d; ++_k) { '
+                      '_pc_%s.v[_k] = _p_%s[(ptrdiff_t)_cc * _sb_%s]; if (++_cc == _nc) _cc = 0; } }' % (
+                          idx_t, pad, pad, vec, op.name, op.name, op.name))
+            if partial[op.name] == 'col1':
+                out.append('%sif (_ck + %d <= _nc) _pc_%s = cupy::load_vec<%s, %d, false>(_p_%s + _ck);' % (
+                    pad, vec, op.name, op.store_t, vec, op.name))
+                out.append('%selse %s' % (pad, gather))
+            else:
+                out.append('%s%s' % (pad, gather))
+        return out
+
+    def rc_step(pad):
+        if not row_ops:
+            return []
+        reload = ' '.join('_pr_%s = %s;' % (op.name, part_expr(op)) for op in row_ops)
+        return ['%sif (_k + 1 < %d) { if (++_ck == _nc) { _ck = 0; ++_rk; %s } }' % (
+            pad, vec, reload)]
+
+    def part_value(op):
+        if partial[op.name] == 'row':
+            return '_pr_%s' % op.name
+        return '_pc_%s.v[_k]' % op.name
+
     def vec_load_expr(suffix):
         def f(op):
             if op.name in bcast:
                 return '_b_%s' % op.name
+            if op.name in partial:
+                return part_value(op)
             return '_l_%s%s.v[_k]' % (op.name, suffix)
         return f
 
@@ -214,6 +274,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
         for u in range(unroll):
             body.append('      {')
             body.append('        const %s _base = (_v0 + %d) * %d;' % (idx_t, u * block, vec))
+            body.extend(rc_init('        ', '_base'))
             body.append('#pragma unroll')
             body.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
             if use_i or set_ind:
@@ -221,6 +282,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
             body.append(_element_code(
                 operands, operation, vec_load_expr('_%d' % u),
                 vec_store_stmt('_%d' % u), 10))
+            body.extend(rc_step('          '))
             body.append('        }')
             for op in iter_arrays:
                 if op.is_out:
@@ -244,12 +306,14 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
                                              op.store_t, vec, ntl, op.name))
         else:
             body.append('%scupy::Vec<%s, %d> _l_%s;' % (pad, op.store_t, vec, op.name))
+    body.extend(rc_init(pad, '_base'))
     body.append('#pragma unroll')
     body.append('%sfor (int _k = 0; _k < %d; ++_k) {' % (pad, vec))
     if use_i or set_ind:
         body.append('%s  const ptrdiff_t i = _base + _k; %s' % (pad, set_ind))
     body.append(_element_code(operands, operation, vec_load_expr(''),
                               vec_store_stmt(''), inner_pad + 2))
+    body.extend(rc_step(pad + '  '))
     body.append('%s}' % pad)
     for op in iter_arrays:
         if op.is_out:
@@ -263,6 +327,8 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
     def tail_load(op):
         if op.name in bcast:
             return '_b_%s' % op.name
+        if op.name in partial:
+            return part_expr(op)
         return '_p_%s[_t]' % op.name
 
     def tail_store(op, value):
@@ -273,6 +339,7 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
                 '_t += (%s)gridDim.x * %d) {' % (idx_t, vec, idx_t, block, idx_t, block))
     if use_i or set_ind:
         tail.append('    const ptrdiff_t i = _t; %s' % set_ind)
+    tail.extend(rc_init('    ', '_t', whole_vector=False))
     tail.append(_element_code(operands, operation, tail_load, tail_store, 4))
     tail.append('  }')
 
@@ -342,6 +409,117 @@ def emit_generic(name, operands, operation, typedefs='', preamble='',
     src.append('  CUPY_FOR(i, _ind.size()) {')
     src.append('    _ind.set(i);')
     src.extend(lines)
+    src.append('  }')
+    src.append('  %s;' % after_loop)
+    src.append('}')
+    return '\n'.join(src) + '\n'
+
+
+def emit_rows2d(name, operands, operation, typedefs='', preamble='',
+                loop_prep='', after_loop='', kinds=None, vec=4, idx64=False,
+                stream_hint=True, block=BLOCK):
+    """Kernel for a matrix problem (rows r, columns c) none of whose arrays
+    runs against the columns: every row is walked in vectors of ``vec``
+    columns that start at column 0, 1 * vec, ... of that row, so that no
+    vector reaches into the next row and rows may be spaced in any way.
+    Consecutive lanes take consecutive vectors, across row ends.
+
+    ``kinds[name]`` is
+      'R'    unit stride along columns, any stride along rows: vector access;
+      'row'  zero stride along columns: one value per row;
+      'col1' zero stride along rows, unit stride along columns: one vector
+             load per vector of the problem;
+      'S'    anything else (every second column, columns backwards, ...):
+             element-wise access.
+    The last ``_nc % vec`` columns of a row are handled element by element by
+    the lane that owns them.  Kernel parameters after the operands:
+    ``_nr, _nc``, then per array its row stride and column stride in elements.
+    """
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    arrays = [op for op in operands if op.kind == 'array']
+    _nt_l, _nt_s = stream_hint if isinstance(stream_hint, tuple) else (stream_hint, stream_hint)
+    ntl = 'true' if _nt_l else 'false'
+    nts = 'true' if _nt_s else 'false'
+    use_i = uses_identifier(operation, 'i')
+    parts = [_param_decl(op) for op in operands if op.kind != 'indexer']
+    parts += ['const %s _nr' % idx_t, 'const %s _nc' % idx_t]
+    for op in arrays:
+        parts += ['const %s _sr_%s' % (idx_t, op.name), 'const %s _sc_%s' % (idx_t, op.name)]
+    assert not any(op.kind == 'indexer' for op in operands)
+    params = ', '.join(parts)
+
+    def addr(op, c):
+        return '(_p_%s + (ptrdiff_t)_rk * _sr_%s + (ptrdiff_t)(%s) * _sc_%s)' % (
+            op.name, op.name, c, op.name)
+
+    src = [_header(typedefs, preamble)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        block, name, params))
+    src.append('  %s;' % loop_prep)
+    src.append('  const %s _nvr = (_nc + %d) / %d;' % (idx_t, vec - 1, vec))
+    src.append('  const %s _nv = _nr * _nvr;' % idx_t)
+    src.append('  for (%s _v = (%s)blockIdx.x * %d + threadIdx.x; _v < _nv; '
+               '_v += (%s)gridDim.x * %d) {' % (idx_t, idx_t, block, idx_t, block))
+    src.append('    const %s _rk = _v / _nvr;' % idx_t)
+    src.append('    const %s _ck = (_v - _rk * _nvr) * %d;' % (idx_t, vec))
+    src.append('    if (_ck + %d <= _nc) {' % vec)
+    for op in arrays:
+        k = kinds[op.name]
+        reads = (not op.is_out) or op.read_out
+        if k in ('R', 'col1'):
+            if reads:
+                src.append('      cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
+                    op.store_t, vec, op.name, op.store_t, vec,
+                    ntl if k == 'R' else 'false', addr(op, '_ck')))
+            else:
+                src.append('      cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+        elif k == 'row':
+            if reads:
+                src.append('      const %s _b_%s = *%s;' % (op.store_t, op.name, addr(op, '0')))
+        else:
+            src.append('      cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+            if reads:
+                src.append('#pragma unroll')
+                src.append('      for (int _k = 0; _k < %d; ++_k) _l_%s.v[_k] = *%s;' % (
+                    vec, op.name, addr(op, '_ck + _k')))
+
+    def full_load(op):
+        if kinds[op.name] == 'row':
+            return '_b_%s' % op.name
+        return '_l_%s.v[_k]' % op.name
+
+    def full_store(op, value):
+        return '_l_%s.v[_k] = %s;' % (op.name, value)
+
+    src.append('#pragma unroll')
+    src.append('      for (int _k = 0; _k < %d; ++_k) {' % vec)
+    if use_i:
+        src.append('        const ptrdiff_t i = (ptrdiff_t)_rk * _nc + _ck + _k;')
+    src.append(_element_code(operands, operation, full_load, full_store, 8))
+    src.append('      }')
+    for op in arrays:
+        if op.is_out:
+            if kinds[op.name] == 'R':
+                src.append('      cupy::store_vec<%s, %d, %s>(%s, _l_%s);' % (
+                    op.store_t, vec, nts, addr(op, '_ck'), op.name))
+            else:
+                src.append('#pragma unroll')
+                src.append('      for (int _k = 0; _k < %d; ++_k) *%s = _l_%s.v[_k];' % (
+                    vec, addr(op, '_ck + _k'), op.name))
+    src.append('    } else {')
+
+    def edge_load(op):
+        return '(*%s)' % addr(op, '_ck + _k')
+
+    def edge_store(op, value):
+        return '*%s = %s;' % (addr(op, '_ck + _k'), value)
+
+    src.append('      for (int _k = 0; _k < (int)(_nc - _ck); ++_k) {')
+    if use_i:
+        src.append('        const ptrdiff_t i = (ptrdiff_t)_rk * _nc + _ck + _k;')
+    src.append(_element_code(operands, operation, edge_load, edge_store, 8))
+    src.append('      }')
+    src.append('    }')
     src.append('  }')
     src.append('  %s;' % after_loop)
     src.append('}')

@@ -414,7 +414,26 @@ class _ElementwisePlanner:
                         break
                 if ok:
                     mode = 'flat'
+                elif not self._uses_ind:
+                    # one axis with a stride: a matrix of one row
+                    plan = self._plan_rows2d(
+                        arrays, (1, cshape[0]), [(0, cs[0]) for cs in cstrides], args, nin)
+                    if plan is not None and plan[0][0] == 1:
+                        return self._launch_rows2d(
+                            dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
+                            force_read_out, stream_ptr, kernel_name, rec)
             elif nd == 2 and not self._uses_ind:
+                part = self._plan_flat_bcast(arrays, cshape, cstrides, args, nin)
+                if part is not None:
+                    return self._launch_flat(
+                        dev_id, args, nin, arrays, cstrides, size, var_types, typedefs,
+                        casts, force_read_out, stream_ptr, kernel_name, rec,
+                        partial=part, nc=cshape[1])
+                plan = self._plan_rows2d(arrays, cshape, cstrides, args, nin)
+                if plan is not None:
+                    return self._launch_rows2d(
+                        dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
+                        force_read_out, stream_ptr, kernel_name, rec)
                 mode = self._classify_2d(arrays, cstrides, args, nin)
             elif nd in (3, 4) and not self._uses_ind and not self._uses_i:
                 plan = self._plan_batched(arrays, cshape, cstrides, args, nin)
@@ -440,9 +459,133 @@ class _ElementwisePlanner:
             dev_id, args, nin, shape, var_types, typedefs, casts, force_read_out,
             stream_ptr, block_size or 128, kernel_name, rec)
 
+    def _plan_flat_bcast(self, arrays, cshape, cstrides, args, nin):
+        """Matrix problem whose full-size arrays are all stored row after row
+        without gaps and whose other arrays hold a value per row or a value per
+        column: {parameter name: ('row' | 'col', byte stride)} for the latter,
+        None when the problem is not of this kind."""
+        if not _tuning.get('flat_bcast'):
+            return None
+        nr, nc = cshape
+        names = [p.name for a, p in zip(args, self.params)
+                 if isinstance(a, ndarray) and not p.raw]
+        outs = args[nin:]
+        part = {}
+        n_full = 0
+        for a, cs, nm in zip(arrays, cstrides, names):
+            item = a.dtype.itemsize
+            if cs[1] == item and cs[0] == nc * item:
+                n_full += 1
+                continue
+            if any(a is o for o in outs) or cs[0] % item or cs[1] % item:
+                return None
+            if cs[1] == 0:
+                kind = ('row', cs[0])
+            elif cs[0] == 0:
+                kind = ('col1' if cs[1] == item else 'col', cs[1])
+            else:
+                return None
+            if part.get(nm, kind) != kind:
+                return None       # the same parameter name twice: not expected
+            part[nm] = kind
+        if not n_full or not part:
+            return None
+        return part
+
+    def _plan_rows2d(self, arrays, cshape, cstrides, args, nin):
+        """Matrix problem in which no array runs against the columns: every
+        output has unit stride along the columns, every input unit, zero or a
+        small stride.  Returns (shape, strides per array, kinds per parameter
+        name), with the two axes swapped when that is what makes it fit (all
+        arrays stored column after column), or None."""
+        if not _tuning.get('rows2d'):
+            return None
+        names = [p.name for a, p in zip(args, self.params)
+                 if isinstance(a, ndarray) and not p.raw]
+        outs = args[nin:]
+        for swap in ((False, True) if not self._uses_i else (False,)):
+            kinds = {}
+            ok = True
+            for a, cs, nm in zip(arrays, cstrides, names):
+                sr, sc = (cs[1], cs[0]) if swap else cs
+                item = a.dtype.itemsize
+                is_out = any(a is o for o in outs)
+                if sr % item or sc % item:
+                    ok = False
+                elif sc == item:
+                    kind = 'R'
+                elif is_out:
+                    ok = False
+                elif sc == 0:
+                    kind = 'row'
+                elif sr == 0 and sc == item:
+                    kind = 'col1'
+                elif abs(sc) <= 4 * item and (sr == 0 or abs(sr) >= abs(sc)):
+                    kind = 'S'
+                else:
+                    ok = False
+                if not ok or kinds.get(nm, kind) != kind:
+                    ok = False
+                    break
+                kinds[nm] = kind
+            if ok and any(k == 'R' for k in kinds.values()):
+                if swap:
+                    return ((cshape[1], cshape[0]), [(cs[1], cs[0]) for cs in cstrides], kinds)
+                return cshape, cstrides, kinds
+        return None
+
+    def _launch_rows2d(self, dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
+                       force_read_out, stream_ptr, kernel_name, rec):
+        (nr, nc), cstrides, kinds = plan
+        itemsizes = [a.dtype.itemsize for a in arrays]
+        vec = max(1, 16 // max(itemsizes))
+        span = max(abs(cs[0]) * nr + abs(cs[1]) * nc for cs in cstrides)
+        nvr = (nc + vec - 1) // vec
+        idx64 = span > _INT32_MAX or nr * nvr * vec > _INT32_MAX - (1 << 24)
+        operands = self._make_operands(args, nin, var_types, casts, force_read_out)
+        light = [n for n, k in kinds.items() if k in ('row', 'col1')]
+        in_bytes, out_bytes = self._traffic(args, nin, light)
+        stream_hint = _tuning.stream_policy(_tuning.get('tiled_stream'), in_bytes, out_bytes)
+        block = 256
+        key = ('rows2d', tuple(o.key() for o in operands), typedefs, vec, idx64,
+               tuple(sorted(kinds.items())), dev_id, stream_hint, block)
+        entry = self._memo.get(key)
+        if entry is None:
+            name = kernel_name or self.name
+            code = _cg.emit_rows2d(
+                name, operands, self.operation, typedefs, self.preamble,
+                self.loop_prep, self.after_loop, kinds=kinds, vec=vec, idx64=idx64,
+                stream_hint=stream_hint, block=block)
+            fn = compiler.compile_with_cache(code, self.options).get_function(name)
+            ic = 'q' if idx64 else 'i'
+            fmt = ['@']
+            for o in operands:
+                if o.kind == 'array':
+                    fmt.append('P')
+                elif o.kind == 'raw':
+                    fmt.append('P' + 'q' * (1 + 2 * o.ndim))
+                elif o.kind == 'scalar':
+                    fmt.append(_scalar_struct_code(o.store_t))
+            fmt.append(ic * (2 + 2 * len(arrays)))
+            entry = (fn, _make_packer(fmt), code)
+            with self._lock:
+                entry = self._memo.setdefault(key, entry)
+            self._remember_code(args, entry[2])
+        fn, packer, _ = entry
+        block_args = self._flat_values(args)
+        block_args.const(nr, nc)
+        for a, cs in zip(arrays, cstrides):
+            item = a.dtype.itemsize
+            block_args.const(cs[0] // item, cs[1] // item)
+        grid = max(1, min((nr * nvr + block - 1) // block,
+                          _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu')) * 4))
+        _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
+                            stream_ptr)
+
     # -- flat ---------------------------------------------------------------------------
     def _launch_flat(self, dev_id, args, nin, arrays, cstrides, size, var_types,
-                     typedefs, casts, force_read_out, stream_ptr, kernel_name, rec):
+                     typedefs, casts, force_read_out, stream_ptr, kernel_name, rec,
+                     partial=None, nc=None):
         params = self.params
         bcast = []
         itemsizes = []
@@ -451,6 +594,8 @@ class _ElementwisePlanner:
             if isinstance(a, ndarray) and not p.raw:
                 cs = cstrides[ai]
                 ai += 1
+                if partial and p.name in partial:
+                    continue
                 if size > 1 and (len(cs) == 1 and cs[0] == 0):
                     bcast.append(p.name)
                 else:
@@ -466,7 +611,7 @@ class _ElementwisePlanner:
         ai = 0
         for a, p in zip(args, params):
             if isinstance(a, ndarray) and not p.raw:
-                if p.name not in bcast:
+                if p.name not in bcast and not (partial and p.name in partial):
                     while vec > 1 and not _aligned(
                             a.data.ptr, min(16, vec * a.dtype.itemsize)):
                         vec //= 2
@@ -478,7 +623,7 @@ class _ElementwisePlanner:
         if mixed and vec > 1:
             unroll = _tuning.get('flat_mixed_unroll') if len(itemsizes) <= 2 else 1
         block = _tuning.get('flat_block')
-        in_bytes, out_bytes = self._traffic(args, nin, bcast)
+        in_bytes, out_bytes = self._traffic(args, nin, bcast + list(partial or ()))
         # nothing streams in (a fill): full-size workgroups and four times the
         # usual grid, so that a thread stores a few vectors only (2^28 float32:
         # 197 -> 174 us)
@@ -493,17 +638,20 @@ class _ElementwisePlanner:
         if self._uses_ind:
             operands.append(_cg.Operand('indexer', '_ind', '', ndim=1,
                                         index_32=not idx64))
+        part_kinds = tuple(sorted((n, k[0]) for n, k in partial.items())) if partial else ()
         key = ('flat', tuple(o.key() for o in operands), typedefs, vec, unroll,
-               idx64, tuple(bcast), dev_id, block, stream_hint)
+               idx64, tuple(bcast), dev_id, block, stream_hint, part_kinds)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
             code = _cg.emit_flat(
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, vec=vec, unroll=unroll,
-                idx64=idx64, bcast=tuple(bcast), stream_hint=stream_hint, block=block)
+                idx64=idx64, bcast=tuple(bcast), stream_hint=stream_hint, block=block,
+                partial=dict(part_kinds))
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
-            fmt = self._arg_format(operands, 'q' if idx64 else 'i', flat=True)
+            fmt = self._arg_format(operands, 'q' if idx64 else 'i', flat=True,
+                                   extra=(1 + len(part_kinds)) if partial else 0)
             entry = (fn, _make_packer(fmt), code)
             with self._lock:
                 entry = self._memo.setdefault(key, entry)
@@ -511,6 +659,11 @@ class _ElementwisePlanner:
         fn, packer, _ = entry
         block_args = self._flat_values(args)
         block_args.const(size)
+        if partial:
+            block_args.const(nc)
+            for a, p in zip(args, params):
+                if isinstance(a, ndarray) and not p.raw and p.name in partial:
+                    block_args.const(partial[p.name][1] // a.dtype.itemsize)
         if self._uses_ind:
             block_args.const(size, size, 0)
         nvec = size // vec
@@ -556,8 +709,9 @@ class _ElementwisePlanner:
                 out.scalar(ref, a)
         return out
 
-    def _arg_format(self, operands, idx_code, flat):
-        """struct format of the kernel's argument block."""
+    def _arg_format(self, operands, idx_code, flat, extra=0):
+        """struct format of the kernel's argument block (``extra`` more index
+        values after the element count)."""
         fmt = ['@']
         for o in operands:
             if o.kind == 'array':
@@ -566,7 +720,7 @@ class _ElementwisePlanner:
                 fmt.append('P' + 'q' * (1 + 2 * o.ndim))
             elif o.kind == 'scalar':
                 fmt.append(_scalar_struct_code(o.store_t))
-        fmt.append(idx_code)
+        fmt.append(idx_code * (1 + extra))
         for o in operands:
             if o.kind == 'indexer':
                 fmt.append('q' * (1 + 2 * o.ndim))

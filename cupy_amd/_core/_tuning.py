@@ -15,6 +15,12 @@ _params = {
     'flat_block': 1024,         # threads per workgroup
     'flat_unroll': 1,           # vectors per thread per trip
     'flat_blocks_per_cu': 64,   # grid cap, in workgroups per CU
+    # matrices stored row after row combined with a value per row or per column
+    # stay in the flat kernel (row and column by one division per vector)
+    'flat_bcast': True,
+    # matrices whose rows are spaced apart (windows, every second row or
+    # column) are walked row by row in vectors instead of in square tiles
+    'rows2d': True,
     # Operands of different widths: the widest moves 16 bytes per access
     # ('wide'; the narrower ones then move less, but consecutive lanes stay on
     # consecutive addresses in every operand) or the narrowest does ('narrow';

@@ -162,3 +162,85 @@ def test_array_that_ends_with_its_allocation():
             assert_exact((v + v).get(), hv + hv)
             np.testing.assert_allclose(v.sum().get(), hv.sum(dtype=np.float64), rtol=1e-5, atol=1e-3)
             assert_exact(v.argmax().get(), hv.argmax())
+
+
+@pytest.mark.parametrize('shape', [(70001, 3), (5000, 1000), (3, 70001), (4099, 67), (2, 2), (1000, 1),
+                                   (129, 4099), (100000, 2)])
+def test_matrix_with_a_value_per_row_or_per_column(shape):
+    nr, nc = shape
+    x = shaped_random(shape, 'float32', 61)
+    row = shaped_random((1, nc), 'float32', 62)
+    col = shaped_random((nr, 1), 'float16', 63)
+    one = shaped_random((1, 1), 'float64', 64)
+    dx, drow, dcol, done = map(cp.asarray, (x, row, col, one))
+    assert_exact((dx + drow).get(), x + row)
+    assert_exact((dx * dcol).get(), x * col)
+    assert_exact(((dx - drow) * dcol).get(), (x - row) * col)
+    assert_exact((drow - dx).get(), row - x)
+    assert_exact((dx + done).get(), x + one)
+    out = cp.zeros(shape, 'float32')
+    cp.add(drow, dcol, out)
+    assert_exact(out.get(), (row + col).astype(np.float32))
+    assert_exact(cp.where(dx > drow, dx, dcol).get(), np.where(x > row, x, col))
+    # 1-d row vector (broadcast from the left), strided column vector
+    assert_exact((dx + drow[0]).get(), x + row[0])
+    wide = shaped_random((nr, 3), 'float32', 65)
+    assert_exact((dx * cp.asarray(wide)[:, 1:2]).get(), x * wide[:, 1:2])
+    assert_exact((dx * cp.asarray(wide.T.copy())[1][:, None]).get(), x * wide[:, 1:2])
+    long_row = shaped_random((1, 2 * nc), 'float32', 66)
+    assert_exact((dx - cp.asarray(long_row)[:, ::2]).get(), x - long_row[:, ::2])
+    # the element index of a user kernel runs over the matrix row after row
+    k = cp.ElementwiseKernel('T x, T r', 'T y, int64 at', 'y = x + r; at = i', 'row_add_with_index')
+    y, at = k(dx, drow)
+    assert_exact(y.get(), x + row)
+    assert_exact(at.get(), np.arange(nr * nc, dtype=np.int64).reshape(shape))
+
+
+@pytest.mark.parametrize('dtype', ['int8', 'float16', 'float32', 'float64'])
+@pytest.mark.parametrize('shape', [(300, 1001), (1000, 3), (70, 4099), (5, 5), (2000, 130)])
+def test_rows_spaced_apart_and_strided_columns(dtype, shape):
+    nr, nc = shape
+    x = shaped_random((nr + 3, 2 * nc + 6), dtype, 71)
+    y = shaped_random((nr + 3, 2 * nc + 6), dtype, 72)
+    dx, dy = cp.asarray(x), cp.asarray(y)
+    views = [
+        lambda a: a[1:nr + 1, 2:nc + 2],            # window
+        lambda a: a[:nr, 1:2 * nc + 1:2],           # every second column
+        lambda a: a[:nr, nc - 1::-1],               # columns backwards
+        lambda a: a[:2 * (nr // 2):2, :nc],         # every second row
+        lambda a: a[nr - 1::-1, 3:nc + 3],          # rows backwards
+    ]
+    for va in views:
+        for vb in views:
+            p, q = va(x), vb(y)
+            if p.shape != q.shape:
+                continue
+            assert_exact((va(dx) + vb(dy)).get(), p + q)
+    # into a window, in place, with a value per row and a user kernel's index
+    out = cp.zeros_like(dx)
+    w = out[1:nr + 1, 2:nc + 2]
+    cp.multiply(dx[:nr, :nc], dy[2:nr + 2, 3:4], out=w)
+    want = np.zeros_like(x)
+    np.multiply(x[:nr, :nc], y[2:nr + 2, 3:4], out=want[1:nr + 1, 2:nc + 2])
+    assert_exact(out.get(), want)
+    w += dx[:nr, 1:2 * nc + 1:2]
+    want[1:nr + 1, 2:nc + 2] += x[:nr, 1:2 * nc + 1:2]
+    assert_exact(out.get(), want)
+    k = cp.ElementwiseKernel('T a', 'int64 at', 'at = i + (a == a ? 0 : 1)', 'index_of_window')
+    assert_exact(k(dx[1:nr + 1, 2:nc + 2]).get(), np.arange(nr * nc, dtype=np.int64).reshape(shape))
+    # matrices stored column after column
+    xf, yf = np.asfortranarray(x[:nr, :nc]), np.asfortranarray(y[:nr, :nc])
+    dxf, dyf = cp.asarray(x[:nr, :nc].T.copy()).T, cp.asarray(y[:nr, :nc].T.copy()).T
+    of = cp.zeros((nc, nr), dtype).T
+    cp.add(dxf, dyf, out=of)
+    assert_exact(of.get(), xf + yf)
+    assert_exact((dxf[1:, :] - dyf[:-1, :]).get(), xf[1:, :] - yf[:-1, :])
+    # one strided axis
+    flat, dflat = x.reshape(-1), dx.reshape(-1)
+    assert_exact((dflat[::2] * dflat[1::2]).get(), flat[::2] * flat[1::2])
+    assert_exact((dflat[::-1] + dflat).get(), flat[::-1] + flat)
+    o1 = cp.zeros(flat.size + 3, dtype)
+    cp.negative(dflat[::3], out=o1[1::3][:dflat[::3].size])
+    w1 = np.zeros(flat.size + 3, dtype)
+    np.negative(flat[::3], out=w1[1::3][:flat[::3].size])
+    assert_exact(o1.get(), w1)
