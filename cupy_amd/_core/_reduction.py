@@ -298,6 +298,24 @@ class _AbstractReductionKernel:
                     [a.dtype.itemsize for a in outs], map_expr, reduce_expr,
                     post_map_expr, reduce_type, typedefs, device_id, stream_ptr, rec,
                     batch=(n_batch, n_inner, [os_[0] for os_ in o_in]))
+        # reduction over an outer and the innermost axis, in[r0, c, r1] -> out[c]
+        # (e.g. per-channel statistics of a batch of images): the rows kernel
+        # reduces r1 for every (r0, c) into partial results, which the combine
+        # kernel reduces over r0
+        if (len(rshape) == 2 and len(oshape) == 1 and not has_raw and not needs_indexers
+                and in_arr_idx and not any(uses_identifier(e, '_J') for e in exprs)):
+            ins = [in_args[i] for i in in_arr_idx]
+            n_outer, n_inner = rshape
+            n_keep = oshape[0]
+            if all(rs[1] == a.dtype.itemsize and os_[0] % a.dtype.itemsize == 0
+                   and rs[0] == n_keep * os_[0] and os_[0] >= n_inner * a.dtype.itemsize
+                   for rs, os_, a in zip(rstrides, o_in, ins)) and n_inner > 1:
+                return self._launch_rows(
+                    in_args, out_args, in_arr_idx, out_arr_idx, n_outer * n_keep, n_inner,
+                    [os_[0] for os_ in o_in], [rs[1] for rs in rstrides],
+                    [os_[0] for os_ in o_out], map_expr, reduce_expr, post_map_expr,
+                    reduce_type, typedefs, device_id, stream_ptr, rec,
+                    stage=(n_outer, n_keep))
         # generic: views with the reduced axes in front, merged where possible
         g_in = list(in_args)
         for k, i in enumerate(in_arr_idx):
@@ -525,10 +543,13 @@ class _AbstractReductionKernel:
     # -- rows ---------------------------------------------------------------------------------
     def _launch_rows(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                      so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
-                     reduce_type, typedefs, device_id, stream_ptr, rec=None):
+                     reduce_type, typedefs, device_id, stream_ptr, rec=None, stage=None):
+        """``stage`` = (n_outer, n_keep): the ``n_out = n_outer * n_keep`` rows
+        are not the final outputs; their results are partial results that a
+        second launch combines over ``n_outer`` into ``n_keep`` outputs."""
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
-        flat = self._rows_flat_geometry(ins, n_out, n_red, so_in, sr)
+        flat = None if stage else self._rows_flat_geometry(ins, n_out, n_red, so_in, sr)
         if flat is not None:
             return self._launch_rows_flat(
                 flat, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red, so_in,
@@ -566,13 +587,13 @@ class _AbstractReductionKernel:
                 chunk = (n_red + n_split - 1) // n_split
                 chunk = (chunk + trip - 1) // trip * trip
                 n_split = (n_red + chunk - 1) // chunk
-        partial = n_split > 1
+        partial = n_split > 1 or bool(stage)
         span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
                    + [abs(s) * n_out for s in so_out] + [n_red + chunk])
         idx64 = span > _INT32_MAX - (1 << 24)
         batch = _tuning.get('rows_batch')
         trips = 1
-        batched = (group < _cg.BLOCK and batch >= 1 and n_red <= group * vec
+        batched = (group < _cg.BLOCK and batch >= 1 and n_red <= group * vec and not stage
                    and n_out >= 4 * batch and _tuning.get('rows_trips') >= 1)
         if batched:
             # Fewer lanes per row with several loads per lane shorten the
@@ -627,8 +648,12 @@ class _AbstractReductionKernel:
             _launch_plan.launch(
                 rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
                 _make_packer(self._fast_format(rargs, ic, 'P' + ic)), vals, stream_ptr)
+            if stage:
+                n_split, n_final = n_split * stage[0], stage[1]
+            else:
+                n_final = n_out
             self._finalize_partials(
-                partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
+                partials, n_split, out_args, out_arr_idx, n_final, so_out, in_args,
                 reduce_expr, post_map_expr, reduce_type, typedefs, device_id,
                 stream_ptr, rec, pref, n_out * n_red)
         else:
