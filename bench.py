@@ -283,6 +283,110 @@ def build_next_cases(cp):
     return cases
 
 
+def build_layout_cases(cp):
+    """Operand layouts beyond the five configurations, at the same size class
+    (2^26 float32 elements unless stated): views at an element offset, rows of
+    odd length, tall narrow matrices with a value per row or column, windows,
+    permuted axes, operands of different widths, reductions over a middle axis
+    or over the outer and the innermost axis.  ``bytes`` as in the other
+    suites: every input element read once, every output element written once."""
+    cases = []
+
+    def add(name, nbytes, gpu, cpu, check, kernel):
+        cases.append(dict(name=name, config='layouts', bytes=int(nbytes), gpu=gpu, cpu=cpu,
+                          check=check, kernel=kernel))
+
+    def same(out, want):
+        return bool(np.array_equal(out.get(), want))
+
+    def close(got, want, rtol, scale):
+        err = np.abs(got.get().astype(np.float64) - want)
+        return bool(np.all(err <= rtol * scale + 1e-30))
+
+    rng = np.random.default_rng(12)
+    n = 1 << 26
+    flat = rng.standard_normal(n, dtype=np.float32)
+    dflat = cp.asarray(flat)
+    res = {}
+
+    def run(key, fn):
+        def call():
+            res[key] = fn()
+        return call
+
+    # ---- elementwise ------------------------------------------------------------------
+    add('x[1:] + x[:-1] f32 2^26 (x counted once)', 2 * 4 * (n - 1), run('off', lambda: dflat[1:] + dflat[:-1]),
+        lambda: flat[1:] + flat[:-1], lambda: same(res['off'], flat[1:] + flat[:-1]), 'cupy_add')
+    rows3 = n // 3
+    a3, d3 = flat[:rows3 * 3].reshape(rows3, 3), dflat[:rows3 * 3].reshape(rows3, 3)
+    row3 = rng.standard_normal((1, 3), dtype=np.float32)
+    drow3 = cp.asarray(row3)
+    add('(N,3) - row f32', 2 * a3.nbytes, run('n3', lambda: d3 - drow3), lambda: a3 - row3,
+        lambda: same(res['n3'], a3 - row3), 'cupy_subtract')
+    sq, dsq = flat.reshape(8192, 8192), dflat.reshape(8192, 8192)
+    col = rng.standard_normal((8192, 1), dtype=np.float32)
+    row = rng.standard_normal((1, 8192), dtype=np.float32)
+    dcol, drow = cp.asarray(col), cp.asarray(row)
+    add('a * col(n,1) f32 8192x8192', 2 * sq.nbytes, run('col', lambda: dsq * dcol), lambda: sq * col,
+        lambda: same(res['col'], sq * col), 'cupy_multiply')
+    add('col + row -> 8192x8192 f32', sq.nbytes, run('outer', lambda: dcol + drow), lambda: col + row,
+        lambda: same(res['outer'], col + row), 'cupy_add')
+    add('a[1:-1,1:-1] + a[:-2,2:] f32 8192x8192 (a counted once)', 2 * 4 * 8190 * 8190,
+        run('win', lambda: dsq[1:-1, 1:-1] + dsq[:-2, 2:]), lambda: sq[1:-1, 1:-1] + sq[:-2, 2:],
+        lambda: same(res['win'], sq[1:-1, 1:-1] + sq[:-2, 2:]), 'cupy_add')
+    cube, dcube = flat.reshape(256, 512, 512), dflat.reshape(256, 512, 512)
+    for perm in ((0, 2, 1), (2, 1, 0), (1, 0, 2)):
+        key = 'perm%d%d%d' % perm
+        add('transpose%r copy f32 256x512x512' % (perm,), 2 * cube.nbytes,
+            run(key, lambda perm=perm: cp.ascontiguousarray(dcube.transpose(perm))),
+            lambda perm=perm: np.ascontiguousarray(cube.transpose(perm)),
+            lambda perm=perm, key=key: same(res[key], cube.transpose(perm)), 'cupy_copy')
+    q, dq = flat.reshape(16, 512, 64, 128), dflat.reshape(16, 512, 64, 128)
+    add('(B,S,H,D) -> (B,H,S,D) copy f32 16x512x64x128', 2 * q.nbytes,
+        run('bshd', lambda: cp.ascontiguousarray(dq.transpose(0, 2, 1, 3))),
+        lambda: np.ascontiguousarray(q.transpose(0, 2, 1, 3)),
+        lambda: same(res['bshd'], q.transpose(0, 2, 1, 3)), 'cupy_copy')
+    add('f32 > 0 -> bool 2^26', 5 * n, run('gt', lambda: dflat > 0), lambda: flat > 0,
+        lambda: same(res['gt'], flat > 0), 'cupy_greater')
+    mask = flat > 0
+    dmask = cp.asarray(mask)
+    other = rng.standard_normal(n, dtype=np.float32)
+    dother = cp.asarray(other)
+    add('where(mask, f32, f32) 2^26', 13 * n, run('where', lambda: cp.where(dmask, dflat, dother)),
+        lambda: np.where(mask, flat, other), lambda: same(res['where'], np.where(mask, flat, other)),
+        'cupy_where')
+    add('astype f32 -> f16 2^26', 6 * n, run('half', lambda: dflat.astype(np.float16)),
+        lambda: flat.astype(np.float16), lambda: same(res['half'], flat.astype(np.float16)),
+        'cupy_copy')
+    i8 = rng.integers(-100, 100, n).astype(np.int8)
+    di8 = cp.asarray(i8)
+    add('astype int8 -> int64 2^26', 9 * n, run('wide', lambda: di8.astype(np.int64)),
+        lambda: i8.astype(np.int64), lambda: same(res['wide'], i8.astype(np.int64)), 'cupy_copy')
+    # ---- reductions -------------------------------------------------------------------
+    def red(name, arr, darr, axis, kernel='cupy_sum'):
+        want = arr.sum(axis=axis, dtype=np.float64)
+        scale = np.abs(arr).sum(axis=axis, dtype=np.float64)
+        key = name
+        add(name, arr.nbytes + want.size * 4, run(key, lambda: darr.sum(axis=axis)),
+            lambda: arr.sum(axis=axis), lambda: close(res[key], want, 1e-5, scale), kernel)
+    r67 = 1000003
+    a67, d67 = flat[:r67 * 67].reshape(r67, 67), dflat[:r67 * 67].reshape(r67, 67)
+    red('sum f32 1000003x67 axis=0', a67, d67, 0)
+    red('sum f32 1000003x67 axis=1', a67, d67, 1)
+    r7 = n // 7
+    a7, d7 = flat[:r7 * 7].reshape(r7, 7), dflat[:r7 * 7].reshape(r7, 7)
+    red('sum f32 (2^26/7)x7 axis=1', a7, d7, 1)
+    add('argmax f32 (2^26/7)x7 axis=1', a7.nbytes + r7 * 8, run('am7', lambda: d7.argmax(axis=1)),
+        lambda: a7.argmax(axis=1), lambda: same(res['am7'], a7.argmax(axis=1)), 'cupy_argmax')
+    am, dm3 = flat[:33 * 65 * 31277].reshape(33, 65, 31277), dflat[:33 * 65 * 31277].reshape(33, 65, 31277)
+    red('sum f32 33x65x31277 axis=1', am, dm3, 1)
+    ac, dc = flat.reshape(512, 256, 512), dflat.reshape(512, 256, 512)
+    red('sum f32 512x256x512 axis=(0,2)', ac, dc, (0, 2))
+    a2, d2 = flat.reshape(2, n // 2), dflat.reshape(2, n // 2)
+    red('sum f32 2x2^25 axis=0', a2, d2, 0)
+    return cases
+
+
 def time_case_events(cp, fn, repeats, inner):
     """Median over ``repeats`` of the time per call, each sample being
     ``inner`` back-to-back calls bracketed by two events on the launch stream."""
@@ -357,10 +461,11 @@ def main():
     ap.add_argument('--no-detail', action='store_true',
                     help='skip per-operation event timing and launch latency')
     ap.add_argument('--only', default='', help='run only cases whose name contains this')
-    ap.add_argument('--suite', default='configs', choices=('configs', 'next'),
+    ap.add_argument('--suite', default='configs', choices=('configs', 'next', 'layouts'),
                     help="'configs': the five benchmark configurations (the headline figure); "
                          "'next': scans, statistics, complex types and multi-kernel fused "
-                         "functions at shapes of the same size class")
+                         "functions at shapes of the same size class; 'layouts': offset views, "
+                         "odd and narrow rows, windows, permuted axes, mixed widths")
     ap.add_argument('--calibrate', action='store_true',
                     help='add a plain copy kernel of known size (256 MiB in, 256 MiB out) to '
                          'every step, as the yardstick for hardware traffic counters')
@@ -376,7 +481,8 @@ def main():
     props = cp.cuda.device.get_device_properties(0)
     log('device:', props['arch'], props['compute_units'], 'CUs')
     t0 = time.perf_counter()
-    cases = build_cases(cp, args.scale) if args.suite == 'configs' else build_next_cases(cp)
+    cases = (build_cases(cp, args.scale) if args.suite == 'configs' else
+             build_next_cases(cp) if args.suite == 'next' else build_layout_cases(cp))
     if args.only:
         cases = [c for c in cases if args.only in c['name']]
     log('inputs ready in %.1f s' % (time.perf_counter() - t0))
@@ -484,6 +590,9 @@ def main():
                    'NOT the benchmark figure: scans, statistics, complex types and multi-kernel '
                    'fused functions, %d operations per step' % len(cases)
                    if args.suite == 'next' and not args.only else
+                   'NOT the benchmark figure: offset views, odd and narrow rows, windows, permuted '
+                   'axes, mixed widths, %d operations per step' % len(cases)
+                   if args.suite == 'layouts' and not args.only else
                    'REDUCED run (scale=%d only=%r): not the benchmark figure' % (args.scale, args.only),
                    'bytes_per_step': total_bytes, 'operations': len(cases)},
         'frac_of_hbm_peak': round(value / HBM_PEAK_GBPS, 4),
