@@ -507,18 +507,32 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
                 src.append('      for (int _k = 0; _k < %d; ++_k) *%s = _l_%s.v[_k];' % (
                     vec, addr(op, '_ck + _k'), op.name))
     src.append('    } else {')
-
-    def edge_load(op):
-        return '(*%s)' % addr(op, '_ck + _k')
-
-    def edge_store(op, value):
-        return '*%s = %s;' % (addr(op, '_ck + _k'), value)
-
-    src.append('      for (int _k = 0; _k < (int)(_nc - _ck); ++_k) {')
+    # the last, partial vector of a row: the same three phases under a
+    # per-element test, so that all loads are in flight together (a loop of
+    # unknown length would wait for every element in turn)
+    for op in arrays:
+        k = kinds[op.name]
+        reads = (not op.is_out) or op.read_out
+        if k == 'row':
+            if reads:
+                src.append('      const %s _b_%s = *%s;' % (op.store_t, op.name, addr(op, '0')))
+            continue
+        src.append('      cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+        if reads:
+            src.append('#pragma unroll')
+            src.append('      for (int _k = 0; _k < %d; ++_k) if (_ck + _k < _nc) _l_%s.v[_k] = *%s;' % (
+                vec, op.name, addr(op, '_ck + _k')))
+    src.append('#pragma unroll')
+    src.append('      for (int _k = 0; _k < %d; ++_k) if (_ck + _k < _nc) {' % vec)
     if use_i:
         src.append('        const ptrdiff_t i = (ptrdiff_t)_rk * _nc + _ck + _k;')
-    src.append(_element_code(operands, operation, edge_load, edge_store, 8))
+    src.append(_element_code(operands, operation, full_load, full_store, 8))
     src.append('      }')
+    for op in arrays:
+        if op.is_out:
+            src.append('#pragma unroll')
+            src.append('      for (int _k = 0; _k < %d; ++_k) if (_ck + _k < _nc) *%s = _l_%s.v[_k];' % (
+                vec, addr(op, '_ck + _k'), op.name))
     src.append('    }')
     src.append('  }')
     src.append('  %s;' % after_loop)

@@ -499,7 +499,7 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
 def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
               partial_in=False, partial_out=False, stream_hint=False, unroll=4,
-              solo=False, batched=False, clamp_tail=False):
+              solo=False, batched=False, clamp_tail=False, vec_out=False, solo_block=BLOCK):
     """Output-axis-contiguous kernel.  Thread layout: ``tx`` threads across
     the output axis (each owning ``vec`` adjacent outputs) times 256/tx slices
     of the reduce axis; gridDim.y further slices.  ``partial_in``: the single
@@ -516,15 +516,16 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     # moves its own columns to the front of its accumulators at the end; no
     # lane then walks the reduce axis element by element.  Needs loads that
     # may start at any element.
+    block = solo_block if solo else BLOCK
     if solo:
-        tx = BLOCK
+        tx = block
     clamp_tail = clamp_tail and vec > 1 and not partial_in
     assert tx in (1, 2, 4, 8, 16, 32, 64) or solo
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     nt = 'true' if stream_hint else 'false'
     ins = [a for a in args if a.kind == 'in']
-    ty = BLOCK // tx
-    waves = BLOCK // WAVE
+    ty = block // tx
+    waves = block // WAVE
     params = _fast_params(args, idx_t, partial_in, partial_out)
     if batched:
         assert not partial_in and not any(a.bcast_o for a in ins)
@@ -534,7 +535,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         params += ''.join(', const %s _sb_%s' % (idx_t, a.name) for a in ins)
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
-        BLOCK, name, params))
+        block, name, params))
     src.append(_SIZE_INDEXERS)
     if not solo:
         src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (
@@ -673,6 +674,26 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         src.append('    }')
         src.append('  }')
     if solo:
+        outs = [a for a in args if a.kind == 'out']
+        if vec_out and vec > 1 and not partial_out:
+            # outputs stored next to one another: the thread's results leave as
+            # one vector per output (with few rows to reduce, the outputs are a
+            # large share of the traffic)
+            src.append('  if (_c + %d <= _ncol) {' % vec)
+            for a in outs:
+                src.append('    cupy::Vec<%s, %d> _o_%s;' % (a.store_t, vec, a.name))
+            src.append('#pragma unroll')
+            src.append('    for (int _k = 0; _k < %d; ++_k) {' % vec)
+            src.append('      _type_reduce _s = _acc[_k];')
+            src.append('      const %s _i = _i0 + _c + _k; (void)_i;' % idx_t)
+            for a in outs:
+                src.append('      %s &%s = _o_%s.v[_k];' % (a.var_t, a.name, a.name))
+            src.append('      POST_MAP(_s);')
+            src.append('    }')
+            for a in outs:
+                src.append('    cupy::store_vec<%s, %d, %s>(_p_%s + _i0 + _c, _o_%s);' % (
+                    a.store_t, vec, nt, a.name, a.name))
+            src.append('  } else')
         src.append('  if (_c < _ncol) {')
         src.append('#pragma unroll')
         src.append('    for (int _k = 0; _k < %d; ++_k) if (_c + _k < _ncol) {' % vec)
@@ -812,10 +833,14 @@ def emit_finalize_generic(name, args, identity, reduce_expr, post_map_expr,
     parts.append('CIndexer<%d, %d> _out_ind' % (out_ndim, out_index_32))
     parts.append('const _type_reduce* _partials')
     parts.append('const int _n_split')
+    parts.append('const long long _in_total')     # element count of the whole problem
     params = ', '.join(parts)
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         BLOCK, name, params))
+    # post-maps ask the input indexer for its size only (a mean divides by
+    # `_in_ind.size() / _out_ind.size()`)
+    src.append('  const SizeOnly _in_ind((ptrdiff_t)_in_total); (void)_in_ind;')
     src.append('  const ptrdiff_t _n_out = _out_ind.size();')
     src.append('  CUPY_FOR(_i, _n_out) {')
     src.append('    _type_reduce _s = %s;' % _identity_decl(identity))

@@ -309,7 +309,8 @@ class _AbstractReductionKernel:
             n_keep = oshape[0]
             if all(rs[1] == a.dtype.itemsize and os_[0] % a.dtype.itemsize == 0
                    and rs[0] == n_keep * os_[0] and os_[0] >= n_inner * a.dtype.itemsize
-                   for rs, os_, a in zip(rstrides, o_in, ins)) and n_inner > 1:
+                   for rs, os_, a in zip(rstrides, o_in, ins)) and n_inner > 1 and (
+                       n_outer * n_keep * n_inner >= 1 << 16):     # else one launch is quicker
                 return self._launch_rows(
                     in_args, out_args, in_arr_idx, out_arr_idx, n_outer * n_keep, n_inner,
                     [os_[0] for os_ in o_in], [rs[1] for rs in rstrides],
@@ -705,16 +706,18 @@ class _AbstractReductionKernel:
             vec //= 2
         tx = max(1, min(64, internal.clp2((n_cols + vec - 1) // vec)))
         # a handful of rows and plenty of columns: a thread per column vector
-        solo = (n_red <= 8 and n_out >= cus * _cg.BLOCK * vec
-                and n_cols >= _cg.BLOCK * vec)
+        solo_block = _tuning.get('cols_solo_block')
+        solo = (n_red <= 8 and n_out >= cus * solo_block * vec
+                and n_cols >= solo_block * vec)
+        block = solo_block if solo else _cg.BLOCK
         if solo:
-            tx = _cg.BLOCK
-        ty = _cg.BLOCK // tx
+            tx = block
+        ty = block // tx
         nbc = (n_cols + tx * vec - 1) // (tx * vec)
         gx = nbc * n_batch
         # the kernel does not loop over column blocks: beyond what grid.x may
         # hold they continue along grid.z
-        gz = (gx + _max_blocks(_cg.BLOCK) - 1) // _max_blocks(_cg.BLOCK)
+        gz = (gx + _max_blocks(block) - 1) // _max_blocks(block)
         gx = (gx + gz - 1) // gz
         want = (cus * _tuning.get('target_blocks_per_cu') + gx * gz - 1) // (gx * gz)
         most = max(1, n_red // (ty * 8))
@@ -729,8 +732,11 @@ class _AbstractReductionKernel:
         idx64 = span > _INT32_MAX - (1 << 24)
         rargs = self._rargs(in_args, out_args, bcast_r=[s == 0 for s in sr], bcast_o=bcast_o)
         clamp = bool(n_cols % vec and n_cols >= vec and _tuning.get('unaligned_vectors'))
+        outs = [out_args[i] for i in out_arr_idx]
+        vec_out = bool(solo and all(s == a.dtype.itemsize for s, a in zip(so_out, outs)))
         if solo:
-            unroll = 1
+            # all rows of a column are requested together
+            unroll = max(1, min(4, internal.flp2(n_red)))
         elif partial and all(s % 128 == 0 for s in sr):
             unroll = _tuning.get('cols_unroll')
         else:
@@ -739,7 +745,7 @@ class _AbstractReductionKernel:
             _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
-               stream_hint, solo, bool(batch), clamp, unroll, _tuning.signature())
+               stream_hint, solo, bool(batch), clamp, unroll, vec_out, block, _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
@@ -747,7 +753,7 @@ class _AbstractReductionKernel:
                 post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
                 idx64=idx64, partial_out=partial,
                 stream_hint=stream_hint, unroll=unroll, solo=solo,
-                batched=bool(batch), clamp_tail=clamp)
+                batched=bool(batch), clamp_tail=clamp, vec_out=vec_out, solo_block=solo_block)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
@@ -762,7 +768,7 @@ class _AbstractReductionKernel:
             if batch:
                 vals.const(*batch_vals)
             _launch_plan.launch(
-                rec, fn, (gx, n_split, gz), (_cg.BLOCK, 1, 1),
+                rec, fn, (gx, n_split, gz), (block, 1, 1),
                 _make_packer(self._fast_format(rargs, ic, 'P' + tail)), vals, stream_ptr)
             self._finalize_partials(
                 partials, n_split, out_args, out_arr_idx, n_out, so_out, in_args,
@@ -772,7 +778,7 @@ class _AbstractReductionKernel:
             if batch:
                 vals.const(*batch_vals)
             _launch_plan.launch(
-                rec, fn, (gx, 1, gz), (_cg.BLOCK, 1, 1),
+                rec, fn, (gx, 1, gz), (block, 1, 1),
                 _make_packer(self._fast_format(rargs, ic, tail)), vals, stream_ptr)
 
     # -- generic ------------------------------------------------------------------------------
@@ -877,9 +883,9 @@ class _AbstractReductionKernel:
         fmt.append('q' * (1 + 2 * out_ind.ndim))
         vals.const(out_ind.size, *out_ind.shape)
         vals.const(*((0,) * out_ind.ndim))
-        fmt.append('Pi')
+        fmt.append('Piq')
         vals.ptr(pref, partials.ptr)
-        vals.const(n_split)
+        vals.const(n_split, in_ind.size)
         grid = max(1, min((n_out + _cg.BLOCK - 1) // _cg.BLOCK, cus * 8))
         _launch_plan.launch(rec, ffn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
                             _make_packer(fmt), vals, stream_ptr)

@@ -65,6 +65,7 @@ _params = {
     # 509: 78.5 -> 60.6 us)
     'cols_unroll': 1,
     'cols_unroll_near': 4,
+    'cols_solo_block': 1024,    # workgroup of the thread-per-column variant
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
     # fused row-wise functions: words per lane up to which a wave takes a whole row

@@ -428,6 +428,9 @@ def test_reduction_over_the_outer_and_the_innermost_axis(shape, dtype):
     if shape[2] > 4:
         w, dw = x[:, :, 1:-1], dx[:, :, 1:-1]
         assert_exact(dw.max(axis=(0, 2)).get(), w.max(axis=(0, 2)))
+        # a post-map that asks for the number of reduced elements, after a split
+        np.testing.assert_allclose(dw.mean(axis=(0, 2)).get().astype(np.float64),
+                                   w.astype(np.float64).mean(axis=(0, 2)), rtol=2e-3, atol=2e-2)
     out = cp.zeros((2 * shape[1],), dx.max().dtype)
     dx.max(axis=(0, 2), out=out[::2])
     assert_exact(out.get()[::2], x.max(axis=(0, 2)))
