@@ -181,3 +181,81 @@ def test_scans_random_views(block):
             assert_close(got.get(), want, 1e-12, np.maximum(np.cumsum(np.abs(a), axis=axis), 1))
         else:
             assert_exact(got.get(), want), tag
+
+
+def _fused_templates(xp):
+    def chain(x, y):
+        return xp.sqrt(xp.abs(x)) + y * 2 - xp.minimum(x, y)
+
+    def dot_last(x, y):
+        return xp.sum(x * y, axis=-1)
+
+    def dot_first(x, y):
+        return xp.sum(x * y, axis=0)
+
+    def centre(x, y):
+        return x - xp.sum(x, axis=-1, keepdims=True) / x.shape[-1] + y
+
+    def softmax(x, y):
+        e = xp.exp(x - xp.amax(x, axis=-1, keepdims=True))
+        return e / xp.sum(e, axis=-1, keepdims=True)
+
+    def two_results(x, y):
+        return xp.sum(x, axis=0), xp.amax(x * y, axis=0)
+
+    def normalise(x, y):
+        m = xp.sum(x, axis=-1, keepdims=True) / x.shape[-1]
+        d = x - m
+        v = xp.sum(d * d, axis=-1, keepdims=True) / x.shape[-1]
+        return d / xp.sqrt(v + 1e-3) * y
+
+    def total(x, y):
+        return xp.sum(xp.where(x > y, x, y))
+
+    return [chain, dot_last, dot_first, centre, softmax, two_results, normalise, total]
+
+
+@pytest.mark.parametrize('template', range(8))
+def test_fused_functions_random_views(template):
+    rng = np.random.default_rng(4000 + template)
+    host_f = _fused_templates(np)[template]
+    dev_f = cp.fuse(_fused_templates(cp)[template])
+    for case in range(40):
+        ndim = int(rng.integers(1, 4))
+        if case % 4 == 0:
+            shape = tuple(int(d) for d in rng.integers(2, 9, ndim - 1)) + (
+                int(rng.choice([64, 100, 256, 1000, 4096, 5000])),)
+        else:
+            shape = tuple(int(d) for d in rng.integers(1, 30, ndim))
+        dt = str(rng.choice(['float32', 'float64', 'float32', 'float16']))
+        plain = rng.random() < 0.5
+        if plain:
+            r = np.random.default_rng(case)
+            a = (r.random(shape) * 4 - 2).astype(dt)
+            b = (r.random(shape) * 4 - 2).astype(dt)
+            xa, xb = cp.asarray(a), cp.asarray(b)
+        else:
+            a, xa = random_view(rng, shape, dt, int(rng.integers(1 << 30)))
+            b, xb = random_view(rng, shape, dt, int(rng.integers(1 << 30)))
+            a, b = a / 4, b / 4
+            xa, xb = xa / 4, xb / 4
+            if rng.random() < 0.5:
+                # the division above made them dense; take views of those again
+                a, b, xa, xb = a[..., ::-1], b[..., 1:], xa[..., ::-1], xb[..., 1:]
+                a, xa = a[..., 1:], xa[..., 1:]
+        if a.shape[-1] == 0:
+            continue
+        with np.errstate(all='ignore'):
+            want = host_f(a.astype(np.float64), b.astype(np.float64))
+            like = host_f(a, b)
+        got = dev_f(xa, xb)
+        wants = want if isinstance(want, tuple) else (want,)
+        likes = like if isinstance(like, tuple) else (like,)
+        gots = got if isinstance(got, tuple) else (got,)
+        tol = {'float16': 2e-2, 'float32': 2e-4, 'float64': 1e-9}[dt]
+        for g, w, l in zip(gots, wants, likes):
+            tag = (template, case, shape, dt, plain, xa.strides, xb.strides)
+            assert g.shape == np.shape(w) and g.dtype == np.asarray(l).dtype, tag
+            if dt == 'float16':
+                w = np.where(np.abs(w) > 65504, np.sign(w) * np.inf, w)     # overflows like the result
+            assert_close(g.get(), w, tol, np.maximum(np.abs(w), 1) * (a.shape[-1] ** 0.5))
