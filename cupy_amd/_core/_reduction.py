@@ -579,7 +579,10 @@ class _AbstractReductionKernel:
             group = max(1, min(64, internal.clp2(lanes_needed)))
         n_split = 1
         chunk = n_red
-        if group == _cg.BLOCK and n_out < cus * _tuning.get('min_blocks_per_cu'):
+        # (a second launch costs about 8 us: below 128 KiB per row a workgroup
+        # on its own is quicker)
+        if (group == _cg.BLOCK and n_out < cus * _tuning.get('min_blocks_per_cu')
+                and (n_red * max_item >= 128 * 1024 or stage)):
             trip = _cg.BLOCK * vec
             want = (cus * _tuning.get('target_blocks_per_cu') + n_out - 1) // n_out
             most = max(1, n_red // (trip * 4))

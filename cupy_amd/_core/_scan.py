@@ -488,7 +488,9 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         # enough waves to fill the device: cut rows into chunks if there are few
         want = cus * _tuning.get('scan_waves_per_cu')
         n_chunks = 1
-        if may_chunk and group == _WAVE and outer < want and n > 2 * per_group:
+        # (three launches cost about 30 us: a wave on its own is quicker for
+        # up to a dozen rounds)
+        if may_chunk and group == _WAVE and outer < want and n > 12 * per_group:
             n_chunks = min((want + outer - 1) // outer, (n + per_group - 1) // per_group)
         chunk_len = (n + n_chunks - 1) // n_chunks
         chunk_len = (chunk_len + per_group - 1) // per_group * per_group
