@@ -677,14 +677,29 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
                        '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (vec, op.name, pitch))
         src.append('      }')
         src.append('    } else {')
-        src.append('      for (int _v = threadIdx.x; _v < %d; _v += %d) {' % (
-            tile_r * tile_c, threads))
-        src.append('        const int _lr = _v %% %d;' % tile_r)
-        src.append('        const int _lc = _v / %d;' % tile_r)
-        src.append('        if (_r0 + _lr < _nr && _c0 + _lc < _nc) {')
+        # edge tile: the same vectors where they lie inside the array, element by
+        # element (under a test each) where they cross its border
+        src.append('#pragma unroll')
+        src.append('      for (int _it = 0; _it < %d; ++_it) {' % (n_stage // threads))
+        src.append('        const int _v = threadIdx.x + _it * %d;' % threads)
+        src.append('        const int _lr = (_v %% %d) * %d;' % (tile_r // vec, vec))
+        src.append('        const int _lc = _v / %d;' % (tile_r // vec))
+        src.append('        if (_c0 + _lc < _nc) {')
+        src.append('          if (_r0 + _lr + %d <= _nr) {' % vec)
         for op in c_ops:
-            src.append('          _t_%s[_lr * %d + _lc] = *%s;' % (
-                op.name, pitch, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
+            src.append('            { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s);' % (
+                op.store_t, vec, op.store_t, vec, ntl, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
+            src.append('#pragma unroll')
+            src.append('              for (int _k = 0; _k < %d; ++_k) '
+                       '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (vec, op.name, pitch))
+        src.append('          } else {')
+        src.append('#pragma unroll')
+        src.append('            for (int _k = 0; _k < %d; ++_k) if (_r0 + _lr + _k < _nr) {' % vec)
+        for op in c_ops:
+            src.append('              _t_%s[(_lr + _k) * %d + _lc] = *%s;' % (
+                op.name, pitch, gaddr(op, '_r0 + _lr + _k', '_c0 + _lc')))
+        src.append('            }')
+        src.append('          }')
         src.append('        }')
         src.append('      }')
         src.append('    }')
@@ -740,21 +755,48 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     def edge_load(op):
         lay = layouts[op.name]
         if lay == 'C':
-            return '_t_%s[_lr * %d + _lc]' % (op.name, pitch)
-        return '(*%s)' % gaddr(op, '_r', '_c')
+            return '_t_%s[_lr * %d + _lc + _k]' % (op.name, pitch)
+        return '(*%s)' % gaddr(op, '_r', '_c + _k')
 
     def edge_store(op, value):
-        return '*%s = %s;' % (gaddr(op, '_r', '_c'), value)
+        return '*%s = %s;' % (gaddr(op, '_r', '_c + _k'), value)
 
-    src.append('      for (int _w = threadIdx.x; _w < %d; _w += %d) {' % (tile_r * tile_c, threads))
-    src.append('        const int _lc = _w %% %d;' % tile_c)
-    src.append('        const int _lr = _w / %d;' % tile_c)
+    src.append('#pragma unroll')
+    src.append('      for (int _it = 0; _it < %d; ++_it) {' % (n_work // threads))
+    src.append('        const int _w = threadIdx.x + _it * %d;' % threads)
+    src.append('        const int _lc = (_w %% %d) * %d;' % (tile_c // vec, vec))
+    src.append('        const int _lr = _w / %d;' % (tile_c // vec))
     src.append('        const %s _r = _r0 + _lr;' % idx_t)
     src.append('        const %s _c = _c0 + _lc;' % idx_t)
-    src.append('        if (_r < _nr && _c < _nc) {')
+    src.append('        if (_r < _nr && _c + %d <= _nc) {' % vec)
+    for op in arrays:
+        lay = layouts[op.name]
+        reads = (not op.is_out) or op.read_out
+        if lay == 'R':
+            if reads:
+                src.append('          cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
+                    op.store_t, vec, op.name, op.store_t, vec, ntl, gaddr(op, '_r', '_c')))
+            else:
+                src.append('          cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+        elif lay == 'R0':
+            src.append('          const %s _b_%s = *%s;' % (op.store_t, op.name, gaddr(op, '_r', '0')))
+    src.append('#pragma unroll')
+    src.append('          for (int _k = 0; _k < %d; ++_k) {' % vec)
     if use_i or set_ind:
-        src.append('          const ptrdiff_t i = (ptrdiff_t)_r * _nc + _c; %s' % set_ind)
-    src.append(_element_code(operands, operation, edge_load, edge_store, 10))
+        src.append('            const ptrdiff_t i = (ptrdiff_t)_r * _nc + _c + _k; %s' % set_ind)
+    src.append(_element_code(operands, operation, full_load, full_store, 12))
+    src.append('          }')
+    for op in arrays:
+        if op.is_out:
+            src.append('          cupy::store_vec<%s, %d, %s>(%s, _l_%s);' % (
+                op.store_t, vec, nts, gaddr(op, '_r', '_c'), op.name))
+    src.append('        } else if (_r < _nr) {')
+    src.append('#pragma unroll')
+    src.append('          for (int _k = 0; _k < %d; ++_k) if (_c + _k < _nc) {' % vec)
+    if use_i or set_ind:
+        src.append('            const ptrdiff_t i = (ptrdiff_t)_r * _nc + _c + _k; %s' % set_ind)
+    src.append(_element_code(operands, operation, edge_load, edge_store, 12))
+    src.append('          }')
     src.append('        }')
     src.append('      }')
     src.append('    }')
