@@ -899,15 +899,18 @@ class _ElementwisePlanner:
         stream_hint = _tuning.stream_policy(
             _tuning.get('tiled_stream'),
             *self._traffic(args, nin, [n for n, l in layouts.items() if l == 'R0']))
-        if stream_hint[1]:
-            # a tile row is a short run of the output (256-512 bytes): where such
-            # runs do not start and end on cache-line boundaries, non-temporal
-            # stores leave partly written lines behind (transposed copy of
-            # 4099 x 16363 float32: 183 us with the hint, 116 us without)
-            for a, cs in zip(arrays, cstrides):
-                if any(a is o for o in args[nin:]) and (
-                        a.data.ptr % 128 or cs[0] % 128 or (tile_c * a.dtype.itemsize) % 128):
-                    stream_hint = (stream_hint[0], False)
+        if stream_hint[1] and n_transposed and _tuning.get('tiled_stream') == 'auto':
+            # a tile row is a short run of the output (256-512 bytes), written
+            # by a few lanes while neighbouring tiles write the rest of the same
+            # cache lines later: plain stores let the cache put the lines together
+            # (transposed copy of 4099 x 16363 float32: 183 us with non-temporal
+            # stores, 116 us without; C2a within the benchmark step 84.6 -> 80.8 us)
+            # (batches of aligned tiles measure 2-6 % better with the hint)
+            unaligned = any(
+                any(a is o for o in args[nin:]) and (a.data.ptr % 128 or cs[0] % 128)
+                for a, cs in zip(arrays, cstrides))
+            if not batch or unaligned:
+                stream_hint = (stream_hint[0], False)
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
                threads, bool(batch))
