@@ -539,6 +539,11 @@ class _ElementwisePlanner:
         (nr, nc), cstrides, kinds = plan
         itemsizes = [a.dtype.itemsize for a in arrays]
         vec = max(1, 16 // max(itemsizes))
+        if _tuning.get('rows2d_narrow_vec') and nc < 12 * vec:
+            # few vectors per row: a partial one at every row end would split
+            # the lanes of a wave between two code paths
+            while vec > 1 and nc % vec:
+                vec //= 2
         span = max(abs(cs[0]) * nr + abs(cs[1]) * nc for cs in cstrides)
         nvr = (nc + vec - 1) // vec
         idx64 = span > _INT32_MAX or nr * nvr * vec > _INT32_MAX - (1 << 24)

@@ -640,6 +640,9 @@ class _AbstractReductionKernel:
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
         if group == _cg.BLOCK:
             gx = min(n_out, _max_blocks(_cg.BLOCK))
+            cap = _tuning.get('rows_block_grid_per_cu')
+            if cap and n_split == 1:
+                gx = min(gx, cus * cap)
         else:
             rows_per_block = _cg.BLOCK // group * (batch if batched else 1)
             gx = min((n_out + rows_per_block - 1) // rows_per_block,

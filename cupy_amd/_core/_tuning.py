@@ -21,6 +21,10 @@ _params = {
     # matrices whose rows are spaced apart (windows, every second row or
     # column) are walked row by row in vectors instead of in square tiles
     'rows2d': True,
+    # ... with shorter vectors for rows of fewer than 12 vectors, so that no row
+    # ends in a partial one (window of 7 columns: 235 -> 142 us; from 12
+    # vectors per row on, the partial vector costs less than shorter accesses)
+    'rows2d_narrow_vec': True,
     # Operands of different widths: the widest moves 16 bytes per access
     # ('wide'; the narrower ones then move less, but consecutive lanes stay on
     # consecutive addresses in every operand) or the narrowest does ('narrow';
@@ -46,6 +50,7 @@ _params = {
     'rows_stream': True,       # non-temporal loads: True / False / 'auto' (by footprint);
                                # measured better or equal from 16 MiB inputs upwards
     'rows_unroll': 4,
+    'rows_block_grid_per_cu': 0,   # workgroups per CU when a workgroup owns a row (0: one per row)
     'rows_block_mode_bytes': 32768,   # row length from which a workgroup owns a row
     'rows_batch': 2,            # short rows handled per lane group at a time
     'rows_trips': 4,            # ... with up to this many vector loads per lane and row
