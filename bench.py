@@ -41,19 +41,19 @@ HBM_PEAK_GBPS = 8000.0
 # device); the summary of those runs is profiles/pmc_traffic_bench_suite.md.
 # Two-pass reductions count both of their kernels.
 MEASURED_TRAFFIC_BYTES = {
-    'C1 saxpy f32 2^26': 536849410 + 268402180,
-    'C2a x.T*y f32(T)xf16 8192^2': 269332789 + 268446079,
-    'C2b tmp+1 f32 8192^2': 268435456 + 268507639,
-    'C3 sum float32 axis=1 16384^2': 1073677829 + 524735,
-    'C3 sum float32 axis=0 16384^2': 1073677317 + 2096892 + 2122574 + 65528,
-    'C3 sum float32 axis=None 16384^2': 1073678341 + 65688 + 11391 + 32,
-    'C3 sum float64 axis=1 8192^2': 536851714 + 262239,
-    'C3 sum float64 axis=0 8192^2': 536851458 + 2096892 + 2122574 + 65528,
-    'C3 sum float64 axis=None 8192^2': 536852482 + 65592 + 19582 + 32,
-    'C4 argmax i32 (2^20,128)': 536870912 + 8392368,
-    'C4 argmin i32 (2^20,128)': 536869888 + 8396207,
-    'C4 argmax f32 (2^16,4096)': 1073710979 + 525599,
-    'C5 fused sum((x-y)^2*w) f16 (2^18,256)': 268443647 + 1048446,
+    'C1 saxpy f32 2^26': 536849410 + 268397829,
+    'C2a x.T*y f32(T)xf16 8192^2': 271083170 + 268397701,
+    'C2b tmp+1 f32 8192^2': 268435456 + 268720216,
+    'C3 sum float32 axis=1 16384^2': 1073677445 + 524886,
+    'C3 sum float32 axis=0 16384^2': 1073677317 + 2096857 + 2122574 + 65527,
+    'C3 sum float32 axis=None 16384^2': 1073678341 + 65719 + 11391 + 32,
+    'C3 sum float64 axis=1 8192^2': 536851842 + 262427,
+    'C3 sum float64 axis=0 8192^2': 536851458 + 2096857 + 2122574 + 65527,
+    'C3 sum float64 axis=None 8192^2': 536852482 + 65591 + 19582 + 32,
+    'C4 argmax i32 (2^20,128)': 536870912 + 8392036,
+    'C4 argmin i32 (2^20,128)': 536869888 + 8396707,
+    'C4 argmax f32 (2^16,4096)': 1073711235 + 525942,
+    'C5 fused sum((x-y)^2*w) f16 (2^18,256)': 268443647 + 1048429,
 }
 
 
