@@ -268,7 +268,9 @@ def _emit_lanes(in_t, out_t, op, skip_nan, vec, trips, idx64, lstride, stream):
     ``lstride`` adjacent lanes, a wave holds ``64 / lstride`` consecutive rows
     per load -- contiguous in memory, so accesses stay coalesced however narrow
     the array is -- and the scan runs across the lanes in steps of ``lstride``
-    (Kogge-Stone over rows; the ``vec`` columns of a lane never mix)."""
+    (Kogge-Stone over rows; the ``vec`` columns of a lane never mix).
+    ``lstride`` need not be a power of two: the lanes past the last whole row
+    of a wave stay idle."""
     acc_t = _acc_type(out_t)
     op_c = '+' if op == _SUM else '*'
     ident = '0' if op == _SUM else '1'
@@ -326,7 +328,8 @@ __device__ __forceinline__ void scan_lanes_impl(
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t) {
         const _idx_t r = rb + t * TRIP_ROWS + lrow;
-        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + (ptrdiff_t)(r < r1 ? r : r0) * INNER);
+        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(
+            src + (ptrdiff_t)((r < r1 && lrow < TRIP_ROWS) ? r : r0) * INNER);
       }
       _acc_t v[TRIPS][VEC];
 #pragma unroll
@@ -334,7 +337,7 @@ __device__ __forceinline__ void scan_lanes_impl(
         const _idx_t r = rb + t * TRIP_ROWS + lrow;
 #pragma unroll
         for (int k = 0; k < VEC; ++k)
-          v[t][k] = (r < r1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+          v[t][k] = (r < r1 && lrow < TRIP_ROWS) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
       }
       if (kMode == 1) {
         // only the column totals of the chunk are wanted: every lane adds up
@@ -366,21 +369,27 @@ __device__ __forceinline__ void scan_lanes_impl(
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
           // the trip's total of this column sits in the last row of the wave
-          const _acc_t total = cupy::shfl_idx<64>(v[t][k], 64 - LSTRIDE + lane %% LSTRIDE);
+          const _acc_t total = cupy::shfl_idx<64>(
+              v[t][k], (TRIP_ROWS - 1) * LSTRIDE + lane %% LSTRIDE);
           res.v[k] = static_cast<_out_t>(SCAN_OP(carry[k], v[t][k]));
           carry[k] = SCAN_OP(carry[k], total);
         }
-        if (kMode != 1 && r < r1)
+        if (kMode != 1 && r < r1 && lrow < TRIP_ROWS)
           cupy::store_vec<_out_t, VEC, NT_STORE>(dst + (ptrdiff_t)r * INNER, res);
       }
     }
     if (kMode == 1) {
+      // the rows of the wave are combined like a scan; its last row then holds
+      // the totals
 #pragma unroll
-      for (int m = LSTRIDE; m < 64; m <<= 1) {
+      for (int d = LSTRIDE; d < 64; d <<= 1) {
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) carry[k] = SCAN_OP(carry[k], cupy::shfl_xor(carry[k], m));
+        for (int k = 0; k < VEC; ++k) {
+          const _acc_t up = cupy::shfl_up<64>(carry[k], d);
+          carry[k] = (lane >= d) ? SCAN_OP(up, carry[k]) : carry[k];
+        }
       }
-      if (lrow == 0) {
+      if (lrow == TRIP_ROWS - 1) {
 #pragma unroll
         for (int k = 0; k < VEC; ++k)
           totals[((ptrdiff_t)o * n_chunks + chunk) * INNER + lcol + k] = carry[k];
@@ -435,8 +444,8 @@ def _acc_dtype(out_dtype):
 
 
 def _lanes_geometry(src, dst, inner, item):
-    """(vec, lanes per row) for the lane-interleaved kernel, or None when the
-    inner extent is not a small power-of-two number of vectors."""
+    """(vec, lanes per row) for the lane-interleaved kernel, or None when a row
+    of the inner extent does not fit half a wave."""
     if inner < 2:
         return None
     vec = max(1, 16 // item)
@@ -444,8 +453,9 @@ def _lanes_geometry(src, dst, inner, item):
         if (inner % vec == 0 and _aligned(src.data.ptr, vec * src.dtype.itemsize)
                 and _aligned(dst.data.ptr, vec * dst.dtype.itemsize)):
             lstride = inner // vec
-            if lstride <= 16 and lstride & (lstride - 1) == 0:
+            if lstride <= 32:
                 return vec, lstride
+            return None
         vec //= 2
     return None
 

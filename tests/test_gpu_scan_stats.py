@@ -261,7 +261,11 @@ def test_one_pass_variance_is_stable_and_matches_numpy(dtype):
 
 @pytest.mark.parametrize('shape,axis', [((1000, 8), 0), ((7, 1000, 2), 1), ((5000, 64), 0),
                                         ((100001, 16), 0), ((3, 70000, 4), 1), ((50, 32), 0),
-                                        ((2, 3, 999, 8), 2)])
+                                        ((2, 3, 999, 8), 2),
+                                        # rows that do not fill a power-of-two number of lanes
+                                        ((100001, 3), 0), ((5000, 7), 0), ((3, 70000, 5), 1),
+                                        ((40000, 12), 0), ((999, 20), 0), ((70001, 48), 0),
+                                        ((6000, 100), 0), ((2, 9000, 31), 1), ((64, 6), 0)])
 @pytest.mark.parametrize('dtype', ['float32', 'float64', 'int32', 'float16'])
 def test_scans_along_an_axis_with_a_narrow_tail(shape, axis, dtype):
     """The axes after the scanned one span a few vectors only: rows sit in
