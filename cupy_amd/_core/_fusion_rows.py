@@ -178,7 +178,10 @@ def _build(nodes, pieces, returns, single, args, name):
     items = [leaf_value[n.order].dtype.itemsize for n in full_leaves + col_leaves]
     vec = max(1, 16 // max(items))
     while vec > 1:
-        ok = n_cols % vec == 0
+        # a row length that is not a whole number of vectors is fine where
+        # vectors may start at any element: the last, partial vector of a row
+        # is then read and written element by element
+        ok = n_cols % vec == 0 or (_tuning.get('unaligned_vectors') and n_cols >= 4 * vec)
         for n in full_leaves + col_leaves:
             a = leaf_value[n.order]
             ok = ok and _aligned(a.data.ptr, min(16, vec * a.dtype.itemsize))
@@ -191,6 +194,9 @@ def _build(nodes, pieces, returns, single, args, name):
     # a wave per row while the row fits its registers: no barrier, and every
     # lane keeps many loads in flight; a workgroup per row beyond that
     group = WAVE if words_for(WAVE) <= _tuning.get('fused_rows_wave_words') else BLOCK
+    if group == WAVE:
+        # short rows: as many lanes as the row has vectors, several rows per wave
+        group = max(4, min(WAVE, internal.clp2((n_cols + vec - 1) // vec)))
     per_lane = (n_cols + group * vec - 1) // (group * vec)          # vectors per lane and operand
     words = words_for(group)
     if words > _ROW_WORDS_PER_LANE or n_cols < 16:
@@ -291,6 +297,22 @@ def _build(nodes, pieces, returns, single, args, name):
     src.append('#define GROUP %d' % group)
     src.append('#define VEC %d' % vec)
     src.append('#define PER_LANE %d' % per_lane)
+    # a vector of a row: whole where it lies within the row, element by element
+    # where the row ends inside it (rows that are not a multiple of VEC long)
+    src.append('''template <typename T, bool kStream>
+__device__ __forceinline__ cupy::Vec<T, VEC> _row_vec(const T* row, int col) {
+  if (NCOLS % VEC == 0 || col + VEC <= NCOLS) return cupy::load_vec<T, VEC, kStream>(row + col);
+  cupy::Vec<T, VEC> v;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) v.v[k] = (col + k < NCOLS) ? row[col + k] : T();
+  return v;
+}
+template <typename T, bool kStream>
+__device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, VEC>& v) {
+  if (NCOLS % VEC == 0 || col + VEC <= NCOLS) { cupy::store_vec<T, VEC, kStream>(row + col, v); return; }
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) if (col + k < NCOLS) row[col + k] = v.v[k];
+}''')
     for k, (p, d) in enumerate(zip(pieces, described)):
         src.append('namespace piece%d {' % k)
         if d['kind'] == 'reduce':
@@ -324,7 +346,7 @@ def _build(nodes, pieces, returns, single, args, name):
         src.append('#pragma unroll')
         src.append('  for (int _e = 0; _e < PER_LANE; ++_e) {')
         src.append('    const int _col = (_e * GROUP + _lane) * VEC;')
-        src.append('    _c%d[_e] = cupy::load_vec<%s, VEC, false>(_p%d + (_col < NCOLS ? _col : 0));'
+        src.append('    _c%d[_e] = _row_vec<%s, false>(_p%d, _col < NCOLS ? _col : 0);'
                    % (n.order, t, n.order))
         src.append('  }')
     for n in nodes:
@@ -345,7 +367,7 @@ def _build(nodes, pieces, returns, single, args, name):
     src.append('      const int _cc = _col < NCOLS ? _col : 0;')
     for n in full_leaves:
         t = get_typename(leaf_value[n.order].dtype)
-        src.append('      _f%d[_e] = cupy::load_vec<%s, VEC, %s>(_p%d + (ptrdiff_t)_row * NCOLS + _cc);'
+        src.append('      _f%d[_e] = _row_vec<%s, %s>(_p%d + (ptrdiff_t)_row * NCOLS, _cc);'
                    % (n.order, t, ntl, n.order))
     src.append('    }')
     for n in nodes:
@@ -383,8 +405,8 @@ def _build(nodes, pieces, returns, single, args, name):
                 k, k, k, k, ', '.join(call_args)))
             src.append('      }')
             src.append('    }')
-            if group == WAVE:
-                src.append('    _a%d = cupy::group_allreduce<64>(_a%d, piece%d::Op());' % (k, k, k))
+            if group <= WAVE:
+                src.append('    _a%d = cupy::group_allreduce<GROUP>(_a%d, piece%d::Op());' % (k, k, k))
             else:
                 src.append('    _a%d = cupy::group_allreduce<64>(_a%d, piece%d::Op());' % (k, k, k))
                 src.append('    if ((threadIdx.x & 63) == 0) _sm%d[threadIdx.x >> 6] = _a%d;' % (k, k))
@@ -423,8 +445,8 @@ def _build(nodes, pieces, returns, single, args, name):
                 for t in p.targets:
                     if not any(t is m for m in out_nodes):
                         raise _Unsupported('elementwise value that is not a result')
-                    src.append('      if (_col < NCOLS) cupy::store_vec<%s, VEC, %s>('
-                               '_o%d + (ptrdiff_t)_row * NCOLS + _col, _v%d);' % (
+                    src.append('      if (_col < NCOLS) _row_store<%s, %s>('
+                               '_o%d + (ptrdiff_t)_row * NCOLS, _col, _v%d);' % (
                                    get_typename(dtype_of[t.order]), nts, t.order, t.order))
                 src.append('    }')
             else:
