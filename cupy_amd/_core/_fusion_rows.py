@@ -140,6 +140,8 @@ def build(nodes, pieces, returns, single, args, name):
 
     ``pieces``: the ``_Piece`` objects of ``_fusion_split`` in evaluation order;
     ``returns``: node order numbers or ('const', value)."""
+    if not _tuning.get('fused_rows'):
+        return None
     try:
         return _build(nodes, pieces, returns, single, args, name)
     except _Unsupported:
@@ -181,7 +183,7 @@ def _build(nodes, pieces, returns, single, args, name):
         # a row length that is not a whole number of vectors is fine where
         # vectors may start at any element: the last, partial vector of a row
         # is then read and written element by element
-        ok = n_cols % vec == 0 or (_tuning.get('unaligned_vectors') and n_cols >= 4 * vec)
+        ok = n_cols % vec == 0 or (_tuning.get('unaligned_vectors') and n_cols > vec)
         for n in full_leaves + col_leaves:
             a = leaf_value[n.order]
             ok = ok and _aligned(a.data.ptr, min(16, vec * a.dtype.itemsize))
@@ -196,10 +198,10 @@ def _build(nodes, pieces, returns, single, args, name):
     group = WAVE if words_for(WAVE) <= _tuning.get('fused_rows_wave_words') else BLOCK
     if group == WAVE:
         # short rows: as many lanes as the row has vectors, several rows per wave
-        group = max(4, min(WAVE, internal.clp2((n_cols + vec - 1) // vec)))
+        group = max(1, min(WAVE, internal.clp2((n_cols + vec - 1) // vec)))
     per_lane = (n_cols + group * vec - 1) // (group * vec)          # vectors per lane and operand
     words = words_for(group)
-    if words > _ROW_WORDS_PER_LANE or n_cols < 16:
+    if words > _ROW_WORDS_PER_LANE or n_cols < 2:
         raise _Unsupported('row of %d elements does not fit the registers of a group' % n_cols)
 
     # ---- trace every piece into device functions -----------------------------------------
@@ -405,7 +407,9 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
                 k, k, k, k, ', '.join(call_args)))
             src.append('      }')
             src.append('    }')
-            if group <= WAVE:
+            if group == 1:
+                pass
+            elif group <= WAVE:
                 src.append('    _a%d = cupy::group_allreduce<GROUP>(_a%d, piece%d::Op());' % (k, k, k))
             else:
                 src.append('    _a%d = cupy::group_allreduce<64>(_a%d, piece%d::Op());' % (k, k, k))

@@ -75,6 +75,7 @@ _params = {
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
     # fused row-wise functions: words per lane up to which a wave takes a whole row
+    'fused_rows': True,         # row-wise fused functions as one kernel (False: one kernel per piece)
     'fused_rows_wave_words': 64,
     # Vector accesses need only the alignment of one element: an access of 16
     # bytes at an address that is a multiple of 4 measures within 4 % of an

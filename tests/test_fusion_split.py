@@ -157,8 +157,16 @@ CASES = {
 }
 
 
+@pytest.fixture
+def one_kernel_per_piece():
+    from cupy_amd._core import _tuning
+    _tuning.set(fused_rows=False)
+    yield
+    _tuning.set(fused_rows=True)
+
+
 @pytest.mark.parametrize('name', sorted(CASES))
-def test_recorded_shapes_and_kernel_counts(name):
+def test_recorded_shapes_and_kernel_counts(name, one_kernel_per_piece):
     make, n_arrays, extra, n_kernels, shapes = CASES[name]
     captured = cp.asarray(np.ones(4, np.float32))
     f = cp.fuse(make(cp, captured))

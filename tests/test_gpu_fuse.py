@@ -305,7 +305,8 @@ def test_kernel_sequence_cases_match_numpy():
 
 
 @pytest.mark.parametrize('shape', [(301, 77), (70, 33), (64, 4096), (17, 5, 1000), (1000,),
-                                   (129, 8192), (300, 1001), (64, 4099), (128, 777), (33, 18)])
+                                   (129, 8192), (300, 1001), (64, 4099), (128, 777), (33, 18),
+                                   (5000, 10), (777, 3), (100, 2), (4099, 7)])
 def test_row_wise_functions_in_one_kernel_match_numpy(shape):
     """Functions whose reductions all run along short rows compile to a single
     kernel that holds the row in registers (wave-per-row and workgroup-per-row
