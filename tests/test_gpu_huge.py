@@ -235,3 +235,57 @@ def test_three_dimensional_view_that_does_not_merge():
         '  if (v > best) { best = v; at = a; } }'
         'ok = k == at'.replace('VALUE', value), 'is_view_leading_argmax')
     assert bool(check3(k).all().get())
+
+
+def test_matrix_plus_row_vector_beyond_2_to_31_elements():
+    m = 2 ** 30 + 1
+    a = _fill_mod100_i8(size=3 * m).reshape(m, 3)
+    row = cp.asarray(np.array([[1, 2, 3]], np.int8))
+    r = a + row                                       # flat kernel, row and column by division
+    check = cp.ElementwiseKernel(
+        'int8 v', 'bool ok', 'ok = v == (signed char)(i % 100 + i % 3 + 1)', 'is_plus_row')
+    assert bool(check(r).all().get())
+    del r
+    col = _fill_mod50_i8(size=m).reshape(m, 1)
+    r = a - col
+    check2 = cp.ElementwiseKernel(
+        'int8 v', 'bool ok', 'ok = v == (signed char)(i % 100 - (i / 3) % 50)', 'is_minus_col')
+    assert bool(check2(r).all().get())
+
+
+def test_short_odd_rows_and_windows_beyond_2_to_31_elements():
+    n_rows = 2 ** 29
+    a = _fill_mod100_i8(size=n_rows * 5).reshape(n_rows, 5)
+    rows = a.sum(axis=1)                              # rows staged through the LDS
+    check = cp.ElementwiseKernel(
+        'int64 s', 'bool ok',
+        'const long long b = (long long)i * 5; long long w = 0;'
+        'for (int k = 0; k < 5; ++k) w += (b + k) % 100; ok = s == w', 'is_rowsum5_mod100')
+    assert bool(check(rows).all().get())
+    del rows
+    w = a[:, 1:4] + a[:, 0:3]                         # windows: row by row in vectors
+    check2 = cp.ElementwiseKernel(
+        'int8 v', 'bool ok',
+        'const long long r = i / 3, c = i % 3;'
+        'ok = v == (signed char)((r * 5 + c + 1) % 100 + (r * 5 + c) % 100)', 'is_window_sum')
+    assert bool(check2(w).all().get())
+
+
+def test_permuted_axes_beyond_2_to_31_elements():
+    nb, n = 3, 30000                                  # 2.7e9 elements
+    a = _fill_mod100_i8(size=nb * n * n).reshape(nb, n, n)
+    t = cp.ascontiguousarray(a.transpose(0, 2, 1))    # tiled kernel with a batch axis
+    check = cp.ElementwiseKernel(
+        'int8 v', 'bool ok',
+        'const long long n = 30000, c = i % n, r = (i / n) % n, b = i / (n * n);'
+        'ok = v == (signed char)((b * n * n + c * n + r) % 100)', 'is_batch_transposed')
+    assert bool(check(t).all().get())
+    del t
+    s = a.sum(axis=1)                                 # reduction over the middle axis
+    assert s.shape == (nb, n) and s.dtype == np.int64
+    check2 = cp.ElementwiseKernel(
+        'int64 s', 'bool ok',
+        'const long long n = 30000, c = i % n, b = i / n; long long w = 0;'
+        'for (long long r = 0; r < n; ++r) w += (b * n * n + r * n + c) % 100; ok = s == w',
+        'is_middle_sum')
+    assert bool(check2(s).all().get())

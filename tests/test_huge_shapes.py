@@ -27,6 +27,12 @@ CASES = {
     'rows_few': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=1),
     'rows_many': lambda: cp.empty((2 ** 25, 64), np.int8).sum(axis=1),
     'rows_very_many': lambda: cp.empty((2 ** 29, 4), np.int8).sum(axis=1),
+    'flat_row_vector': lambda: cp.empty((2 ** 30 + 1, 3), np.int8) + cp.empty((1, 3), np.int8),
+    'rows_flat': lambda: cp.empty((2 ** 29, 5), np.int8).sum(axis=1),
+    'windows': lambda: cp.empty((2 ** 29, 5), np.int8)[:, 1:4] + cp.empty((2 ** 29, 5), np.int8)[:, 0:3],
+    'batched_transpose': lambda: cp.ascontiguousarray(
+        cp.empty((3, 30000, 30000), np.int8).transpose(0, 2, 1)),
+    'middle_axis': lambda: cp.empty((3, 30000, 30000), np.int8).sum(axis=1),
     'cols_wide': lambda: cp.empty((9, 2 ** 30 + 1), np.int8).sum(axis=0),
     'cols_wide_few_rows': lambda: cp.empty((3, 2 ** 30 + 1), np.int8).sum(axis=0),
     'cols_split': lambda: cp.empty((2 ** 16, 2 ** 16), np.int8).sum(axis=0),
