@@ -384,6 +384,26 @@ def build_layout_cases(cp):
     red('sum f32 512x256x512 axis=(0,2)', ac, dc, (0, 2))
     a2, d2 = flat.reshape(2, n // 2), dflat.reshape(2, n // 2)
     red('sum f32 2x2^25 axis=0', a2, d2, 0)
+    # ---- scan along an axis with an odd tail, fused rows of 100 ---------------------------
+    want_scan = np.cumsum(a3, axis=0, dtype=np.float64)
+    scale_scan = np.cumsum(np.abs(a3), axis=0, dtype=np.float64)
+    add('cumsum f32 (2^26/3)x3 axis=0', 2 * a3.nbytes, run('scan3', lambda: cp.cumsum(d3, axis=0)),
+        lambda: np.cumsum(a3, axis=0), lambda: close(res['scan3'], want_scan, 1e-5, scale_scan),
+        'cupy_scan_lanes')
+    r100 = n // 100
+    a100, d100 = flat[:r100 * 100].reshape(r100, 100), dflat[:r100 * 100].reshape(r100, 100)
+
+    @cp.fuse(kernel_name='softmax_rows_of_100')
+    def softmax(x):
+        e = cp.exp(x - cp.amax(x, axis=1, keepdims=True))
+        return e / cp.sum(e, axis=1, keepdims=True)
+
+    def cpu_softmax():
+        e = np.exp(a100 - a100.max(axis=1, keepdims=True))
+        return e / e.sum(axis=1, keepdims=True)
+    add('fused softmax f32 (2^26/100)x100', 2 * a100.nbytes, run('sm100', lambda: softmax(d100)),
+        cpu_softmax, lambda: close(res['sm100'], cpu_softmax().astype(np.float64), 1e-5, 1.0),
+        'softmax_rows_of_100')
     return cases
 
 
