@@ -427,8 +427,6 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
     ``kinds[name]`` is
       'R'    unit stride along columns, any stride along rows: vector access;
       'row'  zero stride along columns: one value per row;
-      'col1' zero stride along rows, unit stride along columns: one vector
-             load per vector of the problem;
       'S'    anything else (every second column, columns backwards, ...):
              element-wise access.
     The last ``_nc % vec`` columns of a row are handled element by element by
@@ -466,11 +464,10 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
     for op in arrays:
         k = kinds[op.name]
         reads = (not op.is_out) or op.read_out
-        if k in ('R', 'col1'):
+        if k == 'R':
             if reads:
                 src.append('      cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s);' % (
-                    op.store_t, vec, op.name, op.store_t, vec,
-                    ntl if k == 'R' else 'false', addr(op, '_ck')))
+                    op.store_t, vec, op.name, op.store_t, vec, ntl, addr(op, '_ck')))
             else:
                 src.append('      cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
         elif k == 'row':

@@ -466,7 +466,7 @@ class _ElementwisePlanner:
         None when the problem is not of this kind."""
         if not _tuning.get('flat_bcast'):
             return None
-        nr, nc = cshape
+        nc = cshape[1]
         names = [p.name for a, p in zip(args, self.params)
                  if isinstance(a, ndarray) and not p.raw]
         outs = args[nin:]
@@ -518,8 +518,6 @@ class _ElementwisePlanner:
                     ok = False
                 elif sc == 0:
                     kind = 'row'
-                elif sr == 0 and sc == item:
-                    kind = 'col1'
                 elif abs(sc) <= 4 * item and (sr == 0 or abs(sr) >= abs(sc)):
                     kind = 'S'
                 else:
@@ -537,8 +535,7 @@ class _ElementwisePlanner:
     def _launch_rows2d(self, dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
                        force_read_out, stream_ptr, kernel_name, rec):
         (nr, nc), cstrides, kinds = plan
-        itemsizes = [a.dtype.itemsize for a in arrays]
-        vec = max(1, 16 // max(itemsizes))
+        vec = max(1, 16 // max(a.dtype.itemsize for a in arrays))
         if _tuning.get('rows2d_narrow_vec') and nc < 12 * vec:
             # few vectors per row: a partial one at every row end would split
             # the lanes of a wave between two code paths
@@ -548,7 +545,10 @@ class _ElementwisePlanner:
         nvr = (nc + vec - 1) // vec
         idx64 = span > _INT32_MAX or nr * nvr * vec > _INT32_MAX - (1 << 24)
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
-        light = [n for n, k in kinds.items() if k in ('row', 'col1')]
+        names = [p.name for a, p in zip(args, self.params)
+                 if isinstance(a, ndarray) and not p.raw]
+        # a value per row, or one row repeated: not counted as streamed traffic
+        light = [n for n, cs in zip(names, cstrides) if cs[0] == 0 or cs[1] == 0]
         in_bytes, out_bytes = self._traffic(args, nin, light)
         stream_hint = _tuning.stream_policy(_tuning.get('tiled_stream'), in_bytes, out_bytes)
         block = 256
