@@ -3,6 +3,7 @@ ReductionKernel, ufuncs, ``fuse`` and the device memory pool) built natively
 for AMD Instinct MI355X (gfx950).  ``import cupy_amd as cupy`` keeps existing
 call sites of that path working."""
 import numpy as _numpy
+from cupy_amd._core._structured import make_aligned_dtype  # noqa: F401
 
 from cupy_amd import _rt  # noqa: loads the native shim or fails loudly
 from cupy_amd import cuda  # noqa

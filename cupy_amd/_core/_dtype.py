@@ -25,6 +25,16 @@ def get_dtype(t):
 def check_supported_dtype(dtype, error=True):
     if dtype.char in SUPPORTED_CHARS and dtype.isnative:
         return True
+    if dtype.kind == 'V' and dtype.fields is not None:
+        # structured: any layout can be stored and moved; kernels check the
+        # alignment of the fields when one is built for it
+        from cupy_amd._core import _structured
+        if not _structured.has_references(dtype):
+            return True
+        if error:
+            raise ValueError('dtypes that hold Python objects cannot live in device memory: %s'
+                             % dtype)
+        return False
     if error:
         raise ValueError('Unsupported dtype %s' % dtype)
     return False

@@ -403,6 +403,10 @@ class _ElementwisePlanner:
         stream_ptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
         mode = 'generic'
         cshape = cstrides = None
+        if arrays and any(a.dtype.fields is not None for a in arrays):
+            # elements that are structures go one by one through the indexer
+            # kernel (the vector helpers want element sizes that are powers of two)
+            force_generic = True
         if not (force_generic or self._force_generic) and arrays:
             cshape, cstrides = _canonical_dims(arrays, shape)
             nd = len(cshape)
@@ -1535,6 +1539,9 @@ class ufunc:
                     self, *args, **kwargs)
         if _fusion_thread_local.is_fusing():
             return _fusion_thread_local.call_ufunc(self, *args, **kwargs)
+        for arg in args:
+            if getattr(getattr(arg, 'dtype', None), 'fields', None) is not None:
+                return _call_structured(self, args, kwargs)
 
         # A call that looks like an earlier one replays that call's launch.
         fast_key = rec = fast_args = None
@@ -1747,6 +1754,67 @@ class ufunc:
     def reduceat(self, array, indices, axis=0, dtype=None, out=None):
         raise NotImplementedError(
             f'`{self.name}.reduceat` is not supported yet')
+
+
+_struct_kernels = {}
+
+
+def _call_structured(ufunc_obj, args, kwargs):
+    """Copy and (in)equality of arrays whose elements are structures: the
+    loops the reference has for them (cupy/_core/_routines_logic.pyx:76-117,
+    field-wise assignment in include/cupy/structview.cuh)."""
+    from cupy_amd._core import _structured
+    from cupy_amd._core.core import array
+    out = kwargs.pop('out', None)
+    kwargs.pop('casting', None)
+    if kwargs:
+        raise TypeError('Wrong arguments %s' % kwargs)
+    name = ufunc_obj.name
+    if name not in ('cupy_copy', 'cupy_equal', 'cupy_not_equal'):
+        raise TypeError('ufunc %r is not supported for structured dtypes' % name)
+    args = list(args)
+    if len(args) == ufunc_obj.nin + 1 and out is None:
+        out = args.pop()
+    if len(args) != ufunc_obj.nin:
+        raise TypeError('Wrong number of arguments for %r' % name)
+    if isinstance(out, tuple):
+        (out,) = out
+    ins = [a if isinstance(a, ndarray) else array(a) for a in args]
+    if name == 'cupy_copy':
+        (src,) = ins
+        if out is None:
+            out = ndarray._new_contiguous(src.shape, src.dtype)
+        if src.dtype.fields is not None and out.dtype.fields is not None and \
+                not numpy.can_cast(src.dtype, out.dtype, 'unsafe'):
+            raise TypeError(f'Cannot cast array data from {src.dtype!r} to {out.dtype!r}')
+        if src.dtype.fields is not None and out.dtype.fields is None:
+            raise TypeError(f'Cannot cast array data from {src.dtype!r} to {out.dtype!r}')
+        kern = _struct_kernels.get('copy')
+        if kern is None:
+            kern = _struct_kernels['copy'] = ElementwiseKernel(
+                'X x', 'Y y', 'y = x', 'cupy_copy_struct')
+        if out.size:
+            kern(src, out)
+        return out
+    a, b = ins
+    common = _structured.comparison_dtype(a.dtype, b.dtype)
+    if any(f[0].subdtype is not None for f in (common.fields or {}).values()):
+        raise ValueError('comparison of structured arrays with subarray dtypes is not supported')
+    # both sides in the common dtype first, as the reference's loop resolution
+    # has it: field values are then compared like with like
+    if a.dtype != common:
+        a = a.astype(common)
+    if b.dtype != common:
+        b = b.astype(common)
+    key = 'eq' if name == 'cupy_equal' else 'ne'
+    kern = _struct_kernels.get(key)
+    if kern is None:
+        kern = _struct_kernels[key] = ElementwiseKernel(
+            'X a, Y b', 'bool z', 'z = (a %s b)' % ('==' if key == 'eq' else '!='),
+            'cupy_%s_struct' % ('equal' if key == 'eq' else 'not_equal'))
+    if out is None:
+        return kern(a, b)
+    return kern(a, b, out)
 
 
 def _make_cast(src_dtype, dst_dtype):

@@ -38,8 +38,14 @@ def get_typename(dtype, type_decls=None):
     except TypeError:
         name = None
     if name is None:
-        name = _typenames.get(get_dtype(dtype))
+        dt = get_dtype(dtype)
+        name = _typenames.get(dt)
         if name is None:
+            if dt.kind == 'V' and dt.fields is not None:
+                # a struct written out for this dtype; not memoised here: the
+                # registry of definitions keeps its own table
+                from cupy_amd._core import _structured
+                return _structured.struct_typename(dt)[0]
             raise ValueError(f'Unsupported dtype {dtype}')
         try:
             _typenames_by_key[dtype] = name

@@ -340,10 +340,47 @@ class ndarray:
         return self._view(shape, strides, dtype)
 
     def __getitem__(self, key):
+        if self.dtype.fields is not None and (
+                isinstance(key, str) or (isinstance(key, list) and key
+                                         and all(isinstance(k, str) for k in key))):
+            return self._field_view(key)
         shape, strides, offset = _basic_index(self._shape, self._strides, key)
         v = self._view(shape, strides)
         if offset:
             v.data = self.data + offset
+        return v
+
+    def _field_view(self, key):
+        """View of one field, or of several fields at their places in the
+        element (as NumPy does it)."""
+        fields = self.dtype.fields
+        if isinstance(key, str):
+            if key not in fields:
+                raise ValueError('no field of name %s' % key)
+            sub, offset = fields[key][0], fields[key][1]
+            if sub.subdtype is not None:
+                raise ValueError('CuPy does not yet support accessing nested subarrays')
+        else:
+            for k in key:
+                if k not in fields:
+                    raise ValueError('no field of name %s' % k)
+            if len(set(key)) != len(key):
+                raise ValueError('duplicate field of name %s' % key)
+            sub = numpy.dtype(dict(names=list(key), formats=[fields[k][0] for k in key],
+                                   offsets=[fields[k][1] for k in key],
+                                   itemsize=self.dtype.itemsize))
+            offset = 0
+        v = ndarray(self._shape, sub, memptr=self.data + offset, strides=self._strides)
+        v.base = self.base if self.base is not None else self
+        if sub.fields is None and v.size:
+            # every element of a plain field must sit at a multiple of its size
+            # (cupy/_core/internal.pyx:532-562)
+            mask = sub.itemsize - 1
+            if v.data.ptr & mask or any(st & mask for st in v._strides):
+                raise ValueError(
+                    f'result array with dtype {sub} would not be sufficiently aligned for GPU '
+                    'operations. When using structured dtypes you must manually align the '
+                    'dtype and its fields; CuPy may provide utilities for this in the future.')
         return v
 
     def __setitem__(self, key, value):
@@ -446,6 +483,9 @@ class ndarray:
         dt = _dtype.get_dtype(dtype)
         if casting is not None:
             _dtype._raise_if_invalid_cast(self.dtype, dt, casting)
+        if (dt.fields is not None or self.dtype.fields is not None) and \
+                not numpy.can_cast(self.dtype, dt, 'unsafe'):
+            raise TypeError(f'Cannot cast array data from {self.dtype!r} to {dt!r}')
         if dt == self.dtype and not copy:
             return self
         if order in ('K', 'k', 'A', 'a'):
@@ -462,6 +502,9 @@ class ndarray:
         from cupy_amd._core._ufuncs import elementwise_copy
         if isinstance(value, ndarray) and value.ndim != 0:
             raise ValueError('non-scalar cupy.ndarray cannot be used for fill')
+        if self.dtype.fields is not None and not isinstance(value, ndarray):
+            # a structured value travels as a one-element array of this dtype
+            value = array(numpy.asarray(value, dtype=self.dtype).reshape(()))
         elementwise_copy(value, self, casting='unsafe')
 
     def item(self):
@@ -953,8 +996,7 @@ def array(obj, dtype=None, copy=True, order='K', subok=False, ndmin=0):
             out = src.astype(dtype)
     else:
         host = numpy.asarray(obj, dtype=dtype)
-        if host.dtype.char not in _dtype.SUPPORTED_CHARS or not host.dtype.isnative:
-            raise ValueError('Unsupported dtype %s' % host.dtype)
+        _dtype.check_supported_dtype(host.dtype)
         keep_f = (order in ('K', 'A', 'F', 'k', 'a', 'f') and host.ndim > 1
                   and host.flags.f_contiguous and not host.flags.c_contiguous) \
             or (order in ('F', 'f') and host.ndim > 1)

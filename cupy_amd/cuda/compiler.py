@@ -217,6 +217,10 @@ def get_code_object(source, options=()):
 def compile_with_cache(source, options=()):
     """Loaded module for ``source`` on the current device (memoised)."""
     options = tuple(options)
+    if 'cupy_struct_' in source:
+        # structured element types: their definitions follow the device header
+        from cupy_amd._core import _structured
+        source = _structured.splice_definitions(source)
     dev = _device.get_device_id()
     key = (dev, source, options)
     mod = _module_memo.get(key)
