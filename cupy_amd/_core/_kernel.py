@@ -1540,7 +1540,7 @@ class ufunc:
         if _fusion_thread_local.is_fusing():
             return _fusion_thread_local.call_ufunc(self, *args, **kwargs)
         for arg in args:
-            if getattr(getattr(arg, 'dtype', None), 'fields', None) is not None:
+            if type(arg) is ndarray and arg.dtype.fields is not None:
                 return _call_structured(self, args, kwargs)
 
         # A call that looks like an earlier one replays that call's launch.

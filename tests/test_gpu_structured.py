@@ -159,3 +159,20 @@ def test_fields_feed_the_other_kernels():
     got = (dev['f0'] * dev['f1'] + dev['f2']).get()
     assert np.array_equal(got, host['f0'] * host['f1'] + host['f2'])
     assert np.array_equal(cp.cumsum(dev['f1']).get(), np.cumsum(host['f1']))
+
+
+def test_user_kernel_over_structures():
+    dt = cp.make_aligned_dtype('i4,f8')
+    host = np.zeros(5000, dtype=dt)
+    host['f0'] = np.arange(5000)
+    host['f1'] = np.arange(5000) * 0.5
+    dev = cp.asarray(host)
+    k = cp.ElementwiseKernel('T x', 'float64 y', 'y = x.template at<0>() + x.template at<1>()',
+                             'sum_of_fields')
+    assert np.array_equal(k(dev).get(), host['f0'] + host['f1'])
+    swap = cp.ElementwiseKernel(
+        'T x', 'T y', 'y = x; y.template at<0>() = -x.template at<0>()', 'negate_first_field')
+    got = swap(dev).get()
+    want = host.copy()
+    want['f0'] = -want['f0']
+    assert np.array_equal(got, want)
