@@ -25,6 +25,9 @@ def get_dtype(t):
 def check_supported_dtype(dtype, error=True):
     if dtype.char in SUPPORTED_CHARS and dtype.isnative:
         return True
+    if dtype.kind == 'V' and dtype.fields is None and dtype.subdtype is None \
+            and dtype.itemsize > 0:
+        return True                      # raw bytes
     if dtype.kind == 'V' and dtype.fields is not None:
         # structured: any layout can be stored and moved; kernels check the
         # alignment of the fields when one is built for it

@@ -403,7 +403,7 @@ class _ElementwisePlanner:
         stream_ptr = _stream.get_current_stream_ptr() if stream is None else stream.ptr
         mode = 'generic'
         cshape = cstrides = None
-        if arrays and any(a.dtype.fields is not None for a in arrays):
+        if arrays and any(a.dtype.kind == 'V' for a in arrays):
             # elements that are structures go one by one through the indexer
             # kernel (the vector helpers want element sizes that are powers of two)
             force_generic = True
@@ -1540,7 +1540,7 @@ class ufunc:
         if _fusion_thread_local.is_fusing():
             return _fusion_thread_local.call_ufunc(self, *args, **kwargs)
         for arg in args:
-            if type(arg) is ndarray and arg.dtype.fields is not None:
+            if type(arg) is ndarray and arg.dtype.kind == 'V':
                 return _call_structured(self, args, kwargs)
 
         # A call that looks like an earlier one replays that call's launch.
@@ -1789,6 +1789,9 @@ def _call_structured(ufunc_obj, args, kwargs):
             raise TypeError(f'Cannot cast array data from {src.dtype!r} to {out.dtype!r}')
         if src.dtype.fields is not None and out.dtype.fields is None:
             raise TypeError(f'Cannot cast array data from {src.dtype!r} to {out.dtype!r}')
+        if out.dtype.kind == 'V' and out.dtype.fields is None and src.dtype != out.dtype:
+            raise TypeError('raw bytes are only copied between arrays of the same dtype, '
+                            f'not from {src.dtype!r} to {out.dtype!r}')
         kern = _struct_kernels.get('copy')
         if kern is None:
             kern = _struct_kernels['copy'] = ElementwiseKernel(

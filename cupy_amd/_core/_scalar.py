@@ -46,6 +46,9 @@ def get_typename(dtype, type_decls=None):
                 # registry of definitions keeps its own table
                 from cupy_amd._core import _structured
                 return _structured.struct_typename(dt)[0]
+            if dt.kind == 'V' and dt.subdtype is None and dt.itemsize > 0:
+                from cupy_amd._core import _structured
+                return _structured.void_typename(dt.itemsize)       # a blob of bytes
             raise ValueError(f'Unsupported dtype {dtype}')
         try:
             _typenames_by_key[dtype] = name

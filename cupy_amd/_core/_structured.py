@@ -137,7 +137,8 @@ def struct_typename(dtype):
     if type_name not in _definitions:
         lines = ['struct alignas(%d) %s {' % (alignment, type_name),
                  '  char _d[%d];' % dtype.itemsize,
-                 '  static const int n_fields = %d;' % len(fields)]
+                 '  static const int n_fields = %d;' % len(fields),
+                 '  static const int field_count = %d;' % len(fields)]
         for const in ('', 'const '):
             lines.append('  template <int I> __device__ __forceinline__ %sauto& at() %s{' % (const, const))
             for k, (sub_name, offset) in enumerate(fields):
@@ -161,6 +162,24 @@ def struct_typename(dtype):
     if not dtype.metadata:
         _names[dtype] = (type_name, alignment)
     return type_name, alignment
+
+
+def void_typename(itemsize):
+    """C++ type of an unstructured void element: ``itemsize`` raw bytes that can
+    be copied and compared (include/cupy/unstructured_void.cuh in the
+    reference)."""
+    type_name = 'cupy_struct_' + hashlib.sha1(b'void/%d' % itemsize).hexdigest()[:16]
+    if type_name not in _definitions:
+        _definitions[type_name] = ('''struct %(n)s {
+  char _d[%(size)d];
+  __device__ __forceinline__ bool operator==(const %(n)s& o) const {
+    bool same = true;
+    for (int k = 0; k < %(size)d; ++k) same = same && (_d[k] == o._d[k]);
+    return same;
+  }
+  __device__ __forceinline__ bool operator!=(const %(n)s& o) const { return !(*this == o); }
+};''' % dict(n=type_name, size=itemsize), ())
+    return type_name
 
 
 def splice_definitions(source):

@@ -176,3 +176,56 @@ def test_user_kernel_over_structures():
     want = host.copy()
     want['f0'] = -want['f0']
     assert np.array_equal(got, want)
+
+
+def test_field_count_and_in_place_field_update_of_a_user_kernel():
+    kernel = cp.ElementwiseKernel(
+        'T in', 'T out',
+        'static_assert(T::field_count == 2, "expected 2 fields"); out.at<1>() = -in.at<0>();',
+        'test_struct_access')
+    x = cp.array(np.array([(1, 0), (2, 0), (3, 0)], dtype='i,i'))
+    y = cp.array(np.array([(4, 0), (5, 0), (6, 0)], dtype='i,i'))
+    kernel(x, y)
+    assert np.array_equal(y.get(), np.array([(4, -1), (5, -2), (6, -3)], dtype='i,i'))
+
+
+def test_multifield_assignment_with_holes_and_casts():
+    def f(xp):
+        a = xp.ones(10, 'i,f,i,f,i,f')
+        for i in range(6):
+            a['f%d' % i] = xp.arange(i, 10 + i)
+        a[['f1', 'f0', 'f4']] = a[['f2', 'f1', 'f5']].copy()
+        return a
+    both(f)
+
+
+@pytest.mark.parametrize('scalar', [
+    1.0, np.int32(-1),
+    np.void((1, 2, 3, 4, 5, 6), dtype='q,q,q,q,i,i'),
+    np.void((-1, 2, 3, 4, 5, -6), dtype='d,d,d,d,d,d')])
+def test_scalars_into_structures(scalar):
+    def full(xp):
+        return xp.full(10, scalar, dtype='i,i,q,q,q,q')
+
+    def assign(xp):
+        a = xp.zeros(10, dtype='i,i,q,q,q,q')
+        a[...] = scalar
+        return a
+    both(full)
+    both(assign)
+
+
+def test_raw_bytes():
+    assert cp.empty(10, dtype='V10').dtype == np.dtype('V10')
+    assert not cp.zeros(3, dtype='V10').get().view('uint8').any()
+    host = np.array([b'1', b'2', b'3'], dtype='V10')
+    dev = cp.array(host)
+    assert np.array_equal(dev.get(), host) and np.array_equal(dev[::-1].copy().get(), host[::-1])
+    a = np.array([b'87654321', b'12345678'], dtype='V8')
+    b = np.array([b'87654321', b'1234567_'], dtype='V8')
+    assert np.array_equal((cp.array(a) == cp.array(b)).get(), a == b)
+    assert np.array_equal((cp.array(a) != cp.array(b)).get(), a != b)
+    with pytest.raises(ValueError, match='Unsupported dtype'):
+        cp.empty(3, dtype='3i')
+    with pytest.raises(ValueError, match='Unsupported dtype'):
+        cp.empty(3, dtype='V')
