@@ -421,9 +421,11 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     around), so that the lanes of a wave are spread over the LDS banks for
     even widths too.
 
-    Every input must have element strides (width, 1).  Same parameters as the
+    Every input must have element strides (width, 1), or (0, 1): one row that
+    all outputs share (``bcast_o``), read in place.  Same parameters as the
     rows kernel."""
-    ins = [a for a in args if a.kind == 'in']
+    all_ins = [a for a in args if a.kind == 'in']
+    ins = [a for a in all_ins if not a.bcast_o]
     assert ins and group in (1, 2, 4, 8, 16, 32, 64) and rows % (BLOCK // group) == 0
     nt = 'true' if stream_hint else 'false'
     params = _fast_params(args, 'ptrdiff_t', False, False)
@@ -478,8 +480,11 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     src.append('    for (int _jq = _g; _jq < %d; _jq += %d) {' % (width, group))
     src.append('      const int _j = (_jq + _rot >= %d) ? (_jq + _rot - %d) : (_jq + _rot);' % (width, width))
     src.append('      const IndexT _J = _j;')
-    for a in ins:
-        src.append('      const %s %s(_slab_%s[_r * %d + _j]);' % (a.var_t, a.name, a.name, width))
+    for a in all_ins:
+        if a.bcast_o:
+            src.append('      const %s %s(_p_%s[_j]);' % (a.var_t, a.name, a.name))
+        else:
+            src.append('      const %s %s(_slab_%s[_r * %d + _j]);' % (a.var_t, a.name, a.name, width))
     src.append('      _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
     src.append('      _s = REDUCE(_s, _a);')
     src.append('    }')

@@ -493,9 +493,17 @@ class _AbstractReductionKernel:
         items = [a.dtype.itemsize for a in ins]
         if n_red * max(items) > _tuning.get('rows_flat_max_bytes'):
             return None
+        dense = 0
         for a, s_o, s_r in zip(ins, so_in, sr):
-            if s_r != a.dtype.itemsize or s_o != n_red * a.dtype.itemsize:
+            if s_r != a.dtype.itemsize:
                 return None
+            if s_o == n_red * a.dtype.itemsize:
+                dense += 1
+            elif s_o != 0:            # one row shared by all outputs is read in place
+                return None
+        if not dense:
+            return None
+        items = [a.dtype.itemsize for a, s_o in zip(ins, so_in) if s_o]
         if mode == 'auto':
             # a lane group per row does as well when a row is a whole number
             # of vectors that fills a power-of-two group of lanes, or three
@@ -524,7 +532,7 @@ class _AbstractReductionKernel:
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
         group, rows = geometry
-        rargs = self._rargs(in_args, out_args)
+        rargs = self._rargs(in_args, out_args, bcast_o=[s == 0 for s in so_in])
         stream_hint = _tuning.stream_policy(
             _tuning.get('rows_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('rows_flat', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,

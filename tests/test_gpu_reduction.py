@@ -434,3 +434,28 @@ def test_reduction_over_the_outer_and_the_innermost_axis(shape, dtype):
     out = cp.zeros((2 * shape[1],), dx.max().dtype)
     dx.max(axis=(0, 2), out=out[::2])
     assert_exact(out.get()[::2], x.max(axis=(0, 2)))
+
+
+@pytest.mark.parametrize('width', [3, 7, 10, 33, 100])
+def test_short_rows_with_a_row_of_weights_shared_by_all_rows(width):
+    rng = np.random.default_rng(44)
+    x = rng.standard_normal((50001, width)).astype(np.float32)
+    y = rng.standard_normal((50001, width)).astype(np.float32)
+    w = rng.uniform(0, 1, width).astype(np.float32)
+    k = cp.ReductionKernel('T x, T y, T w', 'T z', '(x - y) * (x - y) * w', 'a + b', 'z = a', '0',
+                           'weighted_sqdiff_rows')
+    got = k(cp.asarray(x), cp.asarray(y), cp.asarray(w), axis=1).get()
+    want = (((x.astype(np.float64) - y) ** 2) * w).sum(axis=1)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-5)
+    fused = cp.fuse(lambda a, b, c: cp.sum((a - b) ** 2 * c, axis=-1))
+    np.testing.assert_allclose(fused(cp.asarray(x), cp.asarray(y), cp.asarray(w)).get(), want,
+                               rtol=2e-5, atol=1e-5)
+    am = cp.ReductionKernel('T x, T w', 'int64 z', 'cupy_pair(x * w, _J)', 'a.v >= b.v ? a : b',
+                            'z = a.i', 'cupy_pair(-1e30f, 0)', 'weighted_argmax_rows',
+                            reduce_type='cupy_pair',
+                            preamble='struct cupy_pair { float v; long long i; '
+                                     '__device__ cupy_pair() : v(0), i(0) {} '
+                                     '__device__ cupy_pair(float a, long long b) : v(a), i(b) {} };')
+    got = am(cp.asarray(x), cp.asarray(w), axis=1).get()
+    prod = x * w
+    assert np.array_equal(prod[np.arange(len(got)), got], prod.max(axis=1))
