@@ -422,10 +422,10 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     even widths too.
 
     Every input must have element strides (width, 1), or (0, 1): one row that
-    all outputs share (``bcast_o``), read in place.  Same parameters as the
-    rows kernel."""
+    all outputs share (``bcast_o``), or a value per row (``bcast_r``), both
+    read in place.  Same parameters as the rows kernel."""
     all_ins = [a for a in args if a.kind == 'in']
-    ins = [a for a in all_ins if not a.bcast_o]
+    ins = [a for a in all_ins if not (a.bcast_o or a.bcast_r)]
     assert ins and group in (1, 2, 4, 8, 16, 32, 64) and rows % (BLOCK // group) == 0
     nt = 'true' if stream_hint else 'false'
     params = _fast_params(args, 'ptrdiff_t', False, False)
@@ -481,7 +481,10 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     src.append('      const int _j = (_jq + _rot >= %d) ? (_jq + _rot - %d) : (_jq + _rot);' % (width, width))
     src.append('      const IndexT _J = _j;')
     for a in all_ins:
-        if a.bcast_o:
+        if a.bcast_r:
+            src.append('      const %s %s(_p_%s[(_row0 + _r) * _so_%s]);' % (
+                a.var_t, a.name, a.name, a.name))
+        elif a.bcast_o:
             src.append('      const %s %s(_p_%s[_j]);' % (a.var_t, a.name, a.name))
         else:
             src.append('      const %s %s(_slab_%s[_r * %d + _j]);' % (a.var_t, a.name, a.name, width))

@@ -495,6 +495,8 @@ class _AbstractReductionKernel:
             return None
         dense = 0
         for a, s_o, s_r in zip(ins, so_in, sr):
+            if s_r == 0 and s_o % a.dtype.itemsize == 0:
+                continue              # a value per row, read in place
             if s_r != a.dtype.itemsize:
                 return None
             if s_o == n_red * a.dtype.itemsize:
@@ -503,7 +505,7 @@ class _AbstractReductionKernel:
                 return None
         if not dense:
             return None
-        items = [a.dtype.itemsize for a, s_o in zip(ins, so_in) if s_o]
+        items = [a.dtype.itemsize for a, s_o, s_r in zip(ins, so_in, sr) if s_o and s_r]
         if mode == 'auto':
             # a lane group per row does as well when a row is a whole number
             # of vectors that fills a power-of-two group of lanes, or three
@@ -532,7 +534,8 @@ class _AbstractReductionKernel:
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
         group, rows = geometry
-        rargs = self._rargs(in_args, out_args, bcast_o=[s == 0 for s in so_in])
+        rargs = self._rargs(in_args, out_args, bcast_r=[s == 0 for s in sr],
+                            bcast_o=[s_o == 0 and s_r != 0 for s_o, s_r in zip(so_in, sr)])
         stream_hint = _tuning.stream_policy(
             _tuning.get('rows_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('rows_flat', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,

@@ -450,6 +450,11 @@ def test_short_rows_with_a_row_of_weights_shared_by_all_rows(width):
     fused = cp.fuse(lambda a, b, c: cp.sum((a - b) ** 2 * c, axis=-1))
     np.testing.assert_allclose(fused(cp.asarray(x), cp.asarray(y), cp.asarray(w)).get(), want,
                                rtol=2e-5, atol=1e-5)
+    # a value per row beside the row itself: the variance's pivot
+    np.testing.assert_allclose(cp.asarray(x).var(axis=1).get(), x.astype(np.float64).var(axis=1),
+                               rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(cp.asarray(x + 1000).std(axis=1, ddof=1).get(),
+                               (x + 1000).astype(np.float64).std(axis=1, ddof=1), rtol=2e-3)
     am = cp.ReductionKernel('T x, T w', 'int64 z', 'cupy_pair(x * w, _J)', 'a.v >= b.v ? a : b',
                             'z = a.i', 'cupy_pair(-1e30f, 0)', 'weighted_argmax_rows',
                             reduce_type='cupy_pair',
