@@ -457,6 +457,12 @@ def _var_pivot(a, axis):
         key = tuple(slice(pick(n), pick(n) + 1) if ax in axis else slice(None)
                     for ax, n in enumerate(a.shape))
         probes.append(a[key])
+    if internal.prod([a.shape[ax] for ax in axis]) <= 64:
+        # few elements per output: any of them is close enough (the error grows
+        # with the number of elements times the squared distance of the pivot
+        # from the mean, and the pivot is one of the elements); the first one is
+        # a view, no kernel
+        return probes[0]
     return _median3(*probes)
 
 
