@@ -412,6 +412,14 @@ __device__ __forceinline__ var_st<T> operator+(const var_st<T>& a, const var_st<
   r.s2 = a.s2 + b.s2;
   return r;
 }
+// Median of three probes of the data: the pivot.  A NaN probe may give any
+// value here, the probe itself then makes the sums NaN.
+template <typename S>
+__device__ __forceinline__ S var_med3(S a, S b, S c) {
+  const S lo = a < b ? a : b;
+  const S hi = a < b ? b : a;
+  return c < lo ? lo : (c > hi ? hi : c);
+}
 template <typename T>
 __device__ __forceinline__ T var_finish(const var_st<T>& a, T inv_n, T alpha) {
   const T m2 = a.s2 - a.s1 * a.s1 * inv_n;
@@ -420,38 +428,36 @@ __device__ __forceinline__ T var_finish(const var_st<T>& a, T inv_n, T alpha) {
 '''
 
 _var_onepass_cores = {}
-_median3 = None
 
 
-def _var_onepass(out_name):
+def _var_onepass(out_name, probes=1):
     """ReductionKernel of the one-pass variance, accumulating in double for a
-    float64 result and in float otherwise (as the sums of those types do)."""
+    float64 result and in float otherwise (as the sums of those types do).
+    The pivot is one probe of the data per output, or the median of three,
+    taken inside the kernel."""
     from cupy_amd._core._reduction import ReductionKernel
-    ker = _var_onepass_cores.get(out_name)
+    ker = _var_onepass_cores.get((out_name, probes))
     if ker is None:
         work, scalar_t = ('double', 'float64') if out_name == 'float64' else ('float', 'float32')
+        if probes == 1:
+            params, pivot = 'S k', 'k'
+        else:
+            params, pivot = 'S k0, S k1, S k2', 'var_med3(k0, k1, k2)'
         ker = ReductionKernel(
-            'S x, S k, %s inv_n, %s alpha' % (scalar_t, scalar_t), '%s out' % out_name,
-            'var_st<%s>(static_cast<%s>(x) - static_cast<%s>(k))' % (work, work, work),
+            'S x, %s, %s inv_n, %s alpha' % (params, scalar_t, scalar_t), '%s out' % out_name,
+            'var_st<%s>(static_cast<%s>(x) - static_cast<%s>(%s))' % (work, work, work, pivot),
             'a + b', 'out = var_finish<%s>(a, inv_n, alpha)' % work, 'var_st<%s>()' % work,
-            'cupy_var_' + out_name, reduce_type='var_st<%s>' % work,
+            'cupy_var%d_%s' % (probes, out_name), reduce_type='var_st<%s>' % work,
             preamble=_var_onepass_preamble)
-        _var_onepass_cores[out_name] = ker
+        _var_onepass_cores[(out_name, probes)] = ker
     return ker
 
 
 def _var_pivot(a, axis):
-    """Per output, the median of the first, middle and last element along the
-    reduced axes (shape of ``a`` with the reduced axes of length one): a value
-    near the data unless two of the three probes are outliers."""
-    global _median3
-    if _median3 is None:
-        from cupy_amd._core._kernel import ElementwiseKernel
-        _median3 = ElementwiseKernel(
-            'T a, T b, T c', 'T k',
-            'const T lo = a < b ? a : b; const T hi = a < b ? b : a;'
-            'k = (a != a || b != b) ? (a != a ? a : b) : (c < lo ? lo : (c > hi ? hi : c))',
-            'cupy_var_pivot')
+    """Per output, the probes of the data that give the pivot, as views (shape
+    of ``a`` with the reduced axes of length one): the first, middle and last
+    element along the reduced axes, whose median is near the data unless two
+    of the three are outliers."""
     probes = []
     for pick in (lambda n: 0, lambda n: n // 2, lambda n: n - 1):
         key = tuple(slice(pick(n), pick(n) + 1) if ax in axis else slice(None)
@@ -460,10 +466,9 @@ def _var_pivot(a, axis):
     if internal.prod([a.shape[ax] for ax in axis]) <= 64:
         # few elements per output: any of them is close enough (the error grows
         # with the number of elements times the squared distance of the pivot
-        # from the mean, and the pivot is one of the elements); the first one is
-        # a view, no kernel
-        return probes[0]
-    return _median3(*probes)
+        # from the mean, and the pivot is one of the elements)
+        return probes[:1]
+    return probes
 
 
 def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
@@ -495,9 +500,9 @@ def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
     if (a.dtype.kind in 'biuf' and dtype_out.kind == 'f' and dtype_out.itemsize <= 8
             and items > 0 and (out is None or out.dtype == dtype_out)):
         axis = tuple(internal._normalize_axis_index(ax, a.ndim) for ax in axis)
-        pivot = _var_pivot(a, axis)
-        args = (a, pivot, 1. / items, alpha) + (() if out is None else (out,))
-        return _var_onepass(dtype_out.name)(*args, axis=axis, keepdims=keepdims)
+        probes = _var_pivot(a, axis)
+        args = (a, *probes, 1. / items, alpha) + (() if out is None else (out,))
+        return _var_onepass(dtype_out.name, len(probes))(*args, axis=axis, keepdims=keepdims)
     arrmean = a.mean(axis=axis, dtype=dtype_mean, out=None, keepdims=True)
     if out is None:
         name = dtype_out.name if dtype_out.name in ('float16', 'float32') else 'float64'
