@@ -458,6 +458,28 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
         src.append('    if (_q + _V_%s <= _count) _st_%s[_t] = cupy::load_vec<%s, _V_%s, %s>(_src_%s + _q);' % (
             a.name, a.name, a.store_t, a.name, nt, a.name))
         src.append('  }')
+    # values per row are requested along with the rows and handed over through
+    # the LDS as well: a load after the barrier would be waited for by itself
+    row_vals = [a for a in all_ins if a.bcast_r]
+    n_rv = (rows + BLOCK - 1) // BLOCK
+    for a in row_vals:
+        src.append('  __shared__ __attribute__((aligned(16))) char _rowv_raw_%s[%d * sizeof(%s)];' % (
+            a.name, rows, a.store_t))
+        src.append('  %s* _rowv_%s = reinterpret_cast<%s*>(_rowv_raw_%s);' % (
+            a.store_t, a.name, a.store_t, a.name))
+        src.append('  %s _rvst_%s[%d];' % (a.store_t, a.name, n_rv))
+        src.append('#pragma unroll')
+        src.append('  for (int _t = 0; _t < %d; ++_t) {' % n_rv)
+        src.append('    const int _rr = _t * %d + threadIdx.x;' % BLOCK)
+        src.append('    if (_rr < _nrows) _rvst_%s[_t] = _p_%s[(_row0 + _rr) * _so_%s];' % (
+            a.name, a.name, a.name))
+        src.append('  }')
+    for a in row_vals:
+        src.append('#pragma unroll')
+        src.append('  for (int _t = 0; _t < %d; ++_t) {' % n_rv)
+        src.append('    const int _rr = _t * %d + threadIdx.x;' % BLOCK)
+        src.append('    if (_rr < _nrows) _rowv_%s[_rr] = _rvst_%s[_t];' % (a.name, a.name))
+        src.append('  }')
     for a in ins:
         src.append('#pragma unroll')
         src.append('  for (int _t = 0; _t < _T_%s; ++_t) {' % a.name)
@@ -482,8 +504,7 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     src.append('      const IndexT _J = _j;')
     for a in all_ins:
         if a.bcast_r:
-            src.append('      const %s %s(_p_%s[(_row0 + _r) * _so_%s]);' % (
-                a.var_t, a.name, a.name, a.name))
+            src.append('      const %s %s(_rowv_%s[_r]);' % (a.var_t, a.name, a.name))
         elif a.bcast_o:
             src.append('      const %s %s(_p_%s[_j]);' % (a.var_t, a.name, a.name))
         else:
