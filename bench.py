@@ -231,7 +231,7 @@ def build_next_cases(cp):
 
     def gpu_var():
         res_var[0] = dm.var(axis=0)
-    add('var f32 16384x8192 axis=0 (one pass; pivot and combine kernels included)', m.nbytes + 8192 * 4,
+    add('var f32 16384x8192 axis=0 (one pass; combine kernel included)', m.nbytes + 8192 * 4,
         gpu_var, lambda: m.var(axis=0),
         lambda: close(res_var[0], m.var(axis=0, dtype=np.float64), 1e-4), 'cupy_var_core')
     mn = m.copy()
