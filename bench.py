@@ -233,7 +233,7 @@ def build_next_cases(cp):
         res_var[0] = dm.var(axis=0)
     add('var f32 16384x8192 axis=0 (one pass; combine kernel included)', m.nbytes + 8192 * 4,
         gpu_var, lambda: m.var(axis=0),
-        lambda: close(res_var[0], m.var(axis=0, dtype=np.float64), 1e-4), 'cupy_var_core')
+        lambda: close(res_var[0], m.var(axis=0, dtype=np.float64), 1e-4), 'cupy_var3_float32')
     mn = m.copy()
     mn[::7, ::5] = np.nan
     dmn = cp.asarray(mn)

@@ -428,6 +428,7 @@ __device__ __forceinline__ T var_finish(const var_st<T>& a, T inv_n, T alpha) {
 '''
 
 _var_onepass_cores = {}
+_FLOAT_NAMES = {'e': 'float16', 'f': 'float32', 'd': 'float64'}
 
 
 def _var_onepass(out_name, probes=1):
@@ -458,11 +459,19 @@ def _var_pivot(a, axis):
     of ``a`` with the reduced axes of length one): the first, middle and last
     element along the reduced axes, whose median is near the data unless two
     of the three are outliers."""
-    probes = []
-    for pick in (lambda n: 0, lambda n: n // 2, lambda n: n - 1):
-        key = tuple(slice(pick(n), pick(n) + 1) if ax in axis else slice(None)
-                    for ax, n in enumerate(a.shape))
-        probes.append(a[key])
+    # the three views share shape and strides: one is built, the others are
+    # copies of it that start elsewhere (slicing three times costs more host
+    # time than the kernel runs for mid-sized arrays)
+    shape = tuple(1 if ax in axis else n for ax, n in enumerate(a.shape))
+    first = a._view(shape, a.strides)
+    probes = [first]
+    for pick in (lambda n: n // 2, lambda n: n - 1):
+        offset = sum(pick(a.shape[ax]) * a.strides[ax] for ax in axis)
+        v = object.__new__(type(first))
+        v.__dict__.update(first.__dict__)
+        if offset:
+            v.data = first.data + offset
+        probes.append(v)
     if internal.prod([a.shape[ax] for ax in axis]) <= 64:
         # few elements per output: any of them is close enough (the error grows
         # with the number of elements times the squared distance of the pivot
@@ -502,7 +511,9 @@ def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
         axis = tuple(internal._normalize_axis_index(ax, a.ndim) for ax in axis)
         probes = _var_pivot(a, axis)
         args = (a, *probes, 1. / items, alpha) + (() if out is None else (out,))
-        return _var_onepass(dtype_out.name, len(probes))(*args, axis=axis, keepdims=keepdims)
+        # (numpy's dtype.name is computed on every access)
+        out_name = _FLOAT_NAMES[dtype_out.char]
+        return _var_onepass(out_name, len(probes))(*args, axis=axis, keepdims=keepdims)
     arrmean = a.mean(axis=axis, dtype=dtype_mean, out=None, keepdims=True)
     if out is None:
         name = dtype_out.name if dtype_out.name in ('float16', 'float32') else 'float64'
