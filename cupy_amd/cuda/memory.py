@@ -10,7 +10,6 @@ import ctypes
 import gc
 import threading
 import warnings
-import weakref
 
 from cupy_amd import _dryrun
 from cupy_amd import _rt
@@ -100,13 +99,17 @@ class PooledMemory(BaseMemory):
         self.ptr = ptr
         self.size = size
         self.device_id = device_id
-        self._pool = weakref.ref(pool)
+        # A strong reference to the native pool's holder, not a weak one to
+        # the Python pool: the collector clears weak references that are part
+        # of a garbage cycle BEFORE it runs the cycle's finalisers, so a block
+        # owned by such a cycle would find its pool gone and never return.
+        self._pool = pool._native
 
     def free(self):
         ptr, self.ptr = self.ptr, 0
         if not ptr:
             return
-        pool = self._pool()
+        pool = self._pool
         hooks = _memory_hook.get_memory_hooks() if _memory_hook._has_memory_hooks() else None
         if hooks:
             kw = dict(device_id=self.device_id, mem_size=self.size, mem_ptr=ptr,
@@ -262,6 +265,34 @@ def _parse_limit_string(limit=None):
     return {'size': size, 'fraction': fraction}
 
 
+class _NativePool:
+    """Owner of one native pool handle and of the callbacks it calls.  Shared by
+    the Python pool and every block it handed out, so the native bookkeeping
+    lives until the last block has come back."""
+
+    __slots__ = ('handle', 'callbacks', 'live')
+
+    def __init__(self, alloc_cb, free_cb, live):
+        self.live = live
+        self.callbacks = (_rt.POOL_ALLOC_FN(alloc_cb), _rt.POOL_FREE_FN(free_cb))
+        self.handle = ctypes.c_void_p()
+        _rt.check(_rt.lib.rt_pool_create_with_allocator(
+            ctypes.byref(self.handle), self.callbacks[0], self.callbacks[1], None))
+
+    def _free(self, ptr, size):
+        handle = self.handle
+        if handle:
+            _rt.lib.rt_pool_free(handle, ptr)
+
+    def __del__(self):
+        handle, self.handle = getattr(self, 'handle', None), None
+        if handle:
+            try:
+                _rt.lib.rt_pool_destroy(handle)
+            except Exception:
+                pass
+
+
 class SingleDeviceMemoryPool:
     """Caching pool of one device.
 
@@ -271,9 +302,7 @@ class SingleDeviceMemoryPool:
 
     def __init__(self, allocator=None):
         self._device_id = _device.get_device_id()
-        self._handle = ctypes.c_void_p()
         self._live = {}      # address -> MemoryPointer from a Python allocator
-        self._callbacks = None
         # Fresh memory always comes through this Python callback (a pool hit
         # never gets here, and a device allocation costs far more than the
         # call): that is where a custom allocator plugs in and where the
@@ -308,21 +337,11 @@ class SingleDeviceMemoryPool:
         def free_cb(ctx, address, size):
             live.pop(address, None)
 
-        self._callbacks = (_rt.POOL_ALLOC_FN(alloc_cb), _rt.POOL_FREE_FN(free_cb))
-        _rt.check(_rt.lib.rt_pool_create_with_allocator(
-            ctypes.byref(self._handle), self._callbacks[0],
-            self._callbacks[1], None))
+        self._native = _NativePool(alloc_cb, free_cb, live)
+        self._handle = self._native.handle
         limit = _parse_limit_string()
         if limit['size'] is not None or limit['fraction'] is not None:
             self.set_limit(**limit)
-
-    def __del__(self):
-        handle, self._handle = getattr(self, '_handle', None), None
-        if handle:
-            try:
-                _rt.lib.rt_pool_destroy(handle)
-            except Exception:
-                pass
 
     # -- allocation -------------------------------------------------------------
     def malloc(self, size):
@@ -366,9 +385,7 @@ class SingleDeviceMemoryPool:
         return MemoryPointer(mem, 0)
 
     def _free(self, ptr, size):
-        handle = self._handle
-        if handle:
-            _rt.lib.rt_pool_free(handle, ptr)
+        self._native._free(ptr, size)
 
     def free_all_blocks(self, stream=None):
         if stream is None:

@@ -355,3 +355,181 @@ def test_threads_hammering_one_pool(pool):
     assert not errors
     assert pool.used_bytes() == 0
     assert pool.used_bytes() + pool.free_bytes() == pool.total_bytes()
+
+
+def _run_with_deadline(fn, seconds=20):
+    """Runs ``fn`` in a thread of its own: a pool that locks itself up fails
+    the test instead of wedging the whole run."""
+    result = {}
+
+    def body():
+        try:
+            result['value'] = fn()
+        except BaseException as e:      # pragma: no cover
+            result['error'] = e
+
+    t = threading.Thread(target=body, daemon=True)
+    t.start()
+    t.join(seconds)
+    assert not t.is_alive(), 'the pool did not return (self-deadlock)'
+    if 'error' in result:
+        raise result['error']
+    return result.get('value')
+
+
+def test_allocator_may_free_into_the_same_pool(monkeypatch):
+    # The allocator callback runs arbitrary code; here it drops the last
+    # reference to another block of the very pool that is calling it.
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+    held = []
+
+    def alloc(size):
+        if held:
+            held.pop()          # PooledMemory.__del__ -> rt_pool_free
+        return mock_alloc(size)
+
+    pool = memory.SingleDeviceMemoryPool(allocator=alloc)
+
+    def scenario():
+        held.append(pool.malloc(unit * 2))
+        big = pool.malloc(unit * 64)     # cache miss -> callback -> free
+        return big.ptr, pool.used_bytes(), pool.n_free_blocks()
+
+    ptr, used, nfree = _run_with_deadline(scenario)
+    assert ptr
+    assert not held
+    assert used == unit * 64
+    assert nfree == 1
+
+
+def test_gc_inside_the_allocator_callback(monkeypatch):
+    # A collector pass that starts inside the callback and finalises a
+    # PooledMemory owned by a garbage cycle re-enters the pool on the same
+    # thread.
+    import gc
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+
+    def alloc(size):
+        gc.collect()
+        return mock_alloc(size)
+
+    pool = memory.SingleDeviceMemoryPool(allocator=alloc)
+
+    class Node:
+        pass
+
+    def scenario():
+        for k in range(4):
+            a, b = Node(), Node()
+            a.other, b.other = b, a
+            a.block = pool.malloc(unit * (k + 1))
+            del a, b                         # a cycle that owns a pool block
+            pool.malloc(unit * (100 + k))    # miss -> callback -> gc -> free
+        gc.collect()
+        return pool.used_bytes()
+
+    gc.disable()
+    try:
+        used = _run_with_deadline(scenario)
+    finally:
+        gc.enable()
+    assert used == 0
+    assert pool.used_bytes() + pool.free_bytes() == pool.total_bytes()
+
+
+def test_hook_may_query_the_pool_from_the_callback(monkeypatch):
+    from cupy_amd.cuda import memory_hook
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+    pool = memory.SingleDeviceMemoryPool(allocator=mock_alloc)
+    seen = []
+
+    class Hook(memory_hook.MemoryHook):
+        name = 'QueryHook'
+
+        def alloc_preprocess(self, **kwargs):
+            seen.append(pool.used_bytes())
+
+        def alloc_postprocess(self, **kwargs):
+            seen.append(pool.total_bytes())
+
+    def scenario():
+        with Hook():
+            p = pool.malloc(unit * 3)
+        return p.ptr
+
+    assert _run_with_deadline(scenario)
+    assert seen == [0, 0]
+
+
+def test_slow_allocator_calls_overlap(monkeypatch):
+    # Eight threads miss the cache at the same time; the allocator takes
+    # 0.2 s.  With the pool's lock held across the callback this would take
+    # 8 x 0.2 s and never show two calls in flight.
+    import time
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+    state = {'now': 0, 'peak': 0}
+    guard = threading.Lock()
+
+    def alloc(size):
+        with guard:
+            state['now'] += 1
+            state['peak'] = max(state['peak'], state['now'])
+        time.sleep(0.2)
+        with guard:
+            state['now'] -= 1
+        return mock_alloc(size)
+
+    pool = memory.SingleDeviceMemoryPool(allocator=alloc)
+    start = threading.Barrier(8)
+    blocks = []
+
+    def worker(k):
+        start.wait()
+        blocks.append(pool.malloc(unit * (k + 1)))
+
+    def scenario():
+        threads = [threading.Thread(target=worker, args=(k,)) for k in range(8)]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        return time.perf_counter() - t0
+
+    elapsed = _run_with_deadline(scenario)
+    assert len({b.ptr for b in blocks}) == 8
+    assert state['peak'] >= 2
+    assert elapsed < 1.2
+    assert pool.used_bytes() == sum(unit * (k + 1) for k in range(8))
+
+
+def test_limit_holds_for_requests_side_by_side(monkeypatch):
+    import time
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+
+    def alloc(size):
+        time.sleep(0.05)
+        return mock_alloc(size)
+
+    pool = memory.SingleDeviceMemoryPool(allocator=alloc)
+    pool.set_limit(size=unit * 10)
+    start = threading.Barrier(4)
+    got, refused = [], []
+
+    def worker():
+        start.wait()
+        try:
+            got.append(pool.malloc(unit * 4))
+        except memory.OutOfMemoryError:
+            refused.append(1)
+
+    def scenario():
+        threads = [threading.Thread(target=worker) for _ in range(4)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+
+    _run_with_deadline(scenario)
+    assert len(got) == 2 and len(refused) == 2
+    assert pool.total_bytes() <= unit * 10
