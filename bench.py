@@ -37,24 +37,18 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch (read + written) from the rocprofv3 FETCH_SIZE and
 # WRITE_SIZE counters, scaled by what the same counters read for the plain copy
-# kernel that --calibrate adds (2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE on this
-# device); the summary of those runs is profiles/pmc_traffic_bench_suite.md.
-# Two-pass reductions count both of their kernels.
-MEASURED_TRAFFIC_BYTES = {
-    'C1 saxpy f32 2^26': 536849410 + 268397829,
-    'C2a x.T*y f32(T)xf16 8192^2': 271083170 + 268397701,
-    'C2b tmp+1 f32 8192^2': 268435456 + 268720216,
-    'C3 sum float32 axis=1 16384^2': 1073677445 + 524886,
-    'C3 sum float32 axis=0 16384^2': 1073677317 + 2096857 + 2122574 + 65527,
-    'C3 sum float32 axis=None 16384^2': 1073678341 + 65719 + 11391 + 32,
-    'C3 sum float64 axis=1 8192^2': 536851842 + 262427,
-    'C3 sum float64 axis=0 8192^2': 536851458 + 2096857 + 2122574 + 65527,
-    'C3 sum float64 axis=None 8192^2': 536852482 + 65591 + 19582 + 32,
-    'C4 argmax i32 (2^20,128)': 536870912 + 8392036,
-    'C4 argmin i32 (2^20,128)': 536869888 + 8396707,
-    'C4 argmax f32 (2^16,4096)': 1073711235 + 525942,
-    'C5 fused sum((x-y)^2*w) f16 (2^18,256)': 268443647 + 1048429,
-}
+# kernel that --calibrate adds.  `python bench_profiles.py pmc` digests the
+# counter runs into this file (operation name -> bytes; two-pass reductions
+# count both of their kernels); an operation it does not list reports null.
+TRAFFIC_FILE = os.path.join(ROOT, 'bench_traffic.json')
+
+
+def measured_traffic():
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f).get('hbm_bytes_per_launch', {})
+    except (OSError, ValueError):
+        return {}
 
 
 def log(*a):
@@ -130,10 +124,17 @@ def build_cases(cp, scale=1):
             def cpu(a=a, axis=axis, hout=hout):
                 return np.sum(a, axis=axis, out=hout)
 
-            def check(a=a, axis=axis, out=out, rtol=rtol):
+            def check(a=a, axis=axis, out=out, rtol=rtol, dt=dt):
+                # backward bound against NumPy's own sum, and the bound on the
+                # result itself: |got - float64 sum| <= rtol * max(|float64
+                # sum|, sigma * sqrt(N reduced)), which a missing partial breaks
+                got = out.get()
                 mag = np.abs(a).sum(axis=axis, dtype=np.float64)
-                err = np.abs(out.get().astype(np.float64) - np.sum(a, axis=axis))
-                return bool(np.all(err <= rtol * mag))
+                err = np.abs(got.astype(np.float64) - np.sum(a, axis=axis))
+                ratio = oracle.check_sum_forward(got, a, axis, dt)
+                log('  forward bound %s axis=%s: largest err/bound %.3g' % (
+                    np.dtype(dt).name, axis, ratio))
+                return bool(np.all(err <= rtol * mag)) and ratio <= 1.0
 
             add('C3 sum %s axis=%s %d^2' % (np.dtype(dt).name, axis, n), 'C3',
                 a.nbytes + (item if axis is None else n * item), gpu, cpu, check, 'cupy_sum')
@@ -407,6 +408,141 @@ def build_layout_cases(cp):
     return cases
 
 
+CEILING_SOURCE = r'''
+#include <cupy/carray.cuh>
+typedef float T;
+typedef cupy::Vec<T, 4> V4;
+#define KBLOCK 512
+#define KUN 4
+// Plain streaming kernels, written by hand in the shape that measured best on
+// this device: 16 bytes per lane and access, four accesses in flight per lane
+// before the first is used, grid-stride over whole blocks of work, streaming
+// (non-temporal) hints on loads and stores.  n is a multiple of 4*KBLOCK*KUN.
+extern "C" __global__ void __launch_bounds__(KBLOCK)
+ceil_read(const T* __restrict__ x, T* __restrict__ sink, long nvec) {
+  const long per_iter = (long)KBLOCK * KUN;
+  float s = 0;
+  for (long base = (long)blockIdx.x * per_iter; base + per_iter <= nvec;
+       base += (long)gridDim.x * per_iter) {
+    V4 a[KUN];
+#pragma unroll
+    for (int u = 0; u < KUN; ++u)
+      a[u] = cupy::load_vec<T, 4, true>(x + (base + u * KBLOCK + threadIdx.x) * 4);
+#pragma unroll
+    for (int u = 0; u < KUN; ++u) s += a[u].v[0] + a[u].v[1] + a[u].v[2] + a[u].v[3];
+  }
+  if (s == 12345.678f) sink[0] = s;   // keeps the loads alive, never true for the zeros read
+}
+extern "C" __global__ void __launch_bounds__(KBLOCK)
+ceil_fill(T* __restrict__ z, long nvec) {
+  const long per_iter = (long)KBLOCK * KUN;
+  V4 a;
+  a.v[0] = a.v[1] = a.v[2] = a.v[3] = 1.0f;
+  for (long base = (long)blockIdx.x * per_iter; base + per_iter <= nvec;
+       base += (long)gridDim.x * per_iter) {
+#pragma unroll
+    for (int u = 0; u < KUN; ++u)
+      cupy::store_vec<T, 4, true>(z + (base + u * KBLOCK + threadIdx.x) * 4, a);
+  }
+}
+extern "C" __global__ void __launch_bounds__(KBLOCK)
+ceil_copy(const T* __restrict__ x, T* __restrict__ z, long nvec) {
+  const long per_iter = (long)KBLOCK * KUN;
+  for (long base = (long)blockIdx.x * per_iter; base + per_iter <= nvec;
+       base += (long)gridDim.x * per_iter) {
+    V4 a[KUN];
+#pragma unroll
+    for (int u = 0; u < KUN; ++u)
+      a[u] = cupy::load_vec<T, 4, true>(x + (base + u * KBLOCK + threadIdx.x) * 4);
+#pragma unroll
+    for (int u = 0; u < KUN; ++u)
+      cupy::store_vec<T, 4, true>(z + (base + u * KBLOCK + threadIdx.x) * 4, a[u]);
+  }
+}
+extern "C" __global__ void __launch_bounds__(KBLOCK)
+ceil_saxpy(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ z, long nvec) {
+  const long per_iter = (long)KBLOCK * (KUN / 2);
+  for (long base = (long)blockIdx.x * per_iter; base + per_iter <= nvec;
+       base += (long)gridDim.x * per_iter) {
+    V4 a[KUN / 2], b[KUN / 2];
+#pragma unroll
+    for (int u = 0; u < KUN / 2; ++u) {
+      a[u] = cupy::load_vec<T, 4, true>(x + (base + u * KBLOCK + threadIdx.x) * 4);
+      b[u] = cupy::load_vec<T, 4, true>(y + (base + u * KBLOCK + threadIdx.x) * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < KUN / 2; ++u) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) a[u].v[k] = 2.5f * a[u].v[k] + b[u].v[k];
+      cupy::store_vec<T, 4, true>(z + (base + u * KBLOCK + threadIdx.x) * 4, a[u]);
+    }
+  }
+}
+'''
+
+
+def build_ceiling_cases(cp):
+    """The streaming ceiling of the device: what plain read-only, write-only,
+    copy and two-in-one-out kernels reach, (a) written by hand (RawKernel), (b)
+    through ElementwiseKernel / ``sum`` / ``fill`` of this package, (c) as a
+    device-to-device ``rt_memcpy_async``.  Arrays of 256 MiB and 1 GiB; every
+    call works on the next of several buffer sets, so that nothing of a call's
+    operands is left in the 256 MB memory-side cache from the call before."""
+    cases = []
+
+    def add(name, nbytes, gpu, kernel):
+        cases.append(dict(name=name, config='ceiling', bytes=int(nbytes), gpu=gpu,
+                          cpu=lambda: None, check=lambda: True, kernel=kernel))
+
+    mod = cp.RawModule(code=CEILING_SOURCE)
+    k_read, k_fill = mod.get_function('ceil_read'), mod.get_function('ceil_fill')
+    k_copy, k_saxpy = mod.get_function('ceil_copy'), mod.get_function('ceil_saxpy')
+    e_copy = cp.ElementwiseKernel('T x', 'T y', 'y = x', 'ew_copy')
+    e_saxpy = cp.ElementwiseKernel('float32 x, float32 y, float32 a', 'float32 z',
+                                   'z = a * x + y', 'ew_saxpy')
+    sink = cp.zeros((4,), np.float32)
+    block = 512
+    for mib in (256, 1024):
+        n = mib * (1 << 20) // 4
+        nvec = n // 4
+        sets = 6 if mib == 256 else 3
+        xs = [cp.zeros((n,), np.float32) for _ in range(sets)]
+        ys = [cp.zeros((n,), np.float32) for _ in range(sets)]
+        zs = [cp.empty((n,), np.float32) for _ in range(sets)]
+        souts = [cp.empty((), np.float32) for _ in range(sets)]
+        turn = [0]
+
+        def rot(fn, sets=sets, turn=turn):
+            def call():
+                turn[0] = (turn[0] + 1) % sets
+                fn(turn[0])
+            return call
+        grid = (256 * 8,)
+        tag = '%d MiB' % mib
+        add('read   hand-written %s' % tag, 4 * n,
+            rot(lambda i, xs=xs, nvec=nvec: k_read(grid, (block,), (xs[i], sink, nvec))), 'ceil_read')
+        add('read   sum() of this package %s' % tag, 4 * n,
+            rot(lambda i, xs=xs, souts=souts: xs[i].sum(out=souts[i])), 'cupy_sum')
+        add('fill   hand-written %s' % tag, 4 * n,
+            rot(lambda i, zs=zs, nvec=nvec: k_fill(grid, (block,), (zs[i], nvec))), 'ceil_fill')
+        add('fill   ndarray.fill %s' % tag, 4 * n,
+            rot(lambda i, zs=zs: zs[i].fill(1.0)), 'cupy_fill')
+        add('copy   hand-written %s' % tag, 8 * n,
+            rot(lambda i, xs=xs, zs=zs, nvec=nvec: k_copy(grid, (block,), (xs[i], zs[i], nvec))),
+            'ceil_copy')
+        add('copy   ElementwiseKernel %s' % tag, 8 * n,
+            rot(lambda i, xs=xs, zs=zs: e_copy(xs[i], zs[i])), 'ew_copy')
+        add('copy   rt_memcpy_async D2D %s' % tag, 8 * n,
+            rot(lambda i, xs=xs, zs=zs, n=n: zs[i].data.copy_from_device_async(xs[i].data, 4 * n)),
+            'hipMemcpyAsync')
+        add('saxpy  hand-written %s' % tag, 12 * n,
+            rot(lambda i, xs=xs, ys=ys, zs=zs, nvec=nvec:
+                k_saxpy(grid, (block,), (xs[i], ys[i], zs[i], nvec))), 'ceil_saxpy')
+        add('saxpy  ElementwiseKernel %s' % tag, 12 * n,
+            rot(lambda i, xs=xs, ys=ys, zs=zs: e_saxpy(xs[i], ys[i], 2.5, zs[i])), 'ew_saxpy')
+    return cases
+
+
 def time_case_events(cp, fn, repeats, inner):
     """Median over ``repeats`` of the time per call, each sample being
     ``inner`` back-to-back calls bracketed by two events on the launch stream."""
@@ -481,11 +617,17 @@ def main():
     ap.add_argument('--no-detail', action='store_true',
                     help='skip per-operation event timing and launch latency')
     ap.add_argument('--only', default='', help='run only cases whose name contains this')
-    ap.add_argument('--suite', default='configs', choices=('configs', 'next', 'layouts'),
+    ap.add_argument('--suite', default='configs', choices=('configs', 'next', 'layouts', 'ceiling'),
                     help="'configs': the five benchmark configurations (the headline figure); "
                          "'next': scans, statistics, complex types and multi-kernel fused "
                          "functions at shapes of the same size class; 'layouts': offset views, "
-                         "odd and narrow rows, windows, permuted axes, mixed widths")
+                         "odd and narrow rows, windows, permuted axes, mixed widths; 'ceiling': plain "
+                         "read / fill / copy / saxpy streams over rotating buffers, the "
+                         "yardstick the other suites are read against")
+    ap.add_argument('--plan', default='',
+                    help='write the names of the kernels every operation launches, in step '
+                         'order, to this JSON file (bench_profiles.py maps profiler rows to '
+                         'operations with it)')
     ap.add_argument('--calibrate', action='store_true',
                     help='add a plain copy kernel of known size (256 MiB in, 256 MiB out) to '
                          'every step, as the yardstick for hardware traffic counters')
@@ -502,7 +644,10 @@ def main():
     log('device:', props['arch'], props['compute_units'], 'CUs')
     t0 = time.perf_counter()
     cases = (build_cases(cp, args.scale) if args.suite == 'configs' else
-             build_next_cases(cp) if args.suite == 'next' else build_layout_cases(cp))
+             build_next_cases(cp) if args.suite == 'next' else
+             build_ceiling_cases(cp) if args.suite == 'ceiling' else build_layout_cases(cp))
+    if args.suite == 'ceiling':
+        args.no_cpu = True
     if args.only:
         cases = [c for c in cases if args.only in c['name']]
     log('inputs ready in %.1f s' % (time.perf_counter() - t0))
@@ -527,6 +672,29 @@ def main():
     for _ in range(max(args.warmup, 1)):
         step()
     dev.synchronize()
+    if args.plan:
+        from cupy_amd.cuda import function as _function
+        seen = []
+        real_launch = _function.Function.launch_packed
+
+        def spy(self, *a, **k):
+            seen.append(self.name)
+            return real_launch(self, *a, **k)
+        _function.Function.launch_packed = spy
+        plan = []
+        try:
+            for c in cases + ([dict(name='calibration copy 256 MiB', bytes=2 << 28,
+                                    gpu=calib)] if calib is not None else []):
+                del seen[:]
+                c['gpu']()
+                plan.append({'name': c['name'], 'bytes': c['bytes'], 'kernels': list(seen)})
+        finally:
+            _function.Function.launch_packed = real_launch
+        dev.synchronize()
+        os.makedirs(os.path.dirname(os.path.abspath(args.plan)), exist_ok=True)
+        with open(args.plan, 'w') as f:
+            json.dump({'suite': args.suite, 'scale': args.scale, 'steps': args.steps,
+                       'warmup': max(args.warmup, 1), 'operations': plan}, f, indent=1)
     parity = {}
     for c in cases:
         parity[c['name']] = bool(c['check']())
@@ -561,7 +729,7 @@ def main():
         roof = {'bound': 'hbm', 'kernel': dom['kernel'], 'operation': dom['name'],
                 'achieved': dom['gbps'], 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
                 'frac': dom['frac'],
-                'traffic': MEASURED_TRAFFIC_BYTES.get(dom['name'])
+                'traffic': measured_traffic().get(dom['name'])
                 if args.scale == 1 and args.suite == 'configs' else None,
                 'launch_us': dom['us'], 'algorithmic_bytes': dom['bytes']}
     else:
@@ -570,10 +738,10 @@ def main():
 
     cpu = None
     if not args.no_cpu:
-        # NumPy, single-threaded, one warm pass then the best of three passes
-        # over the whole suite (about 10-20 s of CPU work)
+        # NumPy, single-threaded, one warm pass then the best of five passes
+        # over the whole suite (about 15-25 s of CPU work)
         best = None
-        for _ in range(4):
+        for _ in range(6):
             c0 = time.perf_counter()
             for c in cases:
                 c['cpu']()
@@ -587,7 +755,7 @@ def main():
         cpu = {'value': round(total_bytes / best / 1e9, 2), 'unit': 'GB/s', 'cores': 1,
                'kind': 'port',
                'sample': 'one full pass of the same %d operations with NumPy %s on the host '
-                         '(best of 3 after a warm pass, outputs preallocated where NumPy allows); '
+                         '(best of 5 after a warm pass, outputs preallocated where NumPy allows); '
                          '%d host cores visible, CPU: %s' % (
                              len(cases), np.__version__, os.cpu_count(), model),
                'seconds_per_pass': round(best, 3)}
@@ -613,6 +781,9 @@ def main():
                    'NOT the benchmark figure: offset views, odd and narrow rows, windows, permuted '
                    'axes, mixed widths, %d operations per step' % len(cases)
                    if args.suite == 'layouts' and not args.only else
+                   'NOT the benchmark figure: plain streaming kernels over rotating buffers, '
+                   '%d operations per step' % len(cases)
+                   if args.suite == 'ceiling' and not args.only else
                    'REDUCED run (scale=%d only=%r): not the benchmark figure' % (args.scale, args.only),
                    'bytes_per_step': total_bytes, 'operations': len(cases)},
         'frac_of_hbm_peak': round(value / HBM_PEAK_GBPS, 4),

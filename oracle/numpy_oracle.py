@@ -85,6 +85,51 @@ def sum_fp(a, axis=None, dtype=None):
     return np.sum(a, axis=axis, dtype=dtype)
 
 
+def sum_tolerances(dtype):
+    """rtol for floating-point reductions whose order differs from NumPy's."""
+    return {'float16': 1e-3, 'float32': 1e-5, 'float64': 1e-12}[np.dtype(dtype).name]
+
+
+def _square_sum64(a, axis):
+    """Sum of squares in float64, without a float64 copy of a large array."""
+    a = np.asarray(a)
+    if a.size <= 1 << 24 or a.ndim == 0:
+        return np.sum(np.square(a, dtype=np.float64), axis=axis)
+    # large arrays in the tests are matrices: go through them in row blocks
+    step = max(1, (1 << 24) // max(1, a.size // a.shape[0]))
+    axes = tuple(range(a.ndim)) if axis is None else \
+        tuple(ax % a.ndim for ax in (axis if isinstance(axis, tuple) else (axis,)))
+    if 0 in axes:
+        total = None
+        for i in range(0, a.shape[0], step):
+            part = np.sum(np.square(a[i:i + step], dtype=np.float64), axis=axes)
+            total = part if total is None else total + part
+        return total
+    parts = [np.sum(np.square(a[i:i + step], dtype=np.float64), axis=axes)
+             for i in range(0, a.shape[0], step)]
+    return np.concatenate(parts, axis=0)
+
+
+def forward_sum_bound(data, axis, dtype):
+    """``(ref64, bound)`` of the forward check on a floating-point sum:
+    ``|got - ref64| <= rtol * max(|ref64|, sigma * sqrt(N))`` with ``ref64``
+    NumPy's float64 sum of the same data and ``sigma * sqrt(N)`` the root of the
+    addends' square sum -- the size a sum of N values of spread sigma has when
+    its mean is zero, so heavy cancellation does not turn rtol into nothing,
+    while a dropped or doubled block of addends (which moves the result by
+    about sigma * sqrt(block)) is far outside."""
+    ref64 = np.sum(data, axis=axis, dtype=np.float64)
+    floor = np.sqrt(_square_sum64(data, axis))
+    return ref64, sum_tolerances(dtype) * np.maximum(np.abs(ref64), floor)
+
+
+def check_sum_forward(got, data, axis, dtype):
+    """Largest ``err / bound`` of the forward check (<= 1 passes)."""
+    ref64, bound = forward_sum_bound(data, axis, dtype)
+    err = np.abs(np.asarray(got).astype(np.float64).reshape(np.shape(ref64)) - ref64)
+    return float(np.max(err / (bound + 1e-300))) if err.size else 0.0
+
+
 def sum_exact(values):
     """Correctly rounded float64 sum of a 1-d sequence (``math.fsum``)."""
     return math.fsum(float(v) for v in np.asarray(values).ravel())

@@ -1,6 +1,9 @@
 """Comparison helpers shared by the tests."""
 import numpy as np
 
+from oracle.numpy_oracle import (  # noqa: F401  (re-exported for the tests)
+    _square_sum64, check_sum_forward, forward_sum_bound, sum_tolerances)
+
 
 def ulp_distance(a, b):
     """Largest distance, in units in the last place, between two float arrays
@@ -42,15 +45,14 @@ def assert_exact(got, expect):
     assert np.array_equal(got, expect, equal_nan=got.dtype.kind in 'fc')
 
 
-def sum_tolerances(dtype):
-    """rtol for floating-point reductions whose order differs from NumPy's."""
-    return {'float16': 1e-3, 'float32': 1e-5, 'float64': 1e-12}[np.dtype(dtype).name]
+def assert_sum_close(got, expect, addends_abs_sum, dtype, data=None, axis=None):
+    """Two bounds on a floating-point sum whose order differs from NumPy's.
 
-
-def assert_sum_close(got, expect, addends_abs_sum, dtype):
-    """|got - expect| <= rtol * sum(|addends|): the bound any summation order of
-    the same addends meets with room to spare, and that a dropped or doubled
-    addend breaks."""
+    Backward: ``|got - expect| <= rtol * sum(|addends|)``, which any summation
+    order of the same addends meets.  On data that cancels this is very wide
+    (the sum of |a| dwarfs the result), so when the addends themselves are
+    given (``data``, ``axis``) the forward bound of ``forward_sum_bound`` must
+    hold as well: that one a missing partial result does break."""
     got = np.asarray(got)
     expect = np.asarray(expect)
     assert got.dtype == expect.dtype, (got.dtype, expect.dtype)
@@ -59,6 +61,11 @@ def assert_sum_close(got, expect, addends_abs_sum, dtype):
     err = np.abs(got.astype(np.float64) - expect.astype(np.float64))
     bound = rtol * np.asarray(addends_abs_sum, dtype=np.float64) + 1e-300
     assert np.all(err <= bound), 'max err/bound = %g' % float(np.max(err / bound))
+    if data is not None:
+        ratio = check_sum_forward(got, data, axis, dtype)
+        assert ratio <= 1.0, 'forward bound: max err/bound = %g' % ratio
+        return ratio
+    return None
 
 
 def shaped_random(shape, dtype, seed=0, scale=10):

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import cupy_amd as cp
-from helpers import assert_exact, assert_sum_close, assert_ulp
+from helpers import assert_exact, assert_sum_close, assert_ulp, check_sum_forward
 from oracle import numpy_oracle as o
 
 pytestmark = pytest.mark.gpu
@@ -58,9 +58,26 @@ def test_c3_sums_full(dtype, n, seed):
     s1 = d.sum(axis=1)
     s0 = d.sum(axis=0)
     sa = d.sum()
-    assert_sum_close(s1.get(), o.sum_fp(a, 1), mag.sum(axis=1, dtype=np.float64), dtype)
-    assert_sum_close(s0.get(), o.sum_fp(a, 0), mag.sum(axis=0, dtype=np.float64), dtype)
-    assert_sum_close(sa.get(), np.asarray(o.sum_fp(a)), mag.sum(dtype=np.float64), dtype)
+    # backward bound (rtol * sum|a|) AND forward bound on the result itself:
+    # |got - float64 sum| <= rtol * max(|float64 sum|, sigma * sqrt(N reduced))
+    r1 = assert_sum_close(s1.get(), o.sum_fp(a, 1), mag.sum(axis=1, dtype=np.float64), dtype,
+                          data=a, axis=1)
+    r0 = assert_sum_close(s0.get(), o.sum_fp(a, 0), mag.sum(axis=0, dtype=np.float64), dtype,
+                          data=a, axis=0)
+    ra = assert_sum_close(sa.get(), np.asarray(o.sum_fp(a)), mag.sum(dtype=np.float64), dtype,
+                          data=a, axis=None)
+    print('forward bound, largest err/bound: axis=1 %.3g, axis=0 %.3g, all %.3g' % (r1, r0, ra))
+    # the gate bites: had the kernel dropped one partial result's worth of input
+    # (131072 consecutive elements = 1/2048 of the f32 matrix), the value it
+    # would have produced -- the sum of everything else -- is rejected
+    chunk = 131072
+    cut = a.reshape(-1)[5 * chunk:6 * chunk]
+    missing = np.asarray(float(sa.get()) - cut.sum(dtype=np.float64)).astype(a.dtype)
+    assert check_sum_forward(missing, a, None, dtype) > 1.0
+    rows = chunk // n
+    short1 = s1.get().copy()
+    short1[:rows] = 0
+    assert check_sum_forward(short1, a, 1, dtype) > 1.0
     # a sum of sums is the same total, whichever axis goes first
     t1 = float(s1.astype(np.float64).sum().get())
     t0 = float(s0.astype(np.float64).sum().get())

@@ -23,7 +23,7 @@ def check_sum(a, axis=None, keepdims=False, dtype=None, view=None):
     expect = a.sum(axis=axis, keepdims=keepdims, dtype=dtype)
     if expect.dtype.kind == 'f':
         mag = np.abs(a.astype(np.float64)).sum(axis=axis, keepdims=keepdims)
-        assert_sum_close(got.get(), np.asarray(expect), mag, expect.dtype)
+        assert_sum_close(got.get(), np.asarray(expect), mag, expect.dtype, data=a, axis=axis)
     else:
         assert_exact(got.get(), np.asarray(expect))
     return got
@@ -76,7 +76,8 @@ def test_sum_small_config(small_configs):
         d = cp.asarray(a)
         for axis, key in ((0, 'ax0'), (1, 'ax1'), (None, 'all')):
             mag = np.abs(a.astype(np.float64)).sum(axis=axis)
-            assert_sum_close(d.sum(axis=axis).get(), c['c3_%s_%s' % (name, key)], mag, a.dtype)
+            assert_sum_close(d.sum(axis=axis).get(), c['c3_%s_%s' % (name, key)], mag, a.dtype,
+                             data=a, axis=axis)
 
 
 TRANSPOSES = [
@@ -103,9 +104,9 @@ def test_sum_strided_and_broadcast_views():
     d = cp.broadcast_to(cp.asarray(b), (64, 16, 32))
     e = np.broadcast_to(b, (64, 16, 32))
     assert_sum_close(d.sum(axis=2).get(), e.sum(axis=2),
-                     np.abs(e.astype(np.float64)).sum(axis=2), np.float32)
+                     np.abs(e.astype(np.float64)).sum(axis=2), np.float32, data=e, axis=2)
     assert_sum_close(d.sum(axis=1).get(), e.sum(axis=1),
-                     np.abs(e.astype(np.float64)).sum(axis=1), np.float32)
+                     np.abs(e.astype(np.float64)).sum(axis=1), np.float32, data=e, axis=1)
 
 
 def test_sum_many_dims_keepdims():
@@ -119,7 +120,8 @@ def test_sum_out_and_dtype_arguments():
     d = cp.asarray(a)
     out = cp.empty((50,), np.float32)
     assert d.sum(axis=0, out=out) is out
-    assert_sum_close(out.get(), a.sum(axis=0), np.abs(a).sum(axis=0, dtype=np.float64), np.float32)
+    assert_sum_close(out.get(), a.sum(axis=0), np.abs(a).sum(axis=0, dtype=np.float64), np.float32,
+                     data=a, axis=0)
     out64 = cp.empty((30,), np.float64)
     d.sum(axis=1, out=out64)
     assert np.allclose(out64.get(), a.sum(axis=1), rtol=1e-5)

@@ -64,7 +64,8 @@ def test_reductions_repeated(dtype):
             got = d.sum(axis=axis).get()
             want = h.sum(axis=axis)
             if np.dtype(dtype).kind == 'f':
-                assert_sum_close(got, want, np.abs(h).sum(axis=axis, dtype=np.float64), dtype)
+                assert_sum_close(got, want, np.abs(h).sum(axis=axis, dtype=np.float64), dtype,
+                                 data=h, axis=axis)
             else:
                 assert_exact(got, want)
         h[rng.integers(0, 700), :] = h.max()          # ties
@@ -84,7 +85,7 @@ def test_large_split_reduction_repeated_uses_fresh_partials():
         d = cp.asarray(h)
         got = d.sum().get()
         assert_sum_close(got, h.sum(dtype=np.float32), np.abs(h).sum(dtype=np.float64),
-                         np.float32)
+                         np.float32, data=h, axis=None)
 
 
 def test_fused_and_reduction_kernel_repeated():
@@ -99,7 +100,8 @@ def test_fused_and_reduction_kernel_repeated():
         got = f(cp.asarray(x), cp.asarray(y), cp.asarray(w)).get()
         want = oracle.fused_sqdiff_wsum(x, y, w)
         bound = np.abs(((x - y) ** 2).astype(np.float32) * w).sum(axis=-1, dtype=np.float64)
-        assert_sum_close(got, want, bound, np.float32)
+        terms = ((x - y) ** 2).astype(np.float32) * w
+        assert_sum_close(got, want, bound, np.float32, data=terms, axis=-1)
         xf, yf = x.astype(np.float32), y.astype(np.float32)
         got = l2(cp.asarray(xf), cp.asarray(yf), axis=1).get()
         want = np.sqrt(((xf - yf) ** 2).sum(axis=1))
