@@ -234,7 +234,7 @@ def build_next_cases(cp):
         res_var[0] = dm.var(axis=0)
     add('var f32 16384x8192 axis=0 (one pass; combine kernel included)', m.nbytes + 8192 * 4,
         gpu_var, lambda: m.var(axis=0),
-        lambda: close(res_var[0], m.var(axis=0, dtype=np.float64), 1e-4), 'cupy_var3_float32')
+        lambda: close(res_var[0], m.var(axis=0, dtype=np.float64), 1e-4), 'cupy_var_float32')
     mn = m.copy()
     mn[::7, ::5] = np.nan
     dmn = cp.asarray(mn)
@@ -412,12 +412,12 @@ CEILING_SOURCE = r'''
 #include <cupy/carray.cuh>
 typedef float T;
 typedef cupy::Vec<T, 4> V4;
-#define KBLOCK 512
-#define KUN 4
-// Plain streaming kernels, written by hand in the shape that measured best on
-// this device: 16 bytes per lane and access, four accesses in flight per lane
-// before the first is used, grid-stride over whole blocks of work, streaming
-// (non-temporal) hints on loads and stores.  n is a multiple of 4*KBLOCK*KUN.
+// Plain streaming kernels written by hand: 16 bytes per lane and access, KUN
+// accesses per operand in flight per lane before the first is used, grid-stride
+// over whole blocks of work, streaming (non-temporal) hints on loads and stores.
+// KBLOCK (workgroup size) and KUN come from the command line: the suite runs a
+// grid of variants and the best one per stream kind is the yardstick.  n is a
+// multiple of 4*KBLOCK*KUN.
 extern "C" __global__ void __launch_bounds__(KBLOCK)
 ceil_read(const T* __restrict__ x, T* __restrict__ sink, long nvec) {
   const long per_iter = (long)KBLOCK * KUN;
@@ -461,17 +461,17 @@ ceil_copy(const T* __restrict__ x, T* __restrict__ z, long nvec) {
 }
 extern "C" __global__ void __launch_bounds__(KBLOCK)
 ceil_saxpy(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ z, long nvec) {
-  const long per_iter = (long)KBLOCK * (KUN / 2);
+  const long per_iter = (long)KBLOCK * KUN;
   for (long base = (long)blockIdx.x * per_iter; base + per_iter <= nvec;
        base += (long)gridDim.x * per_iter) {
-    V4 a[KUN / 2], b[KUN / 2];
+    V4 a[KUN], b[KUN];
 #pragma unroll
-    for (int u = 0; u < KUN / 2; ++u) {
+    for (int u = 0; u < KUN; ++u) {
       a[u] = cupy::load_vec<T, 4, true>(x + (base + u * KBLOCK + threadIdx.x) * 4);
       b[u] = cupy::load_vec<T, 4, true>(y + (base + u * KBLOCK + threadIdx.x) * 4);
     }
 #pragma unroll
-    for (int u = 0; u < KUN / 2; ++u) {
+    for (int u = 0; u < KUN; ++u) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) a[u].v[k] = 2.5f * a[u].v[k] + b[u].v[k];
       cupy::store_vec<T, 4, true>(z + (base + u * KBLOCK + threadIdx.x) * 4, a[u]);
@@ -483,7 +483,8 @@ ceil_saxpy(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ z, 
 
 def build_ceiling_cases(cp):
     """The streaming ceiling of the device: what plain read-only, write-only,
-    copy and two-in-one-out kernels reach, (a) written by hand (RawKernel), (b)
+    copy and two-in-one-out kernels reach, (a) written by hand (RawKernel) over
+    a grid of workgroup sizes, accesses in flight per lane and grid sizes, (b)
     through ElementwiseKernel / ``sum`` / ``fill`` of this package, (c) as a
     device-to-device ``rt_memcpy_async``.  Arrays of 256 MiB and 1 GiB; every
     call works on the next of several buffer sets, so that nothing of a call's
@@ -494,14 +495,16 @@ def build_ceiling_cases(cp):
         cases.append(dict(name=name, config='ceiling', bytes=int(nbytes), gpu=gpu,
                           cpu=lambda: None, check=lambda: True, kernel=kernel))
 
-    mod = cp.RawModule(code=CEILING_SOURCE)
-    k_read, k_fill = mod.get_function('ceil_read'), mod.get_function('ceil_fill')
-    k_copy, k_saxpy = mod.get_function('ceil_copy'), mod.get_function('ceil_saxpy')
+    mods = {}
+    for block in (256, 512, 1024):
+        for un in (1, 2, 4):
+            mods[block, un] = cp.RawModule(
+                code=CEILING_SOURCE, options=('-DKBLOCK=%d' % block, '-DKUN=%d' % un))
     e_copy = cp.ElementwiseKernel('T x', 'T y', 'y = x', 'ew_copy')
     e_saxpy = cp.ElementwiseKernel('float32 x, float32 y, float32 a', 'float32 z',
                                    'z = a * x + y', 'ew_saxpy')
     sink = cp.zeros((4,), np.float32)
-    block = 512
+    cus = 256
     for mib in (256, 1024):
         n = mib * (1 << 20) // 4
         nvec = n // 4
@@ -517,28 +520,36 @@ def build_ceiling_cases(cp):
                 turn[0] = (turn[0] + 1) % sets
                 fn(turn[0])
             return call
-        grid = (256 * 8,)
         tag = '%d MiB' % mib
-        add('read   hand-written %s' % tag, 4 * n,
-            rot(lambda i, xs=xs, nvec=nvec: k_read(grid, (block,), (xs[i], sink, nvec))), 'ceil_read')
+        for (block, un), mod in mods.items():
+            k_read, k_fill = mod.get_function('ceil_read'), mod.get_function('ceil_fill')
+            k_copy, k_saxpy = mod.get_function('ceil_copy'), mod.get_function('ceil_saxpy')
+            full = nvec // (block * un)
+            for per_cu in (1, 4, 0):         # resident workgroups' worth of grid; 0 = no loop
+                grid = (full if per_cu == 0 else min(full, cus * (2048 // block) * per_cu),)
+                var = ' [block %d, %d in flight, grid %d]' % (block, un, grid[0])
+                add('read   hand-written %s%s' % (tag, var), 4 * n,
+                    rot(lambda i, k=k_read, g=grid, b=block, xs=xs, nvec=nvec:
+                        k(g, (b,), (xs[i], sink, nvec))), 'ceil_read')
+                add('fill   hand-written %s%s' % (tag, var), 4 * n,
+                    rot(lambda i, k=k_fill, g=grid, b=block, zs=zs, nvec=nvec:
+                        k(g, (b,), (zs[i], nvec))), 'ceil_fill')
+                add('copy   hand-written %s%s' % (tag, var), 8 * n,
+                    rot(lambda i, k=k_copy, g=grid, b=block, xs=xs, zs=zs, nvec=nvec:
+                        k(g, (b,), (xs[i], zs[i], nvec))), 'ceil_copy')
+                add('saxpy  hand-written %s%s' % (tag, var), 12 * n,
+                    rot(lambda i, k=k_saxpy, g=grid, b=block, xs=xs, ys=ys, zs=zs, nvec=nvec:
+                        k(g, (b,), (xs[i], ys[i], zs[i], nvec))), 'ceil_saxpy')
         add('read   sum() of this package %s' % tag, 4 * n,
             rot(lambda i, xs=xs, souts=souts: xs[i].sum(out=souts[i])), 'cupy_sum')
-        add('fill   hand-written %s' % tag, 4 * n,
-            rot(lambda i, zs=zs, nvec=nvec: k_fill(grid, (block,), (zs[i], nvec))), 'ceil_fill')
-        add('fill   ndarray.fill %s' % tag, 4 * n,
+        add('fill   ndarray.fill of this package %s' % tag, 4 * n,
             rot(lambda i, zs=zs: zs[i].fill(1.0)), 'cupy_fill')
-        add('copy   hand-written %s' % tag, 8 * n,
-            rot(lambda i, xs=xs, zs=zs, nvec=nvec: k_copy(grid, (block,), (xs[i], zs[i], nvec))),
-            'ceil_copy')
-        add('copy   ElementwiseKernel %s' % tag, 8 * n,
+        add('copy   ElementwiseKernel of this package %s' % tag, 8 * n,
             rot(lambda i, xs=xs, zs=zs: e_copy(xs[i], zs[i])), 'ew_copy')
-        add('copy   rt_memcpy_async D2D %s' % tag, 8 * n,
+        add('copy   rt_memcpy_async device to device %s' % tag, 8 * n,
             rot(lambda i, xs=xs, zs=zs, n=n: zs[i].data.copy_from_device_async(xs[i].data, 4 * n)),
             'hipMemcpyAsync')
-        add('saxpy  hand-written %s' % tag, 12 * n,
-            rot(lambda i, xs=xs, ys=ys, zs=zs, nvec=nvec:
-                k_saxpy(grid, (block,), (xs[i], ys[i], zs[i], nvec))), 'ceil_saxpy')
-        add('saxpy  ElementwiseKernel %s' % tag, 12 * n,
+        add('saxpy  ElementwiseKernel of this package %s' % tag, 12 * n,
             rot(lambda i, xs=xs, ys=ys, zs=zs: e_saxpy(xs[i], ys[i], 2.5, zs[i])), 'ew_saxpy')
     return cases
 
@@ -716,7 +727,8 @@ def main():
     roof = None
     if not args.no_detail:
         for c in cases:
-            med, mn = time_case_events(cp, c['gpu'], repeats=15, inner=10)
+            med, mn = time_case_events(cp, c['gpu'], repeats=7 if args.suite == 'ceiling' else 15,
+                                       inner=10)
             gbps = c['bytes'] / med / 1e9
             per_config.append({
                 'name': c['name'], 'config': c['config'], 'kernel': c['kernel'],

@@ -201,24 +201,34 @@ def cmd_occupancy(a):
     vals = {}
     for c in ('SQ_WAVES', 'SQ_WAVE_CYCLES', 'SQ_BUSY_CYCLES', 'GRBM_GUI_ACTIVE'):
         vals[c], per = _counter_by_position(path, c, positions, a.skip)
+    derived = {}
+    if a.derived_dir:
+        dpath = _one(os.path.join(a.derived_dir, '**', '*counter_collection.csv'))
+        for c in ('OccupancyPercent', 'MeanOccupancyPerCU'):
+            derived[c], _ = _counter_by_position(dpath, c, positions, a.skip)
     out = _header(a.title, a.command, a.note)
-    out += ['Waves = wavefronts launched (SQ_WAVES).  Occupancy = wave slots held, averaged over the '
-            'kernel\'s run and over all %d CUs: 4 x SQ_WAVE_CYCLES / GRBM_GUI_ACTIVE / CUs, as waves '
-            'per CU and as a share of the %d slots a CU has (the expression of rocprofv3\'s '
-            '`OccupancyPercent`).  LDS and VGPR columns are what bound the slots a kernel can hold.'
-            % (a.cus, MAX_WAVES_PER_CU), '',
+    out += ['Waves = wavefronts launched (SQ_WAVES).  "Waves per CU" = wave slots held, averaged over '
+            'the kernel\'s run and over all %d CUs: 4 x SQ_WAVE_CYCLES / (GRBM_GUI_ACTIVE / %d) / CUs '
+            '(the CSV holds GRBM_GUI_ACTIVE summed over the %d XCDs); "occupancy" is that as a share '
+            'of the %d slots of a CU.  The last two columns are rocprofv3\'s own derived metrics '
+            '`MeanOccupancyPerCU` and `OccupancyPercent` from a second run.  Workgroup size, VGPRs '
+            'and LDS are what bound the slots a kernel can hold.'
+            % (a.cus, a.xcds, a.xcds, MAX_WAVES_PER_CU), '',
             '| # | Operation | Kernel | Workgroup | VGPRs | LDS B | Waves | GPU cycles | '
-            'Waves per CU (mean) | Occupancy |', '|---|---|---|---|---|---|---|---|---|---|']
+            'Waves per CU | Occupancy | MeanOccupancyPerCU | OccupancyPercent |',
+            '|---|---|---|---|---|---|---|---|---|---|---|---|']
     for k, (op, kern, first) in enumerate(positions):
         r = per[k][0]
         waves = statistics.median(vals['SQ_WAVES'][k])
         wc = statistics.median(vals['SQ_WAVE_CYCLES'][k])
-        ga = statistics.median(vals['GRBM_GUI_ACTIVE'][k])
+        ga = statistics.median(vals['GRBM_GUI_ACTIVE'][k]) / a.xcds
         mean = 4.0 * wc / ga / a.cus if ga else 0.0
-        out.append('| %d | %s | %s | %s | %s | %s | %d | %d | %.1f | %.0f %% |' % (
-            k, op if first else '  (continued)', kern, r.get('Workgroup_Size', r.get('Workgroup_Size_X', '')),
-            r.get('VGPR_Count', r.get('Arch_VGPR_Count', '')), r.get('LDS_Block_Size', ''),
-            waves, ga, mean, 100.0 * mean / MAX_WAVES_PER_CU))
+        d1 = '%.1f' % statistics.median(derived['MeanOccupancyPerCU'][k]) if derived else ''
+        d2 = '%.0f %%' % statistics.median(derived['OccupancyPercent'][k]) if derived else ''
+        out.append('| %d | %s | %s | %s | %s | %s | %d | %d | %.1f | %.0f %% | %s | %s |' % (
+            k, op if first else '  (continued)', kern, r.get('Workgroup_Size', ''),
+            r.get('VGPR_Count', ''), r.get('LDS_Block_Size', ''),
+            waves, ga, mean, 100.0 * mean / MAX_WAVES_PER_CU, d1, d2))
     _write(a.out, out)
 
 
@@ -235,7 +245,17 @@ def cmd_table(a):
         out += ['`%s`: %s' % (os.path.basename(path), res['config']['workload']), '',
                 '| Operation | Algorithmic bytes | us (median of 15 x 10 calls) | min us | GB/s | of 8 TB/s |',
                 '|---|---|---|---|---|---|']
-        for e in res['per_config']:
+        entries = res['per_config']
+        if a.best_variant:
+            # 'name [variant]' entries: keep the fastest variant of every name
+            best = collections.OrderedDict()
+            for e in entries:
+                base, _, var = e['name'].partition(' [')
+                if base not in best or e['us'] < best[base]['us']:
+                    best[base] = dict(e, name=base + (' -- best of the variants: ' + var.rstrip(']')
+                                                      if var else ''))
+            entries = list(best.values())
+        for e in entries:
             out.append('| %s | %d | %.1f | %.1f | %.0f | %.1f %% |' % (
                 e['name'], e['bytes'], e['us'], e['min_us'], e['gbps'], e['frac'] * 100))
         out.append('')
@@ -273,11 +293,14 @@ def main():
     p.add_argument('--dir', required=True)
     p.add_argument('--plan', required=True)
     p.add_argument('--cus', type=int, default=256)
+    p.add_argument('--xcds', type=int, default=8)
+    p.add_argument('--derived-dir', default='')
     p.set_defaults(fn=cmd_occupancy)
     p = sub.add_parser('table')
     common(p)
     p.add_argument('--json', action='append', required=True)
     p.add_argument('--ceiling', default='')
+    p.add_argument('--best-variant', action='store_true')
     p.set_defaults(fn=cmd_table)
     a = ap.parse_args()
     a.fn(a)

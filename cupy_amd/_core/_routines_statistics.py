@@ -394,36 +394,65 @@ def _var_core(out_type):
 
 
 _var_onepass_preamble = '''
-// Sums of d and d*d for d = x - k, k a pivot near the data (shifted-data
-// algorithm, Chan, Golub, LeVeque 1983): with sum(d*d) - sum(d)^2 / n the
-// variance comes out of ONE pass.  The cancellation in that difference grows
-// with (distance of the pivot from the mean / standard deviation)^2, which the
-// choice of the pivot keeps near one.
+// One-pass variance that no input can make cancel.  State of a set of values:
+// their number n, a pivot k (the first value that joined), and -- of the values
+// counted from the pivot, y = x - k -- the mean m and the sum of squared
+// deviations from that mean, M2.
+//  * A value joins the set by Welford's update, d = y - m, m += d / n,
+//    M2 += d * (y - m): the mean the deviations are taken from follows the data
+//    with every value, so nothing large is ever subtracted from something
+//    large.  Counting from the pivot keeps m small next to the data (data at
+//    3e5 with a spread of 1 has |m| of order 1), so that rounding m costs
+//    nothing; a pivot far from the rest of the set is a member of the set whose
+//    distance is part of the true variance.  1 / n is the hardware's
+//    reciprocal (one more Newton step for double): the update needs a mean
+//    that is close, not one that is correctly rounded, because what m misses
+//    enters the result squared.
+//  * Two sets merge by M2 = M2a + M2b + delta^2 na nb / n (Chan, Golub,
+//    LeVeque 1983) with delta, the difference of the means, formed as
+//    (kb - ka) + (mb - ma).
+// The reference takes two passes instead (mean, then squared deviations:
+// cupy/_core/_routines_statistics.pyx:553-598).
+__device__ __forceinline__ float var_rcp(float n) { return __builtin_amdgcn_rcpf(n); }
+__device__ __forceinline__ double var_rcp(double n) {
+  const double r = __builtin_amdgcn_rcp(n);
+  return r * (2.0 - n * r);
+}
+#ifndef VAR_COUNT_T
+#define VAR_COUNT_T long long
+#endif
 template <typename T>
 struct var_st {
-  T s1, s2;
-  __device__ __forceinline__ var_st() : s1(0), s2(0) {}
-  __device__ __forceinline__ explicit var_st(T d) : s1(d), s2(d * d) {}
+  VAR_COUNT_T n;
+  T k, m, m2;
+  __device__ __forceinline__ var_st() : n(0), k(0), m(0), m2(0) {}
+  __device__ __forceinline__ explicit var_st(T x) : n(1), k(x), m(0), m2(0) {}
 };
 template <typename T>
 __device__ __forceinline__ var_st<T> operator+(const var_st<T>& a, const var_st<T>& b) {
   var_st<T> r;
-  r.s1 = a.s1 + b.s1;
-  r.s2 = a.s2 + b.s2;
+  if (b.n == 1) {                       // a value joins a set (also an empty one)
+    r.n = a.n + 1;
+    r.k = a.n == 0 ? b.k : a.k;
+    const T y = b.k - r.k;
+    const T d = y - a.m;
+    r.m = a.m + d * var_rcp(static_cast<T>(r.n));
+    r.m2 = a.m2 + d * (y - r.m);
+    return r;
+  }
+  if (a.n == 0) return b;
+  if (b.n == 0) return a;
+  const T delta = (b.k - a.k) + (b.m - a.m);
+  r.n = a.n + b.n;
+  const T w = static_cast<T>(b.n) / static_cast<T>(r.n);
+  r.k = a.k;
+  r.m = a.m + delta * w;
+  r.m2 = a.m2 + b.m2 + delta * delta * (static_cast<T>(a.n) * w);
   return r;
 }
-// Median of three probes of the data: the pivot.  A NaN probe may give any
-// value here, the probe itself then makes the sums NaN.
-template <typename S>
-__device__ __forceinline__ S var_med3(S a, S b, S c) {
-  const S lo = a < b ? a : b;
-  const S hi = a < b ? b : a;
-  return c < lo ? lo : (c > hi ? hi : c);
-}
 template <typename T>
-__device__ __forceinline__ T var_finish(const var_st<T>& a, T inv_n, T alpha) {
-  const T m2 = a.s2 - a.s1 * a.s1 * inv_n;
-  return alpha * (m2 < 0 ? T(0) : m2);          // NaN stays NaN
+__device__ __forceinline__ T var_finish(const var_st<T>& a, T alpha) {
+  return alpha * (a.m2 < 0 ? T(0) : a.m2);          // NaN stays NaN
 }
 '''
 
@@ -431,60 +460,30 @@ _var_onepass_cores = {}
 _FLOAT_NAMES = {'e': 'float16', 'f': 'float32', 'd': 'float64'}
 
 
-def _var_onepass(out_name, probes=1):
+def _var_onepass(out_name):
     """ReductionKernel of the one-pass variance, accumulating in double for a
-    float64 result and in float otherwise (as the sums of those types do).
-    The pivot is one probe of the data per output, or the median of three,
-    taken inside the kernel."""
+    float64 result and in float otherwise (as the sums of those types do)."""
     from cupy_amd._core._reduction import ReductionKernel
-    ker = _var_onepass_cores.get((out_name, probes))
+    import os
+    count_t = os.environ.get('CUPY_AMD_VAR_COUNT', 'long long')
+    ker = _var_onepass_cores.get((out_name, count_t))
     if ker is None:
         work, scalar_t = ('double', 'float64') if out_name == 'float64' else ('float', 'float32')
-        if probes == 1:
-            params, pivot = 'S k', 'k'
-        else:
-            params, pivot = 'S k0, S k1, S k2', 'var_med3(k0, k1, k2)'
         ker = ReductionKernel(
-            'S x, %s, %s inv_n, %s alpha' % (params, scalar_t, scalar_t), '%s out' % out_name,
-            'var_st<%s>(static_cast<%s>(x) - static_cast<%s>(%s))' % (work, work, work, pivot),
-            'a + b', 'out = var_finish<%s>(a, inv_n, alpha)' % work, 'var_st<%s>()' % work,
-            'cupy_var%d_%s' % (probes, out_name), reduce_type='var_st<%s>' % work,
-            preamble=_var_onepass_preamble)
-        _var_onepass_cores[(out_name, probes)] = ker
+            'S x, %s alpha' % scalar_t, '%s out' % out_name,
+            'var_st<%s>(static_cast<%s>(x))' % (work, work),
+            'a + b', 'out = var_finish<%s>(a, alpha)' % work, 'var_st<%s>()' % work,
+            'cupy_var_%s' % out_name, reduce_type='var_st<%s>' % work,
+            preamble='#define VAR_COUNT_T %s\n' % count_t + _var_onepass_preamble)
+        _var_onepass_cores[(out_name, count_t)] = ker
     return ker
 
 
-def _var_pivot(a, axis):
-    """Per output, the probes of the data that give the pivot, as views (shape
-    of ``a`` with the reduced axes of length one): the first, middle and last
-    element along the reduced axes, whose median is near the data unless two
-    of the three are outliers."""
-    # the three views share shape and strides: one is built, the others are
-    # copies of it that start elsewhere (slicing three times costs more host
-    # time than the kernel runs for mid-sized arrays)
-    shape = tuple(1 if ax in axis else n for ax, n in enumerate(a.shape))
-    first = a._view(shape, a.strides)
-    probes = [first]
-    for pick in (lambda n: n // 2, lambda n: n - 1):
-        offset = sum(pick(a.shape[ax]) * a.strides[ax] for ax in axis)
-        v = object.__new__(type(first))
-        v.__dict__.update(first.__dict__)
-        if offset:
-            v.data = first.data + offset
-        probes.append(v)
-    if internal.prod([a.shape[ax] for ax in axis]) <= 64:
-        # few elements per output: any of them is close enough (the error grows
-        # with the number of elements times the squared distance of the pivot
-        # from the mean, and the pivot is one of the elements)
-        return probes[:1]
-    return probes
-
-
 def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
-    """Variance.  Real inputs take one pass over the data around a pivot read
-    from the data itself (the reference reads them twice: the mean first, then
-    the squared deviations, cupy/_core/_routines_statistics.pyx:553-598);
-    complex inputs keep that two-pass form."""
+    """Variance.  Real inputs take one pass over the data (``var_st`` above;
+    the reference reads them twice: the mean first, then the squared
+    deviations, cupy/_core/_routines_statistics.pyx:553-598); complex inputs
+    keep that two-pass form."""
     import numpy
     if axis is None:
         axis = tuple(range(a.ndim))
@@ -509,11 +508,10 @@ def _ndarray_var(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False):
     if (a.dtype.kind in 'biuf' and dtype_out.kind == 'f' and dtype_out.itemsize <= 8
             and items > 0 and (out is None or out.dtype == dtype_out)):
         axis = tuple(internal._normalize_axis_index(ax, a.ndim) for ax in axis)
-        probes = _var_pivot(a, axis)
-        args = (a, *probes, 1. / items, alpha) + (() if out is None else (out,))
+        args = (a, alpha) + (() if out is None else (out,))
         # (numpy's dtype.name is computed on every access)
         out_name = _FLOAT_NAMES[dtype_out.char]
-        return _var_onepass(out_name, len(probes))(*args, axis=axis, keepdims=keepdims)
+        return _var_onepass(out_name)(*args, axis=axis, keepdims=keepdims)
     arrmean = a.mean(axis=axis, dtype=dtype_mean, out=None, keepdims=True)
     if out is None:
         name = dtype_out.name if dtype_out.name in ('float16', 'float32') else 'float64'

@@ -204,9 +204,9 @@ def test_nan_reductions(dtype):
 @pytest.mark.parametrize('dtype', ['float32', 'float64'])
 def test_one_pass_variance_is_stable_and_matches_numpy(dtype):
     """The variance is computed in one pass over the data, as sums of (x - k)
-    and (x - k)**2 around a pivot k taken from the data.  Data with a mean far
-    above its spread is where a plain sum-of-squares formula cancels
-    catastrophically; with the pivot it must not."""
+    and (x - k)**2 around pivots k that follow the data (see ``var_st``).  Data
+    with a mean far above its spread is where a plain sum-of-squares formula
+    cancels catastrophically; here it must not."""
     rng = np.random.default_rng(91)
     rtol = 2e-5 if dtype == 'float32' else 1e-11
     for offset in (0.0, 1.0e3, 1.0e4, -3.0e5):
@@ -218,8 +218,7 @@ def test_one_pass_variance_is_stable_and_matches_numpy(dtype):
                 got = d.var(axis=axis, ddof=ddof)
                 assert got.dtype == np.dtype(dtype)
                 np.testing.assert_allclose(got.get(), want, rtol=rtol)
-    # an outlier where a probe of the pivot looks: the median of three probes
-    # ignores it
+    # outliers at the first and the last position of every row and column
     h = rng.standard_normal((513, 1031)).astype(dtype)
     h[0, :] = 1.0e6
     h[:, 1030] = -1.0e6
@@ -306,3 +305,48 @@ def test_scans_along_an_axis_with_a_narrow_tail(shape, axis, dtype):
     tol = {'float16': 2e-2, 'float32': 1e-5, 'float64': 1e-12, 'int32': 0}[dtype]
     scale = np.cumsum(np.abs(h.astype(np.float64)), axis=axis)
     assert (np.abs(got - want) <= tol * scale + tol).all()
+
+
+@pytest.mark.parametrize('dtype', ['float32', 'float64'])
+def test_variance_with_unrepresentative_edges_and_sentinels(dtype):
+    """Tightly clustered data far from zero, with padding / sentinel values at
+    the places a sampled pivot would look (first, middle, last element) and
+    elsewhere: a one-pass formula around such a pivot is off by tens of
+    percent; the result must stay within the tolerance of a two-pass one."""
+    rng = np.random.default_rng(92)
+    rtol = 2e-5 if dtype == 'float32' else 1e-11
+    n = 1 << 22
+    x = (rng.standard_normal(n) * 0.1 + 100).astype(dtype)
+    for bad in ([0, n - 1], [0, n // 2, n - 1], [0, 1, 2, 3, n // 2, n - 2, n - 1],
+                list(range(0, n, 65537))):
+        h = x.copy()
+        h[bad] = 0
+        want = h.astype(np.float64).var()
+        np.testing.assert_allclose(cp.asarray(h).var().get(), want, rtol=rtol)
+        np.testing.assert_allclose(cp.asarray(h).std(ddof=1).get(),
+                                   h.astype(np.float64).std(ddof=1), rtol=rtol)
+    # the same along rows and columns of a matrix, whole leading rows / columns padded
+    m = (rng.standard_normal((2048, 1500)) * 0.01 + 100).astype(dtype)
+    m[:3, :] = 0
+    m[-2:, :] = 0
+    m[:, :5] = 0
+    m[:, 749:751] = 0
+    m[:, -1] = 0
+    d = cp.asarray(m)
+    for axis in (0, 1, None):
+        np.testing.assert_allclose(d.var(axis=axis).get(), m.astype(np.float64).var(axis=axis),
+                                   rtol=rtol)
+    # short rows and narrow matrices (other kernels), mean far from the spread
+    for shape in ((100000, 7), (30000, 33), (7, 100000), (64, 4096)):
+        h = (rng.standard_normal(shape) * 0.05 - 3000).astype(dtype)
+        h[0] = 0
+        h[:, 0] = 0
+        d = cp.asarray(h)
+        for axis in (0, 1):
+            np.testing.assert_allclose(d.var(axis=axis).get(),
+                                       h.astype(np.float64).var(axis=axis), rtol=rtol)
+    # constant data has variance exactly zero, whatever the constant
+    c = np.full((1000, 300), 123456.7, dtype)
+    assert not cp.asarray(c).var(axis=0).get().any()
+    assert not cp.asarray(c).var(axis=1).get().any()
+    assert float(cp.asarray(c).var().get()) == 0.0
