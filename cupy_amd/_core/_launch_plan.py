@@ -18,6 +18,7 @@ cupy/_core/_reduction.pyx:309-427 for reductions); its kernel memo
 """
 import numpy
 
+from cupy_amd import _rt
 from cupy_amd._core import _tuning
 from cupy_amd._core._scalar import CScalar
 from cupy_amd.cuda import memory as _memory
@@ -37,6 +38,8 @@ _INF = float('inf')
 
 # Recorded calls kept per kernel object.
 _MAX_PLANS = 256
+
+_SLOT_MARK = 0x5ca7c4a5c4a7c4a5       # stands in for a pointer while its byte offset is looked up
 
 
 def scalar_value(v, descr):
@@ -166,6 +169,8 @@ class FastCall:
             a, b = args[i], args[o]
             if a is not b and ranges_overlap(a, b):
                 return NotImplemented
+        if _memory.static_scratch_active():
+            return self._run_static(args, stream_ptr)
         refs = list(args)
         for shape, dtype in self.out_specs:
             refs.append(ndarray._new_contiguous(shape, dtype))
@@ -190,6 +195,57 @@ class FastCall:
         if type(ret) is tuple:
             return tuple(refs[r] for r in ret)
         return refs[ret]
+
+
+def _run_static(self, args, stream_ptr):
+    """``FastCall.run`` without any allocation (``cuda.memory.static_scratch``):
+    the one temporary the call may use is the runtime library's static device
+    array, handed to the kernels by ``rt_launch_packed_scratch``."""
+    refuse_allocation = _memory.refuse_allocation
+    if self.out_specs:
+        refuse_allocation('an output array')
+    if len(self.temps) > 1:
+        refuse_allocation('a second temporary')
+    if self.temps and self.temps[0] > _rt.RT_SCRATCH_MAX_BYTES:
+        raise RuntimeError(
+            'static_scratch: the call needs %d bytes of scratch memory, the runtime '
+            'library holds %d' % (self.temps[0], _rt.RT_SCRATCH_MAX_BYTES))
+    refs = args
+    n_arr = len(refs)
+    if stream_ptr is None:
+        stream_ptr = _stream.get_current_stream_ptr()
+    for fn, grid, block, packer, template, ptrs, scalars, shmem in self.launches:
+        vals = template[:]
+        scratch_slot = None
+        for slot, ref in ptrs:
+            if ref < n_arr:
+                vals[slot] = refs[ref].data.ptr
+            else:
+                if scratch_slot is not None:
+                    refuse_allocation('a kernel with two scratch pointers')
+                scratch_slot = slot
+                vals[slot] = _SLOT_MARK
+        for slot, ref, descr in scalars:
+            vals[slot] = scalar_value(refs[ref], descr)
+        block_bytes = packer.pack(*vals)
+        if scratch_slot is None:
+            fn.launch_packed(grid, block, block_bytes, shmem, stream_ptr)
+            continue
+        mark = _SLOT_MARK.to_bytes(8, 'little')
+        offset = block_bytes.find(mark)
+        if offset < 0 or offset % 8 or block_bytes.find(mark, offset + 1) >= 0:
+            raise RuntimeError('static_scratch: cannot locate the scratch pointer of %s' % fn.name)
+        fn.launch_packed_scratch(grid, block, block_bytes, offset, self.temps[0],
+                                 shmem, stream_ptr)
+    ret = self.ret
+    if ret is None:
+        return None
+    if type(ret) is tuple:
+        return tuple(refs[r] for r in ret)
+    return refs[ret]
+
+
+FastCall._run_static = _run_static
 
 
 def remember(table, key, fast):

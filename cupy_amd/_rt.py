@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, '_lib', 'libmi355rt.so')
 RT_ERR_RTC_BASE = 10000
 RT_ERR_POOL_OOM = 20001
 RT_ERR_INVALID = 20002
+RT_SCRATCH_MAX_BYTES = 8 << 20      # size of the library's static scratch array per GPU
 
 MEMCPY_H2H, MEMCPY_H2D, MEMCPY_D2H, MEMCPY_D2D, MEMCPY_DEFAULT = range(5)
 
@@ -119,6 +120,8 @@ _PROTOTYPES = {
         _vp, _c.c_int, _c.c_size_t, _c.POINTER(_c.c_int)]),
     'rt_launch': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [_vp, _c.POINTER(_vp)]),
     'rt_launch_packed': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [_vp, _vp, _c.c_size_t]),
+    'rt_launch_packed_scratch': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [
+        _vp, _vp, _c.c_size_t, _c.c_size_t, _c.c_size_t]),
     'rt_malloc': (_c.c_int, [_c.POINTER(_vp), _c.c_size_t]),
     'rt_free': (_c.c_int, [_vp]),
     'rt_host_alloc': (_c.c_int, [_c.POINTER(_vp), _c.c_size_t]),

@@ -10,7 +10,17 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
+
+// Device memory owned by the library itself, for rt_launch_packed_scratch: the
+// place where a kernel keeps data beyond its inputs and outputs (the partial
+// results of a reduction split over workgroups) when the caller may not
+// allocate.  Every GPU the library runs on holds its own copy until the
+// process ends.  In host code this name is a stand-in, not an address: the
+// address on a device comes from hipGetSymbolAddress (scratch_address below)
+// and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[RT_SCRATCH_MAX_BYTES];
 
 namespace {
 
@@ -39,6 +49,26 @@ int fail_invalid(const char* what) {
     hipError_t e_ = (call);                        \
     if (e_ != hipSuccess) return fail_hip(e_, #call); \
   } while (0)
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Address of `scratch` on the CURRENT device, looked up once per device.
+int scratch_address(void** out) {
+  int dev = 0;
+  RT_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail_invalid("scratch: device number out of range");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    RT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail_invalid("scratch: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
 
 char* dup_string(const std::string& s) {
   char* p = static_cast<char*>(std::malloc(s.size() + 1));
@@ -76,7 +106,10 @@ const char* rt_last_error_string(void) { return g_last_error.c_str(); }
 
 int rt_init(void) {
   RT_HIP(hipInit(0));
-  return 0;
+  // the library's scratch array on the device that is current now; other
+  // devices are looked up by the first rt_launch_packed_scratch on them
+  void* p = nullptr;
+  return scratch_address(&p);
 }
 
 int rt_device_count(int* count) {
@@ -314,6 +347,41 @@ int rt_launch_packed(void* function, unsigned gx, unsigned gy, unsigned gz, unsi
   size_t size = arg_block_size;
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(arg_block),
                    HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  RT_HIP(hipModuleLaunchKernel(static_cast<hipFunction_t>(function), gx, gy, gz, bx, by, bz,
+                               shared_mem, static_cast<hipStream_t>(stream), nullptr, extra));
+  return 0;
+}
+
+int rt_launch_packed_scratch(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                             unsigned by, unsigned bz, unsigned shared_mem, void* stream,
+                             const void* arg_block, size_t arg_block_size,
+                             size_t scratch_arg_offset, size_t scratch_bytes) {
+  if (!function) return fail_invalid("rt_launch_packed_scratch: null function");
+  if (gx == 0 || gy == 0 || gz == 0 || bx == 0 || by == 0 || bz == 0)
+    return fail_invalid("rt_launch_packed_scratch: zero-sized grid or block");
+  if (scratch_bytes > RT_SCRATCH_MAX_BYTES) {
+    char msg[160];
+    std::snprintf(msg, sizeof(msg),
+                  "rt_launch_packed_scratch: %zu bytes of scratch requested, the library holds %zu",
+                  scratch_bytes, static_cast<size_t>(RT_SCRATCH_MAX_BYTES));
+    return fail_invalid(msg);
+  }
+  unsigned char block[RT_SCRATCH_MAX_ARG_BLOCK];
+  if (!arg_block || arg_block_size > sizeof(block))
+    return fail_invalid("rt_launch_packed_scratch: argument block missing or larger than "
+                        "RT_SCRATCH_MAX_ARG_BLOCK bytes");
+  if (scratch_arg_offset % sizeof(void*) != 0 ||
+      scratch_arg_offset + sizeof(void*) > arg_block_size)
+    return fail_invalid("rt_launch_packed_scratch: the pointer slot lies outside the argument "
+                        "block or is not 8-byte aligned");
+  void* ptr = nullptr;
+  int status = scratch_address(&ptr);
+  if (status != 0) return status;
+  std::memcpy(block, arg_block, arg_block_size);
+  std::memcpy(block + scratch_arg_offset, &ptr, sizeof(ptr));
+  size_t size = arg_block_size;
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, block, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                   HIP_LAUNCH_PARAM_END};
   RT_HIP(hipModuleLaunchKernel(static_cast<hipFunction_t>(function), gx, gy, gz, bx, by, bz,
                                shared_mem, static_cast<hipStream_t>(stream), nullptr, extra));
   return 0;

@@ -183,6 +183,37 @@ class Function:
         if status != 0:
             _rt.check(status)
 
+    def launch_packed_scratch(self, grid, block, arg_block, scratch_arg_offset,
+                              scratch_bytes, shared_mem=0, stream_ptr=None):
+        """``launch_packed`` for a kernel whose scratch buffer is the runtime
+        library's own static device array instead of an allocation: the
+        pointer parameter at byte ``scratch_arg_offset`` of the argument block
+        receives the array's address (``rt_launch_packed_scratch``).  Nothing
+        is allocated on the way."""
+        if stream_ptr is None:
+            stream_ptr = _stream.get_current_stream_ptr()
+        gx, gy, gz = grid
+        bx, by, bz = block
+        if gx * bx > 0xffffffff or gy * by > 0xffffffff or gz * bz > 0xffffffff:
+            raise ValueError(
+                'kernel %s: grid %r x block %r exceeds 2**32 - 1 work-items in one dimension'
+                % (self.name, grid, block))
+        n = len(arg_block)
+        if n > self._arg_size or n < self._arg_min:
+            raise ValueError(
+                'kernel %s expects an argument block of %d bytes, got %d'
+                % (self.name, self._arg_size, n))
+        if n < self._arg_size:
+            arg_block = bytes(arg_block) + b'\0' * (self._arg_size - n)
+        if _dryrun.enabled():
+            _dryrun.record_launch(self.name, grid, block, shared_mem, bytes(arg_block))
+            return
+        status = _rt.lib.rt_launch_packed_scratch(
+            self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr,
+            arg_block, len(arg_block), scratch_arg_offset, scratch_bytes)
+        if status != 0:
+            _rt.check(status)
+
     def __call__(self, grid, block, args, shared_mem=0, stream=None):
         """Launch with one Python object per kernel parameter.  Each object's
         bytes are placed at the parameter's offset in the argument block, cut

@@ -494,7 +494,42 @@ _thread_local = threading.local()
 
 def alloc(size):
     """Allocates through the current allocator (thread-local override first)."""
+    if getattr(_thread_local, 'static_scratch', False):
+        refuse_allocation('a request for %d bytes' % size)
     return get_allocator()(size)
+
+
+class static_scratch:
+    """Context manager: calls made inside allocate NO device memory.
+
+    For callers that cannot allocate: code under HIP graph capture, tight
+    serving loops.  Outputs must be passed in (``out=``), and the one temporary
+    a call may use -- the partial results of a reduction split over workgroups
+    -- lives in the runtime library's static device array
+    (``rt_launch_packed_scratch``, ``RT_SCRATCH_MAX_BYTES``) instead of coming
+    from the pool.  The call must have run once before with arguments of the
+    same signature (outside the context), so that its kernels are compiled and
+    its launches recorded; whatever would allocate raises ``RuntimeError``
+    instead.  All calls on one GPU share the one array: calls that overlap in
+    time on one GPU (other streams, other threads) race on it."""
+
+    def __enter__(self):
+        self._prev = getattr(_thread_local, 'static_scratch', False)
+        _thread_local.static_scratch = True
+        return self
+
+    def __exit__(self, *exc):
+        _thread_local.static_scratch = self._prev
+
+
+def static_scratch_active():
+    return getattr(_thread_local, 'static_scratch', False)
+
+
+def refuse_allocation(what):
+    raise RuntimeError(
+        'static_scratch: %s would allocate device memory; run the call once outside the '
+        'context and pass every output with out=' % what)
 
 
 def set_allocator(allocator=None):

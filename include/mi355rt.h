@@ -136,6 +136,32 @@ int rt_launch_packed(void* function,
                      unsigned shared_mem, void* stream,
                      const void* arg_block, size_t arg_block_size);
 
+/*
+ * No counterpart in the reference.  For callers that cannot allocate device
+ * memory -- code under HIP graph capture, serving loops, harnesses that forbid
+ * hipMalloc: rt_launch_packed for a kernel that needs a scratch buffer (the
+ * partial results of a reduction split over workgroups, which the Python layer
+ * otherwise takes from the memory pool), with that buffer inside the library:
+ * a static device array of RT_SCRATCH_MAX_BYTES per GPU.  The 8 bytes at
+ * `scratch_arg_offset` of the argument block (the kernel's pointer parameter
+ * for the buffer) are replaced by the array's address on the current device;
+ * `scratch_bytes` is what the kernel will use of it and is refused with
+ * RT_ERR_INVALID beyond RT_SCRATCH_MAX_BYTES, as is an argument block of more
+ * than RT_SCRATCH_MAX_ARG_BLOCK bytes.  Allocates nothing, on the host or the
+ * device.  All calls on one GPU share the one array: it keeps what the last
+ * call left (the reduction kernels write every partial before they read it, so
+ * nothing needs clearing), and two calls that overlap in time on one GPU --
+ * different streams or threads -- race on it.
+ */
+#define RT_SCRATCH_MAX_BYTES (8u << 20)
+#define RT_SCRATCH_MAX_ARG_BLOCK 4096
+int rt_launch_packed_scratch(void* function,
+                             unsigned gx, unsigned gy, unsigned gz,
+                             unsigned bx, unsigned by, unsigned bz,
+                             unsigned shared_mem, void* stream,
+                             const void* arg_block, size_t arg_block_size,
+                             size_t scratch_arg_offset, size_t scratch_bytes);
+
 /* ---- raw device / pinned host memory --------------------------------------- */
 
 /* runtime.pyx:515 malloc, :588 free */
