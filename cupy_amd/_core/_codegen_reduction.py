@@ -366,7 +366,7 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
         src.append('          _acc = REDUCE(_acc, _a);')
     else:
         src.append('          const _type_reduce _n = REDUCE(_acc, _a);')
-        src.append('          _acc = _JOK(_t) ? _n : _acc;')
+        src.append('          _acc = cupy::select_value(_JOK(_t), _n, _acc);')
     src.append('        }')
     src.append('      }')
     if not exact:

@@ -12,19 +12,20 @@ once.  The reference has no counterpart on this platform: its general tracer
 needs a grid-wide barrier (cupy/_core/_fusion_kernel.pyx:99-115).
 
 The pieces of the function (one map-reduce function per reduction, one
-elementwise function per result) are traced by the single-kernel tracer of
-``fusion.py`` in "describe" mode; this module only composes the device
-functions it produced.
+elementwise function per result) come from ``_fusion_emit`` as bare device
+functions; this module composes them.
 """
 import numpy
 
 from cupy_amd._core import _codegen_reduction as _cg
+from cupy_amd._core import _fusion_emit
 from cupy_amd._core import _launch_plan
 from cupy_amd._core import _tuning
 from cupy_amd._core import internal
 from cupy_amd._core._kernel import _make_packer, _scalar_struct_code, _aligned
 from cupy_amd._core._scalar import CScalar, get_typename
 from cupy_amd._core.core import ndarray
+from cupy_amd._core.fusion import _collect, _leaf_reader
 from cupy_amd.cuda import compiler
 from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import stream as _stream
@@ -60,17 +61,19 @@ def _classify(nodes, full):
     kinds = {}
     last = len(full) - 1
     for n in nodes:
-        if n.kind == 'leaf':
+        if n.kind in ('array', 'scalar'):
             k = _kind_of_leaf(n.shape, full)
+        elif n.kind == 'const':
+            k = 'uni'
         elif n.kind == 'reduce':
-            src = n.args[0]
-            if kinds.get(src.order) != 'full' or n.kwargs['axes'] != (last,):
+            src = n.src
+            if kinds.get(src.order) != 'full' or n.axes != (last,):
                 raise _Unsupported('a reduction that is not along the last axis of a row')
             k = 'row'
         elif n.kind == 'keepdims':
             k = 'rowk'
         else:
-            ks = set(kinds[a.order] for a in n.args if hasattr(a, 'order'))
+            ks = set(kinds[a.order] for a in n.inputs)
             ks.discard('uni')
             if not ks:
                 k = 'uni'
@@ -86,7 +89,8 @@ def _classify(nodes, full):
                 k, = ks
         expect = {'full': tuple(full), 'row': tuple(full[:-1]),
                   'rowk': tuple(full[:-1]) + (1,)}.get(k)
-        if n.kind != 'leaf' and expect is not None and n.shape is not None \
+        if n.kind not in ('array', 'scalar', 'const') and expect is not None \
+                and n.shape is not None \
                 and tuple(n.shape) != expect:
             raise _Unsupported('shape %r of a %s value' % (n.shape, k))
         kinds[n.order] = k
@@ -101,19 +105,20 @@ class RowPlan:
         self.packer = packer
         self.grid = grid
         self.n_rows = n_rows
-        # per kernel argument ('arg', position, x) or ('const', array, x); x is the
+        # per kernel argument (reader of the call's arguments, x); x is the
         # alignment in bytes required of an array's data, or the dtype of a scalar
         self.in_slots = tuple(in_slots)
         self.out_specs = tuple(out_specs)    # (shape, dtype) per output pointer
-        self.returns = tuple(returns)        # ('out', k) | ('arg', position) | ('const', value)
+        self.returns = tuple(returns)        # as fusion._collect takes them
+        self.store_positions = ()
         self.single = single
         self.fallback = None
         self.steps = (('kernel', self),)
 
     def run(self, *args):
         vals = []
-        for what, ref, descr in self.in_slots:
-            v = args[ref] if what == 'arg' else ref
+        for read, descr in self.in_slots:
+            v = read(args)
             if type(descr) is int:
                 # an array: contiguous and aligned as the kernel's vector
                 # accesses assume, or the call goes the general way
@@ -128,18 +133,16 @@ class RowPlan:
         vals.append(self.n_rows)
         self.fn.launch_packed(self.grid, (BLOCK, 1, 1), self.packer.pack(*vals), 0,
                               _stream.get_current_stream_ptr())
-        res = []
-        for what, ref in self.returns:
-            res.append(outs[ref] if what == 'out' else args[ref] if what == 'arg' else ref)
-        return res[0] if self.single else tuple(res)
+        return _collect(self.returns, outs, args, self.single)
 
 
 def build(nodes, pieces, returns, single, args, name):
     """RowPlan for the recorded function, or None when it does not have the
     row-wise form (the caller then launches the pieces one by one).
 
-    ``pieces``: the ``_Piece`` objects of ``_fusion_split`` in evaluation order;
-    ``returns``: node order numbers or ('const', value)."""
+    ``nodes``: the values of the recording that the results depend on;
+    ``pieces``: the ``Piece`` objects of ``_fusion_split`` in evaluation order;
+    ``returns``: as ``fusion.Recording`` lists them."""
     if not _tuning.get('fused_rows'):
         return None
     try:
@@ -149,30 +152,28 @@ def build(nodes, pieces, returns, single, args, name):
 
 
 def _build(nodes, pieces, returns, single, args, name):
-    from cupy_amd._core import fusion
     reduces = [n for n in nodes if n.kind == 'reduce']
     if not reduces:
         raise _Unsupported('no reduction')
-    full = tuple(reduces[0].args[0].shape)
+    full = tuple(reduces[0].src.shape)
     if len(full) < 1 or internal.prod(full) == 0:
         raise _Unsupported('empty')
     n_cols = full[-1]
     n_rows = internal.prod(full[:-1])
     kinds = _classify(nodes, full)
-    by_order = {n.order: n for n in nodes}
 
     # ---- the values every piece starts from --------------------------------------------
     leaf_value = {}
-    for n in nodes:
-        if n.kind == 'leaf':
-            leaf_value[n.order] = args[n.fn] if isinstance(n.fn, int) else n.fn
-    for n in nodes:
-        if n.kind == 'leaf' and kinds[n.order] != 'uni':
+    leaf_nodes = [n for n in nodes if n.kind in ('array', 'scalar')]
+    for n in leaf_nodes:
+        leaf_value[n.order] = _leaf_reader(n)(args)
+    for n in leaf_nodes:
+        if kinds[n.order] != 'uni':
             a = leaf_value[n.order]
             if not isinstance(a, ndarray) or not a._c_contiguous:
                 raise _Unsupported('operand that is not C-contiguous')
-    full_leaves = [n for n in nodes if n.kind == 'leaf' and kinds[n.order] == 'full']
-    col_leaves = [n for n in nodes if n.kind == 'leaf' and kinds[n.order] == 'col']
+    full_leaves = [n for n in leaf_nodes if kinds[n.order] == 'full']
+    col_leaves = [n for n in leaf_nodes if kinds[n.order] == 'col']
     if not full_leaves:
         raise _Unsupported('no full-size operand')
 
@@ -204,32 +205,14 @@ def _build(nodes, pieces, returns, single, args, name):
     if words > _ROW_WORDS_PER_LANE or n_cols < 2:
         raise _Unsupported('row of %d elements does not fit the registers of a group' % n_cols)
 
-    # ---- trace every piece into device functions -----------------------------------------
-    dtype_of = {}
-    for n in nodes:
-        if n.kind == 'leaf':
-            v = leaf_value[n.order]
-            dtype_of[n.order] = v.dtype if isinstance(v, (ndarray, numpy.generic)) else None
-
-    def stand_in(n):
-        if n.kind == 'leaf':
-            return leaf_value[n.order]
-        source = n.args[0] if n.kind == 'keepdims' else n
-        return ndarray._new_contiguous((1,) * len(n.shape), dtype_of[source.order])
-
+    # ---- every piece as device functions -------------------------------------------------
+    dtype_of = dict((n.order, n.dtype) for n in nodes)
     described = []
     for p in pieces:
-        desc = fusion.describe(p.func, [stand_in(l) for l in p.leaves], name)
-        if desc['kind'] == 'reduce':
-            (target,) = p.targets
-            dtype_of[target.order] = desc['out_params'][0].dtype
+        if p.reduce is not None:
+            described.append(_fusion_emit.describe_reduction(p.reduce, p.leaves))
         else:
-            for t, v in zip(p.targets, desc['out_params']):
-                dtype_of[t.order] = v.dtype
-        described.append(desc)
-    for n in nodes:
-        if n.kind == 'keepdims':
-            dtype_of[n.order] = dtype_of[n.args[0].order]
+            described.append(_fusion_emit.describe_elementwise(p.leaves, p.targets))
 
     # ---- kernel parameters ---------------------------------------------------------------
     params = []
@@ -237,37 +220,28 @@ def _build(nodes, pieces, returns, single, args, name):
     in_slots = []
     cname = {}
 
-    def slot_of(n):
-        return ('arg', n.fn, ) if isinstance(n.fn, int) else ('const', n.fn)
-
-    for n in nodes:
-        if n.kind != 'leaf':
-            continue
+    for n in leaf_nodes:
         v = leaf_value[n.order]
-        what, ref = slot_of(n)
+        read = _leaf_reader(n)
         if isinstance(v, ndarray):
             t = get_typename(v.dtype)
             params.append('const %s* __restrict__ _p%d' % (t, n.order))
             fmt.append('P')
             vector = kinds[n.order] in ('full', 'col')
-            in_slots.append((what, ref, min(16, vec * v.dtype.itemsize) if vector
+            in_slots.append((read, min(16, vec * v.dtype.itemsize) if vector
                              else v.dtype.itemsize))
         else:
             s = CScalar(v)
             t = get_typename(s.descr)
             params.append('const %s _s%d' % (t, n.order))
             fmt.append(_scalar_struct_code(t))
-            in_slots.append((what, ref, s.descr))
+            in_slots.append((read, s.descr))
             cname[n.order] = '_s%d' % n.order
     out_nodes = []
     out_returns = []
-    for r in returns:
-        if isinstance(r, tuple):
-            out_returns.append(r)
-            continue
-        n = by_order[r]
-        if n.kind == 'leaf':
-            out_returns.append(slot_of(n) if isinstance(n.fn, int) else ('const', n.fn))
+    for kind, n in returns:
+        if kind != 'value':
+            out_returns.append((kind, n))
             continue
         if not any(n is m for m in out_nodes):
             out_nodes.append(n)
@@ -317,17 +291,12 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
 }''')
     for k, (p, d) in enumerate(zip(pieces, described)):
         src.append('namespace piece%d {' % k)
+        src.append(d['functions'])
         if d['kind'] == 'reduce':
-            src.append(d['defs'])
             src.append('typedef %s reduce_t;' % d['reduce_ctype'])
             src.append('struct Op { __device__ __forceinline__ reduce_t operator()('
                        'const reduce_t& a, const reduce_t& b) const { return (%s); } };'
                        % d['reduce_expr'])
-        else:
-            sig = ['%s v%d' % (get_typename(v.dtype), v.index) for v in d['in_params']]
-            sig += ['%s& v%d' % (get_typename(v.dtype), v.index) for v in d['out_params']]
-            src.append('__device__ __forceinline__ void elementwise(%s) {\n%s\n}' % (
-                ', '.join(sig), d['operation']))
         src.append('}  // namespace piece%d' % k)
     params.append('const %s _n_rows' % idx_t)
     fmt.append('q' if idx_t == 'ptrdiff_t' else 'i')
@@ -351,8 +320,8 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
         src.append('    _c%d[_e] = _row_vec<%s, false>(_p%d, _col < NCOLS ? _col : 0);'
                    % (n.order, t, n.order))
         src.append('  }')
-    for n in nodes:
-        if n.kind == 'leaf' and kinds[n.order] == 'uni' and n.order not in cname:
+    for n in leaf_nodes:
+        if kinds[n.order] == 'uni' and n.order not in cname:
             t = get_typename(leaf_value[n.order].dtype)
             src.append('  const %s _u%d = _p%d[0];' % (t, n.order, n.order))
             cname[n.order] = '_u%d' % n.order
@@ -372,8 +341,8 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
         src.append('      _f%d[_e] = _row_vec<%s, %s>(_p%d + (ptrdiff_t)_row * NCOLS, _cc);'
                    % (n.order, t, ntl, n.order))
     src.append('    }')
-    for n in nodes:
-        if n.kind == 'leaf' and kinds[n.order] == 'rowk':
+    for n in leaf_nodes:
+        if kinds[n.order] == 'rowk':
             t = get_typename(leaf_value[n.order].dtype)
             src.append('    const %s _r%d = _p%d[_row];' % (t, n.order, n.order))
             cname[n.order] = '_r%d' % n.order
@@ -385,10 +354,10 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
         if n.order in cname:
             return cname[n.order]
         if n.kind == 'keepdims':
-            return operand(n.args[0])
-        if k == 'full' and n.kind == 'leaf':
+            return operand(n.src)
+        if k == 'full' and n.kind == 'array':
             return '_f%d[_e].v[_k]' % n.order
-        if k == 'col' and n.kind == 'leaf':
+        if k == 'col' and n.kind == 'array':
             return '_c%d[_e].v[_k]' % n.order
         raise _Unsupported('value %d (%s, %s) is not available here' % (n.order, n.kind, k))
 
@@ -403,7 +372,7 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
             src.append('      const int _col = (_e * GROUP + _lane) * VEC;')
             src.append('#pragma unroll')
             src.append('      for (int _k = 0; _k < VEC; ++_k) if (_col + _k < NCOLS) {')
-            src.append('        _a%d = piece%d::Op()(_a%d, piece%d::_pre_map(%s));' % (
+            src.append('        _a%d = piece%d::Op()(_a%d, piece%d::_fz_map(%s));' % (
                 k, k, k, k, ', '.join(call_args)))
             src.append('      }')
             src.append('    }')
@@ -421,8 +390,7 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
                 src.append('    __syncthreads();')
             t = get_typename(dtype_of[target.order])
             src.append('    %s _t%d;' % (t, target.order))
-            src.append('    piece%d::_post_map(piece%d::_postmap_cast(_a%d), _t%d);' % (
-                k, k, k, target.order))
+            src.append('    piece%d::_fz_finish(_a%d, _t%d);' % (k, k, target.order))
             cname[target.order] = '_t%d' % target.order
         else:
             target_kinds = set(kinds[t.order] for t in p.targets)

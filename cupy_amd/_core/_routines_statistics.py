@@ -418,13 +418,13 @@ __device__ __forceinline__ double var_rcp(double n) {
   const double r = __builtin_amdgcn_rcp(n);
   return r * (2.0 - n * r);
 }
-#ifndef VAR_COUNT_T
-#define VAR_COUNT_T long long
-#endif
+// The count is kept in T: exact far beyond what one thread folds (2^24 values
+// in float), and where it saturates the update degrades into a moving average
+// with a very long window instead of overflowing; merged counts only serve as
+// weights.
 template <typename T>
 struct var_st {
-  VAR_COUNT_T n;
-  T k, m, m2;
+  T n, k, m, m2;
   __device__ __forceinline__ var_st() : n(0), k(0), m(0), m2(0) {}
   __device__ __forceinline__ explicit var_st(T x) : n(1), k(x), m(0), m2(0) {}
 };
@@ -436,7 +436,7 @@ __device__ __forceinline__ var_st<T> operator+(const var_st<T>& a, const var_st<
     r.k = a.n == 0 ? b.k : a.k;
     const T y = b.k - r.k;
     const T d = y - a.m;
-    r.m = a.m + d * var_rcp(static_cast<T>(r.n));
+    r.m = a.m + d * var_rcp(r.n);
     r.m2 = a.m2 + d * (y - r.m);
     return r;
   }
@@ -444,10 +444,10 @@ __device__ __forceinline__ var_st<T> operator+(const var_st<T>& a, const var_st<
   if (b.n == 0) return a;
   const T delta = (b.k - a.k) + (b.m - a.m);
   r.n = a.n + b.n;
-  const T w = static_cast<T>(b.n) / static_cast<T>(r.n);
+  const T w = b.n / r.n;
   r.k = a.k;
   r.m = a.m + delta * w;
-  r.m2 = a.m2 + b.m2 + delta * delta * (static_cast<T>(a.n) * w);
+  r.m2 = a.m2 + b.m2 + delta * delta * (a.n * w);
   return r;
 }
 template <typename T>
@@ -464,9 +464,7 @@ def _var_onepass(out_name):
     """ReductionKernel of the one-pass variance, accumulating in double for a
     float64 result and in float otherwise (as the sums of those types do)."""
     from cupy_amd._core._reduction import ReductionKernel
-    import os
-    count_t = os.environ.get('CUPY_AMD_VAR_COUNT', 'long long')
-    ker = _var_onepass_cores.get((out_name, count_t))
+    ker = _var_onepass_cores.get(out_name)
     if ker is None:
         work, scalar_t = ('double', 'float64') if out_name == 'float64' else ('float', 'float32')
         ker = ReductionKernel(
@@ -474,8 +472,8 @@ def _var_onepass(out_name):
             'var_st<%s>(static_cast<%s>(x))' % (work, work),
             'a + b', 'out = var_finish<%s>(a, alpha)' % work, 'var_st<%s>()' % work,
             'cupy_var_%s' % out_name, reduce_type='var_st<%s>' % work,
-            preamble='#define VAR_COUNT_T %s\n' % count_t + _var_onepass_preamble)
-        _var_onepass_cores[(out_name, count_t)] = ker
+            preamble=_var_onepass_preamble)
+        _var_onepass_cores[out_name] = ker
     return ker
 
 

@@ -92,18 +92,51 @@ def get_rtc_version():
 _header_digest = None
 
 
-def _get_header_digest():
-    """Hash of the bundled device headers: part of every cache key."""
-    global _header_digest
-    if _header_digest is None:
+_include_re = re.compile(r'#\s*include\s*[<"](cupy/[^>"]+)[>"]')
+_header_files = {}          # relative name -> (bytes, names it includes)
+_header_digests = {}        # frozenset of names -> digest
+
+
+def _header_file(name):
+    entry = _header_files.get(name)
+    if entry is None:
+        try:
+            with open(os.path.join(_INCLUDE_DIR, name), 'rb') as f:
+                data = f.read()
+        except OSError:
+            data = b''
+        entry = (data, tuple(_include_re.findall(data.decode('utf-8', 'replace'))))
+        _header_files[name] = entry
+    return entry
+
+
+def _get_header_digest(source=None):
+    """Hash of the bundled device headers a source includes, directly or
+    through other bundled headers: part of its cache key (a change to one
+    header leaves the cached kernels that never saw it valid).  Without a
+    source: of all bundled headers."""
+    if source is None:
+        names = set()
+        for root, _, files in os.walk(_INCLUDE_DIR):
+            for name in files:
+                names.add(os.path.relpath(os.path.join(root, name), _INCLUDE_DIR))
+    else:
+        names = set()
+        todo = list(_include_re.findall(source))
+        while todo:
+            name = todo.pop()
+            if name not in names:
+                names.add(name)
+                todo.extend(_header_file(name)[1])
+    key = frozenset(names)
+    digest = _header_digests.get(key)
+    if digest is None:
         h = hashlib.sha1()
-        for root, _, files in sorted(os.walk(_INCLUDE_DIR)):
-            for name in sorted(files):
-                with open(os.path.join(root, name), 'rb') as f:
-                    h.update(name.encode())
-                    h.update(f.read())
-        _header_digest = h.hexdigest()
-    return _header_digest
+        for name in sorted(names):
+            h.update(name.encode())
+            h.update(_header_file(name)[0])
+        digest = _header_digests[key] = h.hexdigest()
+    return digest
 
 
 def get_arch(device_id=None):
@@ -176,7 +209,7 @@ def compile_source(source, options=(), arch='gfx950', name='kernel.hip',
 def _cache_key(source, options, arch):
     h = hashlib.sha1()
     for part in (arch, repr(_BASE_OPTIONS), repr(tuple(options)),
-                 repr(get_rtc_version()), _get_header_digest(), source):
+                 repr(get_rtc_version()), _get_header_digest(source), source):
         h.update(part.encode())
         h.update(b'\0')
     return h.hexdigest() + '.hsaco'

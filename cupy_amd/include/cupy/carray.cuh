@@ -362,6 +362,23 @@ _CUPY_DEV T shfl_idx(const T& v, int src) {
   return r;
 }
 
+// `c ? a : b` for a value of any trivially copyable type, word by word.  The
+// conditional operator on a structure of more than two words is compiled into
+// stores of both operands to scratch memory and a load through a selected
+// address; words selected one by one stay in registers.
+template <typename T>
+_CUPY_DEV T select_value(bool c, const T& a, const T& b) {
+  constexpr int kWords = (sizeof(T) + 3) / 4;
+  unsigned wa[kWords] = {}, wb[kWords] = {};
+  __builtin_memcpy(wa, &a, sizeof(T));
+  __builtin_memcpy(wb, &b, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) wa[k] = c ? wa[k] : wb[k];
+  T r = b;
+  __builtin_memcpy(&r, wa, sizeof(T));
+  return r;
+}
+
 // One value moved between lanes by a data-parallel-primitive modifier
 // (`kCtrl`: quad permutation, row mirror / half mirror, row rotation), word by
 // word.  These run in the vector ALU; a general shuffle goes through the LDS

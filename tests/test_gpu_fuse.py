@@ -391,3 +391,197 @@ def test_row_kernel_follows_scalars_types_and_captured_arrays():
             else:
                 # a comparison may flip where x + shift and the mean agree to rounding
                 assert (g.get() != w).mean() < 0.01
+
+
+# ---- in-place operators, out= and indexing inside fused functions --------------------------
+# Scenarios of the reference's fusion_tests/test_misc.py:32-54,126-141 and
+# test_indexing.py:48-124, evaluated on NumPy and by the fused kernel on the
+# same seeded inputs; integer results bit-exact, float results too (every step is
+# one IEEE operation in the same order).
+
+ALL_DTYPES = ['int8', 'int16', 'int32', 'int64', 'uint8', 'uint16', 'uint32', 'uint64',
+              'float16', 'float32', 'float64']
+
+
+def _inputs(n, dtype, shape=(3, 4)):
+    return [shaped_random(shape, dtype, seed) for seed in range(n)]
+
+
+def _run_both(make, host_args):
+    """Runs ``make(numpy)`` on copies of the host arrays and the fused
+    ``make(cupy)`` on device copies; returns (numpy result, numpy args after,
+    fused result, device args after)."""
+    h = [a.copy() if isinstance(a, np.ndarray) else a for a in host_args]
+    d = [cp.asarray(a) if isinstance(a, np.ndarray) else a for a in host_args]
+    with np.errstate(all='ignore'):
+        want = make(np)(*h)
+    got = cp.fuse(make(cp))(*d)
+    return want, h, got, d
+
+
+def _same(got, want):
+    if want is None:
+        assert got is None
+        return
+    if isinstance(want, tuple):
+        assert isinstance(got, tuple) and len(got) == len(want)
+        for g, w in zip(got, want):
+            _same(g, w)
+        return
+    g = got.get() if isinstance(got, cp.ndarray) else np.asarray(got)
+    assert g.dtype == np.asarray(want).dtype, (g.dtype, np.asarray(want).dtype)
+    assert g.shape == np.asarray(want).shape
+    assert np.array_equal(g, want, equal_nan=True)
+
+
+@pytest.mark.parametrize('dtype', ALL_DTYPES)
+def test_out_arguments_mixed(dtype):
+    def make(xp):
+        def func(x, y, z, u, v):
+            xp.add(x, y, out=z)
+            xp.subtract(z, x, out=u)
+            xp.multiply(z, x, out=v)
+            return u
+        return func
+    want, h, got, d = _run_both(make, _inputs(5, dtype))
+    _same(got, want)
+    for a, b in zip(d, h):
+        _same(a, b)                      # z, u and v were written, x and y were not
+    assert got is d[3]
+
+
+@pytest.mark.parametrize('dtype', ALL_DTYPES)
+def test_in_place_add_several_times(dtype):
+    def thrice(xp):
+        def func(x, y):
+            x += y
+            x += y
+            x += y
+            return x
+        return func
+
+    def once(xp):
+        def func(x):
+            x += 2
+        return func
+
+    def twice(xp):
+        def func(x):
+            x += x
+            x += x
+        return func
+    for make, n in ((thrice, 2), (once, 1), (twice, 1)):
+        want, h, got, d = _run_both(make, _inputs(n, dtype))
+        _same(got, want)
+        for a, b in zip(d, h):
+            _same(a, b)
+
+
+@pytest.mark.parametrize('dtype', ['int32', 'uint8', 'float16', 'float32', 'float64', 'bool'])
+def test_tuples_swaps_and_casts(dtype):
+    def swap(xp):
+        def func(x, y, z):
+            w = x * y + z
+            (x, w) = (w, x)
+            return z * w + y + x
+        return func
+
+    def triple(xp):
+        return lambda x, y, z: (x + y, y + z, z * x)
+
+    def casts(xp):
+        def func(x, y, z):
+            x = x.astype('int32')
+            y = x.astype('float32')
+            return x + y, y + z, z + x
+        return func
+    for make in (swap, triple, casts):
+        want, h, got, d = _run_both(make, _inputs(3, dtype))
+        _same(got, want)
+    x = cp.asarray(_inputs(1, dtype)[0])
+    assert cp.fuse(lambda a: ())(x) == ()
+    (only,) = cp.fuse(lambda a: (a,))(x)
+    assert only is x
+    assert cp.fuse(lambda: None)() is None
+
+
+FUSE_INDICES = [
+    1, -1, (1,), (1, 0), (1, 0, 2), (-1, 0, -2), slice(None), slice(None, None, -1),
+    (slice(None), slice(None, None, -1)), Ellipsis, None, (None, None, None),
+    (slice(None), 0, slice(None, None, -1)), (1, None, slice(None, None, -1), None, 2),
+    (Ellipsis, 2), (1, Ellipsis),
+]
+
+
+@pytest.mark.parametrize('indices', FUSE_INDICES, ids=str)
+def test_getitem_inside_a_fused_function(indices):
+    for dtype in ('int16', 'float32', 'bool'):
+        x = shaped_random((2, 3, 4), dtype, 0)
+        want, _, got, _ = _run_both(lambda xp: lambda a: a[indices], [x])
+        _same(got, want)
+        # and as an operand of arithmetic
+        want, _, got, _ = _run_both(lambda xp: lambda a: a[indices] + a[indices], [x])
+        _same(got, want)
+    x4 = shaped_random((2, 3, 4, 5), 'float32', 1)
+    want, _, got, _ = _run_both(lambda xp: lambda a: a[1, ..., 3] * 2, [x4])
+    _same(got, want)
+
+
+@pytest.mark.parametrize('dtype1', ['int8', 'int32', 'uint16', 'float16', 'float32', 'float64'])
+@pytest.mark.parametrize('dtype2', ['int16', 'uint32', 'float32', 'float64'])
+def test_indexing_combined_with_arithmetic(dtype1, dtype2):
+    x = shaped_random((3, 4), dtype1, 0)
+    y = shaped_random((4,), dtype2, 1)
+    z = shaped_random((1,), dtype1, 2)
+    cases = [
+        lambda xp: lambda x, y, z: x + y[1],
+        lambda xp: lambda x, y, z: x + z[0] + y,
+        lambda xp: lambda x, y, z: x + x[0] + x[1],
+        lambda xp: lambda x, y, z: x + x[0, 1] + x[1] + x + x[2, 1],
+        lambda xp: lambda x, y, z: x[0][1],
+        lambda xp: lambda x, y, z: x[0][1] + x[1][0],
+        lambda xp: lambda x, y, z: x[::-1] - y[::-1],
+    ]
+    for make in cases:
+        want, _, got, _ = _run_both(make, [x, y, z])
+        _same(got, want)
+
+
+def test_in_place_with_reductions_and_overlapping_arguments():
+    rng = np.random.default_rng(50)
+    a = rng.standard_normal((40, 30)).astype(np.float32)
+    b = rng.standard_normal((40, 30)).astype(np.float32)
+
+    def various(xp):
+        def func(x, y):
+            s = x + y
+            t = xp.sum(s, axis=0)
+            x += t
+            c = xp.sum(x, axis=0)
+            y += c
+            return c, t, x, y, s
+        return func
+    want, h, got, d = _run_both(various, [a, b])
+    for g, w in zip(got, want):
+        np.testing.assert_allclose(g.get(), w, rtol=1e-5, atol=1e-4)
+    assert got[2] is d[0] and got[3] is d[1]
+    np.testing.assert_allclose(d[0].get(), h[0], rtol=1e-5, atol=1e-4)
+    np.testing.assert_allclose(d[1].get(), h[1], rtol=1e-5, atol=1e-4)
+
+    # the written array overlaps another argument: what NumPy does, step by step
+    @cp.fuse()
+    def shift(x, y):
+        x += y
+        x += y
+        return x
+    base = cp.asarray(np.arange(20, dtype=np.float32))
+    hbase = np.arange(20, dtype=np.float32)
+    shift(base[1:], base[:-1])
+    hx, hy = hbase[1:], hbase[:-1]
+    hx += hy
+    hx += hy
+    _same(base, hbase)
+    # the same array twice
+    c = cp.asarray(a)
+    shift(c, c)
+    _same(c, a * 4)
