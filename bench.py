@@ -685,6 +685,8 @@ def main():
     dev.synchronize()
     if args.plan:
         from cupy_amd.cuda import function as _function
+        from cupy_amd._core import _launch_plan
+        _launch_plan.use_quick = False      # every launch through Function.launch_packed
         seen = []
         real_launch = _function.Function.launch_packed
 
@@ -701,6 +703,7 @@ def main():
                 plan.append({'name': c['name'], 'bytes': c['bytes'], 'kernels': list(seen)})
         finally:
             _function.Function.launch_packed = real_launch
+            _launch_plan.use_quick = True
         dev.synchronize()
         os.makedirs(os.path.dirname(os.path.abspath(args.plan)), exist_ok=True)
         with open(args.plan, 'w') as f:

@@ -1734,7 +1734,16 @@ class ufunc:
         return self(A, B, **kwargs)
 
     def at(self, a, indices, b=None):
-        raise NotImplementedError(f'`{self.name}.at` is not supported yet')
+        """Applies the operation in place at ``a[indices]``, once per
+        occurrence of an index (``numpy.ufunc.at``); available for the ufuncs
+        that carry a scatter operation: add, subtract, maximum, minimum,
+        bitwise_and / or / xor (cupy/_core/_kernel.pyx:1447-1456)."""
+        if self._scatter_op is None:
+            raise NotImplementedError(f'`{self.name}.at` is not supported yet')
+        if b is None:
+            raise ValueError('second operand needed for ufunc')
+        from cupy_amd._core import _scatter
+        _scatter.scatter_op(a, indices, b, self._scatter_op)
 
     def reduce(self, array, axis=0, dtype=None, out=None, keepdims=False):
         if self.name == 'cupy_add':
@@ -1752,6 +1761,10 @@ class ufunc:
             f'`{self.name}.accumulate` is not supported yet')
 
     def reduceat(self, array, indices, axis=0, dtype=None, out=None):
+        """``numpy.ufunc.reduceat`` for add (cupy/_core/_kernel.pyx:1485-1493)."""
+        if self.name == 'cupy_add':
+            from cupy_amd._core import _scatter
+            return _scatter.add_reduceat(array, indices, axis, dtype, out)
         raise NotImplementedError(
             f'`{self.name}.reduceat` is not supported yet')
 

@@ -16,6 +16,8 @@ The reference repeats its whole per-call path on every call
 cupy/_core/_reduction.pyx:309-427 for reductions); its kernel memo
 (_kernel.pyx:948-975) saves only the compilation.
 """
+import struct
+
 import numpy
 
 from cupy_amd import _rt
@@ -38,6 +40,10 @@ _INF = float('inf')
 
 # Recorded calls kept per kernel object.
 _MAX_PLANS = 256
+
+# False: replays go through Function.launch_packed like first calls do (for
+# code that watches launches there, e.g. to list the kernels of an operation)
+use_quick = True
 
 _SLOT_MARK = 0x5ca7c4a5c4a7c4a5       # stands in for a pointer while its byte offset is looked up
 
@@ -153,7 +159,7 @@ def ranges_overlap(a, b):
 class FastCall:
     """Recorded call: allocates outputs and temporaries, patches pointers and
     scalar values, launches."""
-    __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap')
+    __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap', 'quick')
 
     def __init__(self, n_user, out_specs, rec, ret, overlap=()):
         self.n_user = n_user
@@ -162,6 +168,7 @@ class FastCall:
         self.launches = tuple(rec.launches)
         self.ret = ret                        # ref, tuple of refs, or None
         self.overlap = tuple(overlap)         # (input ref, output ref) pairs to check
+        self.quick = _quick_launches(self.launches)
 
     def run(self, args, stream_ptr=None):
         from cupy_amd._core.core import ndarray
@@ -179,22 +186,85 @@ class FastCall:
             refs.append(_memory.alloc(nbytes))
         if stream_ptr is None:
             stream_ptr = _stream.get_current_stream_ptr()
-        for fn, grid, block, packer, template, ptrs, scalars, shmem in self.launches:
-            vals = template[:]
-            for slot, ref in ptrs:
-                if ref < n_arr:
-                    vals[slot] = refs[ref].data.ptr
-                else:
-                    vals[slot] = refs[ref].ptr
-            for slot, ref, descr in scalars:
-                vals[slot] = scalar_value(refs[ref], descr)
-            fn.launch_packed(grid, block, packer.pack(*vals), shmem, stream_ptr)
+        quick = self.quick
+        if quick is not None and use_quick:
+            # pointer-only argument blocks: the recorded bytes with the
+            # addresses spliced in, handed to the library as they are
+            launch = _rt.lib.rt_launch_packed
+            for fptr, dims, shmem, packer, pieces, slots, size, fn in quick:
+                pieces = pieces[:]            # (other threads replay the same record)
+                k = 1
+                for ref in slots:
+                    pieces[k] = refs[ref].data.ptr if ref < n_arr else refs[ref].ptr
+                    k += 2
+                status = launch(fptr, *dims, shmem, stream_ptr, packer.pack(*pieces), size)
+                if status != 0:
+                    _rt.check(status)
+        else:
+            for fn, grid, block, packer, template, ptrs, scalars, shmem in self.launches:
+                vals = template[:]
+                for slot, ref in ptrs:
+                    if ref < n_arr:
+                        vals[slot] = refs[ref].data.ptr
+                    else:
+                        vals[slot] = refs[ref].ptr
+                for slot, ref, descr in scalars:
+                    vals[slot] = scalar_value(refs[ref], descr)
+                fn.launch_packed(grid, block, packer.pack(*vals), shmem, stream_ptr)
         ret = self.ret
         if ret is None:
             return None
         if type(ret) is tuple:
             return tuple(refs[r] for r in ret)
         return refs[ret]
+
+
+def _quick_launches(launches):
+    """Per recorded launch whose argument block changes only in its pointers:
+    everything ``rt_launch_packed`` takes, with the block cut at the pointer
+    slots -- ``(function handle, grid and block, shared memory, packer of
+    [bytes, pointer, bytes, ...], that list with the bytes filled in, ref per
+    pointer, block size, Function)``.  None if any launch takes a scalar that
+    changes from call to call, or when launches are only recorded."""
+    from cupy_amd import _dryrun
+    if _dryrun.enabled():
+        return None
+    out = []
+    for fn, grid, block, packer, template, ptrs, scalars, shmem in launches:
+        if scalars or not ptrs:
+            return None
+        gx, gy, gz = grid
+        bx, by, bz = block
+        if gx * bx > 0xffffffff or gy * by > 0xffffffff or gz * bz > 0xffffffff:
+            return None
+        vals = list(template)
+        marks = {}
+        for i, (slot, ref) in enumerate(ptrs):
+            vals[slot] = _SLOT_MARK + i
+            marks[(_SLOT_MARK + i).to_bytes(8, 'little')] = ref
+        blob = packer.pack(*vals)
+        if len(blob) > fn._arg_size or len(blob) < fn._arg_min:
+            return None
+        blob += b'\0' * (fn._arg_size - len(blob))
+        found = []
+        for mark, ref in marks.items():
+            off = blob.find(mark)
+            if off < 0 or off % 8 or blob.find(mark, off + 1) >= 0:
+                return None
+            found.append((off, ref))
+        found.sort()
+        pieces, fmt, pos = [], ['<'], 0
+        for off, ref in found:
+            pieces.append(blob[pos:off])
+            fmt.append('%ds' % (off - pos))
+            pieces.append(0)
+            fmt.append('Q')
+            pos = off + 8
+        pieces.append(blob[pos:])
+        fmt.append('%ds' % (len(blob) - pos))
+        out.append((fn.ptr, (gx, gy, gz, bx, by, bz), shmem, struct.Struct(''.join(fmt)),
+                    pieces, tuple(ref for _, ref in found), len(blob), fn))
+    return tuple(out)
 
 
 def _run_static(self, args, stream_ptr):

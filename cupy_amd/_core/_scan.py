@@ -48,7 +48,7 @@ def _acc_type(t):
 
 
 def _emit(in_t, out_t, op, skip_nan, vec, trips, idx64, group=64, stream=(True, False),
-          ragged=True):
+          ragged=True, reuse=False):
     acc_t = _acc_type(out_t)
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     op_c = '+' if op == _SUM else '*'
@@ -68,6 +68,13 @@ typedef %(idx_t)s _idx_t;
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
 #define NT_STORE %(nts)s
+// CHUNK_REUSE: the totals pass and the seeded pass of a chunked scan read the
+// input with plain loads, the seeded pass works through the chunks from the
+// last to the first and stores past the cache: what the totals pass read last
+// is still in the memory-side cache when the seeded pass asks for it first.
+#define CHUNK_REUSE %(reuse)d
+#define NT_LOAD_OF(MODE) ((MODE) == 0 || !CHUNK_REUSE ? NT_LOAD : false)
+#define NT_STORE_OF(MODE) ((MODE) == 2 && CHUNK_REUSE ? true : NT_STORE)
 #define GROUP %(group)d
 // RAGGED: a row may end inside a vector (its length is no multiple of VEC)
 #define RAGGED %(ragged)d
@@ -76,6 +83,7 @@ __device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
 // One round of loads of a group: TRIPS vectors per lane, all unconditional (a
 // vector that would start past the end of the chunk is read from the row start
 // instead, which always holds one; its values are not used).
+template <bool kStream>
 __device__ __forceinline__ void _rows_load(
     cupy::Vec<_in_t, VEC> (&raw)[TRIPS], const _in_t* __restrict__ src, const _idx_t base,
     const _idx_t j0, const _idx_t j1, const int lane) {
@@ -83,7 +91,7 @@ __device__ __forceinline__ void _rows_load(
   for (int t = 0; t < TRIPS; ++t) {
     const _idx_t j = base + (t * GROUP + lane) * VEC;
     const _idx_t jc = (j + VEC <= j1) ? j : 0;
-    if (VEC > 1) raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + jc);
+    if (VEC > 1) raw[t] = cupy::load_vec<_in_t, VEC, kStream>(src + jc);
     else raw[t].v[0] = src[(j < j1) ? j : j0];
   }
 }
@@ -97,8 +105,9 @@ __device__ __forceinline__ void scan_rows_impl(
   const int lane = threadIdx.x %% GROUP;
   const _idx_t n_work = n_rows * n_chunks;
   const _idx_t group_step = (_idx_t)gridDim.x * (%(block)d / GROUP);
-  for (_idx_t w = (_idx_t)blockIdx.x * (%(block)d / GROUP) + threadIdx.x / GROUP; w < n_work;
-       w += group_step) {
+  for (_idx_t w0 = (_idx_t)blockIdx.x * (%(block)d / GROUP) + threadIdx.x / GROUP; w0 < n_work;
+       w0 += group_step) {
+    const _idx_t w = (kMode == 2 && CHUNK_REUSE) ? n_work - 1 - w0 : w0;
     const _idx_t row = w / n_chunks;
     const _idx_t chunk = w - row * n_chunks;
     const _idx_t j0 = chunk * chunk_len;
@@ -109,11 +118,11 @@ __device__ __forceinline__ void scan_rows_impl(
     // the vectors of the first round; later rounds are requested one round
     // ahead, before the current one is scanned
     cupy::Vec<_in_t, VEC> raw[TRIPS];
-    _rows_load(raw, src, j0, j0, j1, lane);
+    _rows_load<NT_LOAD_OF(kMode)>(raw, src, j0, j0, j1, lane);
     for (_idx_t base = j0; base < j1; base += GROUP * VEC * TRIPS) {
       cupy::Vec<_in_t, VEC> next[TRIPS];
       const _idx_t nbase = base + GROUP * VEC * TRIPS;
-      if (nbase < j1) _rows_load(next, src, nbase, j0, j1, lane);
+      if (nbase < j1) _rows_load<NT_LOAD_OF(kMode)>(next, src, nbase, j0, j1, lane);
       _acc_t v[TRIPS][VEC];
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t) {
@@ -161,7 +170,7 @@ __device__ __forceinline__ void scan_rows_impl(
             cupy::Vec<_out_t, VEC> r;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(SCAN_OP(before, v[t][k]));
-            cupy::store_vec<_out_t, VEC, NT_STORE>(dst, r);
+            cupy::store_vec<_out_t, VEC, NT_STORE_OF(kMode)>(dst, r);
           } else if (RAGGED || VEC == 1) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k)
@@ -188,8 +197,9 @@ __device__ __forceinline__ void scan_cols_impl(
     const _idx_t chunk_len) {
   const _idx_t inner_v = inner / VEC;            // the host guarantees inner %% VEC == 0
   const _idx_t n_work = n_outer * n_chunks * inner_v;
-  for (_idx_t w = (_idx_t)blockIdx.x * %(block)d + threadIdx.x; w < n_work;
-       w += (_idx_t)gridDim.x * %(block)d) {
+  for (_idx_t w0 = (_idx_t)blockIdx.x * %(block)d + threadIdx.x; w0 < n_work;
+       w0 += (_idx_t)gridDim.x * %(block)d) {
+    const _idx_t w = (kMode == 2 && CHUNK_REUSE) ? n_work - 1 - w0 : w0;
     const _idx_t iv = w %% inner_v;
     const _idx_t oc = w / inner_v;
     const _idx_t chunk = oc %% n_chunks;
@@ -210,7 +220,7 @@ __device__ __forceinline__ void scan_cols_impl(
       cupy::Vec<_in_t, VEC> raw[TRIPS];
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t)
-        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + col + (ptrdiff_t)(j + t) * inner);
+        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD_OF(kMode)>(in + col + (ptrdiff_t)(j + t) * inner);
 #pragma unroll
       for (int t = 0; t < TRIPS; ++t) {
         cupy::Vec<_out_t, VEC> r;
@@ -219,18 +229,18 @@ __device__ __forceinline__ void scan_cols_impl(
           run[k] = SCAN_OP(run[k], _load_value(raw[t].v[k]));
           r.v[k] = static_cast<_out_t>(run[k]);
         }
-        if (kMode != 1) cupy::store_vec<_out_t, VEC, NT_STORE>(out + col + (ptrdiff_t)(j + t) * inner, r);
+        if (kMode != 1) cupy::store_vec<_out_t, VEC, NT_STORE_OF(kMode)>(out + col + (ptrdiff_t)(j + t) * inner, r);
       }
     }
     for (; j < j1; ++j) {
-      const cupy::Vec<_in_t, VEC> raw = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + col + (ptrdiff_t)j * inner);
+      const cupy::Vec<_in_t, VEC> raw = cupy::load_vec<_in_t, VEC, NT_LOAD_OF(kMode)>(in + col + (ptrdiff_t)j * inner);
       cupy::Vec<_out_t, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) {
         run[k] = SCAN_OP(run[k], _load_value(raw.v[k]));
         r.v[k] = static_cast<_out_t>(run[k]);
       }
-      if (kMode != 1) cupy::store_vec<_out_t, VEC, NT_STORE>(out + col + (ptrdiff_t)j * inner, r);
+      if (kMode != 1) cupy::store_vec<_out_t, VEC, NT_STORE_OF(kMode)>(out + col + (ptrdiff_t)j * inner, r);
     }
     if (kMode == 1) {
 #pragma unroll
@@ -259,7 +269,7 @@ COLS_KERNEL(cupy_scan_cols_seeded, 2)
 ''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident,
            vec=vec, trips=trips, conv=conv, block=_BLOCK, group=group,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
-           ragged=1 if ragged else 0)
+           ragged=1 if ragged else 0, reuse=1 if reuse else 0)
 
 
 def _emit_lanes(in_t, out_t, op, skip_nan, vec, trips, idx64, lstride, stream):
@@ -426,13 +436,13 @@ def _module_lanes(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, lstride,
 
 
 def _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group=64,
-            stream=(True, False), ragged=True):
+            stream=(True, False), ragged=True, reuse=False):
     key = (_device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
-           trips, idx64, group, stream, ragged)
+           trips, idx64, group, stream, ragged, reuse)
     mod = _memo.get(key)
     if mod is None:
         src = _emit(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
-                    vec, trips, idx64, group, stream, ragged)
+                    vec, trips, idx64, group, stream, ragged, reuse)
         mod = compiler.compile_with_cache(src)
         with _lock:
             mod = _memo.setdefault(key, mod)
@@ -480,6 +490,11 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
     else:
         stream = _tuning.stream_policy(setting, total * in_dtype.itemsize,
                                        total * out_dtype.itemsize)
+    # A chunked scan reads its input twice.  While the input is not much larger
+    # than the memory-side cache, the second reading starts where the first
+    # ended and finds (part of) it there.
+    reuse_ok = (_tuning.get('scan_chunk_reuse')
+                and total * in_dtype.itemsize <= 2 * _tuning.get('cache_bytes'))
     if inner == 1:
         vec = max(1, 16 // item)
         while vec > 1 and (not _aligned(src.data.ptr, vec * in_dtype.itemsize)
@@ -506,7 +521,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         chunk_len = (chunk_len + per_group - 1) // per_group * per_group
         n_chunks = (n + chunk_len - 1) // chunk_len
         mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, group, stream,
-                      ragged=n % vec != 0)
+                      ragged=n % vec != 0, reuse=n_chunks > 1 and reuse_ok)
         groups = outer * n_chunks
         per_block = _BLOCK // group
         grid = max(1, min((groups + per_block - 1) // per_block, cus * 32))
@@ -561,7 +576,8 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
             n_chunks = min((want + threads - 1) // threads, n // 64)
         chunk_len = (n + n_chunks - 1) // n_chunks
         n_chunks = (n + chunk_len - 1) // chunk_len
-        mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, 64, stream)
+        mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, 64, stream,
+                      reuse=n_chunks > 1 and reuse_ok)
         work = threads * n_chunks
         grid = max(1, min((work + _BLOCK - 1) // _BLOCK, cus * 64))
         fmt = '@PPP' + ic * 5

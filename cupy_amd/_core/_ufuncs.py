@@ -376,6 +376,14 @@ invert = create_ufunc(
     'cupy_invert', (('?->?', 'out0 = !in0'),) + _sig(_INTS, 1),
     'out0 = ~in0', doc='Elementwise bitwise NOT.')
 bitwise_not = invert
+
+# in-place application at indices (ufunc.at): the operation each of these
+# applies atomically (cupy/_core/_routines_math.pyx:905,1060,
+# cupy/_core/_routines_binary.pyx:23-47 pass the same names as scatter_op=)
+for _uf, _op in ((add, 'add'), (subtract, 'sub'), (maximum, 'max'), (minimum, 'min'),
+                 (bitwise_and, 'and'), (bitwise_or, 'or'), (bitwise_xor, 'xor')):
+    _uf._scatter_op = _op
+del _uf, _op
 left_shift = create_ufunc(
     'cupy_left_shift', _sig(_INTS, 2),
     'out0 = (in1 < 0 || in1 >= (int)(sizeof(in0_type) * 8)) ? (out0_type)0 : (out0_type)(in0 << in1)',

@@ -157,6 +157,29 @@ class _KernelPlan:
             out = (out,)
         return _collect(self.returns, out, args, self.single)
 
+    def replay_runner(self, args):
+        """After ``run(*args)``: a callable that goes straight to the launch
+        record the kernel made for arguments of this signature (skipping the
+        kernel object's own argument checks and signature lookup), or None."""
+        kargs = [r(args) for r in self.readers]
+        key = _launch_plan.call_signature(kargs, _device.get_device_id())
+        if key is None:
+            return None
+        if 'axis' in self.kwargs or hasattr(self.kernel, 'map_expr'):
+            key = key + ((self.kwargs.get('axis'), False),)
+        fast = getattr(self.kernel, '_fast_calls', {}).get(key)
+        if fast is None:
+            return None
+        readers, returns, single, one = self.readers, self.returns, self.single, self.n_targets == 1
+        slow = self.run
+
+        def run(*a):
+            out = fast.run([r(a) for r in readers])
+            if out is NotImplemented:       # an output overlaps an input this time
+                return slow(*a)
+            return _collect(returns, (out,) if one else out, a, single)
+        return run
+
 
 def _collect(returns, outs, args, single):
     """The call's return value from the kernels' outputs and the arguments."""
@@ -302,6 +325,12 @@ class Fusion:
         if plan is _EAGER:
             return self.func(*args)
         run = plan.run
+        first = None
+        if type(plan) is _KernelPlan and not plan.store_positions:
+            # the first call makes the kernel's launch record; later calls with
+            # this signature replay it directly
+            first = plan.run(*args)
+            run = plan.replay_runner(args) or plan.run
         if getattr(plan, 'store_positions', None):
             def run(*a, _plan=plan):
                 if self._writes_overlap(_plan, a):
@@ -311,6 +340,8 @@ class Fusion:
             if len(self._fast) >= 256:
                 self._fast.clear()
             self._fast[sig] = run
+        if type(plan) is _KernelPlan and not plan.store_positions:
+            return first
         return run(*args)
 
     @staticmethod

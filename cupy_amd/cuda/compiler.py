@@ -247,9 +247,19 @@ def get_code_object(source, options=()):
     return payload
 
 
+def _debug_options():
+    """``CUPY_CUDA_COMPILE_WITH_DEBUG=1``: every kernel is compiled with debug
+    information and without optimisation (the reference adds ``--device-debug
+    --generate-line-info``, cupy/cuda/compiler.py:673-674).  The options are part
+    of the cache key, so optimised and debug builds never mix."""
+    if os.environ.get('CUPY_CUDA_COMPILE_WITH_DEBUG', '0') in ('', '0'):
+        return ()
+    return ('-g', '-O0')
+
+
 def compile_with_cache(source, options=()):
     """Loaded module for ``source`` on the current device (memoised)."""
-    options = tuple(options)
+    options = tuple(options) + _debug_options()
     if 'cupy_struct_' in source:
         # structured element types: their definitions follow the device header
         from cupy_amd._core import _structured

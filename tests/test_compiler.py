@@ -100,3 +100,28 @@ def test_get_code_object_uses_disk_cache(tmp_path, monkeypatch):
     # a different option set is a different entry
     compiler.get_code_object(src, ('-DX=1',))
     assert len([n for n in os.listdir(tmp_path) if n.endswith('.hsaco')]) == 2
+
+
+def test_compile_with_debug_switch(tmp_path, monkeypatch):
+    """CUPY_CUDA_COMPILE_WITH_DEBUG (cupy/cuda/compiler.py:673 in the reference):
+    debug information, no optimisation, and a cache entry of its own."""
+    monkeypatch.setenv('CUPY_CACHE_DIR', str(tmp_path))
+    src = ('extern "C" __global__ void debug_probe_kernel(float* x, float a) '
+           '{ x[threadIdx.x] = x[threadIdx.x] * a + 1.0f; }')
+    monkeypatch.delenv('CUPY_CUDA_COMPILE_WITH_DEBUG', raising=False)
+    assert compiler._debug_options() == ()
+    plain = compiler.compile_with_cache(src)
+    monkeypatch.setenv('CUPY_CUDA_COMPILE_WITH_DEBUG', '1')
+    assert compiler._debug_options() == ('-g', '-O0')
+    debug = compiler.compile_with_cache(src)
+    assert debug is not plain
+    assert b'.debug_info' in debug.code and b'.debug_info' not in plain.code
+    assert len([n for n in os.listdir(tmp_path) if n.endswith('.hsaco')]) == 2
+    # header changes reach only the kernels that include the header
+    a = compiler._cache_key('#include <cupy/carray.cuh>\n', (), 'gfx950')
+    b = compiler._cache_key('#include <cupy/carray.cuh>\n#include <cupy/atomics.cuh>\n', (), 'gfx950')
+    assert compiler._get_header_digest('int x;') != compiler._get_header_digest(
+        '#include <cupy/carray.cuh>\n')
+    assert a != b
+    assert compiler._get_header_digest('#include <cupy/carray.cuh>') == \
+        compiler._get_header_digest('#include "cupy/complex.cuh"\n#include <cupy/carray.cuh>')

@@ -33,10 +33,12 @@ def _record_launches(fn):
         seen.append((self.ptr, tuple(grid), tuple(block), shared_mem, bytes(arg_block)))
         return real(self, grid, block, arg_block, shared_mem, stream_ptr)
     _function.Function.launch_packed = spy
+    _launch_plan.use_quick = False       # replays through Function.launch_packed too
     try:
         fn()
     finally:
         _function.Function.launch_packed = real
+        _launch_plan.use_quick = True
     return seen
 
 
