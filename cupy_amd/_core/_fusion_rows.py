@@ -151,6 +151,87 @@ def build(nodes, pieces, returns, single, args, name):
         return None
 
 
+class _RowPiece:
+    """A piece of the row kernel: like ``_fusion_split.Piece`` without a kernel
+    object; ``keep``: the target stays in registers for later pieces."""
+    __slots__ = ('leaves', 'targets', 'reduce', 'keep')
+
+    def __init__(self, leaves, targets, reduce=None, keep=False):
+        self.leaves, self.targets, self.reduce, self.keep = leaves, targets, reduce, keep
+
+
+def _with_kept_values(nodes, pieces, kinds, returns, full_leaves, row_words, lane_elems):
+    from cupy_amd._core._fusion_split import leaves_of
+    consumers = {}
+    for n in nodes:
+        for a in n.inputs:
+            consumers.setdefault(a.order, []).append(n)
+    keep = []
+    for p in pieces:
+        if p.reduce is None:
+            continue
+        src = p.reduce.src
+        if src.kind != 'apply' or kinds.get(src.order) != 'full':
+            continue
+        if len(consumers.get(src.order, ())) < 2:
+            continue
+        keep.append(src)
+    if not keep:
+        return pieces
+    # register budget: a kept array that replaces the row operands it came from
+    # is free, any other counts like one more row operand
+    later_roots = [v for kind, v in returns if kind == 'value']
+    words = row_words
+    accepted = []
+    for src in keep:
+        feeds = [l for l in leaves_of([src], set(n.order for n in full_leaves))]
+        others = [n for n in nodes if n.order > src.order and n.kind in ('apply', 'reduce')
+                  and not _depends_only_through(n, src, feeds)]
+        replaces = bool(feeds) and not others
+        cost = lane_elems * max(1, src.dtype.itemsize // 4)
+        if replaces or words + cost <= _ROW_WORDS_PER_LANE:
+            accepted.append(src)
+            if not replaces:
+                words += cost
+    if not accepted:
+        return pieces
+    # the pieces again, with the kept values as starting points
+    stored = set(n.order for n in nodes if n.kind in ('array', 'scalar'))
+    out = []
+    kept_orders = set(v.order for v in accepted)
+    for p in pieces:
+        if p.reduce is not None:
+            src = p.reduce.src
+            if src.order in kept_orders and src.order not in stored:
+                out.append(_RowPiece(leaves_of([src], stored), [src], keep=True))
+                stored.add(src.order)
+            out.append(_RowPiece(leaves_of([src], stored), list(p.targets), reduce=p.reduce))
+            stored.add(p.reduce.order)
+            for n in nodes:
+                if n.kind == 'keepdims' and n.src is p.reduce:
+                    stored.add(n.order)
+        else:
+            out.append(_RowPiece(leaves_of(list(p.targets), stored), list(p.targets)))
+    return out
+
+
+def _depends_only_through(n, kept, feeds):
+    """True unless ``n`` reads one of the row operands ``feeds`` by a path that
+    does not pass through ``kept``."""
+    feed_orders = set(f.order for f in feeds)
+    stack = [n]
+    seen = set()
+    while stack:
+        v = stack.pop()
+        if v.order in seen or v is kept:
+            continue
+        seen.add(v.order)
+        if v.order in feed_orders:
+            return False
+        stack.extend(v.inputs)
+    return True
+
+
 def _build(nodes, pieces, returns, single, args, name):
     reduces = [n for n in nodes if n.kind == 'reduce']
     if not reduces:
@@ -204,6 +285,16 @@ def _build(nodes, pieces, returns, single, args, name):
     words = words_for(group)
     if words > _ROW_WORDS_PER_LANE or n_cols < 2:
         raise _Unsupported('row of %d elements does not fit the registers of a group' % n_cols)
+
+    # ---- values kept in registers between pieces -------------------------------------------
+    # The source of a reduction that later pieces need again (the exponentials
+    # of a softmax: summed, then divided by the sum) is evaluated once, into a
+    # register array of its own, instead of once per piece -- when that does not
+    # raise the register count: the row operands it is computed from must not be
+    # needed afterwards (the array then takes their place), or everything still
+    # fits the budget of one row.
+    pieces = _with_kept_values(nodes, pieces, kinds, returns, full_leaves,
+                               words, per_lane * vec)
 
     # ---- every piece as device functions -------------------------------------------------
     dtype_of = dict((n.order, n.dtype) for n in nodes)
@@ -357,12 +448,29 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
             return operand(n.src)
         if k == 'full' and n.kind == 'array':
             return '_f%d[_e].v[_k]' % n.order
+        if k == 'full' and n.order in kept_names:
+            return '_m%d[_e].v[_k]' % n.order
         if k == 'col' and n.kind == 'array':
             return '_c%d[_e].v[_k]' % n.order
         raise _Unsupported('value %d (%s, %s) is not available here' % (n.order, n.kind, k))
 
+    kept_names = set()
     for k, (p, d) in enumerate(zip(pieces, described)):
         call_args = [operand(l) for l in p.leaves]
+        if getattr(p, 'keep', False):
+            (t,) = p.targets
+            src.append('    cupy::Vec<%s, VEC> _m%d[PER_LANE];' % (
+                get_typename(dtype_of[t.order]), t.order))
+            src.append('#pragma unroll')
+            src.append('    for (int _e = 0; _e < PER_LANE; ++_e) {')
+            src.append('#pragma unroll')
+            src.append('      for (int _k = 0; _k < VEC; ++_k) {')
+            src.append('        piece%d::elementwise(%s);' % (
+                k, ', '.join(call_args + ['_m%d[_e].v[_k]' % t.order])))
+            src.append('      }')
+            src.append('    }')
+            kept_names.add(t.order)
+            continue
         if d['kind'] == 'reduce':
             (target,) = p.targets
             ident = _cg._identity_decl(d['identity']).replace('_type_reduce', 'piece%d::reduce_t' % k)

@@ -357,6 +357,10 @@ class _ElementwisePlanner:
             _cg.uses_identifier(loop_prep, '_ind') or \
             _cg.uses_identifier(after_loop, '_ind')
         self._uses_i = _cg.uses_identifier(operation, 'i')
+        # False: the kernel sees the axes of the broadcast arguments as they
+        # are (``reduce_dims=False``): no axes are merged, ``_ind`` and the
+        # arrays keep their number of dimensions
+        self.reduce_dims = True
 
     # One operand description per kernel parameter -------------------------------------
     def _make_operands(self, args, nin, var_types, casts, force_read_out):
@@ -406,6 +410,8 @@ class _ElementwisePlanner:
         if arrays and any(a.dtype.kind == 'V' for a in arrays):
             # elements that are structures go one by one through the indexer
             # kernel (the vector helpers want element sizes that are powers of two)
+            force_generic = True
+        if not self.reduce_dims:
             force_generic = True
         if not (force_generic or self._force_generic) and arrays:
             cshape, cstrides = _canonical_dims(arrays, shape)
@@ -972,7 +978,7 @@ class _ElementwisePlanner:
         arrays_idx = [i for i, (a, p) in enumerate(zip(args, params))
                       if isinstance(a, ndarray) and not p.raw]
         args = list(args)
-        if arrays_idx:
+        if arrays_idx and self.reduce_dims:
             arrays = [args[i] for i in arrays_idx]
             cshape, cstrides = _canonical_dims(arrays, shape)
             if len(cshape) != len(shape):
@@ -1156,6 +1162,7 @@ class ElementwiseKernel:
         self._planner = _ElementwisePlanner(
             name, self.in_params + self.out_params, operation, preamble,
             loop_prep, after_loop, options, is_ufunc=False)
+        self._planner.reduce_dims = bool(reduce_dims)
         self._cached_codes = self._planner._codes
         self._fast_calls = {}
 

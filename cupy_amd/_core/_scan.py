@@ -422,6 +422,191 @@ LANES_KERNEL(cupy_scan_lanes_seeded, 2)
            nts='true' if stream[1] else 'false')
 
 
+def _tile_geometry(inner, vec, trips):
+    """(rows per round, segments, rows per segment, words between segments in
+    the LDS) of the staged kernel for ``inner`` columns."""
+    tile = _WAVE * vec * trips
+    seg = _WAVE // inner
+    lrows = (tile // inner) // seg
+    # segments start `inner` banks apart, so the lanes of one access touch
+    # distinct banks
+    pad = (inner - (lrows * inner) % 32) % 32
+    return seg * lrows, seg, lrows, lrows * inner + pad
+
+
+def _emit_tile(in_t, out_t, op, skip_nan, vec, trips, idx64, inner, stream, reuse):
+    """Scan along the middle axis of (outer, n, inner) for 2 <= inner <= 32.
+
+    A wave takes ``ROWS_T`` consecutive rows per round -- one contiguous piece
+    of memory, read with full 128-bit vectors on consecutive lanes whatever the
+    width of the array -- and lays them out in the LDS.  Lane (s, c) then owns
+    ``LROWS`` consecutive rows of column c (segment s of the tile): it scans them
+    in registers, the totals of the segments of a column are scanned across the
+    lanes (shuffles in steps of ``INNER`` lanes), every lane adds what came
+    before its segment, and the tile goes back through the LDS into one
+    contiguous store.  No barrier: a wave only ever reads what it wrote itself."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    rows_t, seg, lrows, stride = _tile_geometry(inner, vec, trips)
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define CHUNK_REUSE %(reuse)d
+#define NT_LOAD_OF(MODE) ((MODE) == 0 || !CHUNK_REUSE ? NT_LOAD : false)
+#define NT_STORE_OF(MODE) ((MODE) == 2 && CHUNK_REUSE ? true : NT_STORE)
+#define INNER %(inner)d
+#define ROWS_T %(rows_t)d
+#define SEG %(seg)d
+#define LROWS %(lrows)d
+#define SEG_STRIDE %(stride)d
+#define LDS_WORDS (SEG * SEG_STRIDE)
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+// position in the LDS of element p of the tile (p = row * INNER + column)
+__device__ __forceinline__ int _lds_at(int p) { return p + (p / (LROWS * INNER)) * (SEG_STRIDE - LROWS * INNER); }
+
+template <int kMode>
+__device__ __forceinline__ void scan_tile_impl(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, _acc_t* __restrict__ totals,
+    const _idx_t n_outer, const _idx_t n, const _idx_t n_chunks, const _idx_t chunk_rows) {
+  __shared__ _acc_t _lds_all[%(block)d / 64][LDS_WORDS];
+  _acc_t* lds = _lds_all[threadIdx.x / 64];
+  const int lane = threadIdx.x %% 64;
+  const int seg = lane / INNER;
+  const int col = lane - seg * INNER;
+  const bool active = lane < SEG * INNER;
+  const _idx_t n_work = n_outer * n_chunks;
+  const _idx_t wave_step = (_idx_t)gridDim.x * (%(block)d / 64);
+  for (_idx_t w0 = (_idx_t)blockIdx.x * (%(block)d / 64) + threadIdx.x / 64; w0 < n_work;
+       w0 += wave_step) {
+    const _idx_t w = (kMode == 2 && CHUNK_REUSE) ? n_work - 1 - w0 : w0;
+    const _idx_t o = w / n_chunks;
+    const _idx_t chunk = w - o * n_chunks;
+    const _idx_t r0 = chunk * chunk_rows;
+    const _idx_t r1 = (r0 + chunk_rows < n) ? (r0 + chunk_rows) : n;
+    _acc_t carry = SCAN_IDENTITY;
+    if (kMode == 2 && chunk > 0 && active)
+      carry = totals[((ptrdiff_t)o * n_chunks + chunk - 1) * INNER + col];
+    for (_idx_t rb = r0; rb < r1; rb += ROWS_T) {
+      const int rows_here = (r1 - rb < ROWS_T) ? (int)(r1 - rb) : ROWS_T;
+      const int valid = rows_here * INNER;
+      const _in_t* src = in + ((ptrdiff_t)o * n + rb) * INNER;
+      _out_t* dst = out + ((ptrdiff_t)o * n + rb) * INNER;
+      // every load of the round is requested before the first value is used
+      cupy::Vec<_in_t, VEC> raw[TRIPS];
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const int p = (t * 64 + lane) * VEC;
+        if (p + VEC <= valid) {
+          raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD_OF(kMode)>(src + p);
+        } else {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) raw[t].v[k] = (p + k < valid) ? src[p + k] : _in_t();
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const int p = (t * 64 + lane) * VEC;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          if (p + k < ROWS_T * INNER)
+            lds[_lds_at(p + k)] = (p + k < valid) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      // the lane's own rows of its column, scanned in registers
+      _acc_t v[LROWS];
+      if (active) {
+#pragma unroll
+        for (int i = 0; i < LROWS; ++i) v[i] = lds[seg * SEG_STRIDE + i * INNER + col];
+#pragma unroll
+        for (int i = 1; i < LROWS; ++i) v[i] = SCAN_OP(v[i - 1], v[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < LROWS; ++i) v[i] = SCAN_IDENTITY;
+      }
+      // totals of the segments of one column sit INNER lanes apart
+      _acc_t incl = v[LROWS - 1];
+#pragma unroll
+      for (int d = 1; d < SEG; d <<= 1) {
+        const _acc_t other = cupy::shfl_up<64>(incl, d * INNER);
+        incl = (lane >= d * INNER) ? SCAN_OP(other, incl) : incl;
+      }
+      const _acc_t column_total = cupy::shfl_idx<64>(incl, (SEG - 1) * INNER + col);
+      if (kMode != 1) {
+        _acc_t before = cupy::shfl_up<64>(incl, INNER);
+        before = (seg == 0) ? carry : SCAN_OP(carry, before);
+        if (active) {
+#pragma unroll
+          for (int i = 0; i < LROWS; ++i)
+            lds[seg * SEG_STRIDE + i * INNER + col] = SCAN_OP(before, v[i]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < TRIPS; ++t) {
+          const int p = (t * 64 + lane) * VEC;
+          if (p + VEC <= valid) {
+            cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(lds[_lds_at(p + k)]);
+            cupy::store_vec<_out_t, VEC, NT_STORE_OF(kMode)>(dst + p, r);
+          } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k)
+              if (p + k < valid) dst[p + k] = static_cast<_out_t>(lds[_lds_at(p + k)]);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+      carry = SCAN_OP(carry, column_total);
+    }
+    if (kMode == 1 && lane < INNER)
+      totals[((ptrdiff_t)o * n_chunks + chunk) * INNER + col] = carry;
+  }
+}
+
+#define TILE_KERNEL(NAME, MODE) \\
+extern "C" __global__ void __launch_bounds__(%(block)d) NAME( \\
+    const _in_t* in, _out_t* out, _acc_t* totals, const _idx_t n_outer, const _idx_t n, \\
+    const _idx_t n_chunks, const _idx_t chunk_rows) { \\
+  scan_tile_impl<MODE>(in, out, totals, n_outer, n, n_chunks, chunk_rows); }
+TILE_KERNEL(cupy_scan_tile, 0)
+TILE_KERNEL(cupy_scan_tile_totals, 1)
+TILE_KERNEL(cupy_scan_tile_seeded, 2)
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           inner=inner, rows_t=rows_t, seg=seg, lrows=lrows, stride=stride,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
+           reuse=1 if reuse else 0)
+
+
+def _module_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream, reuse):
+    key = ('tile', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
+           trips, idx64, inner, stream, reuse)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_tile(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                         vec, trips, idx64, inner, stream, reuse)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
 def _module_lanes(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, lstride, stream):
     key = ('lanes', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
            trips, idx64, lstride, stream)
@@ -535,6 +720,32 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         prefix = 'cupy_scan_rows'
         totals_shape = (outer, n_chunks, 1)
         middle_round = _WAVE * 4 * 4          # elements one wave takes per round
+    elif 2 <= inner <= 32 and _tuning.get('scan_tile'):
+        vec = max(1, 16 // item)
+        trips = 4
+        rows_t, _, _, _ = _tile_geometry(inner, vec, trips)
+        want = cus * _tuning.get('scan_waves_per_cu')
+        n_chunks = 1
+        if may_chunk and outer < want and n > 2 * rows_t:
+            n_chunks = min((want + outer - 1) // outer, (n + rows_t - 1) // rows_t)
+        chunk_len = (n + n_chunks - 1) // n_chunks
+        chunk_len = (chunk_len + rows_t - 1) // rows_t * rows_t
+        n_chunks = (n + chunk_len - 1) // chunk_len
+        mod = _module_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream,
+                           n_chunks > 1 and reuse_ok)
+        waves = outer * n_chunks
+        per_block = _BLOCK // _WAVE
+        grid = max(1, min((waves + per_block - 1) // per_block, cus * 32))
+        fmt = '@PPP' + ic * 4
+
+        def launch(name, totals_ptr):
+            blob = struct.pack(fmt, src.data.ptr, dst.data.ptr, totals_ptr, outer, n,
+                               n_chunks, chunk_len)
+            mod.get_function(name).launch_packed(
+                (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+        prefix = 'cupy_scan_tile'
+        totals_shape = (outer, n_chunks, inner)
+        middle_round = rows_t
     elif _lanes_geometry(src, dst, inner, item) is not None:
         vec, lstride = _lanes_geometry(src, dst, inner, item)
         trips = 4

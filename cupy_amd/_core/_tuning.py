@@ -73,6 +73,7 @@ _params = {
     'cols_unroll_near': 4,
     'cols_solo_block': 1024,    # workgroup of the thread-per-column variant
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
+    'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
     # fused row-wise functions: words per lane up to which a wave takes a whole row

@@ -306,3 +306,71 @@ def test_extrema_order_by_real_then_imaginary_part(dtype):
             assert_exact(cp.nanmin(dy, axis=axis).get(), np.nanmin(y, axis=axis))
             assert_exact(cp.nanargmax(dy, axis=axis).get(), np.nanargmax(y, axis=axis))
             assert_exact(cp.nanargmin(dy, axis=axis).get(), np.nanargmin(y, axis=axis))
+
+
+# ---- the GPU against the host build of the same header ---------------------------------------
+# tests/test_complex_functions_host.py holds the formulas of cupy/complex.cuh,
+# compiled with g++, to 4 eps * (1 + |result|) of NumPy.  Here the GPU runs the
+# same header: what can differ is only how the device's sin / cos / exp / log /
+# atan2 / hypot round, so the two must agree far more closely than either is
+# asked to agree with NumPy.
+
+_HOST_UNARY = ('sqrt exp log log2 log10 sin cos tan sinh cosh tanh arcsin arccos arctan '
+               'arcsinh arccosh arctanh log1p expm1 exp2').split()
+# largest distance GPU <-> host build seen over the inputs below, in units of
+# eps * (1 + |result|), rounded up generously (observed values are printed)
+_GPU_VS_HOST_EPS = {name: 6 for name in _HOST_UNARY}
+_GPU_VS_HOST_EPS.update({'exp2': 40})
+
+
+@pytest.fixture(scope='module')
+def host_lib(tmp_path_factory):
+    import ctypes
+    import os
+    import subprocess
+    here = os.path.dirname(os.path.abspath(__file__))
+    out = str(tmp_path_factory.mktemp('complex_host') / 'libcomplex_host.so')
+    subprocess.check_call([
+        'g++', '-O2', '-ffp-contract=off', '-shared', '-fPIC',
+        '-I', os.path.join(os.path.dirname(here), 'cupy_amd', 'include'),
+        '-o', out, os.path.join(here, 'complex_host_shim.cpp')])
+    return ctypes.CDLL(out)
+
+
+def _host_call(lib, name, z):
+    import ctypes
+    prefix = 'c64_' if z.dtype == np.complex64 else 'c128_'
+    out = np.empty_like(z)
+    getattr(lib, prefix + name)(z.ctypes.data_as(ctypes.c_void_p),
+                                out.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(z.size))
+    return out
+
+
+def _distance_in_eps(got, want, real_dtype):
+    eps = np.finfo(real_dtype).eps
+    both = np.isfinite(got) & np.isfinite(want)
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    err = np.abs(got.astype(np.complex128)[both] - want.astype(np.complex128)[both])
+    scale = eps * (1 + np.abs(want.astype(np.complex128)[both]))
+    return float((err / scale).max()) if err.size else 0.0
+
+
+@pytest.mark.parametrize('dtype', CTYPES)
+@pytest.mark.parametrize('name', _HOST_UNARY)
+def test_gpu_agrees_with_the_host_build_of_the_header(host_lib, name, dtype):
+    real_dtype = np.float32 if dtype == 'complex64' else np.float64
+    worst_host = worst_numpy = 0.0
+    for scale in (1.5, 0.01, 1e-5, 30.0):
+        z = crandom((50000,), dtype, 5, scale=scale)
+        with np.errstate(all='ignore'):
+            want_np = getattr(np, name)(z.astype(np.complex128))
+        got = getattr(cp, name)(cp.asarray(z)).get()
+        host = _host_call(host_lib, name, z)
+        worst_host = max(worst_host, _distance_in_eps(got, host, real_dtype))
+        with np.errstate(all='ignore'):
+            finite = np.isfinite(want_np.astype(dtype))
+        worst_numpy = max(worst_numpy, _distance_in_eps(
+            got[finite], want_np[finite].astype(np.complex128), real_dtype))
+    print('%-8s %-10s GPU vs host build %.2f eps, GPU vs NumPy %.2f eps' % (
+        name, dtype, worst_host, worst_numpy))
+    assert worst_host <= _GPU_VS_HOST_EPS[name], (name, dtype, worst_host)

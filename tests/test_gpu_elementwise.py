@@ -521,3 +521,29 @@ def test_permuted_windows_and_mixed_types():
     assert_exact((da + db).get(), a + b)
     assert_exact((da.transpose(1, 0, 2) > db.transpose(1, 0, 2)).get(),
                  a.transpose(1, 0, 2) > b.transpose(1, 0, 2))
+
+
+def test_reduce_dims_false_keeps_the_axes_for_the_kernel():
+    """``reduce_dims=False`` (cupy/_core/_kernel.pyx:802-868): the kernel sees the
+    broadcast arguments with all their axes, so ``_ind.get()[k]`` is the index
+    along axis k and raw arrays can be addressed with it."""
+    k = cp.ElementwiseKernel(
+        'T x', 'int64 y',
+        'y = _ind.get()[0] * 10000 + _ind.get()[1] * 100 + _ind.get()[2] + (x > 1e30f ? 1 : 0)',
+        'multi_index', reduce_dims=False)
+    x = cp.asarray(np.zeros((7, 11, 13), np.float32))
+    i0, i1, i2 = np.meshgrid(np.arange(7), np.arange(11), np.arange(13), indexing='ij')
+    assert_exact(k(x).get(), (i0 * 10000 + i1 * 100 + i2).astype(np.int64))
+    # a transposed view keeps its axes too
+    got = k(x.transpose(2, 0, 1)).get()
+    j0, j1, j2 = np.meshgrid(np.arange(13), np.arange(7), np.arange(11), indexing='ij')
+    assert_exact(got, (j0 * 10000 + j1 * 100 + j2).astype(np.int64))
+    # gather along the last two axes of a raw array with the loop's own indices
+    g = cp.ElementwiseKernel(
+        'raw T src, int32 row', 'T out',
+        'ptrdiff_t idx[2] = {row, _ind.get()[1]}; out = src[idx]', 'gather_rows',
+        reduce_dims=False)
+    src = np.arange(5 * 6, dtype=np.float32).reshape(5, 6)
+    rows = np.array([[4], [0], [2]], np.int32)
+    out = g(cp.asarray(src), cp.broadcast_to(cp.asarray(rows), (3, 6)))
+    assert_exact(out.get(), src[rows[:, 0]])

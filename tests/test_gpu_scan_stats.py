@@ -264,7 +264,10 @@ def test_one_pass_variance_is_stable_and_matches_numpy(dtype):
                                         # rows that do not fill a power-of-two number of lanes
                                         ((100001, 3), 0), ((5000, 7), 0), ((3, 70000, 5), 1),
                                         ((40000, 12), 0), ((999, 20), 0), ((70001, 48), 0),
-                                        ((6000, 100), 0), ((2, 9000, 31), 1), ((64, 6), 0)])
+                                        ((6000, 100), 0), ((2, 9000, 31), 1), ((64, 6), 0),
+                                        # whole rounds of the staged kernel, one row more, one less
+                                        ((336 * 3, 3), 0), ((336 * 50 + 1, 3), 0), ((204 * 7 - 1, 5), 0),
+                                        ((2000003, 3), 0), ((5, 64 * 9 + 1, 32), 1), ((300001, 2), 0)])
 @pytest.mark.parametrize('dtype', ['float32', 'float64', 'int32', 'float16'])
 def test_scans_along_an_axis_with_a_narrow_tail(shape, axis, dtype):
     """The axes after the scanned one span a few vectors only: rows sit in
@@ -350,3 +353,27 @@ def test_variance_with_unrepresentative_edges_and_sentinels(dtype):
     assert not cp.asarray(c).var(axis=0).get().any()
     assert not cp.asarray(c).var(axis=1).get().any()
     assert float(cp.asarray(c).var().get()) == 0.0
+
+
+def test_narrow_scans_of_other_types_and_operations():
+    """int8 -> int64, complex and products through the kernel that stages
+    narrow arrays in the LDS."""
+    rng = np.random.default_rng(94)
+    h8 = rng.integers(-100, 100, (150001, 3)).astype(np.int8)
+    assert np.array_equal(cp.cumsum(cp.asarray(h8), axis=0).get(), np.cumsum(h8, axis=0))
+    hu = rng.integers(0, 255, (4, 30011, 7)).astype(np.uint8)
+    assert np.array_equal(cp.cumsum(cp.asarray(hu), axis=1).get(), np.cumsum(hu, axis=1))
+    hc = (rng.standard_normal((70001, 5)) + 1j * rng.standard_normal((70001, 5))).astype(np.complex64)
+    got = cp.cumsum(cp.asarray(hc), axis=0).get()
+    want = np.cumsum(hc.astype(np.complex128), axis=0)
+    scale = np.cumsum(np.abs(hc).astype(np.float64), axis=0)
+    assert (np.abs(got - want) <= 1e-5 * scale + 1e-5).all()
+    hp = rng.choice(np.array([-1, 1, 1, 2], dtype=np.int64), size=(40, 6))
+    hp = np.concatenate([hp, np.ones((60000, 6), np.int64)])
+    rng.shuffle(hp, axis=0)
+    assert np.array_equal(cp.cumprod(cp.asarray(hp), axis=0).get(), np.cumprod(hp, axis=0))
+    hb = rng.integers(0, 2, (100000, 12)).astype(bool)
+    assert np.array_equal(cp.cumsum(cp.asarray(hb), axis=0).get(), np.cumsum(hb, axis=0))
+    out = cp.empty((150001, 3), np.float64)
+    r = cp.cumsum(cp.asarray(h8), axis=0, out=out)
+    assert r is out and np.array_equal(out.get(), np.cumsum(h8, axis=0, dtype=np.float64))

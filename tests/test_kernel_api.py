@@ -308,3 +308,19 @@ def test_fuse_decorator_forms_and_argument_checks():
     # not expressible in the single fused kernel: runs as a kernel sequence
     assert keep(x).shape == (1,)
     assert list(keep._memo.values()) == ['by shape'] and len(keep._plans) == 1
+
+
+def test_reduce_dims_false_is_passed_to_the_launch():
+    from cupy_amd import _dryrun
+    if not _dryrun.enabled():
+        pytest.skip('inspects recorded launches')
+    body = 'y = x + _ind.get()[0]'
+    x = cp.zeros((3, 4, 5), np.float32)
+    sizes = {}
+    for flag in (True, False):
+        k = cp.ElementwiseKernel('T x', 'T y', body, 'keeps_axes', reduce_dims=flag)
+        k(x)
+        sizes[flag] = len(_dryrun.launches[-1][4])
+    # kept: two 3-d arrays and a 3-d indexer; merged: one axis, far fewer bytes
+    assert sizes[False] == (8 + 8 * 7) * 2 + 8 * 7
+    assert sizes[True] < sizes[False]
