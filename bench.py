@@ -576,6 +576,7 @@ def launch_latency(cp):
     out = {}
     x = cp.zeros((1,), np.float32)
     y = cp.zeros((1,), np.float32)
+    y0 = y.reshape(())
     k = cp.ElementwiseKernel('T x', 'T y', 'y = x + 1', 'tiny_add')
 
     @cp.fuse(kernel_name='tiny_fused')
@@ -588,7 +589,7 @@ def launch_latency(cp):
         pool.malloc(4096)
 
     ops = {'ElementwiseKernel': lambda: k(x, y), 'ufunc_add': lambda: cp.add(x, x, y),
-           'sum': lambda: x.sum(out=y.reshape(())), 'fuse': lambda: fz(x),
+           'sum': lambda: x.sum(out=y0), 'fuse': lambda: fz(x),
            'pool_malloc_free': pool_cycle}
     for name, fn in ops.items():
         for _ in range(20):

@@ -34,10 +34,15 @@ def _indexer_init(shape):
     return Indexer(shape)
 
 
+_byte_extent = None      # core._byte_extent, bound at the first call (core imports this module)
+
+
 def may_share_bounds(a, b):
     """True if the byte ranges spanned by two arrays of one allocation
     intersect (reference: cupy/_core/_memory_range.pyx:46-59)."""
-    from cupy_amd._core.core import _byte_extent
+    global _byte_extent
+    if _byte_extent is None:
+        from cupy_amd._core.core import _byte_extent
     if (a.data.device_id != b.data.device_id
             or a.data.mem.ptr != b.data.mem.ptr
             or a.size == 0 or b.size == 0):

@@ -147,9 +147,9 @@ def _finish(args, partial_out, pad, i_expr='_i', s_expr='_s', split_expr='blockI
 
 def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', group=64, vec=4,
-              idx64=False, partial_out=False, stream_hint=False, unroll=2):
+              idx64=False, partial_out=False, stream_hint=False, unroll=2, block=BLOCK):
     """Reduce-axis-contiguous kernel.  ``group`` lanes per row (power of two up
-    to 64) or 256 for a workgroup per row.  With ``partial_out`` the reduce
+    to 64) or ``BLOCK`` for a workgroup (of ``block`` threads) per row.  With ``partial_out`` the reduce
     range is cut into gridDim.y chunks of ``_chunk`` elements (an extra kernel
     parameter) and each (chunk, row) writes one ``_type_reduce`` partial."""
     idx_t = 'ptrdiff_t' if idx64 else 'int'
@@ -159,13 +159,14 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     if partial_out:
         params += ', const %s _chunk' % idx_t
     block_mode = group >= BLOCK
-    lanes = BLOCK if block_mode else group
+    wg = block if block_mode else BLOCK
+    lanes = wg if block_mode else group
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
-        BLOCK, name, params))
+        wg, name, params))
     src.append(_SIZE_INDEXERS)
     if block_mode:
-        src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (BLOCK // WAVE))
+        src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (wg // WAVE))
         src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
         src.append('  const int _lane = threadIdx.x;')
         src.append('  const %s _first = blockIdx.x;' % idx_t)
@@ -256,7 +257,7 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         src.append('    __syncthreads();')
         src.append('    if (threadIdx.x == 0) {')
         src.append('      _s = _sm[0];')
-        src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[_w]);' % (BLOCK // WAVE))
+        src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[_w]);' % (wg // WAVE))
         src.extend(_finish(args, partial_out, '      '))
         src.append('    }')
         src.append('    __syncthreads();')

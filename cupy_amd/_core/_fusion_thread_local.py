@@ -3,14 +3,30 @@ trace is in progress (reference: cupy/_core/_fusion_thread_local.pyx:1-46)."""
 import threading
 
 thread_local = threading.local()
+# recordings in progress in any thread: callers on the launch path test this
+# before they look at their own thread's state
+recording = 0
+_recording_lock = threading.Lock()
+
+
+def begin_recording():
+    global recording
+    with _recording_lock:
+        recording += 1
+
+
+def end_recording():
+    global recording
+    with _recording_lock:
+        recording -= 1
 
 
 def is_fusing():
-    return getattr(thread_local, 'history', None) is not None
+    return recording != 0 and getattr(thread_local, 'history', None) is not None
 
 
 def is_old_fusing():
-    return getattr(thread_local, 'is_old_fusing', False)
+    return recording != 0 and getattr(thread_local, 'is_old_fusing', False)
 
 
 def call_ufunc(fusion_op, *args, **kwargs):

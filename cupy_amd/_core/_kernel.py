@@ -1177,6 +1177,13 @@ class ElementwiseKernel:
             block_size (int): Threads per workgroup of the strided fallback
                 kernel (default 128).
         """
+        if not kwargs and len(args) == self.nargs:
+            # the common call, seen before: straight to its recorded launches
+            fast_key = _launch_plan.call_signature(args, _device.get_device_id())
+            if fast_key is not None:
+                fast = self._fast_calls.get(fast_key)
+                if fast is not None:
+                    return fast.run(args)
         size = kwargs.pop('size', -1)
         stream = kwargs.pop('stream', None)
         block_size = kwargs.pop('block_size', 128)
@@ -1540,17 +1547,17 @@ class ufunc:
             casting (str): Rule for casting results into given outputs
                 (default ``'same_kind'``).
         """
-        for arg in args:
-            if hasattr(arg, '__cupy_override_elementwise_kernel__'):
-                return arg.__cupy_override_elementwise_kernel__(
-                    self, *args, **kwargs)
-        if _fusion_thread_local.is_fusing():
+        if _fusion_thread_local.recording and _fusion_thread_local.is_fusing():
+            for arg in args:
+                if hasattr(arg, '__cupy_override_elementwise_kernel__'):
+                    return arg.__cupy_override_elementwise_kernel__(
+                        self, *args, **kwargs)
             return _fusion_thread_local.call_ufunc(self, *args, **kwargs)
-        for arg in args:
-            if type(arg) is ndarray and arg.dtype.kind == 'V':
-                return _call_structured(self, args, kwargs)
 
         # A call that looks like an earlier one replays that call's launch.
+        # (Only plain arrays and scalars have a signature, and calls with
+        # structured arrays are never recorded, so a hit needs none of the
+        # checks below.)
         fast_key = rec = fast_args = None
         nk = len(kwargs)
         if nk == 0:
@@ -1567,8 +1574,15 @@ class ufunc:
                     if ret is not NotImplemented:
                         return ret
                     fast_key = None
-                else:
-                    rec = _launch_plan.Recorder(self.nargs)
+        for arg in args:
+            if hasattr(arg, '__cupy_override_elementwise_kernel__'):
+                return arg.__cupy_override_elementwise_kernel__(
+                    self, *args, **kwargs)
+        for arg in args:
+            if type(arg) is ndarray and arg.dtype.kind == 'V':
+                return _call_structured(self, args, kwargs)
+        if fast_key is not None:
+            rec = _launch_plan.Recorder(self.nargs)
 
         out = kwargs.pop('out', None)
         where = kwargs.pop('_where', None)

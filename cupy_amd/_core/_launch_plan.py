@@ -20,7 +20,9 @@ import struct
 
 import numpy
 
+from cupy_amd import _dryrun
 from cupy_amd import _rt
+from cupy_amd._core import _carray
 from cupy_amd._core import _tuning
 from cupy_amd._core._scalar import CScalar
 from cupy_amd.cuda import memory as _memory
@@ -126,34 +128,20 @@ def launch(rec, fn, grid, block, packer, argblock, stream_ptr, shared_mem=0):
 
 
 def call_signature(args, dev_id):
-    """Hashable description of everything about ``args`` that launch decisions
-    may depend on, or None if the call must take the full path."""
-    from cupy_amd._core.core import ndarray
-    sig = [dev_id, _tuning.version()]
-    for a in args:
-        t = type(a)
-        if t is ndarray:
-            d = a.data
-            if d.device_id != dev_id:
-                return None
-            sig.append((a.dtype, a._shape, a._strides, d.ptr & 15))
-        elif t is float or t is bool or t is complex:
-            sig.append(t)
-        elif t is int:
-            if not (_INT64_MIN <= a <= _INT64_MAX):
-                return None
-            sig.append(t)
-        elif isinstance(a, numpy.generic):
-            sig.append(t)
-        else:
-            return None
-    return tuple(sig)
+    """Hashable description of everything about ``args`` (a tuple) that launch
+    decisions may depend on, or None if the call must take the full path:
+    per array ``(dtype, shape, strides, address & 15)``, per scalar its type
+    (Python ints beyond 64 bits, arrays of other devices and objects of other
+    kinds take the full path).  Computed by the extension module."""
+    return _signature(args, dev_id, _tuning.version())
+
+
+_signature = _rt.hot.signature
 
 
 def ranges_overlap(a, b):
     """True if the memory spans of two arrays intersect."""
-    from cupy_amd._core._carray import may_share_bounds
-    return may_share_bounds(a, b)
+    return _carray.may_share_bounds(a, b)
 
 
 class FastCall:
@@ -174,9 +162,11 @@ class FastCall:
         from cupy_amd._core.core import ndarray
         for i, o in self.overlap:
             a, b = args[i], args[o]
-            if a is not b and ranges_overlap(a, b):
+            # (arrays of different allocations cannot overlap)
+            if (a is not b and a.data.mem.ptr == b.data.mem.ptr
+                    and _carray.may_share_bounds(a, b)):
                 return NotImplemented
-        if _memory.static_scratch_active():
+        if _memory._static_scratch_open and _memory.static_scratch_active():
             return self._run_static(args, stream_ptr)
         refs = list(args)
         for shape, dtype in self.out_specs:
@@ -188,18 +178,11 @@ class FastCall:
             stream_ptr = _stream.get_current_stream_ptr()
         quick = self.quick
         if quick is not None and use_quick:
-            # pointer-only argument blocks: the recorded bytes with the
-            # addresses spliced in, handed to the library as they are
-            launch = _rt.lib.rt_launch_packed
-            for fptr, dims, shmem, packer, pieces, slots, size, fn in quick:
-                pieces = pieces[:]            # (other threads replay the same record)
-                k = 1
-                for ref in slots:
-                    pieces[k] = refs[ref].data.ptr if ref < n_arr else refs[ref].ptr
-                    k += 2
-                status = launch(fptr, *dims, shmem, stream_ptr, packer.pack(*pieces), size)
-                if status != 0:
-                    _rt.check(status)
+            # pointer-only argument blocks: the extension splices the
+            # addresses into the recorded bytes and launches
+            status = _replay(quick[0], refs, n_arr, stream_ptr)
+            if status != 0:
+                _rt.check(status)
         else:
             for fn, grid, block, packer, template, ptrs, scalars, shmem in self.launches:
                 vals = template[:]
@@ -220,16 +203,14 @@ class FastCall:
 
 
 def _quick_launches(launches):
-    """Per recorded launch whose argument block changes only in its pointers:
-    everything ``rt_launch_packed`` takes, with the block cut at the pointer
-    slots -- ``(function handle, grid and block, shared memory, packer of
-    [bytes, pointer, bytes, ...], that list with the bytes filled in, ref per
-    pointer, block size, Function)``.  None if any launch takes a scalar that
-    changes from call to call, or when launches are only recorded."""
-    from cupy_amd import _dryrun
-    if _dryrun.enabled():
-        return None
-    out = []
+    """The launches of a recorded call whose argument blocks change only in
+    their pointers, as the record ``_rt.hot.replay`` takes: per launch the
+    function handle, grid and block, shared memory, the byte offsets of the
+    pointer slots with the ref each receives, and the argument block as
+    recorded.  Returns ``(record, Functions kept alive)``, or None if any
+    launch takes a scalar that changes from call to call."""
+    out = [struct.pack('<II', len(launches), 0)]
+    recorded_only = _dryrun.enabled()
     for fn, grid, block, packer, template, ptrs, scalars, shmem in launches:
         if scalars or not ptrs:
             return None
@@ -253,18 +234,29 @@ def _quick_launches(launches):
                 return None
             found.append((off, ref))
         found.sort()
-        pieces, fmt, pos = [], ['<'], 0
-        for off, ref in found:
-            pieces.append(blob[pos:off])
-            fmt.append('%ds' % (off - pos))
-            pieces.append(0)
-            fmt.append('Q')
-            pos = off + 8
-        pieces.append(blob[pos:])
-        fmt.append('%ds' % (len(blob) - pos))
-        out.append((fn.ptr, (gx, gy, gz, bx, by, bz), shmem, struct.Struct(''.join(fmt)),
-                    pieces, tuple(ref for _, ref in found), len(blob), fn))
-    return tuple(out)
+        handle = fn.ptr
+        if recorded_only:
+            # no function handles exist: a stand-in that names the kernel
+            handle = id(fn)
+            _function_names[handle] = fn.name
+        out.append(struct.pack('<Q3I3IIIQ', handle, gx, gy, gz, bx, by, bz, shmem,
+                               len(found), len(blob)))
+        out.append(b''.join(struct.pack('<II', off, ref) for off, ref in found))
+        out.append(blob + b'\0' * (-len(blob) % 8))
+    return b''.join(out), tuple(launch[0] for launch in launches)
+
+
+def _replay_recorded_only(record, refs, n_arr, stream_ptr):
+    """Stand-in for ``_rt.hot.replay`` where launches are only recorded: the
+    extension patches the argument blocks as it would for a launch and hands
+    them back."""
+    for handle, grid, block, shmem, blob in _rt.hot.splice(record, refs, n_arr):
+        _dryrun.record_launch(_function_names[handle], grid, block, shmem, blob)
+    return 0
+
+
+_function_names = {}
+_replay = _replay_recorded_only if _dryrun.enabled() else _rt.hot.replay
 
 
 def _run_static(self, args, stream_ptr):

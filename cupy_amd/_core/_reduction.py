@@ -590,13 +590,14 @@ class _AbstractReductionKernel:
             group = max(1, min(64, internal.clp2(lanes_needed)))
         n_split = 1
         chunk = n_red
+        wg = _tuning.get('rows_block') if group == _cg.BLOCK else _cg.BLOCK
         # (a second launch costs about 8 us: below 128 KiB per row a workgroup
         # on its own is quicker)
         if (group == _cg.BLOCK and n_out < cus * _tuning.get('min_blocks_per_cu')
                 and (n_red * max_item >= 128 * 1024 or stage)):
-            trip = _cg.BLOCK * vec
+            trip = wg * vec
             want = (cus * _tuning.get('target_blocks_per_cu') + n_out - 1) // n_out
-            most = max(1, n_red // (trip * 4))
+            most = max(1, n_red // (trip * _tuning.get('rows_split_min_trips')))
             n_split = max(1, min(want, most, 65535))
             if n_split > 1:
                 chunk = (n_red + n_split - 1) // n_split
@@ -631,7 +632,7 @@ class _AbstractReductionKernel:
         rargs = self._rargs(in_args, out_args, bcast_r=bcast_r, bcast_o=bcast_o)
         key = ('rows', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, group, vec, idx64, partial, device_id,
-               batched, trips, exact, stream_hint, _tuning.signature())
+               batched, trips, exact, stream_hint, wg, _tuning.signature())
 
         def emit():
             if batched:
@@ -645,12 +646,12 @@ class _AbstractReductionKernel:
                 post_map_expr, reduce_type, typedefs, preamble, group=group,
                 vec=vec, idx64=idx64, partial_out=partial,
                 stream_hint=stream_hint,
-                unroll=_tuning.get('rows_unroll'))
+                unroll=_tuning.get('rows_unroll'), block=wg)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
         if group == _cg.BLOCK:
-            gx = min(n_out, _max_blocks(_cg.BLOCK))
+            gx = min(n_out, _max_blocks(wg))
             cap = _tuning.get('rows_block_grid_per_cu')
             if cap and n_split == 1:
                 gx = min(gx, cus * cap)
@@ -664,7 +665,7 @@ class _AbstractReductionKernel:
             vals.ptr(pref, partials.ptr)
             vals.const(chunk)
             _launch_plan.launch(
-                rec, fn, (gx, n_split, 1), (_cg.BLOCK, 1, 1),
+                rec, fn, (gx, n_split, 1), (wg, 1, 1),
                 _make_packer(self._fast_format(rargs, ic, 'P' + ic)), vals, stream_ptr)
             if stage:
                 n_split, n_final = n_split * stage[0], stage[1]
@@ -676,7 +677,7 @@ class _AbstractReductionKernel:
                 stream_ptr, rec, pref, n_out * n_red)
         else:
             _launch_plan.launch(
-                rec, fn, (gx, 1, 1), (_cg.BLOCK, 1, 1),
+                rec, fn, (gx, 1, 1), (wg, 1, 1),
                 _make_packer(self._fast_format(rargs, ic)), vals, stream_ptr)
 
     @staticmethod

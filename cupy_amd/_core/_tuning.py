@@ -50,6 +50,8 @@ _params = {
     'rows_stream': True,       # non-temporal loads: True / False / 'auto' (by footprint);
                                # measured better or equal from 16 MiB inputs upwards
     'rows_unroll': 4,
+    'rows_block': 256,          # threads of a workgroup that owns a row
+    'rows_split_min_trips': 4,  # a split row leaves every workgroup at least this many trips
     'rows_block_grid_per_cu': 0,   # workgroups per CU when a workgroup owns a row (0: one per row)
     'rows_block_mode_bytes': 32768,   # row length from which a workgroup owns a row
     'rows_batch': 2,            # short rows handled per lane group at a time

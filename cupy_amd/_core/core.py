@@ -11,6 +11,7 @@ import operator
 import numpy
 
 from cupy_amd import _dryrun
+from cupy_amd import _rt
 from cupy_amd._core import _dtype
 from cupy_amd._core import internal
 from cupy_amd.cuda import device as _device
@@ -1023,3 +1024,7 @@ def asnumpy(a, stream=None, order='C', out=None, blocking=True):
     if hasattr(a, '__cuda_array_interface__'):
         return _from_cuda_array_interface(a).get(stream=stream, out=out)
     return numpy.asarray(a, order=order)
+
+
+# the extension module recognises this package's arrays and NumPy's scalars by type
+_rt.hot.setup(ndarray, numpy.generic)

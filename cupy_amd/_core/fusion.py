@@ -73,12 +73,14 @@ class Recording:
         proxies = [rec.argument(i, a) for i, a in enumerate(args)]
         saved = (getattr(_thread_local, 'history', None),
                  getattr(_thread_local, 'is_old_fusing', False))
+        _fusion_thread_local.begin_recording()
         _thread_local.history = rec
         _thread_local.is_old_fusing = True
         try:
             ret = func(*proxies)
         finally:
             _thread_local.history, _thread_local.is_old_fusing = saved
+            _fusion_thread_local.end_recording()
         self.recorder = rec
         self.single = not isinstance(ret, tuple)
         # every returned item: ('value', Value) | ('arg', position) | ('const', object)

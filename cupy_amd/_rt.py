@@ -163,7 +163,7 @@ def _load():
         raise ImportError(
             'cupy_amd: the native runtime shim %s is missing. Build it with '
             '`python -c "import __graft_entry__ as g; g.build()"` from the '
-            'repository root (or `python -m cupy_amd.csrc.build`). There is '
+            'repository root (or `python cupy_amd/csrc/build.py`). There is '
             'no fallback path without it.' % LIB_PATH)
     try:
         handle = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
@@ -179,6 +179,30 @@ def _load():
 
 
 lib = _load()
+
+HOTPATH_PATH = os.path.join(_HERE, '_lib', '_hotpath.so')
+
+
+def _load_hotpath():
+    """The extension module with the per-launch calls (``launch``, ``replay``,
+    ``pool_malloc``, ``pool_free``): callers of ``rt_launch_packed``,
+    ``rt_pool_malloc`` and ``rt_pool_free`` that skip ctypes' conversion of
+    every argument.  Mandatory like the library it links against."""
+    import importlib.machinery
+    import importlib.util
+    if not os.path.exists(HOTPATH_PATH):
+        raise ImportError(
+            'cupy_amd: the extension module %s is missing. Build it with '
+            '`python -c "import __graft_entry__ as g; g.build()"` from the '
+            'repository root (or `python cupy_amd/csrc/build.py`).' % HOTPATH_PATH)
+    loader = importlib.machinery.ExtensionFileLoader('_hotpath', HOTPATH_PATH)
+    spec = importlib.util.spec_from_loader('_hotpath', loader)
+    module = importlib.util.module_from_spec(spec)
+    loader.exec_module(module)
+    return module
+
+
+hot = _load_hotpath()
 
 
 def check(status):

@@ -1,17 +1,21 @@
-"""Builds ``_lib/libmi355rt.so`` (the C-ABI runtime shim) with hipcc.
+"""Builds ``_lib/libmi355rt.so`` (the C-ABI runtime shim) with hipcc and
+``_lib/_hotpath.so`` (CPython extension: the per-launch calls into that
+library without ctypes' argument conversion) with gcc.
 
-Usage: ``python -m cupy_amd.csrc.build``.  Nothing is imported from the package
-itself, so this also works before the library exists.
+Usage: ``python cupy_amd/csrc/build.py`` (run as a script, so that nothing of
+the package is imported: importing the package needs what this builds).
 """
 import os
 import subprocess
 import sys
+import sysconfig
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 ROOT = os.path.dirname(PKG)
 SOURCES = ['mi355rt.cpp', 'pool.cpp']
 OUTPUT = os.path.join(PKG, '_lib', 'libmi355rt.so')
+HOTPATH_OUTPUT = os.path.join(PKG, '_lib', '_hotpath.so')
 
 
 def build_shim(verbose=False):
@@ -27,7 +31,23 @@ def build_shim(verbose=False):
         print(' '.join(cmd))
     subprocess.check_call(cmd)
     os.replace(OUTPUT + '.tmp', OUTPUT)
+    build_hotpath(verbose)
     return OUTPUT
+
+
+def build_hotpath(verbose=False):
+    """The extension module links against the shim beside it (found through
+    ``$ORIGIN``) and is built for the interpreter that runs this script."""
+    cc = os.environ.get('CC', 'gcc')
+    cmd = [cc, '-shared', '-fPIC', '-O2', '-std=c11', '-Wall', '-Wextra',
+           '-I' + os.path.join(ROOT, 'include'), '-I' + sysconfig.get_paths()['include'],
+           os.path.join(HERE, 'hotpath.c'), '-o', HOTPATH_OUTPUT + '.tmp',
+           '-L' + os.path.dirname(OUTPUT), '-lmi355rt', '-Wl,-rpath,$ORIGIN']
+    if verbose:
+        print(' '.join(cmd))
+    subprocess.check_call(cmd)
+    os.replace(HOTPATH_OUTPUT + '.tmp', HOTPATH_OUTPUT)
+    return HOTPATH_OUTPUT
 
 
 if __name__ == '__main__':

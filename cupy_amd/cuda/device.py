@@ -24,9 +24,13 @@ def get_device_id():
     """Index of the calling thread's current device."""
     if _dryrun.enabled():
         return 0
-    dev = ctypes.c_int(0)
-    _rt.check(_rt.lib.rt_get_device(ctypes.byref(dev)))
-    return dev.value
+    dev = _hot_get_device()
+    if dev < 0:
+        _rt.check(-dev)
+    return dev
+
+
+_hot_get_device = _rt.hot.get_device
 
 
 def get_device_count():

@@ -177,9 +177,8 @@ class Function:
         if _dryrun.enabled():
             _dryrun.record_launch(self.name, grid, block, shared_mem, bytes(arg_block))
             return
-        status = _rt.lib.rt_launch_packed(
-            self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr,
-            arg_block, len(arg_block))
+        status = _rt.hot.launch(
+            self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr, arg_block)
         if status != 0:
             _rt.check(status)
 

@@ -270,22 +270,25 @@ class _NativePool:
     the Python pool and every block it handed out, so the native bookkeeping
     lives until the last block has come back."""
 
-    __slots__ = ('handle', 'callbacks', 'live')
+    __slots__ = ('handle', 'value', 'callbacks', 'live')
 
     def __init__(self, alloc_cb, free_cb, live):
         self.live = live
         self.callbacks = (_rt.POOL_ALLOC_FN(alloc_cb), _rt.POOL_FREE_FN(free_cb))
         self.handle = ctypes.c_void_p()
+        self.value = 0
         _rt.check(_rt.lib.rt_pool_create_with_allocator(
             ctypes.byref(self.handle), self.callbacks[0], self.callbacks[1], None))
+        self.value = self.handle.value or 0      # the handle as the integer the extension takes
 
     def _free(self, ptr, size):
-        handle = self.handle
-        if handle:
-            _rt.lib.rt_pool_free(handle, ptr)
+        value = self.value
+        if value:
+            _rt.hot.pool_free(value, ptr)
 
     def __del__(self):
         handle, self.handle = getattr(self, 'handle', None), None
+        self.value = 0
         if handle:
             try:
                 _rt.lib.rt_pool_destroy(handle)
@@ -339,6 +342,7 @@ class SingleDeviceMemoryPool:
 
         self._native = _NativePool(alloc_cb, free_cb, live)
         self._handle = self._native.handle
+        self._handle_value = self._native.value
         limit = _parse_limit_string()
         if limit['size'] is not None or limit['fraction'] is not None:
             self.set_limit(**limit)
@@ -369,19 +373,20 @@ class SingleDeviceMemoryPool:
             return MemoryPointer(Memory(0), 0)
         rounded = _round_size(size)
         stream_ident = _stream.get_current_stream_ptr()
-        addr = ctypes.c_uint64(0)
-        lib = _rt.lib
-        status = lib.rt_pool_malloc(self._handle, rounded, stream_ident, ctypes.byref(addr))
-        if status == _rt.RT_ERR_POOL_OOM:
-            # Last resort before giving up: collect garbage cycles that may be
-            # keeping arrays (and so pool blocks) alive.
-            gc.collect()
-            status = lib.rt_pool_malloc(
-                self._handle, rounded, stream_ident, ctypes.byref(addr))
-            if status == _rt.RT_ERR_POOL_OOM:
-                raise OutOfMemoryError(rounded, self.total_bytes(), self.get_limit())
-        _rt.check(status)
-        mem = PooledMemory(addr.value, rounded, self._device_id, self)
+        handle = self._handle_value
+        pool_malloc = _rt.hot.pool_malloc
+        addr = pool_malloc(handle, rounded, stream_ident)
+        if addr < 0:
+            if -addr == _rt.RT_ERR_POOL_OOM:
+                # Last resort before giving up: collect garbage cycles that may
+                # be keeping arrays (and so pool blocks) alive.
+                gc.collect()
+                addr = pool_malloc(handle, rounded, stream_ident)
+                if -addr == _rt.RT_ERR_POOL_OOM:
+                    raise OutOfMemoryError(rounded, self.total_bytes(), self.get_limit())
+            if addr < 0:
+                _rt.check(-addr)
+        mem = PooledMemory(addr, rounded, self._device_id, self)
         return MemoryPointer(mem, 0)
 
     def _free(self, ptr, size):
@@ -460,7 +465,12 @@ class MemoryPool:
         return pool
 
     def malloc(self, size):
-        return self._pool().malloc(size)
+        pool = self._pools.get(_device.get_device_id())
+        if pool is None:
+            pool = self._pool()
+        if _memory_hook._n_registered > 0:
+            return pool.malloc(size)
+        return pool._malloc(size)
 
     def free_all_blocks(self, stream=None):
         self._pool().free_all_blocks(stream)
@@ -492,11 +502,20 @@ _current_allocator = _malloc
 _thread_local = threading.local()
 
 
+# number of ``static_scratch`` contexts open in any thread: the per-call checks
+# look at the thread's own flag only while this is non-zero
+_static_scratch_open = 0
+_static_scratch_lock = threading.Lock()
+_allocator_overrides = 0        # ``using_allocator`` contexts open in any thread
+
+
 def alloc(size):
     """Allocates through the current allocator (thread-local override first)."""
-    if getattr(_thread_local, 'static_scratch', False):
+    if _static_scratch_open and getattr(_thread_local, 'static_scratch', False):
         refuse_allocation('a request for %d bytes' % size)
-    return get_allocator()(size)
+    if _allocator_overrides:
+        return get_allocator()(size)
+    return _current_allocator(size)
 
 
 class static_scratch:
@@ -514,16 +533,22 @@ class static_scratch:
     time on one GPU (other streams, other threads) race on it."""
 
     def __enter__(self):
+        global _static_scratch_open
         self._prev = getattr(_thread_local, 'static_scratch', False)
+        with _static_scratch_lock:
+            _static_scratch_open += 1
         _thread_local.static_scratch = True
         return self
 
     def __exit__(self, *exc):
+        global _static_scratch_open
         _thread_local.static_scratch = self._prev
+        with _static_scratch_lock:
+            _static_scratch_open -= 1
 
 
 def static_scratch_active():
-    return getattr(_thread_local, 'static_scratch', False)
+    return bool(_static_scratch_open) and getattr(_thread_local, 'static_scratch', False)
 
 
 def refuse_allocation(what):
@@ -551,9 +576,14 @@ def using_allocator(allocator=None):
     """Thread-local, nestable allocator override."""
     if allocator is None:
         allocator = _malloc
+    global _allocator_overrides
     previous = getattr(_thread_local, 'allocator', None)
+    with _static_scratch_lock:
+        _allocator_overrides += 1
     _thread_local.allocator = allocator
     try:
         yield
     finally:
         _thread_local.allocator = previous
+        with _static_scratch_lock:
+            _allocator_overrides -= 1
