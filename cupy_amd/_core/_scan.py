@@ -21,6 +21,7 @@ along the scanned axis: pass 1 reduces every chunk to its total, the totals
 are scanned by the same code, pass 3 scans the chunks seeded with the total of
 everything before them.  Nothing spins on another workgroup's progress.
 """
+import ctypes
 import struct
 import threading
 
@@ -594,6 +595,351 @@ TILE_KERNEL(cupy_scan_tile_seeded, 2)
            reuse=1 if reuse else 0)
 
 
+_CHAIN_WAVES = _BLOCK // _WAVE
+_CHAIN_HEADER_WORDS = 64            # the ticket counter, padded to 256 bytes
+
+
+def _emit_chain(in_t, out_t, op, skip_nan, vec, trips, idx64, stream, ragged, parts=2):
+    """One-pass scan of long rows: a workgroup per tile of 256 x VEC x TRIPS
+    elements scans its tile in registers, publishes the tile's total and adds
+    up the totals published by the tiles before it: the input is read once and
+    the result written once.
+
+    A tile waits only for tiles with smaller numbers (``blockIdx.x``), and
+    workgroups start in the order of their numbers on every compute die, so
+    the unfinished tile with the smallest number is always running and waits
+    for nobody.  Every wait is bounded by ``spin_limit`` polls all the same:
+    a tile that runs out of patience flags the failure in ``fault`` and still
+    runs to its end, so the grid always drains.
+
+    The totals before a tile are combined in an order that depends only on the
+    tile's number: tiles form groups of ``group_tiles``; the last tile of a
+    group publishes the group's total; a tile adds the totals of the groups
+    before its own and the totals of the tiles before it in its group, each
+    set folded lane by lane and then across the lanes.  Results therefore do
+    not vary from run to run (a look-back that stops at whatever prefix happens
+    to be published would make floating-point results depend on timing)."""
+    acc_t = _acc_type(out_t)
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    return '''#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define RAGGED %(ragged)d
+#define WAVE 64
+#define WAVES %(waves)d
+#define PARTS %(parts)d
+#define SPIN_SLEEP %(sleep)d      // pause between two polls, in units of 64 clocks
+#define PART_ELEMS (WAVE * VEC * TRIPS)
+#define WAVE_ELEMS (PARTS * PART_ELEMS)
+#define TILE (WAVES * WAVE_ELEMS)
+#define HEADER_WORDS %(header)d
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+
+// A published value travels as 32-bit words, each in the low half of a 64-bit
+// slot whose high half holds the number of this launch (`epoch`, never zero):
+// one atomic store publishes a word together with its mark and one atomic load
+// fetches both, so that no fence (and no write-back of a die's cache) is
+// needed on either side, and nothing has to be cleared between launches: what
+// an earlier launch left in a slot carries an older number.  The accesses have
+// device scope: they pass the caches of the compute dies.
+constexpr int kWords = (sizeof(_acc_t) + 3) / 4;
+typedef unsigned long long _slot_t;
+
+__device__ __forceinline__ void _publish(_slot_t* slots, const ptrdiff_t i, const _acc_t& v,
+                                         const unsigned epoch) {
+  unsigned w[kWords];
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) w[k] = 0u;
+  __builtin_memcpy(w, &v, sizeof(_acc_t));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k)
+    __hip_atomic_store(slots + i * kWords + k, ((_slot_t)epoch << 32) | w[k], __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// `count` published values from `first`, waited for and combined in an order
+// that depends on `count` alone: every lane takes the values lane, lane + 64,
+// ... as they appear, then the lanes are combined (every lane ends with the
+// same value).  One wave, all lanes call.  `ok` turns false if the wave gave
+// up after `spin_limit` rounds of polling (the value is then meaningless).
+__device__ __forceinline__ _acc_t _await_fold(_slot_t* slots, const ptrdiff_t first,
+                                              const int count, const int lane,
+                                              const unsigned epoch, const unsigned spin_limit,
+                                              bool& ok) {
+  _acc_t s = SCAN_IDENTITY;
+  int i = lane;
+  unsigned spins = 0;
+  // Tiles publish roughly in the order of their numbers: wait for the newest
+  // value alone first (one address for the whole wave, so that thousands of
+  // waiting workgroups do not hammer the few memory channels that hold the
+  // slots), then collect all of them.
+  for (;;) {
+    const _slot_t x = __hip_atomic_load(slots + (first + count) * kWords - 1, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    if ((unsigned)(x >> 32) == epoch) break;
+    if (spins >= spin_limit) { ok = false; break; }
+    ++spins;
+    __builtin_amdgcn_s_sleep(SPIN_SLEEP);
+  }
+  for (;;) {
+    while (i < count) {
+      _slot_t x[kWords];
+#pragma unroll
+      for (int k = 0; k < kWords; ++k)
+        x[k] = __hip_atomic_load(slots + (first + i) * kWords + k, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      bool written = true;
+      unsigned w[kWords];
+#pragma unroll
+      for (int k = 0; k < kWords; ++k) {
+        written = written && (unsigned)(x[k] >> 32) == epoch;
+        w[k] = (unsigned)x[k];
+      }
+      if (!written) break;
+      _acc_t v;
+      __builtin_memcpy(&v, w, sizeof(_acc_t));
+      s = SCAN_OP(s, v);
+      i += WAVE;
+    }
+    if (__ballot(i < count) == 0) break;
+    if (spins >= spin_limit) { ok = false; break; }
+    ++spins;
+    __builtin_amdgcn_s_sleep(SPIN_SLEEP);
+  }
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) s = SCAN_OP(s, cupy::shfl_xor(s, m));
+  return s;
+}
+
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_clear(
+    unsigned* desc, const unsigned words) {
+  for (unsigned i = blockIdx.x * %(block)d + threadIdx.x; i < words; i += gridDim.x * %(block)d)
+    desc[i] = 0u;
+}
+
+// The TRIPS vectors of a lane for the part of tile `t_row` of a row that wave
+// `wv` scans, all requested at once (a vector that would start past the end of
+// the row is read from the row's start instead; its values are not used).
+__device__ __forceinline__ void _tile_load(
+    cupy::Vec<_in_t, VEC> (&raw)[TRIPS], const _in_t* __restrict__ src, const _idx_t j0,
+    const _idx_t j1, const int lane) {
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    const _idx_t j = j0 + (t * WAVE + lane) * VEC;
+    const _idx_t jc = (j + VEC <= j1) ? j : 0;
+    if (VEC > 1) raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + jc);
+    else raw[t].v[0] = src[(j < j1) ? j : 0];
+  }
+}
+
+// One part of a wave's share of the tile (TRIPS vectors per lane, from `j0`):
+// the values of every lane scanned in place (`v`), what precedes each of the
+// lane's vectors inside the part (`pre`), and -- returned -- the part's total.
+__device__ __forceinline__ _acc_t _part_scan(
+    const cupy::Vec<_in_t, VEC> (&raw)[TRIPS], const _in_t* __restrict__ src, const _idx_t j0,
+    const _idx_t j1, const int lane, _acc_t (&v)[TRIPS][VEC], _acc_t (&pre)[TRIPS]) {
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    const _idx_t j = j0 + (t * WAVE + lane) * VEC;
+    if (RAGGED && VEC > 1 && j + VEC > j1) {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        v[t][k] = (j + k < j1) ? _load_value(src[j + k]) : SCAN_IDENTITY;
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        v[t][k] = ((RAGGED ? j + k : j) < j1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+    }
+#pragma unroll
+    for (int k = 1; k < VEC; ++k) v[t][k] = SCAN_OP(v[t][k - 1], v[t][k]);
+  }
+  // inclusive scans of the lane totals across the wave, the trips side by side
+  _acc_t incl[TRIPS];
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) incl[t] = v[t][VEC - 1];
+#pragma unroll
+  for (int d = 1; d < WAVE; d <<= 1) {
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const _acc_t o = cupy::shfl_up<WAVE>(incl[t], d);
+      incl[t] = (lane >= d) ? SCAN_OP(o, incl[t]) : incl[t];
+    }
+  }
+  _acc_t carry = SCAN_IDENTITY;
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    const _acc_t trip_total = cupy::shfl_idx<WAVE>(incl[t], WAVE - 1);
+    const _acc_t before = cupy::shfl_up<WAVE>(incl[t], 1);
+    pre[t] = (lane == 0) ? carry : SCAN_OP(carry, before);
+    carry = (t == 0) ? trip_total : SCAN_OP(carry, trip_total);
+  }
+  return carry;
+}
+
+// The results of one part: `base` (if `has_base`) before everything.
+__device__ __forceinline__ void _part_store(
+    _out_t* __restrict__ row_out, const _idx_t j0, const _idx_t j1, const int lane,
+    const _acc_t (&v)[TRIPS][VEC], const _acc_t (&pre)[TRIPS], const _acc_t base,
+    const bool has_base) {
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    const _idx_t j = j0 + (t * WAVE + lane) * VEC;
+    const bool has_pre = (t > 0) || (lane > 0);
+    const _acc_t before = has_base ? (has_pre ? SCAN_OP(base, pre[t]) : base) : pre[t];
+    const bool any = has_base || has_pre;
+    _out_t* dst = row_out + j;
+    if (VEC > 1 && (RAGGED ? j + VEC <= j1 : j < j1)) {
+      cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        r.v[k] = static_cast<_out_t>(any ? SCAN_OP(before, v[t][k]) : v[t][k]);
+      cupy::store_vec<_out_t, VEC, NT_STORE>(dst, r);
+    } else if (RAGGED || VEC == 1) {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        if (j + k < j1) dst[k] = static_cast<_out_t>(any ? SCAN_OP(before, v[t][k]) : v[t][k]);
+    }
+  }
+}
+
+// desc: [HEADER_WORDS unused 32-bit words][slots of the tile totals][slots of
+//       the group totals]; zero before its first use, then only ever written
+//       by launches of this kernel, each with a number of its own.
+// One workgroup per tile, tiles numbered by blockIdx.x: a tile waits only for
+// tiles with smaller numbers.  Workgroups are handed to each compute die in the
+// order of their numbers, so the unfinished tile with the smallest number is
+// always running and owes nothing to anyone: every wait ends.  (Should that
+// order ever not hold, the waits are bounded: see `spin_limit`.)
+//
+// A wave's share of the tile comes in PARTS parts of TRIPS vectors per lane,
+// all requested at the start.  While the workgroup waits for its neighbours it
+// has nothing in flight, so what it holds in registers meanwhile is what
+// keeps the memory system busy: the first part is held scanned, the others as
+// loaded (they are scanned twice: once for their total, once for the result).
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, unsigned* desc,
+    const _idx_t n_rows, const _idx_t n, const _idx_t tiles_per_row, const _idx_t group_tiles,
+    const _idx_t groups_per_row, const unsigned epoch, const unsigned spin_limit,
+    unsigned* fault) {
+  __shared__ __attribute__((aligned(16))) char sm_raw[(WAVES + 2) * sizeof(_acc_t)];
+  _acc_t* sm_wave = reinterpret_cast<_acc_t*>(sm_raw);
+  const ptrdiff_t n_tiles = (ptrdiff_t)n_rows * tiles_per_row;
+  _slot_t* tile_totals = reinterpret_cast<_slot_t*>(desc + HEADER_WORDS);
+  _slot_t* group_totals = tile_totals + n_tiles * kWords;
+  const int lane = threadIdx.x %% WAVE;
+  const int wv = threadIdx.x / WAVE;
+  const _idx_t j1 = n;
+  const ptrdiff_t tile = blockIdx.x;
+  if (tile >= n_tiles) return;
+  const _idx_t row = (_idx_t)(tile / tiles_per_row);
+  const _idx_t t_row = (_idx_t)(tile - (ptrdiff_t)row * tiles_per_row);
+  const _in_t* src = in + (ptrdiff_t)row * n;
+  _out_t* row_out = out + (ptrdiff_t)row * n;
+  const _idx_t j0 = t_row * TILE + wv * WAVE_ELEMS;        // this wave's share of the tile
+  cupy::Vec<_in_t, VEC> raw[PARTS][TRIPS];
+#pragma unroll
+  for (int p = 0; p < PARTS; ++p) _tile_load(raw[p], src, j0 + p * PART_ELEMS, j1, lane);
+  _acc_t v[TRIPS][VEC];
+  _acc_t pre[TRIPS];
+  _acc_t part_total[PARTS];
+  part_total[0] = _part_scan(raw[0], src, j0, j1, lane, v, pre);
+  _acc_t carry = part_total[0];
+#pragma unroll
+  for (int p = 1; p < PARTS; ++p) {
+    _acc_t v2[TRIPS][VEC];
+    _acc_t pre2[TRIPS];
+    part_total[p] = _part_scan(raw[p], src, j0 + p * PART_ELEMS, j1, lane, v2, pre2);
+    carry = SCAN_OP(carry, part_total[p]);
+  }
+  if (lane == 0) sm_wave[wv] = carry;
+  __syncthreads();
+  _acc_t wave_before = SCAN_IDENTITY;
+  _acc_t tile_total = sm_wave[0];
+#pragma unroll
+  for (int w = 1; w < WAVES; ++w) {
+    if (w == wv) wave_before = tile_total;
+    tile_total = SCAN_OP(tile_total, sm_wave[w]);
+  }
+  // ---- what precedes the tile in its row: the first wave collects the totals
+  // of the tiles before it in its group, the second those of the groups before
+  // its own
+  const _idx_t g = t_row / group_tiles;
+  const int t_group = (int)(t_row - g * group_tiles);
+  const bool closes_group = (t_group == group_tiles - 1) || (t_row == tiles_per_row - 1);
+  const ptrdiff_t row_groups = (ptrdiff_t)row * groups_per_row;
+  if (wv == 0) {
+    if (lane == 0) _publish(tile_totals, tile, tile_total, epoch);
+    bool ok = true;
+    _acc_t in_group = SCAN_IDENTITY;
+    if (t_group > 0)
+      in_group = _await_fold(tile_totals, tile - t_group, t_group, lane, epoch, spin_limit, ok);
+    if (lane == 0) {
+      if (closes_group)
+        _publish(group_totals, row_groups + g,
+                 (t_group > 0) ? SCAN_OP(in_group, tile_total) : tile_total, epoch);
+      sm_wave[WAVES] = in_group;
+      if (!ok && fault) *reinterpret_cast<volatile unsigned*>(fault) = 1u;
+    }
+  } else if (wv == 1 && g > 0) {
+    bool ok = true;
+    const _acc_t groups_before =
+        _await_fold(group_totals, row_groups, (int)g, lane, epoch, spin_limit, ok);
+    if (lane == 0) {
+      sm_wave[WAVES + 1] = groups_before;
+      if (!ok && fault) *reinterpret_cast<volatile unsigned*>(fault) = 1u;
+    }
+  }
+  __syncthreads();
+  const bool seeded = t_row > 0;
+  _acc_t base = (g > 0) ? ((t_group > 0) ? SCAN_OP(sm_wave[WAVES + 1], sm_wave[WAVES])
+                                         : sm_wave[WAVES + 1])
+                        : sm_wave[WAVES];
+  if (wv > 0) base = seeded ? SCAN_OP(base, wave_before) : wave_before;
+  bool has_base = seeded || wv > 0;
+  // ---- results
+  _part_store(row_out, j0, j1, lane, v, pre, base, has_base);
+#pragma unroll
+  for (int p = 1; p < PARTS; ++p) {
+    base = has_base ? SCAN_OP(base, part_total[p - 1]) : part_total[p - 1];
+    has_base = true;
+    (void)_part_scan(raw[p], src, j0 + p * PART_ELEMS, j1, lane, v, pre);
+    _part_store(row_out, j0 + p * PART_ELEMS, j1, lane, v, pre, base, has_base);
+  }
+}
+''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident,
+           vec=vec, trips=trips, conv=conv, block=_BLOCK, waves=_CHAIN_WAVES,
+           header=_CHAIN_HEADER_WORDS, parts=parts, sleep=_tuning.get('scan_chain_sleep'),
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
+           ragged=1 if ragged else 0)
+
+
+def _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream, ragged, parts):
+    key = ('chain', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
+           trips, idx64, stream, ragged, parts, _tuning.get('scan_chain_sleep'))
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_chain(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                          vec, trips, idx64, stream, ragged, parts)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
 def _module_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream, reuse):
     key = ('tile', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
            trips, idx64, inner, stream, reuse)
@@ -655,6 +1001,115 @@ def _lanes_geometry(src, dst, inner, item):
     return None
 
 
+_chain_fault = {}        # device id -> address of the word in pinned host memory a tile
+                         # that gave up waiting writes to (0 where none could be allocated)
+_chain_disabled = set()  # devices on which that has happened
+
+
+def _chain_fault_word(dev_id):
+    address = _chain_fault.get(dev_id)
+    if address is None:
+        from cupy_amd import _dryrun
+        address = 0
+        if not _dryrun.enabled():
+            from cupy_amd.cuda import runtime
+            address = runtime.hostAlloc(64, 0)
+            ctypes.memset(address, 0, 64)
+        with _lock:
+            address = _chain_fault.setdefault(dev_id, address)
+    return address
+
+
+_chain_arenas = {}       # (device id, stream) -> [slots array, number of the last launch]
+
+
+def _chain_slots(dev_id, stream_ptr, words, mod):
+    """Memory for the published totals of one launch on ``stream_ptr`` and the
+    launch's number.  A stream keeps its array from call to call (launches on
+    one stream run one after the other, and each marks what it publishes with
+    its own number, so nothing needs clearing in between); the array is
+    cleared when it is created, when it has to grow and when the numbers wrap
+    around."""
+    if stream_ptr is None:
+        stream_ptr = _stream.get_current_stream_ptr()
+    key = (dev_id, stream_ptr)
+    with _lock:
+        arena = _chain_arenas.get(key)
+        if arena is None or arena[0].size < words or arena[1] >= 0xffffffff:
+            if len(_chain_arenas) >= 64:
+                _chain_arenas.clear()
+            size = max(words, 1 << 16)
+            if arena is not None:
+                size = max(size, 2 * arena[0].size)
+            desc = ndarray._new_contiguous((size,), numpy.dtype('uint32'))
+            # (a kernel, not a memset: the caller may be capturing the stream)
+            mod.get_function('cupy_scan_chain_clear').launch_packed(
+                (max(1, min(1024, (size + _BLOCK - 1) // _BLOCK)), 1, 1), (_BLOCK, 1, 1),
+                struct.pack('@PI', desc.data.ptr, size), 0, stream_ptr)
+            arena = _chain_arenas[key] = [desc, 0]
+        arena[1] += 1
+        return arena[0], arena[1]
+
+
+def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_ptr):
+    """The one-pass scan of a few long rows (``_emit_chain``): input read once,
+    output written once.  Returns False where it does not apply (the caller
+    then takes the three-pass route)."""
+    if not _tuning.get('scan_chain'):
+        return False
+    dev_id = _device.get_device_id()
+    if dev_id in _chain_disabled:
+        return False
+    fault = _chain_fault_word(dev_id)
+    if fault and ctypes.c_uint32.from_address(fault).value:
+        # A tile of an earlier scan gave up waiting for the tiles before it and
+        # left wrong results.  Not expected to happen: say so, and stay away
+        # from the kernel from here on.
+        _chain_disabled.add(dev_id)
+        ctypes.c_uint32.from_address(fault).value = 0
+        raise RuntimeError(
+            'an earlier one-pass scan on device %d gave up waiting for its neighbouring '
+            'tiles: its result is wrong.  Scans use the three-pass kernels from now on.'
+            % dev_id)
+    in_dtype, out_dtype = src.dtype, dst.dtype
+    trips = 4
+    parts = _tuning.get('scan_chain_parts')
+    if not parts:
+        # Bigger tiles mean fewer waits per byte but fewer workgroups per CU;
+        # measured on 2^20 .. 2^26 float32: 8 parts (128 KiB of input per tile)
+        # are best from 64 MiB on, 4 from 16 MiB on
+        # (with 8-byte and wider values 8 parts do not fit the registers of a lane)
+        nbytes = n_rows * n * in_dtype.itemsize
+        parts = 8 if nbytes >= 64 << 20 else 4 if nbytes >= 16 << 20 else 2
+        if max(in_dtype.itemsize, _acc_dtype(out_dtype).itemsize) > 4:
+            parts = min(parts, 4)
+    tile = _BLOCK * vec * trips * parts
+    tiles_per_row = (n + tile - 1) // tile
+    n_tiles = n_rows * tiles_per_row
+    if n_tiles < 2 or n_tiles * _BLOCK > 0xffffffff:
+        return False
+    # groups of about sqrt(tiles per row) tiles: a tile then reads about
+    # 2 sqrt(tiles per row) published totals
+    group_tiles = max(32, min(2048, internal.clp2(int(tiles_per_row ** 0.5))))
+    groups_per_row = (tiles_per_row + group_tiles - 1) // group_tiles
+    n_groups = n_rows * groups_per_row
+    # every 32-bit word of a published total sits in a 64-bit slot beside its mark
+    words_per_value = (_acc_dtype(out_dtype).itemsize + 3) // 4
+    desc_words = _CHAIN_HEADER_WORDS + 2 * words_per_value * (n_tiles + n_groups)
+    if desc_words > 0xffffffff:
+        return False
+    mod = _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream,
+                        n % vec != 0, parts)
+    desc, epoch = _chain_slots(dev_id, stream_ptr, desc_words, mod)
+    ic = 'q' if idx64 else 'i'
+    blob = struct.pack('@PPP' + ic * 5 + 'IIP', src.data.ptr, dst.data.ptr, desc.data.ptr,
+                       n_rows, n, tiles_per_row, group_tiles, groups_per_row, epoch,
+                       _tuning.get('scan_chain_spin_limit'), fault)
+    mod.get_function('cupy_scan_chain').launch_packed(
+        (n_tiles, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+    return True
+
+
 def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_chunk=True):
     """Scans the middle axis of C-contiguous (outer, n, inner) ``src`` into
     ``dst`` (same layout; may be the same memory if the dtypes agree)."""
@@ -702,6 +1157,9 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         # up to a dozen rounds)
         if may_chunk and group == _WAVE and outer < want and n > 12 * per_group:
             n_chunks = min((want + outer - 1) // outer, (n + per_group - 1) // per_group)
+        if n_chunks > 1 and _scan_chained(src, dst, outer, n, op, skip_nan, vec, idx64, stream,
+                                          stream_ptr):
+            return
         chunk_len = (n + n_chunks - 1) // n_chunks
         chunk_len = (chunk_len + per_group - 1) // per_group * per_group
         n_chunks = (n + chunk_len - 1) // chunk_len
@@ -779,7 +1237,6 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                            or not _aligned(dst.data.ptr, vec * out_dtype.itemsize)
                            or inner % vec):
             vec //= 2
-        trips = 4
         threads = outer * (inner // vec)
         want = cus * 1024
         n_chunks = 1
@@ -787,6 +1244,13 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
             n_chunks = min((want + threads - 1) // threads, n // 64)
         chunk_len = (n + n_chunks - 1) // n_chunks
         n_chunks = (n + chunk_len - 1) // chunk_len
+        # Rows a thread requests at a time.  Enough threads for one pass: many
+        # (64 x 2^20 float32 along axis 0: 98 us with 4, 96 with 8, 83 with
+        # 16); chunked, every thread has few rows and more only costs
+        # registers (16 x 4096 x 1024 along axis 1: 136 us with 4, 149 with 16).
+        trips = _tuning.get('scan_cols_trips')
+        if not trips:
+            trips = 16 if n_chunks == 1 and n >= 32 else 4
         mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, 64, stream,
                       reuse=n_chunks > 1 and reuse_ok)
         work = threads * n_chunks

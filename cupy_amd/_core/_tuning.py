@@ -77,10 +77,20 @@ _params = {
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
+    'scan_cols_trips': 0,       # rows a thread of the column kernel requests at a time (0: by shape)
+    'scan_chain': True,         # a few long rows: one pass, tiles chained through published totals
+    'scan_chain_parts': 0,      # ... a wave holds this many times 4 vectors per lane of its tile
+                                # (0: by the size of the input)
+    'scan_chain_sleep': 8,      # ... and pauses this many times 64 clocks between two polls
+    'scan_chain_spin_limit': 1 << 18,   # polls after which a tile of that kernel gives up waiting
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
     # fused row-wise functions: words per lane up to which a wave takes a whole row
     'fused_rows': True,         # row-wise fused functions as one kernel (False: one kernel per piece)
-    'fused_rows_wave_words': 64,
+    # (measured with a softmax: rows of 4096 float32 74.7 % of peak with a
+    # workgroup per row against 70.9 % with a wave per row; rows of 2048 73 %
+    # with a wave against 68 % with a workgroup.  Requesting the next row before
+    # the current one is worked on did not help: 62 % against 76 % on rows of 8192)
+    'fused_rows_wave_words': 32,
     # Vector accesses need only the alignment of one element: an access of 16
     # bytes at an address that is a multiple of 4 measures within 4 % of an
     # aligned one (reads of 2^28 bytes: 82 % of peak against 86 %), one at an odd

@@ -1,0 +1,145 @@
+"""The one-pass scan of long rows (tiles chained through published totals)
+against NumPy and against the three-pass kernels on the same seeded inputs."""
+import numpy as np
+import pytest
+
+import cupy_amd as cp
+from cupy_amd._core import _scan, _tuning
+from helpers import assert_exact
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _restore():
+    yield
+    _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0)
+    _scan._chain_disabled.clear()
+
+
+def three_pass(fn):
+    _tuning.set(scan_chain=False)
+    try:
+        return fn()
+    finally:
+        _tuning.set(scan_chain=True)
+
+
+def launched(fn):
+    """Names of the kernels ``fn`` launches."""
+    from cupy_amd.cuda import function
+    names = []
+    orig = function.Function.launch_packed
+
+    def spy(self, *a, **k):
+        names.append(self.name)
+        return orig(self, *a, **k)
+    function.Function.launch_packed = spy
+    try:
+        fn()
+    finally:
+        function.Function.launch_packed = orig
+    return names
+
+
+@pytest.mark.parametrize('n', [(1 << 22) + 12345, 1 << 22, (1 << 20) + 1, 3 * 4096 * 32 + 7])
+def test_integer_scans_are_exact(n):
+    rng = np.random.default_rng(n & 0xffff)
+    h = rng.integers(-5, 6, n).astype(np.int32)
+    d = cp.asarray(h)
+    assert 'cupy_scan_chain' in launched(lambda: d.cumsum())
+    assert_exact(d.cumsum().get(), h.cumsum())
+    out = cp.empty(n, np.int32)
+    cp.cumsum(d, out=out)
+    assert_exact(out.get(), h.cumsum(dtype=np.int32))
+
+
+@pytest.mark.parametrize('dtype,rtol', [('float32', 1e-5), ('float64', 1e-13), ('float16', 2e-3),
+                                        ('complex64', 1e-5), ('complex128', 1e-13)])
+def test_floating_scans(dtype, rtol):
+    rng = np.random.default_rng(17)
+    n = (1 << 21) + 4321
+    h = rng.uniform(0, 1, n)
+    if np.dtype(dtype).kind == 'c':
+        h = h + 1j * rng.uniform(-1, 1, n)
+    if dtype == 'float16':
+        h = h * 1e-3                      # the running sum stays representable
+    h = h.astype(dtype)
+    d = cp.asarray(h)
+    assert 'cupy_scan_chain' in launched(lambda: d.cumsum())
+    got = d.cumsum().get()
+    wide = np.complex128 if np.dtype(dtype).kind == 'c' else np.float64
+    want = np.cumsum(h.astype(wide))
+    scale = np.cumsum(np.abs(h).astype(np.float64))
+    assert (np.abs(got - want) <= rtol * scale + 1e-30).all()
+    # same bits on every run, and close to the three-pass result
+    assert_exact(d.cumsum().get(), got)
+    other = three_pass(lambda: d.cumsum().get())
+    assert (np.abs(got - other) <= 2 * rtol * scale + 1e-30).all()
+
+
+@pytest.mark.parametrize('parts', [1, 2, 3, 8])
+def test_every_tile_size_and_many_launches_on_one_stream(parts):
+    """The slots of the published totals are reused from call to call without
+    being cleared: totals of an earlier call (other data, other tile size) must
+    never be taken for this call's."""
+    _tuning.set(scan_chain_parts=parts)
+    rng = np.random.default_rng(parts)
+    for n in ((1 << 21) + 77, 1 << 20, (1 << 21) + 77, 3 << 19):
+        h = rng.integers(-50, 51, n).astype(np.int32)
+        d = cp.asarray(h)
+        assert_exact(d.cumsum().get(), h.cumsum())
+    stream = cp.cuda.Stream()
+    with stream:
+        h = rng.integers(-50, 51, 1 << 21).astype(np.int64)
+        d = cp.asarray(h)
+        for _ in range(3):
+            got = d.cumsum()
+        stream.synchronize()
+        assert_exact(got.get(), h.cumsum())
+
+
+def test_few_long_rows_products_and_nans():
+    rng = np.random.default_rng(5)
+    h = rng.integers(-5, 6, (3, 300001)).astype(np.int64)
+    d = cp.asarray(h)
+    assert 'cupy_scan_chain' in launched(lambda: d.cumsum(axis=1))
+    assert_exact(d.cumsum(axis=1).get(), h.cumsum(axis=1))
+    # int8 in, int64 out; int8 all the way (wraps as NumPy wraps)
+    h8 = rng.integers(-100, 100, 1 << 21).astype(np.int8)
+    assert_exact(cp.asarray(h8).cumsum().get(), h8.cumsum())
+    assert_exact(cp.cumsum(cp.asarray(h8), dtype=np.int8).get(), h8.cumsum(dtype=np.int8))
+    # products of +-1 and a few 2s
+    hp = np.ones(1 << 21, np.int64)
+    hp[rng.choice(hp.size, 40, replace=False)] = rng.choice([-1, 2], 40)
+    assert_exact(cp.cumprod(cp.asarray(hp)).get(), np.cumprod(hp))
+    # NaNs count as zero
+    hf = rng.uniform(0, 1, (2, 700001)).astype(np.float32)
+    hf[0, ::1000] = np.nan
+    got = cp.nancumsum(cp.asarray(hf), axis=1).get()
+    want = np.nancumsum(hf.astype(np.float64), axis=1)
+    assert (np.abs(got - want) <= 1e-5 * want + 1e-6).all()
+    # a row whose length is no multiple of the vector, rows not aligned to it
+    ho = rng.integers(-5, 6, (5, 99991)).astype(np.int32)
+    assert_exact(cp.asarray(ho).cumsum(axis=1).get(), ho.cumsum(axis=1))
+    hv = rng.integers(-5, 6, (1 << 21) + 3).astype(np.int32)
+    assert_exact(cp.asarray(hv)[1:].cumsum().get(), hv[1:].cumsum())
+
+
+def test_a_tile_that_gives_up_is_reported_and_the_kernel_retired():
+    """With no patience at all (one poll per wait) some tile finds its
+    neighbours unfinished, gives up and says so: every workgroup still runs to
+    its end, the next chained scan raises, and scans go on through the
+    three-pass kernels."""
+    rng = np.random.default_rng(6)
+    h = rng.integers(-5, 6, 1 << 23).astype(np.int32)
+    d = cp.asarray(h)
+    _tuning.set(scan_chain_spin_limit=0)
+    d.cumsum()
+    cp.cuda.Device().synchronize()
+    _tuning.set(scan_chain_spin_limit=1 << 18)
+    with pytest.raises(RuntimeError, match='gave up waiting'):
+        d.cumsum()
+    names = launched(lambda: d.cumsum())
+    assert 'cupy_scan_chain' not in names and 'cupy_scan_rows_seeded' in names
+    assert_exact(d.cumsum().get(), h.cumsum())

@@ -57,7 +57,19 @@ def test_cumsum_floats(shape, dtype, rtol):
         assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
 
 
-def test_large_one_dimensional_scans_use_every_pass():
+@pytest.mark.parametrize('chain', [True, False])
+def test_large_one_dimensional_scans_use_every_pass(chain):
+    """Long rows: through the one-pass kernel and (with it switched off)
+    through the three passes of the chunked kernels."""
+    from cupy_amd._core import _tuning
+    _tuning.set(scan_chain=chain)
+    try:
+        _large_scans()
+    finally:
+        _tuning.set(scan_chain=True)
+
+
+def _large_scans():
     rng = np.random.default_rng(24)
     h = rng.integers(-5, 6, (1 << 23) + 12345).astype(np.int32)
     d = cp.asarray(h)
