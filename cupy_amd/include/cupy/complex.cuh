@@ -192,9 +192,28 @@ __device__ __forceinline__ complex<T> expm1(const complex<T>& z) {
   const T sh = sin(z.im / 2);
   return complex<T>(expm1(z.re) * cos(z.im) - 2 * sh * sh, exp(z.re) * sin(z.im));
 }
+// 2^z = exp(z log 2).  The rounded product z log 2 alone would cost |z| eps
+// (at |z| = 30 some 30 eps): both components keep the rounding error of their
+// product (from an fma) and the part of log 2 beyond its leading digits, and
+// the error term is applied to first order, e^(x + d) = e^x (1 + d),
+// cos(y + d) = cos y - d sin y, sin(y + d) = sin y + d cos y.
 template <typename T>
 __device__ __forceinline__ complex<T> exp2(const complex<T>& z) {
-  return exp(complex<T>(z.re * T(0.69314718055994530942), z.im * T(0.69314718055994530942)));
+  if (z.im == 0) return complex<T>(exp2(z.re), z.im);
+  const T ln2 = T(0.69314718055994530942);
+  const T ln2_rest = sizeof(T) == 4 ? T(-1.904654299957767878541823431924e-9)
+                                    : T(2.319046813846299616e-17);
+  const T x = z.re * ln2;
+  const T dx = fma(z.re, ln2, -x) + z.re * ln2_rest;
+  const T y = z.im * ln2;
+  const T dy = fma(z.im, ln2, -y) + z.im * ln2_rest;
+  T c = cos(y), s = sin(y);
+  if (isfinite(dx) && isfinite(dy)) {
+    const T c1 = c - dy * s, s1 = s + dy * c;
+    c = c1 + c1 * dx;
+    s = s1 + s1 * dx;
+  }
+  return _exp_times(x, c, s);
 }
 template <typename T>
 __device__ __forceinline__ complex<T> rint(const complex<T>& z) {

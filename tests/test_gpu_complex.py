@@ -5,10 +5,13 @@ Multiply, square, divide and reciprocal are within 4 eps * (1 + |result|) in the
 complex plane: NumPy's own result for them depends on the host (its vectorised
 loops fuse one product into the sum where the CPU can, its scalar tails and
 strided loops are left to the C compiler), so there is no single bit pattern to
-match.  Absolute value within 2 ulp; the elementary functions, computed here by
-their textbook formulas and there by the C library's, within
-32 eps * (1 + |result|); sums within the reduction tolerance of the real
-types."""
+match.  Absolute value within 2 ulp.  The elementary functions: within
+4 eps * (1 + |result|) of the g++ build of the same header run on the host
+(observed: at most 2.01), which tests/test_complex_functions_host.py in turn
+holds to 4 eps of extended-precision NumPy; and within 8 eps of NumPy's own
+result in the same precision, whose C library routines are a few eps off
+themselves (observed GPU against double-precision NumPy: at most 2.14).  Sums
+within the reduction tolerance of the real types."""
 import numpy as np
 import pytest
 
@@ -26,7 +29,7 @@ def crandom(shape, dtype, seed, scale=1.0):
     return (z * scale).astype(dtype)
 
 
-def assert_cclose(got, want, eps_factor=32):
+def assert_cclose(got, want, eps_factor=8):
     got, want = np.asarray(got), np.asarray(want)
     assert got.dtype == want.dtype and got.shape == want.shape, (got.dtype, want.dtype)
     eps = np.finfo(want.real.dtype).eps
@@ -317,10 +320,11 @@ def test_extrema_order_by_real_then_imaginary_part(dtype):
 
 _HOST_UNARY = ('sqrt exp log log2 log10 sin cos tan sinh cosh tanh arcsin arccos arctan '
                'arcsinh arccosh arctanh log1p expm1 exp2').split()
-# largest distance GPU <-> host build seen over the inputs below, in units of
-# eps * (1 + |result|), rounded up generously (observed values are printed)
-_GPU_VS_HOST_EPS = {name: 6 for name in _HOST_UNARY}
-_GPU_VS_HOST_EPS.update({'exp2': 40})
+# Bound on the distance GPU <-> host build over the inputs below, in units of
+# eps * (1 + |result|).  Observed (printed by the test): 0.5 (arctan, arctanh)
+# to 2.01 (tanh, complex128); exp, sin, cos, sinh, cosh, tan, expm1, exp2 1.7
+# to 2.0; sqrt, the logarithms, arcsin, arccos, arcsinh, arccosh 0.8 to 1.8.
+_GPU_VS_HOST_EPS = {name: 4 for name in _HOST_UNARY}
 
 
 @pytest.fixture(scope='module')
@@ -363,7 +367,7 @@ def test_gpu_agrees_with_the_host_build_of_the_header(host_lib, name, dtype):
     for scale in (1.5, 0.01, 1e-5, 30.0):
         z = crandom((50000,), dtype, 5, scale=scale)
         with np.errstate(all='ignore'):
-            want_np = getattr(np, name)(z.astype(np.complex128))
+            want_np = getattr(np, name)(z.astype(np.clongdouble)).astype(np.complex128)
         got = getattr(cp, name)(cp.asarray(z)).get()
         host = _host_call(host_lib, name, z)
         worst_host = max(worst_host, _distance_in_eps(got, host, real_dtype))
@@ -374,3 +378,5 @@ def test_gpu_agrees_with_the_host_build_of_the_header(host_lib, name, dtype):
     print('%-8s %-10s GPU vs host build %.2f eps, GPU vs NumPy %.2f eps' % (
         name, dtype, worst_host, worst_numpy))
     assert worst_host <= _GPU_VS_HOST_EPS[name], (name, dtype, worst_host)
+    # ... and the GPU itself within 4 eps of extended-precision NumPy
+    assert worst_numpy <= 4, (name, dtype, worst_numpy)
