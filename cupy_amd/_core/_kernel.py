@@ -643,6 +643,8 @@ class _ElementwisePlanner:
         # usual grid, so that a thread stores a few vectors only (2^28 float32:
         # 197 -> 174 us)
         write_only = in_bytes == 0
+        if write_only:
+            block = _tuning.get('flat_fill_block')
         if len(itemsizes) <= 2 and block > 512 and not write_only:
             # one stream in, one out: measured 2 % faster with smaller
             # workgroups (the grid cap below keeps threads per CU the same)

@@ -940,6 +940,339 @@ def _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream, 
     return mod
 
 
+def _emit_chain_tile(in_t, out_t, op, skip_nan, vec, trips, idx64, inner, stream, parts, sleep):
+    """One-pass scan along the middle axis of (outer, n, inner) for
+    2 <= inner <= 32 and few, long (outer) slices: the staging of
+    ``_emit_tile`` (a wave lays a run of whole rows out in the LDS and scans its
+    columns) inside the tile protocol of ``_emit_chain`` (a workgroup per tile
+    publishes the tile's totals -- one per column -- and folds those published
+    before it, in an order fixed by the tile's number).  A wave holds PARTS
+    rounds of rows as loaded; they go through the LDS twice, once for the
+    totals and once, after the totals before the tile are known, for the
+    results."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    rows_t, seg, lrows, stride = _tile_geometry(inner, vec, trips)
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define INNER %(inner)d
+#define ROWS_T %(rows_t)d
+#define SEG %(seg)d
+#define LROWS %(lrows)d
+#define SEG_STRIDE %(stride)d
+#define LDS_WORDS (SEG * SEG_STRIDE)
+#define WAVES %(waves)d
+#define PARTS %(parts)d
+#define WAVE_ROWS (PARTS * ROWS_T)
+#define TILE_ROWS (WAVES * WAVE_ROWS)
+#define HEADER_WORDS %(header)d
+#define SPIN_SLEEP %(sleep)d
+// tiles whose totals one round of a wave's polling covers, one per group of INNER lanes
+#define FOLD_TILES (64 / INNER)
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+// position in the LDS of element p of the round (p = row * INNER + column)
+__device__ __forceinline__ int _lds_at(int p) { return p + (p / (LROWS * INNER)) * (SEG_STRIDE - LROWS * INNER); }
+
+// Published values: see the one-pass kernel for contiguous rows.  Value
+// `i * INNER + column` belongs to column `column` of tile (or group) `i`.
+constexpr int kWords = (sizeof(_acc_t) + 3) / 4;
+typedef unsigned long long _slot_t;
+
+__device__ __forceinline__ void _publish(_slot_t* slots, const ptrdiff_t i, const _acc_t& v,
+                                         const unsigned epoch) {
+  unsigned w[kWords];
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) w[k] = 0u;
+  __builtin_memcpy(w, &v, sizeof(_acc_t));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k)
+    __hip_atomic_store(slots + i * kWords + k, ((_slot_t)epoch << 32) | w[k], __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Totals of `count` tiles (or groups) from `first`, per column: lane (s, c)
+// takes column c of the tiles s, s + FOLD_TILES, ...; the partial results of a
+// column are then combined across the lane groups in order.  Every lane ends
+// with the value of its column (lanes past the last whole group: undefined).
+// A lane asks for FOLD_AHEAD of its values at a time (with wide rows a wave
+// covers few tiles per round, and every round is a trip to memory).
+#define FOLD_AHEAD 4
+__device__ __forceinline__ _acc_t _await_fold(_slot_t* slots, const ptrdiff_t first,
+                                              const int count, const int lane,
+                                              const unsigned epoch, const unsigned spin_limit,
+                                              bool& ok) {
+  const int sub = lane / INNER;
+  const int col = lane - sub * INNER;
+  const bool active = sub < FOLD_TILES;
+  _acc_t s = SCAN_IDENTITY;
+  int i = active ? sub : count;
+  unsigned spins = 0;
+  // the newest totals first, alone (see the kernel for contiguous rows)
+  for (;;) {
+    const _slot_t x = __hip_atomic_load(slots + ((first + count) * INNER) * kWords - 1,
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((unsigned)(x >> 32) == epoch) break;
+    if (spins >= spin_limit) { ok = false; break; }
+    ++spins;
+    __builtin_amdgcn_s_sleep(SPIN_SLEEP);
+  }
+  for (;;) {
+    while (i < count) {
+      _slot_t x[FOLD_AHEAD][kWords];
+#pragma unroll
+      for (int a = 0; a < FOLD_AHEAD; ++a) {
+        // (past the last value: the last one again, not used)
+        const int ia = (i + a * FOLD_TILES < count) ? i + a * FOLD_TILES : i;
+#pragma unroll
+        for (int k = 0; k < kWords; ++k)
+          x[a][k] = __hip_atomic_load(slots + ((first + ia) * INNER + col) * kWords + k,
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      bool stalled = false;
+#pragma unroll
+      for (int a = 0; a < FOLD_AHEAD; ++a) {
+        if (stalled || i >= count) break;
+        bool written = true;
+        unsigned w[kWords];
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) {
+          written = written && (unsigned)(x[a][k] >> 32) == epoch;
+          w[k] = (unsigned)x[a][k];
+        }
+        if (!written) { stalled = true; break; }
+        _acc_t v;
+        __builtin_memcpy(&v, w, sizeof(_acc_t));
+        s = SCAN_OP(s, v);
+        i += FOLD_TILES;
+      }
+      if (stalled) break;
+    }
+    if (__ballot(i < count) == 0) break;
+    if (spins >= spin_limit) { ok = false; break; }
+    ++spins;
+    __builtin_amdgcn_s_sleep(SPIN_SLEEP);
+  }
+  // running combination down the lane groups of a column; the last group holds all
+#pragma unroll
+  for (int d = 1; d < FOLD_TILES; d <<= 1) {
+    const _acc_t other = cupy::shfl_up<64>(s, d * INNER);
+    s = (lane >= d * INNER && active) ? SCAN_OP(other, s) : s;
+  }
+  return cupy::shfl_idx<64>(s, (FOLD_TILES - 1) * INNER + col);
+}
+
+// One round of a wave: its rows as loaded -> the LDS -> every lane's own rows
+// of its column scanned in registers (`v`), the running combination of the
+// segments of a column across the lanes (`incl`).  Returns the column's total.
+__device__ __forceinline__ _acc_t _round_scan(
+    const cupy::Vec<_in_t, VEC> (&raw)[TRIPS], _acc_t* lds, const int valid, const int lane,
+    const int seg, const int col, const bool active, _acc_t (&v)[LROWS], _acc_t& incl) {
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    const int p = (t * 64 + lane) * VEC;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k)
+      if (p + k < ROWS_T * INNER)
+        lds[_lds_at(p + k)] = (p + k < valid) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < LROWS; ++i) v[i] = lds[seg * SEG_STRIDE + i * INNER + col];
+#pragma unroll
+    for (int i = 1; i < LROWS; ++i) v[i] = SCAN_OP(v[i - 1], v[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < LROWS; ++i) v[i] = SCAN_IDENTITY;
+  }
+  incl = v[LROWS - 1];
+#pragma unroll
+  for (int d = 1; d < SEG; d <<= 1) {
+    const _acc_t other = cupy::shfl_up<64>(incl, d * INNER);
+    incl = (lane >= d * INNER) ? SCAN_OP(other, incl) : incl;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  return cupy::shfl_idx<64>(incl, (SEG - 1) * INNER + col);
+}
+
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_clear(
+    unsigned* desc, const unsigned words) {
+  for (unsigned i = blockIdx.x * %(block)d + threadIdx.x; i < words; i += gridDim.x * %(block)d)
+    desc[i] = 0u;
+}
+
+// One workgroup per tile of TILE_ROWS rows of one (outer) slice, tiles numbered
+// by blockIdx.x; waits, slots and the order of combination as in the kernel for
+// contiguous rows, with INNER values per tile instead of one.
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_tile(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, unsigned* desc,
+    const _idx_t n_outer, const _idx_t n, const _idx_t tiles_per_row, const _idx_t group_tiles,
+    const _idx_t groups_per_row, const unsigned epoch, const unsigned spin_limit,
+    unsigned* fault) {
+  __shared__ _acc_t _lds_all[WAVES][LDS_WORDS];
+  __shared__ _acc_t sm_wave[WAVES + 2][INNER];
+  const ptrdiff_t n_tiles = (ptrdiff_t)n_outer * tiles_per_row;
+  _slot_t* tile_totals = reinterpret_cast<_slot_t*>(desc + HEADER_WORDS);
+  _slot_t* group_totals = tile_totals + n_tiles * INNER * kWords;
+  const int lane = threadIdx.x %% 64;
+  const int wv = threadIdx.x / 64;
+  _acc_t* lds = _lds_all[wv];
+  const int seg = lane / INNER;
+  const int col = lane - seg * INNER;
+  const bool active = lane < SEG * INNER;
+  const ptrdiff_t tile = blockIdx.x;
+  if (tile >= n_tiles) return;
+  const _idx_t o = (_idx_t)(tile / tiles_per_row);
+  const _idx_t t_row = (_idx_t)(tile - (ptrdiff_t)o * tiles_per_row);
+  const _idx_t r0 = t_row * TILE_ROWS + wv * WAVE_ROWS;      // this wave's first row
+  // ---- the wave's rows as loaded, all requested at once
+  cupy::Vec<_in_t, VEC> raw[PARTS][TRIPS];
+  int valid[PARTS];
+#pragma unroll
+  for (int q = 0; q < PARTS; ++q) {
+    const _idx_t rb = r0 + q * ROWS_T;
+    const _idx_t left = n - rb;
+    const int rows_here = left <= 0 ? 0 : (left < ROWS_T ? (int)left : ROWS_T);
+    valid[q] = rows_here * INNER;
+    const _in_t* src = in + ((ptrdiff_t)o * n + rb) * INNER;
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * 64 + lane) * VEC;
+      if (p + VEC <= valid[q]) {
+        raw[q][t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + p);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) raw[q][t].v[k] = (p + k < valid[q]) ? src[p + k] : _in_t();
+      }
+    }
+  }
+  // ---- totals: of every round, of the wave, of the tile (per column)
+  _acc_t round_total[PARTS];
+  _acc_t carry = SCAN_IDENTITY;
+#pragma unroll
+  for (int q = 0; q < PARTS; ++q) {
+    _acc_t v[LROWS];
+    _acc_t incl;
+    round_total[q] = _round_scan(raw[q], lds, valid[q], lane, seg, col, active, v, incl);
+    carry = (q == 0) ? round_total[q] : SCAN_OP(carry, round_total[q]);
+  }
+  if (lane < INNER) sm_wave[wv][lane] = carry;
+  __syncthreads();
+  _acc_t wave_before = SCAN_IDENTITY;
+  _acc_t tile_total = sm_wave[0][col];
+#pragma unroll
+  for (int w = 1; w < WAVES; ++w) {
+    if (w == wv) wave_before = tile_total;
+    tile_total = SCAN_OP(tile_total, sm_wave[w][col]);
+  }
+  // ---- what precedes the tile in its slice
+  const _idx_t g = t_row / group_tiles;
+  const int t_group = (int)(t_row - g * group_tiles);
+  const bool closes_group = (t_group == group_tiles - 1) || (t_row == tiles_per_row - 1);
+  const ptrdiff_t row_groups = (ptrdiff_t)o * groups_per_row;
+  if (wv == 0) {
+    if (lane < INNER) _publish(tile_totals, tile * INNER + lane, tile_total, epoch);
+    bool ok = true;
+    _acc_t in_group = SCAN_IDENTITY;
+    if (t_group > 0)
+      in_group = _await_fold(tile_totals, tile - t_group, t_group, lane, epoch, spin_limit, ok);
+    if (lane < INNER) {
+      if (closes_group)
+        _publish(group_totals, (row_groups + g) * INNER + lane,
+                 (t_group > 0) ? SCAN_OP(in_group, tile_total) : tile_total, epoch);
+      sm_wave[WAVES][lane] = in_group;
+    }
+    if (!ok && lane == 0 && fault) *reinterpret_cast<volatile unsigned*>(fault) = 1u;
+  } else if (wv == 1 && g > 0) {
+    bool ok = true;
+    const _acc_t groups_before =
+        _await_fold(group_totals, row_groups, (int)g, lane, epoch, spin_limit, ok);
+    if (lane < INNER) sm_wave[WAVES + 1][lane] = groups_before;
+    if (!ok && lane == 0 && fault) *reinterpret_cast<volatile unsigned*>(fault) = 1u;
+  }
+  __syncthreads();
+  _acc_t base = SCAN_IDENTITY;
+  if (g > 0) base = sm_wave[WAVES + 1][col];
+  if (t_group > 0) base = (g > 0) ? SCAN_OP(base, sm_wave[WAVES][col]) : sm_wave[WAVES][col];
+  if (wv > 0) base = (t_row > 0) ? SCAN_OP(base, wave_before) : wave_before;
+  // ---- results, round by round
+  carry = base;
+  bool seeded = t_row > 0 || wv > 0;
+#pragma unroll
+  for (int q = 0; q < PARTS; ++q) {
+    _acc_t v[LROWS];
+    _acc_t incl;
+    (void)_round_scan(raw[q], lds, valid[q], lane, seg, col, active, v, incl);
+    _acc_t before = cupy::shfl_up<64>(incl, INNER);
+    const bool has_before = seg > 0;
+    before = seeded ? (has_before ? SCAN_OP(carry, before) : carry) : before;
+    const bool any = seeded || has_before;
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < LROWS; ++i)
+        lds[seg * SEG_STRIDE + i * INNER + col] = any ? SCAN_OP(before, v[i]) : v[i];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    _out_t* dst = out + ((ptrdiff_t)o * n + r0 + q * ROWS_T) * INNER;
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * 64 + lane) * VEC;
+      if (p + VEC <= valid[q]) {
+        cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(lds[_lds_at(p + k)]);
+        cupy::store_vec<_out_t, VEC, NT_STORE>(dst + p, r);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          if (p + k < valid[q]) dst[p + k] = static_cast<_out_t>(lds[_lds_at(p + k)]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    carry = seeded ? SCAN_OP(carry, round_total[q]) : round_total[q];
+    seeded = true;
+  }
+}
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           inner=inner, rows_t=rows_t, seg=seg, lrows=lrows, stride=stride,
+           waves=_CHAIN_WAVES, parts=parts, header=_CHAIN_HEADER_WORDS, sleep=sleep,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
+
+
+def _module_chain_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream,
+                       parts):
+    sleep = _tuning.get('scan_chain_sleep')
+    key = ('chain tile', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan,
+           vec, trips, idx64, inner, stream, parts, sleep)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_chain_tile(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                               vec, trips, idx64, inner, stream, parts, sleep)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
 def _module_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream, reuse):
     key = ('tile', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
            trips, idx64, inner, stream, reuse)
@@ -1051,10 +1384,12 @@ def _chain_slots(dev_id, stream_ptr, words, mod):
         return arena[0], arena[1]
 
 
-def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_ptr):
-    """The one-pass scan of a few long rows (``_emit_chain``): input read once,
-    output written once.  Returns False where it does not apply (the caller
-    then takes the three-pass route)."""
+def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_ptr, inner=1):
+    """The one-pass scan of a few long rows (``_emit_chain``) or, with
+    ``inner`` > 1, of a few long slices of rows of ``inner`` elements scanned
+    down their columns (``_emit_chain_tile``): input read once, output written
+    once.  Returns False where it does not apply (the caller then takes the
+    three-pass route)."""
     if not _tuning.get('scan_chain'):
         return False
     dev_id = _device.get_device_id()
@@ -1079,11 +1414,19 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
         # measured on 2^20 .. 2^26 float32: 8 parts (128 KiB of input per tile)
         # are best from 64 MiB on, 4 from 16 MiB on
         # (with 8-byte and wider values 8 parts do not fit the registers of a lane)
-        nbytes = n_rows * n * in_dtype.itemsize
+        nbytes = n_rows * n * inner * in_dtype.itemsize
         parts = 8 if nbytes >= 64 << 20 else 4 if nbytes >= 16 << 20 else 2
-        if max(in_dtype.itemsize, _acc_dtype(out_dtype).itemsize) > 4:
+        if max(in_dtype.itemsize, _acc_dtype(out_dtype).itemsize) > 4 or inner > 1:
             parts = min(parts, 4)
-    tile = _BLOCK * vec * trips * parts
+        if 1 < inner <= 6:
+            # (2^26 float32 as (n,3): 115 us with 2 parts, 123 with 4; as (n,5)
+            # 133 / 138; as (n,12) 131 / 113; as (n,16) 128 / 120)
+            parts = min(parts, 2)
+    if inner > 1:
+        vec = max(1, 16 // max(in_dtype.itemsize, out_dtype.itemsize))
+        tile = _CHAIN_WAVES * parts * _tile_geometry(inner, vec, trips)[0]     # rows
+    else:
+        tile = _BLOCK * vec * trips * parts
     tiles_per_row = (n + tile - 1) // tile
     n_tiles = n_rows * tiles_per_row
     if n_tiles < 2 or n_tiles * _BLOCK > 0xffffffff:
@@ -1095,17 +1438,23 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
     n_groups = n_rows * groups_per_row
     # every 32-bit word of a published total sits in a 64-bit slot beside its mark
     words_per_value = (_acc_dtype(out_dtype).itemsize + 3) // 4
-    desc_words = _CHAIN_HEADER_WORDS + 2 * words_per_value * (n_tiles + n_groups)
+    desc_words = _CHAIN_HEADER_WORDS + 2 * words_per_value * inner * (n_tiles + n_groups)
     if desc_words > 0xffffffff:
         return False
-    mod = _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream,
-                        n % vec != 0, parts)
+    if inner > 1:
+        mod = _module_chain_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner,
+                                 stream, parts)
+        name = 'cupy_scan_chain_tile'
+    else:
+        mod = _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream,
+                            n % vec != 0, parts)
+        name = 'cupy_scan_chain'
     desc, epoch = _chain_slots(dev_id, stream_ptr, desc_words, mod)
     ic = 'q' if idx64 else 'i'
     blob = struct.pack('@PPP' + ic * 5 + 'IIP', src.data.ptr, dst.data.ptr, desc.data.ptr,
                        n_rows, n, tiles_per_row, group_tiles, groups_per_row, epoch,
                        _tuning.get('scan_chain_spin_limit'), fault)
-    mod.get_function('cupy_scan_chain').launch_packed(
+    mod.get_function(name).launch_packed(
         (n_tiles, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
     return True
 
@@ -1186,6 +1535,9 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         n_chunks = 1
         if may_chunk and outer < want and n > 2 * rows_t:
             n_chunks = min((want + outer - 1) // outer, (n + rows_t - 1) // rows_t)
+        if n_chunks > 1 and _scan_chained(src, dst, outer, n, op, skip_nan, vec, idx64, stream,
+                                          stream_ptr, inner=inner):
+            return
         chunk_len = (n + n_chunks - 1) // n_chunks
         chunk_len = (chunk_len + rows_t - 1) // rows_t * rows_t
         n_chunks = (n + chunk_len - 1) // chunk_len

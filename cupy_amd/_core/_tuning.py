@@ -14,7 +14,14 @@ _params = {
     # flat elementwise kernel
     'flat_block': 1024,         # threads per workgroup
     'flat_unroll': 1,           # vectors per thread per trip
-    'flat_blocks_per_cu': 64,   # grid cap, in workgroups per CU
+    # Grid cap, in workgroups per CU.  A workgroup per 16 KiB of every operand
+    # and no loop is best at every size measured; with the cap at 64 arrays of
+    # 1 GiB looped four times and lost six points (copy 76.6 -> 82.2 % of peak,
+    # saxpy 73.7 -> 80.4 %; 256 MiB arrays, which fit under either cap: 83 / 82 %)
+    'flat_blocks_per_cu': 1024,
+    # Threads per workgroup of a launch that only writes (fill 256 MiB: 70.7 %
+    # of peak with 1024, 76.7 % with 256; 1 GiB: 76.8 -> 84.5 %)
+    'flat_fill_block': 256,
     # matrices stored row after row combined with a value per row or per column
     # stay in the flat kernel (row and column by one division per vector)
     'flat_bcast': True,

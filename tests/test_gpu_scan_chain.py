@@ -143,3 +143,48 @@ def test_a_tile_that_gives_up_is_reported_and_the_kernel_retired():
     names = launched(lambda: d.cumsum())
     assert 'cupy_scan_chain' not in names and 'cupy_scan_rows_seeded' in names
     assert_exact(d.cumsum().get(), h.cumsum())
+
+
+@pytest.mark.parametrize('shape,axis', [((700001, 3), 0), ((2, 300000, 5), 1), ((1 << 20, 2), 0),
+                                        ((150000, 32), 0), ((3, 99999, 7), 1), ((400000, 12), 0)])
+def test_columns_of_narrow_arrays_in_one_pass(shape, axis):
+    """Long columns of arrays with a narrow tail: tiles of whole rows, one
+    published total per column."""
+    rng = np.random.default_rng(shape[-1])
+    h = rng.integers(-5, 6, shape).astype(np.int32)
+    d = cp.asarray(h)
+    assert 'cupy_scan_chain_tile' in launched(lambda: d.cumsum(axis=axis))
+    assert_exact(d.cumsum(axis=axis).get(), h.cumsum(axis=axis))
+    hf = rng.uniform(0, 1, shape).astype(np.float32)
+    df = cp.asarray(hf)
+    got = df.cumsum(axis=axis).get()
+    want = np.cumsum(hf.astype(np.float64), axis=axis)
+    assert (np.abs(got - want) <= 1e-5 * want + 1e-6).all()
+    assert_exact(df.cumsum(axis=axis).get(), got)                 # same bits on every run
+    other = three_pass(lambda: df.cumsum(axis=axis).get())
+    assert (np.abs(got - other) <= 2e-5 * want + 1e-6).all()
+
+
+@pytest.mark.parametrize('parts', [1, 2, 4])
+def test_narrow_arrays_other_types_and_tile_sizes(parts):
+    _tuning.set(scan_chain_parts=parts)
+    rng = np.random.default_rng(40 + parts)
+    h8 = rng.integers(-100, 100, (500001, 3)).astype(np.int8)
+    assert_exact(cp.cumsum(cp.asarray(h8), axis=0).get(), np.cumsum(h8, axis=0))
+    hd = rng.standard_normal((300000, 5))
+    got = cp.cumsum(cp.asarray(hd), axis=0).get()
+    scale = np.cumsum(np.abs(hd), axis=0)
+    assert (np.abs(got - np.cumsum(hd, axis=0)) <= 1e-13 * scale).all()
+    hc = (rng.standard_normal((200001, 6)) + 1j * rng.standard_normal((200001, 6))).astype(np.complex64)
+    got = cp.cumsum(cp.asarray(hc), axis=0).get()
+    want = np.cumsum(hc.astype(np.complex128), axis=0)
+    scale = np.cumsum(np.abs(hc).astype(np.float64), axis=0)
+    assert (np.abs(got - want) <= 1e-5 * scale + 1e-5).all()
+    hp = np.ones((400000, 4), np.int64)
+    hp[rng.choice(400000, 30, replace=False), rng.integers(0, 4, 30)] = rng.choice([-1, 2], 30)
+    assert_exact(cp.cumprod(cp.asarray(hp), axis=0).get(), np.cumprod(hp, axis=0))
+    hn = rng.uniform(0, 1, (500000, 3)).astype(np.float32)
+    hn[::777, 1] = np.nan
+    got = cp.nancumsum(cp.asarray(hn), axis=0).get()
+    want = np.nancumsum(hn.astype(np.float64), axis=0)
+    assert (np.abs(got - want) <= 1e-5 * want + 1e-6).all()
