@@ -541,6 +541,7 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
     fn = compiler.compile_with_cache(code, ('-DCUPY_FUSED_ROWS',)).get_function(name)
     rows_per_block = BLOCK // group
     cus = _device.get_compute_units(_device.get_device_id())
-    grid = max(1, min((n_rows + rows_per_block - 1) // rows_per_block, cus * 16))
+    grid = max(1, min((n_rows + rows_per_block - 1) // rows_per_block,
+                      cus * _tuning.get('fused_rows_blocks_per_cu')))
     return RowPlan(fn, _make_packer(fmt), (grid, 1, 1), n_rows, in_slots, out_specs,
                    out_returns, single)

@@ -1516,7 +1516,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                       ragged=n % vec != 0, reuse=n_chunks > 1 and reuse_ok)
         groups = outer * n_chunks
         per_block = _BLOCK // group
-        grid = max(1, min((groups + per_block - 1) // per_block, cus * 32))
+        grid = max(1, min((groups + per_block - 1) // per_block, cus * _tuning.get('scan_blocks_per_cu')))
         fmt = '@PPP' + ic * 4
 
         def launch(name, totals_ptr):
@@ -1545,7 +1545,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                            n_chunks > 1 and reuse_ok)
         waves = outer * n_chunks
         per_block = _BLOCK // _WAVE
-        grid = max(1, min((waves + per_block - 1) // per_block, cus * 32))
+        grid = max(1, min((waves + per_block - 1) // per_block, cus * _tuning.get('scan_blocks_per_cu')))
         fmt = '@PPP' + ic * 4
 
         def launch(name, totals_ptr):
@@ -1572,7 +1572,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                             stream)
         waves = outer * n_chunks
         per_block = _BLOCK // _WAVE
-        grid = max(1, min((waves + per_block - 1) // per_block, cus * 32))
+        grid = max(1, min((waves + per_block - 1) // per_block, cus * _tuning.get('scan_blocks_per_cu')))
         fmt = '@PPP' + ic * 4
 
         def launch(name, totals_ptr):
@@ -1606,7 +1606,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, 64, stream,
                       reuse=n_chunks > 1 and reuse_ok)
         work = threads * n_chunks
-        grid = max(1, min((work + _BLOCK - 1) // _BLOCK, cus * 64))
+        grid = max(1, min((work + _BLOCK - 1) // _BLOCK, cus * 2 * _tuning.get('scan_blocks_per_cu')))
         fmt = '@PPP' + ic * 5
 
         def launch(name, totals_ptr):

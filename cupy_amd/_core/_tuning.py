@@ -70,7 +70,9 @@ _params = {
     # the rows are short enough), False (never)
     'rows_flat': 'auto',
     'rows_flat_max_bytes': 2048,
-    'rows_group_rows_per_lane': 64,   # grid cap for sub-wave groups: CUs * this workgroups
+    # Grid cap for sub-wave groups: CUs * this workgroups (2^28 elements in rows
+    # of 1024: sum 83.2 -> 86.4 % of peak, argmax 82.8 -> 86.4 % with 256 instead of 64)
+    'rows_group_rows_per_lane': 256,
     'cols_stream': True,
     # Row-slices a thread of the column kernel loads before it uses the first:
     # 1 when the reduce axis is split across workgroups and the rows start on
@@ -81,6 +83,9 @@ _params = {
     'cols_unroll': 1,
     'cols_unroll_near': 4,
     'cols_solo_block': 1024,    # workgroup of the thread-per-column variant
+    # Grid cap of the scan kernels, in workgroups per CU (cumsum along rows of
+    # 1024 float32, 2^28 elements: 74.9 % of peak with 32, 80.2 % with 256)
+    'scan_blocks_per_cu': 256,
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
@@ -98,6 +103,10 @@ _params = {
     # with a wave against 68 % with a workgroup.  Requesting the next row before
     # the current one is worked on did not help: 62 % against 76 % on rows of 8192)
     'fused_rows_wave_words': 32,
+    # Grid cap of that kernel, in workgroups per CU (softmax 16384x4096: 94.5 us
+    # with 16, 86.0 with 64 or more; rows of 1024: 89.9 -> 85.1; layer
+    # normalisation over rows of 100: 110 -> 96)
+    'fused_rows_blocks_per_cu': 256,
     # Vector accesses need only the alignment of one element: an access of 16
     # bytes at an address that is a multiple of 4 measures within 4 % of an
     # aligned one (reads of 2^28 bytes: 82 % of peak against 86 %), one at an odd
