@@ -417,7 +417,7 @@ def emit_generic(name, operands, operation, typedefs='', preamble='',
 
 def emit_rows2d(name, operands, operation, typedefs='', preamble='',
                 loop_prep='', after_loop='', kinds=None, vec=4, idx64=False,
-                stream_hint=True, block=BLOCK):
+                stream_hint=True, block=BLOCK, outer=1):
     """Kernel for a matrix problem (rows r, columns c) none of whose arrays
     runs against the columns: every row is walked in vectors of ``vec``
     columns that start at column 0, 1 * vec, ... of that row, so that no
@@ -432,6 +432,12 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
     The last ``_nc % vec`` columns of a row are handled element by element by
     the lane that owns them.  Kernel parameters after the operands:
     ``_nr, _nc``, then per array its row stride and column stride in elements.
+
+    ``outer`` > 1: the rows are the positions of ``outer`` axes (C order), each
+    with a stride of its own per array -- a permutation of the leading axes of
+    arrays whose last axis is contiguous.  ``_nr`` is still the number of rows;
+    the extents of all but the first of those axes follow ``_nc``
+    (``_ne1`` .. ), and every array brings one row stride per axis.
     """
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     arrays = [op for op in operands if op.kind == 'array']
@@ -441,14 +447,16 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
     use_i = uses_identifier(operation, 'i')
     parts = [_param_decl(op) for op in operands if op.kind != 'indexer']
     parts += ['const %s _nr' % idx_t, 'const %s _nc' % idx_t]
+    parts += ['const %s _ne%d' % (idx_t, d) for d in range(1, outer)]
     for op in arrays:
-        parts += ['const %s _sr_%s' % (idx_t, op.name), 'const %s _sc_%s' % (idx_t, op.name)]
+        parts += ['const %s _sr_%s' % (idx_t, op.name)]
+        parts += ['const %s _sr%d_%s' % (idx_t, d, op.name) for d in range(1, outer)]
+        parts += ['const %s _sc_%s' % (idx_t, op.name)]
     assert not any(op.kind == 'indexer' for op in operands)
     params = ', '.join(parts)
 
     def addr(op, c):
-        return '(_p_%s + (ptrdiff_t)_rk * _sr_%s + (ptrdiff_t)(%s) * _sc_%s)' % (
-            op.name, op.name, c, op.name)
+        return '(_p_%s + _ro_%s + (ptrdiff_t)(%s) * _sc_%s)' % (op.name, op.name, c, op.name)
 
     src = [_header(typedefs, preamble)]
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
@@ -460,6 +468,20 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
                '_v += (%s)gridDim.x * %d) {' % (idx_t, idx_t, block, idx_t, block))
     src.append('    const %s _rk = _v / _nvr;' % idx_t)
     src.append('    const %s _ck = (_v - _rk * _nvr) * %d;' % (idx_t, vec))
+    # where the row starts in every array
+    if outer == 1:
+        for op in arrays:
+            src.append('    const ptrdiff_t _ro_%s = (ptrdiff_t)_rk * _sr_%s;' % (op.name, op.name))
+    else:
+        src.append('    %s _rest = _rk;' % idx_t)
+        for d in range(outer - 1, 0, -1):
+            src.append('    const %s _q%d = _rest / _ne%d;' % (idx_t, d, d))
+            src.append('    const %s _i%d = _rest - _q%d * _ne%d;' % (idx_t, d, d, d))
+            src.append('    _rest = _q%d;' % d)
+        for op in arrays:
+            terms = ['(ptrdiff_t)_rest * _sr_%s' % op.name]
+            terms += ['(ptrdiff_t)_i%d * _sr%d_%s' % (d, d, op.name) for d in range(1, outer)]
+            src.append('    const ptrdiff_t _ro_%s = %s;' % (op.name, ' + '.join(terms)))
     src.append('    if (_ck + %d <= _nc) {' % vec)
     for op in arrays:
         k = kinds[op.name]

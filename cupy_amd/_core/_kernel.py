@@ -446,6 +446,11 @@ class _ElementwisePlanner:
                         force_read_out, stream_ptr, kernel_name, rec)
                 mode = self._classify_2d(arrays, cstrides, args, nin)
             elif nd in (3, 4) and not self._uses_ind and not self._uses_i:
+                plan = self._plan_rows_nd(arrays, cshape, cstrides, args, nin)
+                if plan is not None:
+                    return self._launch_rows2d(
+                        dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
+                        force_read_out, stream_ptr, kernel_name, rec)
                 plan = self._plan_batched(arrays, cshape, cstrides, args, nin)
                 if plan is not None:
                     done = self._launch_tiled(
@@ -542,35 +547,80 @@ class _ElementwisePlanner:
                 return cshape, cstrides, kinds
         return None
 
+    def _plan_rows_nd(self, arrays, cshape, cstrides, args, nin):
+        """Problem of three or four axes in which every array runs along the
+        last axis with unit stride (or repeats one value along it): a
+        permutation of the leading axes, (B, S, H, D) -> (B, H, S, D), a
+        value per row.  The row kernel then takes the leading axes as ONE run
+        of rows whose start it finds from one stride per axis and array.
+        Returns ((rows, columns), [(row strides per leading axis, column
+        stride) per array], kinds, extents of the leading axes) or None."""
+        if not _tuning.get('rows2d'):
+            return None
+        names = [p.name for a, p in zip(args, self.params)
+                 if isinstance(a, ndarray) and not p.raw]
+        outs = args[nin:]
+        kinds = {}
+        for a, cs, nm in zip(arrays, cstrides, names):
+            item = a.dtype.itemsize
+            if any(s % item for s in cs):
+                return None
+            if cs[-1] == item:
+                kind = 'R'
+            elif cs[-1] == 0 and not any(a is o for o in outs):
+                kind = 'row'
+            else:
+                return None
+            if kinds.get(nm, kind) != kind:
+                return None
+            kinds[nm] = kind
+        if not any(k == 'R' for k in kinds.values()):
+            return None
+        lead = tuple(cshape[:-1])
+        # rows of a vector or two leave most lanes of a wave on different rows
+        # with nothing gained over the tiled kernel
+        if cshape[-1] * max(a.dtype.itemsize for a in arrays) < 256:
+            return None
+        return ((internal.prod(lead), cshape[-1]),
+                [(tuple(cs[:-1]), cs[-1]) for cs in cstrides], kinds, lead)
+
     def _launch_rows2d(self, dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
                        force_read_out, stream_ptr, kernel_name, rec):
-        (nr, nc), cstrides, kinds = plan
+        if len(plan) == 4:
+            (nr, nc), nd_strides, kinds, lead = plan
+        else:
+            (nr, nc), cstrides, kinds = plan
+            nd_strides = [((cs[0],), cs[1]) for cs in cstrides]
+            lead = (nr,)
+        outer = len(lead)
         vec = max(1, 16 // max(a.dtype.itemsize for a in arrays))
         if _tuning.get('rows2d_narrow_vec') and nc < 12 * vec:
             # few vectors per row: a partial one at every row end would split
             # the lanes of a wave between two code paths
             while vec > 1 and nc % vec:
                 vec //= 2
-        span = max(abs(cs[0]) * nr + abs(cs[1]) * nc for cs in cstrides)
+        span = max(sum(abs(s) * e for s, e in zip(rs, lead)) + abs(sc) * nc
+                   for rs, sc in nd_strides)
         nvr = (nc + vec - 1) // vec
         idx64 = span > _INT32_MAX or nr * nvr * vec > _INT32_MAX - (1 << 24)
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
         names = [p.name for a, p in zip(args, self.params)
                  if isinstance(a, ndarray) and not p.raw]
         # a value per row, or one row repeated: not counted as streamed traffic
-        light = [n for n, cs in zip(names, cstrides) if cs[0] == 0 or cs[1] == 0]
+        light = [n for n, (rs, sc) in zip(names, nd_strides)
+                 if sc == 0 or all(r == 0 for r in rs)]
         in_bytes, out_bytes = self._traffic(args, nin, light)
         stream_hint = _tuning.stream_policy(_tuning.get('tiled_stream'), in_bytes, out_bytes)
         block = 256
         key = ('rows2d', tuple(o.key() for o in operands), typedefs, vec, idx64,
-               tuple(sorted(kinds.items())), dev_id, stream_hint, block)
+               tuple(sorted(kinds.items())), dev_id, stream_hint, block, outer)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
             code = _cg.emit_rows2d(
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, kinds=kinds, vec=vec, idx64=idx64,
-                stream_hint=stream_hint, block=block)
+                stream_hint=stream_hint, block=block, outer=outer)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']
@@ -581,17 +631,17 @@ class _ElementwisePlanner:
                     fmt.append('P' + 'q' * (1 + 2 * o.ndim))
                 elif o.kind == 'scalar':
                     fmt.append(_scalar_struct_code(o.store_t))
-            fmt.append(ic * (2 + 2 * len(arrays)))
+            fmt.append(ic * (2 + (outer - 1) + (outer + 1) * len(arrays)))
             entry = (fn, _make_packer(fmt), code)
             with self._lock:
                 entry = self._memo.setdefault(key, entry)
             self._remember_code(args, entry[2])
         fn, packer, _ = entry
         block_args = self._flat_values(args)
-        block_args.const(nr, nc)
-        for a, cs in zip(arrays, cstrides):
+        block_args.const(nr, nc, *lead[1:])
+        for a, (rs, sc) in zip(arrays, nd_strides):
             item = a.dtype.itemsize
-            block_args.const(cs[0] // item, cs[1] // item)
+            block_args.const(*([r // item for r in rs] + [sc // item]))
         grid = max(1, min((nr * nvr + block - 1) // block,
                           _grid_limit(dev_id, _tuning.get('flat_blocks_per_cu')) * 4))
         _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
