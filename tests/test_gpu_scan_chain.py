@@ -188,3 +188,29 @@ def test_narrow_arrays_other_types_and_tile_sizes(parts):
     got = cp.nancumsum(cp.asarray(hn), axis=0).get()
     want = np.nancumsum(hn.astype(np.float64), axis=0)
     assert (np.abs(got - want) <= 1e-5 * want + 1e-6).all()
+
+
+def test_scans_on_two_streams_at_once():
+    """Two one-pass scans in flight together share the CUs: tiles of either
+    wait only for tiles of their own launch that started earlier, so both
+    finish, and each stream has its own slots."""
+    rng = np.random.default_rng(77)
+    ha = rng.integers(-5, 6, (1 << 23) + 17).astype(np.int32)
+    hb = rng.integers(-5, 6, (3, 1 << 22)).astype(np.int64)
+    da, db = cp.asarray(ha), cp.asarray(hb)
+    s1, s2 = cp.cuda.Stream(), cp.cuda.Stream()
+    outs = []
+    for _ in range(4):
+        with s1:
+            ra = da.cumsum()
+        with s2:
+            rb = db.cumsum(axis=1)
+        outs.append((ra, rb))
+    s1.synchronize()
+    s2.synchronize()
+    for ra, rb in outs:
+        assert_exact(ra.get(), ha.cumsum())
+        assert_exact(rb.get(), hb.cumsum(axis=1))
+    # nothing gave up on the way
+    d = cp.asarray(ha)
+    assert 'cupy_scan_chain' in launched(lambda: d.cumsum())
