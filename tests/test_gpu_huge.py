@@ -98,6 +98,18 @@ def test_transposed_operand_beyond_2_to_31_bytes():
     assert np.array_equal(host, (2.0 * ((r * cols + c) % 1000)).astype(np.float32))
 
 
+def test_scan_down_the_columns_of_a_narrow_array_beyond_2_to_31_elements():
+    """(2**29 + 3, 5) int8 along axis 0: the one-pass kernel for narrow arrays
+    with 64-bit offsets; the running count wraps as int8 wraps."""
+    rows = 2 ** 29 + 3
+    a = cp.ones((rows, 5), 'b')
+    r = cp.cumsum(a, axis=0, dtype='b')
+    assert r.shape == (rows, 5) and r.dtype == np.int8
+    check = cp.ElementwiseKernel(
+        'int8 s', 'bool ok', 'ok = s == (signed char)(((i / 5) + 1) & 255)', 'is_row_count_mod256')
+    assert bool(check(r).all().get())
+
+
 def test_axis_reductions_and_scans_with_rows_beyond_2_to_30():
     m = 2 ** 30 + 1
     a = _fill_mod100_i8(size=3 * m).reshape(3, m)
