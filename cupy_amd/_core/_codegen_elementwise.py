@@ -561,7 +561,8 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
 
 def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
                  loop_prep='', after_loop='', layouts=None, vec=4, tile_r=64,
-                 tile_c=64, threads=256, idx64=False, stream_hint=True, batched=False):
+                 tile_c=64, threads=256, idx64=False, stream_hint=True, batched=False,
+                 batch_first=False):
     """Kernel for a 2-d index space (rows r, columns c) where every array
     operand is contiguous along one of the axes.
 
@@ -633,8 +634,15 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     if batched:
         src.append('  const %s _nt2 = _ntr * _ntc;' % idx_t)
         src.append('  for (%s _tile_b = blockIdx.x; _tile_b < _nt2 * _nbt; _tile_b += gridDim.x) {' % idx_t)
-        src.append('    const %s _bt = _tile_b / _nt2;' % idx_t)
-        src.append('    const %s _tile = _tile_b - _bt * _nt2;' % idx_t)
+        if batch_first:
+            # consecutive workgroups take the same tile of consecutive batch
+            # entries: where those lie closer together in memory than the rows
+            # of a tile, workgroups that run side by side share DRAM pages
+            src.append('    const %s _tile = _tile_b / _nbt;' % idx_t)
+            src.append('    const %s _bt = _tile_b - _tile * _nbt;' % idx_t)
+        else:
+            src.append('    const %s _bt = _tile_b / _nt2;' % idx_t)
+            src.append('    const %s _tile = _tile_b - _bt * _nt2;' % idx_t)
         src.append('    const %s _b0 = _bt / _nb1;' % idx_t)
         src.append('    const %s _b1 = _bt - _b0 * _nb1;' % idx_t)
         for op in arrays:

@@ -999,9 +999,16 @@ class _ElementwisePlanner:
                 for a, cs in zip(arrays, cstrides))
             if not batch or unaligned:
                 stream_hint = (stream_hint[0], False)
+        # The order the tiles of a batch are visited in: batch entries that lie
+        # closer together than the rows of a tile go first (see emit_tiled2d)
+        batch_first = False
+        if batch and _tuning.get('tiled_batch_first'):
+            inner_batch = [abs(bs[1] if bshape[1] > 1 else bs[0]) for bs in bstrides]
+            pitch = [max(abs(cs[0]), abs(cs[1])) for cs in cstrides]
+            batch_first = all(b and b < p for b, p in zip(inner_batch, pitch))
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
-               threads, bool(batch))
+               threads, bool(batch), batch_first)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
@@ -1009,7 +1016,7 @@ class _ElementwisePlanner:
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
                 tile_r=tile_r, tile_c=tile_c, threads=threads, idx64=idx64,
-                stream_hint=stream_hint, batched=bool(batch))
+                stream_hint=stream_hint, batched=bool(batch), batch_first=batch_first)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']

@@ -51,6 +51,7 @@ _params = {
     'flat_stream': 'auto',
     # tiled 2-d elementwise kernel
     'tiled_stream': 'auto',
+    'tiled_batch_first': True,  # batched tiles: near batch entries before far rows
     'tiled_big_min': 512,       # extent of both tile axes from which tiles are 128 x 128
     'cache_bytes': 256 << 20,   # capacity of the memory-side cache (Infinity Cache)
     # reductions
