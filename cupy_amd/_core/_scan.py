@@ -1426,10 +1426,20 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
         vec = max(1, 16 // max(in_dtype.itemsize, out_dtype.itemsize))
         tile = _CHAIN_WAVES * parts * _tile_geometry(inner, vec, trips)[0]     # rows
     else:
+        # No tile longer than a row; and rows of few tiles want small ones: a
+        # tile then waits for few others, and there are many rows to go on
+        # with (2^26 float32 over rotating buffers, 1 / 8 parts: 1024 rows of
+        # 65536 93.5 / 101 us, 4096 rows of 16384 94.5 / 99; but 64 rows of
+        # 2^20 183 / 102 and one row 138 / 104)
+        base_tiles = n // (_BLOCK * vec * trips)
+        if not _tuning.get('scan_chain_parts'):
+            parts = min(parts, 1 if base_tiles <= 16 else 2 if base_tiles <= 64
+                        else 4 if base_tiles <= 128 else 8)
+        parts = max(1, min(parts, base_tiles))
         tile = _BLOCK * vec * trips * parts
     tiles_per_row = (n + tile - 1) // tile
     n_tiles = n_rows * tiles_per_row
-    if n_tiles < 2 or n_tiles * _BLOCK > 0xffffffff:
+    if n_tiles < 2 or n_tiles * _BLOCK > 0xffffffff or n < _BLOCK * vec * trips:
         return False
     # groups of about sqrt(tiles per row) tiles: a tile then reads about
     # 2 sqrt(tiles per row) published totals
@@ -1512,8 +1522,9 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         # up to a dozen rounds)
         if may_chunk and group == _WAVE and outer < want and n > 12 * per_group:
             n_chunks = min((want + outer - 1) // outer, (n + per_group - 1) // per_group)
-        if n_chunks > 1 and _scan_chained(src, dst, outer, n, op, skip_nan, vec, idx64, stream,
-                                          stream_ptr):
+        long_rows = n * in_dtype.itemsize >= _tuning.get('scan_chain_min_row_bytes')
+        if (n_chunks > 1 or long_rows) and _scan_chained(
+                src, dst, outer, n, op, skip_nan, vec, idx64, stream, stream_ptr):
             return
         chunk_len = (n + n_chunks - 1) // n_chunks
         chunk_len = (chunk_len + per_group - 1) // per_group * per_group

@@ -91,6 +91,12 @@ _params = {
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
     'scan_cols_trips': 0,       # rows a thread of the column kernel requests at a time (0: by shape)
+    # Rows from this length on take that kernel however many there are: a
+    # workgroup per tile with all of it requested at once, instead of a wave
+    # that walks the row round by round (2^26 float32 over rotating buffers:
+    # rows of 8192 104 -> 91 us, rows of 4096 98 -> 87; rows of 2048 stay with
+    # the wave, 89 us)
+    'scan_chain_min_row_bytes': 16384,
     'scan_chain': True,         # a few long rows: one pass, tiles chained through published totals
     'scan_chain_parts': 0,      # ... a wave holds this many times 4 vectors per lane of its tile
                                 # (0: by the size of the input)
