@@ -208,8 +208,8 @@ def build_next_cases(cp):
 
     rng = np.random.default_rng(11)
     # ---- scans ------------------------------------------------------------------------
-    for shape, axis in (((1 << 20, 64), 1), ((8192, 8192), 1), ((64, 1 << 20), 0),
-                        ((1 << 26,), 0)):
+    for shape, axis in (((1 << 20, 64), 1), ((8192, 8192), 1), ((8192, 8192), 0),
+                        ((64, 1 << 20), 0), ((1 << 26,), 0)):
         a = rng.standard_normal(shape, dtype=np.float32)
         da = cp.asarray(a)
         out = cp.empty(shape, np.float32)

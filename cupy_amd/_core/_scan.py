@@ -1273,6 +1273,274 @@ def _module_chain_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inn
     return mod
 
 
+def _emit_chain_cols(in_t, out_t, op, skip_nan, vec, trips, idx64, waves, stream, sleep):
+    """One-pass scan along the middle axis of (outer, n, inner) where the
+    columns are many and long but too few to give every thread a column of its
+    own: a workgroup per tile of WAVES x TRIPS rows by 64 x VEC columns.  A
+    lane owns VEC adjacent columns and TRIPS consecutive rows of them, which it
+    keeps as loaded: it adds them up for the totals, and once more, from what
+    precedes it, for the results.  Tiles publish their totals per column and
+    fold those of the tiles above them as in ``_emit_chain`` (slots, waits and
+    an order of combination fixed by the tile's number); tiles are numbered
+    row of tiles by row of tiles, so that a tile only ever waits for smaller
+    numbers."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define WAVES %(waves)d
+#define HALF (WAVES / 2)
+#define COLS_T (64 * VEC)
+#define TILE_ROWS (WAVES * TRIPS)
+#define HEADER_WORDS %(header)d
+#define SPIN_SLEEP %(sleep)d
+#define FOLD_AHEAD 4
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+
+// Published values: see the one-pass kernel for contiguous rows.  Value
+// `i * COLS_T + c` belongs to column c of tile (or group) i.
+constexpr int kWords = (sizeof(_acc_t) + 3) / 4;
+typedef unsigned long long _slot_t;
+
+__device__ __forceinline__ void _publish(_slot_t* slots, const ptrdiff_t i, const _acc_t& v,
+                                         const unsigned epoch) {
+  unsigned w[kWords];
+#pragma unroll
+  for (int k = 0; k < kWords; ++k) w[k] = 0u;
+  __builtin_memcpy(w, &v, sizeof(_acc_t));
+#pragma unroll
+  for (int k = 0; k < kWords; ++k)
+    __hip_atomic_store(slots + i * kWords + k, ((_slot_t)epoch << 32) | w[k], __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The values `first + j * stride + k` (j < count, k < VEC) of a lane's own
+// columns, waited for and combined over j in order.  A lane asks for
+// FOLD_AHEAD values of j at a time.  One wave, all lanes call (`count` is 0
+// for a lane without columns); `ok` turns false if the wave gave up after
+// `spin_limit` rounds of polling.
+__device__ __forceinline__ void _await_fold_cols(
+    _slot_t* slots, const ptrdiff_t first, const ptrdiff_t stride, const int count,
+    const unsigned epoch, const unsigned spin_limit, bool& ok, _acc_t (&s)[VEC]) {
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) s[k] = SCAN_IDENTITY;
+  int i = 0;
+  unsigned spins = 0;
+  for (;;) {
+    while (i < count) {
+      _slot_t x[FOLD_AHEAD][VEC * kWords];
+#pragma unroll
+      for (int a = 0; a < FOLD_AHEAD; ++a) {
+        // (past the last value: the last one again, not used)
+        const int ia = (i + a < count) ? i + a : count - 1;
+        const _slot_t* at = slots + (first + (ptrdiff_t)ia * stride) * kWords;
+#pragma unroll
+        for (int m = 0; m < VEC * kWords; ++m)
+          x[a][m] = __hip_atomic_load(at + m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      bool stalled = false;
+#pragma unroll
+      for (int a = 0; a < FOLD_AHEAD; ++a) {
+        if (stalled || i >= count) break;
+        bool written = true;
+#pragma unroll
+        for (int m = 0; m < VEC * kWords; ++m)
+          written = written && (unsigned)(x[a][m] >> 32) == epoch;
+        if (!written) { stalled = true; break; }
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          unsigned w[kWords];
+#pragma unroll
+          for (int m = 0; m < kWords; ++m) w[m] = (unsigned)x[a][k * kWords + m];
+          _acc_t v;
+          __builtin_memcpy(&v, w, sizeof(_acc_t));
+          s[k] = (i == 0) ? v : SCAN_OP(s[k], v);
+        }
+        ++i;
+      }
+      if (stalled) break;
+    }
+    if (__ballot(i < count) == 0) break;
+    if (spins >= spin_limit) { ok = false; break; }
+    ++spins;
+    __builtin_amdgcn_s_sleep(SPIN_SLEEP);
+  }
+}
+
+// (launched with workgroups of any size up to the bound)
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_clear(
+    unsigned* desc, const unsigned words) {
+  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x)
+    desc[i] = 0u;
+}
+
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, unsigned* desc,
+    const _idx_t n_outer, const _idx_t n, const _idx_t inner, const _idx_t col_blocks,
+    const _idx_t row_tiles, const _idx_t group_tiles, const _idx_t groups_per_col,
+    const unsigned epoch, const unsigned spin_limit, unsigned* fault) {
+  __shared__ _acc_t sm_wave[WAVES][COLS_T];
+  __shared__ _acc_t sm_part[WAVES][COLS_T];
+  const ptrdiff_t n_tiles = (ptrdiff_t)n_outer * row_tiles * col_blocks;
+  _slot_t* tile_totals = reinterpret_cast<_slot_t*>(desc + HEADER_WORDS);
+  _slot_t* group_totals = tile_totals + n_tiles * COLS_T * kWords;
+  const int lane = threadIdx.x %% 64;
+  const int wv = threadIdx.x / 64;
+  const ptrdiff_t tile = blockIdx.x;
+  if (tile >= n_tiles) return;
+  const _idx_t cb = (_idx_t)(tile %% col_blocks);
+  const ptrdiff_t slab = tile / col_blocks;                  // (o, t_row)
+  const _idx_t t_row = (_idx_t)(slab %% row_tiles);
+  const _idx_t o = (_idx_t)(slab / row_tiles);
+  const _idx_t c0 = cb * COLS_T + lane * VEC;
+  const bool has_cols = c0 < inner;              // the host guarantees inner %% VEC == 0
+  const _idx_t r0 = t_row * TILE_ROWS + wv * TRIPS;          // this wave's first row
+  const ptrdiff_t at0 = ((ptrdiff_t)o * n + r0) * inner + c0;
+  // ---- the lane's rows as loaded, all requested at once
+  cupy::Vec<_in_t, VEC> raw[TRIPS];
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    if (has_cols && r0 + t < n) {
+      raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + at0 + (ptrdiff_t)t * inner);
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) raw[t].v[k] = _in_t();
+    }
+  }
+  // ---- totals: of the lane, of the waves above it, of the tile
+  _acc_t run[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) run[k] = SCAN_IDENTITY;
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    if (r0 + t < n) {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        run[k] = (t == 0) ? _load_value(raw[t].v[k]) : SCAN_OP(run[k], _load_value(raw[t].v[k]));
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) sm_wave[wv][k * 64 + lane] = run[k];
+  __syncthreads();
+  _acc_t wave_before[VEC], tile_total[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    wave_before[k] = SCAN_IDENTITY;
+    tile_total[k] = sm_wave[0][k * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      if (w == wv) wave_before[k] = tile_total[k];
+      tile_total[k] = SCAN_OP(tile_total[k], sm_wave[w][k * 64 + lane]);
+    }
+  }
+  // ---- what precedes the tile in its columns: the totals of the tiles above
+  // it in its group and of the groups above its own.  The first half of the
+  // waves shares out the former, the second half the latter (every wave a run
+  // of consecutive ones), so that the trips to memory overlap; the partial
+  // results are then combined in the order of the waves.
+  const _idx_t g = t_row / group_tiles;
+  const int t_group = (int)(t_row - g * group_tiles);
+  const bool closes_group = (t_group == group_tiles - 1) || (t_row == row_tiles - 1);
+  const ptrdiff_t tile_stride = (ptrdiff_t)col_blocks * COLS_T;   // values from a tile to the one below
+  if (wv == 0 && has_cols) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k)
+      _publish(tile_totals, tile * COLS_T + lane * VEC + k, tile_total[k], epoch);
+  }
+  const bool tiles_side = wv < HALF;
+  const int side_count = tiles_side ? t_group : (int)g;
+  const int per_wave = (side_count + HALF - 1) / HALF;
+  {
+    const int j0 = (tiles_side ? wv : wv - HALF) * per_wave;
+    int mine = side_count - j0;
+    mine = mine < 0 ? 0 : (mine > per_wave ? per_wave : mine);
+    const ptrdiff_t first =
+        (tiles_side ? (tile - (ptrdiff_t)t_group * col_blocks) * COLS_T
+                    : (((ptrdiff_t)o * groups_per_col) * col_blocks + cb) * COLS_T)
+        + lane * VEC + (ptrdiff_t)j0 * tile_stride;
+    bool ok = true;
+    _acc_t part[VEC];
+    _await_fold_cols(tiles_side ? tile_totals : group_totals, first, tile_stride,
+                     has_cols ? mine : 0, epoch, spin_limit, ok, part);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) sm_part[wv][k * 64 + lane] = part[k];
+    if (!ok && lane == 0 && fault) *reinterpret_cast<volatile unsigned*>(fault) = 1u;
+  }
+  __syncthreads();
+  const int per_tiles = (t_group + HALF - 1) / HALF;
+  const int per_groups = ((int)g + HALF - 1) / HALF;
+  const bool seeded = t_row > 0 || wv > 0;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    _acc_t in_group = SCAN_IDENTITY, groups_before = SCAN_IDENTITY;
+#pragma unroll
+    for (int w = 0; w < HALF; ++w) {
+      if (w * per_tiles < t_group)
+        in_group = (w == 0) ? sm_part[w][k * 64 + lane] : SCAN_OP(in_group, sm_part[w][k * 64 + lane]);
+      if (w * per_groups < (int)g)
+        groups_before = (w == 0) ? sm_part[HALF + w][k * 64 + lane]
+                                 : SCAN_OP(groups_before, sm_part[HALF + w][k * 64 + lane]);
+    }
+    if (wv == 0 && has_cols && closes_group)
+      _publish(group_totals,
+               (((ptrdiff_t)o * groups_per_col + g) * col_blocks + cb) * COLS_T + lane * VEC + k,
+               (t_group > 0) ? SCAN_OP(in_group, tile_total[k]) : tile_total[k], epoch);
+    _acc_t base = SCAN_IDENTITY;
+    if (g > 0) base = groups_before;
+    if (t_group > 0) base = (g > 0) ? SCAN_OP(base, in_group) : in_group;
+    if (wv > 0) base = (t_row > 0) ? SCAN_OP(base, wave_before[k]) : wave_before[k];
+    run[k] = base;
+  }
+  // ---- results
+  if (!has_cols) return;
+#pragma unroll
+  for (int t = 0; t < TRIPS; ++t) {
+    if (r0 + t < n) {
+      cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const _acc_t x = _load_value(raw[t].v[k]);
+        run[k] = (seeded || t > 0) ? SCAN_OP(run[k], x) : x;
+        r.v[k] = static_cast<_out_t>(run[k]);
+      }
+      cupy::store_vec<_out_t, VEC, NT_STORE>(out + at0 + (ptrdiff_t)t * inner, r);
+    }
+  }
+}
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=waves * _WAVE,
+           waves=waves, header=_CHAIN_HEADER_WORDS, sleep=sleep,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
+
+
+def _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, waves, stream):
+    sleep = _tuning.get('scan_chain_sleep')
+    key = ('chain cols', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan,
+           vec, trips, idx64, waves, stream, sleep)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_chain_cols(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                               vec, trips, idx64, waves, stream, sleep)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
 def _module_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream, reuse):
     key = ('tile', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
            trips, idx64, inner, stream, reuse)
@@ -1384,17 +1652,14 @@ def _chain_slots(dev_id, stream_ptr, words, mod):
         return arena[0], arena[1]
 
 
-def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_ptr, inner=1):
-    """The one-pass scan of a few long rows (``_emit_chain``) or, with
-    ``inner`` > 1, of a few long slices of rows of ``inner`` elements scanned
-    down their columns (``_emit_chain_tile``): input read once, output written
-    once.  Returns False where it does not apply (the caller then takes the
-    three-pass route)."""
+def _chain_ready():
+    """(device id, address of the device's fault word) if the one-pass kernels
+    may be used, else None."""
     if not _tuning.get('scan_chain'):
-        return False
+        return None
     dev_id = _device.get_device_id()
     if dev_id in _chain_disabled:
-        return False
+        return None
     fault = _chain_fault_word(dev_id)
     if fault and ctypes.c_uint32.from_address(fault).value:
         # A tile of an earlier scan gave up waiting for the tiles before it and
@@ -1406,6 +1671,19 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
             'an earlier one-pass scan on device %d gave up waiting for its neighbouring '
             'tiles: its result is wrong.  Scans use the three-pass kernels from now on.'
             % dev_id)
+    return dev_id, fault
+
+
+def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_ptr, inner=1):
+    """The one-pass scan of a few long rows (``_emit_chain``) or, with
+    ``inner`` > 1, of a few long slices of rows of ``inner`` elements scanned
+    down their columns (``_emit_chain_tile``): input read once, output written
+    once.  Returns False where it does not apply (the caller then takes the
+    three-pass route)."""
+    ready = _chain_ready()
+    if ready is None:
+        return False
+    dev_id, fault = ready
     in_dtype, out_dtype = src.dtype, dst.dtype
     trips = 4
     parts = _tuning.get('scan_chain_parts')
@@ -1466,6 +1744,65 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
                        _tuning.get('scan_chain_spin_limit'), fault)
     mod.get_function(name).launch_packed(
         (n_tiles, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+    return True
+
+
+def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr):
+    """The one-pass scan down many long columns (``_emit_chain_cols``).  Returns
+    False where it does not apply."""
+    if not _tuning.get('scan_chain_cols'):
+        return False
+    ready = _chain_ready()
+    if ready is None:
+        return False
+    dev_id, fault = ready
+    in_dtype, out_dtype = src.dtype, dst.dtype
+    acc_item = _acc_dtype(out_dtype).itemsize
+    item = max(in_dtype.itemsize, out_dtype.itemsize, acc_item)
+    # Vectors of 8 bytes, or of 4 where those would leave many lanes of the
+    # last block of columns idle; a workgroup of 16 waves, each lane keeping
+    # 256 bytes of its columns.  (2^26 float32 over rotating buffers, us, for
+    # 8192 x 8192 / 16 x 4096 x 1024 / 262144 x 256: 16 waves, 8-byte vectors,
+    # 32 rows a lane 97 / 112 / 110; 8 waves 99 / 110 / 110; 4 waves 105 / 126
+    # / 147; 16-byte vectors with 4 waves and 32 rows 122 / 152 / 188.  The
+    # three-pass kernels: 145 / 149 / 169.)
+    best = None
+    forced = _tuning.get('scan_chain_cols_vec_bytes')
+    for vec_bytes in ((forced,) if forced else (8, 4)):
+        v = max(1, vec_bytes // item)
+        while v > 1 and (not _aligned(src.data.ptr, v * in_dtype.itemsize)
+                         or not _aligned(dst.data.ptr, v * out_dtype.itemsize)
+                         or inner % v):
+            v //= 2
+        cols_t = _WAVE * v
+        blocks = (inner + cols_t - 1) // cols_t
+        used = inner / (blocks * cols_t)
+        if best is None or used > best[0] + 0.1:
+            best = (used, v, blocks)
+    _, vec, col_blocks = best
+    waves = max(2, min(16, _tuning.get('scan_chain_cols_waves')))
+    trips = _tuning.get('scan_chain_cols_trips') or max(4, min(64, 256 // (vec * item)))
+    tile_rows = waves * trips
+    row_tiles = (n + tile_rows - 1) // tile_rows
+    n_tiles = outer * row_tiles * col_blocks
+    if row_tiles < 2 or n_tiles * waves * _WAVE > 0xffffffff:
+        return False
+    # groups of about sqrt(tiles down a column) tiles
+    group_tiles = max(2, 1 << (row_tiles.bit_length() // 2))
+    groups_per_col = (row_tiles + group_tiles - 1) // group_tiles
+    n_groups = outer * groups_per_col * col_blocks
+    words_per_value = (acc_item + 3) // 4
+    desc_words = _CHAIN_HEADER_WORDS + 2 * words_per_value * _WAVE * vec * (n_tiles + n_groups)
+    if desc_words > 0x7fffffff:
+        return False
+    mod = _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, waves, stream)
+    desc, epoch = _chain_slots(dev_id, stream_ptr, desc_words, mod)
+    ic = 'q' if idx64 else 'i'
+    blob = struct.pack('@PPP' + ic * 7 + 'IIP', src.data.ptr, dst.data.ptr, desc.data.ptr,
+                       outer, n, inner, col_blocks, row_tiles, group_tiles, groups_per_col,
+                       epoch, _tuning.get('scan_chain_spin_limit'), fault)
+    mod.get_function('cupy_scan_chain_cols').launch_packed(
+        (n_tiles, 1, 1), (waves * _WAVE, 1, 1), blob, 0, stream_ptr)
     return True
 
 
@@ -1582,6 +1919,9 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         n_chunks = 1
         if may_chunk and outer < want and n > 2 * per_wave:
             n_chunks = min((want + outer - 1) // outer, (n + per_wave - 1) // per_wave)
+        if n_chunks > 1 and _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64,
+                                               stream, stream_ptr):
+            return
         chunk_len = (n + n_chunks - 1) // n_chunks
         chunk_len = (chunk_len + per_wave - 1) // per_wave * per_wave
         n_chunks = (n + chunk_len - 1) // chunk_len
@@ -1601,25 +1941,56 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         totals_shape = (outer, n_chunks, inner)
         middle_round = per_wave
     else:
-        vec = max(1, 16 // item)
-        while vec > 1 and (not _aligned(src.data.ptr, vec * in_dtype.itemsize)
-                           or not _aligned(dst.data.ptr, vec * out_dtype.itemsize)
-                           or inner % vec):
-            vec //= 2
-        threads = outer * (inner // vec)
-        want = cus * 1024
+        # A thread owns ``vec`` adjacent columns and walks down them, ``trips``
+        # rows requested at a time.  Wide vectors need many columns to give
+        # every CU its waves; narrower ones with more rows in flight keep a
+        # narrow array in one pass (two transfers per element) where cutting
+        # the rows into chunks costs three.  2^26 float32 over rotating
+        # buffers, us: 64 x 2^20 16-byte vectors 32 rows 92 (16 rows 98, 4
+        # rows 115); 256 x 2^18 8-byte vectors 32 rows 89 (16-byte 8 rows 95,
+        # 32 rows 141, chunked 131); 1024 x 2^16 4-byte vectors 64 rows 104 (32
+        # rows 125, chunked 128).  Below 256 threads per CU the rows are cut
+        # into chunks: 4096 x 2^14 135 with 8 rows at a time.
+        def threads_with(vec_bytes):
+            v = max(1, vec_bytes // item)
+            while v > 1 and (not _aligned(src.data.ptr, v * in_dtype.itemsize)
+                             or not _aligned(dst.data.ptr, v * out_dtype.itemsize)
+                             or inner % v):
+                v //= 2
+            return v, outer * (inner // v)
+        forced = _tuning.get('scan_cols_vec_bytes')
+        per_cu = _tuning.get('scan_cols_threads_per_cu')
+        one_pass_trips = 0
+        if forced:
+            vec, threads = threads_with(forced)
+        else:
+            for vec_bytes, need, rows in ((16, 2 * per_cu, 32), (8, 2 * per_cu, 32),
+                                          (max(4, min(item, 8)), per_cu, 64)):
+                if vec_bytes < item and vec_bytes != 16:
+                    continue
+                vec, threads = threads_with(vec_bytes)
+                if threads >= cus * need:
+                    one_pass_trips = rows
+                    break
+            else:
+                vec, threads = threads_with(16)
+        want = cus * per_cu
         n_chunks = 1
-        if may_chunk and threads < want and n >= 128:
+        if may_chunk and not one_pass_trips and threads < want and n >= 128:
             n_chunks = min((want + threads - 1) // threads, n // 64)
+        if n_chunks > 1 and _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64,
+                                               stream, stream_ptr):
+            return
         chunk_len = (n + n_chunks - 1) // n_chunks
         n_chunks = (n + chunk_len - 1) // chunk_len
-        # Rows a thread requests at a time.  Enough threads for one pass: many
-        # (64 x 2^20 float32 along axis 0: 98 us with 4, 96 with 8, 83 with
-        # 16); chunked, every thread has few rows and more only costs
-        # registers (16 x 4096 x 1024 along axis 1: 136 us with 4, 149 with 16).
         trips = _tuning.get('scan_cols_trips')
         if not trips:
-            trips = 16 if n_chunks == 1 and n >= 32 else 4
+            if n_chunks > 1:
+                trips = 8
+            else:
+                trips = one_pass_trips or 32
+                while trips > 4 and trips > n:
+                    trips //= 2
         mod = _module(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, 64, stream,
                       reuse=n_chunks > 1 and reuse_ok)
         work = threads * n_chunks

@@ -90,6 +90,12 @@ _params = {
     'scan_stream': 'auto',      # non-temporal hints of the scan kernels
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
+    'scan_cols_threads_per_cu': 256,   # column scans are cut into chunks below this many threads per CU
+    'scan_cols_vec_bytes': 0,
+    'scan_chain_cols': True,    # one-pass kernel for many long columns
+    'scan_chain_cols_waves': 16,
+    'scan_chain_cols_trips': 0,
+    'scan_chain_cols_vec_bytes': 0,
     'scan_cols_trips': 0,       # rows a thread of the column kernel requests at a time (0: by shape)
     # Rows from this length on take that kernel however many there are: a
     # workgroup per tile with all of it requested at once, instead of a wave

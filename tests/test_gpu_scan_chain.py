@@ -13,7 +13,9 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(autouse=True)
 def _restore():
     yield
-    _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0)
+    _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0,
+                scan_chain_cols=True, scan_chain_cols_waves=16, scan_chain_cols_trips=0,
+                scan_chain_cols_vec_bytes=0)
     _scan._chain_disabled.clear()
 
 
@@ -214,3 +216,116 @@ def test_scans_on_two_streams_at_once():
     # nothing gave up on the way
     d = cp.asarray(ha)
     assert 'cupy_scan_chain' in launched(lambda: d.cumsum())
+
+
+# ---- many long columns: tiles of rows x columns, totals published per column
+
+def within(got, want, bound):
+    off = np.abs(got - want) > bound
+    if off.any():
+        where = np.argwhere(off)
+        first = tuple(where[0])
+        raise AssertionError('%d values out of bound, first at %s: got %r, expected %r; rows %s, '
+                             'columns %s' % (len(where), first, got[first], want[first],
+                                             sorted(set(where[:, -2].tolist()))[:8],
+                                             sorted(set(where[:, -1].tolist()))[:8]))
+
+
+@pytest.mark.parametrize('shape,axis', [
+    ((8192, 2048), 0),            # whole blocks of columns, whole tiles of rows
+    ((5000, 1000), 0),            # ragged on both sides
+    ((3, 3001, 516), 1),          # several slices
+    ((70001, 100), 0),            # many tiles down a column, the last block of columns part empty
+    ((1029, 4098), 0),            # the last tile holds few rows
+    ((40000, 37), 0),             # odd row length: single-element vectors
+])
+def test_many_long_columns_in_one_pass(shape, axis):
+    rng = np.random.default_rng(shape[-1])
+    h = rng.integers(-5, 6, shape).astype(np.int32)
+    d = cp.asarray(h)
+    assert launched(lambda: d.cumsum(axis=axis))[-1] == 'cupy_scan_chain_cols'
+    assert_exact(d.cumsum(axis=axis).get(), h.cumsum(axis=axis))
+    hf = rng.uniform(0, 1, shape).astype(np.float32)
+    df = cp.asarray(hf)
+    got = df.cumsum(axis=axis).get()
+    want = np.cumsum(hf.astype(np.float64), axis=axis)
+    assert (np.abs(got - want) <= 1e-5 * want + 1e-6).all()
+    assert_exact(df.cumsum(axis=axis).get(), got)                 # same bits on every run
+    other = three_pass(lambda: df.cumsum(axis=axis).get())
+    assert (np.abs(got - other) <= 2e-5 * want + 1e-6).all()
+
+
+@pytest.mark.parametrize('waves,trips,vec_bytes', [(16, 0, 0), (8, 8, 16), (2, 64, 4), (16, 4, 8),
+                                                   (4, 16, 8)])
+def test_long_columns_other_types_and_tile_shapes(waves, trips, vec_bytes):
+    _tuning.set(scan_chain_cols_waves=waves, scan_chain_cols_trips=trips,
+                scan_chain_cols_vec_bytes=vec_bytes)
+    rng = np.random.default_rng(waves * 100 + trips)
+    h8 = rng.integers(-100, 100, (30001, 200)).astype(np.int8)
+    d8 = cp.asarray(h8)
+    assert launched(lambda: cp.cumsum(d8, axis=0))[-1] == 'cupy_scan_chain_cols'
+    assert_exact(cp.cumsum(d8, axis=0).get(), np.cumsum(h8, axis=0))
+    hd = rng.standard_normal((9000, 300))
+    got = cp.cumsum(cp.asarray(hd), axis=0).get()
+    within(got, np.cumsum(hd, axis=0), 1e-13 * np.cumsum(np.abs(hd), axis=0))
+    hc = (rng.standard_normal((2, 7001, 130)) + 1j * rng.standard_normal((2, 7001, 130)))
+    got = cp.cumsum(cp.asarray(hc), axis=1).get()
+    within(got, np.cumsum(hc, axis=1), 1e-13 * np.cumsum(np.abs(hc), axis=1))
+    hh = rng.uniform(0, 1, (6000, 256)).astype(np.float16)
+    got = cp.cumsum(cp.asarray(hh), axis=0).get().astype(np.float64)
+    want = np.cumsum(hh.astype(np.float64), axis=0)
+    assert (np.abs(got - want) <= 2e-3 * want + 1e-3).all()
+    hp = np.ones((20000, 96), np.int64)
+    hp[rng.choice(20000, 30, replace=False), rng.integers(0, 96, 30)] = rng.choice([-1, 2], 30)
+    assert_exact(cp.cumprod(cp.asarray(hp), axis=0).get(), np.cumprod(hp, axis=0))
+    hn = rng.uniform(0, 1, (25000, 160)).astype(np.float32)
+    hn[::777, 1::7] = np.nan
+    got = cp.nancumsum(cp.asarray(hn), axis=0).get()
+    want = np.nancumsum(hn.astype(np.float64), axis=0)
+    assert (np.abs(got - want) <= 1e-5 * want + 1e-6).all()
+    # negative zeros survive: nothing is added to the first row
+    hz = np.full((5000, 128), -0.0, np.float32)
+    assert_exact(cp.cumsum(cp.asarray(hz), axis=0).get(), np.cumsum(hz, axis=0))
+    # a view that starts off the 16-byte grid
+    hv = rng.integers(-5, 6, 4000 * 256 + 1).astype(np.int32)
+    assert_exact(cp.asarray(hv)[1:].reshape(4000, 256).cumsum(axis=0).get(),
+                 hv[1:].reshape(4000, 256).cumsum(axis=0))
+
+
+def test_a_column_tile_that_gives_up_is_reported():
+    rng = np.random.default_rng(8)
+    h = rng.integers(-5, 6, (1 << 15, 512)).astype(np.int32)
+    d = cp.asarray(h)
+    _tuning.set(scan_chain_spin_limit=0)
+    d.cumsum(axis=0)
+    cp.cuda.Device().synchronize()
+    _tuning.set(scan_chain_spin_limit=1 << 18)
+    with pytest.raises(RuntimeError, match='gave up waiting'):
+        d.cumsum(axis=0)
+    names = launched(lambda: d.cumsum(axis=0))
+    assert 'cupy_scan_chain_cols' not in names
+    assert_exact(d.cumsum(axis=0).get(), h.cumsum(axis=0))
+
+
+def test_slots_of_a_new_stream_start_cleared_whatever_the_memory_held():
+    """The first launch on a stream gets fresh memory for its published
+    totals, which must be cleared whole: here the pool hands back a block
+    filled with what looks like totals marked with the number of that very
+    launch."""
+    rng = np.random.default_rng(21)
+    h = rng.integers(-5, 6, (20000, 512)).astype(np.int32)
+    d = cp.asarray(h)
+    _scan._chain_arenas.clear()
+    assert launched(lambda: d.cumsum(axis=0))[-1] == 'cupy_scan_chain_cols'
+    (arena,) = _scan._chain_arenas.values()
+    words = arena[0].size
+    del arena
+    cp.cuda.Device().synchronize()
+    _scan._chain_arenas.clear()
+    junk = cp.empty(words // 2, np.uint64)
+    junk[...] = (1 << 32) | 0x12345678
+    cp.cuda.Device().synchronize()
+    del junk
+    assert_exact(d.cumsum(axis=0).get(), h.cumsum(axis=0))
+    (arena,) = _scan._chain_arenas.values()
+    assert arena[1] == 1 and arena[0].size == words
