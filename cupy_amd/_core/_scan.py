@@ -1273,7 +1273,8 @@ def _module_chain_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inn
     return mod
 
 
-def _emit_chain_cols(in_t, out_t, op, skip_nan, vec, trips, idx64, waves, stream, sleep):
+def _emit_chain_cols(in_t, out_t, op, skip_nan, vec, trips, idx64, waves, stream, sleep,
+                     ahead=2):
     """One-pass scan along the middle axis of (outer, n, inner) where the
     columns are many and long but too few to give every thread a column of its
     own: a workgroup per tile of WAVES x TRIPS rows by 64 x VEC columns.  A
@@ -1308,7 +1309,7 @@ typedef %(idx_t)s _idx_t;
 #define TILE_ROWS (WAVES * TRIPS)
 #define HEADER_WORDS %(header)d
 #define SPIN_SLEEP %(sleep)d
-#define FOLD_AHEAD 4
+#define FOLD_AHEAD %(ahead)d
 __device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
 
 // Published values: see the one-pass kernel for contiguous rows.  Value
@@ -1399,23 +1400,24 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
   _slot_t* tile_totals = reinterpret_cast<_slot_t*>(desc + HEADER_WORDS);
   _slot_t* group_totals = tile_totals + n_tiles * COLS_T * kWords;
   const int lane = threadIdx.x %% 64;
-  const int wv = threadIdx.x / 64;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const ptrdiff_t tile = blockIdx.x;
   if (tile >= n_tiles) return;
   const _idx_t cb = (_idx_t)(tile %% col_blocks);
   const ptrdiff_t slab = tile / col_blocks;                  // (o, t_row)
   const _idx_t t_row = (_idx_t)(slab %% row_tiles);
   const _idx_t o = (_idx_t)(slab / row_tiles);
-  const _idx_t c0 = cb * COLS_T + lane * VEC;
-  const bool has_cols = c0 < inner;              // the host guarantees inner %% VEC == 0
+  const int lc = lane * VEC;                     // the lane's first column within the block
+  const bool has_cols = cb * COLS_T + lc < inner;            // the host guarantees inner %% VEC == 0
   const _idx_t r0 = t_row * TILE_ROWS + wv * TRIPS;          // this wave's first row
-  const ptrdiff_t at0 = ((ptrdiff_t)o * n + r0) * inner + c0;
+  // (the same for all lanes of a wave: the lanes differ by `lc` alone)
+  const ptrdiff_t at0 = ((ptrdiff_t)o * n + r0) * inner + (ptrdiff_t)cb * COLS_T;
   // ---- the lane's rows as loaded, all requested at once
   cupy::Vec<_in_t, VEC> raw[TRIPS];
 #pragma unroll
   for (int t = 0; t < TRIPS; ++t) {
     if (has_cols && r0 + t < n) {
-      raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + at0 + (ptrdiff_t)t * inner);
+      raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + at0 + (ptrdiff_t)t * inner + lc);
     } else {
 #pragma unroll
       for (int k = 0; k < VEC; ++k) raw[t].v[k] = _in_t();
@@ -1517,13 +1519,13 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
         run[k] = (seeded || t > 0) ? SCAN_OP(run[k], x) : x;
         r.v[k] = static_cast<_out_t>(run[k]);
       }
-      cupy::store_vec<_out_t, VEC, NT_STORE>(out + at0 + (ptrdiff_t)t * inner, r);
+      cupy::store_vec<_out_t, VEC, NT_STORE>(out + at0 + (ptrdiff_t)t * inner + lc, r);
     }
   }
 }
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
            op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=waves * _WAVE,
-           waves=waves, header=_CHAIN_HEADER_WORDS, sleep=sleep,
+           waves=waves, header=_CHAIN_HEADER_WORDS, sleep=sleep, ahead=ahead,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
 
 
@@ -1533,8 +1535,11 @@ def _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, wav
            vec, trips, idx64, waves, stream, sleep)
     mod = _memo.get(key)
     if mod is None:
+        # published totals a lane asks for at a time: what the registers of
+        # a lane in a workgroup of 16 waves hold beside its rows
+        ahead = 4 if (in_dtype.itemsize == 4 and _acc_dtype(out_dtype).itemsize * vec <= 8) else 2
         src = _emit_chain_cols(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
-                               vec, trips, idx64, waves, stream, sleep)
+                               vec, trips, idx64, waves, stream, sleep, ahead)
         mod = compiler.compile_with_cache(src)
         with _lock:
             mod = _memo.setdefault(key, mod)
@@ -1781,7 +1786,7 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
             best = (used, v, blocks)
     _, vec, col_blocks = best
     waves = max(2, min(16, _tuning.get('scan_chain_cols_waves')))
-    trips = _tuning.get('scan_chain_cols_trips') or max(4, min(64, 256 // (vec * item)))
+    trips = _tuning.get('scan_chain_cols_trips') or max(4, min(64, (256 if item < 16 else 128) // (vec * item)))
     tile_rows = waves * trips
     row_tiles = (n + tile_rows - 1) // tile_rows
     n_tiles = outer * row_tiles * col_blocks
