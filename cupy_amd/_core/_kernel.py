@@ -956,6 +956,9 @@ class _ElementwisePlanner:
         else:
             tile_r = tile_c = 64
             threads = 256
+        forced = _tuning.get('tiled_tile')
+        if forced and n_transposed:
+            tile_r, tile_c, threads = forced
         if n_transposed == 0:
             # Nothing is staged: every operand runs along the columns, so the
             # tile is made as wide as divides the row length (up to one vector

@@ -52,7 +52,8 @@ _params = {
     # tiled 2-d elementwise kernel
     'tiled_stream': 'auto',
     'tiled_batch_first': True,  # batched tiles: near batch entries before far rows
-    'tiled_big_min': 512,       # extent of both tile axes from which tiles are 128 x 128
+    'tiled_tile': None,         # (rows, columns, threads) of a staged tile; None: by shape
+    'tiled_big_min': 256,       # extent of both tile axes from which tiles are 128 x 128
     'cache_bytes': 256 << 20,   # capacity of the memory-side cache (Infinity Cache)
     # reductions
     'rows_stream': True,       # non-temporal loads: True / False / 'auto' (by footprint);
