@@ -595,6 +595,170 @@ TILE_KERNEL(cupy_scan_tile_seeded, 2)
            reuse=1 if reuse else 0)
 
 
+def _emit_tile_packed(in_t, out_t, op, skip_nan, vec, trips, idx64, inner, stream):
+    """Scan along the middle axis of (outer, n, inner) for 2 <= inner <= 32 and
+    slices so short that many fit the rows a wave stages per round: the
+    staging of ``_emit_tile``, with the (outer x n) rows taken as one long run
+    cut into rounds of whole slices.  The scan starts over wherever a slice
+    starts: inside a lane's own rows, and -- through a flag that travels with
+    the running values -- in the combination across the lanes.  Rounds are
+    independent of one another: nothing is carried from round to round."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    rows_t, seg, lrows, stride = _tile_geometry(inner, vec, trips)
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define INNER %(inner)d
+#define ROWS_T %(rows_t)d
+#define SEG %(seg)d
+#define LROWS %(lrows)d
+#define SEG_STRIDE %(stride)d
+#define LDS_WORDS (SEG * SEG_STRIDE)
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+// position in the LDS of element p of the round (p = row * INNER + column)
+__device__ __forceinline__ int _lds_at(int p) { return p + (p / (LROWS * INNER)) * (SEG_STRIDE - LROWS * INNER); }
+
+// total_rows = outer * n rows of INNER elements; a round is round_rows of them,
+// a multiple of n not above ROWS_T (so that every round starts a slice).
+extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_tile_packed(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, const _idx_t total_rows,
+    const int n, const int round_rows) {
+  __shared__ _acc_t _lds_all[%(block)d / 64][LDS_WORDS];
+  _acc_t* lds = _lds_all[threadIdx.x / 64];
+  const int lane = threadIdx.x %% 64;
+  const int seg = lane / INNER;
+  const int col = lane - seg * INNER;
+  const bool active = lane < SEG * INNER;
+  // where the lane's rows start over (the same in every round): bit i is set
+  // if its row i is the first of a slice
+  unsigned long long starts = 0ull;      // (LROWS <= 64)
+  {
+    int j = (seg * LROWS) %% n;
+#pragma unroll
+    for (int i = 0; i < LROWS; ++i) {
+      if (j == 0) starts |= 1ull << i;
+      j = (j + 1 == n) ? 0 : j + 1;
+    }
+  }
+  const _idx_t n_rounds = (total_rows + round_rows - 1) / round_rows;
+  const _idx_t wave_step = (_idx_t)gridDim.x * (%(block)d / 64);
+  for (_idx_t w = (_idx_t)blockIdx.x * (%(block)d / 64) + threadIdx.x / 64; w < n_rounds;
+       w += wave_step) {
+    const _idx_t rb = w * round_rows;
+    const int rows_here = (total_rows - rb < round_rows) ? (int)(total_rows - rb) : round_rows;
+    const int valid = rows_here * INNER;
+    const _in_t* src = in + (ptrdiff_t)rb * INNER;
+    _out_t* dst = out + (ptrdiff_t)rb * INNER;
+    // every load of the round is requested before the first value is used
+    cupy::Vec<_in_t, VEC> raw[TRIPS];
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * 64 + lane) * VEC;
+      if (p + VEC <= valid) {
+        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + p);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) raw[t].v[k] = (p + k < valid) ? src[p + k] : _in_t();
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * 64 + lane) * VEC;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        if (p + k < ROWS_T * INNER)
+          lds[_lds_at(p + k)] = (p + k < valid) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // the lane's own rows of its column, scanned in registers
+    _acc_t v[LROWS];
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < LROWS; ++i) v[i] = lds[seg * SEG_STRIDE + i * INNER + col];
+#pragma unroll
+      for (int i = 1; i < LROWS; ++i) v[i] = ((starts >> i) & 1ull) ? v[i] : SCAN_OP(v[i - 1], v[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < LROWS; ++i) v[i] = SCAN_IDENTITY;
+    }
+    // what runs into the next segment of the column: the lane's last value,
+    // and whether a slice started inside the lane (then nothing from the
+    // segments before passes through it)
+    _acc_t run = v[LROWS - 1];
+    bool cut = starts != 0ull;
+#pragma unroll
+    for (int d = 1; d < SEG; d <<= 1) {
+      const _acc_t other = cupy::shfl_up<64>(run, d * INNER);
+      const int other_cut = cupy::shfl_up<64>((int)cut, d * INNER);
+      if (lane >= d * INNER) {
+        run = cut ? run : SCAN_OP(other, run);
+        cut = cut || other_cut != 0;
+      }
+    }
+    const _acc_t before = cupy::shfl_up<64>(run, INNER);
+    if (active) {
+      // rows before the lane's first start continue the segments before it
+      bool open = seg > 0;
+#pragma unroll
+      for (int i = 0; i < LROWS; ++i) {
+        open = open && !((starts >> i) & 1ull);
+        lds[seg * SEG_STRIDE + i * INNER + col] = open ? SCAN_OP(before, v[i]) : v[i];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * 64 + lane) * VEC;
+      if (p + VEC <= valid) {
+        cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(lds[_lds_at(p + k)]);
+        cupy::store_vec<_out_t, VEC, NT_STORE>(dst + p, r);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          if (p + k < valid) dst[p + k] = static_cast<_out_t>(lds[_lds_at(p + k)]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           inner=inner, rows_t=rows_t, seg=seg, lrows=lrows, stride=stride,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
+
+
+def _module_tile_packed(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inner, stream):
+    key = ('tile packed', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan,
+           vec, trips, idx64, inner, stream)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_tile_packed(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                                vec, trips, idx64, inner, stream)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
 _CHAIN_WAVES = _BLOCK // _WAVE
 _CHAIN_HEADER_WORDS = 64            # the ticket counter, padded to 256 bytes
 
@@ -1890,6 +2054,31 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         vec = max(1, 16 // item)
         trips = 4
         rows_t, _, _, _ = _tile_geometry(inner, vec, trips)
+        if 4 * n <= rows_t and outer > 1 and _tuning.get('scan_tile_packed'):
+            # Slices of few rows: many to a round.  (2^26 float32 as 2^22
+            # slices of 4 x 4: 1190 us with a wave per slice; 2^21 of 16 x 2:
+            # 697; 2^20 of 2 x 32: 278)
+            p_trips = trips
+            while _tile_geometry(inner, vec, p_trips)[2] > 32 and p_trips > 1:
+                p_trips //= 2       # (a lane marks the slice starts among its rows in 64 bits)
+            rows_p = _tile_geometry(inner, vec, p_trips)[0]
+        else:
+            rows_p = 0
+        # (with two slices to a round the plain kernel is as good: 2^17 slices
+        # of 32 x 16 floats 86.6 us against 91.5)
+        if 4 * n <= rows_p and _tile_geometry(inner, vec, p_trips)[2] <= 64:
+            round_rows = rows_p // n * n
+            mod = _module_tile_packed(in_dtype, out_dtype, op, skip_nan, vec, p_trips, idx64,
+                                      inner, stream)
+            rounds = (outer * n + round_rows - 1) // round_rows
+            per_block = _BLOCK // _WAVE
+            grid = max(1, min((rounds + per_block - 1) // per_block,
+                              cus * _tuning.get('scan_blocks_per_cu')))
+            blob = struct.pack('@PP' + ic + 'ii', src.data.ptr, dst.data.ptr, outer * n, n,
+                               round_rows)
+            mod.get_function('cupy_scan_tile_packed').launch_packed(
+                (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+            return
         want = cus * _tuning.get('scan_waves_per_cu')
         n_chunks = 1
         if may_chunk and outer < want and n > 2 * rows_t:
@@ -1915,7 +2104,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         prefix = 'cupy_scan_tile'
         totals_shape = (outer, n_chunks, inner)
         middle_round = rows_t
-    elif _lanes_geometry(src, dst, inner, item) is not None:
+    elif _tuning.get('scan_lanes') and _lanes_geometry(src, dst, inner, item) is not None:
         vec, lstride = _lanes_geometry(src, dst, inner, item)
         trips = 4
         trip_rows = _WAVE // lstride
@@ -2062,8 +2251,21 @@ def scan_core(a, axis, op, dtype=None, out=None, skip_nan=False):
         if may_share_bounds(a, out):
             src = a.copy()
     stream_ptr = _stream.get_current_stream_ptr()
-    _scan_contiguous(src, result, outer, n, inner, op, skip_nan and src.dtype.kind in 'fc',
-                     stream_ptr)
+    skip_nan = skip_nan and src.dtype.kind in 'fc'
+    if (op == _SUM and not skip_nan and src.dtype == numpy.complex128 and n >= 1024
+            and src.dtype == result.dtype and _tuning.get('scan_complex_as_real')):
+        # Sums of complex numbers are sums of their parts: long scans of
+        # complex128 go over the array as a real one with twice the columns
+        # (the same additions in the same order).  Values of 16 bytes leave the
+        # one-pass kernels at 35-50 % of peak: 2^24 in one dimension 190 us, as
+        # 2^24 x 2 doubles 118; 8192 rows of 2048 113-129 -> 101; 2^22 x 4 along
+        # axis 0 136 -> 106.  (Short rows and complex64 are as fast or faster
+        # as they are: 2^21 rows of 16 complex64 86 us, as 16 x 2 floats more.)
+        part = numpy.dtype('float64')
+        _scan_contiguous(src.reshape(-1).view(part), result.reshape(-1).view(part), outer, n,
+                         inner * 2, op, False, stream_ptr)
+    else:
+        _scan_contiguous(src, result, outer, n, inner, op, skip_nan, stream_ptr)
     if out is not None and not direct:
         _ufuncs.elementwise_copy(result, out)
         return out

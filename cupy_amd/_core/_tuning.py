@@ -92,6 +92,9 @@ _params = {
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
     'scan_cols_threads_per_cu': 256,   # column scans are cut into chunks below this many threads per CU
+    'scan_lanes': True,
+    'scan_tile_packed': True,   # slices of few rows and a narrow tail: many to a wave
+    'scan_complex_as_real': True,   # cumsum of complex arrays: as real arrays with twice the columns
     'scan_cols_vec_bytes': 0,
     'scan_chain_cols': True,    # one-pass kernel for many long columns
     'scan_chain_cols_waves': 16,

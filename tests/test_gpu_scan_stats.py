@@ -389,3 +389,36 @@ def test_narrow_scans_of_other_types_and_operations():
     out = cp.empty((150001, 3), np.float64)
     r = cp.cumsum(cp.asarray(h8), axis=0, out=out)
     assert r is out and np.array_equal(out.get(), np.cumsum(h8, axis=0, dtype=np.float64))
+
+
+@pytest.mark.parametrize('shape', [(40000, 4, 4), (30001, 16, 2), (5000, 2, 32), (20011, 5, 3),
+                                   (7001, 9, 7), (3, 100, 2), (100000, 3, 2), (1500, 33, 8),
+                                   (2, 7, 4, 5)])
+def test_scans_of_many_short_slices_with_a_narrow_tail(shape):
+    """Slices of few rows: a wave stages many of them per round and starts
+    over at every slice."""
+    rng = np.random.default_rng(sum(shape))
+    axis = len(shape) - 2
+    h = rng.integers(-9, 10, shape).astype(np.int32)
+    d = cp.asarray(h)
+    assert (d.cumsum(axis=axis).get() == h.cumsum(axis=axis)).all()
+    h8 = h.astype(np.int8)
+    assert (cp.cumsum(cp.asarray(h8), axis=axis, dtype=np.int8).get()
+            == h8.cumsum(axis=axis, dtype=np.int8)).all()
+    assert (cp.cumsum(cp.asarray(h8), axis=axis).get() == h8.cumsum(axis=axis)).all()
+    hp = np.where(rng.uniform(size=shape) < 0.2, -1, 1).astype(np.int64)
+    assert (cp.cumprod(cp.asarray(hp), axis=axis).get() == hp.cumprod(axis=axis)).all()
+    hf = rng.standard_normal(shape)
+    got = cp.cumsum(cp.asarray(hf), axis=axis).get()
+    assert np.allclose(got, hf.cumsum(axis=axis), rtol=1e-12, atol=1e-12)
+    hn = rng.uniform(0, 1, shape).astype(np.float32)
+    hn[..., ::3, 1] = np.nan
+    got = cp.nancumsum(cp.asarray(hn), axis=axis).get()
+    assert np.allclose(got, np.nancumsum(hn.astype(np.float64), axis=axis), rtol=1e-5, atol=1e-6)
+    hc = (hf + 1j * rng.standard_normal(shape)).astype(np.complex64)
+    got = cp.cumsum(cp.asarray(hc), axis=axis).get()
+    assert np.allclose(got, hc.astype(np.complex128).cumsum(axis=axis), rtol=1e-4, atol=1e-4)
+    # a view that does not start on a 16-byte boundary
+    flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
+    assert (cp.asarray(flat)[1:].reshape(shape).cumsum(axis=axis).get()
+            == flat[1:].reshape(shape).cumsum(axis=axis)).all()
