@@ -410,7 +410,7 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
 
 def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
                    reduce_type, typedefs='', preamble='', width=3, group=1, rows=256,
-                   stream_hint=False):
+                   stream_hint=False, inner=1):
     """Reduce-axis-contiguous kernel for short rows of ``width`` elements (a
     compile-time constant) that follow one another without gaps and whose
     length in bytes is not a multiple of a vector: a lane group per row would
@@ -424,10 +424,18 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
 
     Every input must have element strides (width, 1), or (0, 1): one row that
     all outputs share (``bcast_o``), or a value per row (``bcast_r``), both
-    read in place.  Same parameters as the rows kernel."""
+    read in place.  Same parameters as the rows kernel.
+
+    ``inner`` > 1: a row is a slice of ``width / inner`` lines of ``inner``
+    columns each, reduced down its columns (the reduction over the middle axis
+    of (slices, lines, columns) with few columns): ``group`` lanes per slice
+    and column, ``inner`` results per slice stored next to one another;
+    ``_n_out`` counts the results.  Plain inputs only."""
     all_ins = [a for a in args if a.kind == 'in']
     ins = [a for a in all_ins if not (a.bcast_o or a.bcast_r)]
-    assert ins and group in (1, 2, 4, 8, 16, 32, 64) and rows % (BLOCK // group) == 0
+    assert ins and group in (1, 2, 4, 8, 16, 32, 64)
+    assert inner == 1 and rows % (BLOCK // group) == 0 or (
+        inner > 1 and width % inner == 0 and len(ins) == len(all_ins))
     nt = 'true' if stream_hint else 'false'
     params = _fast_params(args, 'ptrdiff_t', False, False)
     per_pass = BLOCK // group
@@ -436,7 +444,8 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
         BLOCK, name, params))
     src.append(_SIZE_INDEXERS)
     src.append('  const ptrdiff_t _row0 = (ptrdiff_t)blockIdx.x * %d;' % rows)
-    src.append('  const int _nrows = (_n_out - _row0 < %d) ? (int)(_n_out - _row0) : %d;' % (rows, rows))
+    src.append('  const ptrdiff_t _n_rows_all = _n_out / %d;' % inner)
+    src.append('  const int _nrows = (_n_rows_all - _row0 < %d) ? (int)(_n_rows_all - _row0) : %d;' % (rows, rows))
     src.append('  const int _count = _nrows * %d;' % width)
     vecs = {}
     for a in ins:
@@ -495,6 +504,34 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
         src.append('  }')
     src.append('  __syncthreads();')
     src.append('  const int _g = threadIdx.x %% %d;' % group)
+    if inner > 1:
+        lines = width // inner
+        src.append('  for (int _it = threadIdx.x / %d; _it < _nrows * %d; _it += %d) {' % (
+            group, inner, per_pass))
+        src.append('    const int _r = _it / %d;' % inner)
+        src.append('    const int _c = _it - _r * %d;' % inner)
+        src.append('    _type_reduce _s = %s;' % _identity_decl(identity))
+        if lines // group <= 32:
+            src.append('#pragma unroll')
+        src.append('    for (int _j = _g; _j < %d; _j += %d) {' % (lines, group))
+        src.append('      const IndexT _J = _j;')
+        for a in all_ins:
+            src.append('      const %s %s(_slab_%s[_r * %d + _j * %d + _c]);' % (
+                a.var_t, a.name, a.name, width, inner))
+        src.append('      _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+        src.append('      _s = REDUCE(_s, _a);')
+        src.append('    }')
+        if group > 1:
+            src.append('    _s = cupy::group_allreduce<%d>(_s, _ReduceOp());' % group)
+            src.append('    if (_g == 0) {')
+        else:
+            src.append('    {')
+        src.append('      const ptrdiff_t _i = (_row0 + _r) * %d + _c;' % inner)
+        src.extend(_finish(args, False, '      '))
+        src.append('    }')
+        src.append('  }')
+        src.append('}')
+        return '\n'.join(src) + '\n'
     src.append('  for (int _r = threadIdx.x / %d; _r < _nrows; _r += %d) {' % (group, per_pass))
     src.append('    _type_reduce _s = %s;' % _identity_decl(identity))
     src.append('    const int _rot = (_r * %d) %% %d;' % (group, width))

@@ -292,6 +292,15 @@ class _AbstractReductionKernel:
                     and all(tuple(os_) == (n_inner * a.dtype.itemsize, a.dtype.itemsize)
                             for os_, a in zip(o_out, outs))
                     and all(s % a.dtype.itemsize == 0 for s, a in zip(sr, ins))):
+                n_red = rshape[0] if rshape else 1
+                if (all(tuple(os_) == (n_red * n_inner * a.dtype.itemsize, a.dtype.itemsize)
+                        and s == n_inner * a.dtype.itemsize
+                        for os_, s, a in zip(o_in, sr, ins))
+                        and self._launch_mid_flat(
+                            in_args, out_args, in_arr_idx, out_arr_idx, n_batch, n_red, n_inner,
+                            map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                            device_id, stream_ptr, rec)):
+                    return
                 return self._launch_cols(
                     in_args, out_args, in_arr_idx, out_arr_idx, n_batch * n_inner,
                     rshape[0] if rshape else 1, [a.dtype.itemsize for a in ins], sr,
@@ -551,6 +560,47 @@ class _AbstractReductionKernel:
         _launch_plan.launch(
             rec, fn, ((n_out + rows - 1) // rows, 1, 1), (_cg.BLOCK, 1, 1),
             _make_packer(self._fast_format(rargs, 'q')), vals, stream_ptr)
+
+    def _launch_mid_flat(self, in_args, out_args, in_arr_idx, out_arr_idx, n_batch, n_red,
+                         n_inner, map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                         device_id, stream_ptr, rec=None):
+        """Reduction over the middle axis of dense (n_batch, n_red, n_inner)
+        inputs whose slices are short and have few columns: workgroups stage
+        runs of whole slices in the LDS (``emit_rows_flat`` with ``inner``).
+        Returns False where that does not apply."""
+        ins = [in_args[i] for i in in_arr_idx]
+        items = [a.dtype.itemsize for a in ins]
+        width = n_red * n_inner
+        if (not _tuning.get('mid_flat') or n_inner > 1024 or n_red < 2 or n_batch < 1024
+                or width * sum(items) > 16 * 1024):
+            return False
+        # a lane per slice and column for up to 8 lines, more lanes beyond
+        group = min(64, internal.clp2((n_red + 7) // 8))
+        rows = max(1, min((24 * 1024) // (width * sum(items)), 65536))
+        if (n_batch + rows - 1) // rows > _max_blocks(_cg.BLOCK):
+            return False
+        preamble, _ = self._get_preamble_options()
+        rargs = self._rargs(in_args, out_args)
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('rows_stream'), sum(a.nbytes for a in ins), 0)[0]
+        key = ('mid_flat', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
+               post_map_expr, reduce_type, width, n_inner, group, rows, device_id, stream_hint)
+
+        def emit():
+            return self.name, _cg.emit_rows_flat(
+                self.name, rargs, self.identity, map_expr, reduce_expr, post_map_expr,
+                reduce_type, typedefs, preamble, width=width, group=group, rows=rows,
+                stream_hint=stream_hint, inner=n_inner)
+        fn, _, _ = self._compile(key, emit, in_args)
+        n_out = n_batch * n_inner
+        vals = self._fast_values(
+            in_args, out_args, n_out, n_red, [width * i for i in items],
+            [n_inner * i for i in items],
+            [out_args[i].dtype.itemsize for i in out_arr_idx])
+        _launch_plan.launch(
+            rec, fn, ((n_batch + rows - 1) // rows, 1, 1), (_cg.BLOCK, 1, 1),
+            _make_packer(self._fast_format(rargs, 'q')), vals, stream_ptr)
+        return True
 
     # -- rows ---------------------------------------------------------------------------------
     def _launch_rows(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,

@@ -130,6 +130,7 @@ _params = {
     # byte address reaches 58 % where element-wide accesses stay below 30 %.
     # False restricts vectors to operands aligned to the whole vector.
     'unaligned_vectors': True,
+    'mid_flat': True,           # middle-axis reductions of short slices with few columns through the LDS
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
 }

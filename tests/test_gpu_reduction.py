@@ -466,3 +466,50 @@ def test_short_rows_with_a_row_of_weights_shared_by_all_rows(width):
     got = am(cp.asarray(x), cp.asarray(w), axis=1).get()
     prod = x * w
     assert np.array_equal(prod[np.arange(len(got)), got], prod.max(axis=1))
+
+
+@pytest.mark.parametrize('shape', [(40000, 4, 4), (30001, 16, 2), (5000, 2, 32), (20011, 5, 3),
+                                   (7001, 9, 7), (1500, 33, 8), (100000, 3, 2), (2049, 100, 5),
+                                   (1025, 7, 100), (3, 700, 4, 5), (4096, 2, 128)])
+def test_middle_axis_reductions_of_short_slices_with_few_columns(shape):
+    """(slices, lines, columns) reduced over the lines: workgroups stage runs
+    of whole slices in the LDS."""
+    rng = np.random.default_rng(sum(shape))
+    axis = len(shape) - 2
+    h = rng.integers(-9, 10, shape).astype(np.int32)
+    d = cp.asarray(h)
+    assert_exact(d.sum(axis=axis).get(), h.sum(axis=axis))
+    assert_exact(d.max(axis=axis).get(), h.max(axis=axis))
+    assert_exact(d.argmax(axis=axis).get(), h.argmax(axis=axis))          # first of the ties
+    assert_exact(d.argmin(axis=axis).get(), h.argmin(axis=axis))
+    assert_exact((d > 7).any(axis=axis).get(), (h > 7).any(axis=axis))
+    assert_exact(cp.count_nonzero(d, axis=axis).get(), np.count_nonzero(h, axis=axis))
+    h8 = h.astype(np.int8)
+    assert_exact(cp.asarray(h8).sum(axis=axis).get(), h8.sum(axis=axis))
+    assert_exact(cp.asarray(h8).min(axis=axis).get(), h8.min(axis=axis))
+    hp = np.where(rng.uniform(size=shape) < 0.3, -1, 1).astype(np.int64)
+    assert_exact(cp.asarray(hp).prod(axis=axis).get(), hp.prod(axis=axis))
+    out = cp.empty(h.sum(axis=axis, keepdims=True).shape, np.int64)
+    d.sum(axis=axis, keepdims=True, out=out)
+    assert_exact(out.get(), h.sum(axis=axis, keepdims=True))
+    hf = rng.standard_normal(shape)
+    df = cp.asarray(hf)
+    np.testing.assert_allclose(df.sum(axis=axis).get(), hf.sum(axis=axis), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(df.mean(axis=axis).get(), hf.mean(axis=axis), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(df.var(axis=axis).get(), hf.var(axis=axis), rtol=1e-10, atol=1e-12)
+    hn = hf.astype(np.float32)
+    hn[..., ::3, 1] = np.nan
+    dn = cp.asarray(hn)
+    assert_exact(dn.argmax(axis=axis).get(), hn.argmax(axis=axis))        # the first NaN wins
+    np.testing.assert_allclose(cp.nansum(dn, axis=axis).get(),
+                               np.nansum(hn.astype(np.float64), axis=axis), rtol=1e-5, atol=1e-5)
+    hc = (hf + 1j * rng.standard_normal(shape)).astype(np.complex64)
+    np.testing.assert_allclose(cp.asarray(hc).sum(axis=axis).get(),
+                               hc.astype(np.complex128).sum(axis=axis), rtol=1e-4, atol=1e-4)
+    h16 = rng.uniform(0, 1, shape).astype(np.float16)
+    np.testing.assert_allclose(cp.asarray(h16).sum(axis=axis).get().astype(np.float64),
+                               h16.astype(np.float64).sum(axis=axis), rtol=2e-3, atol=1e-2)
+    # a view that does not start on a 16-byte boundary
+    flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
+    assert_exact(cp.asarray(flat)[1:].reshape(shape).sum(axis=axis).get(),
+                 flat[1:].reshape(shape).sum(axis=axis))
