@@ -511,9 +511,21 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
         src.append('    const int _r = _it / %d;' % inner)
         src.append('    const int _c = _it - _r * %d;' % inner)
         src.append('    _type_reduce _s = %s;' % _identity_decl(identity))
+        # slice r starts its walk r lines down (and wraps around): the lanes of
+        # a wave, which hold the same column of consecutive slices, are then
+        # spread over the LDS banks whatever the length of a slice
+        # (only where slices start a multiple of 16 words apart: elsewhere the
+        # banks are spread as it is, and the plain walk is quicker)
+        rotate = width % 16 == 0
+        src.append('    const int _rot = %s;' % (('_r %% %d' % lines) if rotate else '0'))
         if lines // group <= 32:
             src.append('#pragma unroll')
-        src.append('    for (int _j = _g; _j < %d; _j += %d) {' % (lines, group))
+        src.append('    for (int _jq = _g; _jq < %d; _jq += %d) {' % (lines, group))
+        if rotate:
+            src.append('      const int _j = (_jq + _rot >= %d) ? (_jq + _rot - %d) : (_jq + _rot);' % (
+                lines, lines))
+        else:
+            src.append('      const int _j = _jq;')
         src.append('      const IndexT _J = _j;')
         for a in all_ins:
             src.append('      const %s %s(_slab_%s[_r * %d + _j * %d + _c]);' % (

@@ -572,10 +572,14 @@ class _AbstractReductionKernel:
         items = [a.dtype.itemsize for a in ins]
         width = n_red * n_inner
         if (not _tuning.get('mid_flat') or n_inner > 1024 or n_red < 2 or n_batch < 1024
-                or width * sum(items) > 16 * 1024):
+                or width * sum(items) > 32 * 1024):
             return False
-        # a lane per slice and column for up to 8 lines, more lanes beyond
-        group = min(64, internal.clp2((n_red + 7) // 8))
+        # a lane per slice and column for up to 32 lines, more lanes beyond
+        # (states that are expensive to merge, like those of the variance,
+        # want long walks and few lanes: 130561 slices of 257 x 2 floats, var:
+        # 31 % of peak with 8 lines per lane, 58 % with 32; sums do not care)
+        per_lane = _tuning.get('mid_flat_lines_per_lane')
+        group = min(64, internal.clp2((n_red + per_lane - 1) // per_lane))
         rows = max(1, min((24 * 1024) // (width * sum(items)), 65536))
         if (n_batch + rows - 1) // rows > _max_blocks(_cg.BLOCK):
             return False

@@ -1975,6 +1975,31 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
     return True
 
 
+def _scan_packed(src, dst, outer, n, inner, op, skip_nan, vec, trips, idx64, stream, stream_ptr,
+                 cus):
+    """Launches ``_emit_tile_packed`` where at least four slices fit a round
+    (with two the plain kernels are as good: 2^17 slices of 32 x 16 floats
+    86.6 us against 91.5).  Returns False otherwise."""
+    if outer < 2 or not _tuning.get('scan_tile_packed'):
+        return False
+    while _tile_geometry(inner, vec, trips)[2] > 32 and trips > 1:
+        trips //= 2       # (a lane marks the slice starts among its rows in 64 bits)
+    rows_t, _, lrows, _ = _tile_geometry(inner, vec, trips)
+    if 4 * n > rows_t or lrows > 64:
+        return False
+    round_rows = rows_t // n * n
+    mod = _module_tile_packed(src.dtype, dst.dtype, op, skip_nan, vec, trips, idx64, inner, stream)
+    rounds = (outer * n + round_rows - 1) // round_rows
+    per_block = _BLOCK // _WAVE
+    grid = max(1, min((rounds + per_block - 1) // per_block,
+                      cus * _tuning.get('scan_blocks_per_cu')))
+    blob = struct.pack('@PP' + ('q' if idx64 else 'i') + 'ii', src.data.ptr, dst.data.ptr,
+                       outer * n, n, round_rows)
+    mod.get_function('cupy_scan_tile_packed').launch_packed(
+        (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+    return True
+
+
 def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_chunk=True):
     """Scans the middle axis of C-contiguous (outer, n, inner) ``src`` into
     ``dst`` (same layout; may be the same memory if the dtypes agree)."""
@@ -2008,9 +2033,22 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                 and total * in_dtype.itemsize <= 2 * _tuning.get('cache_bytes'))
     if inner == 1:
         vec = max(1, 16 // item)
-        while vec > 1 and (not _aligned(src.data.ptr, vec * in_dtype.itemsize)
-                           or not _aligned(dst.data.ptr, vec * out_dtype.itemsize)
-                           or (outer > 1 and n % vec) or n < vec):
+        # (rows of any length keep their vectors: wide accesses need the
+        # alignment of an element only, and the kernels end every row element
+        # by element; 2^26 floats as rows of 33: 294 us element-wide)
+        loose = _tuning.get('unaligned_vectors') and _tuning.get('scan_rows_unaligned')
+        if (n % vec and _tuning.get('scan_rows_packed')
+                and _aligned(src.data.ptr, in_dtype.itemsize * vec)
+                and _scan_packed(src, dst, outer, n, 1, op, skip_nan, vec, 4, idx64, stream,
+                                 stream_ptr, cus)):
+            # short rows that are no whole number of vectors: as slices of one
+            # column, many to a wave (2^26 floats as rows of 33: 45 % of peak
+            # with a lane group per row)
+            return
+        while vec > 1 and ((not loose and (
+                not _aligned(src.data.ptr, vec * in_dtype.itemsize)
+                or not _aligned(dst.data.ptr, vec * out_dtype.itemsize)
+                or (outer > 1 and n % vec))) or n < vec):
             vec //= 2
         # short rows: a group of lanes smaller than a wave per row, each lane
         # with up to four vectors; long rows: whole waves
@@ -2054,30 +2092,11 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         vec = max(1, 16 // item)
         trips = 4
         rows_t, _, _, _ = _tile_geometry(inner, vec, trips)
-        if 4 * n <= rows_t and outer > 1 and _tuning.get('scan_tile_packed'):
-            # Slices of few rows: many to a round.  (2^26 float32 as 2^22
-            # slices of 4 x 4: 1190 us with a wave per slice; 2^21 of 16 x 2:
-            # 697; 2^20 of 2 x 32: 278)
-            p_trips = trips
-            while _tile_geometry(inner, vec, p_trips)[2] > 32 and p_trips > 1:
-                p_trips //= 2       # (a lane marks the slice starts among its rows in 64 bits)
-            rows_p = _tile_geometry(inner, vec, p_trips)[0]
-        else:
-            rows_p = 0
-        # (with two slices to a round the plain kernel is as good: 2^17 slices
-        # of 32 x 16 floats 86.6 us against 91.5)
-        if 4 * n <= rows_p and _tile_geometry(inner, vec, p_trips)[2] <= 64:
-            round_rows = rows_p // n * n
-            mod = _module_tile_packed(in_dtype, out_dtype, op, skip_nan, vec, p_trips, idx64,
-                                      inner, stream)
-            rounds = (outer * n + round_rows - 1) // round_rows
-            per_block = _BLOCK // _WAVE
-            grid = max(1, min((rounds + per_block - 1) // per_block,
-                              cus * _tuning.get('scan_blocks_per_cu')))
-            blob = struct.pack('@PP' + ic + 'ii', src.data.ptr, dst.data.ptr, outer * n, n,
-                               round_rows)
-            mod.get_function('cupy_scan_tile_packed').launch_packed(
-                (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+        # Slices of few rows: many to a round.  (2^26 float32 as 2^22 slices of
+        # 4 x 4: 1190 us with a wave per slice; 2^21 of 16 x 2: 697; 2^20 of
+        # 2 x 32: 278)
+        if _scan_packed(src, dst, outer, n, inner, op, skip_nan, vec, trips, idx64, stream,
+                        stream_ptr, cus):
             return
         want = cus * _tuning.get('scan_waves_per_cu')
         n_chunks = 1

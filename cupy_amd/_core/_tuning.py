@@ -92,6 +92,8 @@ _params = {
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
     'scan_cols_threads_per_cu': 256,   # column scans are cut into chunks below this many threads per CU
+    'scan_rows_unaligned': True,   # row scans use vectors whatever the row length and alignment
+    'scan_rows_packed': True,
     'scan_lanes': True,
     'scan_tile_packed': True,   # slices of few rows and a narrow tail: many to a wave
     'scan_complex_as_real': True,   # cumsum of complex arrays: as real arrays with twice the columns
@@ -130,6 +132,7 @@ _params = {
     # byte address reaches 58 % where element-wide accesses stay below 30 %.
     # False restricts vectors to operands aligned to the whole vector.
     'unaligned_vectors': True,
+    'mid_flat_lines_per_lane': 32,
     'mid_flat': True,           # middle-axis reductions of short slices with few columns through the LDS
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this
