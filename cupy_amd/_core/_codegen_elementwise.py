@@ -562,7 +562,7 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
 def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
                  loop_prep='', after_loop='', layouts=None, vec=4, tile_r=64,
                  tile_c=64, threads=256, idx64=False, stream_hint=True, batched=False,
-                 batch_first=False):
+                 batch_first=False, svec=None):
     """Kernel for a 2-d index space (rows r, columns c) where every array
     operand is contiguous along one of the axes.
 
@@ -595,8 +595,13 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     nts = 'true' if _nt_s else 'false'
     use_i = uses_identifier(operation, 'i')
     set_ind = '_ind.set(i);' if needs_ind and uses_identifier(operation, '_ind') else ''
-    assert tile_r % vec == 0 and tile_c % vec == 0
-    n_stage = (tile_r // vec) * tile_c          # staging vectors per tile
+    # ``svec``: elements per staging access of the transposed operands (along
+    # the rows), where that differs from the ``vec`` of the accesses along the
+    # columns: a narrow array has room or alignment for vectors one way only
+    if svec is None:
+        svec = vec
+    assert tile_r % svec == 0 and tile_c % vec == 0
+    n_stage = (tile_r // svec) * tile_c         # staging vectors per tile
     n_work = tile_r * (tile_c // vec)           # compute vectors per tile
     assert n_stage % threads == 0 and n_work % threads == 0
     pitch = tile_c + 1                          # odd pitch: column walks spread over banks
@@ -694,14 +699,14 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         src.append('#pragma unroll')
         src.append('      for (int _it = 0; _it < %d; ++_it) {' % (n_stage // threads))
         src.append('        const int _v = threadIdx.x + _it * %d;' % threads)
-        src.append('        const int _lr = (_v %% %d) * %d;' % (tile_r // vec, vec))
-        src.append('        const int _lc = _v / %d;' % (tile_r // vec))
+        src.append('        const int _lr = (_v %% %d) * %d;' % (tile_r // svec, svec))
+        src.append('        const int _lc = _v / %d;' % (tile_r // svec))
         for op in c_ops:
             src.append('        { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s);' % (
-                op.store_t, vec, op.store_t, vec, ntl, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
+                op.store_t, svec, op.store_t, svec, ntl, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
             src.append('#pragma unroll')
             src.append('          for (int _k = 0; _k < %d; ++_k) '
-                       '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (vec, op.name, pitch))
+                       '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (svec, op.name, pitch))
         src.append('      }')
         src.append('    } else {')
         # edge tile: the same vectors where they lie inside the array, element by
@@ -709,19 +714,19 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
         src.append('#pragma unroll')
         src.append('      for (int _it = 0; _it < %d; ++_it) {' % (n_stage // threads))
         src.append('        const int _v = threadIdx.x + _it * %d;' % threads)
-        src.append('        const int _lr = (_v %% %d) * %d;' % (tile_r // vec, vec))
-        src.append('        const int _lc = _v / %d;' % (tile_r // vec))
+        src.append('        const int _lr = (_v %% %d) * %d;' % (tile_r // svec, svec))
+        src.append('        const int _lc = _v / %d;' % (tile_r // svec))
         src.append('        if (_c0 + _lc < _nc) {')
-        src.append('          if (_r0 + _lr + %d <= _nr) {' % vec)
+        src.append('          if (_r0 + _lr + %d <= _nr) {' % svec)
         for op in c_ops:
             src.append('            { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s);' % (
-                op.store_t, vec, op.store_t, vec, ntl, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
+                op.store_t, svec, op.store_t, svec, ntl, gaddr(op, '_r0 + _lr', '_c0 + _lc')))
             src.append('#pragma unroll')
             src.append('              for (int _k = 0; _k < %d; ++_k) '
-                       '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (vec, op.name, pitch))
+                       '_t_%s[(_lr + _k) * %d + _lc] = _lv.v[_k]; }' % (svec, op.name, pitch))
         src.append('          } else {')
         src.append('#pragma unroll')
-        src.append('            for (int _k = 0; _k < %d; ++_k) if (_r0 + _lr + _k < _nr) {' % vec)
+        src.append('            for (int _k = 0; _k < %d; ++_k) if (_r0 + _lr + _k < _nr) {' % svec)
         for op in c_ops:
             src.append('              _t_%s[(_lr + _k) * %d + _lc] = *%s;' % (
                 op.name, pitch, gaddr(op, '_r0 + _lr + _k', '_c0 + _lc')))

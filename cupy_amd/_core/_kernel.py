@@ -927,24 +927,29 @@ class _ElementwisePlanner:
                 layouts[nm] = 'C'
                 n_transposed += 1
                 lds_item += item
-        # alignment of every vector access
-        while vec > 1:
-            ok = True
-            for a, cs, nm in zip(arrays, cstrides, names):
-                item = a.dtype.itemsize
-                nb = vec * item
-                if layouts[nm] == 'R0':
-                    continue
-                if not _aligned(a.data.ptr, nb):
-                    ok = False
-                elif layouts[nm] == 'R':
-                    if not _aligned(cs[0], nb):
+        # Alignment of every vector access: along the columns (``vec``) for the
+        # row-major operands, along the rows (``svec``) for the staged ones.
+        # Wide accesses need the alignment of an element only; unaligned ones
+        # cost a few per cent, element-wide ones most of the bandwidth.
+        loose = _tuning.get('unaligned_vectors') and _tuning.get('tiled_unaligned')
+
+        def widest(kinds, limit):
+            v = max(1, 16 // max(itemsizes))
+            while v > 1:
+                ok = v <= limit
+                for a, cs, nm in zip(arrays, cstrides, names):
+                    if layouts[nm] not in kinds or loose:
+                        continue
+                    nb = v * a.dtype.itemsize
+                    if not _aligned(a.data.ptr, nb) or not _aligned(
+                            cs[0] if layouts[nm] == 'R' else cs[1], nb):
                         ok = False
-                elif not _aligned(cs[1], nb):
-                    ok = False
-            if ok:
-                break
-            vec //= 2
+                if ok:
+                    break
+                v //= 2
+            return v
+        vec = widest(('R',), nc)
+        svec = widest(('C',), nr) if n_transposed else vec
         # Large tiles give long contiguous runs in memory on both the transposed
         # and the row-major side; they need the LDS for the staged operands.
         big_min = _tuning.get('tiled_big_min')
@@ -956,6 +961,48 @@ class _ElementwisePlanner:
         else:
             tile_r = tile_c = 64
             threads = 256
+        narrow = n_transposed and min(nr, nc) <= 32 and _tuning.get('tiled_narrow')
+        if narrow:
+            # A narrow array (points as rows of three coordinates, say, to or
+            # from three long rows): tiles as narrow as the array and long the
+            # other way, so that no tile has an edge along the narrow side and
+            # both sides move in long contiguous runs.  (2^26 floats over
+            # rotating buffers, (n, 3) to (3, n): 1215 us with square tiles, 118
+            # so; back: 531 -> 108; (n, 2): 1243 -> 105; (n, 15): 340 -> 161.
+            # Tiles of about 1536 elements: of 4096 (n, 3) takes 214 us, of
+            # 12288 615: few workgroups per CU then, each busy with one phase.)
+            # the workgroup is a whole number of lines of the narrow side, so
+            # that both loops of the kernel come out in whole trips
+            want = max(512, min(_tuning.get('tiled_narrow_elements'),
+                                 (48 * 1024) // max(1, lds_item)))
+            if nr <= 32:
+                tile_r = nr
+                while svec > 1 and tile_r % svec:
+                    svec //= 2
+                # (a power of two of lines: tiles then start on whole cache lines)
+                per = internal.flp2(256 // tile_r)
+                threads = tile_r * per
+                m = 1
+                while (vec * m) % svec or threads * vec * m < want:
+                    m += 1
+                tile_c = vec * per * m
+            else:
+                tile_c = nc
+                while vec > 1 and tile_c % vec:
+                    vec //= 2
+                q = tile_c // vec
+                per = internal.flp2(256 // q)
+                threads = q * per
+                m = 1
+                while ((vec * m) % svec or (per * m) % svec or (per * m) % 32
+                       or threads * vec * m < want):
+                    m += 1
+                tile_r = per * m
+            if lds_item * tile_r * (tile_c + 1) > 64 * 1024:
+                tile_r = tile_c = 64        # (many wide staged operands: square tiles)
+                threads = 256
+                vec = min(vec, svec)
+                svec = vec
         forced = _tuning.get('tiled_tile')
         if forced and n_transposed:
             tile_r, tile_c, threads = forced
@@ -1011,7 +1058,7 @@ class _ElementwisePlanner:
             batch_first = all(b and b < p for b, p in zip(inner_batch, pitch))
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
-               threads, bool(batch), batch_first)
+               threads, bool(batch), batch_first, svec)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
@@ -1019,7 +1066,8 @@ class _ElementwisePlanner:
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
                 tile_r=tile_r, tile_c=tile_c, threads=threads, idx64=idx64,
-                stream_hint=stream_hint, batched=bool(batch), batch_first=batch_first)
+                stream_hint=stream_hint, batched=bool(batch), batch_first=batch_first,
+                svec=svec)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']

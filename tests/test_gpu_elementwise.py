@@ -547,3 +547,27 @@ def test_reduce_dims_false_keeps_the_axes_for_the_kernel():
     rows = np.array([[4], [0], [2]], np.int32)
     out = g(cp.asarray(src), cp.broadcast_to(cp.asarray(rows), (3, 6)))
     assert_exact(out.get(), src[rows[:, 0]])
+
+
+@pytest.mark.parametrize('shape', [(100003, 3), (3, 100003), (65536, 15), (31, 40001), (50000, 32),
+                                   (2, 70001), (4099, 1), (7, 5, 20001, 3), (6, 3, 20001)])
+def test_transposes_of_narrow_arrays(shape):
+    """Points as rows of a few coordinates to or from a few long rows: tiles as
+    narrow as the array."""
+    rng = np.random.default_rng(sum(shape))
+    perm = tuple(range(len(shape) - 2)) + (len(shape) - 1, len(shape) - 2)
+    for dtype in (np.float32, np.float64, np.int8, np.complex64, np.float16):
+        h = (rng.uniform(-100, 100, shape)).astype(dtype)
+        d = cp.asarray(h)
+        ht = np.swapaxes(h, -1, -2)
+        dt = d.transpose(perm)
+        assert_exact(cp.ascontiguousarray(dt).get(), np.ascontiguousarray(ht))
+        if np.dtype(dtype).kind == 'f':
+            other = rng.uniform(1, 2, ht.shape).astype(dtype)
+            assert_exact((dt * cp.asarray(other)).get(), ht * other)
+            assert_exact((dt + dt).get(), ht + ht)
+    # a view that does not start on a 16-byte boundary
+    n = int(np.prod(shape))
+    flat = rng.integers(-9, 10, n + 1).astype(np.int32)
+    got = cp.ascontiguousarray(cp.asarray(flat)[1:].reshape(shape).transpose(perm)).get()
+    assert_exact(got, np.ascontiguousarray(np.swapaxes(flat[1:].reshape(shape), -1, -2)))
