@@ -391,6 +391,25 @@ def build_layout_cases(cp):
     add('cumsum f32 (2^26/3)x3 axis=0', 2 * a3.nbytes, run('scan3', lambda: cp.cumsum(d3, axis=0)),
         lambda: np.cumsum(a3, axis=0), lambda: close(res['scan3'], want_scan, 1e-5, scale_scan),
         'cupy_scan_lanes')
+    # ---- narrow arrays and short slices (points, channels-last data) -------------------
+    add('(N,3) -> (3,N) copy f32', 2 * a3.nbytes, run('t3', lambda: cp.ascontiguousarray(d3.T)),
+        lambda: np.ascontiguousarray(a3.T), lambda: same(res['t3'], a3.T), 'cupy_copy')
+    ach, dch = flat.reshape(n // 32, 16, 2), dflat.reshape(n // 32, 16, 2)
+    add('sum f32 (2^21,16,2) axis=1', ach.nbytes + (n // 16) * 4, run('ch', lambda: dch.sum(axis=1)),
+        lambda: ach.sum(axis=1),
+        lambda: close(res['ch'], ach.sum(axis=1, dtype=np.float64), 1e-5,
+                      np.abs(ach).sum(axis=1, dtype=np.float64)), 'cupy_sum')
+    a44, d44 = flat.reshape(n // 16, 4, 4), dflat.reshape(n // 16, 4, 4)
+    add('cumsum f32 (2^22,4,4) axis=1', 2 * a44.nbytes, run('s44', lambda: cp.cumsum(d44, axis=1)),
+        lambda: np.cumsum(a44, axis=1),
+        lambda: close(res['s44'], np.cumsum(a44, axis=1, dtype=np.float64), 1e-5,
+                      np.cumsum(np.abs(a44), axis=1, dtype=np.float64)), 'cupy_scan_tile_packed')
+    r33 = n // 33
+    a33, d33 = flat[:r33 * 33].reshape(r33, 33), dflat[:r33 * 33].reshape(r33, 33)
+    add('cumsum f32 (2^26/33)x33 axis=1', 2 * a33.nbytes, run('s33', lambda: cp.cumsum(d33, axis=1)),
+        lambda: np.cumsum(a33, axis=1),
+        lambda: close(res['s33'], np.cumsum(a33, axis=1, dtype=np.float64), 1e-5,
+                      np.cumsum(np.abs(a33), axis=1, dtype=np.float64)), 'cupy_scan_tile_packed')
     r100 = n // 100
     a100, d100 = flat[:r100 * 100].reshape(r100, 100), dflat[:r100 * 100].reshape(r100, 100)
 
