@@ -1927,7 +1927,9 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
     dev_id, fault = ready
     in_dtype, out_dtype = src.dtype, dst.dtype
     acc_item = _acc_dtype(out_dtype).itemsize
-    item = max(in_dtype.itemsize, out_dtype.itemsize, acc_item)
+    # (a lane keeps its rows as loaded: the width of the accumulator, wider than
+    # the values for float16, does not count)
+    item = max(in_dtype.itemsize, out_dtype.itemsize)
     # Vectors of 8 bytes, or of 4 where those would leave many lanes of the
     # last block of columns idle; a workgroup of 16 waves, each lane keeping
     # 256 bytes of its columns.  (2^26 float32 over rotating buffers, us, for
@@ -1938,7 +1940,9 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
     best = None
     forced = _tuning.get('scan_chain_cols_vec_bytes')
     for vec_bytes in ((forced,) if forced else (8, 4)):
-        v = max(1, vec_bytes // item)
+        # (two columns a lane at most: every column has its running values and
+        # its share of the look-back in registers)
+        v = max(1, min(2, vec_bytes // item))
         while v > 1 and (not _aligned(src.data.ptr, v * in_dtype.itemsize)
                          or not _aligned(dst.data.ptr, v * out_dtype.itemsize)
                          or inner % v):
@@ -1950,7 +1954,9 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
             best = (used, v, blocks)
     _, vec, col_blocks = best
     waves = max(2, min(16, _tuning.get('scan_chain_cols_waves')))
-    trips = _tuning.get('scan_chain_cols_trips') or max(4, min(64, (256 if item < 16 else 128) // (vec * item)))
+    # (values narrower than a register are unpacked: fewer rows then)
+    trips = _tuning.get('scan_chain_cols_trips') or max(4, min(
+        64 if item >= 4 else 32, (256 if item < 16 else 128) // (vec * item)))
     tile_rows = waves * trips
     row_tiles = (n + tile_rows - 1) // tile_rows
     n_tiles = outer * row_tiles * col_blocks

@@ -23,16 +23,18 @@ def scratch_users():
     return bad
 
 
-@pytest.mark.parametrize('dtype', ['float32', 'float64', 'complex64', 'complex128', 'int8'])
+@pytest.mark.parametrize('dtype', ['float32', 'float64', 'complex64', 'complex128', 'int8',
+                                   'float16', 'int16'])
 def test_reductions_scans_and_elementwise_kernels_use_no_scratch(dtype):
     before = scratch_users()
-    shapes = [(513, 1031), (1 << 14, 256), (3, 400001)]
+    shapes = [(513, 1031), (1 << 14, 256), (3, 400001), (40000, 100)]
     for shape in shapes:
         arr = cp.empty(shape, dtype)
         for axis in (0, 1, None):
             arr.sum(axis=axis)
             arr.mean(axis=axis)
             cp.cumsum(arr, axis=axis)
+            cp.cumsum(arr, axis=axis, dtype=arr.dtype)
             if arr.dtype.kind != 'c':
                 arr.argmax(axis=axis)
                 arr.max(axis=axis)
