@@ -196,7 +196,10 @@ __device__ __forceinline__ void scan_cols_impl(
     const _in_t* __restrict__ in, _out_t* __restrict__ out, _acc_t* __restrict__ totals,
     const _idx_t n_outer, const _idx_t n, const _idx_t inner, const _idx_t n_chunks,
     const _idx_t chunk_len) {
-  const _idx_t inner_v = inner / VEC;            // the host guarantees inner %% VEC == 0
+  // vectors per row; where the row is no whole number of them, the last one
+  // starts VEC columns before the end of the row and overlaps its neighbour
+  // (both then compute and store the same values for the shared columns)
+  const _idx_t inner_v = (inner + VEC - 1) / VEC;            // the host guarantees inner >= VEC
   const _idx_t n_work = n_outer * n_chunks * inner_v;
   for (_idx_t w0 = (_idx_t)blockIdx.x * %(block)d + threadIdx.x; w0 < n_work;
        w0 += (_idx_t)gridDim.x * %(block)d) {
@@ -207,14 +210,15 @@ __device__ __forceinline__ void scan_cols_impl(
     const _idx_t o = oc / n_chunks;
     const _idx_t j0 = chunk * chunk_len;
     const _idx_t j1 = (j0 + chunk_len < n) ? (j0 + chunk_len) : n;
-    const ptrdiff_t col = (ptrdiff_t)o * n * inner + (ptrdiff_t)iv * VEC;
+    const _idx_t c0 = (iv * VEC + VEC <= inner) ? iv * VEC : inner - VEC;
+    const ptrdiff_t col = (ptrdiff_t)o * n * inner + c0;
     _acc_t run[VEC];
 #pragma unroll
     for (int k = 0; k < VEC; ++k) run[k] = SCAN_IDENTITY;
     if (kMode == 2 && chunk > 0) {
 #pragma unroll
       for (int k = 0; k < VEC; ++k)
-        run[k] = totals[((ptrdiff_t)o * n_chunks + chunk - 1) * inner + (ptrdiff_t)iv * VEC + k];
+        run[k] = totals[((ptrdiff_t)o * n_chunks + chunk - 1) * inner + c0 + k];
     }
     _idx_t j = j0;
     for (; j + TRIPS <= j1; j += TRIPS) {
@@ -246,7 +250,7 @@ __device__ __forceinline__ void scan_cols_impl(
     if (kMode == 1) {
 #pragma unroll
       for (int k = 0; k < VEC; ++k)
-        totals[((ptrdiff_t)o * n_chunks + chunk) * inner + (ptrdiff_t)iv * VEC + k] = run[k];
+        totals[((ptrdiff_t)o * n_chunks + chunk) * inner + c0 + k] = run[k];
     }
   }
 }
@@ -2170,13 +2174,25 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         # 32 rows 141, chunked 131); 1024 x 2^16 4-byte vectors 64 rows 104 (32
         # rows 125, chunked 128).  Below 256 threads per CU the rows are cut
         # into chunks: 4096 x 2^14 135 with 8 rows at a time.
+        # (not in place: a thread would find its neighbour's results where it
+        # expects the values of the columns they share)
+        # (and rows of 128 columns or more: 2^26 floats in slices of 100 x 33
+        # take 220 us element-wide, 280 with overlapping vectors; in slices of
+        # 2 x 65537 89 us against 141)
+        loose = (_tuning.get('unaligned_vectors') and _tuning.get('scan_cols_unaligned')
+                 and src.data.ptr != dst.data.ptr and inner >= 128)
+
         def threads_with(vec_bytes):
+            # (vectors need the alignment of an element only, and a row that
+            # is no whole number of them ends with one that overlaps its
+            # neighbour)
             v = max(1, vec_bytes // item)
-            while v > 1 and (not _aligned(src.data.ptr, v * in_dtype.itemsize)
-                             or not _aligned(dst.data.ptr, v * out_dtype.itemsize)
-                             or inner % v):
+            while v > 1 and (v > inner or (not loose and (
+                    not _aligned(src.data.ptr, v * in_dtype.itemsize)
+                    or not _aligned(dst.data.ptr, v * out_dtype.itemsize)
+                    or inner % v))):
                 v //= 2
-            return v, outer * (inner // v)
+            return v, outer * ((inner + v - 1) // v)
         forced = _tuning.get('scan_cols_vec_bytes')
         per_cu = _tuning.get('scan_cols_threads_per_cu')
         one_pass_trips = 0

@@ -95,6 +95,7 @@ _params = {
     'scan_tile': True,          # narrow scanned arrays (2..32 columns) staged through the LDS
     'scan_chunk_reuse': True,   # chunked scans: second reading of the input in reverse order
     'scan_cols_threads_per_cu': 256,   # column scans are cut into chunks below this many threads per CU
+    'scan_cols_unaligned': True,   # ... and so do the column scans (the last vector of a row overlaps)
     'scan_rows_unaligned': True,   # row scans use vectors whatever the row length and alignment
     'scan_rows_packed': True,
     'scan_lanes': True,

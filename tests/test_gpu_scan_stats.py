@@ -422,3 +422,31 @@ def test_scans_of_many_short_slices_with_a_narrow_tail(shape):
     flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
     assert (cp.asarray(flat)[1:].reshape(shape).cumsum(axis=axis).get()
             == flat[1:].reshape(shape).cumsum(axis=axis)).all()
+
+
+@pytest.mark.parametrize('shape', [(2000, 100, 33), (50, 257, 257), (300, 1024, 33), (7, 9, 1001),
+                                   (3, 40, 4099), (1, 70000, 37), (5, 3, 65537)])
+def test_column_scans_with_odd_numbers_of_columns(shape):
+    """Rows that are no whole number of vectors: the last vector of a row
+    overlaps its neighbour; in place the kernel falls back to single elements."""
+    rng = np.random.default_rng(sum(shape))
+    h = rng.integers(-9, 10, shape).astype(np.int32)
+    d = cp.asarray(h)
+    assert (d.cumsum(axis=1).get() == h.cumsum(axis=1)).all()
+    out = cp.empty(shape, np.int32)
+    cp.cumsum(d, axis=1, out=out)
+    assert (out.get() == h.cumsum(axis=1)).all()
+    inplace = d.copy()
+    cp.cumsum(inplace, axis=1, out=inplace)
+    assert (inplace.get() == h.cumsum(axis=1)).all()
+    h8 = h.astype(np.int8)
+    assert (cp.cumsum(cp.asarray(h8), axis=1).get() == h8.cumsum(axis=1)).all()
+    hf = rng.standard_normal(shape)
+    got = cp.cumsum(cp.asarray(hf), axis=1).get()
+    assert np.allclose(got, hf.cumsum(axis=1), rtol=1e-12, atol=1e-10)
+    hh = rng.uniform(0, 1, shape).astype(np.float16)
+    got = cp.cumsum(cp.asarray(hh), axis=1, dtype=np.float32).get()
+    assert np.allclose(got, hh.astype(np.float32).cumsum(axis=1), rtol=1e-4, atol=1e-3)
+    flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
+    assert (cp.asarray(flat)[1:].reshape(shape).cumsum(axis=1).get()
+            == flat[1:].reshape(shape).cumsum(axis=1)).all()
