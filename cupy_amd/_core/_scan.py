@@ -2133,7 +2133,11 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         prefix = 'cupy_scan_tile'
         totals_shape = (outer, n_chunks, inner)
         middle_round = rows_t
-    elif _tuning.get('scan_lanes') and _lanes_geometry(src, dst, inner, item) is not None:
+    elif (_tuning.get('scan_lanes') and _lanes_geometry(src, dst, inner, item) is not None
+          # (a slice with fewer rows than a wave takes per trip leaves most of
+          # the wave idle: a thread per column vector instead; 2^19 slices of
+          # 2 x 64 floats: 274 us here)
+          and n > _WAVE // _lanes_geometry(src, dst, inner, item)[1]):
         vec, lstride = _lanes_geometry(src, dst, inner, item)
         trips = 4
         trip_rows = _WAVE // lstride
