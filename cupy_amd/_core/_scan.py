@@ -440,7 +440,7 @@ def _tile_geometry(inner, vec, trips):
 
 
 def _emit_tile(in_t, out_t, op, skip_nan, vec, trips, idx64, inner, stream, reuse):
-    """Scan along the middle axis of (outer, n, inner) for 2 <= inner <= 32.
+    """Scan along the middle axis of (outer, n, inner) for 2 <= inner <= 64.
 
     A wave takes ``ROWS_T`` consecutive rows per round -- one contiguous piece
     of memory, read with full 128-bit vectors on consecutive lanes whatever the
@@ -600,7 +600,7 @@ TILE_KERNEL(cupy_scan_tile_seeded, 2)
 
 
 def _emit_tile_packed(in_t, out_t, op, skip_nan, vec, trips, idx64, inner, stream):
-    """Scan along the middle axis of (outer, n, inner) for 2 <= inner <= 32 and
+    """Scan along the middle axis of (outer, n, inner) for 2 <= inner <= 64 and
     slices so short that many fit the rows a wave stages per round: the
     staging of ``_emit_tile``, with the (outer x n) rows taken as one long run
     cut into rounds of whole slices.  The scan starts over wherever a slice
@@ -2098,7 +2098,12 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         prefix = 'cupy_scan_rows'
         totals_shape = (outer, n_chunks, 1)
         middle_round = _WAVE * 4 * 4          # elements one wave takes per round
-    elif 2 <= inner <= 32 and _tuning.get('scan_tile'):
+    elif (2 <= inner <= (_tuning.get('scan_tile_max_inner') if n < 16384 else 32)
+          and _tuning.get('scan_tile')):
+        # (33 to 64 columns: a lane per column, half the wave idle while it
+        # scans, but whole vectors both ways; 2^26 floats in slices of 16 x 33:
+        # 51 -> 62 % of peak, of 100 x 63: 33 -> 56 %.  Long columns are better
+        # off in the one-pass kernel for many columns.)
         vec = max(1, 16 // item)
         trips = 4
         rows_t, _, _, _ = _tile_geometry(inner, vec, trips)

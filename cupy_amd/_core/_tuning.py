@@ -98,6 +98,7 @@ _params = {
     'scan_cols_unaligned': True,   # ... and so do the column scans (the last vector of a row overlaps)
     'scan_rows_unaligned': True,   # row scans use vectors whatever the row length and alignment
     'scan_rows_packed': True,
+    'scan_tile_max_inner': 64,  # widest tail the staged kernels take
     'scan_lanes': True,
     'scan_tile_packed': True,   # slices of few rows and a narrow tail: many to a wave
     'scan_complex_as_real': True,   # cumsum of complex arrays: as real arrays with twice the columns
