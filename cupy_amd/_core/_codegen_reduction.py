@@ -86,13 +86,148 @@ struct _ReduceOp {
 ''' % (typedefs, preamble, reduce_expr, post_map_expr, reduce_type)
 
 
+# Finishing a split reduction inside the launch that produced the partial
+# results.  Every workgroup publishes its partial result(s) in slots of 64 bits:
+# a 32-bit word of the value beside the number of the launch (``epoch``), one
+# relaxed device-scope store each, so that neither side needs a fence.  The
+# workgroup of a column block (or row) that starts last -- the one with the
+# highest number, workgroups start in the order of their numbers -- waits for
+# the slots of the others, combines them in the order of their numbers and
+# stores the result(s).  The number of the launch is kept in the memory the
+# slots live in (word 0): every workgroup reads it at its start, and the very
+# last workgroup of the grid advances it once every other finishing workgroup
+# has reported (each reports after it has seen the partial results of all its
+# workgroups, which therefore have all read the number).  Launches that share
+# the memory must not overlap: the host keeps one such memory per stream.
+# Every wait is bounded by ``_spin_limit`` polls; a workgroup that gives up
+# says so in ``_fault`` and runs to its end all the same.
+_SYNC_HELPERS = r"""
+typedef unsigned long long _slot_t;
+constexpr int _kWords = (sizeof(_type_reduce) + 3) / 4;
+#define _SYNC_HEADER_WORDS 64
+#define _SYNC_AHEAD %(ahead)d
+
+// (the value by value: taken by reference, structures of four doubles went
+// through the stack)
+__device__ __forceinline__ void _sync_publish(_slot_t* slots, const ptrdiff_t i,
+                                              const _type_reduce v, const unsigned epoch) {
+  unsigned w[_kWords];
+#pragma unroll
+  for (int k = 0; k < _kWords; ++k) w[k] = 0u;
+  __builtin_memcpy(w, &v, sizeof(_type_reduce));
+#pragma unroll
+  for (int k = 0; k < _kWords; ++k)
+    __hip_atomic_store(slots + i * _kWords + k, ((_slot_t)epoch << 32) | w[k], __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The values first, first + stride, ... (`count` of them), waited for and
+// combined in that order onto `acc`.  Asks for _SYNC_AHEAD values at a time.
+// Returns false if it gave up.
+__device__ __forceinline__ bool _sync_fold(_slot_t* slots, const ptrdiff_t first,
+                                           const ptrdiff_t stride, const int count,
+                                           const unsigned epoch, const unsigned spin_limit,
+                                           _type_reduce& acc) {
+  int i = 0;
+  unsigned spins = 0;
+  while (i < count) {
+    _slot_t x[_SYNC_AHEAD][_kWords];
+#pragma unroll
+    for (int a = 0; a < _SYNC_AHEAD; ++a) {
+      // (past the last value: the last one again, not used)
+      const int ia = (i + a < count) ? i + a : count - 1;
+#pragma unroll
+      for (int k = 0; k < _kWords; ++k)
+        x[a][k] = __hip_atomic_load(slots + (first + (ptrdiff_t)ia * stride) * _kWords + k,
+                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // (no early exit from the loop: it unrolls whole, and `x` stays in registers)
+    bool stalled = false;
+#pragma unroll
+    for (int a = 0; a < _SYNC_AHEAD; ++a) {
+      bool written = true;
+      unsigned w[_kWords];
+#pragma unroll
+      for (int k = 0; k < _kWords; ++k) {
+        written = written && (unsigned)(x[a][k] >> 32) == epoch;
+        w[k] = (unsigned)x[a][k];
+      }
+      const bool due = !stalled && i < count;
+      if (due && written) {
+        _type_reduce v;
+        __builtin_memcpy(&v, w, sizeof(_type_reduce));
+        acc = REDUCE(acc, v);
+        ++i;
+      }
+      stalled = stalled || (due && !written);
+    }
+    if (stalled) {
+      if (spins >= spin_limit) return false;
+      ++spins;
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+  return true;
+}
+
+// Number of this launch, read by the first wave of every workgroup at its start.
+__device__ __forceinline__ unsigned _sync_epoch(unsigned* sync) {
+  return __hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+}
+
+// The finishing workgroup `x` of `n_finishers` reports; the last one waits
+// for the reports of the others and advances the number of the launch.  One
+// wave, all lanes call.  `done` are the slots after those of the partial
+// results.
+__device__ __forceinline__ void _sync_report(unsigned* sync, _slot_t* done, const ptrdiff_t x,
+                                             const ptrdiff_t n_finishers, const unsigned epoch,
+                                             const unsigned spin_limit, unsigned* fault,
+                                             const ptrdiff_t all_slots) {
+  const int lane = threadIdx.x & 63;
+  if (lane == 0)
+    __hip_atomic_store(done + x, ((_slot_t)epoch << 32), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  if (x != n_finishers - 1) return;
+  bool ok = true;
+  unsigned spins = 0;
+  for (ptrdiff_t i = lane; i < n_finishers - 1; i += 64) {
+    for (;;) {
+      const _slot_t v = __hip_atomic_load(done + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((unsigned)(v >> 32) == epoch) break;
+      if (spins >= spin_limit) { ok = false; break; }
+      ++spins;
+      __builtin_amdgcn_s_sleep(8);
+    }
+    if (!ok) break;
+  }
+  const bool all_ok = __ballot(!ok) == 0;
+  if (!all_ok && lane == 0 && fault) *reinterpret_cast<volatile unsigned*>(fault) = 1u;
+  unsigned next = epoch;
+  if (epoch == 0xffffffffu) {
+    // the numbers start over: nothing may be left that carries an old one
+    _slot_t* slots = reinterpret_cast<_slot_t*>(sync + _SYNC_HEADER_WORDS);
+    for (ptrdiff_t i = lane; i < all_slots; i += 64)
+      __hip_atomic_store(slots + i, (_slot_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    next = 0u;
+  }
+  if (lane == 0)
+    __hip_atomic_store(sync, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+"""
+
+
+def _sync_helpers(reduce_words_hint=2):
+    # values a lane asks for at a time: what fits the registers beside the rest
+    return _SYNC_HELPERS % dict(ahead=8 if reduce_words_hint <= 2 else 4)
+
+
 def _raw_param(a):
     const = 'const ' if a.is_const else ''
     return '%sCArray<%s, %d, %d, %d> %s' % (
         const, a.store_t, a.ndim, a.c_contiguous, a.index_32, a.name)
 
 
-def _fast_params(args, idx_t, partial_in, partial_out):
+def _fast_params(args, idx_t, partial_in, partial_out, finish=False):
     """Parameter list of the rows / cols kernels."""
     parts = []
     for a in args:
@@ -116,7 +251,13 @@ def _fast_params(args, idx_t, partial_in, partial_out):
             parts.append('const %s _sr_%s' % (idx_t, a.name))   # stride along j
         elif a.kind == 'out':
             parts.append('const %s _so_%s' % (idx_t, a.name))
-    if partial_out:
+    if partial_out and finish:
+        # memory of the slots (see _SYNC_HELPERS), workgroups along the outputs
+        parts.append('unsigned* _sync')
+        parts.append('const unsigned _spin_limit')
+        parts.append('unsigned* _fault')
+        parts.append('const %s _gx' % idx_t)
+    elif partial_out:
         parts.append('_type_reduce* __restrict__ _partials')
     return ', '.join(parts)
 
@@ -133,7 +274,10 @@ def _finish(args, partial_out, pad, i_expr='_i', s_expr='_s', split_expr='blockI
     """Code storing one finished value: either into the partial buffer or
     through POST_MAP into the output element(s)."""
     lines = []
-    if partial_out:
+    if partial_out == 'publish':
+        lines.append('%s_sync_publish(_slots, (ptrdiff_t)%s * _n_out + %s, %s, _epoch);' % (
+            pad, split_expr, i_expr, s_expr))
+    elif partial_out:
         lines.append('%s_partials[(ptrdiff_t)%s * _n_out + %s] = %s;' % (
             pad, split_expr, i_expr, s_expr))
     else:
@@ -147,7 +291,8 @@ def _finish(args, partial_out, pad, i_expr='_i', s_expr='_s', split_expr='blockI
 
 def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', group=64, vec=4,
-              idx64=False, partial_out=False, stream_hint=False, unroll=2, block=BLOCK):
+              idx64=False, partial_out=False, stream_hint=False, unroll=2, block=BLOCK,
+              finish=False, reduce_words=2):
     """Reduce-axis-contiguous kernel.  ``group`` lanes per row (power of two up
     to 64) or ``BLOCK`` for a workgroup (of ``block`` threads) per row.  With ``partial_out`` the reduce
     range is cut into gridDim.y chunks of ``_chunk`` elements (an extra kernel
@@ -155,29 +300,49 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     nt = 'true' if stream_hint else 'false'
     ins = [a for a in args if a.kind == 'in']
-    params = _fast_params(args, idx_t, False, partial_out)
+    finish = bool(finish and partial_out and group >= BLOCK)
+    params = _fast_params(args, idx_t, False, partial_out, finish)
     if partial_out:
         params += ', const %s _chunk' % idx_t
     block_mode = group >= BLOCK
     wg = block if block_mode else BLOCK
     lanes = wg if block_mode else group
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    if finish:
+        src.append(_sync_helpers(reduce_words))
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         wg, name, params))
     src.append(_SIZE_INDEXERS)
+    split_of_block = 'blockIdx.y'
+    if finish:
+        # a grid of one dimension, numbered along the outputs first: the
+        # workgroups of one output start in the order of their chunks
+        src.append('  const %s _bx = (%s)(blockIdx.x %% (unsigned)_gx);' % (idx_t, idx_t))
+        src.append('  const %s _by = (%s)(blockIdx.x / (unsigned)_gx);' % (idx_t, idx_t))
+        src.append('  const %s _gy = (%s)(gridDim.x / (unsigned)_gx);' % (idx_t, idx_t))
+        src.append('  _slot_t* _slots = reinterpret_cast<_slot_t*>(_sync + _SYNC_HEADER_WORDS);')
+        # (asked for now, needed when the partial result is there: the first
+        # wave alone uses it)
+        src.append('  unsigned _epoch = 0u;')
+        src.append('  if (threadIdx.x < %d) _epoch = _sync_epoch(_sync);' % WAVE)
+        split_of_block = '_by'
     if block_mode:
         src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];' % (wg // WAVE))
         src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
         src.append('  const int _lane = threadIdx.x;')
-        src.append('  const %s _first = blockIdx.x;' % idx_t)
-        src.append('  const %s _step = gridDim.x;' % idx_t)
+        if finish:
+            src.append('  const %s _first = _bx;' % idx_t)
+            src.append('  const %s _step = _gx;' % idx_t)
+        else:
+            src.append('  const %s _first = blockIdx.x;' % idx_t)
+            src.append('  const %s _step = gridDim.x;' % idx_t)
     else:
         src.append('  const int _lane = threadIdx.x %% %d;' % group)
         src.append('  const %s _first = ((%s)blockIdx.x * %d + threadIdx.x) / %d;' % (
             idx_t, idx_t, BLOCK, group))
         src.append('  const %s _step = (%s)gridDim.x * %d;' % (idx_t, idx_t, BLOCK // group))
     if partial_out:
-        src.append('  const %s _j_begin = (%s)blockIdx.y * _chunk;' % (idx_t, idx_t))
+        src.append('  const %s _j_begin = (%s)%s * _chunk;' % (idx_t, idx_t, split_of_block))
         src.append('  const %s _j_end = (_j_begin + _chunk < _n_red) ? (_j_begin + _chunk) : _n_red;' % idx_t)
     else:
         src.append('  const %s _j_begin = 0;' % idx_t)
@@ -258,9 +423,30 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         src.append('    if (threadIdx.x == 0) {')
         src.append('      _s = _sm[0];')
         src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[_w]);' % (wg // WAVE))
-        src.extend(_finish(args, partial_out, '      '))
+        src.extend(_finish(args, 'publish' if finish else partial_out, '      ',
+                           split_expr=split_of_block))
         src.append('    }')
         src.append('    __syncthreads();')
+        if finish:
+            # the workgroup of the last chunk of output _i finishes it: the
+            # partial results of the chunks, a lane taking every 64th, then
+            # across the lanes
+            src.append('    if (_by == _gy - 1 && threadIdx.x < %d) {' % WAVE)
+            src.append('      _type_reduce _t = %s;' % _identity_decl(identity))
+            src.append('      const int _mine = (int)((_gy - threadIdx.x + %d) / %d);' % (WAVE - 1, WAVE))
+            src.append('      const bool _ok = _sync_fold(_slots, (ptrdiff_t)threadIdx.x * _n_out + _i, '
+                       '(ptrdiff_t)%d * _n_out, _mine, _epoch, _spin_limit, _t);' % WAVE)
+            src.append('      if (__ballot(!_ok) != 0 && threadIdx.x == 0 && _fault) '
+                       '*reinterpret_cast<volatile unsigned*>(_fault) = 1u;')
+            # (lanes without a chunk hold the identity, as lanes without
+            # elements do in the reduction proper)
+            src.append('      _type_reduce _s = cupy::group_allreduce<%d>(_t, _ReduceOp());' % WAVE)
+            src.append('      if (threadIdx.x == 0) {')
+            src.extend(_finish(args, False, '        '))
+            src.append('      }')
+            src.append('      _sync_report(_sync, _slots + (ptrdiff_t)_gy * _n_out * _kWords, _i, _n_out, '
+                       '_epoch, _spin_limit, _fault, (ptrdiff_t)_gy * _n_out * _kWords + _n_out);')
+            src.append('    }')
     else:
         if group > 1:
             src.append('    _s = cupy::group_allreduce<%d>(_s, _ReduceOp());' % group)
@@ -578,7 +764,8 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
 def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
               partial_in=False, partial_out=False, stream_hint=False, unroll=4,
-              solo=False, batched=False, clamp_tail=False, vec_out=False, solo_block=BLOCK):
+              solo=False, batched=False, clamp_tail=False, vec_out=False, solo_block=BLOCK,
+              finish=False, reduce_words=2):
     """Output-axis-contiguous kernel.  Thread layout: ``tx`` threads across
     the output axis (each owning ``vec`` adjacent outputs) times 256/tx slices
     of the reduce axis; gridDim.y further slices.  ``partial_in``: the single
@@ -605,7 +792,8 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     ins = [a for a in args if a.kind == 'in']
     ty = block // tx
     waves = block // WAVE
-    params = _fast_params(args, idx_t, partial_in, partial_out)
+    finish = bool(finish and partial_out and not solo and not batched and not partial_in)
+    params = _fast_params(args, idx_t, partial_in, partial_out, finish)
     if batched:
         assert not partial_in and not any(a.bcast_o for a in ins)
         for a in ins:
@@ -613,6 +801,8 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         params += ', const %s _n_inner, const %s _nbc' % (idx_t, idx_t)
         params += ''.join(', const %s _sb_%s' % (idx_t, a.name) for a in ins)
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    if finish:
+        src.append(_sync_helpers(reduce_words))
     src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
         block, name, params))
     src.append(_SIZE_INDEXERS)
@@ -622,8 +812,22 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
     src.append('  const int _tx = threadIdx.x %% %d;' % tx)
     src.append('  const int _ty = threadIdx.x / %d;' % tx)
-    # column blocks beyond the capacity of grid.x continue along grid.z
-    src.append('  const %s _blk = (%s)blockIdx.z * gridDim.x + blockIdx.x;' % (idx_t, idx_t))
+    if finish:
+        # a grid of one dimension, numbered along the column blocks first: the
+        # workgroups of one column block start in the order of their slices
+        src.append('  const %s _blk = (%s)(blockIdx.x %% (unsigned)_gx);' % (idx_t, idx_t))
+        src.append('  const %s _by = (%s)(blockIdx.x / (unsigned)_gx);' % (idx_t, idx_t))
+        src.append('  const %s _gy = (%s)(gridDim.x / (unsigned)_gx);' % (idx_t, idx_t))
+        src.append('  _slot_t* _slots = reinterpret_cast<_slot_t*>(_sync + _SYNC_HEADER_WORDS);')
+        # (asked for now, needed when the partial results are there)
+        src.append('  __shared__ unsigned _sh_epoch;')
+        src.append('  unsigned _epoch0 = 0u;')
+        src.append('  if (threadIdx.x == 0) _epoch0 = _sync_epoch(_sync);')
+        by_expr, gy_expr = '_by', '_gy'
+    else:
+        # column blocks beyond the capacity of grid.x continue along grid.z
+        src.append('  const %s _blk = (%s)blockIdx.z * gridDim.x + blockIdx.x;' % (idx_t, idx_t))
+        by_expr, gy_expr = '(%s)blockIdx.y' % idx_t, '(%s)gridDim.y' % idx_t
     if batched:
         src.append('  const %s _b = _blk / _nbc;' % idx_t)
         src.append('  const %s _c = ((_blk - _b * _nbc) * %d + _tx) * %d;' % (idx_t, tx, vec))
@@ -651,8 +855,8 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     else:
         src.append('    const bool _full = _c + %d <= _ncol;' % vec)
     src.append('    if (_full) {')
-    src.append('      const %s _jstep = (%s)gridDim.y * %d;' % (idx_t, idx_t, ty))
-    src.append('      %s _j = (%s)blockIdx.y * %d + _ty;' % (idx_t, idx_t, ty))
+    src.append('      const %s _jstep = %s * %d;' % (idx_t, gy_expr, ty))
+    src.append('      %s _j = %s * %d + _ty;' % (idx_t, by_expr, ty))
     # operands that do not vary along the reduce axis are read once
     for a in ins:
         if a.bcast_r and not partial_in:
@@ -719,8 +923,8 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     accumulate('        ', '_j', '')
     src.append('      }')
     src.append('    } else {')
-    src.append('      for (%s _j = (%s)blockIdx.y * %d + _ty; _j < _n_red; _j += (%s)gridDim.y * %d) {' % (
-        idx_t, idx_t, ty, idx_t, ty))
+    src.append('      for (%s _j = %s * %d + _ty; _j < _n_red; _j += %s * %d) {' % (
+        idx_t, by_expr, ty, gy_expr, ty))
     src.append('        const IndexT _J = _j;')
     # a constant trip count with the bound tested inside: the accumulators are
     # then indexed by constants only and stay in registers whatever their type
@@ -795,16 +999,41 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('    for (int _k = 0; _k < %d; ++_k) _sm[(_wave * %d + _tx) * %d + _k] = _acc[_k];' % (
         vec, tx, vec))
     src.append('  }')
+    if finish:
+        src.append('  if (threadIdx.x == 0) _sh_epoch = _epoch0;')
     src.append('  __syncthreads();')
+    if finish:
+        src.append('  const unsigned _epoch = _sh_epoch;')
     src.append('  if (threadIdx.x < %d && _c < _ncol) {' % tx)
     src.append('    for (int _k = 0; _k < %d && _c + _k < _ncol; ++_k) {' % vec)
     src.append('      _type_reduce _s = _sm[_tx * %d + _k];' % vec)
     src.append('      for (int _w = 1; _w < %d; ++_w) _s = REDUCE(_s, _sm[(_w * %d + _tx) * %d + _k]);' % (
         waves, tx, vec))
     src.append('      const %s _i = _i0 + _c + _k;' % idx_t)
-    src.extend(_finish(args, partial_out, '      '))
+    src.extend(_finish(args, 'publish' if finish else partial_out, '      ',
+                       split_expr='_by' if finish else 'blockIdx.y'))
     src.append('    }')
     src.append('  }')
+    if finish:
+        # the workgroup of the last slice finishes the columns of its block: a
+        # thread per column combines the partial results of the slices in
+        # their order
+        src.append('  if (_by == _gy - 1) {')
+        src.append('    bool _ok = true;')
+        src.append('    for (%s _c1 = _blk * %d + threadIdx.x; _c1 < (_blk + 1) * %d && _c1 < _ncol; '
+                   '_c1 += %d) {' % (idx_t, tx * vec, tx * vec, block))
+        src.append('      _type_reduce _s = %s;' % _identity_decl(identity))
+        src.append('      _ok = _sync_fold(_slots, (ptrdiff_t)_i0 + _c1, (ptrdiff_t)_n_out, (int)_gy, '
+                   '_epoch, _spin_limit, _s) && _ok;')
+        src.append('      const %s _i = _i0 + _c1;' % idx_t)
+        src.extend(_finish(args, False, '      '))
+        src.append('    }')
+        src.append('    if (!_ok && _fault) *reinterpret_cast<volatile unsigned*>(_fault) = 1u;')
+        src.append('    __syncthreads();')
+        src.append('    if (threadIdx.x < %d)' % WAVE)
+        src.append('      _sync_report(_sync, _slots + (ptrdiff_t)_gy * _n_out * _kWords, _blk, _gx, '
+                   '_epoch, _spin_limit, _fault, (ptrdiff_t)_gy * _n_out * _kWords + _gx);')
+        src.append('  }')
     src.append('}')
     return '\n'.join(src) + '\n'
 

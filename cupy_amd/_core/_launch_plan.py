@@ -102,12 +102,18 @@ class ArgBlock:
 
 class Recorder:
     """Collects the launches and temporaries of one call."""
-    __slots__ = ('n_refs', 'launches', 'temps')
+    __slots__ = ('n_refs', 'launches', 'temps', 'stream')
 
     def __init__(self, n_refs):
         self.n_refs = n_refs      # user arguments + allocated outputs
         self.launches = []
         self.temps = []
+        self.stream = None        # the one stream the launches may be replayed on
+
+    def bind_stream(self, stream_ptr):
+        """The recorded launches name memory that belongs to ``stream_ptr``:
+        a replay on another stream takes the full path."""
+        self.stream = stream_ptr
 
     def temp(self, nbytes):
         """Registers a temporary of ``nbytes``; returns its ref number."""
@@ -147,7 +153,8 @@ def ranges_overlap(a, b):
 class FastCall:
     """Recorded call: allocates outputs and temporaries, patches pointers and
     scalar values, launches."""
-    __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap', 'quick')
+    __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap', 'quick',
+                 'stream')
 
     def __init__(self, n_user, out_specs, rec, ret, overlap=()):
         self.n_user = n_user
@@ -157,9 +164,15 @@ class FastCall:
         self.ret = ret                        # ref, tuple of refs, or None
         self.overlap = tuple(overlap)         # (input ref, output ref) pairs to check
         self.quick = _quick_launches(self.launches)
+        self.stream = rec.stream
 
     def run(self, args, stream_ptr=None):
         from cupy_amd._core.core import ndarray
+        if self.stream is not None:
+            if stream_ptr is None:
+                stream_ptr = _stream.get_current_stream_ptr()
+            if stream_ptr != self.stream:
+                return NotImplemented
         for i, o in self.overlap:
             a, b = args[i], args[o]
             # (arrays of different allocations cannot overlap)

@@ -22,6 +22,7 @@ from cupy_amd._core import _carray
 from cupy_amd._core import _codegen_reduction as _cg
 from cupy_amd._core import _kernel
 from cupy_amd._core import _launch_plan
+from cupy_amd._core import _reduce_sync
 from cupy_amd._core import _tuning
 from cupy_amd._core import internal
 from cupy_amd._core._codegen_elementwise import uses_identifier
@@ -97,6 +98,43 @@ _known_type_sizes = {
     'unsigned short': 2, 'int': 4, 'unsigned int': 4, 'long long': 8,
     'unsigned long long': 8, 'float16': 2, 'float': 4, 'double': 8,
 }
+
+
+_TYPEDEF = re.compile(r'typedef\s+(.+?)\s+(\w+)\s*;')
+_WRAPPED = re.compile(r'(mm_val|arg_state|var_st)\s*<\s*([^,>]+(?:<[^>]*>)?)\s*(?:,[^>]*)?>(?:::type)?')
+
+
+def _reduce_type_bytes(reduce_type, typedefs):
+    """Upper bound of ``sizeof`` of a reduction type, from its name alone
+    (the same with and without a device): exact for the arithmetic types, the
+    complex types and the structures of the min/max, argmin/argmax and
+    variance reductions, 64 for anything else."""
+    names = dict((name, what) for what, name in _TYPEDEF.findall(typedefs))
+
+    def plain(t):
+        t = names.get(t.strip(), t.strip())
+        size = _known_type_sizes.get(t)
+        if size is None:
+            size = {'complex<float>': 8, 'complex<double>': 16}.get(t.replace(' ', ''))
+        return size
+
+    size = plain(reduce_type)
+    if size is not None:
+        return size
+    m = _WRAPPED.fullmatch(reduce_type.strip())
+    inner = plain(m.group(2)) if m else None
+    if inner is None:
+        return 64
+    if m.group(1) == 'mm_val':
+        return inner
+    if m.group(1) == 'var_st':
+        return 4 * inner
+    # argmin / argmax: values of 4 bytes at most with 32-bit indices travel as
+    # one 64-bit key, the others as (value, index of 8 bytes)
+    if inner <= 4 and names.get('IndexT', '').strip() == 'int' and 'complex' not in (
+            names.get(m.group(2).strip(), m.group(2))):
+        return 8
+    return 8 + (inner + 7) // 8 * 8
 
 
 _SIZE_CALL = re.compile(r'\b_(?:in|out)_ind\s*\.\s*size\s*\(\s*\)')
@@ -661,6 +699,12 @@ class _AbstractReductionKernel:
         span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
                    + [abs(s) * n_out for s in so_out] + [n_red + chunk])
         idx64 = span > _INT32_MAX - (1 << 24)
+        finish, words_hint = None, 2
+        if n_split > 1 and not stage and n_out <= _max_blocks(wg):
+            words_hint, finish = self._finish_memory(
+                ins, n_out, n_red, so_in, sr, reduce_type, typedefs,
+                lambda words: n_split * n_out * words + n_out, (n_split + 63) // 64,
+                False, device_id, stream_ptr)
         batch = _tuning.get('rows_batch')
         trips = 1
         batched = (group < _cg.BLOCK and batch >= 1 and n_red <= group * vec and not stage
@@ -686,7 +730,7 @@ class _AbstractReductionKernel:
         rargs = self._rargs(in_args, out_args, bcast_r=bcast_r, bcast_o=bcast_o)
         key = ('rows', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, group, vec, idx64, partial, device_id,
-               batched, trips, exact, stream_hint, wg, _tuning.signature())
+               batched, trips, exact, stream_hint, wg, bool(finish), _tuning.signature())
 
         def emit():
             if batched:
@@ -700,7 +744,8 @@ class _AbstractReductionKernel:
                 post_map_expr, reduce_type, typedefs, preamble, group=group,
                 vec=vec, idx64=idx64, partial_out=partial,
                 stream_hint=stream_hint,
-                unroll=_tuning.get('rows_unroll'), block=wg)
+                unroll=_tuning.get('rows_unroll'), block=wg,
+                finish=bool(finish), reduce_words=words_hint)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
@@ -713,7 +758,16 @@ class _AbstractReductionKernel:
             rows_per_block = _cg.BLOCK // group * (batch if batched else 1)
             gx = min((n_out + rows_per_block - 1) // rows_per_block,
                      cus * _tuning.get('rows_group_rows_per_lane'))
-        if partial:
+        if finish:
+            # one launch: the workgroup of the last chunk of every row combines
+            # the partial results of the others
+            if rec is not None:
+                rec.bind_stream(stream_ptr)
+            vals.const(finish[0], _tuning.get('reduce_finish_spin_limit'), finish[1], gx, chunk)
+            _launch_plan.launch(
+                rec, fn, (gx * n_split, 1, 1), (wg, 1, 1),
+                _make_packer(self._fast_format(rargs, ic, 'PIP' + ic + ic)), vals, stream_ptr)
+        elif partial:
             rsize = self._reduce_type_size(reduce_type, mod)
             partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
             vals.ptr(pref, partials.ptr)
@@ -742,6 +796,34 @@ class _AbstractReductionKernel:
         for a, s_o, s_r in zip(ins, so_in, sr):
             total += a.dtype.itemsize * (n_out if s_o else 1) * (n_red if s_r else 1)
         return total
+
+    def _finish_memory(self, ins, n_out, n_red, so_in, sr, reduce_type, typedefs, n_slots_of,
+                       per_lane, by_thread, device_id, stream_ptr):
+        """Decides whether a split reduction finishes inside its one launch.
+        Returns ``(hint, None)`` or ``(hint, (block address, fault address))``:
+        ``hint`` tells whether the reduction type fits two 32-bit words, as far
+        as its name tells (2 or 4: it selects how many partial results a lane
+        asks for at a time), the pair
+        names the memory of the slots.  ``n_slots_of(words)`` gives the slots
+        the launch needs for a type of that many words, ``per_lane`` is the
+        number of partial results the busiest lane of a finishing workgroup
+        combines; ``by_thread`` says that a thread does so for a column on its
+        own (no other lanes share the work: the words it has to fetch are
+        limited as well)."""
+        words = (_reduce_type_bytes(reduce_type, typedefs) + 3) // 4
+        hint = 2 if words <= 2 else 4
+        if self._read_bytes(ins, n_out, n_red, so_in, sr) > _tuning.get('reduce_finish_max_bytes'):
+            return hint, None
+        # a lane asks for 8 partial results at a time (4 of the wider types)
+        # and waits for them: beyond a few such round trips the second launch
+        # is quicker
+        if per_lane > _tuning.get('reduce_finish_round_trips') * (8 if hint == 2 else 4):
+            return hint, None
+        if by_thread and per_lane * words > 32:
+            return hint, None
+        got = _reduce_sync.acquire(device_id, stream_ptr, _stream.get_current_stream_ptr(),
+                                   n_slots_of(words))
+        return hint, got
 
     @staticmethod
     def _alloc_partials(rec, nbytes):
@@ -802,6 +884,12 @@ class _AbstractReductionKernel:
                 abs(s_b) * n_batch + abs(s_r) * n_red + s_o * n_cols
                 for s_b, s_r, s_o in zip(sb, sr, so_in)])
         idx64 = span > _INT32_MAX - (1 << 24)
+        finish, words_hint = None, 2
+        if partial and not batch and not solo and gz == 1:
+            words_hint, finish = self._finish_memory(
+                ins, n_out, n_red, so_in, sr, reduce_type, typedefs,
+                lambda words: n_split * n_out * words + gx, n_split, True, device_id,
+                stream_ptr)
         rargs = self._rargs(in_args, out_args, bcast_r=[s == 0 for s in sr], bcast_o=bcast_o)
         clamp = bool(n_cols % vec and n_cols >= vec and _tuning.get('unaligned_vectors'))
         outs = [out_args[i] for i in out_arr_idx]
@@ -817,7 +905,8 @@ class _AbstractReductionKernel:
             _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
-               stream_hint, solo, bool(batch), clamp, unroll, vec_out, block, _tuning.signature())
+               stream_hint, solo, bool(batch), clamp, unroll, vec_out, block, bool(finish),
+               _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
@@ -825,7 +914,8 @@ class _AbstractReductionKernel:
                 post_map_expr, reduce_type, typedefs, preamble, tx=tx, vec=vec,
                 idx64=idx64, partial_out=partial,
                 stream_hint=stream_hint, unroll=unroll, solo=solo,
-                batched=bool(batch), clamp_tail=clamp, vec_out=vec_out, solo_block=solo_block)
+                batched=bool(batch), clamp_tail=clamp, vec_out=vec_out, solo_block=solo_block,
+                finish=bool(finish), reduce_words=words_hint)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
@@ -833,7 +923,16 @@ class _AbstractReductionKernel:
         if batch:
             tail = ic * (2 + len(ins))
             batch_vals = [n_cols, nbc] + [s // a.dtype.itemsize for s, a in zip(sb, ins)]
-        if partial:
+        if finish:
+            # one launch: the workgroup of the last slice of every column block
+            # combines the partial results of the others
+            if rec is not None:
+                rec.bind_stream(stream_ptr)
+            vals.const(finish[0], _tuning.get('reduce_finish_spin_limit'), finish[1], gx)
+            _launch_plan.launch(
+                rec, fn, (gx * n_split, 1, 1), (block, 1, 1),
+                _make_packer(self._fast_format(rargs, ic, 'PIP' + ic)), vals, stream_ptr)
+        elif partial:
             rsize = self._reduce_type_size(reduce_type, mod)
             partials, pref = self._alloc_partials(rec, rsize * n_split * n_out)
             vals.ptr(pref, partials.ptr)

@@ -2,7 +2,7 @@
 from cupy_amd._core import _fusion_thread_local
 from cupy_amd._core._reduction import create_reduction_func
 
-_all_sigs = tuple('%s->?' % c for c in '?bBhHiIlLqQefd')
+_all_sigs = tuple('%s->?' % c for c in '?bBhHiIlLqQefdFD')
 
 _all = create_reduction_func(
     'cupy_all', _all_sigs,

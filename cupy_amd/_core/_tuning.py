@@ -138,6 +138,11 @@ _params = {
     # False restricts vectors to operands aligned to the whole vector.
     'unaligned_vectors': True,
     'mid_flat_lines_per_lane': 32,
+    'reduce_finish': True,      # split reductions of moderate size finish inside the launch that makes the partial results
+    'reduce_finish_max_bytes': 16 << 20,   # ... up to this much input (beyond, a second launch is quicker)
+    'reduce_finish_round_trips': 4,        # ... and while a finishing lane waits for partial results this often at most
+    'reduce_finish_max_slots': 1 << 20,    # ... and up to this many words of partial results
+    'reduce_finish_spin_limit': 1 << 22,   # polls before a waiting workgroup gives up
     'mid_flat': True,           # middle-axis reductions of short slices with few columns through the LDS
     'target_blocks_per_cu': 8,  # split the reduce axis until the grid has this many
     'min_blocks_per_cu': 2,     # ... but only if it would otherwise have fewer than this

@@ -202,6 +202,11 @@ def test_launch_plans_of_the_benchmark_shapes():
     ls = launches_of(lambda: a.sum())
     assert [x[0] for x in ls] == ['cupy_sum', 'cupy_sum_combine']
     assert ls[0][1][0] == 1 and ls[0][1][1] >= 256     # split over the grid
+    # up to 16 MiB a split reduction finishes in its one launch (the first on a
+    # stream also clears the memory the workgroups hand their results over in)
+    c = cp.ndarray((1 << 21,), np.float32)
+    ls = [x for x in launches_of(lambda: c.sum()) if not x[0].startswith('cupy_copy')]
+    assert [x[0] for x in ls] == ['cupy_sum'] and ls[0][1][0] >= 256 and ls[0][1][1] == 1
 
     m = cp.ndarray((4096, 128), np.int32)
     (l,) = launches_of(lambda: m.argmax(axis=-1))

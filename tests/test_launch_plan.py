@@ -219,8 +219,43 @@ def test_reduction_replay_with_and_without_partials():
         return (cp.ndarray((1 << 22,), np.float32), cp.ndarray((), np.float32))
 
     from cupy_amd._core import _routines_math as rm
+    from cupy_amd._core import _tuning
     sumk = rm._sum_auto_dtype
     check_replay(lambda: [sumk._fast_calls], lambda a, o: sumk(a, 1, None, o, False), rows, known)
+    _tuning.set(reduce_finish=False)
+    try:
+        _split_reductions_in_two_launches(sumk, cols_split, full, known)
+    finally:
+        _tuning.set(reduce_finish=True)
+    # split reductions that finish in their one launch: the first call on a
+    # stream also clears the memory the workgroups hand their results over in;
+    # replays launch the one kernel with the same arguments
+    def cols_short():
+        return (cp.ndarray((512, 512), np.float64), cp.ndarray((512,), np.float64))
+
+    for make, axis in ((cols_short, 0), (full, None)):
+        a, o = make()
+        _, first = launches_of(lambda: sumk(a, axis, None, o, False))
+        assert [l[0] for l in first if not l[0].startswith('cupy_copy')] == ['cupy_sum']
+        _, again = launches_of(lambda: sumk(a, axis, None, o, False))
+        assert [l[0] for l in again] == ['cupy_sum']
+        k = known((a, o))
+        assert describe(again, k) == describe(first[-1:], k)
+        b, p = make()
+        _, other = launches_of(lambda: sumk(b, axis, None, p, False))
+        assert describe(other, known((b, p))) == describe(again, k)
+        # on another stream the recorded call is not used: that stream gets
+        # memory of its own
+        side = cp.cuda.Stream()
+        with side:
+            _, elsewhere = launches_of(lambda: sumk(a, axis, None, o, False))
+        assert [l[0] for l in elsewhere if not l[0].startswith('cupy_copy')] == ['cupy_sum']
+        if side.ptr != cp.cuda.get_current_stream().ptr:
+            assert (words(elsewhere[-1][4], names((a, o)))
+                    != words(again[-1][4], names((a, o))))
+
+
+def _split_reductions_in_two_launches(sumk, cols_split, full, known):
     check_replay(lambda: [sumk._fast_calls], lambda a, o: sumk(a, 0, None, o, False), cols_split, known)
     check_replay(lambda: [sumk._fast_calls], lambda a, o: sumk(a, None, None, o, False), full, known)
     # the split reductions launch two kernels sharing one temporary

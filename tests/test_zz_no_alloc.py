@@ -65,6 +65,19 @@ def _recorded_call(fn):
     return found[-1]
 
 
+@pytest.fixture(autouse=True)
+def _reductions_with_scratch_memory():
+    """The calls here are reductions that keep partial results in scratch
+    memory for a second launch; reductions of this size would otherwise finish
+    inside their one launch and use none."""
+    from cupy_amd._core import _tuning
+    _tuning.set(reduce_finish=False)
+    try:
+        yield
+    finally:
+        _tuning.set(reduce_finish=True)
+
+
 _MARK = 0x1badc0de1badc0de
 
 
