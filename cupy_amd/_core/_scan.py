@@ -1985,17 +1985,38 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
     return True
 
 
+def _chunk_below(cus, n, want):
+    """Number of slices below which the staged and the lane-interleaved kernels
+    cut the slices into chunks.  Slices of fewer than 4096 rows are better off
+    whole, a wave each, while there are four waves per CU: 2^26 floats in
+    slices of 1024 x 16 143 us cut up, 114 whole; of 1024 x 36 148 -> 113, of
+    512 x 64 142 -> 117, of 257 x 100 186 -> 132; with fewer waves than that
+    whole slices lose (8192 x 16 from 512 waves: 186 against 105), and longer
+    slices do well in the one-pass kernels (16384 x 3: 107 against 125)."""
+    if n < 4096:
+        return min(want, cus * _tuning.get('scan_whole_slices_waves_per_cu'))
+    return want
+
+
 def _scan_packed(src, dst, outer, n, inner, op, skip_nan, vec, trips, idx64, stream, stream_ptr,
                  cus):
-    """Launches ``_emit_tile_packed`` where at least four slices fit a round
-    (with two the plain kernels are as good: 2^17 slices of 32 x 16 floats
-    86.6 us against 91.5).  Returns False otherwise."""
+    """Launches ``_emit_tile_packed`` where several slices fit a round: two for
+    rows that are no whole vectors, else four (with two the plain kernels are
+    as good there: 2^17 slices of 32 x 16 floats 86.6 us against 91.5).
+    Returns False otherwise."""
     if outer < 2 or not _tuning.get('scan_tile_packed'):
         return False
     while _tile_geometry(inner, vec, trips)[2] > 32 and trips > 1:
         trips //= 2       # (a lane marks the slice starts among its rows in 64 bits)
     rows_t, _, lrows, _ = _tile_geometry(inner, vec, trips)
-    if 4 * n > rows_t or lrows > 64:
+    # (rows that are whole vectors do as well a slice to a wave down to a third
+    # of a round: 2^26 floats in slices of 24 x 16 88 us against 96 here; others
+    # do not: 100 x 3 180 against 97, 60 x 5 241 against 95, 12 x 31 130
+    # against 93, 10 x 33 176 against 98)
+    least = _tuning.get('scan_tile_packed_min_slices')
+    if not least:
+        least = 4 if inner == 1 or inner % vec == 0 else 2
+    if least * n > rows_t or lrows > 64:
         return False
     round_rows = rows_t // n * n
     mod = _module_tile_packed(src.dtype, dst.dtype, op, skip_nan, vec, trips, idx64, inner, stream)
@@ -2115,7 +2136,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
             return
         want = cus * _tuning.get('scan_waves_per_cu')
         n_chunks = 1
-        if may_chunk and outer < want and n > 2 * rows_t:
+        if may_chunk and outer < _chunk_below(cus, n, want) and n > 2 * rows_t:
             n_chunks = min((want + outer - 1) // outer, (n + rows_t - 1) // rows_t)
         if n_chunks > 1 and _scan_chained(src, dst, outer, n, op, skip_nan, vec, idx64, stream,
                                           stream_ptr, inner=inner):
@@ -2149,7 +2170,7 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         per_wave = trip_rows * trips
         want = cus * _tuning.get('scan_waves_per_cu')
         n_chunks = 1
-        if may_chunk and outer < want and n > 2 * per_wave:
+        if may_chunk and outer < _chunk_below(cus, n, want) and n > 2 * per_wave:
             n_chunks = min((want + outer - 1) // outer, (n + per_wave - 1) // per_wave)
         if n_chunks > 1 and _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64,
                                                stream, stream_ptr):
@@ -2213,7 +2234,10 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
                 if vec_bytes < item and vec_bytes != 16:
                     continue
                 vec, threads = threads_with(vec_bytes)
-                if threads >= cus * need:
+                # (8-byte vectors from three quarters of that on: 2^26 floats
+                # in slices of 257 x 100, 130550 threads, 167 us against 204
+                # element-wide)
+                if threads >= cus * need * (0.75 if vec_bytes == 8 else 1):
                     one_pass_trips = rows
                     break
             else:

@@ -101,6 +101,7 @@ _params = {
     'scan_tile_max_inner': 64,  # widest tail the staged kernels take
     'scan_lanes': True,
     'scan_tile_packed': True,   # slices of few rows and a narrow tail: many to a wave
+    'scan_tile_packed_min_slices': 0,   # ... when at least this many slices fit one round of a wave (0: by the shape)
     'scan_complex_as_real': True,   # cumsum of complex arrays: as real arrays with twice the columns
     'scan_cols_vec_bytes': 0,
     'scan_chain_cols': True,    # one-pass kernel for many long columns
@@ -120,6 +121,7 @@ _params = {
     'scan_chain_sleep': 8,      # ... and pauses this many times 64 clocks between two polls
     'scan_chain_spin_limit': 1 << 18,   # polls after which a tile of that kernel gives up waiting
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
+    'scan_whole_slices_waves_per_cu': 4,   # ... slices of fewer than 4096 rows with a narrow tail stay whole from this many on
     # fused row-wise functions: words per lane up to which a wave takes a whole row
     'fused_rows': True,         # row-wise fused functions as one kernel (False: one kernel per piece)
     # (measured with a softmax: rows of 4096 float32 74.7 % of peak with a

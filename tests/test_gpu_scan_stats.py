@@ -394,7 +394,12 @@ def test_narrow_scans_of_other_types_and_operations():
 @pytest.mark.parametrize('shape', [(40000, 4, 4), (30001, 16, 2), (5000, 2, 32), (20011, 5, 3),
                                    (7001, 9, 7), (3, 100, 2), (100000, 3, 2), (1500, 33, 8),
                                    (2, 7, 4, 5), (9000, 3, 33), (701, 100, 63), (40, 5000, 64),
-                                   (3, 20000, 40)])
+                                   (3, 20000, 40),
+                                   # two or three slices to a round
+                                   (3001, 100, 3), (2000, 150, 3), (3000, 60, 5), (999, 70, 7),
+                                   (4001, 12, 31), (3000, 10, 33), (2500, 6, 48),
+                                   # slices of several rounds, a wave each
+                                   (1100, 300, 36), (1030, 257, 100), (1025, 500, 16)])
 def test_scans_of_many_short_slices_with_a_narrow_tail(shape):
     """Slices of few rows: a wave stages many of them per round and starts
     over at every slice."""
