@@ -763,6 +763,184 @@ def _module_tile_packed(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, in
     return mod
 
 
+_SLAB_TRIPS = 8
+
+
+def _emit_slab(in_t, out_t, op, skip_nan, vec, idx64, stream):
+    """Scan along the middle axis of (outer, n, inner) where a whole slice of
+    n x inner elements fits the LDS of a workgroup, however wide and however
+    aligned its rows: a workgroup takes a slab of consecutive whole slices --
+    one contiguous piece of memory, read with full vectors on consecutive
+    lanes --, lays it out in the LDS, a thread per column walks down the rows
+    there, and the slab goes back in one contiguous store."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define BLOCK %(block)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define SLAB_ELEMS (BLOCK * VEC * TRIPS)
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+
+// total = outer * n * inner elements; a slab is slab_elems of them, a whole
+// number of slices and SLAB_ELEMS at most.
+extern "C" __global__ void __launch_bounds__(BLOCK) cupy_scan_slab(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, const _idx_t total,
+    const int n, const int inner, const int slab_elems) {
+  __shared__ _acc_t lds[SLAB_ELEMS];
+  const int slice_elems = n * inner;
+  const _idx_t n_slabs = (total + slab_elems - 1) / slab_elems;
+  for (_idx_t slab = blockIdx.x; slab < n_slabs; slab += gridDim.x) {
+    const _idx_t base = slab * slab_elems;
+    const int valid = (total - base < slab_elems) ? (int)(total - base) : slab_elems;
+    const _in_t* src = in + (ptrdiff_t)base;
+    _out_t* dst = out + (ptrdiff_t)base;
+    // every load of the slab is requested before the first value is used
+    cupy::Vec<_in_t, VEC> raw[TRIPS];
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * BLOCK + (int)threadIdx.x) * VEC;
+      if (p + VEC <= valid) {
+        raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + p);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) raw[t].v[k] = (p + k < valid) ? src[p + k] : _in_t();
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * BLOCK + (int)threadIdx.x) * VEC;
+      if (p < valid) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) lds[p + k] = _load_value(raw[t].v[k]);
+      }
+    }
+    __syncthreads();
+    // a thread per column of a slice
+    const int columns = (valid / slice_elems) * inner;
+    for (int q = threadIdx.x; q < columns; q += BLOCK) {
+      const int s = q / inner;
+      _acc_t* at = lds + s * slice_elems + (q - s * inner);
+      _acc_t acc = at[0];
+#pragma unroll 4
+      for (int r = 1; r < n; ++r) {
+        acc = SCAN_OP(acc, at[(ptrdiff_t)r * inner]);
+        at[(ptrdiff_t)r * inner] = acc;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < TRIPS; ++t) {
+      const int p = (t * BLOCK + (int)threadIdx.x) * VEC;
+      if (p + VEC <= valid) {
+        cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(lds[p + k]);
+        cupy::store_vec<_out_t, VEC, NT_STORE>(dst + p, r);
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          if (p + k < valid) dst[p + k] = static_cast<_out_t>(lds[p + k]);
+      }
+    }
+    // (the next slab overwrites what the stores above read)
+    __syncthreads();
+  }
+}
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, vec=vec, trips=_SLAB_TRIPS, conv=conv, block=_BLOCK,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
+
+
+def _module_slab(in_dtype, out_dtype, op, skip_nan, vec, idx64, stream):
+    key = ('slab', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan,
+           vec, idx64, stream)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_slab(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                         vec, idx64, stream)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
+def _slab_pays(src, dst, n, inner, item):
+    """Whether slices that fit the LDS of a workgroup go through
+    ``_emit_slab``, which runs at 65-70 % of peak whatever the shape, rather
+    than through the kernels for narrow, medium and wide rows.  Measured on
+    2^26 floats (us, slab against the others): rows that are no whole vectors
+    -- 2 x 65 103 / 165, 64 x 65 109 / 178, 16 x 257 111 / 168, 33 x 33
+    101 / 131, 33 x 17 102 / 130 -- and rows that leave lanes of the
+    lane-interleaved kernel idle -- 2 x 100 98 / 138, 33 x 100 99 / 126 -- gain;
+    rows of whole vectors that fill the lanes do not: 2 x 128 97 / 89, 2 x 4096
+    97 / 88, 7 x 64 96 / 90, but 7 x 1000 98 / 107."""
+    setting = _tuning.get('scan_slab_min_inner')
+    if setting is not None:
+        return inner > setting
+    vec = max(1, 16 // item)
+    # (a thread walks down a column: long columns want a wave's worth of them
+    # to a slab; 400 x 3: 180 us against 98, 126 x 65: 113 against 205)
+    if n > 64 and (_BLOCK * min(vec, 4) * _SLAB_TRIPS) // (n * inner) * inner < _WAVE:
+        return False
+    whole = (inner % vec == 0 and _aligned(src.data.ptr, 16) and _aligned(dst.data.ptr, 16))
+    if inner > 64:
+        if not whole:
+            return True
+        lstride = inner // vec
+        if lstride <= 32:
+            return 64 % lstride != 0
+        return n >= 5
+    if whole:
+        return False
+    # narrow rows: where the staged kernels leave much of a round empty
+    rows_t = _tile_geometry(inner, vec, 4)[0]
+    if 2 * n <= rows_t:
+        used = rows_t // n * n          # whole slices to a round
+        rounds = 1
+    else:
+        used = n
+        rounds = (n + rows_t - 1) // rows_t
+    return used < 0.7 * rounds * rows_t
+
+
+def _scan_slab(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr, cus):
+    """Launches ``_emit_slab`` where a slice fits the LDS; returns False
+    otherwise."""
+    if not _tuning.get('scan_slab'):
+        return False
+    item = max(src.dtype.itemsize, dst.dtype.itemsize, _acc_dtype(dst.dtype).itemsize)
+    vec = max(1, min(4, 16 // item))
+    capacity = _BLOCK * vec * _SLAB_TRIPS
+    slice_elems = n * inner
+    if slice_elems > capacity:
+        return False
+    # whole slices to a slab, and slabs enough for every CU
+    per_slab = max(1, min(capacity // slice_elems, outer // (cus * 8)))
+    slab_elems = per_slab * slice_elems
+    n_slabs = (outer + per_slab - 1) // per_slab
+    mod = _module_slab(src.dtype, dst.dtype, op, skip_nan, vec, idx64, stream)
+    grid = max(1, min(n_slabs, cus * _tuning.get('scan_blocks_per_cu')))
+    blob = struct.pack('@PP' + ('q' if idx64 else 'i') + 'iii', src.data.ptr, dst.data.ptr,
+                       outer * n * inner, n, inner, slab_elems)
+    mod.get_function('cupy_scan_slab').launch_packed(
+        (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+    return True
+
+
+
 _CHAIN_WAVES = _BLOCK // _WAVE
 _CHAIN_HEADER_WORDS = 64            # the ticket counter, padded to 256 bytes
 
@@ -2119,6 +2297,9 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         prefix = 'cupy_scan_rows'
         totals_shape = (outer, n_chunks, 1)
         middle_round = _WAVE * 4 * 4          # elements one wave takes per round
+    elif (inner >= 2 and n >= 2 and _slab_pays(src, dst, n, inner, item)
+          and _scan_slab(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr, cus)):
+        return
     elif (2 <= inner <= (_tuning.get('scan_tile_max_inner') if n < 16384 else 32)
           and _tuning.get('scan_tile')):
         # (33 to 64 columns: a lane per column, half the wave idle while it

@@ -100,6 +100,8 @@ _params = {
     'scan_rows_packed': True,
     'scan_tile_max_inner': 64,  # widest tail the staged kernels take
     'scan_lanes': True,
+    'scan_slab': True,          # slices with wide rows that fit the LDS: a workgroup stages whole slices
+    'scan_slab_min_inner': None,   # ... for rows wider than this (None: by the shape)
     'scan_tile_packed': True,   # slices of few rows and a narrow tail: many to a wave
     'scan_tile_packed_min_slices': 0,   # ... when at least this many slices fit one round of a wave (0: by the shape)
     'scan_complex_as_real': True,   # cumsum of complex arrays: as real arrays with twice the columns

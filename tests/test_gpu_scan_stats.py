@@ -399,7 +399,10 @@ def test_narrow_scans_of_other_types_and_operations():
                                    (3001, 100, 3), (2000, 150, 3), (3000, 60, 5), (999, 70, 7),
                                    (4001, 12, 31), (3000, 10, 33), (2500, 6, 48),
                                    # slices of several rounds, a wave each
-                                   (1100, 300, 36), (1030, 257, 100), (1025, 500, 16)])
+                                   (1100, 300, 36), (1030, 257, 100), (1025, 500, 16),
+                                   # wide rows, slices that fit the LDS of a workgroup
+                                   (700, 16, 257), (300, 3, 1000), (50, 33, 100), (9, 2, 4096),
+                                   (1000, 81, 100), (5, 8, 65), (2100, 7, 129)])
 def test_scans_of_many_short_slices_with_a_narrow_tail(shape):
     """Slices of few rows: a wave stages many of them per round and starts
     over at every slice."""
