@@ -44,6 +44,23 @@ _memo = {}
 _lock = threading.Lock()
 
 
+def _start_text(op, acc_t):
+    """Arguments of the accumulator's constructor for the value a scan starts
+    from.  For sums of floating-point values that is the NEGATIVE zero, the
+    one value that leaves every other unchanged when added to it
+    (0.0 + -0.0 is 0.0: a scan that starts from 0.0 turns a leading -0.0 into
+    0.0, which neither NumPy nor the reference's in-place scan does;
+    cupy/_core/_routines_math.pyx:160-751).  A NaN that ``nancumsum`` skips
+    still counts as 0.0."""
+    if op != _SUM:
+        return '1'
+    if acc_t.startswith('complex'):
+        return '-0.0, -0.0'
+    if acc_t in ('float', 'double'):
+        return '-0.0'
+    return '0'
+
+
 def _acc_type(t):
     return 'float' if t == 'float16' else t
 
@@ -64,7 +81,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -271,7 +288,7 @@ ROWS_KERNEL(cupy_scan_rows_seeded, 2)
 COLS_KERNEL(cupy_scan_cols, 0)
 COLS_KERNEL(cupy_scan_cols_totals, 1)
 COLS_KERNEL(cupy_scan_cols_seeded, 2)
-''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident,
+''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident, start=_start_text(op, acc_t),
            vec=vec, trips=trips, conv=conv, block=_BLOCK, group=group,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
            ragged=1 if ragged else 0, reuse=1 if reuse else 0)
@@ -299,7 +316,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -422,7 +439,7 @@ LANES_KERNEL(cupy_scan_lanes, 0)
 LANES_KERNEL(cupy_scan_lanes_totals, 1)
 LANES_KERNEL(cupy_scan_lanes_seeded, 2)
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
-           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=trips, conv=conv, block=_BLOCK,
            lstride=lstride, ntl='true' if stream[0] else 'false',
            nts='true' if stream[1] else 'false')
 
@@ -464,7 +481,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -593,7 +610,7 @@ TILE_KERNEL(cupy_scan_tile, 0)
 TILE_KERNEL(cupy_scan_tile_totals, 1)
 TILE_KERNEL(cupy_scan_tile_seeded, 2)
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
-           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=trips, conv=conv, block=_BLOCK,
            inner=inner, rows_t=rows_t, seg=seg, lrows=lrows, stride=stride,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
            reuse=1 if reuse else 0)
@@ -621,7 +638,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -745,7 +762,7 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_tile_packed(
   }
 }
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
-           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=trips, conv=conv, block=_BLOCK,
            inner=inner, rows_t=rows_t, seg=seg, lrows=lrows, stride=stride,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
 
@@ -834,10 +851,22 @@ extern "C" __global__ void __launch_bounds__(BLOCK) cupy_scan_slab(
       const int s = q / inner;
       _acc_t* at = lds + s * slice_elems + (q - s * inner);
       _acc_t acc = at[0];
-#pragma unroll 4
-      for (int r = 1; r < n; ++r) {
-        acc = SCAN_OP(acc, at[(ptrdiff_t)r * inner]);
-        at[(ptrdiff_t)r * inner] = acc;
+      int r = 1;
+      // (eight rows requested before the first is used: the compiler keeps
+      // every read behind the write before it, which would cost the latency
+      // of the LDS per row)
+      for (; r + 8 <= n; r += 8) {
+        _acc_t x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = at[(r + u) * inner];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { acc = SCAN_OP(acc, x[u]); x[u] = acc; }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) at[(r + u) * inner] = x[u];
+      }
+      for (; r < n; ++r) {
+        acc = SCAN_OP(acc, at[r * inner]);
+        at[r * inner] = acc;
       }
     }
     __syncthreads();
@@ -860,7 +889,7 @@ extern "C" __global__ void __launch_bounds__(BLOCK) cupy_scan_slab(
   }
 }
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
-           op_c=op_c, ident=ident, vec=vec, trips=_SLAB_TRIPS, conv=conv, block=_BLOCK,
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=_SLAB_TRIPS, conv=conv, block=_BLOCK,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
 
 
@@ -941,6 +970,165 @@ def _scan_slab(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_pt
 
 
 
+_SLAB_LONG_COLUMNS = 2       # columns a thread may own in the kernel below
+
+
+def _emit_slab_long(in_t, out_t, op, skip_nan, vec, idx64, stream):
+    """``_emit_slab`` for slices that do not fit the LDS: a workgroup takes a
+    slice, ``round_rows`` rows at a time -- again one contiguous piece of
+    memory per round --, and every thread carries the running values of its
+    columns (two at most) from round to round."""
+    acc_t = _acc_type(out_t)
+    op_c = '+' if op == _SUM else '*'
+    ident = '0' if op == _SUM else '1'
+    if skip_nan:
+        conv = ('(_x != _x) ? _acc_t(%s) : static_cast<_acc_t>(_x)' % ident)
+    else:
+        conv = 'static_cast<_acc_t>(_x)'
+    return """#include <cupy/carray.cuh>
+typedef %(in_t)s _in_t;
+typedef %(out_t)s _out_t;
+typedef %(acc_t)s _acc_t;
+typedef %(idx_t)s _idx_t;
+#define SCAN_OP(a, b) ((a) %(op_c)s (b))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
+#define VEC %(vec)d
+#define TRIPS %(trips)d
+#define BLOCK %(block)d
+#define COLUMNS %(columns)d
+#define NT_LOAD %(ntl)s
+#define NT_STORE %(nts)s
+#define SLAB_ELEMS (BLOCK * VEC * TRIPS)
+__device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
+
+// inner <= COLUMNS * BLOCK; round_rows * inner <= SLAB_ELEMS
+extern "C" __global__ void __launch_bounds__(BLOCK) cupy_scan_slab_long(
+    const _in_t* __restrict__ in, _out_t* __restrict__ out, const _idx_t outer,
+    const int n, const int inner, const int round_rows) {
+  __shared__ _acc_t lds[SLAB_ELEMS];
+  for (_idx_t slice = blockIdx.x; slice < outer; slice += gridDim.x) {
+    _acc_t carry[COLUMNS];
+#pragma unroll
+    for (int j = 0; j < COLUMNS; ++j) carry[j] = SCAN_IDENTITY;
+    for (int r0 = 0; r0 < n; r0 += round_rows) {
+      const int rows = (n - r0 < round_rows) ? n - r0 : round_rows;
+      const int valid = rows * inner;
+      const ptrdiff_t base = ((ptrdiff_t)slice * n + r0) * inner;
+      const _in_t* src = in + base;
+      _out_t* dst = out + base;
+      cupy::Vec<_in_t, VEC> raw[TRIPS];
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const int p = (t * BLOCK + (int)threadIdx.x) * VEC;
+        if (p + VEC <= valid) {
+          raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(src + p);
+        } else {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) raw[t].v[k] = (p + k < valid) ? src[p + k] : _in_t();
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const int p = (t * BLOCK + (int)threadIdx.x) * VEC;
+        if (p < valid) {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) lds[p + k] = _load_value(raw[t].v[k]);
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < COLUMNS; ++j) {
+        const int c = j * BLOCK + (int)threadIdx.x;
+        if (c < inner) {
+          // (the first row of a slice as it is: adding it to a zero would
+          // lose the sign of a negative zero)
+          _acc_t acc = (r0 == 0) ? lds[c] : carry[j];
+          int r = (r0 == 0) ? 1 : 0;
+          // (eight rows requested before the first is used: the compiler
+          // keeps every read behind the write before it, which would cost
+          // the latency of the LDS per row)
+          for (; r + 8 <= rows; r += 8) {
+            _acc_t x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = lds[(r + u) * inner + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { acc = SCAN_OP(acc, x[u]); x[u] = acc; }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) lds[(r + u) * inner + c] = x[u];
+          }
+          for (; r < rows; ++r) {
+            acc = SCAN_OP(acc, lds[r * inner + c]);
+            lds[r * inner + c] = acc;
+          }
+          carry[j] = acc;
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int t = 0; t < TRIPS; ++t) {
+        const int p = (t * BLOCK + (int)threadIdx.x) * VEC;
+        if (p + VEC <= valid) {
+          cupy::Vec<_out_t, VEC> r;
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) r.v[k] = static_cast<_out_t>(lds[p + k]);
+          cupy::store_vec<_out_t, VEC, NT_STORE>(dst + p, r);
+        } else {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k)
+            if (p + k < valid) dst[p + k] = static_cast<_out_t>(lds[p + k]);
+        }
+      }
+      // (the next round overwrites what the stores above read)
+      __syncthreads();
+    }
+  }
+}
+""" % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=_SLAB_TRIPS, conv=conv, block=_BLOCK,
+           columns=_SLAB_LONG_COLUMNS,
+           ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
+
+
+def _module_slab_long(in_dtype, out_dtype, op, skip_nan, vec, idx64, stream):
+    key = ('slab long', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan,
+           vec, idx64, stream)
+    mod = _memo.get(key)
+    if mod is None:
+        src = _emit_slab_long(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
+                              vec, idx64, stream)
+        mod = compiler.compile_with_cache(src)
+        with _lock:
+            mod = _memo.setdefault(key, mod)
+    return mod
+
+
+def _scan_slab_long(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr, cus):
+    """Launches ``_emit_slab_long`` for many slices of rows that are no whole
+    vectors, or that leave lanes of the lane-interleaved kernel idle; returns
+    False where it does not apply."""
+    if not _tuning.get('scan_slab_long'):
+        return False
+    item = max(src.dtype.itemsize, dst.dtype.itemsize, _acc_dtype(dst.dtype).itemsize)
+    vec = max(1, min(4, 16 // item))
+    capacity = _BLOCK * vec * _SLAB_TRIPS
+    round_rows = capacity // inner
+    if (inner <= 64 or inner > _SLAB_LONG_COLUMNS * _BLOCK or round_rows < 8
+            or outer < cus * _tuning.get('scan_slab_long_slices_per_cu')):
+        return False
+    full = max(1, 16 // max(src.dtype.itemsize, dst.dtype.itemsize))
+    whole = (inner % full == 0 and _aligned(src.data.ptr, 16) and _aligned(dst.data.ptr, 16))
+    if whole and (inner // full > 32 or 64 % (inner // full) == 0):
+        return False
+    mod = _module_slab_long(src.dtype, dst.dtype, op, skip_nan, vec, idx64, stream)
+    grid = max(1, min(outer, cus * _tuning.get('scan_blocks_per_cu')))
+    blob = struct.pack('@PP' + ('q' if idx64 else 'i') + 'iii', src.data.ptr, dst.data.ptr,
+                       outer, n, inner, round_rows)
+    mod.get_function('cupy_scan_slab_long').launch_packed(
+        (grid, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+    return True
+
+
+
 _CHAIN_WAVES = _BLOCK // _WAVE
 _CHAIN_HEADER_WORDS = 64            # the ticket counter, padded to 256 bytes
 
@@ -979,7 +1167,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -1266,7 +1454,7 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain(
     _part_store(row_out, j0 + p * PART_ELEMS, j1, lane, v, pre, base, has_base);
   }
 }
-''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident,
+''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident, start=_start_text(op, acc_t),
            vec=vec, trips=trips, conv=conv, block=_BLOCK, waves=_CHAIN_WAVES,
            header=_CHAIN_HEADER_WORDS, parts=parts, sleep=_tuning.get('scan_chain_sleep'),
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
@@ -1310,7 +1498,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -1598,7 +1786,7 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_tile(
   }
 }
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
-           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=_BLOCK,
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=trips, conv=conv, block=_BLOCK,
            inner=inner, rows_t=rows_t, seg=seg, lrows=lrows, stride=stride,
            waves=_CHAIN_WAVES, parts=parts, header=_CHAIN_HEADER_WORDS, sleep=sleep,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
@@ -1644,7 +1832,7 @@ typedef %(out_t)s _out_t;
 typedef %(acc_t)s _acc_t;
 typedef %(idx_t)s _idx_t;
 #define SCAN_OP(a, b) ((a) %(op_c)s (b))
-#define SCAN_IDENTITY (_acc_t(%(ident)s))
+#define SCAN_IDENTITY (_acc_t(%(start)s))
 #define VEC %(vec)d
 #define TRIPS %(trips)d
 #define NT_LOAD %(ntl)s
@@ -1870,7 +2058,7 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
   }
 }
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
-           op_c=op_c, ident=ident, vec=vec, trips=trips, conv=conv, block=waves * _WAVE,
+           op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=trips, conv=conv, block=waves * _WAVE,
            waves=waves, header=_CHAIN_HEADER_WORDS, sleep=sleep, ahead=ahead,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
 
@@ -2299,6 +2487,10 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         middle_round = _WAVE * 4 * 4          # elements one wave takes per round
     elif (inner >= 2 and n >= 2 and _slab_pays(src, dst, n, inner, item)
           and _scan_slab(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr, cus)):
+        return
+    elif (inner > 64 and n >= 2
+          and _scan_slab_long(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr,
+                              cus)):
         return
     elif (2 <= inner <= (_tuning.get('scan_tile_max_inner') if n < 16384 else 32)
           and _tuning.get('scan_tile')):

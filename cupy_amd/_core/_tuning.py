@@ -102,6 +102,8 @@ _params = {
     'scan_lanes': True,
     'scan_slab': True,          # slices with wide rows that fit the LDS: a workgroup stages whole slices
     'scan_slab_min_inner': None,   # ... for rows wider than this (None: by the shape)
+    'scan_slab_long': True,     # ... and longer slices of such rows round by round, a workgroup per slice
+    'scan_slab_long_slices_per_cu': 2,   # ... when there are this many slices per CU
     'scan_tile_packed': True,   # slices of few rows and a narrow tail: many to a wave
     'scan_tile_packed_min_slices': 0,   # ... when at least this many slices fit one round of a wave (0: by the shape)
     'scan_complex_as_real': True,   # cumsum of complex arrays: as real arrays with twice the columns

@@ -461,3 +461,78 @@ def test_column_scans_with_odd_numbers_of_columns(shape):
     flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
     assert (cp.asarray(flat)[1:].reshape(shape).cumsum(axis=1).get()
             == flat[1:].reshape(shape).cumsum(axis=1)).all()
+
+
+@pytest.mark.parametrize('shape', [(40, 300, 257), (7, 1000, 100), (3, 70, 500), (5, 80, 129),
+                                   (600, 40, 321)])
+def test_scans_of_long_slices_of_rows_that_are_no_whole_vectors(shape):
+    """A workgroup per slice, a few rows per round, running values carried from
+    round to round (taken from two slices per CU on; here from the first)."""
+    from cupy_amd._core import _tuning
+    rng = np.random.default_rng(sum(shape))
+    _tuning.set(scan_slab_long_slices_per_cu=0)
+    try:
+        h = rng.integers(-9, 10, shape).astype(np.int32)
+        assert (cp.asarray(h).cumsum(axis=1).get() == h.cumsum(axis=1)).all()
+        h8 = h.astype(np.int8)
+        assert (cp.cumsum(cp.asarray(h8), axis=1, dtype=np.int8).get()
+                == h8.cumsum(axis=1, dtype=np.int8)).all()
+        assert (cp.cumsum(cp.asarray(h8), axis=1).get() == h8.cumsum(axis=1)).all()
+        hp = np.where(rng.uniform(size=shape) < 0.2, -1, 1).astype(np.int64)
+        assert (cp.cumprod(cp.asarray(hp), axis=1).get() == hp.cumprod(axis=1)).all()
+        hf = rng.standard_normal(shape)
+        hf[:, 0, :3] = -0.0
+        got = cp.cumsum(cp.asarray(hf), axis=1).get()
+        bound = 1e-13 * np.cumsum(np.abs(hf), axis=1) + 1e-15
+        assert (np.abs(got - hf.cumsum(axis=1)) <= bound).all()
+        assert np.signbit(got[:, 0, :3]).all()
+        hn = rng.uniform(0, 1, shape).astype(np.float32)
+        hn[:, ::3, 1] = np.nan
+        got = cp.nancumsum(cp.asarray(hn), axis=1).get()
+        assert np.allclose(got, np.nancumsum(hn.astype(np.float64), axis=1), rtol=1e-5, atol=1e-6)
+        hh = rng.uniform(0, 1, shape).astype(np.float16)
+        got = cp.cumsum(cp.asarray(hh), axis=1).get()
+        assert np.allclose(got, hh.astype(np.float64).cumsum(axis=1), rtol=2e-3, atol=1e-2)
+        # in place, and from a view that does not start on a 16-byte boundary
+        d = cp.asarray(h)
+        r = cp.cumsum(d, axis=1, out=d)
+        assert r is d and (d.get() == h.cumsum(axis=1)).all()
+        flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
+        assert (cp.asarray(flat)[1:].reshape(shape).cumsum(axis=1).get()
+                == flat[1:].reshape(shape).cumsum(axis=1)).all()
+        from test_gpu_scan_chain import launched
+        if shape[2] % 4:      # (rows of 500 floats are whole vectors: a thread per vector)
+            floats = cp.asarray(h.astype(np.float32))
+            assert 'cupy_scan_slab_long' in launched(lambda: floats.cumsum(axis=1))
+        bytes_ = cp.asarray(h8)
+        assert 'cupy_scan_slab_long' in launched(lambda: cp.cumsum(bytes_, axis=1, dtype=np.int8))
+    finally:
+        _tuning.set(scan_slab_long_slices_per_cu=2)
+
+
+@pytest.mark.parametrize('shape,axis', [((1 << 20,), 0), ((1000, 1000), 0), ((1000, 1000), 1),
+                                        ((3000, 7, 5), 1), ((200, 100, 100), 1), ((64, 1 << 14), 0),
+                                        ((64, 1 << 14), 1), ((100000, 3), 0), ((16, 257, 257), 1),
+                                        ((40, 3, 1000), 1), ((5000, 2, 64), 1), ((1 << 16, 40), 0)])
+@pytest.mark.parametrize('dtype', [np.float32, np.float64, np.complex64])
+def test_sums_of_negative_zeros_stay_negative(shape, axis, dtype):
+    """-0.0 + -0.0 is -0.0 and anything else added to a zero gives +0.0: the
+    signs of a scan of signed zeros do not depend on the order of the additions
+    -- only on what a scan starts from (NumPy and the reference's in-place scan,
+    cupy/_core/_routines_math.pyx:160-751, start from the first element)."""
+    rng = np.random.default_rng(len(shape) + axis)
+    h = np.where(rng.uniform(size=shape) < 2.0 / shape[axis], 0.0, -0.0).astype(dtype)
+    if dtype == np.complex64:
+        h.imag = np.where(rng.uniform(size=shape) < 2.0 / shape[axis], 0.0, -0.0)
+    want = np.cumsum(h, axis=axis)
+    got = cp.cumsum(cp.asarray(h), axis=axis).get()
+    assert (np.signbit(got.real) == np.signbit(want.real)).all()
+    if dtype == np.complex64:
+        assert (np.signbit(got.imag) == np.signbit(want.imag)).all()
+    else:
+        hn = h.copy()
+        hn.reshape(-1)[::7] = np.nan
+        # (a NaN that is skipped counts as +0.0)
+        want = np.nancumsum(hn, axis=axis)
+        got = cp.nancumsum(cp.asarray(hn), axis=axis).get()
+        assert (np.signbit(got) == np.signbit(want)).all()
