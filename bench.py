@@ -410,6 +410,13 @@ def build_layout_cases(cp):
         lambda: np.cumsum(a33, axis=1),
         lambda: close(res['s33'], np.cumsum(a33, axis=1, dtype=np.float64), 1e-5,
                       np.cumsum(np.abs(a33), axis=1, dtype=np.float64)), 'cupy_scan_tile_packed')
+    rw = n // (16 * 257)
+    aw = flat[:rw * 16 * 257].reshape(rw, 16, 257)
+    dw = dflat[:rw * 16 * 257].reshape(rw, 16, 257)
+    add('cumsum f32 (2^26/4112)x16x257 axis=1', 2 * aw.nbytes, run('sw', lambda: cp.cumsum(dw, axis=1)),
+        lambda: np.cumsum(aw, axis=1),
+        lambda: close(res['sw'], np.cumsum(aw, axis=1, dtype=np.float64), 1e-5,
+                      np.cumsum(np.abs(aw), axis=1, dtype=np.float64)), 'cupy_scan_slab')
     r100 = n // 100
     a100, d100 = flat[:r100 * 100].reshape(r100, 100), dflat[:r100 * 100].reshape(r100, 100)
 
