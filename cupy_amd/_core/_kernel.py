@@ -1701,16 +1701,26 @@ class ufunc:
         # (Only plain arrays and scalars have a signature, and calls with
         # structured arrays are never recorded, so a hit needs none of the
         # checks below.)
-        fast_key = rec = fast_args = None
+        fast_key = rec = fast_args = casting_given = None
         nk = len(kwargs)
         if nk == 0:
             fast_args = args
-        elif nk == 1 and len(args) == self.nin and 'out' in kwargs:
-            o = kwargs['out']
-            fast_args = args + (o if type(o) is tuple else (o,))
+        elif nk <= 2:
+            # (``out`` and ``casting``: the rule only decides whether the types
+            # of the call, which the signature holds, may be cast; it joins the
+            # key.  astype, copies and fills pass it.)
+            o = kwargs.get('out')
+            casting_given = kwargs.get('casting')
+            if (o is not None) + (type(casting_given) is str) == nk:
+                if o is None:
+                    fast_args = args
+                elif len(args) == self.nin:
+                    fast_args = args + (o if type(o) is tuple else (o,))
         if fast_args is not None and self.nin <= len(fast_args) <= self.nargs:
             fast_key = _launch_plan.call_signature(fast_args, _device.get_device_id())
             if fast_key is not None:
+                if casting_given is not None:
+                    fast_key = fast_key + (casting_given,)
                 fast = self._fast_calls.get(fast_key)
                 if fast is not None:
                     ret = fast.run(fast_args)
@@ -1842,7 +1852,11 @@ class ufunc:
             dev_id, all_args, nin_total, shape, var_types, typedefs, casts=casts,
             force_generic=False, force_read_out=has_where,
             kernel_name=self._get_name_with_type(all_args, has_where), rec=rec)
-        if rec is not None and len(rec.launches) == 1:
+        # (a cast that warns -- complex to real under 'unsafe' -- warns every time)
+        warns = casting == 'unsafe' and any(
+            get_dtype(lt).kind == 'c' and a.dtype.kind in 'iuf'
+            for a, lt in zip(out_args, core_out_dtypes))
+        if rec is not None and len(rec.launches) == 1 and not warns:
             n_user = len(fast_args)
             n_given = n_user - self.nin
             ret_refs = self.nin if self.nout == 1 else tuple(range(self.nin, self.nargs))

@@ -68,6 +68,8 @@ def scalar_value(v, descr):
                 return v
         elif descr == _float64 and -(1 << 53) <= v <= (1 << 53):
             return float(v)
+        elif descr == _float32 and -(1 << 24) <= v <= (1 << 24):
+            return float(v)     # (exact in 24 bits of mantissa)
     elif t is bool:
         if descr == _bool:
             return v

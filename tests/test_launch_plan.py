@@ -347,3 +347,36 @@ def test_other_calls_take_the_full_path():
     assert len(k._fast_calls) == 1
     with pytest.raises(TypeError):
         k(x, y, x)
+
+
+def test_casting_rule_joins_the_signature():
+    """``astype``, copies and fills pass ``casting='unsafe'``: such calls are
+    recorded and replayed too, under a key of their own; a cast that warns is
+    never recorded, so it warns on every call."""
+    import warnings
+    from cupy_amd._core._ufuncs import elementwise_copy
+    a = cp.ndarray((1 << 16,), np.float32)
+    n0 = len(elementwise_copy._fast_calls)
+    r1, first = launches_of(lambda: a.astype(np.float64))
+    assert len(elementwise_copy._fast_calls) == n0 + 1
+    assert any(key[-1] == 'unsafe' for key in elementwise_copy._fast_calls)
+    r2, again = launches_of(lambda: a.astype(np.float64))
+    assert r1.dtype == r2.dtype == np.float64 and r1.data.ptr != r2.data.ptr
+    k = names((a,))
+    assert [(l[0], l[1], l[2]) for l in again] == [(l[0], l[1], l[2]) for l in first]
+    assert words(again[0][4], k)[0] == 'arg0'
+    # stricter rules refuse what 'unsafe' allows, recorded or not
+    b = cp.ndarray((1 << 16,), np.int32)
+    elementwise_copy(a, b, casting='unsafe')
+    elementwise_copy(a, b, casting='unsafe')
+    with pytest.raises(TypeError):
+        elementwise_copy(a, b, casting='same_kind')
+    with pytest.raises(TypeError):
+        elementwise_copy(a, b, casting='safe')
+    # complex to real warns every time
+    c = cp.ndarray((100,), np.complex64)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter('always')
+        for _ in range(3):
+            c.astype(np.float32)
+    assert len(seen) == 3
