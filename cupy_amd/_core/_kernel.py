@@ -1701,17 +1701,34 @@ class ufunc:
         # (Only plain arrays and scalars have a signature, and calls with
         # structured arrays are never recorded, so a hit needs none of the
         # checks below.)
-        fast_key = rec = fast_args = casting_given = None
+        fast_key = rec = fast_args = extra = None
         nk = len(kwargs)
         if nk == 0:
             fast_args = args
-        elif nk <= 2:
-            # (``out`` and ``casting``: the rule only decides whether the types
-            # of the call, which the signature holds, may be cast; it joins the
-            # key.  astype, copies and fills pass it.)
+        else:
+            # (``out``, ``casting`` and ``dtype``: the casting rule only decides
+            # whether the types of the call, which the signature holds, may be
+            # cast, and the dtype selects the loop: both join the key.  astype,
+            # copies and fills pass the rule.  Keywords given as None --
+            # wrappers hand ``out=None, dtype=None`` on -- count as absent.)
             o = kwargs.get('out')
-            casting_given = kwargs.get('casting')
-            if (o is not None) + (type(casting_given) is str) == nk:
+            known = 0 if o is None else 1
+            value = kwargs.get('casting')
+            if type(value) is str:
+                known += 1
+                extra = value
+            value = kwargs.get('dtype')
+            if value is not None:
+                try:
+                    extra = (extra, get_dtype(value).char)
+                    known += 1
+                except TypeError:
+                    pass
+            live = 0
+            for value in kwargs.values():
+                if value is not None:
+                    live += 1
+            if known == live:
                 if o is None:
                     fast_args = args
                 elif len(args) == self.nin:
@@ -1719,8 +1736,8 @@ class ufunc:
         if fast_args is not None and self.nin <= len(fast_args) <= self.nargs:
             fast_key = _launch_plan.call_signature(fast_args, _device.get_device_id())
             if fast_key is not None:
-                if casting_given is not None:
-                    fast_key = fast_key + (casting_given,)
+                if extra is not None:
+                    fast_key = fast_key + (extra,)
                 fast = self._fast_calls.get(fast_key)
                 if fast is not None:
                     ret = fast.run(fast_args)

@@ -752,6 +752,12 @@ class ndarray:
         from cupy_amd._core import _routines_statistics
         return _routines_statistics._ndarray_ptp(self, axis, out, keepdims)
 
+    def clip(self, min=None, max=None, out=None):
+        """Values limited to ``[min, max]`` (reference: cupy/_core/core.pyx
+        ``ndarray.clip`` -> ``_routines_math._ndarray_clip``)."""
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.clip(self, min, max, out=out)
+
     def cumsum(self, axis=None, dtype=None, out=None):
         from cupy_amd._core import _scan
         return _scan.cumsum(self, axis, dtype, out)
