@@ -2428,6 +2428,13 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
     # ended and finds (part of) it there.
     reuse_ok = (_tuning.get('scan_chunk_reuse')
                 and total * in_dtype.itemsize <= 2 * _tuning.get('cache_bytes'))
+    if inner > 1 and n <= 256 and total * item <= _tuning.get('scan_whole_max_bytes'):
+        # Small arrays scanned down short columns: three launches and a
+        # temporary cost more than the few rounds of a single pass (us per
+        # call, whole against cut: 128 x 128 floats along axis 0 13 / 36,
+        # 256 x 256 25 / 40, 128 x 2048 16 / 39, 256 x 1024 29 / 40; longer
+        # columns are better off cut: 1024 x 64 41 / 31).
+        may_chunk = False
     if inner == 1:
         vec = max(1, 16 // item)
         # (rows of any length keep their vectors: wide accesses need the
