@@ -2258,6 +2258,12 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
     n_tiles = n_rows * tiles_per_row
     if n_tiles < 2 or n_tiles * _BLOCK > 0xffffffff or n < _BLOCK * vec * trips:
         return False
+    if (inner == 1 and tiles_per_row * tile > _tuning.get('scan_chain_max_waste') * n
+            and n_rows >= _device.get_compute_units(dev_id) * _tuning.get('scan_waves_per_cu')):
+        # Many rows a little longer than a whole number of tiles: the last
+        # tile of every row would be all but empty (rows of 4099 floats: two
+        # tiles of 4096); a wave per row does better.
+        return False
     # groups of about sqrt(tiles per row) tiles: a tile then reads about
     # 2 sqrt(tiles per row) published totals
     group_tiles = max(32, min(2048, internal.clp2(int(tiles_per_row ** 0.5))))

@@ -125,6 +125,7 @@ _params = {
     'scan_chain_sleep': 8,      # ... and pauses this many times 64 clocks between two polls
     'scan_chain_spin_limit': 1 << 18,   # polls after which a tile of that kernel gives up waiting
     'scan_waves_per_cu': 32,    # long rows are cut into chunks until this many waves exist
+    'scan_chain_max_waste': 1.9,    # rows whose tiles would hold this many times their elements take a wave per row instead (rows of 4099 floats: 127 -> 118 us; at 1.25 rows of 5500 lose: 106 -> 118)
     'scan_whole_max_bytes': 1 << 20,   # column scans of up to 256 rows of arrays up to this size are never cut into chunks
     'scan_whole_slices_waves_per_cu': 4,   # ... slices of fewer than 4096 rows with a narrow tail stay whole from this many on
     # fused row-wise functions: words per lane up to which a wave takes a whole row
