@@ -973,8 +973,21 @@ class _ElementwisePlanner:
             # 12288 615: few workgroups per CU then, each busy with one phase.)
             # the workgroup is a whole number of lines of the narrow side, so
             # that both loops of the kernel come out in whole trips
-            want = max(512, min(_tuning.get('tiled_narrow_elements'),
-                                 (48 * 1024) // max(1, lds_item)))
+            want = _tuning.get('tiled_narrow_elements')
+            if not want:
+                # (widths that are no power of two want longer tiles, i.e.
+                # longer runs per line of the other side: (n, 24) to (24, n)
+                # 184 us with 1536 elements, 118 with 6144; (n, 20) 163 -> 116;
+                # (n, 26) 187 -> 138 with 3072; odd widths and powers of two
+                # are best at 1536)
+                narrow_side = min(nr, nc)
+                if narrow_side & (narrow_side - 1) == 0 or narrow_side % 2:
+                    want = 1536
+                elif narrow_side % 4:
+                    want = 3072
+                else:
+                    want = 6144
+            want = max(512, min(want, (48 * 1024) // max(1, lds_item)))
             if nr <= 32:
                 tile_r = nr
                 while svec > 1 and tile_r % svec:

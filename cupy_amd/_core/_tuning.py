@@ -52,7 +52,7 @@ _params = {
     # tiled 2-d elementwise kernel
     'tiled_stream': 'auto',
     'tiled_batch_first': True,  # batched tiles: near batch entries before far rows
-    'tiled_narrow_elements': 1536,   # ... of about this many elements
+    'tiled_narrow_elements': 0,      # ... of about this many elements (0: 1536 to 6144 by the width)
     'tiled_narrow': True,       # tiles as narrow as the array where an axis has at most 32 elements
     'tiled_unaligned': True,    # vectors whatever the alignment of rows and columns
     'tiled_tile': None,         # (rows, columns, threads) of a staged tile; None: by shape

@@ -550,7 +550,10 @@ def test_reduce_dims_false_keeps_the_axes_for_the_kernel():
 
 
 @pytest.mark.parametrize('shape', [(100003, 3), (3, 100003), (65536, 15), (31, 40001), (50000, 32),
-                                   (2, 70001), (4099, 1), (7, 5, 20001, 3), (6, 3, 20001)])
+                                   (2, 70001), (4099, 1), (7, 5, 20001, 3), (6, 3, 20001),
+                                   # widths that are no power of two: longer tiles
+                                   (30011, 12), (24, 30011), (20001, 26), (28, 9001), (70001, 20),
+                                   (18, 33333)])
 def test_transposes_of_narrow_arrays(shape):
     """Points as rows of a few coordinates to or from a few long rows: tiles as
     narrow as the array."""
