@@ -562,7 +562,7 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
 def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
                  loop_prep='', after_loop='', layouts=None, vec=4, tile_r=64,
                  tile_c=64, threads=256, idx64=False, stream_hint=True, batched=False,
-                 batch_first=False, svec=None):
+                 batch_first=False, svec=None, flat_stage=0):
     """Kernel for a 2-d index space (rows r, columns c) where every array
     operand is contiguous along one of the axes.
 
@@ -693,7 +693,40 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
             src.append('        _prer_%s[_it] = *%s;' % (op.name, gaddr(op, '_r', '0')))
         src.append('      }')
         src.append('    }')
-    if c_ops:
+    if c_ops and flat_stage:
+        # ---- stage transposed operands whose tile is ONE contiguous piece of
+        # memory (the tile spans their whole fast extent, and their lines follow
+        # one another without gaps): vectors of ``flat_stage`` elements over the
+        # piece, whatever the length of a line; element _f of the piece is row
+        # _f %% tile_r of column _f / tile_r
+        n_flat = -(-(tile_r * tile_c) // (flat_stage * threads))
+        src.append('    {')
+        src.append('      const int _limit = ((_nc - _c0 < %d) ? (int)(_nc - _c0) : %d) * %d;' % (
+            tile_c, tile_c, tile_r))
+        src.append('#pragma unroll')
+        src.append('      for (int _it = 0; _it < %d; ++_it) {' % n_flat)
+        src.append('        const int _f = (threadIdx.x + _it * %d) * %d;' % (threads, flat_stage))
+        src.append('        if (_f + %d <= _limit) {' % flat_stage)
+        for op in c_ops:
+            src.append('          { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s + _f);' % (
+                op.store_t, flat_stage, op.store_t, flat_stage, ntl, gaddr(op, '0', '_c0')))
+            src.append('#pragma unroll')
+            src.append('            for (int _k = 0; _k < %d; ++_k) { const int _lc = (_f + _k) / %d; '
+                       '_t_%s[(_f + _k - _lc * %d) * %d + _lc] = _lv.v[_k]; } }' % (
+                           flat_stage, tile_r, op.name, tile_r, pitch))
+        src.append('        } else {')
+        src.append('#pragma unroll')
+        src.append('          for (int _k = 0; _k < %d; ++_k) if (_f + _k < _limit) {' % flat_stage)
+        src.append('            const int _lc = (_f + _k) / %d;' % tile_r)
+        for op in c_ops:
+            src.append('            _t_%s[(_f + _k - _lc * %d) * %d + _lc] = (%s)[_f + _k];' % (
+                op.name, tile_r, pitch, gaddr(op, '0', '_c0')))
+        src.append('          }')
+        src.append('        }')
+        src.append('      }')
+        src.append('    }')
+        src.append('    __syncthreads();')
+    elif c_ops:
         # ---- stage transposed operands: rows are the fast direction -------------------
         src.append('    if (_interior) {')
         src.append('#pragma unroll')

@@ -1081,9 +1081,23 @@ class _ElementwisePlanner:
             inner_batch = [abs(bs[1] if bshape[1] > 1 else bs[0]) for bs in bstrides]
             pitch = [max(abs(cs[0]), abs(cs[1])) for cs in cstrides]
             batch_first = all(b and b < p for b, p in zip(inner_batch, pitch))
+        # Staged operands whose lines are no whole vectors (3, 7, 17, 31 ...
+        # elements) and follow one another without gaps: a tile that spans the
+        # lines is one contiguous piece of memory and is read with full vectors
+        # all the same ((n, 17) to (17, n): 183 us element by element).
+        flat_stage = 0
+        if (narrow and nr <= 32 and tile_r == nr and svec == 1 and n_transposed
+                and _tuning.get('tiled_flat_stage')):
+            staged = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names)
+                      if layouts[nm] == 'C']
+            if staged and all(cs[0] == a.dtype.itemsize and cs[1] == nr * a.dtype.itemsize
+                              for a, cs in staged):
+                flat_stage = min(4, 16 // max(a.dtype.itemsize for a, cs in staged))
+                if flat_stage < 2:
+                    flat_stage = 0
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
-               threads, bool(batch), batch_first, svec)
+               threads, bool(batch), batch_first, svec, flat_stage)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
@@ -1092,7 +1106,7 @@ class _ElementwisePlanner:
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
                 tile_r=tile_r, tile_c=tile_c, threads=threads, idx64=idx64,
                 stream_hint=stream_hint, batched=bool(batch), batch_first=batch_first,
-                svec=svec)
+                svec=svec, flat_stage=flat_stage)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']

@@ -53,6 +53,7 @@ _params = {
     'tiled_stream': 'auto',
     'tiled_batch_first': True,  # batched tiles: near batch entries before far rows
     'tiled_narrow_elements': 0,      # ... of about this many elements (0: 1536 to 6144 by the width)
+    'tiled_flat_stage': True,   # ... read as one contiguous piece where the lines are no whole vectors
     'tiled_narrow': True,       # tiles as narrow as the array where an axis has at most 32 elements
     'tiled_unaligned': True,    # vectors whatever the alignment of rows and columns
     'tiled_tile': None,         # (rows, columns, threads) of a staged tile; None: by shape

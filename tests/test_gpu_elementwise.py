@@ -553,7 +553,10 @@ def test_reduce_dims_false_keeps_the_axes_for_the_kernel():
                                    (2, 70001), (4099, 1), (7, 5, 20001, 3), (6, 3, 20001),
                                    # widths that are no power of two: longer tiles
                                    (30011, 12), (24, 30011), (20001, 26), (28, 9001), (70001, 20),
-                                   (18, 33333)])
+                                   (18, 33333),
+                                   # odd widths: the staged tile is read as one piece
+                                   (40001, 31), (50001, 17), (70001, 7), (4, 30001, 5), (1, 3),
+                                   (300, 13)])
 def test_transposes_of_narrow_arrays(shape):
     """Points as rows of a few coordinates to or from a few long rows: tiles as
     narrow as the array."""
