@@ -901,6 +901,20 @@ class _ElementwisePlanner:
             bstrides = [bs + (0,) for bs in bstrides]
         return shape2, strides2, (bshape, bstrides)
 
+    @staticmethod
+    def _flat_stage_width(arrays, cstrides, names, layouts, nr):
+        """Elements per access with which the staged operands of a tile that
+        spans their ``nr`` contiguous elements per line can be read as one
+        piece (their lines follow one another without gaps), or 0."""
+        if not _tuning.get('tiled_flat_stage'):
+            return 0
+        staged = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if layouts[nm] == 'C']
+        if not staged or not all(cs[0] == a.dtype.itemsize and cs[1] == nr * a.dtype.itemsize
+                                 for a, cs in staged):
+            return 0
+        width = min(4, 16 // max(a.dtype.itemsize for a, cs in staged))
+        return width if width >= 2 else 0
+
     def _launch_tiled(self, dev_id, args, nin, arrays, cshape, cstrides, var_types,
                       typedefs, casts, force_read_out, stream_ptr, kernel_name, swap,
                       rec, batch=None):
@@ -981,7 +995,13 @@ class _ElementwisePlanner:
                 # (n, 26) 187 -> 138 with 3072; odd widths and powers of two
                 # are best at 1536)
                 narrow_side = min(nr, nc)
-                if narrow_side & (narrow_side - 1) == 0 or narrow_side % 2:
+                if narrow_side % 2 and narrow_side > 9 and nr <= 32 and self._flat_stage_width(
+                        arrays, cstrides, names, layouts, nr):
+                    # (odd widths whose staged tile is read as one piece, see
+                    # below: (n, 13) 126 -> 114, (n, 19) 159 -> 123, (n, 31)
+                    # 184 -> 125)
+                    want = 3072 if narrow_side < 25 else 6144
+                elif narrow_side & (narrow_side - 1) == 0 or narrow_side % 2:
                     want = 1536
                 elif narrow_side % 4:
                     want = 3072
@@ -1086,15 +1106,8 @@ class _ElementwisePlanner:
         # lines is one contiguous piece of memory and is read with full vectors
         # all the same ((n, 17) to (17, n): 183 us element by element).
         flat_stage = 0
-        if (narrow and nr <= 32 and tile_r == nr and svec == 1 and n_transposed
-                and _tuning.get('tiled_flat_stage')):
-            staged = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names)
-                      if layouts[nm] == 'C']
-            if staged and all(cs[0] == a.dtype.itemsize and cs[1] == nr * a.dtype.itemsize
-                              for a, cs in staged):
-                flat_stage = min(4, 16 // max(a.dtype.itemsize for a, cs in staged))
-                if flat_stage < 2:
-                    flat_stage = 0
+        if narrow and nr <= 32 and tile_r == nr and svec == 1 and n_transposed:
+            flat_stage = self._flat_stage_width(arrays, cstrides, names, layouts, nr)
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
                threads, bool(batch), batch_first, svec, flat_stage)
