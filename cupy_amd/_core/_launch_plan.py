@@ -25,6 +25,7 @@ from cupy_amd import _rt
 from cupy_amd._core import _carray
 from cupy_amd._core import _tuning
 from cupy_amd._core._scalar import CScalar
+from cupy_amd.cuda import _giveup
 from cupy_amd.cuda import memory as _memory
 from cupy_amd.cuda import stream as _stream
 
@@ -104,18 +105,22 @@ class ArgBlock:
 
 class Recorder:
     """Collects the launches and temporaries of one call."""
-    __slots__ = ('n_refs', 'launches', 'temps', 'stream')
+    __slots__ = ('n_refs', 'launches', 'temps', 'stream', 'device')
 
     def __init__(self, n_refs):
         self.n_refs = n_refs      # user arguments + allocated outputs
         self.launches = []
         self.temps = []
         self.stream = None        # the one stream the launches may be replayed on
+        self.device = None        # ... and the device that stream belongs to
 
-    def bind_stream(self, stream_ptr):
-        """The recorded launches name memory that belongs to ``stream_ptr``:
-        a replay on another stream takes the full path."""
+    def bind_stream(self, stream_ptr, dev_id):
+        """The recorded launches finish a split reduction inside one launch
+        through memory that belongs to ``stream_ptr`` of device ``dev_id``: a
+        replay on another stream takes the full path, and so does every replay
+        once a kernel of that kind gave up a wait on the device."""
         self.stream = stream_ptr
+        self.device = dev_id
 
     def temp(self, nbytes):
         """Registers a temporary of ``nbytes``; returns its ref number."""
@@ -156,7 +161,7 @@ class FastCall:
     """Recorded call: allocates outputs and temporaries, patches pointers and
     scalar values, launches."""
     __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap', 'quick',
-                 'stream')
+                 'stream', 'device')
 
     def __init__(self, n_user, out_specs, rec, ret, overlap=()):
         self.n_user = n_user
@@ -167,6 +172,14 @@ class FastCall:
         self.overlap = tuple(overlap)         # (input ref, output ref) pairs to check
         self.quick = _quick_launches(self.launches)
         self.stream = rec.stream
+        self.device = rec.device
+
+    def stale(self):
+        """True for a record that must not be replayed any more, on any
+        stream: it finishes a reduction inside one launch and a kernel of that
+        kind has given up a wait on its device.  The full path then reports
+        that (once) and records the two-launch form in this record's place."""
+        return self.stream is not None and not _giveup.usable(self.device, _giveup.REDUCTION)
 
     def run(self, args, stream_ptr=None):
         from cupy_amd._core.core import ndarray
@@ -174,6 +187,10 @@ class FastCall:
             if stream_ptr is None:
                 stream_ptr = _stream.get_current_stream_ptr()
             if stream_ptr != self.stream:
+                return NotImplemented
+            # (a wrong result must not be handed out twice: the reference's
+            # reduction is a plain launch, cupy/_core/_reduction.pyx:481-508)
+            if not _giveup.usable(self.device, _giveup.REDUCTION):
                 return NotImplemented
         for i, o in self.overlap:
             a, b = args[i], args[o]

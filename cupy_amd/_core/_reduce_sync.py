@@ -8,38 +8,38 @@ so that a recorded launch can be replayed without any change -- followed by
 slots of 64 bits.  Launches on one stream run one after the other, and every
 launch marks what it writes with its own number, so nothing is cleared between
 launches.  A block is cleared once, when it is created; a block that has become
-too small is left to the recorded calls that still name it and a larger one
-takes its place.
+too small is retired (see ``_retired``) and a larger one takes its place.
 """
-import ctypes
 import threading
 
 import numpy
 
-from cupy_amd import _dryrun
 from cupy_amd._core import _tuning
+from cupy_amd.cuda import _giveup
 from cupy_amd.cuda import memory as _memory
 
 HEADER_WORDS = 64
+MAX_STREAMS = 64    # (device, stream) pairs that hold a block at a time
 
 _lock = threading.Lock()
 _blocks = {}        # (device id, stream) -> (array of uint32, slots it holds)
-_retired = []       # blocks that recorded calls may still name
-_fault = {}         # device id -> address of a word in pinned host memory
-_disabled = set()   # devices on which a workgroup gave up waiting
+# Blocks that were replaced or evicted.  Recorded calls name a block by its
+# address, so whenever blocks are retired the tuning version moves on (no
+# earlier record is replayed again) and the blocks stay allocated until the
+# retirement after the next: a thread that had picked up a record just before
+# still finds the memory in place.
+_retired = [[], []]
 
 
 def _fault_word(dev_id):
-    address = _fault.get(dev_id)
-    if address is None:
-        address = 0
-        if not _dryrun.enabled():
-            from cupy_amd.cuda import runtime
-            address = runtime.hostAlloc(64, 0)
-            ctypes.memset(address, 0, 64)
-        with _lock:
-            address = _fault.setdefault(dev_id, address)
-    return address
+    """Address of the word a workgroup that gives up waiting writes to."""
+    return _giveup.word(dev_id, _giveup.REDUCTION)
+
+
+def _retire(blocks):
+    _retired[1] = _retired[0]       # (drops the generation before: freed)
+    _retired[0] = list(blocks)
+    _tuning.invalidate_records()
 
 
 def acquire(dev_id, stream_ptr, current_stream_ptr, n_slots):
@@ -48,21 +48,15 @@ def acquire(dev_id, stream_ptr, current_stream_ptr, n_slots):
     has to take two launches: switched off, a stream other than the current
     one (the block is cleared on the current stream), more slots than a block
     may hold, no allocation allowed, or an earlier failure on this device."""
-    if not _tuning.get('reduce_finish') or dev_id in _disabled:
+    if not _tuning.get('reduce_finish') or dev_id in _giveup.disabled[_giveup.REDUCTION]:
         return None
     if stream_ptr != current_stream_ptr or n_slots > _tuning.get('reduce_finish_max_slots'):
         return None
     if _memory._static_scratch_open and _memory.static_scratch_active():
         return None
     fault = _fault_word(dev_id)
-    if fault and ctypes.c_uint32.from_address(fault).value:
-        # Not expected to happen: say so, and stay away from the kernels.
-        _disabled.add(dev_id)
-        ctypes.c_uint32.from_address(fault).value = 0
-        raise RuntimeError(
-            'an earlier reduction on device %d gave up waiting for the partial results of '
-            'its workgroups: its result is wrong.  Reductions take two launches from now on.'
-            % dev_id)
+    # Not expected to happen: say so, and stay away from the kernels.
+    _giveup.poll(dev_id)
     key = (dev_id, stream_ptr)
     with _lock:
         block = _blocks.get(key)
@@ -71,10 +65,12 @@ def acquire(dev_id, stream_ptr, current_stream_ptr, n_slots):
             slots = max(n_slots, 1 << 16)
             if block is not None:
                 slots = max(slots, 2 * block[1])
-                _retired.append(block)
-            if len(_blocks) >= 64:
-                _retired.extend(_blocks.values())
+                del _blocks[key]
+                _retire([block])
+            elif len(_blocks) >= MAX_STREAMS:
+                evicted = list(_blocks.values())
                 _blocks.clear()
+                _retire(evicted)
             array = ndarray._new_contiguous((HEADER_WORDS + 2 * slots,), numpy.dtype('uint32'))
             # (a kernel on the current stream, not a memset: the caller may be
             # capturing the stream)

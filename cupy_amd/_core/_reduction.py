@@ -221,6 +221,20 @@ class _AbstractReductionKernel:
             fast = self._fast_calls.get(key)
         except TypeError:       # unhashable axis / dtype argument
             return False, None, None, None
+        if fast is not None and fast.stream is not None:
+            # A record that finishes the reduction inside its one launch names
+            # memory of the stream it was made on: other streams keep records
+            # of their own under the key extended by the stream.  Once a
+            # kernel of that kind gave up a wait on the device none of them is
+            # replayed; the full path reports it and records over them.
+            cur = _stream.get_current_stream_ptr()
+            if fast.stale():
+                fast = None
+            elif fast.stream != cur:
+                key = key + (cur,)
+                fast = self._fast_calls.get(key)
+                if fast is not None and fast.stale():
+                    fast = None
         if fast is not None:
             ret = fast.run(fast_args)
             if ret is not NotImplemented:
@@ -762,7 +776,7 @@ class _AbstractReductionKernel:
             # one launch: the workgroup of the last chunk of every row combines
             # the partial results of the others
             if rec is not None:
-                rec.bind_stream(stream_ptr)
+                rec.bind_stream(stream_ptr, device_id)
             vals.const(finish[0], _tuning.get('reduce_finish_spin_limit'), finish[1], gx, chunk)
             _launch_plan.launch(
                 rec, fn, (gx * n_split, 1, 1), (wg, 1, 1),
@@ -927,7 +941,7 @@ class _AbstractReductionKernel:
             # one launch: the workgroup of the last slice of every column block
             # combines the partial results of the others
             if rec is not None:
-                rec.bind_stream(stream_ptr)
+                rec.bind_stream(stream_ptr, device_id)
             vals.const(finish[0], _tuning.get('reduce_finish_spin_limit'), finish[1], gx)
             _launch_plan.launch(
                 rec, fn, (gx * n_split, 1, 1), (block, 1, 1),

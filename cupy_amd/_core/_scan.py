@@ -21,7 +21,6 @@ along the scanned axis: pass 1 reduces every chunk to its total, the totals
 are scanned by the same code, pass 3 scans the chunks seeded with the total of
 everything before them.  Nothing spins on another workgroup's progress.
 """
-import ctypes
 import struct
 import threading
 
@@ -32,6 +31,7 @@ from cupy_amd._core import internal
 from cupy_amd._core._kernel import _aligned
 from cupy_amd._core._scalar import get_typename as _get_typename
 from cupy_amd._core.core import ndarray
+from cupy_amd.cuda import _giveup
 from cupy_amd.cuda import compiler
 from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import stream as _stream
@@ -2141,23 +2141,10 @@ def _lanes_geometry(src, dst, inner, item):
     return None
 
 
-_chain_fault = {}        # device id -> address of the word in pinned host memory a tile
-                         # that gave up waiting writes to (0 where none could be allocated)
-_chain_disabled = set()  # devices on which that has happened
-
-
 def _chain_fault_word(dev_id):
-    address = _chain_fault.get(dev_id)
-    if address is None:
-        from cupy_amd import _dryrun
-        address = 0
-        if not _dryrun.enabled():
-            from cupy_amd.cuda import runtime
-            address = runtime.hostAlloc(64, 0)
-            ctypes.memset(address, 0, 64)
-        with _lock:
-            address = _chain_fault.setdefault(dev_id, address)
-    return address
+    """Address of the word in pinned host memory a tile that gave up waiting
+    writes to (0 where none could be allocated)."""
+    return _giveup.word(dev_id, _giveup.SCAN)
 
 
 _chain_arenas = {}       # (device id, stream) -> [slots array, number of the last launch]
@@ -2197,19 +2184,13 @@ def _chain_ready():
     if not _tuning.get('scan_chain'):
         return None
     dev_id = _device.get_device_id()
-    if dev_id in _chain_disabled:
+    if dev_id in _giveup.disabled[_giveup.SCAN]:
         return None
     fault = _chain_fault_word(dev_id)
-    if fault and ctypes.c_uint32.from_address(fault).value:
-        # A tile of an earlier scan gave up waiting for the tiles before it and
-        # left wrong results.  Not expected to happen: say so, and stay away
-        # from the kernel from here on.
-        _chain_disabled.add(dev_id)
-        ctypes.c_uint32.from_address(fault).value = 0
-        raise RuntimeError(
-            'an earlier one-pass scan on device %d gave up waiting for its neighbouring '
-            'tiles: its result is wrong.  Scans use the three-pass kernels from now on.'
-            % dev_id)
+    # A tile of an earlier scan that gave up waiting for the tiles before it
+    # left wrong results.  Not expected to happen: poll() says so, and the
+    # kernels stay unused from there on.
+    _giveup.poll(dev_id)
     return dev_id, fault
 
 

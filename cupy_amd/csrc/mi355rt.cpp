@@ -370,8 +370,9 @@ int rt_launch_packed_scratch(void* function, unsigned gx, unsigned gy, unsigned 
   if (!arg_block || arg_block_size > sizeof(block))
     return fail_invalid("rt_launch_packed_scratch: argument block missing or larger than "
                         "RT_SCRATCH_MAX_ARG_BLOCK bytes");
-  if (scratch_arg_offset % sizeof(void*) != 0 ||
-      scratch_arg_offset + sizeof(void*) > arg_block_size)
+  // (compared without adding to the offset: an offset near SIZE_MAX must not wrap)
+  if (scratch_arg_offset % sizeof(void*) != 0 || arg_block_size < sizeof(void*) ||
+      scratch_arg_offset > arg_block_size - sizeof(void*))
     return fail_invalid("rt_launch_packed_scratch: the pointer slot lies outside the argument "
                         "block or is not 8-byte aligned");
   void* ptr = nullptr;

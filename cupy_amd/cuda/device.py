@@ -4,6 +4,7 @@ import threading
 
 from cupy_amd import _dryrun
 from cupy_amd import _rt
+from cupy_amd.cuda import _giveup
 
 _props_cache = {}
 _props_lock = threading.Lock()
@@ -116,6 +117,9 @@ class Device:
             return
         with self:
             _rt.check(_rt.lib.rt_device_synchronize())
+        # results become visible to the host here: none may be a wrong one
+        if _giveup.armed:
+            _giveup.poll(self.id)
 
     @property
     def attributes(self):

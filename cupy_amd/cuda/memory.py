@@ -13,6 +13,7 @@ import warnings
 
 from cupy_amd import _dryrun
 from cupy_amd import _rt
+from cupy_amd.cuda import _giveup
 from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import stream as _stream
 from cupy_amd.cuda import memory_hook as _memory_hook
@@ -219,6 +220,10 @@ class MemoryPointer:
         if size > 0:
             _rt.check(_rt.lib.rt_memcpy(
                 _as_host_address(mem), self.ptr, size, _rt.MEMCPY_D2H))
+            # the copy waited for the kernels before it: a value one of them
+            # reported as wrong must not reach the caller
+            if _giveup.armed:
+                _giveup.poll()
 
     def copy_to_host_async(self, mem, size, stream=None):
         if _dryrun.enabled():

@@ -3,6 +3,7 @@
 import ctypes
 
 from cupy_amd import _rt
+from cupy_amd.cuda import _giveup
 from cupy_amd.cuda import device as _device
 
 is_hip = True
@@ -39,6 +40,8 @@ def getDeviceProperties(device):
 
 def deviceSynchronize():
     _rt.check(_rt.lib.rt_device_synchronize())
+    if _giveup.armed:
+        _giveup.poll()
 
 
 def driverGetVersion():
@@ -98,3 +101,5 @@ def memsetAsync(ptr, value, size, stream):
 
 def streamSynchronize(stream):
     _rt.check(_rt.lib.rt_stream_synchronize(stream))
+    if _giveup.armed:
+        _giveup.poll()

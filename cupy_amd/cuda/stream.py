@@ -5,6 +5,7 @@ import threading
 
 from cupy_amd import _dryrun
 from cupy_amd import _rt
+from cupy_amd.cuda import _giveup
 
 _tls = threading.local()
 
@@ -63,6 +64,9 @@ class Event:
         if _dryrun.enabled():
             return
         _rt.check(_rt.lib.rt_event_synchronize(self.ptr))
+        # results become visible to the host here: none may be a wrong one
+        if _giveup.armed:
+            _giveup.poll()
 
 
 def get_elapsed_time(start_event, end_event):
@@ -135,6 +139,9 @@ class Stream:
         if _dryrun.enabled():
             return
         _rt.check(_rt.lib.rt_stream_synchronize(self.ptr))
+        # results become visible to the host here: none may be a wrong one
+        if _giveup.armed:
+            _giveup.poll()
 
     def record(self, event=None):
         if event is None:

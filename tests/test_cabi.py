@@ -48,3 +48,20 @@ def test_invalid_arguments_are_reported_not_crashed():
     minor = ctypes.c_int(0)
     assert _rt.lib.rt_rtc_version(ctypes.byref(major), ctypes.byref(minor)) == 0
     assert major.value >= 7 or major.value == 9 or major.value > 0
+
+
+def test_scratch_launch_refuses_a_pointer_slot_outside_the_argument_block():
+    """Every check of ``rt_launch_packed_scratch`` comes before anything
+    touches a device, so the refusals can be seen without one.  An offset near
+    the top of ``size_t`` must not wrap the bounds check around."""
+    from cupy_amd import _rt
+    args = (ctypes.c_ubyte * 64)()
+    fn = ctypes.addressof(args)         # never called: the checks refuse first
+    launch = _rt.lib.rt_launch_packed_scratch
+    for offset in (2 ** 64 - 8, 2 ** 64 - 16, 64, 60, 57, 2 ** 63):
+        assert launch(fn, 1, 1, 1, 64, 1, 1, 0, None, args, 64, offset, 16) == _rt.RT_ERR_INVALID
+        assert b'pointer slot' in _rt.lib.rt_last_error_string()
+    assert launch(fn, 1, 1, 1, 64, 1, 1, 0, None, args, 4, 0, 16) == _rt.RT_ERR_INVALID
+    assert launch(fn, 1, 1, 1, 64, 1, 1, 0, None, args, 64, 0,
+                  _rt.RT_SCRATCH_MAX_BYTES + 1) == _rt.RT_ERR_INVALID
+    assert launch(fn, 1, 1, 1, 64, 1, 1, 0, None, args, 8192, 0, 16) == _rt.RT_ERR_INVALID

@@ -141,24 +141,122 @@ def test_large_inputs_take_two_launches():
     assert float(got) == float(1 << 25)
 
 
-def test_a_workgroup_that_gives_up_is_reported():
-    from cupy_amd._core import _reduce_sync
-    a = cp.ones(1 << 22, 'int32')
-    assert int(a.sum()) == 1 << 22
+@contextlib.contextmanager
+def _reported_give_up(family):
+    """Writes what a workgroup that gave up would have written into the
+    device's word (every kernel still exits normally) and restores the state
+    of the device afterwards."""
+    from cupy_amd.cuda import _giveup
     dev = cp.cuda.Device().id
-    fault = _reduce_sync._fault_word(dev)
-    # (what a workgroup that gave up would have written)
+    fault = _giveup.word(dev, family)
     ctypes.c_uint32.from_address(fault).value = 1
     try:
-        _tuning.set()
+        yield
+    finally:
+        _giveup.disabled[family].discard(dev)
+        ctypes.c_uint32.from_address(fault).value = 0
+
+
+def test_a_workgroup_that_gives_up_is_reported():
+    """The recorded one-launch call is NOT replayed once the word is set: the
+    call raises, and later calls take two launches (and are replayed as such)."""
+    from cupy_amd.cuda import _giveup
+    a = cp.ones(1 << 22, 'int32')
+    out = cp.zeros((), 'int64')
+    assert int(a.sum()) == 1 << 22
+    assert int(a.sum()) == 1 << 22          # (a replay)
+    a.sum(out=out)
+    a.sum(out=out)
+    with _reported_give_up(_giveup.REDUCTION):
         with pytest.raises(RuntimeError, match='gave up waiting'):
             a.sum()
-        # two launches from here on
-        got, names = _launched(lambda: a.sum())
-        assert len(names) == 2 and int(got) == 1 << 22
+        # two launches from here on, for the other recorded call as well
+        from cupy_amd.cuda import function
+        names = []
+        orig = function.Function.launch_packed
+        from cupy_amd._core import _launch_plan
+        _launch_plan.use_quick = False
+        function.Function.launch_packed = lambda self, *x, **k: (names.append(self.name),
+                                                                orig(self, *x, **k))[1]
+        try:
+            got = a.sum()
+            a.sum(out=out)
+            again = a.sum()
+        finally:
+            function.Function.launch_packed = orig
+            _launch_plan.use_quick = True
+        assert names == ['cupy_sum', 'cupy_sum_combine'] * 3, names
+        assert int(got) == int(out) == int(again) == 1 << 22
+
+
+def test_a_give_up_cannot_reach_the_host_unnoticed():
+    """Whatever makes device results visible to the host raises when a kernel
+    has reported a wait that ran out."""
+    from cupy_amd.cuda import _giveup
+    a = cp.ones(1 << 20, 'int32')
+    r = a.sum()
+    for family in (_giveup.REDUCTION, _giveup.SCAN):
+        for look in (lambda: r.get(), lambda: int(r), lambda: cp.cuda.Device().synchronize(),
+                     lambda: cp.cuda.Stream.null.synchronize(),
+                     lambda: cp.cuda.get_current_stream().record().synchronize()):
+            with _reported_give_up(family):
+                with pytest.raises(RuntimeError, match='gave up waiting'):
+                    look()
+                look()      # reported once
+        s = cp.cuda.Stream()
+        with s:
+            with _reported_give_up(family):
+                with pytest.raises(RuntimeError, match='gave up waiting'):
+                    r.get()
+    assert int(r) == 1 << 20
+
+
+def test_a_wait_that_runs_out_never_delivers_its_value():
+    """With no patience at all (one poll per wait) a finishing workgroup may
+    find partial results missing: then the value must not come back."""
+    from cupy_amd.cuda import _giveup
+    dev = cp.cuda.Device().id
+    a = cp.ones((1 << 22) + 17, 'int32')
+    try:
+        with tuned(reduce_finish_spin_limit=0):
+            for _ in range(4):
+                r = a.sum()
+                try:
+                    value = int(r)
+                except RuntimeError as e:
+                    assert 'gave up waiting' in str(e)
+                    break
+                assert value == (1 << 22) + 17
     finally:
-        _reduce_sync._disabled.discard(dev)
-        ctypes.c_uint32.from_address(fault).value = 0
+        _giveup.disabled[_giveup.REDUCTION].discard(dev)
+    assert int(a.sum()) == (1 << 22) + 17
+
+
+def test_a_second_stream_records_a_replay_of_its_own():
+    rng = np.random.default_rng(9)
+    h = rng.integers(-100, 100, 1 << 21).astype('int32')
+    a = cp.asarray(h)
+    out = cp.zeros((), 'int64')
+    from cupy_amd._core import _routines_math as rm
+    a.sum(out=out)
+    s = cp.cuda.Stream()
+    with s:
+        a.sum(out=out)
+        n = len(rm._sum_auto_dtype._fast_calls)
+        calls = []
+        orig = rm._sum_auto_dtype._call
+        rm._sum_auto_dtype._call = lambda *x, **k: (calls.append(1), orig(*x, **k))[1]
+        try:
+            for _ in range(3):
+                a.sum(out=out)
+        finally:
+            del rm._sum_auto_dtype._call
+        s.synchronize()
+        assert not calls                    # replays, not the full path
+        assert len(rm._sum_auto_dtype._fast_calls) == n
+        assert int(out) == int(h.sum())
+    a.sum(out=out)
+    assert int(out) == int(h.sum())
 
 
 @pytest.mark.parametrize('dtype', ['complex64', 'complex128'])

@@ -5,6 +5,7 @@ import pytest
 
 import cupy_amd as cp
 from cupy_amd._core import _scan, _tuning
+from cupy_amd.cuda import _giveup
 from helpers import assert_exact
 
 pytestmark = pytest.mark.gpu
@@ -16,7 +17,7 @@ def _restore():
     _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0,
                 scan_chain_cols=True, scan_chain_cols_waves=16, scan_chain_cols_trips=0,
                 scan_chain_cols_vec_bytes=0)
-    _scan._chain_disabled.clear()
+    _giveup.disabled[_giveup.SCAN].clear()
 
 
 def three_pass(fn):
@@ -139,11 +140,11 @@ def test_a_tile_that_gives_up_is_reported_and_the_kernel_retired():
     h = rng.integers(-5, 6, 1 << 23).astype(np.int32)
     d = cp.asarray(h)
     _tuning.set(scan_chain_spin_limit=0)
-    d.cumsum()
-    cp.cuda.Device().synchronize()
-    _tuning.set(scan_chain_spin_limit=1 << 18)
+    wrong = d.cumsum()
+    # the result cannot be looked at without the report
     with pytest.raises(RuntimeError, match='gave up waiting'):
-        d.cumsum()
+        wrong.get()
+    _tuning.set(scan_chain_spin_limit=1 << 18)
     names = launched(lambda: d.cumsum())
     assert 'cupy_scan_chain' not in names and 'cupy_scan_rows_seeded' in names
     assert_exact(d.cumsum().get(), h.cumsum())
@@ -294,16 +295,36 @@ def test_long_columns_other_types_and_tile_shapes(waves, trips, vec_bytes):
                  hv[1:].reshape(4000, 256).cumsum(axis=0))
 
 
+def test_a_reported_scan_raises_on_the_next_scan_and_retires_the_kernel():
+    """The twin of the reduction's test: the host writes what a tile that gave
+    up would have written (every kernel exits normally); the next scan raises,
+    later ones take three passes."""
+    import ctypes
+    rng = np.random.default_rng(12)
+    h = rng.integers(-5, 6, 1 << 22).astype(np.int32)
+    d = cp.asarray(h)
+    assert 'cupy_scan_chain' in launched(lambda: d.cumsum())
+    fault = _giveup.word(cp.cuda.Device().id, _giveup.SCAN)
+    ctypes.c_uint32.from_address(fault).value = 1
+    try:
+        with pytest.raises(RuntimeError, match='gave up waiting'):
+            d.cumsum()
+    finally:
+        ctypes.c_uint32.from_address(fault).value = 0
+    names = launched(lambda: d.cumsum())
+    assert 'cupy_scan_chain' not in names and 'cupy_scan_rows_seeded' in names
+    assert_exact(d.cumsum().get(), h.cumsum())
+
+
 def test_a_column_tile_that_gives_up_is_reported():
     rng = np.random.default_rng(8)
     h = rng.integers(-5, 6, (1 << 15, 512)).astype(np.int32)
     d = cp.asarray(h)
     _tuning.set(scan_chain_spin_limit=0)
     d.cumsum(axis=0)
-    cp.cuda.Device().synchronize()
-    _tuning.set(scan_chain_spin_limit=1 << 18)
     with pytest.raises(RuntimeError, match='gave up waiting'):
-        d.cumsum(axis=0)
+        cp.cuda.Device().synchronize()
+    _tuning.set(scan_chain_spin_limit=1 << 18)
     names = launched(lambda: d.cumsum(axis=0))
     assert 'cupy_scan_chain_cols' not in names
     assert_exact(d.cumsum(axis=0).get(), h.cumsum(axis=0))

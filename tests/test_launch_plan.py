@@ -380,3 +380,115 @@ def test_casting_rule_joins_the_signature():
         for _ in range(3):
             c.astype(np.float32)
     assert len(seen) == 3
+
+
+@pytest.fixture
+def giveup_words():
+    """Stands in for the pinned words of device 0 (none exist where launches
+    are only recorded): 16 words of host memory the test may write."""
+    import ctypes
+    from cupy_amd.cuda import _giveup
+    words = (ctypes.c_uint32 * 16)()
+    saved = dict(_giveup._base), _giveup.armed
+    _giveup._base[0] = ctypes.addressof(words)
+    _giveup.armed = True
+    try:
+        yield words
+    finally:
+        _giveup._base.clear()
+        _giveup._base.update(saved[0])
+        _giveup.armed = saved[1]
+        for family in _giveup.disabled:
+            family.clear()
+
+
+def test_a_one_launch_reduction_is_not_replayed_after_a_give_up(giveup_words):
+    """A recorded call whose kernel waits for other workgroups is left to the
+    full path as soon as the device's word is set; that path raises once and
+    records the two-launch form in its place."""
+    from cupy_amd._core import _routines_math as rm
+    from cupy_amd.cuda import _giveup
+    sumk = rm._sum_auto_dtype
+    a, o = cp.ndarray((1 << 22,), np.float32), cp.ndarray((), np.float32)
+    b, p = cp.ndarray((512, 512), np.float64), cp.ndarray((512,), np.float64)
+
+    def kernels(ls):
+        return [l[0] for l in ls if not l[0].startswith('cupy_copy')]
+    for x, out, axis in ((a, o, None), (b, p, 0)):
+        sumk(x, axis, None, out, False)
+        _, again = launches_of(lambda: sumk(x, axis, None, out, False))
+        assert kernels(again) == ['cupy_sum']
+    giveup_words[_giveup.REDUCTION] = 1
+    assert not _giveup.usable(0, _giveup.REDUCTION)
+    with pytest.raises(RuntimeError, match='gave up waiting'):
+        sumk(a, None, None, o, False)
+    assert giveup_words[_giveup.REDUCTION] == 0 and 0 in _giveup.disabled[_giveup.REDUCTION]
+    for x, out, axis in ((a, o, None), (b, p, 0), (a, o, None), (b, p, 0)):
+        _, ls = launches_of(lambda: sumk(x, axis, None, out, False))
+        assert kernels(ls) == ['cupy_sum', 'cupy_sum_combine']
+    # the scans' word is a different one
+    assert _giveup.usable(0, _giveup.SCAN)
+
+
+def test_poll_reports_each_family_once(giveup_words):
+    from cupy_amd.cuda import _giveup
+    _giveup.poll()
+    giveup_words[_giveup.SCAN] = 1
+    with pytest.raises(RuntimeError, match='one-pass scan on device 0 gave up waiting'):
+        _giveup.poll()
+    _giveup.poll()
+    assert 0 in _giveup.disabled[_giveup.SCAN] and 0 not in _giveup.disabled[_giveup.REDUCTION]
+    giveup_words[_giveup.REDUCTION] = 1
+    _giveup.poll(5)             # another device: nothing to say
+    with pytest.raises(RuntimeError, match='a reduction on device 0 gave up waiting'):
+        _giveup.poll(0)
+
+
+def test_a_second_stream_replays_a_record_of_its_own():
+    """One-launch reductions are recorded per stream: the third call on a
+    second stream is a replay, not the full path."""
+    from cupy_amd._core import _routines_math as rm
+    sumk = rm._sum_auto_dtype
+    a, o = cp.ndarray((1 << 21,), np.float32), cp.ndarray((), np.float32)
+    sumk(a, None, None, o, False)
+    side = cp.cuda.Stream()
+    side.ptr = 0x5151            # (streams have no handles here: any other number)
+    calls = []
+    orig = sumk._call
+    sumk._call = lambda *x, **k: (calls.append(1), orig(*x, **k))[1]
+    try:
+        with side:
+            _, first = launches_of(lambda: sumk(a, None, None, o, False))
+            assert len(calls) == 1
+            n = len(sumk._fast_calls)
+            _, second = launches_of(lambda: sumk(a, None, None, o, False))
+            _, third = launches_of(lambda: sumk(a, None, None, o, False))
+        assert len(calls) == 1 and len(sumk._fast_calls) == n
+        _, home = launches_of(lambda: sumk(a, None, None, o, False))
+        assert len(calls) == 1
+    finally:
+        del sumk._call
+        side.ptr = 0
+    k = names((a, o))
+    assert describe(second, k) == describe(third, k) == describe(first[-1:], k)
+    # each stream hands its partial results over in memory of its own
+    assert home[-1][4] != third[-1][4]
+
+
+def test_retired_blocks_are_freed_two_retirements_later():
+    """Streams come and go: the blocks of evicted streams do not pile up."""
+    from cupy_amd._core import _reduce_sync, _tuning
+    saved = dict(_reduce_sync._blocks)
+    try:
+        _reduce_sync._blocks.clear()
+        v0 = _tuning.version()
+        for s in range(3 * _reduce_sync.MAX_STREAMS + 5):
+            assert _reduce_sync.acquire(0, 1000 + s, 1000 + s, 100) is not None
+            held = (len(_reduce_sync._blocks) + len(_reduce_sync._retired[0])
+                    + len(_reduce_sync._retired[1]))
+            assert held <= 3 * _reduce_sync.MAX_STREAMS
+        # records that name retired blocks are never replayed again
+        assert _tuning.version() == v0 + 3
+    finally:
+        _reduce_sync._blocks.clear()
+        _reduce_sync._blocks.update(saved)
