@@ -36,33 +36,37 @@ _INT32_MAX = (1 << 31) - 1
 
 class ParameterInfo:
     """One entry of an ``in_params`` / ``out_params`` string:
-    ``[raw] [_non_const] <dtype name | single-letter placeholder> <name>``."""
+    ``[raw] [_non_const] <dtype name | single-letter placeholder> <name>``
+    (reference: cupy/_core/_kernel.pyx:464-518; same attributes, same errors)."""
+
+    # what a leading keyword sets
+    _KEYWORDS = {'raw': ('raw', True), '_non_const': ('is_const', False)}
 
     def __init__(self, param, is_const):
-        self.name = None
-        self.dtype = None
-        self.ctype = None
+        words = param.split()
+        if len(words) < 2:
+            raise Exception('Syntax error: %s' % param)
+        *keywords, type_word, self.name = words
+        self.dtype, self.ctype = self._read_type(type_word)
         self.raw = False
         self.is_const = is_const
-        s = tuple(i for i in param.split() if len(i) != 0)
-        if len(s) < 2:
-            raise Exception('Syntax error: %s' % param)
-        t, self.name = s[-2:]
-        if t == 'CIndexer':
-            pass
-        elif len(t) == 1:
-            self.ctype = t
-        else:
-            dtype = get_dtype(t)
-            self.dtype = dtype
-            self.ctype = _get_typename(dtype)
-        for i in s[:-2]:
-            if i == 'raw':
-                self.raw = True
-            elif i == '_non_const':
-                self.is_const = False
-            else:
-                raise Exception('Unknown keyword "%s"' % i)
+        for word in keywords:
+            if word not in self._KEYWORDS:
+                raise Exception('Unknown keyword "%s"' % word)
+            attribute, value = self._KEYWORDS[word]
+            setattr(self, attribute, value)
+
+    @staticmethod
+    def _read_type(word):
+        """(dtype, C type name) of the type word: the indexer pseudo-type has
+        neither, a single letter is a placeholder bound at call time, anything
+        else names a dtype."""
+        if word == 'CIndexer':
+            return None, None
+        if len(word) == 1:
+            return None, word
+        dtype = get_dtype(word)
+        return dtype, _get_typename(dtype)
 
     def _key(self):
         return (self.name, self.dtype, self.ctype, self.raw, self.is_const)
@@ -82,15 +86,15 @@ _param_info_memo = {}
 
 
 def _get_param_info(s, is_const):
-    key = (s, is_const)
-    ret = _param_info_memo.get(key)
-    if ret is None:
-        if len(s) == 0:
-            ret = ()
-        else:
-            ret = tuple(ParameterInfo(i, is_const) for i in s.strip().split(','))
-        _param_info_memo[key] = ret
-    return ret
+    """Tuple of ParameterInfo for a comma-separated parameter string (memoised)."""
+    try:
+        return _param_info_memo[s, is_const]
+    except KeyError:
+        pass
+    entries = s.strip().split(',') if s else ()
+    infos = _param_info_memo[s, is_const] = tuple(
+        ParameterInfo(entry, is_const) for entry in entries)
+    return infos
 
 
 class _TypeMap:
@@ -115,45 +119,37 @@ class _TypeMap:
 
 def _decide_params_type_core(in_params, out_params, in_args_dtype, out_args_dtype):
     """Binds single-letter type placeholders from the dtypes of the array
-    arguments (outputs first) and checks fixed-dtype parameters."""
-    type_dict = {}
+    arguments (outputs first) and checks fixed-dtype parameters (reference:
+    cupy/_core/_kernel.pyx:557-604; same error texts)."""
+    bound = {}
+
+    def settle(param, given, as_dtype):
+        # a parameter of fixed dtype only has to agree with the argument; a
+        # placeholder takes the first dtype it meets and must meet no other
+        if param.dtype is not None:
+            if as_dtype(given) != as_dtype(param.dtype):
+                raise TypeError('Type is mismatched. %s %s %s' % (
+                    param.name, given, param.dtype))
+            return
+        known = bound.setdefault(param.ctype, given)
+        if as_dtype(known) != as_dtype(given):
+            raise TypeError('Type is mismatched. %s %s %s %s' % (
+                param.name, given, known, param.ctype))
+
     if out_args_dtype:
         assert len(out_params) == len(out_args_dtype)
-        for p, a in zip(out_params, out_args_dtype):
-            if a is None:
+        for param, given in zip(out_params, out_args_dtype):
+            if given is None:
                 raise TypeError('Output arguments must be cupy.ndarray')
-            if p.dtype is not None:
-                if get_dtype(a) != get_dtype(p.dtype):
-                    raise TypeError(
-                        'Type is mismatched. %s %s %s' % (p.name, a, p.dtype))
-            elif p.ctype in type_dict:
-                t = type_dict[p.ctype]
-                if get_dtype(t) != get_dtype(a):
-                    raise TypeError('Type is mismatched. %s %s %s %s' % (
-                        p.name, a, t, p.ctype))
-            else:
-                type_dict[p.ctype] = a
+            settle(param, given, get_dtype)
     assert len(in_params) == len(in_args_dtype)
-    for p, a in zip(in_params, in_args_dtype):
-        if a is None:
-            continue
-        if p.dtype is not None:
-            if numpy.dtype(a) != numpy.dtype(p.dtype):
-                raise TypeError(
-                    'Type is mismatched. %s %s %s' % (p.name, a, p.dtype))
-        elif p.ctype in type_dict:
-            t = type_dict[p.ctype]
-            if numpy.dtype(t) != numpy.dtype(a):
-                raise TypeError('Type is mismatched. %s %s %s %s' % (
-                    p.name, a, t, p.ctype))
-        else:
-            type_dict[p.ctype] = a
-    in_types = tuple(type_dict[p.ctype] if p.dtype is None else p.dtype
-                     for p in in_params)
-    out_types = tuple(type_dict[p.ctype] if p.dtype is None else p.dtype
-                      for p in out_params)
-    type_map = _TypeMap(sorted(type_dict.items(), key=lambda kv: kv[0]))
-    return in_types, out_types, type_map
+    for param, given in zip(in_params, in_args_dtype):
+        if given is not None:           # (scalars take the type they are given)
+            settle(param, given, numpy.dtype)
+
+    def resolved(params):
+        return tuple(bound[p.ctype] if p.dtype is None else p.dtype for p in params)
+    return resolved(in_params), resolved(out_params), _TypeMap(sorted(bound.items()))
 
 
 _decide_memo = {}
@@ -203,28 +199,23 @@ def _preprocess_optional_args(dev_id, args):
 
 
 def _broadcast(args, params, use_size):
-    """Broadcasts the non-raw arrays of ``args`` against each other.
-    Returns (new args, broadcast shape)."""
-    value = []
-    any_nonraw_array = False
-    for a, p in zip(args, params):
-        if not p.raw and isinstance(a, ndarray):
-            any_nonraw_array = True
-            value.append(a)
-        else:
-            value.append(None)
-    if use_size:
-        if any_nonraw_array:
-            raise ValueError('Specified \'size\' can be used only '
-                             'if all of the ndarray are \'raw\'.')
-    else:
-        if not any_nonraw_array:
-            raise ValueError('Loop size is undecided.')
-    shape = internal._broadcast_core(value)
-    for i, a in enumerate(value):
-        if a is None:
-            value[i] = args[i]
-    return value, shape
+    """Broadcasts the arrays of ``args`` that take part in the loop (arrays of
+    parameters not marked ``raw``) against each other; everything else passes
+    through.  Returns (new args, loop shape).  ``use_size``: the caller gave
+    ``size=``, which is allowed exactly when no array takes part (reference:
+    cupy/_core/_kernel.pyx:607-640)."""
+    looped = [i for i, (a, p) in enumerate(zip(args, params))
+              if isinstance(a, ndarray) and not p.raw]
+    if use_size and looped:
+        raise ValueError('Specified \'size\' can be used only '
+                         'if all of the ndarray are \'raw\'.')
+    if not use_size and not looped:
+        raise ValueError('Loop size is undecided.')
+    views = [None] * len(args)
+    for i in looped:
+        views[i] = args[i]
+    shape = internal._broadcast_core(views)      # (replaces the arrays by views)
+    return [a if v is None else v for a, v in zip(args, views)], shape
 
 
 def _get_out_args_from_optionals(subtype, out_args, out_types, out_shape, casting, obj):
@@ -1318,36 +1309,45 @@ class ElementwiseKernel:
                  return_tuple=False, **kwargs):
         if not compiler.is_valid_kernel_name(name):
             raise ValueError('Invalid kernel name: "%s"' % name)
-        self.in_params = _get_param_info(in_params, True)
-        self.out_params = _get_param_info(out_params, False)
-        self.nin = len(self.in_params)
-        self.nout = len(self.out_params)
-        self.nargs = self.nin + self.nout
-        param_rest = _get_param_info('CIndexer _ind', False)
-        self.params = self.in_params + self.out_params + param_rest
+        self.name = self.__name__ = name
         self.operation = operation
-        self.name = name
-        self.__name__ = name
-        self.reduce_dims = reduce_dims
         self.preamble = preamble
+        self.reduce_dims = reduce_dims
         self.no_return = no_return
         self.return_tuple = return_tuple
         self.kwargs = dict(kwargs)
-        options = kwargs.pop('options', ())
-        loop_prep = kwargs.pop('loop_prep', '')
-        after_loop = kwargs.pop('after_loop', '')
-        if kwargs:
-            raise TypeError('Wrong arguments %s' % kwargs)
-        names = [p.name for p in self.in_params + self.out_params]
-        if 'i' in names:
+        extras = dict(options=(), loop_prep='', after_loop='')
+        unknown = {k: v for k, v in kwargs.items() if k not in extras}
+        if unknown:
+            raise TypeError('Wrong arguments %s' % unknown)
+        extras.update(kwargs)
+
+        self.in_params = _get_param_info(in_params, True)
+        self.out_params = _get_param_info(out_params, False)
+        declared = self.in_params + self.out_params
+        self.nin, self.nout, self.nargs = len(self.in_params), len(self.out_params), len(declared)
+        # (the loop index `i` belongs to the generated loop)
+        if any(p.name == 'i' for p in declared):
             raise ValueError('Can not use \'i\' as a parameter name')
+        # what broadcasting sees: the declared parameters and the indexer
+        self.params = declared + _get_param_info('CIndexer _ind', False)
         self._params_type_memo = {}
         self._planner = _ElementwisePlanner(
-            name, self.in_params + self.out_params, operation, preamble,
-            loop_prep, after_loop, options, is_ufunc=False)
+            name, declared, operation, preamble, extras['loop_prep'], extras['after_loop'],
+            extras['options'], is_ufunc=False)
         self._planner.reduce_dims = bool(reduce_dims)
         self._cached_codes = self._planner._codes
         self._fast_calls = {}
+
+    def _result(self, out_args, as_refs=False):
+        """What a call hands back from its output arrays: nothing, the one
+        array, or a tuple (``as_refs``: their positions among the arguments)."""
+        if self.no_return:
+            return None
+        outs = tuple(range(self.nin, self.nargs)) if as_refs else tuple(out_args)
+        if self.nout == 1 and not self.return_tuple:
+            return outs[0]
+        return outs
 
     def __call__(self, *args, **kwargs):
         """Compiles (if needed) and launches the kernel.
@@ -1367,15 +1367,16 @@ class ElementwiseKernel:
                 fast = self._fast_calls.get(fast_key)
                 if fast is not None:
                     return fast.run(args)
-        size = kwargs.pop('size', -1)
-        stream = kwargs.pop('stream', None)
-        block_size = kwargs.pop('block_size', 128)
-        if len(kwargs):
-            raise TypeError('Wrong arguments %s' % kwargs)
+        options = dict(size=-1, stream=None, block_size=128)
+        unknown = {k: v for k, v in kwargs.items() if k not in options}
+        if unknown:
+            raise TypeError('Wrong arguments %s' % unknown)
+        options.update(kwargs)
+        size, stream, block_size = options['size'], options['stream'], options['block_size']
         if block_size <= 0:
             raise ValueError('block_size must be greater than zero')
         n_args = len(args)
-        if n_args != self.nin and n_args != self.nargs:
+        if n_args not in (self.nin, self.nargs):
             raise TypeError(
                 'Wrong number of arguments for {!r}. '
                 'It must be either {} or {} (with outputs), '
@@ -1399,26 +1400,17 @@ class ElementwiseKernel:
         bargs, shape = _broadcast(arg_list, self.params, size != -1)
         in_args = bargs[:self.nin]
 
-        in_ndarray_types = tuple(
-            a.dtype if isinstance(a, ndarray) else None for a in in_args)
-        out_ndarray_types = tuple(
-            a.dtype if isinstance(a, ndarray) else None for a in out_args)
+        def array_dtypes(arguments):
+            return tuple(a.dtype if isinstance(a, ndarray) else None for a in arguments)
         in_types, out_types, type_map = self._decide_params_type(
-            in_ndarray_types, out_ndarray_types)
+            array_dtypes(in_args), array_dtypes(out_args))
 
-        is_size_specified = False
-        if size != -1:
+        size_given = size != -1
+        if size_given:
             shape = (int(size),)
-            is_size_specified = True
-
         out_args = _get_out_args_with_params(
-            out_args, out_types, shape, self.out_params, is_size_specified)
-        if self.no_return:
-            ret = None
-        elif not self.return_tuple and self.nout == 1:
-            ret = out_args[0]
-        else:
-            ret = tuple(out_args)
+            out_args, out_types, shape, self.out_params, size_given)
+        ret = self._result(out_args)
         if 0 in shape:
             return ret
 
@@ -1433,12 +1425,7 @@ class ElementwiseKernel:
             type_map.get_typedef_code(), stream=stream, block_size=block_size,
             rec=rec)
         if rec is not None and len(rec.launches) == 1:
-            if self.no_return:
-                ret_refs = None
-            elif not self.return_tuple and self.nout == 1:
-                ret_refs = self.nin
-            else:
-                ret_refs = tuple(range(self.nin, self.nargs))
+            ret_refs = self._result(None, as_refs=True)
             out_specs = () if n_args == self.nargs else tuple(
                 (shape, o.dtype) for o in out_args)
             _launch_plan.remember(
@@ -1497,14 +1484,16 @@ def fix_cast_expr(src_type, dst_type, expr):
     return expr
 
 
+_KIND_LADDER = ((numpy.bool_,), (numpy.integer, int), (numpy.inexact, float, complex))
+
+
 def _get_kind_score(kind):
-    if issubclass(kind, numpy.bool_):
-        return 0
-    if issubclass(kind, (numpy.integer, int)):
-        return 1
-    if issubclass(kind, (numpy.inexact, float, complex)):
-        return 2
-    return 3
+    """0 for booleans, 1 for integers, 2 for floating and complex types, 3 for
+    anything else."""
+    for score, kinds in enumerate(_KIND_LADDER):
+        if issubclass(kind, kinds):
+            return score
+    return len(_KIND_LADDER)
 
 
 def _check_should_use_weak_scalar(in_types, weaks):
@@ -1530,28 +1519,21 @@ class _Op:
     routine (code) or an ``error_func`` raising for a forbidden combination."""
 
     def __init__(self, in_types, out_types, routine, error_func):
-        if error_func is None:
-            assert routine is not None
-        else:
-            assert callable(error_func)
-        self.in_types = in_types
-        self.out_types = out_types
-        self.nin = len(in_types)
-        self.nout = len(out_types)
-        self.routine = routine
-        self.error_func = error_func
-        self._in_dtypes = tuple(get_dtype(t) for t in in_types)
-        self._out_dtypes = tuple(get_dtype(t) for t in out_types)
+        # a loop either has code or refuses its type combination
+        assert callable(error_func) if error_func is not None else routine is not None
+        self.in_types, self.out_types = in_types, out_types
+        self.nin, self.nout = len(in_types), len(out_types)
+        self.routine, self.error_func = routine, error_func
+        self._in_dtypes = tuple(map(get_dtype, in_types))
+        self._out_dtypes = tuple(map(get_dtype, out_types))
 
     @staticmethod
     def _from(typ, routine, error_func):
-        types = typ.split('->')
-        if len(types) == 1:
-            in_types = out_types = tuple(types)
-        else:
-            in_types, out_types = map(tuple, types)
-        in_types = tuple(get_dtype(t).type for t in in_types)
-        out_types = tuple(get_dtype(t).type for t in out_types)
+        """From a signature such as ``'ff->f'``; a signature without an arrow
+        gives the outputs the inputs' types."""
+        ins, arrow, outs = typ.partition('->')
+        in_types = tuple(get_dtype(c).type for c in ins)
+        out_types = tuple(get_dtype(c).type for c in outs) if arrow else in_types
         return _Op(in_types, out_types, routine, error_func)
 
     def check_valid(self):
@@ -1569,107 +1551,129 @@ class _Ops:
 
     def __init__(self, ops):
         assert len(ops) > 0
-        nin = ops[0].nin
-        nout = ops[0].nout
-        for op in ops:
-            if op.nin != nin or op.nout != nout:
-                raise ValueError(f'invalid op {op}, wrong nin or nout.')
         self.ops = ops
-        self.nin = nin
-        self.nout = nout
+        self.nin, self.nout = ops[0].nin, ops[0].nout
+        for op in ops:
+            if (op.nin, op.nout) != (self.nin, self.nout):
+                raise ValueError(f'invalid op {op}, wrong nin or nout.')
 
     @staticmethod
     def from_tuples(ops, routine):
-        ops_ = []
-        for t in ops:
-            if isinstance(t, tuple):
-                typ, rt = t
-                if rt is None:
-                    rt = routine
-                elif isinstance(rt, tuple):
-                    rt = tuple(r1 or r2 for r1, r2 in zip(rt, routine))
-                elif not isinstance(rt, str):
-                    if not callable(rt):
-                        raise ValueError(f'invalid op {t}, expected callable {rt}')
-                    ops_.append(_Op._from(typ, None, rt))
-                    continue
-            else:
-                if not isinstance(t, str):
-                    raise ValueError(f'invalid op {t}, expected string')
-                typ, rt = t, routine
-            ops_.append(_Op._from(typ, rt, None))
-        return _Ops(tuple(ops_))
+        """Loop table from the entries ``create_ufunc`` / ``create_reduction_func``
+        take (reference: cupy/_core/_kernel.pyx:1622-1650)."""
+        return _Ops(tuple(_Op._from(*_read_loop_entry(entry, routine)) for entry in ops))
 
     def guess_routine(self, name, cache, in_args, dtype, out_ops):
+        """The loop for these inputs, or for ``dtype=`` if given; memoised in
+        ``cache`` (reference: cupy/_core/_kernel.pyx:1652-1706)."""
         if dtype is None:
-            weaks_l = []
-            in_types_l = []
-            any_weak = False
-            for a in in_args:
-                if type(a) is CScalar:
-                    t = a.descr
-                    weak_t = a.weak_t
-                    if weak_t is not False:
-                        any_weak = True
-                elif isinstance(a, ndarray):
-                    t = a.dtype
-                    weak_t = False
-                else:
-                    raise RuntimeError(f'Need array or CScalar got {type(a)}')
-                in_types_l.append(t)
-                weaks_l.append(weak_t)
-            in_types = tuple(in_types_l)
-            weaks = tuple(weaks_l) if any_weak else None
-            if not _check_should_use_weak_scalar(in_types, weaks):
-                weaks = (False,) * len(in_args)
-            op = cache.get((in_types, weaks), ())
-            if op == ():
-                op = self._guess_routine_from_in_types(in_types, weaks)
-                cache[(in_types, weaks)] = op
+            in_types, weaks = _loop_selection_types(in_args)
+            key, asked = (in_types, weaks), in_types
+            search, what = self._guess_routine_from_in_types, (in_types, weaks)
         else:
-            op = cache.get(dtype, ())
-            if op == ():
-                ops_ = out_ops or self
-                op = ops_._guess_routine_from_dtype(dtype)
-                cache[dtype] = op
-        if op is not None:
-            op.check_valid()
-            return op
-        if dtype is None:
-            dtype = in_types
-        raise TypeError('Wrong type (%s) of arguments for %s' % (dtype, name))
+            key = asked = dtype
+            search, what = (out_ops or self)._guess_routine_from_dtype, (dtype,)
+        try:
+            op = cache[key]
+        except KeyError:
+            op = cache[key] = search(*what)
+        if op is None:
+            raise TypeError('Wrong type (%s) of arguments for %s' % (asked, name))
+        op.check_valid()        # (raises for a combination the ufunc forbids)
+        return op
 
     def _guess_routine_from_in_types(self, in_types, weaks=None):
         """First loop every input can be safely cast to.  A weak Python scalar
         that cannot be cast safely is still accepted when it would not change
         the loop's type under NumPy's promotion (NEP 50)."""
-        can_cast = numpy.can_cast
+        if weaks is None:
+            weaks = (False,) * len(in_types)
         for op in self.ops:
-            op_types = op.in_types
-            for i in range(self.nin):
-                it = in_types[i]
-                ot = op_types[i]
-                weak_t = weaks[i] if weaks is not None else False
-                if not can_cast(it, ot):
-                    if not weak_t:
-                        break
-                    try:
-                        if numpy.result_type(weak_t(0), ot) != ot:
-                            break
-                    except TypeError:
-                        break
-            else:
+            if all(_input_fits(given, wanted, weak)
+                   for given, wanted, weak in zip(in_types, op.in_types, weaks)):
                 return op
         return None
 
     def _guess_routine_from_dtype(self, dtype):
+        """First loop all of whose outputs have ``dtype``."""
         for op in self.ops:
-            for t in op.out_types:
-                if t != dtype:
-                    break
-            else:
+            if all(t == dtype for t in op.out_types):
                 return op
         return None
+
+
+def _read_loop_entry(entry, default):
+    """``(signature, routine, error function)`` of one loop-table entry.  A
+    bare signature takes the table's default routine; a pair may bring its own
+    routine, a tuple of routines whose gaps the default fills, or a callable
+    that raises for a forbidden type combination."""
+    if not isinstance(entry, tuple):
+        if not isinstance(entry, str):
+            raise ValueError(f'invalid op {entry}, expected string')
+        return entry, default, None
+    signature, own = entry
+    if own is None:
+        return signature, default, None
+    if isinstance(own, tuple):
+        return signature, tuple(mine or theirs for mine, theirs in zip(own, default)), None
+    if isinstance(own, str):
+        return signature, own, None
+    if not callable(own):
+        raise ValueError(f'invalid op {entry}, expected callable {own}')
+    return signature, None, own
+
+
+def _loop_selection_types(in_args):
+    """``(dtypes, weak types or None)`` of preprocessed inputs, as loop selection
+    sees them: a Python scalar counts as weak only where
+    ``_check_should_use_weak_scalar`` lets it."""
+    in_types = []
+    weaks = []
+    for arg in in_args:
+        if type(arg) is CScalar:
+            in_types.append(arg.descr)
+            weaks.append(arg.weak_t)
+        elif isinstance(arg, ndarray):
+            in_types.append(arg.dtype)
+            weaks.append(False)
+        else:
+            raise RuntimeError(f'Need array or CScalar got {type(arg)}')
+    in_types = tuple(in_types)
+    weaks = tuple(weaks) if any(w is not False for w in weaks) else None
+    if not _check_should_use_weak_scalar(in_types, weaks):
+        weaks = (False,) * len(in_types)
+    return in_types, weaks
+
+
+def _input_fits(given, wanted, weak):
+    """Whether an input of dtype ``given`` may feed a loop input of dtype
+    ``wanted``; ``weak`` is the Python type of a weak scalar or False."""
+    if numpy.can_cast(given, wanted):
+        return True
+    if not weak:
+        return False
+    try:
+        # a weak scalar that would promote the loop's type cannot use it
+        return numpy.result_type(weak(0), wanted) == wanted
+    except TypeError:
+        return False
+
+
+_UFUNC_KEYWORDS = frozenset(('out', '_where', 'dtype', 'casting'))
+
+
+def _preprocess_where(dev_id, where):
+    """The ``_where=`` argument as a one-element argument list: a boolean
+    array, or a scalar taken by its truth value."""
+    where_args = _preprocess_args(dev_id, (where,))
+    mask = where_args[0]
+    if not isinstance(mask, ndarray):
+        where_args[0] = CScalar(bool(mask.value))
+    elif mask.dtype != bool:
+        raise TypeError(
+            f'Cannot cast array data from {mask.dtype!r} to '
+            f'{get_dtype(bool)!r} according to the rule \'safe\'')
+    return where_args
 
 
 class ufunc:
@@ -1683,19 +1687,12 @@ class ufunc:
     def __init__(self, name, nin, nout, ops, preamble='', loop_prep='', doc='',
                  default_casting=None, *, out_ops=None, cutensor_op=None,
                  scatter_op=None):
-        self.name = name
-        self.__name__ = name
-        self.nin = nin
-        self.nout = nout
-        self.nargs = nin + nout
-        self._ops = ops
-        self._out_ops = out_ops
-        self._preamble = preamble
-        self._loop_prep = loop_prep
-        self._doc = doc
-        self.__doc__ = doc
-        self._default_casting = 'same_kind' if default_casting is None \
-            else default_casting
+        self.name = self.__name__ = name
+        self._doc = self.__doc__ = doc
+        self.nin, self.nout, self.nargs = nin, nout, nin + nout
+        self._ops, self._out_ops = ops, out_ops
+        self._preamble, self._loop_prep = preamble, loop_prep
+        self._default_casting = default_casting or 'same_kind'
         self._scatter_op = scatter_op
         _in_params = tuple(ParameterInfo('T in%d' % i, True) for i in range(nin))
         _out_params = tuple(ParameterInfo('T out%d' % i, False) for i in range(nout))
@@ -1719,6 +1716,38 @@ class ufunc:
             out_str = ''.join(get_dtype(t).char for t in op.out_types)
             types.append('%s->%s' % (in_str, out_str))
         return types
+
+    def _split_arguments(self, args, kwargs):
+        """``(inputs, outputs, where, dtype, casting)`` of a call; outputs may
+        come after the inputs or through ``out=`` (an array, or a tuple with
+        one entry per output).  Checks follow the reference's order and texts
+        (cupy/_core/_kernel.pyx:1268-1305)."""
+        unknown = {k: v for k, v in kwargs.items() if k not in _UFUNC_KEYWORDS}
+        dtype = kwargs.get('dtype')
+        if dtype is not None:
+            dtype = get_dtype(dtype).type
+        if unknown:
+            raise TypeError('Wrong arguments %s' % unknown)
+        given = len(args)
+        if given < self.nin or given > self.nargs:
+            raise TypeError(
+                'Wrong number of arguments for {!r}. '
+                'It must be either {} or {} (with outputs), '
+                'but given {}.'.format(self.name, self.nin, self.nargs, given))
+        inputs, outputs = args[:self.nin], args[self.nin:]
+        out = kwargs.get('out')
+        if out is not None:
+            if outputs:
+                raise ValueError('Cannot specify \'out\' as both '
+                                 'a positional and keyword argument')
+            as_tuple = isinstance(out, tuple)
+            outputs = out if as_tuple else (out,)
+            if len(outputs) != self.nout:
+                raise ValueError(
+                    "The 'out' tuple must have exactly one entry per ufunc output"
+                    if as_tuple else "'out' must be a tuple of arrays")
+        return (inputs, outputs, kwargs.get('_where'), dtype,
+                kwargs.get('casting', self._default_casting))
 
     def __call__(self, *args, **kwargs):
         """Applies the function elementwise.
@@ -1794,56 +1823,14 @@ class ufunc:
         if fast_key is not None:
             rec = _launch_plan.Recorder(self.nargs)
 
-        out = kwargs.pop('out', None)
-        where = kwargs.pop('_where', None)
+        in_args, out_args, where, dtype, casting = self._split_arguments(args, kwargs)
         has_where = where is not None
-        dtype = kwargs.pop('dtype', None)
-        casting = kwargs.pop('casting', self._default_casting)
-        if dtype is not None:
-            dtype = get_dtype(dtype).type
-        if kwargs:
-            raise TypeError('Wrong arguments %s' % kwargs)
-
-        n_args = len(args)
-        if not (self.nin <= n_args <= self.nargs):
-            raise TypeError(
-                'Wrong number of arguments for {!r}. '
-                'It must be either {} or {} (with outputs), '
-                'but given {}.'.format(self.name, self.nin, self.nargs, n_args))
-        in_args = args[:self.nin]
-        out_args = args[self.nin:]
-        if out is not None:
-            if out_args:
-                raise ValueError('Cannot specify \'out\' as both '
-                                 'a positional and keyword argument')
-            if isinstance(out, tuple):
-                if len(out) != self.nout:
-                    raise ValueError(
-                        "The 'out' tuple must have exactly one entry per "
-                        "ufunc output")
-                out_args = out
-            else:
-                if 1 != self.nout:
-                    raise ValueError("'out' must be a tuple of arrays")
-                out_args = out,
 
         dev_id = _device.get_device_id()
         in_args = _preprocess_args(dev_id, in_args)
         out_args = _preprocess_optional_args(dev_id, out_args)
         given_out_args = [o for o in out_args if o is not None]
-
-        if has_where:
-            where_args = _preprocess_args(dev_id, (where,))
-            x = where_args[0]
-            if isinstance(x, ndarray):
-                if x.dtype != bool:
-                    raise TypeError(
-                        f'Cannot cast array data from {x.dtype!r} to '
-                        f'{get_dtype(bool)!r} according to the rule \'safe\'')
-            else:
-                where_args[0] = CScalar(bool(x.value))
-        else:
-            where_args = []
+        where_args = _preprocess_where(dev_id, where) if has_where else []
 
         if rec is not None:
             before = list(in_args)
@@ -1860,14 +1847,10 @@ class ufunc:
         op = self._ops.guess_routine(
             self.name, self._routine_cache, in_args, dtype, self._out_ops)
 
-        subtype = ndarray
-        template = None
-        for in_arg in in_args:
-            t = type(in_arg)
-            if t is not ndarray and issubclass(t, ndarray):
-                subtype = t
-                template = in_arg
-                break
+        # outputs are of the first array subclass among the inputs
+        template = next((a for a in in_args
+                         if type(a) is not ndarray and isinstance(a, ndarray)), None)
+        subtype = ndarray if template is None else type(template)
 
         core_in_dtypes, core_out_dtypes = op.resolve_dtypes(in_args, out_args)
         out_args = _get_out_args_from_optionals(
@@ -1980,20 +1963,22 @@ class ufunc:
         from cupy_amd._core import _scatter
         _scatter.scatter_op(a, indices, b, self._scatter_op)
 
+    # reductions and scans exist for the two ufuncs whose reduction is an
+    # ndarray method (cupy/_core/_kernel.pyx:1452-1483)
+    _REDUCE_METHODS = {'cupy_add': 'sum', 'cupy_multiply': 'prod'}
+    _ACCUMULATE_METHODS = {'cupy_add': 'cumsum', 'cupy_multiply': 'cumprod'}
+
     def reduce(self, array, axis=0, dtype=None, out=None, keepdims=False):
-        if self.name == 'cupy_add':
-            return array.sum(axis, dtype, out, keepdims)
-        if self.name == 'cupy_multiply':
-            return array.prod(axis, dtype, out, keepdims)
-        raise NotImplementedError(f'`{self.name}.reduce` is not supported yet')
+        method = self._REDUCE_METHODS.get(self.name)
+        if method is None:
+            raise NotImplementedError(f'`{self.name}.reduce` is not supported yet')
+        return getattr(array, method)(axis, dtype, out, keepdims)
 
     def accumulate(self, array, axis=0, dtype=None, out=None):
-        if self.name == 'cupy_add':
-            return array.cumsum(axis, dtype, out)
-        if self.name == 'cupy_multiply':
-            return array.cumprod(axis, dtype, out)
-        raise NotImplementedError(
-            f'`{self.name}.accumulate` is not supported yet')
+        method = self._ACCUMULATE_METHODS.get(self.name)
+        if method is None:
+            raise NotImplementedError(f'`{self.name}.accumulate` is not supported yet')
+        return getattr(array, method)(axis, dtype, out)
 
     def reduceat(self, array, indices, axis=0, dtype=None, out=None):
         """``numpy.ufunc.reduceat`` for add (cupy/_core/_kernel.pyx:1485-1493)."""

@@ -17,6 +17,7 @@ import numpy
 from cupy_amd._core import _tuning
 from cupy_amd.cuda import _giveup
 from cupy_amd.cuda import memory as _memory
+from cupy_amd.cuda import stream as _stream
 
 HEADER_WORDS = 64
 MAX_STREAMS = 64    # (device, stream) pairs that hold a block at a time
@@ -47,10 +48,15 @@ def acquire(dev_id, stream_ptr, current_stream_ptr, n_slots):
     ``stream_ptr`` that needs ``n_slots`` slots, or None where the reduction
     has to take two launches: switched off, a stream other than the current
     one (the block is cleared on the current stream), more slots than a block
-    may hold, no allocation allowed, or an earlier failure on this device."""
+    may hold, the per-thread default stream, no allocation allowed, or an
+    earlier failure on this device."""
     if not _tuning.get('reduce_finish') or dev_id in _giveup.disabled[_giveup.REDUCTION]:
         return None
     if stream_ptr != current_stream_ptr or n_slots > _tuning.get('reduce_finish_max_slots'):
+        return None
+    if stream_ptr == _stream.STREAM_PER_THREAD:
+        # one handle, a different stream in every thread: launches that share
+        # a block could overlap
         return None
     if _memory._static_scratch_open and _memory.static_scratch_active():
         return None

@@ -702,7 +702,8 @@ class _AbstractReductionKernel:
         if (group == _cg.BLOCK and n_out < cus * _tuning.get('min_blocks_per_cu')
                 and (n_red * max_item >= 128 * 1024 or stage)):
             trip = wg * vec
-            want = (cus * _tuning.get('target_blocks_per_cu') + n_out - 1) // n_out
+            want = (cus * (_tuning.get('rows_target_blocks_per_cu')
+                           or _tuning.get('target_blocks_per_cu')) + n_out - 1) // n_out
             most = max(1, n_red // (trip * _tuning.get('rows_split_min_trips')))
             n_split = max(1, min(want, most, 65535))
             if n_split > 1:
@@ -872,7 +873,7 @@ class _AbstractReductionKernel:
             if ok:
                 break
             vec //= 2
-        tx = max(1, min(64, internal.clp2((n_cols + vec - 1) // vec)))
+        tx = max(1, min(_tuning.get('cols_tx'), internal.clp2((n_cols + vec - 1) // vec)))
         # a handful of rows and plenty of columns: a thread per column vector
         solo_block = _tuning.get('cols_solo_block')
         solo = (n_red <= 8 and n_out >= cus * solo_block * vec
@@ -887,9 +888,13 @@ class _AbstractReductionKernel:
         # hold they continue along grid.z
         gz = (gx + _max_blocks(block) - 1) // _max_blocks(block)
         gx = (gx + gz - 1) // gz
-        want = (cus * _tuning.get('target_blocks_per_cu') + gx * gz - 1) // (gx * gz)
+        want = (cus * (_tuning.get('cols_target_blocks_per_cu')
+                       or _tuning.get('target_blocks_per_cu')) + gx * gz - 1) // (gx * gz)
         most = max(1, n_red // (ty * 8))
         n_split = max(1, min(want, most, 65535))
+        if 1 < n_split and cus * 8 < gx * gz * n_split:
+            # (never a few workgroups more than the device holds at once)
+            n_split = max(1, cus * 8 // (gx * gz))
         partial = n_split > 1
         span = max([abs(s_o) * n_out + abs(s_r) * n_red for s_o, s_r in zip(so_in, sr)]
                    + [abs(s) * n_out for s in so_out] + [n_red + n_split * ty])

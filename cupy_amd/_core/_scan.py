@@ -2186,6 +2186,10 @@ def _chain_ready():
     dev_id = _device.get_device_id()
     if dev_id in _giveup.disabled[_giveup.SCAN]:
         return None
+    if _stream.get_current_stream_ptr() == _stream.STREAM_PER_THREAD:
+        # (one handle, a different stream in every thread: the published
+        # totals of two threads' scans would share their memory)
+        return None
     fault = _chain_fault_word(dev_id)
     # A tile of an earlier scan that gave up waiting for the tiles before it
     # left wrong results.  Not expected to happen: poll() says so, and the

@@ -87,6 +87,23 @@ _params = {
     # `cols_unroll_near` (64 x 64 x 16384, axis 1: 56.0 -> 47.8 us; 257 x 511 x
     # 509: 78.5 -> 60.6 us)
     'cols_unroll': 1,
+    # Lanes across the columns of a workgroup, at most (the rest of its 256
+    # threads goes down the reduce axis).  Sums over axis 0 of 16384^2 float32 /
+    # 8192^2 float64, timed between other operations on other arrays: 161 / 84 us
+    # with 64 lanes, 156 / 81 with 32, 166 / 86 with 16 (same number of workgroups)
+    'cols_tx': 32,
+    # How far the reduce axis is split, in workgroups per CU.  A CU holds eight
+    # workgroups of 256 threads: a grid of more than that many runs its last
+    # workgroups alone (16384^2 float32, axis 0, 128 column blocks: 159 us with
+    # 16 slices, 208 with 17), and a grid that fills every slot is slower than
+    # one that leaves a few free (10 to 12 slices: 151 to 153 us; float64
+    # 8192^2: 78.6 to 79.5 against 81.7)
+    'cols_target_blocks_per_cu': 5,
+    # ... and for a row cut into chunks (sum of all elements).  Every lane has
+    # four accesses in flight here, so fewer workgroups saturate the memory:
+    # 2^28 float32 in 2048 / 1024 / 512 / 384 / 256 chunks: 161 / 160 / 154 /
+    # 155 / 183 us; 2^26 float64: 84 / 83 / 80 / 82 / 93
+    'rows_target_blocks_per_cu': 2,
     'cols_unroll_near': 4,
     'cols_solo_block': 1024,    # workgroup of the thread-per-column variant
     # Grid cap of the scan kernels, in workgroups per CU (cumsum along rows of

@@ -14,8 +14,13 @@ from cupy_amd.cuda import memory as _memory
 _module_file_memo = {}
 
 
-def _get_raw_module(code, path, options, name_expressions, log_stream):
+def _get_raw_module(code, path, options, name_expressions, log_stream,
+                    enable_cooperative_groups=False):
     if code is not None:
+        if enable_cooperative_groups:
+            # <hip/hip_cooperative_groups.h> is not among the headers the
+            # run-time compiler carries itself: it comes from the installation
+            options = tuple(options) + ('-I' + _compiler.rocm_include_dir(),)
         return _compiler.compile_raw_with_cache(
             code, options, name_expressions=name_expressions, log_stream=log_stream)
     key = (_device.get_device_id(), path)
@@ -37,8 +42,10 @@ class RawKernel:
         backend (str): ``'nvrtc'`` (the run-time compiler, here hiprtc) is the
             only backend.
         translate_cucomplex (bool): Accepted for compatibility; no effect.
-        enable_cooperative_groups (bool): Must be False: grid-wide
-            synchronisation is not available through this launch path.
+        enable_cooperative_groups (bool): Launch cooperatively (all
+            workgroups resident at once), so that the kernel may use
+            ``cooperative_groups::this_grid().sync()``; the installation's
+            include directory is added for ``<hip/hip_cooperative_groups.h>``.
 
     ``kernel(grid, block, args, shared_mem=0, stream=None)`` launches; array
     arguments are passed as device pointers, NumPy scalars by value with their
@@ -53,8 +60,6 @@ class RawKernel:
             raise TypeError('options must be a tuple')
         if backend not in ('nvrtc', 'hiprtc'):
             raise ValueError('only the run-time compiler backend is available')
-        if enable_cooperative_groups:
-            raise ValueError('cooperative launches are not supported')
         if jitify:
             raise ValueError('jitify is not available')
         self.code = code
@@ -79,7 +84,8 @@ class RawKernel:
             shared_mem (int): Dynamic LDS bytes per workgroup.
             stream: Stream to launch on (default: current stream).
         """
-        self.kernel(grid, block, args, **kwargs)
+        self.kernel(grid, block, args,
+                    enable_cooperative_groups=self.enable_cooperative_groups, **kwargs)
 
     @property
     def kernel(self):
@@ -91,7 +97,8 @@ class RawKernel:
         if ker is None or log_stream is not None:
             assert (self.code is None) != (self.file_path is None)
             mod = _get_raw_module(self.code, self.file_path, self.options,
-                                  self.name_expressions, log_stream)
+                                  self.name_expressions, log_stream,
+                                  self.enable_cooperative_groups)
             ker = mod.get_function(self.name)
             self._kernel_cache[dev] = ker
         return ker
@@ -151,8 +158,7 @@ class RawKernel:
 
     @max_dynamic_shared_size_bytes.setter
     def max_dynamic_shared_size_bytes(self, nbytes):
-        raise RuntimeError('function attributes cannot be changed on this device: '
-                           'every kernel may use the whole LDS of a compute unit')
+        self.kernel.set_attribute('max_dynamic_shared_size_bytes', nbytes)
 
     @property
     def preferred_shared_memory_carveout(self):
@@ -160,8 +166,7 @@ class RawKernel:
 
     @preferred_shared_memory_carveout.setter
     def preferred_shared_memory_carveout(self, fraction):
-        raise RuntimeError('function attributes cannot be changed on this device: '
-                           'LDS and cache do not share storage')
+        self.kernel.set_attribute('preferred_shared_memory_carveout', fraction)
 
 
 class RawModule:
@@ -194,8 +199,6 @@ class RawModule:
             self.name_expressions = None
         if jitify:
             raise ValueError('jitify is not available')
-        if enable_cooperative_groups:
-            raise ValueError('cooperative launches are not supported')
         if not isinstance(options, tuple):
             raise TypeError('options must be a tuple')
         self.code = code
@@ -217,7 +220,8 @@ class RawModule:
 
     def _module(self, log_stream=None):
         return _get_raw_module(self.code, self.file_path, self.options,
-                               self.name_expressions, log_stream)
+                               self.name_expressions, log_stream,
+                               self.enable_cooperative_groups)
 
     def compile(self, log_stream=None):
         """Compiles now instead of at first use."""
@@ -231,7 +235,8 @@ class RawModule:
             if mangled is not None:
                 name = mangled
         ker = RawKernel(self.code if self.code is not None else '', name, self.options,
-                        'nvrtc', translate_cucomplex=self.translate_cucomplex)
+                        'nvrtc', translate_cucomplex=self.translate_cucomplex,
+                        enable_cooperative_groups=self.enable_cooperative_groups)
         if self.code is None:
             ker.code = None
         ker.file_path = self.file_path

@@ -118,8 +118,12 @@ _PROTOTYPES = {
     'rt_func_get_attribute': (_c.c_int, [_c.c_int, _vp, _c.POINTER(_c.c_int)]),
     'rt_occupancy_max_active_blocks': (_c.c_int, [
         _vp, _c.c_int, _c.c_size_t, _c.POINTER(_c.c_int)]),
+    'rt_func_set_attribute': (_c.c_int, [_vp, _c.c_int, _c.c_int]),
     'rt_launch': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [_vp, _c.POINTER(_vp)]),
+    'rt_launch_cooperative': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [_vp, _c.POINTER(_vp)]),
     'rt_launch_packed': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [_vp, _vp, _c.c_size_t]),
+    'rt_launch_packed_timed': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [
+        _vp, _vp, _c.c_size_t, _vp, _vp]),
     'rt_launch_packed_scratch': (_c.c_int, [_vp] + [_c.c_uint] * 7 + [
         _vp, _vp, _c.c_size_t, _c.c_size_t, _c.c_size_t]),
     'rt_malloc': (_c.c_int, [_c.POINTER(_vp), _c.c_size_t]),

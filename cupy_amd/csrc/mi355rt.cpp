@@ -5,6 +5,7 @@
 #include "mi355rt.h"
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hiprtc.h>
 
 #include <cstdio>
@@ -320,6 +321,23 @@ int rt_func_get_attribute(int attribute, void* function, int* value) {
   return 0;
 }
 
+int rt_func_set_attribute(void* function, int attribute, int value) {
+  if (!function) return fail_invalid("rt_func_set_attribute: null function");
+  hipFuncAttribute attr;
+  switch (attribute) {
+    case HIP_FUNC_ATTRIBUTE_MAX_DYNAMIC_SHARED_SIZE_BYTES:
+      attr = hipFuncAttributeMaxDynamicSharedMemorySize;
+      break;
+    case HIP_FUNC_ATTRIBUTE_PREFERRED_SHARED_MEMORY_CARVEOUT:
+      attr = hipFuncAttributePreferredSharedMemoryCarveout;
+      break;
+    default:
+      return fail_invalid("rt_func_set_attribute: this attribute cannot be set");
+  }
+  RT_HIP(hipFuncSetAttribute(function, attr, value));
+  return 0;
+}
+
 int rt_occupancy_max_active_blocks(void* function, int block_size, size_t dynamic_smem,
                                    int* num_blocks) {
   if (!function || !num_blocks) return fail_invalid("rt_occupancy_max_active_blocks: null argument");
@@ -338,6 +356,18 @@ int rt_launch(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx
   return 0;
 }
 
+int rt_launch_cooperative(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                          unsigned by, unsigned bz, unsigned shared_mem, void* stream,
+                          void** params) {
+  if (!function) return fail_invalid("rt_launch_cooperative: null function");
+  if (gx == 0 || gy == 0 || gz == 0 || bx == 0 || by == 0 || bz == 0)
+    return fail_invalid("rt_launch_cooperative: zero-sized grid or block");
+  RT_HIP(hipModuleLaunchCooperativeKernel(static_cast<hipFunction_t>(function), gx, gy, gz, bx,
+                                          by, bz, shared_mem, static_cast<hipStream_t>(stream),
+                                          params));
+  return 0;
+}
+
 int rt_launch_packed(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
                      unsigned by, unsigned bz, unsigned shared_mem, void* stream,
                      const void* arg_block, size_t arg_block_size) {
@@ -349,6 +379,28 @@ int rt_launch_packed(void* function, unsigned gx, unsigned gy, unsigned gz, unsi
                    HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
   RT_HIP(hipModuleLaunchKernel(static_cast<hipFunction_t>(function), gx, gy, gz, bx, by, bz,
                                shared_mem, static_cast<hipStream_t>(stream), nullptr, extra));
+  return 0;
+}
+
+int rt_launch_packed_timed(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                           unsigned by, unsigned bz, unsigned shared_mem, void* stream,
+                           const void* arg_block, size_t arg_block_size, void* start_event,
+                           void* stop_event) {
+  if (!function) return fail_invalid("rt_launch_packed_timed: null function");
+  if (gx == 0 || gy == 0 || gz == 0 || bx == 0 || by == 0 || bz == 0)
+    return fail_invalid("rt_launch_packed_timed: zero-sized grid or block");
+  // (this launch takes its grid in work-items, 32 bits per dimension)
+  if (static_cast<uint64_t>(gx) * bx > 0xffffffffull ||
+      static_cast<uint64_t>(gy) * by > 0xffffffffull ||
+      static_cast<uint64_t>(gz) * bz > 0xffffffffull)
+    return fail_invalid("rt_launch_packed_timed: more than 2^32 - 1 work-items in one dimension");
+  size_t size = arg_block_size;
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(arg_block),
+                   HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  RT_HIP(hipExtModuleLaunchKernel(static_cast<hipFunction_t>(function), gx * bx, gy * by, gz * bz,
+                                  bx, by, bz, shared_mem, static_cast<hipStream_t>(stream),
+                                  nullptr, extra, static_cast<hipEvent_t>(start_event),
+                                  static_cast<hipEvent_t>(stop_event), 0));
   return 0;
 }
 

@@ -318,6 +318,17 @@ def _decode_named_payload(payload, count):
     return names, payload[pos:]
 
 
+def rocm_include_dir():
+    """Include directory of the ROCm installation (``ROCM_HOME`` / ``ROCM_PATH``,
+    else /opt/rocm; the reference looks for the installation the same way,
+    cupy/_environment.py:214-230)."""
+    for var in ('ROCM_HOME', 'ROCM_PATH'):
+        root = os.environ.get(var)
+        if root and os.path.isdir(os.path.join(root, 'include')):
+            return os.path.join(root, 'include')
+    return '/opt/rocm/include'
+
+
 def compile_raw_with_cache(source, options=(), name_expressions=None, log_stream=None):
     """Loaded module for user-written source (cupy/_core/raw.pyx:541-558
     ``_get_raw_module``): no bundled headers are prepended, the user's options

@@ -28,6 +28,10 @@ _FUNC_ATTRIBUTES = {
 }
 
 
+# cupy_amd.profiler.KernelTimer while one is active, else None
+_kernel_timer = None
+
+
 def _arg_to_bytes(arg):
     """Bytes of one kernel argument passed by value."""
     if hasattr(arg, '_kernel_arg_bytes'):      # ndarray, Indexer, CScalar
@@ -137,6 +141,14 @@ class Function:
             _FUNC_ATTRIBUTES[name], self.ptr, ctypes.byref(v)))
         return v.value
 
+    def set_attribute(self, name, value):
+        """Sets 'max_dynamic_shared_size_bytes' or
+        'preferred_shared_memory_carveout' (reference:
+        cupy_backends/cuda/api/driver.pyx:322-330 ``funcSetAttribute``)."""
+        if _dryrun.enabled():
+            return
+        _rt.check(_rt.lib.rt_func_set_attribute(self.ptr, _FUNC_ATTRIBUTES[name], int(value)))
+
     @property
     def attributes(self):
         out = {}
@@ -177,6 +189,12 @@ class Function:
         if _dryrun.enabled():
             _dryrun.record_launch(self.name, grid, block, shared_mem, bytes(arg_block))
             return
+        if _kernel_timer is not None:
+            start, stop = _kernel_timer._next(self.name)
+            _rt.check(_rt.lib.rt_launch_packed_timed(
+                self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr,
+                bytes(arg_block), len(arg_block), start.ptr, stop.ptr))
+            return
         status = _rt.hot.launch(
             self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr, arg_block)
         if status != 0:
@@ -213,7 +231,40 @@ class Function:
         if status != 0:
             _rt.check(status)
 
-    def __call__(self, grid, block, args, shared_mem=0, stream=None):
+    def launch_cooperative(self, grid, block, arg_block, shared_mem=0, stream_ptr=None):
+        """``launch_packed`` as a cooperative launch: every workgroup of the
+        grid is resident at once, so the kernel may synchronise the whole grid
+        (reference: cupy/cuda/function.pyx:113-131 with
+        ``enable_cooperative_groups``, driver.pyx:289-301).  The runtime
+        refuses a grid larger than the device can hold at once."""
+        if stream_ptr is None:
+            stream_ptr = _stream.get_current_stream_ptr()
+        gx, gy, gz = grid
+        bx, by, bz = block
+        if gx * bx > 0xffffffff or gy * by > 0xffffffff or gz * bz > 0xffffffff:
+            raise ValueError(
+                'kernel %s: grid %r x block %r exceeds 2**32 - 1 work-items in one dimension'
+                % (self.name, grid, block))
+        n = len(arg_block)
+        if n > self._arg_size or n < self._arg_min:
+            raise ValueError(
+                'kernel %s expects an argument block of %d bytes, got %d'
+                % (self.name, self._arg_size, n))
+        arg_block = bytes(arg_block) + b'\0' * (self._arg_size - n)
+        if _dryrun.enabled():
+            _dryrun.record_launch(self.name, grid, block, shared_mem, arg_block)
+            return
+        # this launch takes one pointer per parameter: into a copy of the block
+        buf = ctypes.create_string_buffer(arg_block, max(1, len(arg_block)))
+        base = ctypes.addressof(buf)
+        params = self.meta['args']
+        pointers = (ctypes.c_void_p * max(1, len(params)))(
+            *[base + offset for offset, _size, _kind in params])
+        _rt.check(_rt.lib.rt_launch_cooperative(
+            self.ptr, gx, gy, gz, bx, by, bz, shared_mem, stream_ptr, pointers))
+
+    def __call__(self, grid, block, args, shared_mem=0, stream=None,
+                 enable_cooperative_groups=False):
         """Launch with one Python object per kernel parameter.  Each object's
         bytes are placed at the parameter's offset in the argument block, cut
         or zero-padded to the parameter's size as recorded in the code object
@@ -233,7 +284,10 @@ class Function:
             blob[offset:offset + n] = b[:n]
         stream_ptr = (_stream.get_current_stream_ptr() if stream is None
                       else stream.ptr)
-        self.launch_packed(grid, block, bytes(blob), shared_mem, stream_ptr)
+        if enable_cooperative_groups:
+            self.launch_cooperative(grid, block, bytes(blob), shared_mem, stream_ptr)
+        else:
+            self.launch_packed(grid, block, bytes(blob), shared_mem, stream_ptr)
 
     def linear_launch(self, size, args, shared_mem=0, block_max_size=128,
                       stream=None):

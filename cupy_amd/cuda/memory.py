@@ -18,6 +18,8 @@ from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import stream as _stream
 from cupy_amd.cuda import memory_hook as _memory_hook
 
+_STREAM_PER_THREAD = _stream.STREAM_PER_THREAD
+
 _allocation_unit_size = 512
 
 
@@ -378,6 +380,8 @@ class SingleDeviceMemoryPool:
             return MemoryPointer(Memory(0), 0)
         rounded = _round_size(size)
         stream_ident = _stream.get_current_stream_ptr()
+        if stream_ident == _STREAM_PER_THREAD:
+            stream_ident = _stream.stream_identifier(stream_ident)
         handle = self._handle_value
         pool_malloc = _rt.hot.pool_malloc
         addr = pool_malloc(handle, rounded, stream_ident)
@@ -401,7 +405,8 @@ class SingleDeviceMemoryPool:
         if stream is None:
             _rt.check(_rt.lib.rt_pool_free_all_blocks(self._handle, 1, 0))
         else:
-            _rt.check(_rt.lib.rt_pool_free_all_blocks(self._handle, 0, stream.ptr))
+            _rt.check(_rt.lib.rt_pool_free_all_blocks(
+                self._handle, 0, _stream.stream_identifier(stream.ptr)))
 
     def free_all_free(self):
         warnings.warn('free_all_free is deprecated. Use free_all_blocks instead.',

@@ -1,6 +1,8 @@
 """Streams and events (reference: cupy/cuda/stream.pyx:101-186,459-598 and
 cupy_backends/cuda/stream.pyx:14-100 for the thread-local current stream)."""
 import ctypes
+import itertools
+import os
 import threading
 
 from cupy_amd import _dryrun
@@ -9,15 +11,54 @@ from cupy_amd.cuda import _giveup
 
 _tls = threading.local()
 
+# hipStreamLegacy / hipStreamPerThread: handles the runtime itself knows
+STREAM_LEGACY = 1
+STREAM_PER_THREAD = 2
+
+# CUPY_CUDA_PER_THREAD_DEFAULT_STREAM=1: a thread that has made no stream
+# current works on its own default stream instead of the one all threads share
+# (reference: cupy_backends/cuda/stream.pyx:10-11,33-44)
+_ptds = int(os.environ.get('CUPY_CUDA_PER_THREAD_DEFAULT_STREAM', '0') or '0') != 0
+_thread_numbers = itertools.count(1)
+
+
+def is_ptds_enabled():
+    return _ptds
+
+
+def get_default_stream_ptr():
+    """Handle of the default stream (cupy_backends/cuda/stream.pyx:84-94)."""
+    return STREAM_PER_THREAD if _ptds else STREAM_LEGACY
+
 
 def get_current_stream_ptr():
-    """Raw handle of the calling thread's current stream (0 = null stream)."""
-    return getattr(_tls, 'ptr', 0)
+    """Raw handle of the calling thread's current stream (0 = null stream;
+    with per-thread default streams switched on, the per-thread stream where
+    the thread has made no other stream current)."""
+    ptr = getattr(_tls, 'ptr', 0)
+    if _ptds and ptr == 0:
+        return STREAM_PER_THREAD
+    return ptr
 
 
 def get_current_stream():
     cur = getattr(_tls, 'stream', None)
-    return Stream.null if cur is None else cur
+    if cur is None:
+        return Stream.ptds if _ptds else Stream.null
+    return cur
+
+
+def stream_identifier(stream_ptr):
+    """What tells the memory of one stream from another's: the handle, except
+    for the per-thread default stream, whose one handle stands for a different
+    stream in every thread (reference: cupy/cuda/memory.pyx:877-889).  Thread
+    numbers are never reused and have the top bit set, which no handle has."""
+    if stream_ptr != STREAM_PER_THREAD:
+        return stream_ptr
+    ident = getattr(_tls, 'ident', None)
+    if ident is None:
+        ident = _tls.ident = (1 << 63) | next(_thread_numbers)
+    return ident
 
 
 def _set_current(stream):
@@ -80,18 +121,23 @@ def get_elapsed_time(start_event, end_event):
 
 
 class Stream:
-    """hipStream wrapper.  ``Stream.null`` is the default stream.  Streams are
-    created at the default priority."""
+    """hipStream wrapper.  ``Stream.null`` is the default stream all threads
+    share, ``Stream.ptds`` the calling thread's own default stream
+    (``hipStreamPerThread``).  Streams are created at the default priority."""
 
     null = None
+    ptds = None
 
     def __init__(self, null=False, non_blocking=False, ptds=False):
-        if ptds:
-            raise NotImplementedError('per-thread default stream is not supported')
         self._owned = False
         self._prev = []
         self.ptr = 0
-        if null or _dryrun.enabled():
+        if null:
+            return
+        if ptds:
+            self.ptr = STREAM_PER_THREAD
+            return
+        if _dryrun.enabled():
             return
         p = ctypes.c_void_p()
         _rt.check(_rt.lib.rt_stream_create(ctypes.byref(p), int(non_blocking)))
@@ -156,3 +202,4 @@ class Stream:
 
 
 Stream.null = Stream(null=True)
+Stream.ptds = Stream(ptds=True)

@@ -64,3 +64,60 @@ def benchmark(func, args=(), kwargs={}, n_repeat=10000, *, name=None,
         if duration > max_duration:
             break
     return PerfCaseResult(name, cpu_times, gpu_times)
+
+
+class KernelTimer:
+    """Times every kernel launched inside the ``with`` block by the device's
+    own clock: each launch carries two events that receive the start and the
+    end of that kernel's execution (``rt_launch_packed_timed``), which is the
+    duration a profiler's kernel trace shows for the dispatch.  Unlike events
+    recorded between calls, this adds no marker to the stream between the
+    kernels, so back-to-back launches run as they do untimed.
+
+    While a timer is active every launch takes the full Python launch path
+    (recorded calls are replayed launch by launch instead of in one go), so
+    host time per call is higher; device time is what is measured.
+
+    ``durations()`` waits for the device and returns ``[(kernel name,
+    seconds), ...]`` in launch order.  Not thread-safe: one timer at a time.
+    """
+
+    def __init__(self):
+        self._launches = []     # (name, start event, stop event)
+        self._spare = []
+
+    def _next(self, name):
+        pair = self._spare.pop() if self._spare else (_stream.Event(), _stream.Event())
+        self._launches.append((name,) + pair)
+        return pair
+
+    def __enter__(self):
+        from cupy_amd._core import _launch_plan
+        from cupy_amd.cuda import function
+        if function._kernel_timer is not None:
+            raise RuntimeError('another KernelTimer is active')
+        self._quick = _launch_plan.use_quick
+        _launch_plan.use_quick = False
+        function._kernel_timer = self
+        return self
+
+    def __exit__(self, *exc):
+        from cupy_amd._core import _launch_plan
+        from cupy_amd.cuda import function
+        function._kernel_timer = None
+        _launch_plan.use_quick = self._quick
+
+    def mark(self):
+        """Number of launches seen so far (to tell one call's kernels from the
+        next call's)."""
+        return len(self._launches)
+
+    def durations(self):
+        from cupy_amd.cuda import device
+        device.Device().synchronize()
+        out = []
+        for name, start, stop in self._launches:
+            out.append((name, _stream.get_elapsed_time(start, stop) * 1e-3))
+        self._spare.extend((a, b) for _, a, b in self._launches)
+        self._launches = []
+        return out

@@ -117,6 +117,12 @@ int rt_module_get_function(void* module, const char* name, void** function);
 int rt_module_get_global(void* module, const char* name, void** dptr, size_t* bytes);
 /* driver.pyx:309 funcGetAttribute; `attribute` is a hipFunction_attribute value */
 int rt_func_get_attribute(int attribute, void* function, int* value);
+/* driver.pyx:322-330 funcSetAttribute (a stub returning hipErrorUnknown in
+ * cupy_backends/hip/cupy_hip.h:130-132; real here).  `attribute` is a
+ * hipFunction_attribute value as for rt_func_get_attribute; the two settable
+ * ones are MAX_DYNAMIC_SHARED_SIZE_BYTES and PREFERRED_SHARED_MEMORY_CARVEOUT
+ * (cupy/_core/raw.pyx:226-287). */
+int rt_func_set_attribute(void* function, int attribute, int value);
 /* driver.pyx:335 occupancyMaxActiveBlocksPerMultiprocessor (a stub returning
  * hipErrorUnknown in cupy_backends/hip/cupy_hip.h:125-137; real here) */
 int rt_occupancy_max_active_blocks(void* function, int block_size,
@@ -127,6 +133,16 @@ int rt_launch(void* function,
               unsigned gx, unsigned gy, unsigned gz,
               unsigned bx, unsigned by, unsigned bz,
               unsigned shared_mem, void* stream, void** params);
+/* driver.pyx:289-301 launchCooperativeKernel (a stub returning hipErrorUnknown
+ * in cupy_backends/hip/cupy_hip.h:121-123; real here): all workgroups of the
+ * grid are resident at once, so the kernel may synchronise the whole grid
+ * (cooperative_groups::this_grid().sync()).  A grid larger than the device can
+ * hold at once is refused with hipErrorCooperativeLaunchTooLarge.  Used by
+ * RawKernel(enable_cooperative_groups=True) (cupy/cuda/function.pyx:113-131). */
+int rt_launch_cooperative(void* function,
+                          unsigned gx, unsigned gy, unsigned gz,
+                          unsigned bx, unsigned by, unsigned bz,
+                          unsigned shared_mem, void* stream, void** params);
 /* Same launch with the arguments already laid out as the kernel's argument
  * block (each argument at its natural alignment); saves building the pointer
  * array that function.pyx:104-127 builds per call. */
@@ -135,6 +151,19 @@ int rt_launch_packed(void* function,
                      unsigned bx, unsigned by, unsigned bz,
                      unsigned shared_mem, void* stream,
                      const void* arg_block, size_t arg_block_size);
+
+/* No counterpart in the reference (its profiler brackets host calls with
+ * events, cupyx/profiler/_time.py:164-234).  For measurement: rt_launch_packed
+ * with two events that receive the start and the end of THIS kernel's execution
+ * on the device, so that rt_event_elapsed_ms(start, stop) is the duration a
+ * profiler's kernel trace reports for the dispatch, with nothing of the
+ * neighbouring launches in it.  Both events must exist; either may be null. */
+int rt_launch_packed_timed(void* function,
+                           unsigned gx, unsigned gy, unsigned gz,
+                           unsigned bx, unsigned by, unsigned bz,
+                           unsigned shared_mem, void* stream,
+                           const void* arg_block, size_t arg_block_size,
+                           void* start_event, void* stop_event);
 
 /*
  * No counterpart in the reference.  For callers that cannot allocate device

@@ -24,6 +24,14 @@
  * are compared with math.fsum within rtol.  The summation order itself cannot
  * be validated against the reference here (it needs a GPU build of the
  * reference): parity unpinned for the order.
+ *
+ * Who uses this file: tests/test_oracle.py only (through oracle/c_oracle.py).
+ * No GPU test, no benchmark and no product code consumes it: GPU results are
+ * compared with NumPy (oracle/numpy_oracle.py), whose values this restatement
+ * is itself compared with.  ref_get_block_specs exists for the summation
+ * order of ref_block_reduce_*; its table of expected triples in
+ * tests/golden/reference_kats.json was evaluated by hand from the same
+ * formula, which pins nothing beyond a consistent reading of that formula.
  */
 #include <math.h>
 #include <stddef.h>

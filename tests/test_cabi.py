@@ -44,6 +44,13 @@ def test_invalid_arguments_are_reported_not_crashed():
     assert _rt.lib.rt_launch(None, 1, 1, 1, 1, 1, 1, 0, None, None) == _rt.RT_ERR_INVALID
     assert _rt.lib.rt_pool_malloc(None, 16, 0, None) == _rt.RT_ERR_INVALID
     assert b'null' in _rt.lib.rt_last_error_string()
+    assert _rt.lib.rt_launch_cooperative(None, 1, 1, 1, 1, 1, 1, 0, None, None) == _rt.RT_ERR_INVALID
+    assert _rt.lib.rt_func_set_attribute(None, 8, 1024) == _rt.RT_ERR_INVALID
+    fake = ctypes.addressof((ctypes.c_ubyte * 8)())
+    assert _rt.lib.rt_launch_cooperative(fake, 0, 1, 1, 1, 1, 1, 0, None, None) == _rt.RT_ERR_INVALID
+    # only the two attributes the reference can set (cupy/_core/raw.pyx:226-287)
+    assert _rt.lib.rt_func_set_attribute(fake, 4, 1) == _rt.RT_ERR_INVALID
+    assert b'cannot be set' in _rt.lib.rt_last_error_string()
     major = ctypes.c_int(0)
     minor = ctypes.c_int(0)
     assert _rt.lib.rt_rtc_version(ctypes.byref(major), ctypes.byref(minor)) == 0

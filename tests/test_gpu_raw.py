@@ -170,3 +170,105 @@ def test_load_code_object_from_file(tmp_path):
     mod = cp.RawModule(path=str(path))
     h1, h2, y = _run(mod.get_function('test_multiply'), np.float32, seed=6)
     assert np.array_equal(y, h1 * h2)
+
+
+GRID_SYNC_SRC = r'''
+#include <hip/hip_cooperative_groups.h>
+extern "C" __global__
+void test_grid_sync(const float* x1, const float* x2, float* y, int n) {
+    namespace cg = cooperative_groups;
+    cg::grid_group grid = cg::this_grid();
+    int size = gridDim.x * blockDim.x;
+    int tid = blockDim.x * blockIdx.x + threadIdx.x;
+    for (int i = tid; i < n; i += size) y[i] = x1[i];
+    cg::sync(grid);
+    for (int i = n - 1 - tid; i >= 0; i -= size) y[i] += x2[i];
+}
+
+// every workgroup adds up its share; after the grid-wide barrier workgroup 0
+// adds up the shares of all workgroups
+extern "C" __global__
+void grid_sum(const int* x, long long* shares, long long* total, int n) {
+    namespace cg = cooperative_groups;
+    __shared__ long long sm[256];
+    long long s = 0;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) s += x[i];
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = blockDim.x / 2; w > 0; w >>= 1) {
+        if (threadIdx.x < w) sm[threadIdx.x] += sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) shares[blockIdx.x] = sm[0];
+    cg::this_grid().sync();
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        long long t = 0;
+        for (int b = 0; b < gridDim.x; ++b) t += shares[b];
+        total[0] = t;
+    }
+}
+'''
+
+
+@pytest.mark.parametrize('n,block', [(64, 64), (257, 128), (1024, 256)])
+def test_grid_sync_rawkernel_and_rawmodule(n, block):
+    """A grid-wide barrier inside a cooperatively launched kernel (reference:
+    tests/cupy_tests/core_tests/test_raw.py:1364-1397, skipped there on HIP)."""
+    x1 = np.arange(n * n, dtype=np.float32).reshape(n, n)
+    x2 = np.ones((n, n), np.float32)
+    grid = min((n * n + block - 1) // block, 512)
+    ker = cp.RawKernel(GRID_SYNC_SRC, 'test_grid_sync', enable_cooperative_groups=True)
+    y = cp.zeros((n, n), np.float32)
+    ker((grid,), (block,), (cp.asarray(x1), cp.asarray(x2), y, n * n))
+    assert np.array_equal(y.get(), x1 + x2)
+    mod = cp.RawModule(code=GRID_SYNC_SRC, enable_cooperative_groups=True)
+    y = cp.zeros((n, n), np.float32)
+    mod.get_function('test_grid_sync')((grid,), (block,), (cp.asarray(x1), cp.asarray(x2), y, n * n))
+    assert np.array_equal(y.get(), x1 + x2)
+
+
+def test_sum_across_workgroups_after_a_grid_wide_barrier():
+    rng = np.random.default_rng(21)
+    h = rng.integers(-1000, 1000, (1 << 22) + 77).astype(np.int32)
+    mod = cp.RawModule(code=GRID_SYNC_SRC, enable_cooperative_groups=True)
+    ker = mod.get_function('grid_sum')
+    shares = cp.zeros((512,), np.int64)
+    total = cp.zeros((1,), np.int64)
+    ker((512,), (256,), (cp.asarray(h), shares, total, h.size))
+    assert int(total.get()[0]) == int(h.sum(dtype=np.int64))
+    # a grid the device cannot hold at once is refused, and nothing is left broken
+    with pytest.raises(cp.cuda.runtime.HIPError if hasattr(cp.cuda.runtime, 'HIPError') else Exception,
+                       match='CooperativeLaunchTooLarge'):
+        ker((1 << 16,), (256,), (cp.asarray(h), cp.zeros((1 << 16,), np.int64), total, h.size))
+    total.fill(0)
+    ker((256,), (256,), (cp.asarray(h), shares, total, h.size))
+    assert int(total.get()[0]) == int(h.sum(dtype=np.int64))
+
+
+LDS_SRC = r'''
+extern "C" __global__ void reverse_through_lds(const int* x, int* y, int n) {
+    extern __shared__ int buf[];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) buf[i] = x[i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) y[i] = buf[n - 1 - i];
+}
+'''
+
+
+def test_more_than_64_kib_of_dynamic_lds_after_the_setter():
+    """(reference: cupy/_core/raw.pyx:226-255; the setter is a stub on the
+    reference's HIP build)"""
+    ker = cp.RawKernel(LDS_SRC, 'reverse_through_lds')
+    nbytes = 96 * 1024
+    ker.max_dynamic_shared_size_bytes = nbytes
+    assert ker.max_dynamic_shared_size_bytes >= nbytes
+    ker.preferred_shared_memory_carveout = 100      # a hint; accepted
+    n = nbytes // 4
+    h = np.arange(n, dtype=np.int32)
+    y = cp.zeros((n,), np.int32)
+    ker((1,), (1024,), (cp.asarray(h), y, n), shared_mem=nbytes)
+    assert np.array_equal(y.get(), h[::-1])
+    # beyond the LDS of a compute unit the launch is refused
+    with pytest.raises(Exception):
+        ker((1,), (1024,), (cp.asarray(h), y, n), shared_mem=1 << 20)
+        cp.cuda.Device().synchronize()

@@ -226,3 +226,34 @@ def test_threads_with_their_own_streams():
     assert all(results)
     # one compiled kernel per input type tuple, however many threads raced for it
     assert len(kernel._cached_codes) == 1
+
+
+def test_work_on_the_per_thread_default_stream():
+    """Kernels, split reductions and scans on ``Stream.ptds`` from two threads
+    (reference: cupy/cuda/stream.pyx:494-505; the pool keeps the threads'
+    blocks apart, cupy/cuda/memory.pyx:877-889)."""
+    import threading
+    from cupy_amd.cuda import stream as stream_module
+    rng = np.random.default_rng(31)
+    h = rng.integers(-50, 50, 1 << 21).astype(np.int32)
+    results = {}
+
+    def job(key):
+        with cp.cuda.Device(0):
+            with cp.cuda.Stream.ptds as s:
+                assert cp.cuda.get_current_stream().ptr == stream_module.STREAM_PER_THREAD
+                a = cp.asarray(h)
+                total = a.sum()
+                running = (a * 2).cumsum()
+                ptr = a.data.ptr
+                s.synchronize()
+                results[key] = (int(total), running.get(), ptr)
+
+    job('main')
+    t = threading.Thread(target=job, args=('sub',))
+    t.start()
+    t.join()
+    for key in ('main', 'sub'):
+        total, running, _ = results[key]
+        assert total == int(h.sum())
+        assert np.array_equal(running, (h * 2).cumsum())

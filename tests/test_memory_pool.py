@@ -533,3 +533,102 @@ def test_limit_holds_for_requests_side_by_side(monkeypatch):
     _run_with_deadline(scenario)
     assert len(got) == 2 and len(refused) == 2
     assert pool.total_bytes() <= unit * 10
+
+
+# ---- per-thread default stream (reference: cupy/cuda/memory.pyx:877-889 and
+# tests/cupy_tests/cuda_tests/test_memory.py:866-926) ---------------------------
+
+def _reuse_between_threads(pool, stream_main, stream_sub):
+    """A block allocated and freed under ``stream_main`` in this thread, then
+    one of the same size under ``stream_sub`` in another thread: both
+    addresses."""
+    seen = {}
+
+    def job(key, s):
+        with s:
+            p = pool.malloc(unit * 4)
+            seen[key] = p.ptr
+            del p
+
+    job('main', stream_main)
+    t = threading.Thread(target=job, args=('sub', stream_sub), daemon=True)
+    t.start()
+    t.join()
+    return seen['main'], seen['sub']
+
+
+def test_reuse_between_threads_on_the_null_stream(pool):
+    main_ptr, sub_ptr = _reuse_between_threads(pool, FakeStream(0), FakeStream(0))
+    assert main_ptr == sub_ptr
+
+
+def test_reuse_between_threads_on_the_same_stream(pool):
+    main_ptr, sub_ptr = _reuse_between_threads(pool, FakeStream(0x77), FakeStream(0x77))
+    assert main_ptr == sub_ptr
+
+
+def test_no_reuse_between_threads_on_different_streams(pool):
+    main_ptr, sub_ptr = _reuse_between_threads(pool, FakeStream(0x77), FakeStream(0x78))
+    assert main_ptr != sub_ptr
+
+
+def test_no_reuse_between_threads_on_the_per_thread_default_stream(pool):
+    """One handle, another stream in every thread: the arenas are kept apart
+    by thread."""
+    ptds = stream_module.Stream.ptds
+    assert ptds.ptr == stream_module.STREAM_PER_THREAD
+    main_ptr, sub_ptr = _reuse_between_threads(pool, ptds, ptds)
+    assert main_ptr != sub_ptr
+    # ... and the same thread does get its block back
+    with ptds:
+        p = pool.malloc(unit * 4)
+        assert p.ptr == main_ptr
+        del p
+        # free_all_blocks(stream=Stream.ptds) means this thread's arena
+        assert pool.n_free_blocks() == 2
+        pool.free_all_blocks(stream=ptds)
+        assert pool.n_free_blocks() == 1
+
+
+def test_thread_identifiers_of_the_per_thread_stream():
+    ident = stream_module.stream_identifier
+    assert ident(0) == 0 and ident(0x1234) == 0x1234
+    mine = ident(stream_module.STREAM_PER_THREAD)
+    assert mine == ident(stream_module.STREAM_PER_THREAD) and mine >> 63 == 1
+    other = []
+    t = threading.Thread(target=lambda: other.append(ident(stream_module.STREAM_PER_THREAD)))
+    t.start()
+    t.join()
+    assert other[0] != mine and other[0] >> 63 == 1
+
+
+def test_default_stream_follows_the_environment_switch(monkeypatch):
+    """CUPY_CUDA_PER_THREAD_DEFAULT_STREAM=1 makes the per-thread stream the
+    one a thread works on until it chooses another (reference:
+    cupy_backends/cuda/stream.pyx:33-44,84-94; cupy/cuda/stream.pyx:74-75)."""
+    S = stream_module.Stream
+    assert stream_module.get_current_stream() is S.null
+    assert stream_module.get_default_stream_ptr() == stream_module.STREAM_LEGACY
+    monkeypatch.setattr(stream_module, '_ptds', True)
+    assert stream_module.is_ptds_enabled()
+    assert stream_module.get_current_stream_ptr() == stream_module.STREAM_PER_THREAD
+    assert stream_module.get_current_stream() is S.ptds
+    assert stream_module.get_default_stream_ptr() == stream_module.STREAM_PER_THREAD
+    with FakeStream(0x99):
+        assert stream_module.get_current_stream_ptr() == 0x99
+    assert stream_module.get_current_stream_ptr() == stream_module.STREAM_PER_THREAD
+
+
+def test_stream_singletons_compare_like_the_reference():
+    """(tests/cupy_tests/cuda_tests/test_stream.py:32-51)"""
+    S = stream_module.Stream
+    assert S(null=True) == S.null and S(ptds=True) == S.ptds
+    assert S(ptds=True) == S(ptds=True) and S(ptds=True) != S(null=True)
+    assert hash(S(ptds=True)) == hash(S.ptds)
+    s = S(ptds=True)
+    s.__del__()                      # never destroyed
+    assert s.ptr == stream_module.STREAM_PER_THREAD
+    with S.ptds:
+        assert stream_module.get_current_stream() is S.ptds
+        assert stream_module.get_current_stream_ptr() == stream_module.STREAM_PER_THREAD
+    assert stream_module.get_current_stream() is S.null

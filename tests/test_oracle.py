@@ -129,9 +129,27 @@ def test_integer_sums_are_exact_and_wrap(small_configs):
 
 
 def test_reference_block_geometry(golden):
+    """A RESTATEMENT check, not a pin: the expected triples in the fixture were
+    worked out by hand from the very formula the C function restates
+    (cupy/_core/_reduction.pyx:239-253), so agreement only shows that the C
+    text and the hand evaluation read the formula the same way.  What the
+    formula itself guarantees is checked below for a range of sizes: the
+    stride is the largest power of two not above max(contiguous capped at 32,
+    256 / elements per output), it never exceeds the block, and the blocks
+    cover every output exactly once."""
     for case in golden['block_specs']:
         got = c_oracle.get_block_specs(case['in_size'], case['out_size'], case['contiguous'])
         assert list(got) == case['expect']
+    for out_size in (1, 2, 3, 31, 32, 33, 255, 256, 257, 4096, 16384, 1 << 20):
+        for per_out in (1, 2, 7, 8, 100, 256, 257, 4096, 1 << 14):
+            for contiguous in (1, 2, 5, 16, 32, 33, 1000, out_size):
+                block, stride, blocks = c_oracle.get_block_specs(
+                    out_size * per_out, out_size, contiguous)
+                bound = max(min(contiguous, 32), 256 // per_out)
+                assert block == 256
+                assert stride & (stride - 1) == 0 and stride <= max(1, bound) < 2 * stride
+                assert stride <= block
+                assert (blocks - 1) * stride < out_size <= blocks * stride
 
 
 def test_fused_pipeline_rounding():
