@@ -1133,7 +1133,7 @@ _CHAIN_WAVES = _BLOCK // _WAVE
 _CHAIN_HEADER_WORDS = 64            # the ticket counter, padded to 256 bytes
 
 
-def _emit_chain(in_t, out_t, op, skip_nan, vec, trips, idx64, stream, ragged, parts=2):
+def _emit_chain(in_t, out_t, op, skip_nan, vec, trips, idx64, stream, ragged, parts=2, waves=_CHAIN_WAVES):
     """One-pass scan of long rows: a workgroup per tile of 256 x VEC x TRIPS
     elements scans its tile in registers, publishes the tile's total and adds
     up the totals published by the tiles before it: the input is read once and
@@ -1259,9 +1259,8 @@ __device__ __forceinline__ _acc_t _await_fold(_slot_t* slots, const ptrdiff_t fi
   return s;
 }
 
-extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_clear(
-    unsigned* desc, const unsigned words) {
-  for (unsigned i = blockIdx.x * %(block)d + threadIdx.x; i < words; i += gridDim.x * %(block)d)
+extern "C" __global__ void cupy_scan_chain_clear(unsigned* desc, const unsigned words) {
+  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x)
     desc[i] = 0u;
 }
 
@@ -1455,19 +1454,20 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain(
   }
 }
 ''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident, start=_start_text(op, acc_t),
-           vec=vec, trips=trips, conv=conv, block=_BLOCK, waves=_CHAIN_WAVES,
+           vec=vec, trips=trips, conv=conv, block=waves * _WAVE, waves=waves,
            header=_CHAIN_HEADER_WORDS, parts=parts, sleep=_tuning.get('scan_chain_sleep'),
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
            ragged=1 if ragged else 0)
 
 
-def _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream, ragged, parts):
+def _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream, ragged, parts,
+                  waves=_CHAIN_WAVES):
     key = ('chain', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
-           trips, idx64, stream, ragged, parts, _tuning.get('scan_chain_sleep'))
+           trips, idx64, stream, ragged, parts, waves, _tuning.get('scan_chain_sleep'))
     mod = _memo.get(key)
     if mod is None:
         src = _emit_chain(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
-                          vec, trips, idx64, stream, ragged, parts)
+                          vec, trips, idx64, stream, ragged, parts, waves)
         mod = compiler.compile_with_cache(src)
         with _lock:
             mod = _memo.setdefault(key, mod)
@@ -1645,9 +1645,8 @@ __device__ __forceinline__ _acc_t _round_scan(
   return cupy::shfl_idx<64>(incl, (SEG - 1) * INNER + col);
 }
 
-extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_clear(
-    unsigned* desc, const unsigned words) {
-  for (unsigned i = blockIdx.x * %(block)d + threadIdx.x; i < words; i += gridDim.x * %(block)d)
+extern "C" __global__ void cupy_scan_chain_clear(unsigned* desc, const unsigned words) {
+  for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x)
     desc[i] = 0u;
 }
 
@@ -2210,6 +2209,7 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
     dev_id, fault = ready
     in_dtype, out_dtype = src.dtype, dst.dtype
     trips = 4
+    waves, wide = _tuning.get('scan_chain_waves'), 1
     parts = _tuning.get('scan_chain_parts')
     if not parts:
         # Bigger tiles mean fewer waits per byte but fewer workgroups per CU;
@@ -2220,6 +2220,10 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
         parts = 8 if nbytes >= 64 << 20 else 4 if nbytes >= 16 << 20 else 2
         if max(in_dtype.itemsize, _acc_dtype(out_dtype).itemsize) > 4 or inner > 1:
             parts = min(parts, 4)
+            if inner == 1 and parts == 4 and waves >= 2 * _CHAIN_WAVES:
+                # (2^25 float64 in one row: 4 waves x 4 parts 122 us, 8 x 2 114,
+                # 8 x 3 110, 16 x 2 112)
+                parts = 6
         if 1 < inner <= 6:
             # (2^26 float32 as (n,3): 115 us with 2 parts, 123 with 4; as (n,5)
             # 133 / 138; as (n,12) 131 / 113; as (n,16) 128 / 120)
@@ -2227,6 +2231,7 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
     if inner > 1:
         vec = max(1, 16 // max(in_dtype.itemsize, out_dtype.itemsize))
         tile = _CHAIN_WAVES * parts * _tile_geometry(inner, vec, trips)[0]     # rows
+        waves = _CHAIN_WAVES
     else:
         # No tile longer than a row; and rows of few tiles want small ones: a
         # tile then waits for few others, and there are many rows to go on
@@ -2238,10 +2243,16 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
             parts = min(parts, 1 if base_tiles <= 16 else 2 if base_tiles <= 64
                         else 4 if base_tiles <= 128 else 8)
         parts = max(1, min(parts, base_tiles))
-        tile = _BLOCK * vec * trips * parts
+        # the same tile from more waves with fewer vectors per lane
+        while (_CHAIN_WAVES * wide < waves and parts % 2 == 0
+               and parts > _tuning.get('scan_chain_min_parts')):
+            parts //= 2
+            wide *= 2
+        waves = _CHAIN_WAVES * wide
+        tile = waves * _WAVE * vec * trips * parts
     tiles_per_row = (n + tile - 1) // tile
     n_tiles = n_rows * tiles_per_row
-    if n_tiles < 2 or n_tiles * _BLOCK > 0xffffffff or n < _BLOCK * vec * trips:
+    if n_tiles < 2 or n_tiles * max(_BLOCK, waves * _WAVE) > 0xffffffff or n < _BLOCK * vec * trips:
         return False
     if (inner == 1 and tiles_per_row * tile > _tuning.get('scan_chain_max_waste') * n
             and n_rows >= _device.get_compute_units(dev_id) * _tuning.get('scan_waves_per_cu')):
@@ -2265,7 +2276,7 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
         name = 'cupy_scan_chain_tile'
     else:
         mod = _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream,
-                            n % vec != 0, parts)
+                            n % vec != 0, parts, waves)
         name = 'cupy_scan_chain'
     desc, epoch = _chain_slots(dev_id, stream_ptr, desc_words, mod)
     ic = 'q' if idx64 else 'i'
@@ -2273,7 +2284,7 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
                        n_rows, n, tiles_per_row, group_tiles, groups_per_row, epoch,
                        _tuning.get('scan_chain_spin_limit'), fault)
     mod.get_function(name).launch_packed(
-        (n_tiles, 1, 1), (_BLOCK, 1, 1), blob, 0, stream_ptr)
+        (n_tiles, 1, 1), (waves * _WAVE if inner == 1 else _BLOCK, 1, 1), blob, 0, stream_ptr)
     return True
 
 

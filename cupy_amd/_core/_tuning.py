@@ -138,6 +138,16 @@ _params = {
     # the wave, 89 us)
     'scan_chain_min_row_bytes': 16384,
     'scan_chain': True,         # a few long rows: one pass, tiles chained through published totals
+    # ... with this many waves per tile, each lane keeping fewer vectors for the
+    # same tile (2^26 float32 in one row, 128 KiB tiles: 4 waves x 8 parts 102 us,
+    # 8 x 4 98, 16 x 2 105; 64 rows of 2^20: 101 / 98 / 109).  A plain copy made
+    # the same way -- a workgroup loads a whole tile into registers, then
+    # stores it -- reaches 79 % of peak with tiles of 32 KiB, 75 % with 48 KiB
+    # and 70 % with 64 to 128 KiB, whatever the order and pacing of the
+    # accesses inside the tile, against 81 % for a streaming copy: tiles large
+    # enough to make the look-back cheap cost about ten points by themselves
+    'scan_chain_waves': 8,
+    'scan_chain_min_parts': 1,  # ... each lane keeping at least this many times 4 vectors
     'scan_chain_parts': 0,      # ... a wave holds this many times 4 vectors per lane of its tile
                                 # (0: by the size of the input)
     'scan_chain_sleep': 8,      # ... and pauses this many times 64 clocks between two polls

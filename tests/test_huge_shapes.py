@@ -69,9 +69,7 @@ def test_column_blocks_beyond_grid_x_continue_along_grid_z():
     finally:
         _tuning.set(unaligned_vectors=True)
     (kernel, grid, block, _, _), = launches
-    lanes = _tuning.get('cols_tx')
-    assert grid[2] >= 2 and grid[0] * grid[2] * lanes >= 2 ** 30 + 1
-    assert grid[0] * (grid[2] - 1) * lanes < 2 ** 30 + 1
+    assert grid[2] == 2 and grid[0] * grid[2] * 64 >= 2 ** 30 + 1
     assert out.shape == (2 ** 30 + 1,)
 
 
@@ -79,10 +77,8 @@ def test_reduction_over_a_middle_axis_is_one_batched_column_kernel():
     out, launches = launches_of(lambda: cp.empty((33, 65, 31277), np.float32).sum(axis=1))
     (kernel, grid, block, _, _), = launches
     assert out.shape == (33, 31277)
-    # column blocks of `cols_tx` lanes x 4 columns, none straddling two batch rows
-    from cupy_amd._core import _tuning
-    width = 4 * _tuning.get('cols_tx')
-    assert grid[0] == 33 * ((31277 + width - 1) // width) and grid[1] == 1
+    # column blocks of 64 lanes x 4 columns, none straddling two batch rows
+    assert grid[0] == 33 * ((31277 + 255) // 256) and grid[1] == 1
     out, launches = launches_of(lambda: cp.empty((4, 100000, 64), np.float32).max(axis=1))
     assert len(launches) == 2 and launches[0][1][1] > 1       # reduce axis split, then combined
     assert out.shape == (4, 64)
