@@ -32,6 +32,58 @@ def get_default_memory_pool():
     """The pool that backs every ``ndarray`` allocation by default."""
     return _default_memory_pool
 
+
+def _runtime_records():
+    """(label, value) pairs describing the installation, in display order."""
+    import os
+    import platform
+    import shutil
+    from cupy_amd import _dryrun
+    from cupy_amd.cuda import compiler as _compiler
+    from cupy_amd.cuda import _compiler_cache
+    records = [
+        ('OS', platform.platform()),
+        ('Python Version', platform.python_version()),
+        ('CuPy Version', __version__),
+        ('CuPy Platform', 'AMD ROCm (MI355X-native build, gfx950)'),
+        ('NumPy Version', _numpy.__version__),
+        ('ROCm Include Dir', _compiler.rocm_include_dir()),
+        ('HIPCC PATH', shutil.which('hipcc')),
+        ('Runtime Library', _rt.LIB_PATH),
+        ('Kernel Cache Dir', _compiler_cache.get_cache_dir()),
+    ]
+    if _dryrun.enabled():
+        records.append(('Mode', 'compile check only (CUPY_AMD_DRYRUN): nothing runs on a device'))
+        return records
+    records += [
+        ('HIP Driver Version', cuda.runtime.driverGetVersion()),
+        ('HIP Runtime Version', cuda.runtime.runtimeGetVersion()),
+        ('hipRTC Version', '%d.%d' % _compiler.get_rtc_version()),
+        ('Per-Thread Default Stream', cuda.stream.is_ptds_enabled()),
+    ]
+    for device_id in range(cuda.runtime.getDeviceCount()):
+        props = cuda.device.get_device_properties(device_id)
+        label = 'Device %d ' % device_id
+        records += [
+            (label + 'Name', props['name']),
+            (label + 'Arch', props['arch']),
+            (label + 'Compute Units', props['compute_units']),
+            (label + 'Memory', '%.1f GiB' % (props['total_global_mem'] / 2.0 ** 30)),
+        ]
+    return records
+
+
+def show_config(*, _full=False):
+    """Prints the current runtime configuration to standard output
+    (reference: cupy/__init__.py:942-946, cupyx/_runtime.py:309-420)."""
+    import builtins
+    import sys
+    records = _runtime_records()
+    width = builtins.max(len(label) for label, _ in records) + 1
+    sys.stdout.write(''.join('%s: %s\n' % (label.ljust(width), value)
+                             for label, value in records))
+    sys.stdout.flush()
+
 from cupy_amd._core._reduction import (  # noqa
     ReductionKernel, create_reduction_func)
 from cupy_amd._core.fusion import fuse  # noqa

@@ -60,8 +60,57 @@ class Code:
                     name, ', '.join(sig), ' '.join(body), loop.routine))
         return name
 
+    def divide_by_row_value(self):
+        """Name of the float32 division by a value that many elements share,
+        given the value's reciprocal (defined on first use)."""
+        name = '_fz_divide_by_shared'
+        if name not in self._functions.values():
+            self._functions[name] = name
+            self.definitions.append(_DIVIDE_BY_SHARED % name)
+        return name
+
     def text(self):
         return '\n'.join(self.preambles) + '\n' + ''.join(self.definitions)
+
+
+# x / d for a divisor that a whole row shares, from r = 1 / d (correctly rounded,
+# computed once per row): the product x * r is within an ulp or so of the
+# quotient; its residual x - q * d is exact in one fused multiply-add, and adding
+# residual * r gives the correctly rounded quotient except in rare cases that
+# end one ulp away (Markstein's correction step).  Six instructions against the
+# ten to thirteen of the division's full expansion.  Where that reasoning does not hold
+# the division itself is carried out: a quotient that is infinite or NaN (an
+# infinite or NaN dividend, overflow), and every quotient of a row whose
+# reciprocal is zero, subnormal, infinite or NaN -- the caller hands NaN in for
+# such a reciprocal (`shared_reciprocal`), which makes every quotient NaN here.
+_DIVIDE_BY_SHARED = '''__device__ __forceinline__ void %s(
+    const float x, const float d, const float r, float& out) {
+  const float p = x * r;
+  const float e = __builtin_fmaf(-p, d, x);
+  float q = __builtin_fmaf(e, r, p);
+  // (a zero quotient takes its sign from the product: the correction step
+  // turns -0 into +0)
+  q = (q == 0.0f) ? p : q;
+  if (__builtin_expect(__builtin_fabsf(q) < __builtin_inff(), 1)) {
+    out = q;
+  } else {
+    // (the empty statement keeps the division on this side of the branch: as a
+    // plain conditional expression it is evaluated for every element)
+    float dd = d;
+    asm volatile("" : "+v"(dd));
+    out = x / dd;
+  }
+}
+'''
+
+# the reciprocal such a division takes: NaN unless it is a normal number well
+# inside the range (so that neither it nor the products with it lose bits)
+SHARED_RECIPROCAL = '''__device__ __forceinline__ float shared_reciprocal(const float d) {
+  const float r = 1.0f / d;
+  const float a = __builtin_fabsf(r);
+  return (a > 1.0e-30f && a < 1.0e30f) ? r : __builtin_nanf("");
+}
+'''
 
 
 def _name(v):
@@ -82,9 +131,38 @@ def _read(v, as_dtype):
     return 'static_cast<%s>(%s)' % (get_typename(as_dtype), _name(v))
 
 
-def straight_line(code, targets, leaves):
+def _is_float32_divide(call):
+    f32 = numpy.dtype('float32')
+    return (call.ufunc.name == 'cupy_true_divide' and len(call.inputs) == 2
+            and all(numpy.dtype(t) == f32 for t in tuple(call.in_dtypes) + tuple(call.out_dtypes)))
+
+
+def shared_divisors(targets, leaves, shared):
+    """Orders of the leaves among ``shared`` (values that many elements have
+    in common) by which a float32 value is divided on the way to ``targets``."""
+    given = set(v.order for v in leaves)
+    found = []
+    stack = list(targets)
+    seen = set()
+    while stack:
+        v = stack.pop()
+        if v.order in seen or v.order in given or v.kind != 'apply':
+            continue
+        seen.add(v.order)
+        call = v.call
+        d = call.inputs[1] if _is_float32_divide(call) else None
+        if d is not None and d.order in shared and d.order in given and d.order not in found \
+                and d.dtype == numpy.dtype('float32'):
+            found.append(d.order)
+        stack.extend(call.inputs)
+    return sorted(found)
+
+
+def straight_line(code, targets, leaves, reciprocals=None):
     """Statements computing ``targets`` from ``leaves`` (Values whose variables
-    are taken as given), in the order the function made the calls."""
+    are taken as given), in the order the function made the calls.
+    ``reciprocals``: order of a float32 leaf -> name of a variable that holds
+    its reciprocal; divisions by such a leaf use it."""
     given = set(v.order for v in leaves)
     needed = {}
     stack = list(targets)
@@ -115,6 +193,9 @@ def straight_line(code, targets, leaves):
                 outs.append(_name(mate))
                 lines.append('%s %s;' % (get_typename(t), _name(mate)))
         ins = [_read(v, t) for v, t in zip(call.inputs, call.in_dtypes)]
+        if reciprocals and _is_float32_divide(call) and call.inputs[1].order in reciprocals:
+            fn = code.divide_by_row_value()
+            ins.append(reciprocals[call.inputs[1].order])
         lines.append('%s(%s);' % (fn, ', '.join(ins + outs)))
     return lines
 
@@ -153,12 +234,19 @@ def elementwise_kernel(name, leaves, targets, stores=()):
         return_tuple=len(targets) != 1, no_return=not targets)
 
 
-def describe_elementwise(leaves, targets):
+def describe_elementwise(leaves, targets, shared=()):
     """The same computation as a device function
-    ``void elementwise(leaf values..., target references...)``."""
+    ``void elementwise(leaf values..., reciprocals..., target references...)``.
+    ``shared``: orders of leaves whose value many elements have in common (one
+    per row); for those among them that float32 values are divided by, the
+    function takes the reciprocal as one more argument each (``reciprocals``
+    of the result lists their orders) and divides through it."""
     code = Code()
-    lines = straight_line(code, targets, leaves)
+    divisors = shared_divisors(targets, leaves, set(shared)) if shared else []
+    lines = straight_line(code, targets, leaves,
+                          dict((o, '_rcp%d' % o) for o in divisors))
     sig = ['%s %s' % (get_typename(v.dtype), _name(v)) for v in leaves]
+    sig += ['float _rcp%d' % o for o in divisors]
     sig += ['%s& o%d' % (get_typename(t.dtype), i) for i, t in enumerate(targets)]
     for i, t in enumerate(targets):
         lines.append('o%d = %s;' % (i, _read(t, t.dtype)))
@@ -166,7 +254,7 @@ def describe_elementwise(leaves, targets):
         ', '.join(sig), '\n'.join(lines))
     return dict(kind='elementwise', preambles=code.preambles,
                 functions=''.join(code.definitions) + function,
-                out_dtypes=[t.dtype for t in targets])
+                out_dtypes=[t.dtype for t in targets], reciprocals=divisors)
 
 
 # ---------------------------------------------------------------------------------------

@@ -303,7 +303,13 @@ def _build(nodes, pieces, returns, single, args, name):
         if p.reduce is not None:
             described.append(_fusion_emit.describe_reduction(p.reduce, p.leaves))
         else:
-            described.append(_fusion_emit.describe_elementwise(p.leaves, p.targets))
+            # values one row shares: a division by such a value goes through
+            # its reciprocal, taken once per row
+            shared = [l.order for l in p.leaves if kinds[l.order] in ('row', 'rowk', 'uni')]
+            if not _tuning.get('fused_rows_reciprocal') or not any(
+                    kinds[t.order] == 'full' for t in p.targets):
+                shared = ()
+            described.append(_fusion_emit.describe_elementwise(p.leaves, p.targets, shared))
 
     # ---- kernel parameters ---------------------------------------------------------------
     params = []
@@ -380,6 +386,8 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
 #pragma unroll
   for (int k = 0; k < VEC; ++k) if (col + k < NCOLS) row[col + k] = v.v[k];
 }''')
+    if any(d.get('reciprocals') for d in described):
+        src.append(_fusion_emit.SHARED_RECIPROCAL)
     for k, (p, d) in enumerate(zip(pieces, described)):
         src.append('namespace piece%d {' % k)
         src.append(d['functions'])
@@ -457,6 +465,10 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
     kept_names = set()
     for k, (p, d) in enumerate(zip(pieces, described)):
         call_args = [operand(l) for l in p.leaves]
+        for order in d.get('reciprocals', ()):
+            (leaf,) = [l for l in p.leaves if l.order == order]
+            src.append('    const float _rcp%d_%d = shared_reciprocal(%s);' % (k, order, operand(leaf)))
+            call_args.append('_rcp%d_%d' % (k, order))
         if getattr(p, 'keep', False):
             (t,) = p.targets
             src.append('    cupy::Vec<%s, VEC> _m%d[PER_LANE];' % (

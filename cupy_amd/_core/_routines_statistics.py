@@ -210,7 +210,14 @@ template <bool kNan, typename T, bool kMax>
 __device__ __forceinline__ mm_val<T, kMax> mm_pick(const mm_val<T, kMax>& a,
                                                    const mm_val<T, kMax>& b) {
   bool take_b = kMax ? (b.v > a.v) : (b.v < a.v);
-  if (kNan) take_b = (take_b | (b.v != b.v)) & !(a.v != a.v);
+  if (kNan) {
+    // NaN wins and stays.  For real floating types "b beats a, or b is NaN"
+    // is one comparison: the negation of an ordered one is true for NaN
+    // (and for NaN in a, which the second test takes out again).
+    if (_mm_is_float<T>::value) take_b = kMax ? !(b.v <= a.v) : !(b.v >= a.v);
+    else take_b = take_b | (b.v != b.v);
+    take_b = take_b & !(a.v != a.v);
+  }
   mm_val<T, kMax> r;
   r.v = take_b ? b.v : a.v;
   return r;

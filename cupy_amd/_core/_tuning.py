@@ -163,6 +163,9 @@ _params = {
     # with a wave against 68 % with a workgroup.  Requesting the next row before
     # the current one is worked on did not help: 62 % against 76 % on rows of 8192)
     'fused_rows_wave_words': 32,
+    # a float32 division by a value the whole row shares (the sum of a softmax)
+    # goes through the value's reciprocal and one correction step
+    'fused_rows_reciprocal': True,
     # Grid cap of that kernel, in workgroups per CU (softmax 16384x4096: 94.5 us
     # with 16, 86.0 with 64 or more; rows of 1024: 89.9 -> 85.1; layer
     # normalisation over rows of 100: 110 -> 96)

@@ -8,6 +8,8 @@ consumes is here (cupy/_core/core.pyx:134-301 construction and flags,
 import ctypes
 import operator
 
+builtins_type = type
+
 import numpy
 
 from cupy_amd import _dryrun
@@ -272,11 +274,42 @@ class ndarray:
         axes[a], axes[b] = axes[b], axes[a]
         return self.transpose(axes)
 
+    def _index_order(self, order, allow_k=False):
+        """'C' or 'F' (or 'K') for an ``order=`` argument; 'A' means Fortran
+        order exactly for arrays stored that way and not in C order."""
+        letter = 'C' if order is None else str(order).upper()
+        if letter == 'A':
+            letter = 'F' if (self._f_contiguous and not self._c_contiguous) else 'C'
+        if letter not in ('C', 'F') and not (allow_k and letter == 'K'):
+            raise ValueError('order not understood: %r' % (order,))
+        return letter
+
+    def _memory_order_axes(self):
+        """Axes from the one with the largest step in memory to the one with
+        the smallest, as NumPy's iterator orders them for ``order='K'``: an
+        axis moves in front of those with smaller steps; axes without a step
+        (broadcast) stay where they are met, and ties keep the axis order."""
+        steps = [abs(s) for s in self._strides]
+        axes = []
+        for axis in reversed(range(len(steps))):
+            pos = 0
+            if steps[axis]:
+                for k, other in enumerate(axes):
+                    if steps[other] == 0:
+                        continue
+                    if steps[other] <= steps[axis]:
+                        break
+                    pos = k + 1
+            axes.insert(pos, axis)
+        return axes
+
     def reshape(self, *shape, order='C'):
         if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
             shape = tuple(shape[0])
-        if order not in ('C', 'c', None):
-            raise NotImplementedError('reshape supports order=\'C\' only')
+        if self._index_order(order) == 'F':
+            # elements taken and placed with the first index changing fastest:
+            # the C-order reshape of the transposed array, transposed back
+            return self.transpose().reshape(*tuple(shape)[::-1]).transpose()
         shape = internal.infer_unknown_dimension(
             [operator.index(s) for s in shape], self.size)
         if internal.prod(shape) != self.size:
@@ -292,11 +325,26 @@ class ndarray:
         return self._view(shape, strides)
 
     def ravel(self, order='C'):
+        """1-d array of the elements in C, Fortran ('F'), stored ('A') or
+        memory ('K') order; a view where memory allows (reference:
+        cupy/_core/_routines_manipulation.pyx:190-208)."""
+        letter = self._index_order(order, allow_k=True)
+        if letter == 'F':
+            return self.transpose().reshape(-1)
+        if letter == 'K':
+            return self.transpose(self._memory_order_axes()).reshape(-1)
         return self.reshape(-1)
 
-    def flatten(self):
-        return self.copy().reshape(-1) if self._c_contiguous else \
-            _ascontiguous(self).reshape(-1)
+    def flatten(self, order='C'):
+        """Like ``ravel`` but always a copy."""
+        letter = self._index_order(order, allow_k=True)
+        src = self
+        if letter == 'F':
+            src = self.transpose()
+        elif letter == 'K':
+            src = self.transpose(self._memory_order_axes())
+        return src.copy().reshape(-1) if src._c_contiguous else \
+            _ascontiguous(src).reshape(-1)
 
     def squeeze(self, axis=None):
         nd = len(self._shape)
@@ -313,8 +361,18 @@ class ndarray:
                           tuple(self._strides[i] for i in keep))
 
     def view(self, dtype=None, type=None):
-        if type is not None:
-            raise NotImplementedError('view(type=...) is not supported')
+        """View of the same memory as another dtype and / or another array
+        class (reference: cupy/_core/core.pyx:926-990)."""
+        cls = type
+        if isinstance(dtype, builtins_type) and issubclass(dtype, ndarray):
+            if cls is not None:
+                raise ValueError('Cannot specify output type twice.')
+            cls, dtype = dtype, None
+        if cls is not None:
+            if not isinstance(cls, builtins_type) or not issubclass(cls, ndarray):
+                raise ValueError('Type must be a sub-type of ndarray type')
+            plain = self.view(dtype)
+            return plain if builtins_type(plain) is cls else plain._retype(cls, self)
         if dtype is None or _dtype.get_dtype(dtype) == self.dtype:
             return self._view(self._shape, self._strides)
         dt = _dtype.get_dtype(dtype)
@@ -399,16 +457,29 @@ class ndarray:
         """Copies the array to host memory and returns a ``numpy.ndarray``."""
         if _dryrun.enabled():
             _dryrun.forbid('ndarray.get()')
-        if order not in ('C', 'c'):
-            raise NotImplementedError('get() supports order=\'C\' only')
+        if out is None:
+            letter = self._index_order(order)
+        else:
+            if not isinstance(out, numpy.ndarray):
+                raise TypeError('Only numpy.ndarray can be obtained from cupy.ndarray')
+            if out.shape != self._shape or out.dtype != self.dtype:
+                raise ValueError('out must be a numpy.ndarray of the same shape and dtype')
+            if out.flags.c_contiguous:
+                letter = 'C'
+            elif out.flags.f_contiguous:
+                letter = 'F'
+            else:
+                raise ValueError('out must be a C- or Fortran-contiguous numpy.ndarray')
+        if letter == 'F' and len(self._shape) > 1:
+            # a Fortran-ordered host array is the C-ordered array of the
+            # transposed data: fetch that into the transposed host array
+            if out is None:
+                out = numpy.empty(self._shape, dtype=self.dtype, order='F')
+            self.transpose().get(stream=stream, order='C', out=out.T, blocking=blocking)
+            return out
         src = self if self._c_contiguous else _ascontiguous(self)
         if out is None:
             out = numpy.empty(self._shape, dtype=self.dtype)
-        else:
-            if out.shape != self._shape or out.dtype != self.dtype or \
-                    not out.flags.c_contiguous:
-                raise ValueError('out must be a C-contiguous numpy.ndarray of '
-                                 'the same shape and dtype')
         if self.size == 0:
             return out
         if stream is None:

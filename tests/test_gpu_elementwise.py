@@ -577,3 +577,26 @@ def test_transposes_of_narrow_arrays(shape):
     flat = rng.integers(-9, 10, n + 1).astype(np.int32)
     got = cp.ascontiguousarray(cp.asarray(flat)[1:].reshape(shape).transpose(perm)).get()
     assert_exact(got, np.ascontiguousarray(np.swapaxes(flat[1:].reshape(shape), -1, -2)))
+
+
+@pytest.mark.parametrize('perm', [(0, 1, 2), (2, 1, 0), (1, 2, 0)])
+def test_orders_of_reshape_ravel_flatten_and_get(perm):
+    """(reference: cupy/_core/_routines_manipulation.pyx:135-208, core.pyx:2098-2160)"""
+    rng = np.random.default_rng(17)
+    h = rng.standard_normal((6, 10, 14)).astype(np.float32).transpose(perm)
+    d = cp.asarray(np.ascontiguousarray(h.transpose(np.argsort(perm)))).transpose(perm)
+    assert d.strides == h.strides
+    for order in ('C', 'F', 'A', 'K'):
+        assert np.array_equal(d.ravel(order=order).get(), h.ravel(order=order)), order
+        assert np.array_equal(d.flatten(order=order).get(), h.flatten(order=order)), order
+    for order in ('C', 'F', 'A'):
+        want = h.reshape((20, 42), order=order)
+        assert np.array_equal(d.reshape((20, 42), order=order).get(), want), order
+        got = d.get(order=order)
+        assert np.array_equal(got, h)
+        assert got.flags.f_contiguous == np.asarray(h, order=order).flags.f_contiguous
+    out = np.empty(h.shape, np.float32, order='F')
+    assert d.get(out=out) is out and np.array_equal(out, h)
+    part = d[1:, ::2]
+    assert np.array_equal(part.get(order='F'), h[1:, ::2])
+    assert part.get(order='F').flags.f_contiguous

@@ -585,3 +585,59 @@ def test_in_place_with_reductions_and_overlapping_arguments():
     c = cp.asarray(a)
     shift(c, c)
     _same(c, a * 4)
+
+
+def test_division_by_a_value_of_the_row_stays_within_one_ulp():
+    """Fused row kernels divide by a value the row shares through its
+    reciprocal and one correction step; where that is not safe (reciprocal or
+    quotient zero, subnormal, infinite, NaN) they divide.  Against NumPy's
+    division: at most one ulp apart, and identical wherever zeros, infinities
+    or NaN are involved."""
+    rng = np.random.default_rng(71)
+    n_rows, n_cols = 4096, 100
+    scale = np.float32(2.0) ** rng.integers(-60, 60, (n_rows, 1)).astype(np.float32)
+    x = (rng.standard_normal((n_rows, n_cols)) * scale).astype(np.float32)
+    # the divisor of row i is column 0 times the row length (all other columns
+    # of the divisor operand are zero): every magnitude, and the special values
+    d = np.zeros((n_rows, n_cols), np.float32)
+    d[:, 0] = (rng.standard_normal(n_rows) * 2.0 ** rng.integers(-100, 100, n_rows)).astype(np.float32)
+    specials = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-39, -1e-39, 1e-45, 3e38, -3e38, 1e-37, 2e37,
+                1.0, 3.0, np.float32(1) - np.float32(2) ** -24, 1.9999999]
+    d[:len(specials), 0] = specials
+    x[::7, 3] = np.inf
+    x[::11, 5] = -np.inf
+    x[::13, 8] = np.nan
+    x[::5, 9] = 0.0
+    x[::9, 10] = -0.0
+    x[::17, 11] = 1e-40
+    x[::19, 12] = 3.3e38
+    x[::23, 13] = -1e-45
+
+    @cp.fuse()
+    def scaled(x, d):
+        return x / cp.sum(d, axis=1, keepdims=True)
+
+    from cupy_amd._core import _fusion_rows
+    with np.errstate(all='ignore'):
+        want = x / d.sum(axis=1, keepdims=True)
+    got = scaled(cp.asarray(x), cp.asarray(d)).get()
+    (plan,) = scaled._plans.values()
+    assert isinstance(plan, _fusion_rows.RowPlan)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    g, w = got[ok], want[ok]
+    # infinities exactly; the sign of every result, zeros included
+    assert np.array_equal(np.isinf(g), np.isinf(w))
+    assert np.array_equal(np.signbit(g), np.signbit(w))
+
+    def ordered(a):
+        """Floats as integers in their own order (one apart = one ulp apart)."""
+        bits = a.view(np.int32).astype(np.int64)
+        return np.where(bits < 0, -(bits & 0x7fffffff), bits)
+    apart = np.abs(ordered(g) - ordered(w))
+    assert apart.max() <= 1, apart.max()
+    # ... and all but a handful are the correctly rounded quotient itself
+    assert (apart != 0).mean() < 1e-3
+    # the cases that must take the exact route did get exact results
+    exact = np.isinf(w) | (np.abs(w) > 1e30)
+    assert np.array_equal(g[exact].view(np.uint32), w[exact].view(np.uint32))

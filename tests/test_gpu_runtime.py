@@ -257,3 +257,9 @@ def test_work_on_the_per_thread_default_stream():
         total, running, _ = results[key]
         assert total == int(h.sum())
         assert np.array_equal(running, (h * 2).cumsum())
+
+
+def test_show_config_on_the_device(capsys):
+    cp.show_config()
+    text = capsys.readouterr().out
+    assert 'Device 0 Name' in text and 'gfx950' in text and 'hipRTC Version' in text

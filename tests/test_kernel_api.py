@@ -329,3 +329,13 @@ def test_reduce_dims_false_is_passed_to_the_launch():
     # kept: two 3-d arrays and a 3-d indexer; merged: one axis, far fewer bytes
     assert sizes[False] == (8 + 8 * 7) * 2 + 8 * 7
     assert sizes[True] < sizes[False]
+
+
+def test_show_config_lists_the_installation(capsys):
+    """(reference: cupy/__init__.py:942-946)"""
+    cp.show_config()
+    text = capsys.readouterr().out
+    for label in ('OS', 'Python Version', 'CuPy Version', 'CuPy Platform', 'NumPy Version',
+                  'Runtime Library', 'Kernel Cache Dir'):
+        assert any(line.startswith(label) and ':' in line for line in text.splitlines()), label
+    assert 'libmi355rt.so' in text

@@ -101,3 +101,76 @@ def test_array_allocation_goes_through_the_hooks():
     kinds = [e[0] for e in hook.events]
     assert kinds.count('malloc_pre') == 1 and kinds.count('free_post') == 1
     assert hook.events[0][1]['size'] == 4000 and hook.events[0][1]['mem_size'] == 4096
+
+
+# ---- the ready-made hooks (reference: tests/cupy_tests/cuda_tests/memory_hooks_tests/) ----
+
+def _fake_pool(monkeypatch):
+    monkeypatch.setattr(memory._device, 'get_device_id', lambda: 0)
+
+    class Fake(memory.BaseMemory):
+        cur = [1 << 30]
+
+        def __init__(self, size):
+            self.ptr = Fake.cur[0]
+            Fake.cur[0] += size + 4096
+            self.size = size
+            self.device_id = 0
+    return memory.MemoryPool(lambda size: memory.MemoryPointer(Fake(size), 0))
+
+
+def test_debug_print_hook_writes_one_json_line_per_event(monkeypatch):
+    import io
+    import json
+    from cupy_amd.cuda import memory_hooks
+    pool = _fake_pool(monkeypatch)
+    out = io.StringIO()
+    with memory_hooks.DebugPrintHook(file=out):
+        mem = pool.malloc(1)
+        ptr1, pmem1 = mem.ptr, id(mem.mem)
+        del mem
+        mem = pool.malloc(1)
+        ptr2, pmem2 = mem.ptr, id(mem.mem)
+        del mem
+    lines = out.getvalue().splitlines()
+    assert [json.loads(l) for l in lines] == [
+        {'hook': 'alloc', 'device_id': 0, 'mem_size': 512, 'mem_ptr': ptr1},
+        {'hook': 'malloc', 'device_id': 0, 'size': 1, 'mem_size': 512, 'mem_ptr': ptr1,
+         'pmem_id': hex(pmem1)},
+        {'hook': 'free', 'device_id': 0, 'mem_size': 512, 'mem_ptr': ptr1, 'pmem_id': hex(pmem1)},
+        {'hook': 'malloc', 'device_id': 0, 'size': 1, 'mem_size': 512, 'mem_ptr': ptr2,
+         'pmem_id': hex(pmem2)},
+        {'hook': 'free', 'device_id': 0, 'mem_size': 512, 'mem_ptr': ptr2, 'pmem_id': hex(pmem2)}]
+    # the reference's layout: no spaces, keys in its order
+    assert lines[0].startswith('{"hook":"alloc","device_id":0,"mem_size":512,"mem_ptr":')
+    assert memory_hooks.debug_print.DebugPrintHook is memory_hooks.DebugPrintHook
+
+
+def test_line_profile_hook_reports_the_call_tree(monkeypatch):
+    import io
+    import re
+    from cupy_amd.cuda import memory_hooks
+    pool = _fake_pool(monkeypatch)
+    p = pool.malloc(1000)
+    del p
+    hook = memory_hooks.LineProfileHook()
+    with hook:
+        p1 = pool.malloc(1000)      # served from the block freed above
+        p2 = pool.malloc(2000)      # needs memory from the device
+    del p1, p2
+    f = io.StringIO()
+    hook.print_report(file=f)
+    text = f.getvalue()
+    assert re.search(r'\A_root \(3\.00KB, 2\.00KB\)', text)
+    assert re.search(r'.*\.py:[0-9]+:test_line_profile_hook_reports_the_call_tree '
+                     r'\(1\.00KB, 0\.00B\)', text)
+    assert re.search(r'.*\.py:[0-9]+:test_line_profile_hook_reports_the_call_tree '
+                     r'\(2\.00KB, 2\.00KB\)', text)
+    for depth in (1, 2):
+        hook = memory_hooks.LineProfileHook(max_depth=depth)
+        with hook:
+            p = pool.malloc(1000)
+        del p
+        f = io.StringIO()
+        hook.print_report(file=f)
+        assert len(f.getvalue().split('\n')) == depth + 1
