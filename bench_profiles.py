@@ -242,10 +242,14 @@ def cmd_table(a):
             cl = [l for l in open(a.ceiling) if l.lstrip().startswith('{')][-1]
             for e in json.loads(cl)['per_config']:
                 ref[e['name']] = e['gbps']
-        out += ['`%s`: %s' % (os.path.basename(path), res['config']['workload']), '',
-                '| Operation | Algorithmic bytes | us (median of 15 x 10 calls) | min us | GB/s | of 8 TB/s |',
-                '|---|---|---|---|---|---|']
         entries = res['per_config']
+        in_step = bool(entries) and 'inside the step' in entries[0].get('timing', '')
+        out += ['`%s`: %s' % (os.path.basename(path), res['config']['workload']), '',
+                '| Operation | Algorithmic bytes | %s | min us | GB/s | of 8 TB/s |%s' % (
+                    'us inside the step (median of 15 steps)' if in_step
+                    else 'us (median of 7 x 10 calls over rotating buffers)',
+                    ' us, ten calls in a row on the same arrays |' if in_step else ''),
+                '|---|---|---|---|---|---|' + ('---|' if in_step else '')]
         if a.best_variant:
             # 'name [variant]' entries: keep the fastest variant of every name
             best = collections.OrderedDict()
@@ -256,9 +260,15 @@ def cmd_table(a):
                                                       if var else ''))
             entries = list(best.values())
         for e in entries:
-            out.append('| %s | %d | %.1f | %.1f | %.0f | %.1f %% |' % (
-                e['name'], e['bytes'], e['us'], e['min_us'], e['gbps'], e['frac'] * 100))
+            out.append('| %s | %d | %.1f | %.1f | %.0f | %.1f %% |%s' % (
+                e['name'], e['bytes'], e['us'], e['min_us'], e['gbps'], e['frac'] * 100,
+                ' %.1f |' % e['us_repeated_calls'] if in_step else ''))
         out.append('')
+        if in_step:
+            out += ['Step of %d operations: %.1f us wall time per step (%.0f GB/s over the '
+                    'algorithmic bytes), %.1f us as the sum of the kernels\' own durations.' % (
+                        len(entries), res['ms_per_step'] * 1e3, res['value'],
+                        sum(e['us'] for e in entries)), '']
         if 'launch_us' in res:
             out += ['Host cost per call (us): ' + ', '.join(
                 '%s %s' % (k, v['host_enqueue_us']) for k, v in res['launch_us'].items()), '']

@@ -761,6 +761,98 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     return '\n'.join(src) + '\n'
 
 
+def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
+                   reduce_type, typedefs='', preamble='', width=3, vec=4, threads=255,
+                   idx64=False, stream_hint=False, unroll=4):
+    """Reduction down the columns of a NARROW dense matrix (``width`` columns,
+    stored row after row, every input alike), partial results per workgroup.
+
+    A workgroup per column block would leave most lanes idle (67 columns: 17 of
+    32 lanes) and its vectors would start wherever the rows do.  Here the matrix
+    is walked as the one contiguous piece of memory it is: lane ``t`` of the
+    first ``threads`` lanes takes the vectors ``t``, ``t + threads``, ... of its
+    workgroup's trips, all of them aligned.  ``threads * vec`` is a multiple of
+    ``width``, so the columns a lane's ``vec`` elements fall into are the same
+    on every trip -- element ``k`` of lane ``t`` always lies in column
+    ``(t * vec + k) % width`` -- and a lane keeps one accumulator per element.
+    At the end the accumulators of a column are combined through the LDS in a
+    fixed order and written as the workgroup's partial result for that column.
+    Workgroups take trips ``blockIdx.x``, ``+ gridDim.x``, ...: together they
+    walk down the matrix side by side."""
+    assert (threads * vec) % width == 0 and threads <= BLOCK
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    nt = 'true' if stream_hint else 'false'
+    ins = [a for a in args if a.kind == 'in']
+    params = _fast_params(args, idx_t, False, True)
+    src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (BLOCK, name, params))
+    src.append(_SIZE_INDEXERS)
+    src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];'
+               % (threads * vec))
+    src.append('  _type_reduce* _sm = reinterpret_cast<_type_reduce*>(_sm_raw);')
+    src.append('  const int _t = threadIdx.x;')
+    src.append('  const ptrdiff_t _total = (ptrdiff_t)_n_red * %d;' % width)
+    src.append('  _type_reduce _acc[%d];' % vec)
+    src.append('#pragma unroll')
+    src.append('  for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (vec, _identity_decl(identity)))
+    src.append('  if (_t < %d) {' % threads)
+    src.append('    ptrdiff_t _e = ((ptrdiff_t)blockIdx.x * %d + _t) * %d;' % (threads, vec))
+    src.append('    const ptrdiff_t _step = (ptrdiff_t)gridDim.x * %d;' % (threads * vec))
+
+    def loads(pad, e_expr, suffix):
+        for a in ins:
+            src.append('%sconst cupy::Vec<%s, %d> _l_%s%s = cupy::load_vec<%s, %d, %s>(_p_%s + (%s));'
+                       % (pad, a.store_t, vec, a.name, suffix, a.store_t, vec, nt, a.name, e_expr))
+
+    def accumulate(pad, e_expr, suffix):
+        src.append('#pragma unroll')
+        src.append('%sfor (int _k = 0; _k < %d; ++_k) {' % (pad, vec))
+        src.append('%s  const IndexT _J = (IndexT)(((%s) + _k) / %d); (void)_J;' % (pad, e_expr, width))
+        for a in ins:
+            src.append('%s  const %s %s(_l_%s%s.v[_k]);' % (pad, a.var_t, a.name, a.name, suffix))
+        src.append('%s  _type_reduce _a = static_cast<_type_reduce>(%s);' % (pad, pre_map_expr))
+        src.append('%s  _acc[_k] = REDUCE(_acc[_k], _a);' % pad)
+        src.append('%s}' % pad)
+
+    if unroll > 1:
+        src.append('    for (; _e + %d * _step + %d <= _total; _e += %d * _step) {' % (
+            unroll - 1, vec, unroll))
+        for u in range(unroll):
+            loads('      ', '_e + %d * _step' % u, '_%d' % u)
+        for u in range(unroll):
+            accumulate('      ', '_e + %d * _step' % u, '_%d' % u)
+        src.append('    }')
+    src.append('    for (; _e + %d <= _total; _e += _step) {' % vec)
+    loads('      ', '_e', '')
+    accumulate('      ', '_e', '')
+    src.append('    }')
+    # the last vector of the matrix may be a partial one
+    src.append('    if (_e < _total) {')
+    src.append('#pragma unroll')
+    src.append('      for (int _k = 0; _k < %d; ++_k) if (_e + _k < _total) {' % vec)
+    src.append('        const IndexT _J = (IndexT)((_e + _k) / %d); (void)_J;' % width)
+    for a in ins:
+        src.append('        const %s %s(_p_%s[_e + _k]);' % (a.var_t, a.name, a.name))
+    src.append('        _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
+    src.append('        _acc[_k] = REDUCE(_acc[_k], _a);')
+    src.append('      }')
+    src.append('    }')
+    src.append('#pragma unroll')
+    src.append('    for (int _k = 0; _k < %d; ++_k) _sm[_t * %d + _k] = _acc[_k];' % (vec, vec))
+    src.append('  }')
+    src.append('  __syncthreads();')
+    # accumulator f of the workgroup (lane f / vec, element f % vec) belongs
+    # to column f % width: one thread per column folds them in order
+    src.append('  for (int _c = _t; _c < %d; _c += %d) {' % (width, BLOCK))
+    src.append('    _type_reduce _s = _sm[_c];')
+    src.append('    for (int _f = _c + %d; _f < %d; _f += %d) _s = REDUCE(_s, _sm[_f]);' % (
+        width, threads * vec, width))
+    src.append('    _partials[(ptrdiff_t)blockIdx.x * %d + _c] = _s;' % width)
+    src.append('  }')
+    src.append('}')
+    return '\n'.join(src) + '\n'
+
+
 def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
               partial_in=False, partial_out=False, stream_hint=False, unroll=4,

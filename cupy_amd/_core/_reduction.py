@@ -846,6 +846,70 @@ class _AbstractReductionKernel:
         partials = _memory.alloc(nbytes)
         return partials, (rec.temp(nbytes) if rec is not None else -1)
 
+    # -- narrow matrices, down the columns -----------------------------------------------------
+    def _cols_flat_geometry(self, ins, n_out, n_red, so_in, sr, so_out, outs, vec):
+        """(vector width, active lanes) for the kernel that walks a narrow dense
+        matrix as one piece of memory, or None where the column kernel serves:
+        inputs that are not all the same dense matrix, rows that are whole
+        vectors and fill a power-of-two group of lanes, wide or short matrices."""
+        if not _tuning.get('cols_flat') or n_out < 2 or n_out > 256:
+            return None
+        items = set(a.dtype.itemsize for a in ins)
+        if len(items) != 1:
+            return None
+        (item,) = items
+        if any(s_o != item or s_r != n_out * item for s_o, s_r in zip(so_in, sr)):
+            return None
+        if n_out * n_red * item < _tuning.get('cols_flat_min_bytes'):
+            return None
+        vec = max(1, 16 // item)
+        if any(not _aligned(a.data.ptr, min(16, vec * item)) for a in ins):
+            return None
+        lanes = (n_out + vec - 1) // vec
+        if n_out % vec == 0 and lanes * 10 >= internal.clp2(lanes) * 8:
+            return None                  # the column kernel wastes little here
+        import math
+        period = n_out // math.gcd(n_out, vec)       # lanes after which the columns repeat
+        if period > _cg.BLOCK:
+            return None
+        return vec, period * (_cg.BLOCK // period)
+
+    def _launch_cols_flat(self, geometry, in_args, out_args, in_arr_idx, out_arr_idx, n_out,
+                          n_red, so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
+                          reduce_type, typedefs, device_id, stream_ptr, rec=None):
+        preamble, _ = self._get_preamble_options()
+        ins = [in_args[i] for i in in_arr_idx]
+        vec, threads = geometry
+        cus = _device.get_compute_units(device_id)
+        rargs = self._rargs(in_args, out_args)
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
+        unroll = 4
+        idx64 = n_out * n_red > _INT32_MAX - (1 << 24)
+        key = ('cols_flat', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
+               post_map_expr, reduce_type, n_out, vec, threads, idx64, device_id, stream_hint,
+               unroll)
+
+        def emit():
+            return self.name, _cg.emit_cols_flat(
+                self.name, rargs, self.identity, map_expr, reduce_expr, post_map_expr,
+                reduce_type, typedefs, preamble, width=n_out, vec=vec, threads=threads,
+                idx64=idx64, stream_hint=stream_hint, unroll=unroll)
+        fn, mod, _ = self._compile(key, emit, in_args)
+        trips = (n_out * n_red + threads * vec - 1) // (threads * vec)
+        grid = max(1, min(cus * _tuning.get('cols_target_blocks_per_cu'), trips // unroll))
+        ic = 'q' if idx64 else 'i'
+        vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
+        rsize = self._reduce_type_size(reduce_type, mod)
+        partials, pref = self._alloc_partials(rec, rsize * grid * n_out)
+        vals.ptr(pref, partials.ptr)
+        _launch_plan.launch(
+            rec, fn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
+            _make_packer(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
+        self._finalize_partials(
+            partials, grid, out_args, out_arr_idx, n_out, so_out, in_args, reduce_expr,
+            post_map_expr, reduce_type, typedefs, device_id, stream_ptr, rec, pref, n_out * n_red)
+
     # -- cols ---------------------------------------------------------------------------------
     def _launch_cols(self, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red,
                      so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
@@ -857,6 +921,14 @@ class _AbstractReductionKernel:
         ins = [in_args[i] for i in in_arr_idx]
         cus = _device.get_compute_units(device_id)
         vec = _max_vector_width([a.dtype.itemsize for a in ins])
+        if not batch and len(ins) == len([a for a in in_args if isinstance(a, ndarray)]):
+            flat = self._cols_flat_geometry(
+                ins, n_out, n_red, so_in, sr, so_out, [out_args[i] for i in out_arr_idx], vec)
+            if flat is not None:
+                return self._launch_cols_flat(
+                    flat, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red, so_in, sr,
+                    so_out, map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                    device_id, stream_ptr, rec)
         bcast_o = [(s == 0 and n_out > 1) for s in so_in]
         n_batch, n_cols, sb = batch if batch else (1, n_out, None)
         while vec > 1:

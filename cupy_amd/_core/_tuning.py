@@ -87,6 +87,12 @@ _params = {
     # `cols_unroll_near` (64 x 64 x 16384, axis 1: 56.0 -> 47.8 us; 257 x 511 x
     # 509: 78.5 -> 60.6 us)
     'cols_unroll': 1,
+    # Narrow dense matrices (rows that are no whole vectors, or that leave
+    # lanes of a column block idle) reduced down their columns are walked as one
+    # contiguous piece of memory, the columns a lane meets repeating from trip
+    # to trip
+    'cols_flat': True,
+    'cols_flat_min_bytes': 1 << 20,
     # Lanes across the columns of a workgroup, at most (the rest of its 256
     # threads goes down the reduce axis).  Sums over axis 0 of 16384^2 float32 /
     # 8192^2 float64, timed between other operations on other arrays: 161 / 84 us

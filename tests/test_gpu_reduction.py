@@ -513,3 +513,73 @@ def test_middle_axis_reductions_of_short_slices_with_few_columns(shape):
     flat = rng.integers(-9, 10, h.size + 1).astype(np.int32)
     assert_exact(cp.asarray(flat)[1:].reshape(shape).sum(axis=axis).get(),
                  flat[1:].reshape(shape).sum(axis=axis))
+
+
+@pytest.mark.parametrize('width', [2, 3, 5, 7, 10, 12, 17, 33, 67, 100, 129, 255])
+@pytest.mark.parametrize('dtype', ['int8', 'float16', 'float32', 'float64', 'complex64'])
+def test_columns_of_narrow_matrices(width, dtype):
+    """Reductions down the columns of narrow dense matrices walk the matrix as
+    one piece of memory (``emit_cols_flat``): every row count modulo the
+    kernel's trip, a last vector that is a partial one, every reduction
+    family, against NumPy."""
+    from cupy_amd._core import _tuning
+    from cupy_amd import _dryrun  # noqa: F401
+    _tuning.set(cols_flat_min_bytes=0)
+    try:
+        for n_rows in (4096, 5001, 70001):
+            x = shaped_random((n_rows, width), dtype, 43)
+            dx = cp.asarray(x)
+            kind = np.dtype(dtype).kind
+            if kind in 'fc':
+                got = dx.sum(axis=0).get()
+                wide = np.complex128 if kind == 'c' else np.float64
+                want = x.astype(wide).sum(axis=0)
+                tol = {'float16': 2e-3, 'float32': 1e-5, 'float64': 1e-12, 'complex64': 1e-5}[dtype]
+                scale = np.abs(x.astype(wide)).sum(axis=0)
+                assert got.dtype == np.dtype(dtype)
+                assert np.all(np.abs(got - want) <= tol * np.maximum(scale, 1))
+            else:
+                assert_exact(dx.sum(axis=0).get(), x.sum(axis=0))
+            assert_exact(dx.max(axis=0).get(), x.max(axis=0))
+            assert_exact(dx.argmin(axis=0).get(), x.argmin(axis=0))
+            assert_exact(dx.argmax(axis=0).get(), x.argmax(axis=0))
+            if kind == 'f' and dtype != 'float16':
+                v = dx.var(axis=0).get()
+                assert np.allclose(v, x.astype(np.float64).var(axis=0), rtol=1e-4)
+                m = dx.mean(axis=0).get()
+                assert np.allclose(m, x.astype(np.float64).mean(axis=0), rtol=1e-4, atol=1e-5)
+        # NaN in one column, keepdims, an output given
+        if np.dtype(dtype).kind == 'f':
+            x[7, width // 2] = np.nan
+            dx = cp.asarray(x)
+            assert_exact(dx.max(axis=0, keepdims=True).get(), x.max(axis=0, keepdims=True))
+            assert_exact(dx.argmax(axis=0).get(), x.argmax(axis=0))
+            out = cp.zeros((width,), dx.dtype)
+            cp.nanmax(dx, axis=0, out=out)
+            assert_exact(out.get(), np.nanmax(x, axis=0))
+    finally:
+        _tuning.set(cols_flat_min_bytes=1 << 20)
+
+
+def test_columns_of_a_narrow_matrix_use_the_flat_kernel_and_replay():
+    rng = np.random.default_rng(44)
+    h = rng.integers(-100, 100, (300007, 67)).astype(np.int32)
+    d = cp.asarray(h)
+    from cupy_amd.cuda import function
+    seen = []
+    orig = function.Function.launch_packed
+    function.Function.launch_packed = lambda self, grid, *a, **k: (
+        seen.append((self.name, grid)), orig(self, grid, *a, **k))[1]
+    try:
+        got = d.sum(axis=0)
+    finally:
+        function.Function.launch_packed = orig
+    assert [s[0] for s in seen] == ['cupy_sum', 'cupy_sum_combine']
+    assert seen[0][1][1] == 1            # one grid dimension: workgroups walk trips, not column blocks
+    assert_exact(got.get(), h.sum(axis=0))
+    for _ in range(3):                   # replays
+        assert_exact(d.sum(axis=0).get(), h.sum(axis=0))
+    # a view that starts elsewhere takes the same route when aligned, the
+    # column kernel otherwise; both agree with NumPy
+    assert_exact(d[4:].sum(axis=0).get(), h[4:].sum(axis=0))
+    assert_exact(d[1:].sum(axis=0).get(), h[1:].sum(axis=0))
