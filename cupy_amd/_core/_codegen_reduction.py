@@ -842,13 +842,24 @@ def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     src.append('  }')
     src.append('  __syncthreads();')
     # accumulator f of the workgroup (lane f / vec, element f % vec) belongs
-    # to column f % width: one thread per column folds them in order
-    src.append('  for (int _c = _t; _c < %d; _c += %d) {' % (width, BLOCK))
-    src.append('    _type_reduce _s = _sm[_c];')
-    src.append('    for (int _f = _c + %d; _f < %d; _f += %d) _s = REDUCE(_s, _sm[_f]);' % (
-        width, threads * vec, width))
-    src.append('    _partials[(ptrdiff_t)blockIdx.x * %d + _c] = _s;' % width)
-    src.append('  }')
+    # to column f % width: the accumulators j = f / width of a column are
+    # folded pairwise, j with j + m for m halving from the power of two below
+    # their number -- a fixed order, every thread taking several pairs
+    count = threads * vec // width
+    m = 1
+    while m * 2 < count:
+        m *= 2
+    while m >= 1 and count > 1:
+        src.append('  for (int _p = _t; _p < %d; _p += %d) {' % (width * m, BLOCK))
+        src.append('    const int _j = _p / %d;' % width)
+        src.append('    if (_j + %d < %d) _sm[_p] = REDUCE(_sm[_p], _sm[_p + %d]);' % (
+            m, count, m * width))
+        src.append('  }')
+        src.append('  __syncthreads();')
+        count = min(count, m)
+        m //= 2
+    src.append('  for (int _c = _t; _c < %d; _c += %d)' % (width, BLOCK))
+    src.append('    _partials[(ptrdiff_t)blockIdx.x * %d + _c] = _sm[_c];' % width)
     src.append('}')
     return '\n'.join(src) + '\n'
 

@@ -847,7 +847,7 @@ class _AbstractReductionKernel:
         return partials, (rec.temp(nbytes) if rec is not None else -1)
 
     # -- narrow matrices, down the columns -----------------------------------------------------
-    def _cols_flat_geometry(self, ins, n_out, n_red, so_in, sr, so_out, outs, vec):
+    def _cols_flat_geometry(self, ins, n_out, n_red, so_in, sr, so_out, outs, vec, exprs):
         """(vector width, active lanes) for the kernel that walks a narrow dense
         matrix as one piece of memory, or None where the column kernel serves:
         inputs that are not all the same dense matrix, rows that are whole
@@ -865,9 +865,24 @@ class _AbstractReductionKernel:
         vec = max(1, 16 // item)
         if any(not _aligned(a.data.ptr, min(16, vec * item)) for a in ins):
             return None
-        lanes = (n_out + vec - 1) // vec
-        if n_out % vec == 0 and lanes * 10 >= internal.clp2(lanes) * 8:
-            return None                  # the column kernel wastes little here
+        # what the column kernel would make of it: column blocks of up to
+        # `cols_tx` lanes (a power of two) times `vec` columns.  One block across
+        # serves as well or better (2^26 float32 with 3 / 40 / 80 columns: 45 / 45 /
+        # 46 us against 51 / 48 / 47 here; with 33 or 67 the two tie); rows that
+        # take two blocks or more do better here (129 / 160 / 200 / 255 columns:
+        # 72 / 57 / 58 / 59 us against 51 / 48 / 49 / 53), and so do the short rows
+        # of one- and two-byte items that leave most of a block's lanes idle (2^27
+        # float16 with 67 columns: 63 against 52).  Reductions that carry the
+        # position (argmax) over such items pay more for the position than
+        # they gain.
+        positional = any(uses_identifier(e, '_J') for e in exprs)
+        tx = max(1, min(_tuning.get('cols_tx'), internal.clp2((n_out + vec - 1) // vec)))
+        blocks = (n_out + tx * vec - 1) // (tx * vec)
+        if _tuning.get('cols_flat') != 'always':
+            if item < 4 and positional:
+                return None
+            if blocks < 2 and not (item < 4 and n_out * 10 < tx * vec * 6):
+                return None
         import math
         period = n_out // math.gcd(n_out, vec)       # lanes after which the columns repeat
         if period > _cg.BLOCK:
@@ -923,7 +938,8 @@ class _AbstractReductionKernel:
         vec = _max_vector_width([a.dtype.itemsize for a in ins])
         if not batch and len(ins) == len([a for a in in_args if isinstance(a, ndarray)]):
             flat = self._cols_flat_geometry(
-                ins, n_out, n_red, so_in, sr, so_out, [out_args[i] for i in out_arr_idx], vec)
+                ins, n_out, n_red, so_in, sr, so_out, [out_args[i] for i in out_arr_idx], vec,
+                (map_expr, reduce_expr, post_map_expr))
             if flat is not None:
                 return self._launch_cols_flat(
                     flat, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red, so_in, sr,

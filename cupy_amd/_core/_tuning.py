@@ -87,10 +87,11 @@ _params = {
     # `cols_unroll_near` (64 x 64 x 16384, axis 1: 56.0 -> 47.8 us; 257 x 511 x
     # 509: 78.5 -> 60.6 us)
     'cols_unroll': 1,
-    # Narrow dense matrices (rows that are no whole vectors, or that leave
-    # lanes of a column block idle) reduced down their columns are walked as one
-    # contiguous piece of memory, the columns a lane meets repeating from trip
-    # to trip
+    # Narrow dense matrices whose rows take two column blocks or more (or, for
+    # one- and two-byte items, leave most lanes of one idle) are walked as one
+    # contiguous piece of memory when reduced down their columns, the columns
+    # a lane meets repeating from trip to trip.  'always': every width from 2
+    # to 256 whatever the column kernel would make of it (for tests).
     'cols_flat': True,
     'cols_flat_min_bytes': 1 << 20,
     # Lanes across the columns of a workgroup, at most (the rest of its 256

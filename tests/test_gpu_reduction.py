@@ -524,7 +524,7 @@ def test_columns_of_narrow_matrices(width, dtype):
     family, against NumPy."""
     from cupy_amd._core import _tuning
     from cupy_amd import _dryrun  # noqa: F401
-    _tuning.set(cols_flat_min_bytes=0)
+    _tuning.set(cols_flat_min_bytes=0, cols_flat='always')
     try:
         for n_rows in (4096, 5001, 70001):
             x = shaped_random((n_rows, width), dtype, 43)
@@ -558,12 +558,12 @@ def test_columns_of_narrow_matrices(width, dtype):
             cp.nanmax(dx, axis=0, out=out)
             assert_exact(out.get(), np.nanmax(x, axis=0))
     finally:
-        _tuning.set(cols_flat_min_bytes=1 << 20)
+        _tuning.set(cols_flat_min_bytes=1 << 20, cols_flat=True)
 
 
 def test_columns_of_a_narrow_matrix_use_the_flat_kernel_and_replay():
     rng = np.random.default_rng(44)
-    h = rng.integers(-100, 100, (300007, 67)).astype(np.int32)
+    h = rng.integers(-100, 100, (150007, 131)).astype(np.int32)
     d = cp.asarray(h)
     from cupy_amd.cuda import function
     seen = []
