@@ -77,7 +77,7 @@ class Code:
 # computed once per row): the product x * r is within an ulp or so of the
 # quotient; its residual x - q * d is exact in one fused multiply-add, and adding
 # residual * r gives the correctly rounded quotient except in rare cases that
-# end one ulp away (Markstein's correction step).  Six instructions against the
+# end one ulp away (Markstein's correction step).  Four instructions against the
 # ten to thirteen of the division's full expansion.  Where that reasoning does not hold
 # the division itself is carried out: a quotient that is infinite or NaN (an
 # infinite or NaN dividend, overflow), and every quotient of a row whose
@@ -87,12 +87,15 @@ _DIVIDE_BY_SHARED = '''__device__ __forceinline__ void %s(
     const float x, const float d, const float r, float& out) {
   const float p = x * r;
   const float e = __builtin_fmaf(-p, d, x);
-  float q = __builtin_fmaf(e, r, p);
-  // (a zero quotient takes its sign from the product: the correction step
-  // turns -0 into +0)
-  q = (q == 0.0f) ? p : q;
-  if (__builtin_expect(__builtin_fabsf(q) < __builtin_inff(), 1)) {
+  const float q = __builtin_fmaf(e, r, p);
+  // one test of the quotient's class sorts out what the three operations
+  // above do not settle: zeros (0x60), infinities (0x204), NaN (0x3)
+  if (__builtin_expect(!__builtin_amdgcn_classf(q, 0x267), 1)) {
     out = q;
+  } else if (q == 0.0f) {
+    // (a zero quotient takes its sign from the product: the correction step
+    // turns -0 into +0)
+    out = p;
   } else {
     // (the empty statement keeps the division on this side of the branch: as a
     // plain conditional expression it is evaluated for every element)

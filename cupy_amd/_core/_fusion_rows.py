@@ -279,10 +279,22 @@ def _build(nodes, pieces, returns, single, args, name):
     # lane keeps many loads in flight; a workgroup per row beyond that
     group = WAVE if words_for(WAVE) <= _tuning.get('fused_rows_wave_words') else BLOCK
     if group == WAVE:
-        # short rows: as many lanes as the row has vectors, several rows per wave
-        group = max(1, min(WAVE, internal.clp2((n_cols + vec - 1) // vec)))
+        # short rows: several rows per wave, a few vectors of a row per lane
+        n_vec = (n_cols + vec - 1) // vec
+        per = max(1, _tuning.get('fused_rows_vectors_per_lane'))
+        group = max(1, min(WAVE, internal.clp2((n_vec + per - 1) // per)))
     per_lane = (n_cols + group * vec - 1) // (group * vec)          # vectors per lane and operand
     words = words_for(group)
+    # rows a group has in flight: `fused_rows_in_flight` where a lane holds one
+    # vector of a row and the rows are enough for every CU to have several
+    # workgroups (rows of 257 float32, two vectors per lane: a softmax gains
+    # 8 us of 110 with two rows in flight, x / sqrt(sum(x * x)) loses 8 of 92)
+    rows_in_flight = 1
+    if group <= WAVE and per_lane == 1:
+        cus_ = _device.get_compute_units(_device.get_device_id())
+        rows_in_flight = max(1, _tuning.get('fused_rows_in_flight'))
+        while rows_in_flight > 1 and n_rows < cus_ * 8 * (BLOCK // group) * rows_in_flight:
+            rows_in_flight //= 2
     if words > _ROW_WORDS_PER_LANE or n_cols < 2:
         raise _Unsupported('row of %d elements does not fit the registers of a group' % n_cols)
 
@@ -370,6 +382,7 @@ def _build(nodes, pieces, returns, single, args, name):
     src.append('#define GROUP %d' % group)
     src.append('#define VEC %d' % vec)
     src.append('#define PER_LANE %d' % per_lane)
+    src.append('#define ROWS %d' % rows_in_flight)
     # a vector of a row: whole where it lies within the row, element by element
     # where the row ends inside it (rows that are not a multiple of VEC long)
     src.append('''template <typename T, bool kStream>
@@ -425,21 +438,39 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
             src.append('  const %s _u%d = _p%d[0];' % (t, n.order, n.order))
             cname[n.order] = '_u%d' % n.order
     src.append('  const %s _rows_per_block = %d / GROUP;' % (idx_t, BLOCK))
-    src.append('  for (%s _row = (%s)blockIdx.x * _rows_per_block + threadIdx.x / GROUP; '
-               '_row < _n_rows; _row += (%s)gridDim.x * _rows_per_block) {' % (idx_t, idx_t, idx_t))
-    # the row, in registers; every load is issued before any value is used
+    # Short rows: a group has ROWS rows in flight -- the loads of all of them
+    # are issued before the first is worked on (a lane holds a few words of a
+    # row: one row per pass leaves too few bytes on their way to hide the
+    # memory's latency behind the arithmetic)
+    src.append('  for (%s _row0 = (%s)blockIdx.x * (_rows_per_block * ROWS) + threadIdx.x / GROUP; '
+               '_row0 < _n_rows; _row0 += (%s)gridDim.x * (_rows_per_block * ROWS)) {'
+               % (idx_t, idx_t, idx_t))
     for n in full_leaves:
         t = get_typename(leaf_value[n.order].dtype)
-        src.append('    cupy::Vec<%s, VEC> _f%d[PER_LANE];' % (t, n.order))
+        src.append('    cupy::Vec<%s, VEC> _fa%d[ROWS][PER_LANE];' % (t, n.order))
     src.append('#pragma unroll')
-    src.append('    for (int _e = 0; _e < PER_LANE; ++_e) {')
-    src.append('      const int _col = (_e * GROUP + _lane) * VEC;')
-    src.append('      const int _cc = _col < NCOLS ? _col : 0;')
+    src.append('    for (int _r = 0; _r < ROWS; ++_r) {')
+    src.append('      const %s _rr = (_row0 + _r * _rows_per_block < _n_rows) ? '
+               '(_row0 + _r * _rows_per_block) : (_n_rows - 1);' % idx_t)
+    src.append('#pragma unroll')
+    src.append('      for (int _e = 0; _e < PER_LANE; ++_e) {')
+    src.append('        const int _col = (_e * GROUP + _lane) * VEC;')
+    src.append('        const int _cc = _col < NCOLS ? _col : 0;')
     for n in full_leaves:
         t = get_typename(leaf_value[n.order].dtype)
-        src.append('      _f%d[_e] = _row_vec<%s, %s>(_p%d + (ptrdiff_t)_row * NCOLS, _cc);'
+        src.append('        _fa%d[_r][_e] = _row_vec<%s, %s>(_p%d + (ptrdiff_t)_rr * NCOLS, _cc);'
                    % (n.order, t, ntl, n.order))
+    src.append('      }')
     src.append('    }')
+    src.append('#pragma unroll')
+    src.append('    for (int _r = 0; _r < ROWS; ++_r) {')
+    src.append('    const %s _row = _row0 + _r * _rows_per_block;' % idx_t)
+    # (a group's lanes share the row, so this is uniform over every set of
+    # lanes that exchanges values below)
+    src.append('    if (ROWS > 1 && _row >= _n_rows) break;')
+    for n in full_leaves:
+        t = get_typename(leaf_value[n.order].dtype)
+        src.append('    cupy::Vec<%s, VEC> (&_f%d)[PER_LANE] = _fa%d[_r];' % (t, n.order, n.order))
     for n in leaf_nodes:
         if kinds[n.order] == 'rowk':
             t = get_typename(leaf_value[n.order].dtype)
@@ -490,11 +521,18 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
             src.append('#pragma unroll')
             src.append('    for (int _e = 0; _e < PER_LANE; ++_e) {')
             src.append('      const int _col = (_e * GROUP + _lane) * VEC;')
+            # (rows of whole vectors: one test per vector instead of one per element)
+            whole = n_cols % vec == 0
+            if whole:
+                src.append('      if (_col < NCOLS) {')
             src.append('#pragma unroll')
-            src.append('      for (int _k = 0; _k < VEC; ++_k) if (_col + _k < NCOLS) {')
+            src.append('      for (int _k = 0; _k < VEC; ++_k) %s{' % (
+                '' if whole else 'if (_col + _k < NCOLS) '))
             src.append('        _a%d = piece%d::Op()(_a%d, piece%d::_fz_map(%s));' % (
                 k, k, k, k, ', '.join(call_args)))
             src.append('      }')
+            if whole:
+                src.append('      }')
             src.append('    }')
             if group == 1:
                 pass
@@ -547,11 +585,12 @@ __device__ __forceinline__ void _row_store(T* row, int col, const cupy::Vec<T, V
     for n in out_nodes:
         if kinds[n.order] in ('row', 'rowk'):
             src.append('    if (_lane == 0) _o%d[_row] = %s;' % (n.order, operand(n)))
+    src.append('    }')
     src.append('  }')
     src.append('}')
     code = '\n'.join(src) + '\n'
     fn = compiler.compile_with_cache(code, ('-DCUPY_FUSED_ROWS',)).get_function(name)
-    rows_per_block = BLOCK // group
+    rows_per_block = BLOCK // group * rows_in_flight
     cus = _device.get_compute_units(_device.get_device_id())
     grid = max(1, min((n_rows + rows_per_block - 1) // rows_per_block,
                       cus * _tuning.get('fused_rows_blocks_per_cu')))

@@ -170,6 +170,16 @@ _params = {
     # with a wave against 68 % with a workgroup.  Requesting the next row before
     # the current one is worked on did not help: 62 % against 76 % on rows of 8192)
     'fused_rows_wave_words': 32,
+    # Lanes of a short row: as many as it has vectors (1 vector per lane).
+    # Fewer lanes with more vectors each would repeat less of the work that is
+    # done once per row, but their accesses fall apart: softmax over rows of
+    # 100 float32 takes 97 us with 1, 104 with 2, 151 with 4 vectors per lane
+    'fused_rows_vectors_per_lane': 1,
+    # Short rows in flight per group of lanes (softmax over rows of 100 / 33
+    # float32: 98 / 142 us with 1, 94 / 132 with 2, 91 / 127 with 4;
+    # x / sqrt(sum(x * x)) over rows of 100 / 33 / 64: 87 / 124 / 78 with 1,
+    # 90 / 117 / 76 with 4)
+    'fused_rows_in_flight': 4,
     # a float32 division by a value the whole row shares (the sum of a softmax)
     # goes through the value's reciprocal and one correction step
     'fused_rows_reciprocal': True,

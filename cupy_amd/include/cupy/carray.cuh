@@ -382,14 +382,18 @@ _CUPY_DEV T select_value(bool c, const T& a, const T& b) {
 // One value moved between lanes by a data-parallel-primitive modifier
 // (`kCtrl`: quad permutation, row mirror / half mirror, row rotation), word by
 // word.  These run in the vector ALU; a general shuffle goes through the LDS
-// crossbar.
+// crossbar.  Every one of these modifiers is a permutation within a row of 16
+// lanes, so no lane ever lacks a source; saying that such a lane would read
+// zero (the last argument) is what lets the compiler fold the move into the
+// instruction that consumes it (one `v_add_f32 ... row_mirror` instead of
+// two moves and an add).
 template <int kCtrl, typename T>
 _CUPY_DEV T _dpp_move(const T& v) {
   constexpr int kWords = (sizeof(T) + 3) / 4;
   int w[kWords] = {};
   __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
-  for (int k = 0; k < kWords; ++k) w[k] = __builtin_amdgcn_update_dpp(w[k], w[k], kCtrl, 0xf, 0xf, false);
+  for (int k = 0; k < kWords; ++k) w[k] = __builtin_amdgcn_update_dpp(0, w[k], kCtrl, 0xf, 0xf, true);
   T r = v;
   __builtin_memcpy(&r, w, sizeof(T));
   return r;

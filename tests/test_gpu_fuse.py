@@ -306,11 +306,14 @@ def test_kernel_sequence_cases_match_numpy():
 
 @pytest.mark.parametrize('shape', [(301, 77), (70, 33), (64, 4096), (17, 5, 1000), (1000,),
                                    (129, 8192), (300, 1001), (64, 4099), (128, 777), (33, 18),
-                                   (5000, 10), (777, 3), (100, 2), (4099, 7)])
+                                   (5000, 10), (777, 3), (100, 2), (4099, 7),
+                                   (70001, 100), (140003, 33), (600001, 5), (66000, 64)])
 def test_row_wise_functions_in_one_kernel_match_numpy(shape):
     """Functions whose reductions all run along short rows compile to a single
     kernel that holds the row in registers (wave-per-row and workgroup-per-row
-    variants, vector widths 1 to 4, ragged row lengths)."""
+    variants, vector widths 1 to 4, ragged row lengths; with rows in plenty,
+    four or two short rows in flight per group of lanes and a last pass that
+    has fewer)."""
     rng = np.random.default_rng(45)
     h = rng.standard_normal(shape).astype(np.float32)
     w = rng.uniform(0.5, 1.5, shape[-1]).astype(np.float32)
