@@ -350,10 +350,10 @@ def emit_flat(name, operands, operation, typedefs='', preamble='',
     b = bcast_decls()
     if b:
         src.append(b)
-    if vec > 1:
-        src.extend(body)
-    else:
-        src.append('  const %s _nvec = 0;' % idx_t)
+    # (vec == 1 -- items of 16 bytes, arrays aligned for no more than an item --
+    # takes the same loop with vectors of one element: it is the one that marks
+    # accesses as streaming and keeps several in flight per lane)
+    src.extend(body)
     src.extend(tail)
     src.append('  %s;' % after_loop)
     src.append('}')

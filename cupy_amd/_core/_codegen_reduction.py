@@ -358,7 +358,10 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
     src.append('#pragma unroll')
     src.append('    for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (
         vec, _identity_decl(identity)))
-    if vec > 1:
+    # (items that are a whole vector by themselves, or arrays aligned for no
+    # more than one item, take the same loop: it is the one that keeps several
+    # loads in flight per lane and marks them as streaming)
+    if vec > 1 or unroll > 1:
         src.append('    const %s _j_vend = _j_begin + (_j_end - _j_begin) / %d * %d;' % (
             idx_t, vec, vec))
         stride = lanes * vec
