@@ -400,6 +400,19 @@ def emit_rows(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
             for u in range(unroll):
                 accumulate('      ', '_j + %d' % (u * stride), '_%d' % u)
             src.append('    }')
+            # what is left (fewer trips than that) in halves: rows of two or three
+            # trips still have two loads in flight per lane (2^18 rows of 512
+            # float32, a wave per row: one load at a time without this)
+            half = unroll // 2
+            while half >= 2:
+                src.append('    if (_j + %d < _j_vend) {' % ((half - 1) * stride))
+                for u in range(half):
+                    loads('      ', '_j + %d' % (u * stride), '_h%d_%d' % (half, u))
+                for u in range(half):
+                    accumulate('      ', '_j + %d' % (u * stride), '_h%d_%d' % (half, u))
+                src.append('      _j += %d;' % (half * stride))
+                src.append('    }')
+                half //= 2
         src.append('    for (; _j < _j_vend; _j += %d) {' % stride)
         loads('      ', '_j', '')
         accumulate('      ', '_j', '')
@@ -575,13 +588,8 @@ def emit_rows_batched(name, args, identity, pre_map_expr, reduce_expr, post_map_
     src.append('      _s[_r] = _acc;')
     src.append('    }')
     if group > 1:
-        m = 1
-        while m < group:
-            # the steps of the `batch` independent all-reduces side by side
-            src.append('#pragma unroll')
-            src.append('    for (int _r = 0; _r < %d; ++_r) '
-                       '_s[_r] = cupy::xor_combine<%d, false>(_s[_r], _ReduceOp());' % (batch, m))
-            m *= 2
+        # the steps of the `batch` independent all-reduces side by side
+        src.append('    cupy::batch_allreduce<%d>(_s, _ReduceOp());' % group)
     src.append('#pragma unroll')
     src.append('    for (int _r = 0; _r < %d; ++_r) {' % batch)
     src.append('      const %s _i = _i0 + _r * _step;' % idx_t)

@@ -129,6 +129,54 @@ __device__ __forceinline__ arg_key32<T, kMax> arg_pick(arg_key32<T, kMax> a, arg
   return r;
 }
 
+// All-reduces of packed keys over lanes go word by word: first the high words
+// (a 32-bit max or min, whose lane exchange folds into the instruction itself),
+// then the low words of the lanes that hold the winning high word.  A step
+// costs two instructions instead of seven for the 64-bit compare-and-select.
+struct _arg_imax { __device__ __forceinline__ int operator()(int a, int b) const { return a > b ? a : b; } };
+struct _arg_imin { __device__ __forceinline__ int operator()(int a, int b) const { return a < b ? a : b; } };
+struct _arg_umax { __device__ __forceinline__ unsigned int operator()(unsigned int a, unsigned int b) const { return a > b ? a : b; } };
+struct _arg_umin { __device__ __forceinline__ unsigned int operator()(unsigned int a, unsigned int b) const { return a < b ? a : b; } };
+template <bool kMax> struct _arg_word_ops {
+  typedef typename cupy::conditional<kMax, _arg_imax, _arg_imin>::type high;
+  typedef typename cupy::conditional<kMax, _arg_umax, _arg_umin>::type low;
+};
+namespace cupy {
+template <int kFirst, int kTop, bool kKeepLow, typename T, bool kMax, int kBatch>
+__device__ __forceinline__ void _arg_key_allreduce(arg_key32<T, kMax> (&s)[kBatch]) {
+  int hi[kBatch], best[kBatch];
+  unsigned int lo[kBatch];
+#pragma unroll
+  for (int r = 0; r < kBatch; ++r) {
+    hi[r] = static_cast<int>(s[r].k >> 32);
+    best[r] = _AllReduce<kFirst, kTop, kKeepLow>::run(hi[r], typename _arg_word_ops<kMax>::high());
+  }
+#pragma unroll
+  for (int r = 0; r < kBatch; ++r) {
+    lo[r] = (hi[r] == best[r]) ? static_cast<unsigned int>(s[r].k) : (kMax ? 0u : 0xffffffffu);
+    lo[r] = _AllReduce<kFirst, kTop, kKeepLow>::run(lo[r], typename _arg_word_ops<kMax>::low());
+    s[r].k = static_cast<long long>(
+        (static_cast<unsigned long long>(static_cast<unsigned int>(best[r])) << 32) | lo[r]);
+  }
+}
+template <int kGroup, typename T, bool kMax, typename Op>
+__device__ __forceinline__ arg_key32<T, kMax> group_allreduce(arg_key32<T, kMax> v, Op) {
+  arg_key32<T, kMax> s[1] = {v};
+  _arg_key_allreduce<1, kGroup, false>(s);
+  return s[0];
+}
+template <int kStride, typename T, bool kMax, typename Op>
+__device__ __forceinline__ arg_key32<T, kMax> strided_allreduce(arg_key32<T, kMax> v, Op) {
+  arg_key32<T, kMax> s[1] = {v};
+  _arg_key_allreduce<kStride, 64, true>(s);
+  return s[0];
+}
+template <int kGroup, typename T, bool kMax, int kBatch, typename Op>
+__device__ __forceinline__ void batch_allreduce(arg_key32<T, kMax> (&s)[kBatch], Op) {
+  _arg_key_allreduce<1, kGroup, false>(s);
+}
+}  // namespace cupy
+
 template <typename T, bool kMax>
 struct arg_wide {
   min_max_st<T> s;

@@ -470,4 +470,23 @@ _CUPY_DEV T strided_allreduce(T v, Op op) {
   return _AllReduce<kStride, 64, true>::run(v, op);
 }
 
+// kBatch independent all-reduces over groups of kGroup adjacent lanes, step by
+// step side by side: the exchanges of one step do not wait for each other.
+template <int kMask, int kTop> struct _BatchAllReduce {
+  template <typename T, int kBatch, typename Op>
+  static _CUPY_DEV void run(T (&s)[kBatch], Op op) {
+#pragma unroll
+    for (int r = 0; r < kBatch; ++r) s[r] = xor_combine<kMask, false>(s[r], op);
+    _BatchAllReduce<kMask * 2, kTop>::run(s, op);
+  }
+};
+template <int kTop> struct _BatchAllReduce<kTop, kTop> {
+  template <typename T, int kBatch, typename Op>
+  static _CUPY_DEV void run(T (&)[kBatch], Op) {}
+};
+template <int kGroup, typename T, int kBatch, typename Op>
+_CUPY_DEV void batch_allreduce(T (&s)[kBatch], Op op) {
+  _BatchAllReduce<1, kGroup>::run(s, op);
+}
+
 }  // namespace cupy
