@@ -853,7 +853,8 @@ class _AbstractReductionKernel:
         return partials, (rec.temp(nbytes) if rec is not None else -1)
 
     # -- narrow matrices, down the columns -----------------------------------------------------
-    def _cols_flat_geometry(self, ins, n_out, n_red, so_in, sr, so_out, outs, vec, exprs):
+    def _cols_flat_geometry(self, ins, n_out, n_red, so_in, sr, so_out, outs, vec, exprs,
+                            state_bytes):
         """(vector width, active lanes) for the kernel that walks a narrow dense
         matrix as one piece of memory, or None where the column kernel serves:
         inputs that are not all the same dense matrix, rows that are whole
@@ -893,7 +894,13 @@ class _AbstractReductionKernel:
         period = n_out // math.gcd(n_out, vec)       # lanes after which the columns repeat
         if period > _cg.BLOCK:
             return None
-        return vec, period * (_cg.BLOCK // period)
+        threads = period * (_cg.BLOCK // period)
+        # a lane keeps `vec` states, and the workgroup lays all of them out in
+        # the LDS: wide states of narrow items (the variance of int8: 16 states
+        # of four doubles per lane) stay with the column kernel
+        if threads * vec * state_bytes > 32 * 1024:
+            return None
+        return vec, threads
 
     def _launch_cols_flat(self, geometry, in_args, out_args, in_arr_idx, out_arr_idx, n_out,
                           n_red, so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
@@ -945,7 +952,8 @@ class _AbstractReductionKernel:
         if not batch and len(ins) == len([a for a in in_args if isinstance(a, ndarray)]):
             flat = self._cols_flat_geometry(
                 ins, n_out, n_red, so_in, sr, so_out, [out_args[i] for i in out_arr_idx], vec,
-                (map_expr, reduce_expr, post_map_expr))
+                (map_expr, reduce_expr, post_map_expr),
+                _reduce_type_bytes(reduce_type, typedefs))
             if flat is not None:
                 return self._launch_cols_flat(
                     flat, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red, so_in, sr,

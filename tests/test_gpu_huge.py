@@ -158,6 +158,30 @@ def test_column_reduction_whose_blocks_continue_along_grid_z():
     assert bool(check(colsum).all().get())
 
 
+def test_narrow_matrix_walked_as_one_piece_beyond_2_to_31_elements():
+    """Column sums of a (2**24 + 3, 130) int8 matrix: the kernel that walks a
+    narrow matrix as one contiguous piece computes its offsets in 64 bits."""
+    rows, width = 2 ** 24 + 3, 130
+    a = _fill_mod100_i8(size=rows * width).reshape(rows, width)
+    from cupy_amd.cuda import function
+    seen = []
+    orig = function.Function.launch_packed
+    function.Function.launch_packed = lambda self, grid, *args, **kw: (
+        seen.append((self.name, grid)), orig(self, grid, *args, **kw))[1]
+    try:
+        colsum = a.sum(axis=0)
+        colmax = a.max(axis=0)
+    finally:
+        function.Function.launch_packed = orig
+    assert seen[0][0] == 'cupy_sum' and seen[0][1][1] == 1 and seen[0][1][2] == 1
+    # element (r, c) holds (130 r + c) % 100 = (30 (r % 10) + c) % 100
+    r10 = np.arange(10)
+    counts = np.array([(rows - k + 9) // 10 for k in range(10)], dtype=np.int64)
+    table = (30 * r10[:, None] + np.arange(width)[None, :]) % 100          # (10, width)
+    np.testing.assert_array_equal(colsum.get(), (counts[:, None] * table).sum(axis=0))
+    np.testing.assert_array_equal(colmax.get(), table.max(axis=0).astype(np.int8))
+
+
 def test_broadcast_input_of_2_to_31_elements():
     base = _fill_mod100_i8(size=2048 * 1024).reshape(2048, 1, 1024)
     a = cp.broadcast_to(base, (2048, 1024, 1024))
