@@ -774,7 +774,7 @@ def emit_rows_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
 
 def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
                    reduce_type, typedefs='', preamble='', width=3, vec=4, threads=255,
-                   idx64=False, stream_hint=False, unroll=4):
+                   idx64=False, stream_hint=False, unroll=4, block=BLOCK, chunked=False):
     """Reduction down the columns of a NARROW dense matrix (``width`` columns,
     stored row after row, every input alike), partial results per workgroup.
 
@@ -788,15 +788,16 @@ def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     ``(t * vec + k) % width`` -- and a lane keeps one accumulator per element.
     At the end the accumulators of a column are combined through the LDS in a
     fixed order and written as the workgroup's partial result for that column.
-    Workgroups take trips ``blockIdx.x``, ``+ gridDim.x``, ...: together they
-    walk down the matrix side by side."""
-    assert (threads * vec) % width == 0 and threads <= BLOCK
+    ``chunked``: a workgroup takes a run of consecutive trips, one contiguous
+    piece of memory; otherwise trips ``blockIdx.x``, ``+ gridDim.x``, ..., the
+    workgroups walking down the matrix side by side."""
+    assert (threads * vec) % width == 0 and threads <= block
     idx_t = 'ptrdiff_t' if idx64 else 'int'
     nt = 'true' if stream_hint else 'false'
     ins = [a for a in args if a.kind == 'in']
     params = _fast_params(args, idx_t, False, True)
     src = [_prologue(typedefs, preamble, reduce_type, reduce_expr, post_map_expr)]
-    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (BLOCK, name, params))
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (block, name, params))
     src.append(_SIZE_INDEXERS)
     src.append('  __shared__ __attribute__((aligned(16))) char _sm_raw[%d * sizeof(_type_reduce)];'
                % (threads * vec))
@@ -807,18 +808,37 @@ def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     src.append('#pragma unroll')
     src.append('  for (int _k = 0; _k < %d; ++_k) _acc[_k] = %s;' % (vec, _identity_decl(identity)))
     src.append('  if (_t < %d) {' % threads)
-    src.append('    ptrdiff_t _e = ((ptrdiff_t)blockIdx.x * %d + _t) * %d;' % (threads, vec))
-    src.append('    const ptrdiff_t _step = (ptrdiff_t)gridDim.x * %d;' % (threads * vec))
+    if chunked:
+        # a workgroup takes a run of consecutive trips: one contiguous piece of memory
+        src.append('    const ptrdiff_t _trips = (_total + %d) / %d;' % (threads * vec - 1, threads * vec))
+        src.append('    const ptrdiff_t _per = (_trips + gridDim.x - 1) / gridDim.x;')
+        src.append('    const ptrdiff_t _q1 = ((ptrdiff_t)blockIdx.x + 1) * _per < _trips ? '
+                   '((ptrdiff_t)blockIdx.x + 1) * _per : _trips;')
+        src.append('    ptrdiff_t _e = ((ptrdiff_t)blockIdx.x * _per * %d + _t) * %d;' % (threads, vec))
+        src.append('    const ptrdiff_t _step = %d;' % (threads * vec))
+        src.append('    const ptrdiff_t _end = _q1 * %d < _total ? _q1 * %d : _total;' % (
+            threads * vec, threads * vec))
+    else:
+        src.append('    ptrdiff_t _e = ((ptrdiff_t)blockIdx.x * %d + _t) * %d;' % (threads, vec))
+        src.append('    const ptrdiff_t _step = (ptrdiff_t)gridDim.x * %d;' % (threads * vec))
+        src.append('    const ptrdiff_t _end = _total;')
+    # the row of element k of this lane's vector: a step is a whole number of
+    # rows, so the rows advance by a constant from trip to trip and no element
+    # needs a division of its own
+    src.append('    const IndexT _jstep = (IndexT)(_step / %d);' % width)
+    src.append('    IndexT _jb[%d];' % vec)
+    src.append('#pragma unroll')
+    src.append('    for (int _k = 0; _k < %d; ++_k) _jb[_k] = (IndexT)((_e + _k) / %d);' % (vec, width))
 
     def loads(pad, e_expr, suffix):
         for a in ins:
             src.append('%sconst cupy::Vec<%s, %d> _l_%s%s = cupy::load_vec<%s, %d, %s>(_p_%s + (%s));'
                        % (pad, a.store_t, vec, a.name, suffix, a.store_t, vec, nt, a.name, e_expr))
 
-    def accumulate(pad, e_expr, suffix):
+    def accumulate(pad, u, suffix):
         src.append('#pragma unroll')
         src.append('%sfor (int _k = 0; _k < %d; ++_k) {' % (pad, vec))
-        src.append('%s  const IndexT _J = (IndexT)(((%s) + _k) / %d); (void)_J;' % (pad, e_expr, width))
+        src.append('%s  const IndexT _J = _jb[_k] + %d * _jstep; (void)_J;' % (pad, u))
         for a in ins:
             src.append('%s  const %s %s(_l_%s%s.v[_k]);' % (pad, a.var_t, a.name, a.name, suffix))
         src.append('%s  _type_reduce _a = static_cast<_type_reduce>(%s);' % (pad, pre_map_expr))
@@ -826,22 +846,26 @@ def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
         src.append('%s}' % pad)
 
     if unroll > 1:
-        src.append('    for (; _e + %d * _step + %d <= _total; _e += %d * _step) {' % (
+        src.append('    for (; _e + %d * _step + %d <= _end; _e += %d * _step) {' % (
             unroll - 1, vec, unroll))
         for u in range(unroll):
             loads('      ', '_e + %d * _step' % u, '_%d' % u)
         for u in range(unroll):
-            accumulate('      ', '_e + %d * _step' % u, '_%d' % u)
+            accumulate('      ', u, '_%d' % u)
+        src.append('#pragma unroll')
+        src.append('      for (int _k = 0; _k < %d; ++_k) _jb[_k] += %d * _jstep;' % (vec, unroll))
         src.append('    }')
-    src.append('    for (; _e + %d <= _total; _e += _step) {' % vec)
+    src.append('    for (; _e + %d <= _end; _e += _step) {' % vec)
     loads('      ', '_e', '')
-    accumulate('      ', '_e', '')
+    accumulate('      ', 0, '')
+    src.append('#pragma unroll')
+    src.append('      for (int _k = 0; _k < %d; ++_k) _jb[_k] += _jstep;' % vec)
     src.append('    }')
     # the last vector of the matrix may be a partial one
-    src.append('    if (_e < _total) {')
+    src.append('    if (_e < _end) {')
     src.append('#pragma unroll')
-    src.append('      for (int _k = 0; _k < %d; ++_k) if (_e + _k < _total) {' % vec)
-    src.append('        const IndexT _J = (IndexT)((_e + _k) / %d); (void)_J;' % width)
+    src.append('      for (int _k = 0; _k < %d; ++_k) if (_e + _k < _end) {' % vec)
+    src.append('        const IndexT _J = _jb[_k]; (void)_J;')
     for a in ins:
         src.append('        const %s %s(_p_%s[_e + _k]);' % (a.var_t, a.name, a.name))
     src.append('        _type_reduce _a = static_cast<_type_reduce>(%s);' % pre_map_expr)
@@ -861,7 +885,7 @@ def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
     while m * 2 < count:
         m *= 2
     while m >= 1 and count > 1:
-        src.append('  for (int _p = _t; _p < %d; _p += %d) {' % (width * m, BLOCK))
+        src.append('  for (int _p = _t; _p < %d; _p += %d) {' % (width * m, block))
         src.append('    const int _j = _p / %d;' % width)
         src.append('    if (_j + %d < %d) _sm[_p] = REDUCE(_sm[_p], _sm[_p + %d]);' % (
             m, count, m * width))
@@ -869,7 +893,7 @@ def emit_cols_flat(name, args, identity, pre_map_expr, reduce_expr, post_map_exp
         src.append('  __syncthreads();')
         count = min(count, m)
         m //= 2
-    src.append('  for (int _c = _t; _c < %d; _c += %d)' % (width, BLOCK))
+    src.append('  for (int _c = _t; _c < %d; _c += %d)' % (width, block))
     src.append('    _partials[(ptrdiff_t)blockIdx.x * %d + _c] = _sm[_c];' % width)
     src.append('}')
     return '\n'.join(src) + '\n'

@@ -872,42 +872,46 @@ class _AbstractReductionKernel:
         vec = max(1, 16 // item)
         if any(not _aligned(a.data.ptr, min(16, vec * item)) for a in ins):
             return None
-        # what the column kernel would make of it: column blocks of up to
-        # `cols_tx` lanes (a power of two) times `vec` columns.  One block across
-        # serves as well or better (2^26 float32 with 3 / 40 / 80 columns: 45 / 45 /
-        # 46 us against 51 / 48 / 47 here; with 33 or 67 the two tie); rows that
-        # take two blocks or more do better here (129 / 160 / 200 / 255 columns:
-        # 72 / 57 / 58 / 59 us against 51 / 48 / 49 / 53), and so do the short rows
-        # of one- and two-byte items that leave most of a block's lanes idle (2^27
-        # float16 with 67 columns: 63 against 52).  Reductions that carry the
-        # position (argmax) over such items pay more for the position than
-        # they gain.
-        positional = any(uses_identifier(e, '_J') for e in exprs)
-        tx = max(1, min(_tuning.get('cols_tx'), internal.clp2((n_out + vec - 1) // vec)))
-        blocks = (n_out + tx * vec - 1) // (tx * vec)
-        if _tuning.get('cols_flat') != 'always':
-            if item < 4 and positional:
-                return None
-            if blocks < 2 and not (item < 4 and n_out * 10 < tx * vec * 6):
-                return None
         import math
         period = n_out // math.gcd(n_out, vec)       # lanes after which the columns repeat
-        if period > _cg.BLOCK:
+        if period > 1024:
             return None
-        threads = period * (_cg.BLOCK // period)
+        if _tuning.get('cols_flat') != 'always':
+            # Measured over 2^26 float32 / 2^25 float64 / 2^27 float16 (us, this
+            # kernel / the column kernel, combine launch included): 33 columns
+            # 44 / 48, 67: 45 / 49, 100: 43 / 48, 129: 44 / 73, 200: 43 / 57; 3, 5,
+            # 40, 80 columns: 43-45 either way; variances gain most (33: 48 / 59,
+            # float16 x 67: 80 / 114).  Two exceptions.  Rows whose period divides
+            # the workgroup (whole vectors that fill a power-of-two group of lanes:
+            # 32, 64, 128, 256 float32 columns) are what the column kernel is made
+            # for, and here every workgroup's piece would start on a multiple of
+            # 4 KiB: 47 against 42.  Reductions that carry the position over
+            # one-byte items pay more for it than they gain (int8 x 255 argmax:
+            # 69 against 62).
+            if _cg.BLOCK % period == 0:
+                return None
+            if item < 2 and any(uses_identifier(e, '_J') for e in exprs):
+                return None
         # a lane keeps `vec` states, and the workgroup lays all of them out in
         # the LDS: wide states of narrow items (the variance of int8: 16 states
-        # of four doubles per lane) stay with the column kernel
-        if threads * vec * state_bytes > 32 * 1024:
+        # of four doubles per lane) stay with the column kernel.  The active
+        # lanes are a whole number of periods of a workgroup of 256: larger
+        # workgroups would leave fewer lanes idle (67 columns: 201 of 256, 469
+        # of 512, 1005 of 1024; 129 columns: 129, 387, 903) and are slower all
+        # the same (2^26 float32 with 67 / 129 / 255 columns: 45 / 46 / 47 us
+        # with 256 threads, 47 / 49 / 50 with 512, 53 / 55 / 56 with 1024)
+        block = _tuning.get('cols_flat_block') or _cg.BLOCK
+        threads = period * (block // period)
+        if threads == 0 or threads * vec * state_bytes > 32 * 1024:
             return None
-        return vec, threads
+        return vec, threads, block
 
     def _launch_cols_flat(self, geometry, in_args, out_args, in_arr_idx, out_arr_idx, n_out,
                           n_red, so_in, sr, so_out, map_expr, reduce_expr, post_map_expr,
                           reduce_type, typedefs, device_id, stream_ptr, rec=None):
         preamble, _ = self._get_preamble_options()
         ins = [in_args[i] for i in in_arr_idx]
-        vec, threads = geometry
+        vec, threads, block = geometry
         cus = _device.get_compute_units(device_id)
         rargs = self._rargs(in_args, out_args)
         stream_hint = _tuning.stream_policy(
@@ -916,23 +920,25 @@ class _AbstractReductionKernel:
         idx64 = n_out * n_red > _INT32_MAX - (1 << 24)
         key = ('cols_flat', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, n_out, vec, threads, idx64, device_id, stream_hint,
-               unroll)
+               unroll, block, _tuning.get('cols_flat_chunked'))
 
         def emit():
             return self.name, _cg.emit_cols_flat(
                 self.name, rargs, self.identity, map_expr, reduce_expr, post_map_expr,
                 reduce_type, typedefs, preamble, width=n_out, vec=vec, threads=threads,
-                idx64=idx64, stream_hint=stream_hint, unroll=unroll)
+                idx64=idx64, stream_hint=stream_hint, unroll=unroll, block=block,
+                chunked=_tuning.get('cols_flat_chunked'))
         fn, mod, _ = self._compile(key, emit, in_args)
         trips = (n_out * n_red + threads * vec - 1) // (threads * vec)
-        grid = max(1, min(cus * _tuning.get('cols_target_blocks_per_cu'), trips // unroll))
+        grid = max(1, min(cus * _tuning.get('cols_flat_blocks_per_cu') * _cg.BLOCK // block,
+                          trips // unroll))
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)
         rsize = self._reduce_type_size(reduce_type, mod)
         partials, pref = self._alloc_partials(rec, rsize * grid * n_out)
         vals.ptr(pref, partials.ptr)
         _launch_plan.launch(
-            rec, fn, (grid, 1, 1), (_cg.BLOCK, 1, 1),
+            rec, fn, (grid, 1, 1), (block, 1, 1),
             _make_packer(self._fast_format(rargs, ic, 'P')), vals, stream_ptr)
         self._finalize_partials(
             partials, grid, out_args, out_arr_idx, n_out, so_out, in_args, reduce_expr,

@@ -87,13 +87,21 @@ _params = {
     # `cols_unroll_near` (64 x 64 x 16384, axis 1: 56.0 -> 47.8 us; 257 x 511 x
     # 509: 78.5 -> 60.6 us)
     'cols_unroll': 1,
-    # Narrow dense matrices whose rows take two column blocks or more (or, for
-    # one- and two-byte items, leave most lanes of one idle) are walked as one
-    # contiguous piece of memory when reduced down their columns, the columns
-    # a lane meets repeating from trip to trip.  'always': every width from 2
-    # to 256 whatever the column kernel would make of it (for tests).
+    # Narrow dense matrices (2 to 256 columns, except rows of whole vectors that
+    # fill a power-of-two group of lanes) are walked as one contiguous piece
+    # of memory when reduced down their columns, the columns a lane meets
+    # repeating from trip to trip.  'always': every width, whatever the column
+    # kernel would make of it (for tests).
     'cols_flat': True,
     'cols_flat_min_bytes': 1 << 20,
+    # ... every workgroup a run of consecutive trips (one contiguous piece of
+    # memory) rather than every grid-th trip, three workgroups per CU: main
+    # kernel over 2^26 float32 with 67 / 129 / 200 / 255 columns 41.7 / 40.7 /
+    # 39.5 / 40.5 us against 44.6 / 45.6 / 43.1 / 46.6 side by side with five
+    # (two per CU: 39.1 / 47.5 / 52.4 / 40.0 -- uneven)
+    'cols_flat_chunked': True,
+    'cols_flat_blocks_per_cu': 3,
+    'cols_flat_block': 0,       # threads of its workgroups (0: 256; 512 and 1024 measured slower)
     # Lanes across the columns of a workgroup, at most (the rest of its 256
     # threads goes down the reduce axis).  Sums over axis 0 of 16384^2 float32 /
     # 8192^2 float64, timed between other operations on other arrays: 161 / 84 us
