@@ -903,7 +903,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
               reduce_type, typedefs='', preamble='', tx=64, vec=4, idx64=False,
               partial_in=False, partial_out=False, stream_hint=False, unroll=4,
               solo=False, batched=False, clamp_tail=False, vec_out=False, solo_block=BLOCK,
-              finish=False, reduce_words=2):
+              finish=False, reduce_words=2, xcd=False):
     """Output-axis-contiguous kernel.  Thread layout: ``tx`` threads across
     the output axis (each owning ``vec`` adjacent outputs) times 256/tx slices
     of the reduce axis; gridDim.y further slices.  ``partial_in``: the single
@@ -962,6 +962,20 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         src.append('  unsigned _epoch0 = 0u;')
         src.append('  if (threadIdx.x == 0) _epoch0 = _sync_epoch(_sync);')
         by_expr, gy_expr = '_by', '_gy'
+    elif xcd:
+        # Workgroups are handed to the eight compute dies in turn (workgroup w
+        # of the grid, counted along x first, goes to die w % 8), and every die
+        # has a cache of its own.  Neighbouring column blocks share the cache
+        # line their border falls into whenever the rows do not start on line
+        # boundaries: numbered so that a die takes a run of consecutive column
+        # blocks, the line is fetched from memory once instead of once per die
+        # (grid.z is 1 here).
+        src.append('  const unsigned _lin = blockIdx.y * gridDim.x + blockIdx.x;')
+        src.append('  const unsigned _whole = (gridDim.x * gridDim.y) & ~7u;')
+        src.append('  const unsigned _turn = _lin < _whole ? (_lin & 7u) * (_whole >> 3) + (_lin >> 3) : _lin;')
+        src.append('  const %s _blk = (%s)(_turn %% gridDim.x);' % (idx_t, idx_t))
+        src.append('  const %s _by = (%s)(_turn / gridDim.x);' % (idx_t, idx_t))
+        by_expr, gy_expr = '_by', '(%s)gridDim.y' % idx_t
     else:
         # column blocks beyond the capacity of grid.x continue along grid.z
         src.append('  const %s _blk = (%s)blockIdx.z * gridDim.x + blockIdx.x;' % (idx_t, idx_t))
@@ -1149,7 +1163,7 @@ def emit_cols(name, args, identity, pre_map_expr, reduce_expr, post_map_expr,
         waves, tx, vec))
     src.append('      const %s _i = _i0 + _c + _k;' % idx_t)
     src.extend(_finish(args, 'publish' if finish else partial_out, '      ',
-                       split_expr='_by' if finish else 'blockIdx.y'))
+                       split_expr='_by' if (finish or xcd) else 'blockIdx.y'))
     src.append('    }')
     src.append('  }')
     if finish:

@@ -1037,10 +1037,15 @@ class _AbstractReductionKernel:
             unroll = _tuning.get('cols_unroll_near')
         stream_hint = _tuning.stream_policy(
             _tuning.get('cols_stream'), self._read_bytes(ins, n_out, n_red, so_in, sr), 0)[0]
+        # Column blocks numbered so that neighbours run on one compute die,
+        # where their borders do not fall on cache-line boundaries
+        mode = _tuning.get('cols_xcd')
+        xcd = bool(mode) and gz == 1 and not finish and gx > 1 and (mode is True or any(
+            s_r % 128 or a.data.ptr % 128 for a, s_r in zip(ins, sr)))
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
                stream_hint, solo, bool(batch), clamp, unroll, vec_out, block, bool(finish),
-               _tuning.signature())
+               xcd, _tuning.signature())
 
         def emit():
             return self.name, _cg.emit_cols(
@@ -1049,7 +1054,7 @@ class _AbstractReductionKernel:
                 idx64=idx64, partial_out=partial,
                 stream_hint=stream_hint, unroll=unroll, solo=solo,
                 batched=bool(batch), clamp_tail=clamp, vec_out=vec_out, solo_block=solo_block,
-                finish=bool(finish), reduce_words=words_hint)
+                finish=bool(finish), reduce_words=words_hint, xcd=xcd)
         fn, mod, _ = self._compile(key, emit, in_args)
         ic = 'q' if idx64 else 'i'
         vals = self._fast_values(in_args, out_args, n_out, n_red, so_in, sr, so_out)

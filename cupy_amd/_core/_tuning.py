@@ -120,6 +120,7 @@ _params = {
     # 155 / 183 us; 2^26 float64: 84 / 83 / 80 / 82 / 93
     'rows_target_blocks_per_cu': 2,
     'cols_unroll_near': 4,
+    'cols_xcd': 'auto',         # column blocks numbered die by die: 'auto' (rows off the cache lines), True, False
     'cols_solo_block': 1024,    # workgroup of the thread-per-column variant
     # Grid cap of the scan kernels, in workgroups per CU (cumsum along rows of
     # 1024 float32, 2^28 elements: 74.9 % of peak with 32, 80.2 % with 256)

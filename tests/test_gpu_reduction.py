@@ -588,3 +588,30 @@ def test_columns_of_a_narrow_matrix_use_the_flat_kernel_and_replay():
     # column kernel otherwise; both agree with NumPy
     assert_exact(d[4:].sum(axis=0).get(), h[4:].sum(axis=0))
     assert_exact(d[1:].sum(axis=0).get(), h[1:].sum(axis=0))
+
+
+@pytest.mark.parametrize('mode', ['auto', True, False])
+@pytest.mark.parametrize('shape,axis', [((1031, 4099), 0), ((7, 33, 1001), 1), ((300, 70001), 0),
+                                        ((4099, 16363), 0), ((64, 2048), 0), ((9, 65, 31277), 1),
+                                        ((5000, 129 * 8 + 4), 0)])
+def test_column_blocks_numbered_die_by_die(shape, axis, mode):
+    """Column reductions whose workgroups are renumbered so that neighbouring
+    column blocks run on one compute die (grids that are and are not a multiple
+    of eight workgroups, split and unsplit reduce axes, batches): every
+    workgroup still takes exactly one (column block, slice) pair."""
+    from cupy_amd._core import _tuning
+    _tuning.set(cols_xcd=mode)
+    try:
+        rng = np.random.default_rng(51)
+        h = rng.integers(-1000, 1000, shape).astype(np.int32)
+        d = cp.asarray(h)
+        assert_exact(d.sum(axis=axis).get(), h.sum(axis=axis))
+        assert_exact(d.argmax(axis=axis).get(), h.argmax(axis=axis))
+        assert_exact(d.min(axis=axis).get(), h.min(axis=axis))
+        hf = rng.standard_normal(shape).astype(np.float32)
+        got = cp.asarray(hf).sum(axis=axis).get()
+        want = hf.astype(np.float64).sum(axis=axis)
+        scale = np.abs(hf).astype(np.float64).sum(axis=axis)
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(scale, 1))
+    finally:
+        _tuning.set(cols_xcd='auto')
