@@ -559,10 +559,22 @@ def emit_rows2d(name, operands, operation, typedefs='', preamble='',
     return '\n'.join(src) + '\n'
 
 
+def _die_by_die(index, total, idx_t, enabled):
+    """Expression that renumbers work item ``index`` of ``total`` so that each
+    of the eight compute dies, which take the workgroups of a grid in turn
+    (workgroup w goes to die w % 8), works on a run of consecutive items: the
+    items whose borders share cache lines then meet in one die's cache.  The
+    last ``total % 8`` items keep their numbers."""
+    if not enabled:
+        return index
+    return ('((%s) < ((%s) & ~(%s)7) ? ((%s) & 7) * (((%s) & ~(%s)7) >> 3) + ((%s) >> 3) : (%s))'
+            % (index, total, idx_t, index, total, idx_t, index, index))
+
+
 def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
                  loop_prep='', after_loop='', layouts=None, vec=4, tile_r=64,
                  tile_c=64, threads=256, idx64=False, stream_hint=True, batched=False,
-                 batch_first=False, svec=None, flat_stage=0):
+                 batch_first=False, svec=None, flat_stage=0, xcd=False, strip=16):
     """Kernel for a 2-d index space (rows r, columns c) where every array
     operand is contiguous along one of the axes.
 
@@ -638,7 +650,8 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     src.append('  const %s _ntc = (_nc + %d) / %d;' % (idx_t, tile_c - 1, tile_c))
     if batched:
         src.append('  const %s _nt2 = _ntr * _ntc;' % idx_t)
-        src.append('  for (%s _tile_b = blockIdx.x; _tile_b < _nt2 * _nbt; _tile_b += gridDim.x) {' % idx_t)
+        src.append('  for (%s _tile_q = blockIdx.x; _tile_q < _nt2 * _nbt; _tile_q += gridDim.x) {' % idx_t)
+        src.append('    const %s _tile_b = %s;' % (idx_t, _die_by_die('_tile_q', '_nt2 * _nbt', idx_t, xcd)))
         if batch_first:
             # consecutive workgroups take the same tile of consecutive batch
             # entries: where those lie closer together in memory than the rows
@@ -654,15 +667,30 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
             src.append('    const ptrdiff_t _o_%s = (ptrdiff_t)_b0 * _sb0_%s + (ptrdiff_t)_b1 * _sb1_%s;' % (
                 op.name, op.name, op.name))
     else:
-        src.append('  for (%s _tile = blockIdx.x; _tile < _ntr * _ntc; _tile += gridDim.x) {' % idx_t)
+        src.append('  for (%s _tile_q = blockIdx.x; _tile_q < _ntr * _ntc; _tile_q += gridDim.x) {' % idx_t)
+        src.append('    const %s _tile = %s;' % (idx_t, _die_by_die('_tile_q', '_ntr * _ntc', idx_t, xcd)))
     # Diagonal tile order: consecutive workgroups differ in both the row block
     # and the column block.  With power-of-two pitches, walking along one axis
     # only would keep the low address bits of either the transposed reads or the
     # row-major accesses identical across all concurrently running workgroups,
     # and with them the memory channel.
-    src.append('    const %s _tr = _tile %% _ntr;' % idx_t)
-    src.append('    const %s _r0 = _tr * %d;' % (idx_t, tile_r))
-    src.append('    const %s _c0 = ((_tile / _ntr + _tr) %% _ntc) * %d;' % (idx_t, tile_c))
+    if xcd and not batched:
+        # Operands off the cache lines (odd pitches): neighbouring tiles share
+        # the lines at their borders, along the rows in one operand and along
+        # the columns in another.  A die walks strips `strip` tiles wide row by
+        # row, so that the tiles it works on at one time are neighbours both
+        # ways (odd pitches spread over the memory channels by themselves).
+        src.append('    const %s _strip = _tile / (_ntr * %d);' % (idx_t, strip))
+        src.append('    const %s _sw = (_ntc - _strip * %d < %d) ? (_ntc - _strip * %d) : %d;' % (
+            idx_t, strip, strip, strip, strip))
+        src.append('    const %s _sv = _tile - _strip * (_ntr * %d);' % (idx_t, strip))
+        src.append('    const %s _tr = _sv / _sw;' % idx_t)
+        src.append('    const %s _r0 = _tr * %d;' % (idx_t, tile_r))
+        src.append('    const %s _c0 = (_strip * %d + (_sv - _tr * _sw)) * %d;' % (idx_t, strip, tile_c))
+    else:
+        src.append('    const %s _tr = _tile %% _ntr;' % idx_t)
+        src.append('    const %s _r0 = _tr * %d;' % (idx_t, tile_r))
+        src.append('    const %s _c0 = ((_tile / _ntr + _tr) %% _ntc) * %d;' % (idx_t, tile_c))
     src.append('    const bool _interior = (_r0 + %d <= _nr) && (_c0 + %d <= _nc);' % (
         tile_r, tile_c))
     # Row-major inputs of an interior tile are requested first of all, for every

@@ -1099,9 +1099,16 @@ class _ElementwisePlanner:
         flat_stage = 0
         if narrow and nr <= 32 and tile_r == nr and svec == 1 and n_transposed:
             flat_stage = self._flat_stage_width(arrays, cstrides, names, layouts, nr)
+        # Tiles numbered so that neighbours run on one compute die, where
+        # their borders do not fall on cache-line boundaries
+        mode = _tuning.get('tiled_xcd')
+        xcd = bool(mode) and (mode is True or any(
+            a.data.ptr % 128 or max(abs(cs[0]), abs(cs[1])) % 128
+            for a, cs in zip(arrays, cstrides)))
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,
-               threads, bool(batch), batch_first, svec, flat_stage)
+               threads, bool(batch), batch_first, svec, flat_stage, xcd,
+               _tuning.get('tiled_xcd_strip'))
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
@@ -1110,7 +1117,8 @@ class _ElementwisePlanner:
                 self.loop_prep, self.after_loop, layouts=layouts, vec=vec,
                 tile_r=tile_r, tile_c=tile_c, threads=threads, idx64=idx64,
                 stream_hint=stream_hint, batched=bool(batch), batch_first=batch_first,
-                svec=svec, flat_stage=flat_stage)
+                svec=svec, flat_stage=flat_stage, xcd=xcd,
+                strip=_tuning.get('tiled_xcd_strip'))
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
             fmt = ['@']

@@ -57,6 +57,8 @@ _params = {
     'tiled_narrow': True,       # tiles as narrow as the array where an axis has at most 32 elements
     'tiled_unaligned': True,    # vectors whatever the alignment of rows and columns
     'tiled_tile': None,         # (rows, columns, threads) of a staged tile; None: by shape
+    'tiled_xcd': 'auto',        # tiles numbered die by die: 'auto' (operands off the cache lines), True, False
+    'tiled_xcd_strip': 16,      # ... a die walking strips of this many tiles across (transposed copy of 8191 x 8193 float32: 136 us in diagonal order, 116 / 110 / 108 / 105 / 118 with strips of 2 / 4 / 8 / 16 / 64)
     'tiled_big_min': 256,       # extent of both tile axes from which tiles are 128 x 128
     'cache_bytes': 256 << 20,   # capacity of the memory-side cache (Infinity Cache)
     # reductions

@@ -600,3 +600,33 @@ def test_orders_of_reshape_ravel_flatten_and_get(perm):
     part = d[1:, ::2]
     assert np.array_equal(part.get(order='F'), h[1:, ::2])
     assert part.get(order='F').flags.f_contiguous
+
+
+@pytest.mark.parametrize('mode,strip', [('auto', 16), (True, 16), (True, 3), (True, 64), (False, 16)])
+@pytest.mark.parametrize('shape', [(1031, 2053), (2049, 515), (127, 4099), (3001, 129), (1024, 1040)])
+def test_tiles_numbered_die_by_die(shape, mode, strip):
+    """Transposed operands whose rows do not start on cache lines: the tiles are
+    renumbered so that a compute die works on neighbouring ones (strips of
+    tiles, a last strip that is narrower, tile counts that are no multiple of
+    eight).  Every tile must still be visited exactly once."""
+    from cupy_amd._core import _tuning
+    _tuning.set(tiled_xcd=mode, tiled_xcd_strip=strip)
+    try:
+        rng = np.random.default_rng(61)
+        a = rng.integers(-1000, 1000, shape).astype(np.int32)
+        b = rng.integers(-1000, 1000, shape[::-1]).astype(np.int32)
+        da, db = cp.asarray(a), cp.asarray(b)
+        assert_exact(cp.ascontiguousarray(da.T).get(), np.ascontiguousarray(a.T))
+        assert_exact((da.T + db).get(), a.T + b)
+        out = cp.full(shape, -7, np.int32)
+        cp.add(db.T, da, out=out)
+        assert_exact(out.get(), b.T + a)
+        # a batch of such matrices
+        c = rng.integers(-1000, 1000, (5,) + shape[::-1]).astype(np.int32)[:, :301, :257]
+        dc = cp.asarray(c)
+        assert_exact(cp.ascontiguousarray(dc.transpose(0, 2, 1)).get(),
+                     np.ascontiguousarray(c.transpose(0, 2, 1)))
+        assert_exact(cp.ascontiguousarray(dc.transpose(2, 1, 0)).get(),
+                     np.ascontiguousarray(c.transpose(2, 1, 0)))
+    finally:
+        _tuning.set(tiled_xcd='auto', tiled_xcd_strip=16)
