@@ -1807,7 +1807,7 @@ def _module_chain_tile(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, inn
 
 
 def _emit_chain_cols(in_t, out_t, op, skip_nan, vec, trips, idx64, waves, stream, sleep,
-                     ahead=2):
+                     ahead=2, bands=False):
     """One-pass scan along the middle axis of (outer, n, inner) where the
     columns are many and long but too few to give every thread a column of its
     own: a workgroup per tile of WAVES x TRIPS rows by 64 x VEC columns.  A
@@ -1817,7 +1817,17 @@ def _emit_chain_cols(in_t, out_t, op, skip_nan, vec, trips, idx64, waves, stream
     fold those of the tiles above them as in ``_emit_chain`` (slots, waits and
     an order of combination fixed by the tile's number); tiles are numbered
     row of tiles by row of tiles, so that a tile only ever waits for smaller
-    numbers."""
+    numbers.
+
+    ``bands``: workgroups are handed to the eight compute dies in turn
+    (workgroup w goes to die w % 8, each die with a cache of its own), and
+    neighbouring tiles of a row of tiles share the cache lines at their borders
+    whenever the rows of the array do not start on line boundaries.  Workgroup
+    w then takes tile number w / 8 of band w % 8 of the columns (the column
+    blocks cut into eight runs), the band's tiles counted row of tiles by row
+    of tiles: a die works on neighbouring tiles, and a tile still only waits
+    for workgroups with smaller numbers (the tiles above it lie in its own
+    band, earlier in the band's count)."""
     acc_t = _acc_type(out_t)
     op_c = '+' if op == _SUM else '*'
     ident = '0' if op == _SUM else '1'
@@ -1843,6 +1853,7 @@ typedef %(idx_t)s _idx_t;
 #define HEADER_WORDS %(header)d
 #define SPIN_SLEEP %(sleep)d
 #define FOLD_AHEAD %(ahead)d
+#define BANDS %(bands)d
 __device__ __forceinline__ _acc_t _load_value(_in_t _x) { return %(conv)s; }
 
 // Published values: see the one-pass kernel for contiguous rows.  Value
@@ -1934,14 +1945,33 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
   _slot_t* group_totals = tile_totals + n_tiles * COLS_T * kWords;
   const int lane = threadIdx.x %% 64;
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+#if BANDS
+  const _idx_t band = (_idx_t)(blockIdx.x & 7u);
+  const ptrdiff_t seq = (ptrdiff_t)(blockIdx.x >> 3);
+  const _idx_t band_base = col_blocks / 8, band_rest = col_blocks %% 8;
+  const _idx_t band_width = band_base + (band < band_rest ? 1 : 0);
+  if (band_width == 0) return;
+  const _idx_t cb = band * band_base + (band < band_rest ? band : band_rest)
+                    + (_idx_t)(seq %% band_width);
+  const ptrdiff_t slab = seq / band_width;                   // (o, t_row)
+  if (slab >= (ptrdiff_t)n_outer * row_tiles) return;
+  const ptrdiff_t tile = slab * col_blocks + cb;
+#else
   const ptrdiff_t tile = blockIdx.x;
   if (tile >= n_tiles) return;
   const _idx_t cb = (_idx_t)(tile %% col_blocks);
   const ptrdiff_t slab = tile / col_blocks;                  // (o, t_row)
+#endif
   const _idx_t t_row = (_idx_t)(slab %% row_tiles);
   const _idx_t o = (_idx_t)(slab / row_tiles);
   const int lc = lane * VEC;                     // the lane's first column within the block
-  const bool has_cols = cb * COLS_T + lc < inner;            // the host guarantees inner %% VEC == 0
+  const bool has_cols = cb * COLS_T + lc < inner;
+  // A vector that would pass the end of the rows (their length is no multiple
+  // of VEC) starts VEC columns before the end instead and overlaps its
+  // neighbour's: both lanes compute and store the same values for the shared
+  // column (never in place: the host sees to that).  In the LDS and in the
+  // slots the lane keeps its own places.
+  const int lm = (VEC > 1 && cb * COLS_T + lc + VEC > inner) ? (int)(inner - VEC - cb * COLS_T) : lc;
   const _idx_t r0 = t_row * TILE_ROWS + wv * TRIPS;          // this wave's first row
   // (the same for all lanes of a wave: the lanes differ by `lc` alone)
   const ptrdiff_t at0 = ((ptrdiff_t)o * n + r0) * inner + (ptrdiff_t)cb * COLS_T;
@@ -1950,7 +1980,7 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
 #pragma unroll
   for (int t = 0; t < TRIPS; ++t) {
     if (has_cols && r0 + t < n) {
-      raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + at0 + (ptrdiff_t)t * inner + lc);
+      raw[t] = cupy::load_vec<_in_t, VEC, NT_LOAD>(in + at0 + (ptrdiff_t)t * inner + lm);
     } else {
 #pragma unroll
       for (int k = 0; k < VEC; ++k) raw[t].v[k] = _in_t();
@@ -2052,27 +2082,28 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain_cols(
         run[k] = (seeded || t > 0) ? SCAN_OP(run[k], x) : x;
         r.v[k] = static_cast<_out_t>(run[k]);
       }
-      cupy::store_vec<_out_t, VEC, NT_STORE>(out + at0 + (ptrdiff_t)t * inner + lc, r);
+      cupy::store_vec<_out_t, VEC, NT_STORE>(out + at0 + (ptrdiff_t)t * inner + lm, r);
     }
   }
 }
 """ % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t='ptrdiff_t' if idx64 else 'int',
            op_c=op_c, ident=ident, start=_start_text(op, acc_t), vec=vec, trips=trips, conv=conv, block=waves * _WAVE,
-           waves=waves, header=_CHAIN_HEADER_WORDS, sleep=sleep, ahead=ahead,
+           waves=waves, header=_CHAIN_HEADER_WORDS, sleep=sleep, ahead=ahead, bands=1 if bands else 0,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false')
 
 
-def _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, waves, stream):
+def _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, waves, stream,
+                       bands=False):
     sleep = _tuning.get('scan_chain_sleep')
     key = ('chain cols', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan,
-           vec, trips, idx64, waves, stream, sleep)
+           vec, trips, idx64, waves, stream, sleep, bands)
     mod = _memo.get(key)
     if mod is None:
         # published totals a lane asks for at a time: what the registers of
         # a lane in a workgroup of 16 waves hold beside its rows
         ahead = 4 if (in_dtype.itemsize == 4 and _acc_dtype(out_dtype).itemsize * vec <= 8) else 2
         src = _emit_chain_cols(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
-                               vec, trips, idx64, waves, stream, sleep, ahead)
+                               vec, trips, idx64, waves, stream, sleep, ahead, bands)
         mod = compiler.compile_with_cache(src)
         with _lock:
             mod = _memo.setdefault(key, mod)
@@ -2288,6 +2319,13 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
     return True
 
 
+def _may_overlap(src, dst):
+    """True if a scan from ``src`` into ``dst`` may read what it has written
+    (in place, or views of one allocation whose byte ranges meet)."""
+    from cupy_amd._core._carray import may_share_bounds
+    return may_share_bounds(src, dst)
+
+
 def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr):
     """The one-pass scan down many long columns (``_emit_chain_cols``).  Returns
     False where it does not apply."""
@@ -2315,9 +2353,15 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
         # (two columns a lane at most: every column has its running values and
         # its share of the look-back in registers)
         v = max(1, min(2, vec_bytes // item))
-        while v > 1 and (not _aligned(src.data.ptr, v * in_dtype.itemsize)
-                         or not _aligned(dst.data.ptr, v * out_dtype.itemsize)
-                         or inner % v):
+        # (rows of any length and arrays aligned for one element keep their
+        # vectors where wide accesses need no more than that: the last vector
+        # of a row then overlaps its neighbour, which in place would let one
+        # lane read what another has already written)
+        loose = (_tuning.get('unaligned_vectors') and _tuning.get('scan_chain_cols_unaligned')
+                 and inner >= 2 * v and not _may_overlap(src, dst))
+        while v > 1 and not loose and (
+                not _aligned(src.data.ptr, v * in_dtype.itemsize)
+                or not _aligned(dst.data.ptr, v * out_dtype.itemsize) or inner % v):
             v //= 2
         cols_t = _WAVE * v
         blocks = (inner + cols_t - 1) // cols_t
@@ -2342,14 +2386,25 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
     desc_words = _CHAIN_HEADER_WORDS + 2 * words_per_value * _WAVE * vec * (n_tiles + n_groups)
     if desc_words > 0x7fffffff:
         return False
-    mod = _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, waves, stream)
+    # Rows off the cache lines: tiles numbered band by band (see the kernel)
+    mode = _tuning.get('scan_chain_cols_xcd')
+    bands = bool(mode) and col_blocks >= 32 and (
+        mode is True or (inner * in_dtype.itemsize) % 128 != 0 or src.data.ptr % 128 != 0
+        or (inner * out_dtype.itemsize) % 128 != 0 or dst.data.ptr % 128 != 0)
+    launched = n_tiles
+    if bands:
+        launched = 8 * outer * row_tiles * ((col_blocks + 7) // 8)
+        if launched * waves * _WAVE > 0xffffffff:
+            bands, launched = False, n_tiles
+    mod = _module_chain_cols(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, waves, stream,
+                             bands)
     desc, epoch = _chain_slots(dev_id, stream_ptr, desc_words, mod)
     ic = 'q' if idx64 else 'i'
     blob = struct.pack('@PPP' + ic * 7 + 'IIP', src.data.ptr, dst.data.ptr, desc.data.ptr,
                        outer, n, inner, col_blocks, row_tiles, group_tiles, groups_per_col,
                        epoch, _tuning.get('scan_chain_spin_limit'), fault)
     mod.get_function('cupy_scan_chain_cols').launch_packed(
-        (n_tiles, 1, 1), (waves * _WAVE, 1, 1), blob, 0, stream_ptr)
+        (launched, 1, 1), (waves * _WAVE, 1, 1), blob, 0, stream_ptr)
     return True
 
 

@@ -16,7 +16,8 @@ def _restore():
     yield
     _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0,
                 scan_chain_cols=True, scan_chain_cols_waves=16, scan_chain_cols_trips=0,
-                scan_chain_cols_vec_bytes=0)
+                scan_chain_cols_vec_bytes=0, scan_chain_cols_xcd='auto',
+                scan_chain_cols_unaligned=True)
     _giveup.disabled[_giveup.SCAN].clear()
 
 
@@ -240,7 +241,10 @@ def within(got, want, bound):
     ((3, 3001, 516), 1),          # several slices
     ((70001, 100), 0),            # many tiles down a column, the last block of columns part empty
     ((1029, 4098), 0),            # the last tile holds few rows
-    ((40000, 37), 0),             # odd row length: single-element vectors
+    ((40000, 37), 0),             # odd row length: the last vector of a row overlaps its neighbour
+    ((9001, 2113), 0),            # ... with enough blocks of columns for a band per compute die
+    ((2, 5003, 2051), 1),
+    ((20001, 65), 0),             # ... a block of columns with a single column
 ])
 def test_many_long_columns_in_one_pass(shape, axis):
     rng = np.random.default_rng(shape[-1])
@@ -248,6 +252,16 @@ def test_many_long_columns_in_one_pass(shape, axis):
     d = cp.asarray(h)
     assert launched(lambda: d.cumsum(axis=axis))[-1] == 'cupy_scan_chain_cols'
     assert_exact(d.cumsum(axis=axis).get(), h.cumsum(axis=axis))
+    # in place (no overlapping vectors then), and with the bands and the
+    # overlapping vectors switched off
+    e = d.copy()
+    cp.cumsum(e, axis=axis, out=e)
+    assert_exact(e.get(), h.cumsum(axis=axis, dtype=np.int32))
+    _tuning.set(scan_chain_cols_xcd=False, scan_chain_cols_unaligned=False)
+    assert_exact(d.cumsum(axis=axis).get(), h.cumsum(axis=axis))
+    _tuning.set(scan_chain_cols_xcd=True, scan_chain_cols_unaligned=True)
+    assert_exact(d.cumsum(axis=axis).get(), h.cumsum(axis=axis))
+    _tuning.set(scan_chain_cols_xcd='auto')
     hf = rng.uniform(0, 1, shape).astype(np.float32)
     df = cp.asarray(hf)
     got = df.cumsum(axis=axis).get()
