@@ -2371,8 +2371,14 @@ def _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64, stream, s
     _, vec, col_blocks = best
     waves = max(2, min(16, _tuning.get('scan_chain_cols_waves')))
     # (values narrower than a register are unpacked: fewer rows then)
-    trips = _tuning.get('scan_chain_cols_trips') or max(4, min(
-        64 if item >= 4 else 32, (256 if item < 16 else 128) // (vec * item)))
+    trips = _tuning.get('scan_chain_cols_trips')
+    if not trips:
+        trips = max(4, min(64 if item >= 4 else 32, (256 if item < 16 else 128) // (vec * item)))
+        # (columns of a few hundred rows: shorter tiles, so that there are at
+        # least two down a column; 257 slices of 511 x 509 float32: 137 us with
+        # 16 rows a lane, 149 with 8, 204 with 4)
+        while trips > 16 and n < 2 * waves * trips:
+            trips //= 2
     tile_rows = waves * trips
     row_tiles = (n + tile_rows - 1) // tile_rows
     n_tiles = outer * row_tiles * col_blocks
@@ -2683,8 +2689,17 @@ def _scan_contiguous(src, dst, outer, n, inner, op, skip_nan, stream_ptr, may_ch
         n_chunks = 1
         if may_chunk and not one_pass_trips and threads < want and n >= 128:
             n_chunks = min((want + threads - 1) // threads, n // 64)
-        if n_chunks > 1 and _scan_chained_cols(src, dst, outer, n, inner, op, skip_nan, idx64,
-                                               stream, stream_ptr):
+        # (slices with too few columns for wide vectors and rows that start off
+        # the vectors' grid: the tiles of the one-pass kernel, with their
+        # overlapping vectors, do better than a thread per column with single
+        # elements; 257 slices of 511 x 509 float32: 232 -> 137 us, 64 of
+        # 1024 x 1025: 160 -> 151.  With aligned rows the thread per column
+        # wins: 128 slices of 512 x 1024 87 against 106)
+        narrow_one_pass = (one_pass_trips == 64 and not forced and inner >= 128 and n >= 256
+                           and outer >= 2 and (inner * item) % 16 != 0
+                           and _tuning.get('scan_chain_cols_short'))
+        if (n_chunks > 1 or narrow_one_pass) and _scan_chained_cols(
+                src, dst, outer, n, inner, op, skip_nan, idx64, stream, stream_ptr):
             return
         chunk_len = (n + n_chunks - 1) // n_chunks
         n_chunks = (n + chunk_len - 1) // chunk_len

@@ -147,6 +147,7 @@ _params = {
     'scan_chain_cols': True,    # one-pass kernel for many long columns
     'scan_chain_cols_xcd': 'auto',   # tiles numbered band by band of the columns, a band per compute die: 'auto' (rows off the cache lines), True, False
     'scan_chain_cols_unaligned': True,   # 8-byte vectors whatever the length and alignment of the rows (not in place)
+    'scan_chain_cols_short': True,   # ... also for columns of a few hundred rows where a thread per column would take single elements
     'scan_chain_cols_waves': 16,
     'scan_chain_cols_trips': 0,
     'scan_chain_cols_vec_bytes': 0,

@@ -17,7 +17,7 @@ def _restore():
     _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0,
                 scan_chain_cols=True, scan_chain_cols_waves=16, scan_chain_cols_trips=0,
                 scan_chain_cols_vec_bytes=0, scan_chain_cols_xcd='auto',
-                scan_chain_cols_unaligned=True)
+                scan_chain_cols_unaligned=True, scan_chain_cols_short=True)
     _giveup.disabled[_giveup.SCAN].clear()
 
 
@@ -245,6 +245,7 @@ def within(got, want, bound):
     ((9001, 2113), 0),            # ... with enough blocks of columns for a band per compute die
     ((2, 5003, 2051), 1),
     ((20001, 65), 0),             # ... a block of columns with a single column
+    ((130, 511, 509), 1),         # slices of a few hundred odd rows: tiles of 256 rows
 ])
 def test_many_long_columns_in_one_pass(shape, axis):
     rng = np.random.default_rng(shape[-1])
