@@ -1288,15 +1288,9 @@ __device__ __forceinline__ _acc_t _part_scan(
 #pragma unroll
   for (int t = 0; t < TRIPS; ++t) {
     const _idx_t j = j0 + (t * WAVE + lane) * VEC;
-    if (RAGGED && VEC > 1 && j + VEC > j1) {
 #pragma unroll
-      for (int k = 0; k < VEC; ++k)
-        v[t][k] = (j + k < j1) ? _load_value(src[j + k]) : SCAN_IDENTITY;
-    } else {
-#pragma unroll
-      for (int k = 0; k < VEC; ++k)
-        v[t][k] = ((RAGGED ? j + k : j) < j1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
-    }
+    for (int k = 0; k < VEC; ++k)
+      v[t][k] = (j < j1) ? _load_value(raw[t].v[k]) : SCAN_IDENTITY;
 #pragma unroll
     for (int k = 1; k < VEC; ++k) v[t][k] = SCAN_OP(v[t][k - 1], v[t][k]);
   }
@@ -1335,16 +1329,13 @@ __device__ __forceinline__ void _part_store(
     const _acc_t before = has_base ? (has_pre ? SCAN_OP(base, pre[t]) : base) : pre[t];
     const bool any = has_base || has_pre;
     _out_t* dst = row_out + j;
-    if (VEC > 1 && (RAGGED ? j + VEC <= j1 : j < j1)) {
+    if (j < j1) {
       cupy::Vec<_out_t, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k)
         r.v[k] = static_cast<_out_t>(any ? SCAN_OP(before, v[t][k]) : v[t][k]);
-      cupy::store_vec<_out_t, VEC, NT_STORE>(dst, r);
-    } else if (RAGGED || VEC == 1) {
-#pragma unroll
-      for (int k = 0; k < VEC; ++k)
-        if (j + k < j1) dst[k] = static_cast<_out_t>(any ? SCAN_OP(before, v[t][k]) : v[t][k]);
+      if (VEC > 1) cupy::store_vec<_out_t, VEC, NT_STORE>(dst, r);
+      else dst[0] = r.v[0];
     }
   }
 }
@@ -1363,7 +1354,7 @@ __device__ __forceinline__ void _part_store(
 // has nothing in flight, so what it holds in registers meanwhile is what
 // keeps the memory system busy: the first part is held scanned, the others as
 // loaded (they are scanned twice: once for their total, once for the result).
-extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain(
+extern "C" __global__ void __launch_bounds__(%(block)d) %(occupancy)s cupy_scan_chain(
     const _in_t* __restrict__ in, _out_t* __restrict__ out, unsigned* desc,
     const _idx_t n_rows, const _idx_t n, const _idx_t tiles_per_row, const _idx_t group_tiles,
     const _idx_t groups_per_row, const unsigned epoch, const unsigned spin_limit,
@@ -1375,7 +1366,8 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain(
   _slot_t* group_totals = tile_totals + n_tiles * kWords;
   const int lane = threadIdx.x %% WAVE;
   const int wv = threadIdx.x / WAVE;
-  const _idx_t j1 = n;
+  const _idx_t jn = n;
+  const _idx_t j1 = RAGGED ? n - n %% VEC : n;           // the whole vectors of a row end here
   const ptrdiff_t tile = blockIdx.x;
   if (tile >= n_tiles) return;
   const _idx_t row = (_idx_t)(tile / tiles_per_row);
@@ -1452,10 +1444,27 @@ extern "C" __global__ void __launch_bounds__(%(block)d) cupy_scan_chain(
     (void)_part_scan(raw[p], src, j0 + p * PART_ELEMS, j1, lane, v, pre);
     _part_store(row_out, j0 + p * PART_ELEMS, j1, lane, v, pre, base, has_base);
   }
+  // A row whose length is no whole number of vectors ends up to VEC - 1
+  // elements after its last whole vector: the lane that has just stored that
+  // vector goes on through them, one element after the other, from the result
+  // it stored last.  (No tile's total needs them: nothing of the row follows.
+  // Nothing is carried through the loops above for this: a register more
+  // than 128 per lane would halve the workgroups a CU holds.)
+  if (RAGGED) {
+    const _idx_t rel = j1 - VEC - j0;                 // the last whole vector, within this wave's share
+    if (rel >= 0 && rel < WAVE_ELEMS && (int)((rel / VEC) %% WAVE) == lane) {
+      _acc_t a = static_cast<_acc_t>(row_out[j1 - 1]);
+      for (_idx_t i = j1; i < jn; ++i) {
+        a = SCAN_OP(a, _load_value(src[i]));
+        row_out[i] = static_cast<_out_t>(a);
+      }
+    }
+  }
 }
 ''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident, start=_start_text(op, acc_t),
            vec=vec, trips=trips, conv=conv, block=waves * _WAVE, waves=waves,
            header=_CHAIN_HEADER_WORDS, parts=parts, sleep=_tuning.get('scan_chain_sleep'),
+           occupancy='',
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
            ragged=1 if ragged else 0)
 
