@@ -1133,7 +1133,8 @@ _CHAIN_WAVES = _BLOCK // _WAVE
 _CHAIN_HEADER_WORDS = 64            # the ticket counter, padded to 256 bytes
 
 
-def _emit_chain(in_t, out_t, op, skip_nan, vec, trips, idx64, stream, ragged, parts=2, waves=_CHAIN_WAVES):
+def _emit_chain(in_t, out_t, op, skip_nan, vec, trips, idx64, stream, ragged, parts=2, waves=_CHAIN_WAVES,
+                bands=False):
     """One-pass scan of long rows: a workgroup per tile of 256 x VEC x TRIPS
     elements scans its tile in registers, publishes the tile's total and adds
     up the totals published by the tiles before it: the input is read once and
@@ -1173,6 +1174,7 @@ typedef %(idx_t)s _idx_t;
 #define NT_LOAD %(ntl)s
 #define NT_STORE %(nts)s
 #define RAGGED %(ragged)d
+#define BANDS %(bands)d
 #define WAVE 64
 #define WAVES %(waves)d
 #define PARTS %(parts)d
@@ -1368,10 +1370,26 @@ extern "C" __global__ void __launch_bounds__(%(block)d) %(occupancy)s cupy_scan_
   const int wv = threadIdx.x / WAVE;
   const _idx_t jn = n;
   const _idx_t j1 = RAGGED ? n - n %% VEC : n;           // the whole vectors of a row end here
+#if BANDS
+  // Workgroups are handed to the eight compute dies in turn (workgroup w goes
+  // to die w %% 8, each die with a cache of its own), and neighbouring tiles of
+  // a row share the cache lines at their borders when the rows do not start on
+  // line boundaries.  Workgroup w takes tile number w / 8 of the rows r with
+  // r %% 8 == w %% 8, counted row by row: a die works its way along whole rows,
+  // and a tile still only waits for workgroups with smaller numbers (the
+  // tiles before it in its row).
+  const _idx_t band = (_idx_t)(blockIdx.x & 7u);
+  const ptrdiff_t seq = (ptrdiff_t)(blockIdx.x >> 3);
+  const _idx_t row = (_idx_t)(seq / tiles_per_row) * 8 + band;
+  if (row >= n_rows) return;
+  const _idx_t t_row = (_idx_t)(seq %% tiles_per_row);
+  const ptrdiff_t tile = (ptrdiff_t)row * tiles_per_row + t_row;
+#else
   const ptrdiff_t tile = blockIdx.x;
   if (tile >= n_tiles) return;
   const _idx_t row = (_idx_t)(tile / tiles_per_row);
   const _idx_t t_row = (_idx_t)(tile - (ptrdiff_t)row * tiles_per_row);
+#endif
   const _in_t* src = in + (ptrdiff_t)row * n;
   _out_t* row_out = out + (ptrdiff_t)row * n;
   const _idx_t j0 = t_row * TILE + wv * WAVE_ELEMS;        // this wave's share of the tile
@@ -1464,19 +1482,19 @@ extern "C" __global__ void __launch_bounds__(%(block)d) %(occupancy)s cupy_scan_
 ''' % dict(in_t=in_t, out_t=out_t, acc_t=acc_t, idx_t=idx_t, op_c=op_c, ident=ident, start=_start_text(op, acc_t),
            vec=vec, trips=trips, conv=conv, block=waves * _WAVE, waves=waves,
            header=_CHAIN_HEADER_WORDS, parts=parts, sleep=_tuning.get('scan_chain_sleep'),
-           occupancy='',
+           occupancy='', bands=1 if bands else 0,
            ntl='true' if stream[0] else 'false', nts='true' if stream[1] else 'false',
            ragged=1 if ragged else 0)
 
 
 def _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream, ragged, parts,
-                  waves=_CHAIN_WAVES):
+                  waves=_CHAIN_WAVES, bands=False):
     key = ('chain', _device.get_device_id(), in_dtype.char, out_dtype.char, op, skip_nan, vec,
-           trips, idx64, stream, ragged, parts, waves, _tuning.get('scan_chain_sleep'))
+           trips, idx64, stream, ragged, parts, waves, _tuning.get('scan_chain_sleep'), bands)
     mod = _memo.get(key)
     if mod is None:
         src = _emit_chain(_get_typename(in_dtype), _get_typename(out_dtype), op, skip_nan,
-                          vec, trips, idx64, stream, ragged, parts, waves)
+                          vec, trips, idx64, stream, ragged, parts, waves, bands)
         mod = compiler.compile_with_cache(src)
         with _lock:
             mod = _memo.setdefault(key, mod)
@@ -2315,9 +2333,23 @@ def _scan_chained(src, dst, n_rows, n, op, skip_nan, vec, idx64, stream, stream_
                                  stream, parts)
         name = 'cupy_scan_chain_tile'
     else:
+        # Rows off the cache lines, enough of them for every die, two tiles to
+        # a row: a die per row (8192 rows of 8191 float32: 101 -> 95 us; rows of
+        # many tiles lose, their tiles wait for each other on one die: 1024 rows
+        # of 65537 102 -> 131)
+        mode = _tuning.get('scan_chain_xcd')
+        bands = bool(mode) and n_rows >= 64 and tiles_per_row == 2 and (
+            mode is True or (n * in_dtype.itemsize) % 128 != 0 or src.data.ptr % 128 != 0
+            or (n * out_dtype.itemsize) % 128 != 0 or dst.data.ptr % 128 != 0)
+        if bands:
+            launched = 8 * ((n_rows + 7) // 8) * tiles_per_row
+            if launched * waves * _WAVE > 0xffffffff:
+                bands = False
         mod = _module_chain(in_dtype, out_dtype, op, skip_nan, vec, trips, idx64, stream,
-                            n % vec != 0, parts, waves)
+                            n % vec != 0, parts, waves, bands)
         name = 'cupy_scan_chain'
+        if bands:
+            n_tiles = launched
     desc, epoch = _chain_slots(dev_id, stream_ptr, desc_words, mod)
     ic = 'q' if idx64 else 'i'
     blob = struct.pack('@PPP' + ic * 5 + 'IIP', src.data.ptr, dst.data.ptr, desc.data.ptr,

@@ -158,6 +158,7 @@ _params = {
     # rows of 8192 104 -> 91 us, rows of 4096 98 -> 87; rows of 2048 stay with
     # the wave, 89 us)
     'scan_chain_min_row_bytes': 16384,
+    'scan_chain_xcd': 'auto',   # rows of the one-pass row scan dealt out die by die: 'auto' (rows off the cache lines), True, False
     'scan_chain': True,         # a few long rows: one pass, tiles chained through published totals
     # ... with this many waves per tile, each lane keeping fewer vectors for the
     # same tile (2^26 float32 in one row, 128 KiB tiles: 4 waves x 8 parts 102 us,

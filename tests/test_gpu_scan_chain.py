@@ -17,7 +17,8 @@ def _restore():
     _tuning.set(scan_chain=True, scan_chain_spin_limit=1 << 18, scan_chain_parts=0,
                 scan_chain_cols=True, scan_chain_cols_waves=16, scan_chain_cols_trips=0,
                 scan_chain_cols_vec_bytes=0, scan_chain_cols_xcd='auto',
-                scan_chain_cols_unaligned=True, scan_chain_cols_short=True)
+                scan_chain_cols_unaligned=True, scan_chain_cols_short=True,
+                scan_chain_xcd='auto')
     _giveup.disabled[_giveup.SCAN].clear()
 
 
@@ -103,6 +104,23 @@ def test_every_tile_size_and_many_launches_on_one_stream(parts):
             got = d.cumsum()
         stream.synchronize()
         assert_exact(got.get(), h.cumsum())
+
+
+@pytest.mark.parametrize('mode', ['auto', True, False])
+@pytest.mark.parametrize('shape', [(300, 8191), (67, 8190), (1000, 6001)])
+def test_rows_dealt_out_die_by_die(shape, mode):
+    """Rows of two tiles that do not start on cache lines: every compute die
+    takes whole rows (row counts that are no multiple of eight leave some
+    workgroups without a row)."""
+    _tuning.set(scan_chain_xcd=mode)
+    rng = np.random.default_rng(shape[1])
+    h = rng.integers(-5, 6, shape).astype(np.int32)
+    d = cp.asarray(h)
+    assert 'cupy_scan_chain' in launched(lambda: d.cumsum(axis=1))
+    assert_exact(d.cumsum(axis=1).get(), h.cumsum(axis=1))
+    e = d.copy()
+    cp.cumsum(e, axis=1, out=e)
+    assert_exact(e.get(), h.cumsum(axis=1, dtype=np.int32))
 
 
 def test_few_long_rows_products_and_nans():
