@@ -435,6 +435,24 @@ def build_layout_cases(cp):
     add('fused softmax f32 (2^26/100)x100', 2 * a100.nbytes, run('sm100', lambda: softmax(d100)),
         cpu_softmax, lambda: close(res['sm100'], cpu_softmax().astype(np.float64), 1e-5, 1.0),
         'softmax_rows_of_100')
+    # ---- rows that do not start on cache lines: neighbouring workgroups share lines -----------
+    odd = flat[:8191 * 8193].reshape(8191, 8193)
+    dodd = dflat[:8191 * 8193].reshape(8191, 8193)
+    add('transposed copy f32 8191x8193', 2 * odd.nbytes, run('oddT', lambda: cp.ascontiguousarray(dodd.T)),
+        lambda: np.ascontiguousarray(odd.T), lambda: same(res['oddT'], np.ascontiguousarray(odd.T)),
+        'cupy_copy')
+    add('sum f32 8191x8193 axis=0', odd.nbytes + 4 * 8193, run('oddS', lambda: dodd.sum(axis=0)),
+        lambda: odd.sum(axis=0),
+        lambda: close(res['oddS'], odd.sum(axis=0, dtype=np.float64), 1e-5,
+                      np.abs(odd).sum(axis=0, dtype=np.float64)), 'cupy_sum')
+    add('cumsum f32 8191x8193 axis=0', 2 * odd.nbytes, run('oddC', lambda: cp.cumsum(dodd, axis=0)),
+        lambda: np.cumsum(odd, axis=0),
+        lambda: close(res['oddC'], np.cumsum(odd, axis=0, dtype=np.float64), 1e-5,
+                      np.cumsum(np.abs(odd), axis=0, dtype=np.float64)), 'cupy_scan_chain_cols')
+    add('cumsum f32 2^26 - 1 axis=0 (no whole number of vectors)', 2 * 4 * (n - 1),
+        run('odd1', lambda: cp.cumsum(dflat[:n - 1])), lambda: np.cumsum(flat[:n - 1]),
+        lambda: close(res['odd1'], np.cumsum(flat[:n - 1], dtype=np.float64), 1e-5,
+                      np.cumsum(np.abs(flat[:n - 1]), dtype=np.float64)), 'cupy_scan_chain')
     return cases
 
 
