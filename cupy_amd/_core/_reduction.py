@@ -984,8 +984,13 @@ class _AbstractReductionKernel:
         # narrower workgroups where the reduce axis will be split (few column
         # blocks for the device); with column blocks in plenty 64 lanes across
         # do better (sum of 33 x 65 x 31277 over its middle axis: 46 us against 51)
+        # (rows that do not start on cache lines: a column block of 64 lanes
+        # has 9 lines to fetch per row where it would have 8, one of 32 lanes 5
+        # for 4; sum over axis 0 of 8191 x 8193 float32 50.7 -> 47.6 us, of
+        # 4099 x 16363 48.6 -> 45.5)
+        off_lines = any(s_r % 128 or a.data.ptr % 128 for a, s_r in zip(ins, sr))
         tx = 64
-        if (n_cols + 64 * vec - 1) // (64 * vec) * n_batch < cus * _tuning.get(
+        if not off_lines and (n_cols + 64 * vec - 1) // (64 * vec) * n_batch < cus * _tuning.get(
                 'cols_target_blocks_per_cu'):
             tx = _tuning.get('cols_tx')
         tx = max(1, min(tx, internal.clp2((n_cols + vec - 1) // vec)))
@@ -1040,8 +1045,7 @@ class _AbstractReductionKernel:
         # Column blocks numbered so that neighbours run on one compute die,
         # where their borders do not fall on cache-line boundaries
         mode = _tuning.get('cols_xcd')
-        xcd = bool(mode) and gz == 1 and not finish and gx > 1 and (mode is True or any(
-            s_r % 128 or a.data.ptr % 128 for a, s_r in zip(ins, sr)))
+        xcd = bool(mode) and gz == 1 and not finish and gx > 1 and (mode is True or off_lines)
         key = ('cols', tuple(r.key() for r in rargs), typedefs, map_expr, reduce_expr,
                post_map_expr, reduce_type, tx, vec, idx64, partial, device_id,
                stream_hint, solo, bool(batch), clamp, unroll, vec_out, block, bool(finish),
