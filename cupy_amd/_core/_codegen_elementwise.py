@@ -899,3 +899,286 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
     src.append('  %s;' % after_loop)
     src.append('}')
     return '\n'.join(src) + '\n'
+
+
+def emit_packed(name, operands, operation, typedefs='', preamble='',
+                loop_prep='', after_loop='', tile=(), in_order=(), staged=(),
+                zero_last=(), vec=1, svec=1, group=1, unit_first=True, threads=256,
+                idx64=False, stream_hint=True, xcd=False, tile_order=None):
+    """Kernel for an index space of ``len(tile)`` axes whose arrays are
+    permuted differently, with a tile that spans SEVERAL axes: as many of the
+    last axes as give the outputs a long contiguous run, and as many of the
+    axes the ``staged`` inputs run fastest along (``in_order``, fastest first)
+    as give those a long run too.  Small trailing axes -- a (B, 4, 3) array
+    copied as (B, 3, 4), pairs or quadruples kept together under a
+    permutation of the leading axes -- are then part of every tile instead of
+    being its edges.
+
+    A workgroup takes a tile in two passes.  First it reads the staged inputs in
+    THEIR order, ``svec`` elements per access, and puts
+    them into an LDS image of the tile that is laid out in the order of the
+    outputs (padded so that lanes side by side spread over the banks).  Then it goes through the tile in
+    the order of the outputs, ``vec`` elements per access along the last axis:
+    the other arrays (unit stride along the last axis, or zero for the inputs
+    named in ``zero_last``; any stride along the others) come straight from
+    memory, the staged ones from the image.
+
+    ``group``: how many of the first axes of ``in_order`` lie in the staged
+    inputs as ONE contiguous piece within a tile (each but the last of them
+    spanned whole, each starting where the one before ends): the accesses of
+    ``svec`` elements then run over that piece as a whole, whatever the extents
+    of its axes, and every element finds its own place in the image.
+    ``unit_first``: every staged input has unit stride along ``in_order[0]``
+    (else ``svec`` and ``group`` are 1 and the stride is applied).
+
+    ``tile[a]`` elements along axis a; tiles are numbered along the axes of
+    ``tile_order``, fastest first (default: the order of the outputs; ``xcd``:
+    die by die, see ``_die_by_die``).  Kernel parameters after the operands: the extents ``_e<a>``, then
+    per array its strides ``_s<a>_<name>`` in elements.  The element index ``i``
+    and the indexer are not available.
+    """
+    nd = len(tile)
+    idx_t = 'ptrdiff_t' if idx64 else 'int'
+    arrays = [op for op in operands if op.kind == 'array']
+    assert not any(op.kind == 'indexer' for op in operands)
+    _nt_l, _nt_s = stream_hint if isinstance(stream_hint, tuple) else (stream_hint, stream_hint)
+    ntl = 'true' if _nt_l else 'false'
+    nts = 'true' if _nt_s else 'false'
+    s_ops = [op for op in arrays if op.name in staged]
+    d_ops = [op for op in arrays if op.name not in staged]
+    for op in s_ops:
+        assert not op.is_out
+    volume = 1
+    for t in tile:
+        volume *= t
+    last = nd - 1
+    assert tile[last] % vec == 0
+    # position of an element in the image: its number in the order of the outputs
+    lds_step = [1] * nd
+    for a in range(nd - 2, -1, -1):
+        lds_step[a] = lds_step[a + 1] * tile[a + 1]
+    # Lanes side by side in the first pass are ``quantum`` words apart in the
+    # image (the step of the axis they differ in): a step that is a multiple of
+    # eight gets one pad word per step, which makes it odd and spreads the lanes
+    # over the banks
+    quantum = 0
+    if s_ops:
+        for n, a in enumerate(in_order):
+            if tile[a] > (svec if n == 0 else 1):
+                step = lds_step[a] * (svec if n == 0 and tile[a] % svec == 0 else 1)
+                if step % 8 == 0:
+                    quantum = step
+                break
+    padded = volume + (volume // quantum if quantum else 0) + 1
+
+    def pad(expr):
+        if not quantum:
+            return '(%s)' % expr
+        return '((%s) + (%s) / %d)' % (expr, expr, quantum)
+
+    parts = [_param_decl(op) for op in operands]
+    parts += ['const %s _e%d' % (idx_t, a) for a in range(nd)]
+    for op in arrays:
+        parts += ['const %s _s%d_%s' % (idx_t, a, op.name) for a in range(nd)]
+    src = [_header(typedefs, preamble)]
+    src.append('extern "C" __global__ void __launch_bounds__(%d) %s(%s) {' % (
+        threads, name, ', '.join(parts)))
+    src.append('  %s;' % loop_prep)
+    for op in s_ops:
+        src.append('  __shared__ %s _t_%s[%d];' % (op.store_t, op.name, padded))
+    for a in range(nd):
+        src.append('  const %s _nt%d = (_e%d + %d) / %d;' % (idx_t, a, a, tile[a] - 1, tile[a]))
+    src.append('  const %s _ntiles = %s;' % (idx_t, ' * '.join('_nt%d' % a for a in range(nd))))
+    src.append('  for (%s _tile = blockIdx.x; _tile < _ntiles; _tile += gridDim.x) {' % idx_t)
+    src.append('    %s _q = %s;' % (idx_t, _die_by_die('_tile', '_ntiles', idx_t, xcd)))
+    tile_order = list(tile_order) if tile_order else list(range(nd - 1, -1, -1))
+    for a in tile_order[:-1]:
+        src.append('    const %s _o%d = (_q %% _nt%d) * %d; _q /= _nt%d;' % (idx_t, a, a, tile[a], a))
+    src.append('    const %s _o%d = _q * %d;' % (idx_t, tile_order[-1], tile[tile_order[-1]]))
+    src.append('    const bool _interior = %s;' % ' && '.join(
+        '(_o%d + %d <= _e%d)' % (a, tile[a], a) for a in range(nd)))
+
+    def base(op):
+        return '_b_%s' % op.name
+    for op in arrays:
+        src.append('    %s%s* const _b_%s = _p_%s + %s;' % (
+            'const ' if (op.is_const and not op.is_out) else '', op.store_t, op.name, op.name,
+            ' + '.join('(ptrdiff_t)_o%d * _s%d_%s' % (a, a, op.name) for a in range(nd))))
+
+    def offset(op, names, skip=None):
+        terms = ['(ptrdiff_t)%s * _s%d_%s' % (names[a], a, op.name)
+                 for a in range(nd) if tile[a] > 1 and a != skip]
+        return ' + '.join(terms) if terms else '0'
+
+    if s_ops:
+        # ---- first pass: the staged inputs in their own order --------------------------------
+        first = in_order[0]
+        g_axes = list(in_order[:group])
+        g_len = 1
+        for a in g_axes:
+            g_len *= tile[a]
+        assert g_len % svec == 0
+        n_slots = volume // svec
+        trips = -(-n_slots // threads)
+        src.append('#pragma unroll')
+        src.append('    for (int _it = 0; _it < %d; ++_it) {' % trips)
+        src.append('      const int _v = threadIdx.x + _it * %d;' % threads)
+        # where the access starts within the contiguous piece, then the other axes
+        src.append('      const int _g = (_v %% %d) * %d; int _r = _v / %d;' % (
+            g_len // svec, svec, g_len // svec))
+        names = {}
+        rest = list(in_order[group:])
+        for n, a in enumerate(rest):
+            names[a] = '_i%d' % a
+            if tile[a] == 1:
+                src.append('      const int _i%d = 0;' % a)
+            elif n == len(rest) - 1:
+                src.append('      const int _i%d = _r;' % a)
+            else:
+                src.append('      const int _i%d = _r %% %d; _r /= %d;' % (a, tile[a], tile[a]))
+        rest_pos = ' + '.join('_i%d * %d' % (a, lds_step[a]) for a in rest if tile[a] > 1) or '0'
+        src.append('      const int _pos = %s;' % rest_pos)
+
+        def split(expr):
+            """Indices along the axes of the piece of its element number ``expr``."""
+            out = {}
+            left = expr
+            for n, a in enumerate(g_axes):
+                if tile[a] == 1:
+                    out[a] = '0'
+                elif n == len(g_axes) - 1:
+                    out[a] = '(%s)' % left
+                else:
+                    out[a] = '((%s) %% %d)' % (left, tile[a])
+                    left = '(%s) / %d' % (left, tile[a])
+            return out
+
+        def image(expr):
+            idx = split(expr)
+            terms = ['%s * %d' % (idx[a], lds_step[a]) for a in g_axes if tile[a] > 1]
+            return pad(' + '.join(['_pos'] + terms))
+
+        def piece_inside(expr):
+            idx = split(expr)
+            return ' && '.join('(_o%d + %s < _e%d)' % (a, idx[a], a)
+                               for a in g_axes if tile[a] > 1) or 'true'
+        guard = '' if n_slots % threads == 0 else '_v < %d && ' % n_slots
+        rest_inside = ' && '.join('(_o%d + _i%d < _e%d)' % (a, a, a)
+                                  for a in rest if tile[a] > 1) or 'true'
+
+        def rest_offset(op):
+            terms = ['(ptrdiff_t)_i%d * _s%d_%s' % (a, a, op.name) for a in rest if tile[a] > 1]
+            return ' + '.join(terms) if terms else '0'
+
+        def piece_offset(op, expr):
+            # the piece is contiguous in an interior tile: its element number is
+            # the offset; at the border of the array the axes are taken apart
+            idx = split(expr)
+            return ' + '.join('(ptrdiff_t)%s * _s%d_%s' % (idx[a], a, op.name)
+                              for a in g_axes if tile[a] > 1) or '0'
+        assert unit_first or (svec == 1 and group == 1)
+        src.append('      if (%s_interior) {' % guard)
+        for op in s_ops:
+            src.append('        { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s + %s + %s);' % (
+                op.store_t, svec, op.store_t, svec, ntl, base(op), rest_offset(op),
+                '_g' if unit_first else piece_offset(op, '_g')))
+            src.append('#pragma unroll')
+            src.append('          for (int _k = 0; _k < %d; ++_k) _t_%s[%s] = _lv.v[_k]; }' % (
+                svec, op.name, image('_g + _k')))
+        src.append('      } else if (%s%s) {' % (guard, rest_inside))
+        src.append('#pragma unroll')
+        src.append('        for (int _k = 0; _k < %d; ++_k) if (%s) {' % (svec, piece_inside('_g + _k')))
+        for op in s_ops:
+            src.append('          _t_%s[%s] = %s[%s + %s];' % (
+                op.name, image('_g + _k'), base(op), rest_offset(op),
+                piece_offset(op, '_g + _k')))
+        src.append('        }')
+        src.append('      }')
+        src.append('    }')
+        src.append('    __syncthreads();')
+
+    # ---- second pass: the tile in the order of the outputs ---------------------------------------
+    n_slots = volume // vec
+    trips = -(-n_slots // threads)
+    src.append('#pragma unroll')
+    src.append('    for (int _it = 0; _it < %d; ++_it) {' % trips)
+    src.append('      const int _w = threadIdx.x + _it * %d;' % threads)
+    src.append('      int _r = _w;')
+    names = {}
+    for a in range(nd - 1, -1, -1):
+        per = tile[a] // vec if a == last else tile[a]
+        scale = ' * %d' % vec if (a == last and vec > 1) else ''
+        names[a] = '_j%d' % a
+        if tile[a] == 1:
+            src.append('      const int _j%d = 0;' % a)
+        elif a == 0:
+            src.append('      const int _j%d = _r%s;' % (a, scale))
+        else:
+            src.append('      const int _j%d = (_r %% %d)%s; _r /= %d;' % (a, per, scale, per))
+    src.append('      const int _pos = _w * %d;' % vec)
+    guard = '' if n_slots % threads == 0 else '_w < %d && ' % n_slots
+    inside = ' && '.join(
+        '(_o%d + _j%d + %d <= _e%d)' % (a, a, vec if a == last else 1, a)
+        for a in range(nd) if tile[a] > 1) or 'true'
+
+    def unit(op):
+        return op.name not in zero_last
+
+    def full_load(op):
+        if op.name in staged:
+            return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
+        if not unit(op):
+            return '_z_%s' % op.name
+        return '_l_%s.v[_k]' % op.name
+
+    def full_store(op, value):
+        return '_l_%s.v[_k] = %s;' % (op.name, value)
+
+    src.append('      if (%s(_interior || (%s))) {' % (guard, inside))
+    for op in d_ops:
+        reads = (not op.is_out) or op.read_out
+        addr = '%s + %s' % (base(op), offset(op, names, skip=last))
+        if not unit(op):
+            src.append('        const %s _z_%s = *(%s);' % (op.store_t, op.name, addr))
+        elif reads:
+            src.append('        cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s + _j%d);' % (
+                op.store_t, vec, op.name, op.store_t, vec, ntl, addr, last))
+        else:
+            src.append('        cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+    src.append('#pragma unroll')
+    src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
+    src.append(_element_code(operands, operation, full_load, full_store, 10))
+    src.append('        }')
+    for op in d_ops:
+        if op.is_out:
+            src.append('        cupy::store_vec<%s, %d, %s>(%s + %s + _j%d, _l_%s);' % (
+                op.store_t, vec, nts, base(op), offset(op, names, skip=last), last, op.name))
+    if vec > 1:
+        others = ' && '.join('(_o%d + _j%d < _e%d)' % (a, a, a)
+                             for a in range(nd) if tile[a] > 1 and a != last) or 'true'
+
+        def edge_load(op):
+            if op.name in staged:
+                return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
+            if not unit(op):
+                return '(*(%s + %s))' % (base(op), offset(op, names, skip=last))
+            return '(%s + %s)[_j%d + _k]' % (base(op), offset(op, names, skip=last), last)
+
+        def edge_store(op, value):
+            return '(%s + %s)[_j%d + _k] = %s;' % (
+                base(op), offset(op, names, skip=last), last, value)
+
+        src.append('      } else if (%s%s) {' % (guard, others))
+        src.append('#pragma unroll')
+        src.append('        for (int _k = 0; _k < %d; ++_k) if (_o%d + _j%d + _k < _e%d) {' % (
+            vec, last, last, last))
+        src.append(_element_code(operands, operation, edge_load, edge_store, 10))
+        src.append('        }')
+    src.append('      }')
+    src.append('    }')
+    if s_ops:
+        src.append('    __syncthreads();')
+    src.append('  }')
+    src.append('  %s;' % after_loop)
+    src.append('}')
+    return '\n'.join(src) + '\n'

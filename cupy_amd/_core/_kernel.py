@@ -319,6 +319,15 @@ def _grid_limit(dev_id, blocks_per_cu):
     return g
 
 
+def _off_lines(arrays, strides):
+    """Whether an array starts inside a 128-byte line, or has a stride of more
+    than a line that is no whole number of lines: tiles then share the lines at
+    their borders."""
+    return any(
+        a.data.ptr % 128 or any(abs(c) >= 128 and c % 128 for c in cs)
+        for a, cs in zip(arrays, strides))
+
+
 def _max_blocks(block):
     """Most workgroups of ``block`` work-items one grid dimension may hold: a
     dispatch carries its size in work-items in 32 bits per dimension."""
@@ -436,13 +445,33 @@ class _ElementwisePlanner:
                         dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
                         force_read_out, stream_ptr, kernel_name, rec)
                 mode = self._classify_2d(arrays, cstrides, args, nin)
-            elif nd in (3, 4) and not self._uses_ind and not self._uses_i:
-                plan = self._plan_rows_nd(arrays, cshape, cstrides, args, nin)
-                if plan is not None:
-                    return self._launch_rows2d(
-                        dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
-                        force_read_out, stream_ptr, kernel_name, rec)
-                plan = self._plan_batched(arrays, cshape, cstrides, args, nin)
+            elif 3 <= nd <= 6 and not self._uses_ind and not self._uses_i:
+                plan = None
+                if nd <= 4:
+                    plan = self._plan_rows_nd(arrays, cshape, cstrides, args, nin)
+                    if plan is not None:
+                        return self._launch_rows2d(
+                            dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
+                            force_read_out, stream_ptr, kernel_name, rec)
+                    plan = self._plan_batched(arrays, cshape, cstrides, args, nin)
+                # Tiles over several axes (emit_packed) wherever they apply,
+                # except for large tiles of two axes in arrays whose rows do not
+                # start on cache lines: the tiled kernel walks those in strips
+                # that keep neighbours on one die (2^26 float32 over permuted
+                # copies, us, tiles of two axes / of several: (524288, 8, 8) to
+                # (.., 8, 8) transposed 806 / 39; (4, 2^21, 4) reversed 3124 / 38;
+                # (256, 512, 512) as (0, 2, 1) 90 / 76; (255, 511, 513) as
+                # (0, 2, 1) 114 / 136; (4226, 68, 4, 29) as (2, 1, 3, 0) 59 / 97)
+                mode_p = _tuning.get('packed_tiles')
+                if mode_p and not (mode_p == 'auto' and plan is not None
+                                   and plan[0][0] * plan[0][1] >= _tuning.get('packed_tiles_below')
+                                   and min(plan[0]) >= 16
+                                   and _off_lines(arrays, cstrides)):
+                    packed = self._plan_packed(arrays, cshape, cstrides, args, nin)
+                    if packed is not None:
+                        return self._launch_packed(
+                            dev_id, args, nin, arrays, cshape, cstrides, packed, var_types,
+                            typedefs, casts, force_read_out, stream_ptr, kernel_name, rec)
                 if plan is not None:
                     done = self._launch_tiled(
                         dev_id, args, nin, arrays, plan[0], plan[1], var_types, typedefs,
@@ -892,6 +921,232 @@ class _ElementwisePlanner:
             bstrides = [bs + (0,) for bs in bstrides]
         return shape2, strides2, (bshape, bstrides)
 
+    def _plan_packed(self, arrays, cshape, cstrides, args, nin):
+        """Tiles over several axes (``emit_packed``) for a problem of three or
+        more axes.  Arrays whose walk in the order of the outputs gives runs of
+        64 bytes or more (unit stride along the last axis), or one value per
+        vector (zero stride along it), are read straight from memory; the
+        other inputs are staged through the LDS in their own order.  Returns
+        (tile, order of the axes for staging, staged names, zero-stride names,
+        vec, svec, axes of the contiguous piece, unit stride along the first
+        of them?) or None."""
+        nd = len(cshape)
+        names = [p.name for a, p in zip(args, self.params)
+                 if isinstance(a, ndarray) and not p.raw]
+        outs = args[nin:]
+        kinds = {}
+        first_staged = None
+        lds_item = 0
+        max_item = max(a.dtype.itemsize for a in arrays)
+        for a, cs, nm in zip(arrays, cstrides, names):
+            item = a.dtype.itemsize
+            if any(s % item for s in cs):
+                return None
+            is_out = any(a is o for o in outs)
+            if cs[-1] == item:
+                # how far the walk in the order of the outputs stays contiguous
+                run = item
+                for ax in range(nd - 1, -1, -1):
+                    if cs[ax] != run:
+                        break
+                    run *= cshape[ax]
+                kind = 'D' if (is_out or run >= 64) else 'S'
+            elif cs[-1] == 0 and not is_out:
+                kind = 'Z'
+            elif not is_out:
+                kind = 'S'
+            else:
+                return None
+            if kinds.get(nm, kind) != kind:
+                return None
+            if kind == 'S' and nm not in kinds:
+                lds_item += item
+                if first_staged is None:
+                    first_staged = cs
+            kinds[nm] = kind
+        if 'D' not in kinds.values():
+            return None
+        staged = tuple(sorted(n for n, k in kinds.items() if k == 'S'))
+        zero_last = tuple(sorted(n for n, k in kinds.items() if k == 'Z'))
+        out_order = list(range(nd - 1, -1, -1))
+        if first_staged is not None:
+            in_order = sorted(range(nd), key=lambda ax: (
+                first_staged[ax] == 0, abs(first_staged[ax])))
+        else:
+            in_order = out_order
+        last, first = nd - 1, in_order[0]
+        # vectors along the last axis (second pass) and along the fastest axis
+        # of the staged inputs (first pass); short axes that are no whole
+        # number of vectors keep to what divides them
+        def widest(ax, members, limit_item):
+            v = max(1, 16 // limit_item)
+            while v > 1 and (v > cshape[ax] or (cshape[ax] < 12 * v and cshape[ax] % v)):
+                v //= 2
+            while v > 1:
+                nb_ok = True
+                for a, cs in members:
+                    nb = v * a.dtype.itemsize
+                    if not _aligned(a.data.ptr, nb) or not all(
+                            _aligned(c, nb) for k, c in enumerate(cs) if k != ax):
+                        nb_ok = False
+                if nb_ok:
+                    break
+                v //= 2
+            return v
+        direct = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'D']
+        s_arrays = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'S']
+        s_item = max([a.dtype.itemsize for a, cs in s_arrays] or [1])
+        vec = widest(last, direct, max_item)
+        svec = 1
+        if s_arrays and all(cs[first] == a.dtype.itemsize for a, cs in s_arrays):
+            svec = widest(first, s_arrays, s_item)
+        max_v = 8192 if not lds_item else min(8192, (48 * 1024) // lds_item)
+        want = min(max_v, 4096 if max_item <= 4 else 2048 if max_item == 8 else 1024)
+        while True:
+            mult = [1] * nd
+            mult[last] = vec
+            mult[first] = max(mult[first], svec)
+            cap = [-(-e // m) * m for e, m in zip(cshape, mult)]
+            run = max(32, 256 // max_item)
+            while True:
+                tile = list(mult)
+
+                def grow(order):
+                    have = 1
+                    for ax in order:
+                        if have >= run:
+                            break
+                        need = -(-run // have)
+                        tile[ax] = max(tile[ax], min(cap[ax], -(-need // mult[ax]) * mult[ax]))
+                        have *= tile[ax]
+                        if tile[ax] < cshape[ax]:
+                            break
+                grow(out_order)
+                grow(in_order)
+                volume = internal.prod(tile)
+                if volume <= max_v or run <= 1:
+                    break
+                run //= 2
+            if volume > max_v:
+                return None
+            turn = 0
+            while internal.prod(tile) * 2 <= want:
+                for k in range(2):
+                    order = (out_order, in_order)[(turn + k) % 2]
+                    ax = next((x for x in order if tile[x] < cshape[x]), None)
+                    if ax is not None:
+                        tile[ax] = min(cap[ax], tile[ax] * 2)
+                        turn = (turn + k + 1) % 2
+                        break
+                else:
+                    break
+            # an axis cut in two unequal parts: whole if there is room, else in
+            # equal parts
+            for ax in range(nd):
+                if 1 < tile[ax] < cshape[ax]:
+                    if cshape[ax] < 2 * tile[ax] and (
+                            internal.prod(tile) // tile[ax] * cap[ax] <= max_v):
+                        tile[ax] = cap[ax]
+                    else:
+                        parts = -(-cshape[ax] // tile[ax])
+                        even = -(-(-(-cshape[ax] // parts)) // mult[ax]) * mult[ax]
+                        tile[ax] = min(tile[ax], even)
+            # a tile that reaches past an axis that is no whole number of
+            # vectors would have no interior: narrower vectors there
+            if vec > 1 and tile[last] > cshape[last]:
+                vec //= 2
+                continue
+            if svec > 1 and tile[first] > cshape[first]:
+                svec //= 2
+                continue
+            break
+        # The first axes of the staged inputs that lie in them as one piece
+        group = 1
+        if s_arrays and all(cs[first] == a.dtype.itemsize for a, cs in s_arrays):
+            while group < nd:
+                a, b = in_order[group - 1], in_order[group]
+                if tile[a] != cshape[a] or tile[b] == 1 or not all(
+                        cs[b] == cs[a] * cshape[a] for arr, cs in s_arrays):
+                    break
+                group += 1
+            if group > 1:
+                piece = internal.prod(tile[ax] for ax in in_order[:group])
+                svec = max(1, 16 // s_item)
+                while svec > 1 and (piece % svec or not all(
+                        _aligned(arr.data.ptr, svec * arr.dtype.itemsize) and all(
+                            _aligned(cs[ax], svec * arr.dtype.itemsize)
+                            for ax in in_order[group:])
+                        for arr, cs in s_arrays)):
+                    svec //= 2
+        unit_first = all(cs[first] == arr.dtype.itemsize for arr, cs in s_arrays)
+        return tuple(tile), tuple(in_order), staged, zero_last, vec, svec, group, unit_first
+
+    def _launch_packed(self, dev_id, args, nin, arrays, cshape, cstrides, plan, var_types,
+                       typedefs, casts, force_read_out, stream_ptr, kernel_name, rec):
+        tile, in_order, staged, zero_last, vec, svec, group, unit_first = plan
+        nd = len(cshape)
+        threads = 256
+        ntiles = 1
+        span = 0
+        for e, t in zip(cshape, tile):
+            ntiles *= (e + t - 1) // t
+        for a, cs in zip(arrays, cstrides):
+            span = max(span, sum(abs(c) // a.dtype.itemsize * (e + t)
+                                 for c, e, t in zip(cs, cshape, tile)))
+        idx64 = span > _INT32_MAX or ntiles * internal.prod(tile) > _INT32_MAX
+        operands = self._make_operands(args, nin, var_types, casts, force_read_out)
+        stream_hint = _tuning.stream_policy(
+            _tuning.get('tiled_stream'), *self._traffic(args, nin, ()))
+        if _tuning.get('tiled_stream') == 'auto':
+            # tiles share the cache lines at their borders wherever a run is no
+            # whole number of lines: plain accesses let the cache put them together
+            item = min(a.dtype.itemsize for a in arrays)
+            whole = (tile[-1] * item) % 128 == 0 and not _off_lines(arrays, cstrides)
+            stream_hint = (stream_hint[0] and whole and not staged, stream_hint[1] and whole)
+        # tiles whose borders fall inside cache lines: neighbours on one die
+        mode = _tuning.get('packed_xcd')
+        xcd = bool(mode) and (mode is True or _off_lines(arrays, cstrides))
+        tile_order = None
+        if staged and _tuning.get('packed_order') == 'in':
+            tile_order = in_order
+        key = ('packed', tile_order, tuple(o.key() for o in operands), typedefs, tile, in_order, staged,
+               zero_last, vec, svec, group, unit_first, idx64, dev_id, stream_hint, threads,
+               xcd)
+        entry = self._memo.get(key)
+        if entry is None:
+            name = kernel_name or self.name
+            code = _cg.emit_packed(
+                name, operands, self.operation, typedefs, self.preamble,
+                self.loop_prep, self.after_loop, tile=tile, in_order=in_order,
+                staged=staged, zero_last=zero_last, vec=vec, svec=svec, group=group,
+                unit_first=unit_first, threads=threads, idx64=idx64, stream_hint=stream_hint,
+                xcd=xcd, tile_order=tile_order)
+            fn = compiler.compile_with_cache(code, self.options).get_function(name)
+            ic = 'q' if idx64 else 'i'
+            fmt = ['@']
+            for o in operands:
+                if o.kind == 'array':
+                    fmt.append('P')
+                elif o.kind == 'raw':
+                    fmt.append('P' + 'q' * (1 + 2 * o.ndim))
+                elif o.kind == 'scalar':
+                    fmt.append(_scalar_struct_code(o.store_t))
+            fmt.append(ic * (nd * (1 + len(arrays))))
+            entry = (fn, _make_packer(fmt), code)
+            with self._lock:
+                entry = self._memo.setdefault(key, entry)
+            self._remember_code(args, entry[2])
+        fn, packer, _ = entry
+        block_args = self._flat_values(args)
+        block_args.const(*cshape)
+        for a, cs in zip(arrays, cstrides):
+            item = a.dtype.itemsize
+            block_args.const(*(c // item for c in cs))
+        grid = max(1, min(ntiles, _max_blocks(threads)))
+        _launch_plan.launch(rec, fn, (grid, 1, 1), (threads, 1, 1), packer, block_args,
+                            stream_ptr)
+        return True
+
     @staticmethod
     def _flat_stage_width(arrays, cstrides, names, layouts, nr):
         """Elements per access with which the staged operands of a tile that
@@ -1103,7 +1358,8 @@ class _ElementwisePlanner:
         # their borders do not fall on cache-line boundaries
         mode = _tuning.get('tiled_xcd')
         xcd = bool(mode) and (mode is True or any(
-            a.data.ptr % 128 or max(abs(cs[0]), abs(cs[1])) % 128
+            a.data.ptr % 128 or any(
+                abs(c) > a.itemsize and abs(c) % 128 for c in cs[:2])
             for a, cs in zip(arrays, cstrides)))
         key = ('tiled', tuple(o.key() for o in operands), typedefs, vec, idx64,
                tuple(sorted(layouts.items())), dev_id, stream_hint, tile_r, tile_c,

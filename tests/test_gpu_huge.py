@@ -325,3 +325,28 @@ def test_permuted_axes_beyond_2_to_31_elements():
         'for (long long r = 0; r < n; ++r) w += (b * n * n + r * n + c) % 100; ok = s == w',
         'is_middle_sum')
     assert bool(check2(s).all().get())
+
+
+def test_tiles_over_several_axes_beyond_2_to_31_elements():
+    from cupy_amd._core import _tuning
+    nb = 180000001                                    # 2.16e9 elements
+    a = _fill_mod100_i8(size=nb * 12).reshape(nb, 4, 3)
+    t = cp.ascontiguousarray(a.transpose(0, 2, 1))    # every tile spans the two small axes
+    check = cp.ElementwiseKernel(
+        'int8 v', 'bool ok',
+        'const long long c = i % 4, r = (i / 4) % 3, b = i / 12;'
+        'ok = v == (signed char)((b * 12 + c * 3 + r) % 100)', 'is_small_transposed')
+    assert bool(check(t).all().get())
+    del t, a
+    nb, n = 3, 30000                                  # 2.7e9 elements
+    a = _fill_mod100_i8(size=nb * n * n).reshape(nb, n, n)
+    _tuning.set(packed_tiles=True)
+    try:
+        t = cp.ascontiguousarray(a.transpose(0, 2, 1))
+    finally:
+        _tuning.set(packed_tiles='auto')
+    check = cp.ElementwiseKernel(
+        'int8 v', 'bool ok',
+        'const long long n = 30000, c = i % n, r = (i / n) % n, b = i / (n * n);'
+        'ok = v == (signed char)((b * n * n + c * n + r) % 100)', 'is_batch_transposed')
+    assert bool(check(t).all().get())
