@@ -903,8 +903,8 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
 
 def emit_packed(name, operands, operation, typedefs='', preamble='',
                 loop_prep='', after_loop='', tile=(), in_order=(), staged=(),
-                zero_last=(), vec=1, svec=1, group=1, unit_first=True, threads=256,
-                idx64=False, stream_hint=True, xcd=False, tile_order=None):
+                zero_last=(), vec=1, svec=1, group=1, ogroup=1, unit_first=True,
+                threads=256, idx64=False, stream_hint=True, xcd=False, tile_order=None):
     """Kernel for an index space of ``len(tile)`` axes whose arrays are
     permuted differently, with a tile that spans SEVERAL axes: as many of the
     last axes as give the outputs a long contiguous run, and as many of the
@@ -915,13 +915,13 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
     being its edges.
 
     A workgroup takes a tile in two passes.  First it reads the staged inputs in
-    THEIR order, ``svec`` elements per access, and puts
-    them into an LDS image of the tile that is laid out in the order of the
-    outputs (padded so that lanes side by side spread over the banks).  Then it goes through the tile in
-    the order of the outputs, ``vec`` elements per access along the last axis:
-    the other arrays (unit stride along the last axis, or zero for the inputs
-    named in ``zero_last``; any stride along the others) come straight from
-    memory, the staged ones from the image.
+    THEIR order, ``svec`` elements per access, and puts them into an LDS image
+    of the tile that is laid out in the order of the outputs (padded so that
+    lanes side by side spread over the banks).  Then it goes through the tile in
+    the order of the outputs, ``vec`` elements per access: the other arrays
+    (unit stride along the last axis, or zero for the inputs named in
+    ``zero_last``; any stride along the others) come straight from memory, the
+    staged ones from the image.
 
     ``group``: how many of the first axes of ``in_order`` lie in the staged
     inputs as ONE contiguous piece within a tile (each but the last of them
@@ -929,13 +929,16 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
     ``svec`` elements then run over that piece as a whole, whatever the extents
     of its axes, and every element finds its own place in the image.
     ``unit_first``: every staged input has unit stride along ``in_order[0]``
-    (else ``svec`` and ``group`` are 1 and the stride is applied).
+    (else ``svec`` and ``group`` are 1 and the stride is applied).  ``ogroup``:
+    the same for the last axes and the arrays of the second pass (the inputs of
+    ``zero_last`` have zero stride along all of these axes).  At the border of
+    the array a piece is shorter, never split: only its last axis can be cut.
 
     ``tile[a]`` elements along axis a; tiles are numbered along the axes of
     ``tile_order``, fastest first (default: the order of the outputs; ``xcd``:
-    die by die, see ``_die_by_die``).  Kernel parameters after the operands: the extents ``_e<a>``, then
-    per array its strides ``_s<a>_<name>`` in elements.  The element index ``i``
-    and the indexer are not available.
+    die by die, see ``_die_by_die``).  Kernel parameters after the operands: the
+    extents ``_e<a>``, then per array its strides ``_s<a>_<name>`` in elements.
+    The element index ``i`` and the indexer are not available.
     """
     nd = len(tile)
     idx_t = 'ptrdiff_t' if idx64 else 'int'
@@ -948,11 +951,11 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
     d_ops = [op for op in arrays if op.name not in staged]
     for op in s_ops:
         assert not op.is_out
+    assert unit_first or (svec == 1 and group == 1)
     volume = 1
     for t in tile:
         volume *= t
-    last = nd - 1
-    assert tile[last] % vec == 0
+    out_order = list(range(nd - 1, -1, -1))
     # position of an element in the image: its number in the order of the outputs
     lds_step = [1] * nd
     for a in range(nd - 2, -1, -1):
@@ -976,6 +979,9 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
             return '(%s)' % expr
         return '((%s) + (%s) / %d)' % (expr, expr, quantum)
 
+    def unroll(trips):
+        return '#pragma unroll' if trips <= 16 else '#pragma unroll 4'
+
     parts = [_param_decl(op) for op in operands]
     parts += ['const %s _e%d' % (idx_t, a) for a in range(nd)]
     for op in arrays:
@@ -991,189 +997,167 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
     src.append('  const %s _ntiles = %s;' % (idx_t, ' * '.join('_nt%d' % a for a in range(nd))))
     src.append('  for (%s _tile = blockIdx.x; _tile < _ntiles; _tile += gridDim.x) {' % idx_t)
     src.append('    %s _q = %s;' % (idx_t, _die_by_die('_tile', '_ntiles', idx_t, xcd)))
-    tile_order = list(tile_order) if tile_order else list(range(nd - 1, -1, -1))
+    tile_order = list(tile_order) if tile_order else out_order
     for a in tile_order[:-1]:
         src.append('    const %s _o%d = (_q %% _nt%d) * %d; _q /= _nt%d;' % (idx_t, a, a, tile[a], a))
     src.append('    const %s _o%d = _q * %d;' % (idx_t, tile_order[-1], tile[tile_order[-1]]))
     src.append('    const bool _interior = %s;' % ' && '.join(
         '(_o%d + %d <= _e%d)' % (a, tile[a], a) for a in range(nd)))
-
-    def base(op):
-        return '_b_%s' % op.name
     for op in arrays:
         src.append('    %s%s* const _b_%s = _p_%s + %s;' % (
             'const ' if (op.is_const and not op.is_out) else '', op.store_t, op.name, op.name,
             ' + '.join('(ptrdiff_t)_o%d * _s%d_%s' % (a, a, op.name) for a in range(nd))))
 
-    def offset(op, names, skip=None):
-        terms = ['(ptrdiff_t)%s * _s%d_%s' % (names[a], a, op.name)
-                 for a in range(nd) if tile[a] > 1 and a != skip]
-        return ' + '.join(terms) if terms else '0'
-
-    if s_ops:
-        # ---- first pass: the staged inputs in their own order --------------------------------
-        first = in_order[0]
-        g_axes = list(in_order[:group])
+    def one_pass(order, n_group, width, prefix):
+        """Code that numbers the accesses of a pass: ``_g`` where an access
+        starts within the contiguous piece of the first ``n_group`` axes of
+        ``order``, ``<prefix><a>`` the index along each other axis, ``_len``
+        the length of the piece in this tile.  Returns (axes of the piece,
+        other axes, slots, trips)."""
+        g_axes = list(order[:n_group])
+        rest = list(order[n_group:])
         g_len = 1
         for a in g_axes:
             g_len *= tile[a]
-        assert g_len % svec == 0
-        n_slots = volume // svec
-        trips = -(-n_slots // threads)
-        src.append('#pragma unroll')
+        assert g_len % width == 0
+        slots = volume // width
+        trips = -(-slots // threads)
+        cut = g_axes[-1]
+        src.append('    const int _len%s = %d * (int)((_e%d - _o%d < %d) ? (_e%d - _o%d) : %d);' % (
+            prefix, g_len // tile[cut], cut, cut, tile[cut], cut, cut, tile[cut]))
+        src.append(unroll(trips))
         src.append('    for (int _it = 0; _it < %d; ++_it) {' % trips)
         src.append('      const int _v = threadIdx.x + _it * %d;' % threads)
-        # where the access starts within the contiguous piece, then the other axes
         src.append('      const int _g = (_v %% %d) * %d; int _r = _v / %d;' % (
-            g_len // svec, svec, g_len // svec))
-        names = {}
-        rest = list(in_order[group:])
+            g_len // width, width, g_len // width))
         for n, a in enumerate(rest):
-            names[a] = '_i%d' % a
             if tile[a] == 1:
-                src.append('      const int _i%d = 0;' % a)
+                src.append('      const int %s%d = 0;' % (prefix, a))
             elif n == len(rest) - 1:
-                src.append('      const int _i%d = _r;' % a)
+                src.append('      const int %s%d = _r;' % (prefix, a))
             else:
-                src.append('      const int _i%d = _r %% %d; _r /= %d;' % (a, tile[a], tile[a]))
-        rest_pos = ' + '.join('_i%d * %d' % (a, lds_step[a]) for a in rest if tile[a] > 1) or '0'
-        src.append('      const int _pos = %s;' % rest_pos)
+                src.append('      const int %s%d = _r %% %d; _r /= %d;' % (prefix, a, tile[a], tile[a]))
+        return g_axes, rest, slots, trips
 
-        def split(expr):
-            """Indices along the axes of the piece of its element number ``expr``."""
-            out = {}
-            left = expr
-            for n, a in enumerate(g_axes):
-                if tile[a] == 1:
-                    out[a] = '0'
-                elif n == len(g_axes) - 1:
-                    out[a] = '(%s)' % left
-                else:
-                    out[a] = '((%s) %% %d)' % (left, tile[a])
-                    left = '(%s) / %d' % (left, tile[a])
-            return out
+    def split(g_axes, expr):
+        """Indices along the axes of a piece of its element number ``expr``."""
+        out = {}
+        left = expr
+        for n, a in enumerate(g_axes):
+            if tile[a] == 1:
+                out[a] = '0'
+            elif n == len(g_axes) - 1:
+                out[a] = '(%s)' % left
+            else:
+                out[a] = '((%s) %% %d)' % (left, tile[a])
+                left = '(%s) / %d' % (left, tile[a])
+        return out
+
+    def rest_offset(op, rest, prefix):
+        terms = ['(ptrdiff_t)%s%d * _s%d_%s' % (prefix, a, a, op.name) for a in rest if tile[a] > 1]
+        return ' + '.join(terms) if terms else '0'
+
+    def rest_inside(rest, prefix):
+        return ' && '.join('(_o%d + %s%d < _e%d)' % (a, prefix, a, a)
+                           for a in rest if tile[a] > 1) or 'true'
+
+    if s_ops:
+        # ---- first pass: the staged inputs in their own order --------------------------------
+        g_axes, rest, slots, trips = one_pass(in_order, group, svec, '_i')
+        src.append('      const int _pos = %s;' % (
+            ' + '.join('_i%d * %d' % (a, lds_step[a]) for a in rest if tile[a] > 1) or '0'))
 
         def image(expr):
-            idx = split(expr)
+            idx = split(g_axes, expr)
             terms = ['%s * %d' % (idx[a], lds_step[a]) for a in g_axes if tile[a] > 1]
             return pad(' + '.join(['_pos'] + terms))
 
-        def piece_inside(expr):
-            idx = split(expr)
-            return ' && '.join('(_o%d + %s < _e%d)' % (a, idx[a], a)
-                               for a in g_axes if tile[a] > 1) or 'true'
-        guard = '' if n_slots % threads == 0 else '_v < %d && ' % n_slots
-        rest_inside = ' && '.join('(_o%d + _i%d < _e%d)' % (a, a, a)
-                                  for a in rest if tile[a] > 1) or 'true'
-
-        def rest_offset(op):
-            terms = ['(ptrdiff_t)_i%d * _s%d_%s' % (a, a, op.name) for a in rest if tile[a] > 1]
-            return ' + '.join(terms) if terms else '0'
-
-        def piece_offset(op, expr):
-            # the piece is contiguous in an interior tile: its element number is
-            # the offset; at the border of the array the axes are taken apart
-            idx = split(expr)
+        def within(op, expr):
+            if unit_first:
+                return expr
+            idx = split(g_axes, expr)
             return ' + '.join('(ptrdiff_t)%s * _s%d_%s' % (idx[a], a, op.name)
                               for a in g_axes if tile[a] > 1) or '0'
-        assert unit_first or (svec == 1 and group == 1)
-        src.append('      if (%s_interior) {' % guard)
+        guard = '' if slots % threads == 0 else '_v < %d && ' % slots
+        src.append('      if (%s(_interior || (%s))) {' % (guard, rest_inside(rest, '_i')))
+        src.append('        if (_g + %d <= _len_i) {' % svec)
         for op in s_ops:
-            src.append('        { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s + %s + %s);' % (
-                op.store_t, svec, op.store_t, svec, ntl, base(op), rest_offset(op),
-                '_g' if unit_first else piece_offset(op, '_g')))
+            src.append('          { const cupy::Vec<%s, %d> _lv = cupy::load_vec<%s, %d, %s>(%s + %s + %s);' % (
+                op.store_t, svec, op.store_t, svec, ntl, '_b_' + op.name,
+                rest_offset(op, rest, '_i'), within(op, '_g')))
             src.append('#pragma unroll')
-            src.append('          for (int _k = 0; _k < %d; ++_k) _t_%s[%s] = _lv.v[_k]; }' % (
+            src.append('            for (int _k = 0; _k < %d; ++_k) _t_%s[%s] = _lv.v[_k]; }' % (
                 svec, op.name, image('_g + _k')))
-        src.append('      } else if (%s%s) {' % (guard, rest_inside))
-        src.append('#pragma unroll')
-        src.append('        for (int _k = 0; _k < %d; ++_k) if (%s) {' % (svec, piece_inside('_g + _k')))
-        for op in s_ops:
-            src.append('          _t_%s[%s] = %s[%s + %s];' % (
-                op.name, image('_g + _k'), base(op), rest_offset(op),
-                piece_offset(op, '_g + _k')))
+        if svec > 1:
+            src.append('        } else {')
+            src.append('#pragma unroll')
+            src.append('          for (int _k = 0; _k < %d; ++_k) if (_g + _k < _len_i) {' % svec)
+            for op in s_ops:
+                src.append('            _t_%s[%s] = (%s + %s)[%s];' % (
+                    op.name, image('_g + _k'), '_b_' + op.name, rest_offset(op, rest, '_i'),
+                    within(op, '_g + _k')))
+            src.append('          }')
         src.append('        }')
         src.append('      }')
         src.append('    }')
         src.append('    __syncthreads();')
 
     # ---- second pass: the tile in the order of the outputs ---------------------------------------
-    n_slots = volume // vec
-    trips = -(-n_slots // threads)
-    src.append('#pragma unroll')
-    src.append('    for (int _it = 0; _it < %d; ++_it) {' % trips)
-    src.append('      const int _w = threadIdx.x + _it * %d;' % threads)
-    src.append('      int _r = _w;')
-    names = {}
-    for a in range(nd - 1, -1, -1):
-        per = tile[a] // vec if a == last else tile[a]
-        scale = ' * %d' % vec if (a == last and vec > 1) else ''
-        names[a] = '_j%d' % a
-        if tile[a] == 1:
-            src.append('      const int _j%d = 0;' % a)
-        elif a == 0:
-            src.append('      const int _j%d = _r%s;' % (a, scale))
-        else:
-            src.append('      const int _j%d = (_r %% %d)%s; _r /= %d;' % (a, per, scale, per))
-    src.append('      const int _pos = _w * %d;' % vec)
-    guard = '' if n_slots % threads == 0 else '_w < %d && ' % n_slots
-    inside = ' && '.join(
-        '(_o%d + _j%d + %d <= _e%d)' % (a, a, vec if a == last else 1, a)
-        for a in range(nd) if tile[a] > 1) or 'true'
+    g_axes, rest, slots, trips = one_pass(out_order, ogroup, vec, '_j')
+    src.append('      const int _pos = _v * %d;' % vec)
+    guard = '' if slots % threads == 0 else '_v < %d && ' % slots
 
-    def unit(op):
-        return op.name not in zero_last
+    def address(op):
+        return '(_b_%s + %s)' % (op.name, rest_offset(op, rest, '_j'))
 
     def full_load(op):
         if op.name in staged:
             return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
-        if not unit(op):
+        if op.name in zero_last:
             return '_z_%s' % op.name
         return '_l_%s.v[_k]' % op.name
 
     def full_store(op, value):
         return '_l_%s.v[_k] = %s;' % (op.name, value)
 
-    src.append('      if (%s(_interior || (%s))) {' % (guard, inside))
+    def edge_load(op):
+        if op.name in staged:
+            return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
+        if op.name in zero_last:
+            return '_z_%s' % op.name
+        return '%s[_g + _k]' % address(op)
+
+    def edge_store(op, value):
+        return '%s[_g + _k] = %s;' % (address(op), value)
+
+    src.append('      if (%s(_interior || (%s))) {' % (guard, rest_inside(rest, '_j')))
     for op in d_ops:
-        reads = (not op.is_out) or op.read_out
-        addr = '%s + %s' % (base(op), offset(op, names, skip=last))
-        if not unit(op):
-            src.append('        const %s _z_%s = *(%s);' % (op.store_t, op.name, addr))
-        elif reads:
-            src.append('        cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s + _j%d);' % (
-                op.store_t, vec, op.name, op.store_t, vec, ntl, addr, last))
+        if op.name in zero_last:
+            src.append('        const %s _z_%s = *%s;' % (op.store_t, op.name, address(op)))
+    src.append('        if (_g + %d <= _len_j) {' % vec)
+    for op in d_ops:
+        if op.name in zero_last:
+            continue
+        if (not op.is_out) or op.read_out:
+            src.append('          cupy::Vec<%s, %d> _l_%s = cupy::load_vec<%s, %d, %s>(%s + _g);' % (
+                op.store_t, vec, op.name, op.store_t, vec, ntl, address(op)))
         else:
-            src.append('        cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
+            src.append('          cupy::Vec<%s, %d> _l_%s;' % (op.store_t, vec, op.name))
     src.append('#pragma unroll')
-    src.append('        for (int _k = 0; _k < %d; ++_k) {' % vec)
-    src.append(_element_code(operands, operation, full_load, full_store, 10))
-    src.append('        }')
+    src.append('          for (int _k = 0; _k < %d; ++_k) {' % vec)
+    src.append(_element_code(operands, operation, full_load, full_store, 12))
+    src.append('          }')
     for op in d_ops:
         if op.is_out:
-            src.append('        cupy::store_vec<%s, %d, %s>(%s + %s + _j%d, _l_%s);' % (
-                op.store_t, vec, nts, base(op), offset(op, names, skip=last), last, op.name))
+            src.append('          cupy::store_vec<%s, %d, %s>(%s + _g, _l_%s);' % (
+                op.store_t, vec, nts, address(op), op.name))
     if vec > 1:
-        others = ' && '.join('(_o%d + _j%d < _e%d)' % (a, a, a)
-                             for a in range(nd) if tile[a] > 1 and a != last) or 'true'
-
-        def edge_load(op):
-            if op.name in staged:
-                return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
-            if not unit(op):
-                return '(*(%s + %s))' % (base(op), offset(op, names, skip=last))
-            return '(%s + %s)[_j%d + _k]' % (base(op), offset(op, names, skip=last), last)
-
-        def edge_store(op, value):
-            return '(%s + %s)[_j%d + _k] = %s;' % (
-                base(op), offset(op, names, skip=last), last, value)
-
-        src.append('      } else if (%s%s) {' % (guard, others))
+        src.append('        } else {')
         src.append('#pragma unroll')
-        src.append('        for (int _k = 0; _k < %d; ++_k) if (_o%d + _j%d + _k < _e%d) {' % (
-            vec, last, last, last))
-        src.append(_element_code(operands, operation, edge_load, edge_store, 10))
-        src.append('        }')
+        src.append('          for (int _k = 0; _k < %d; ++_k) if (_g + _k < _len_j) {' % vec)
+        src.append(_element_code(operands, operation, edge_load, edge_store, 12))
+        src.append('          }')
+    src.append('        }')
     src.append('      }')
     src.append('    }')
     if s_ops:

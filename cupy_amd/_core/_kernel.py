@@ -7,6 +7,7 @@ loop selection :1532-1753); what happens below the call surface -- stride
 canonicalisation into launch plans, the HIP emitters, argument packing -- is
 specific to this implementation.
 """
+import math
 import struct
 import threading
 import warnings
@@ -928,8 +929,8 @@ class _ElementwisePlanner:
         vector (zero stride along it), are read straight from memory; the
         other inputs are staged through the LDS in their own order.  Returns
         (tile, order of the axes for staging, staged names, zero-stride names,
-        vec, svec, axes of the contiguous piece, unit stride along the first
-        of them?) or None."""
+        vec, svec, axes of the contiguous pieces of the two passes, unit stride
+        along the first axis of the staging?) or None."""
         nd = len(cshape)
         names = [p.name for a, p in zip(args, self.params)
                  if isinstance(a, ndarray) and not p.raw]
@@ -974,116 +975,114 @@ class _ElementwisePlanner:
                 first_staged[ax] == 0, abs(first_staged[ax])))
         else:
             in_order = out_order
-        last, first = nd - 1, in_order[0]
-        # vectors along the last axis (second pass) and along the fastest axis
-        # of the staged inputs (first pass); short axes that are no whole
-        # number of vectors keep to what divides them
-        def widest(ax, members, limit_item):
-            v = max(1, 16 // limit_item)
-            while v > 1 and (v > cshape[ax] or (cshape[ax] < 12 * v and cshape[ax] % v)):
-                v //= 2
-            while v > 1:
-                nb_ok = True
-                for a, cs in members:
-                    nb = v * a.dtype.itemsize
-                    if not _aligned(a.data.ptr, nb) or not all(
-                            _aligned(c, nb) for k, c in enumerate(cs) if k != ax):
-                        nb_ok = False
-                if nb_ok:
-                    break
-                v //= 2
-            return v
+        first = in_order[0]
         direct = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'D']
+        zeros = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'Z']
         s_arrays = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'S']
-        s_item = max([a.dtype.itemsize for a, cs in s_arrays] or [1])
-        vec = widest(last, direct, max_item)
-        svec = 1
-        if s_arrays and all(cs[first] == a.dtype.itemsize for a, cs in s_arrays):
-            svec = widest(first, s_arrays, s_item)
-        max_v = 8192 if not lds_item else min(8192, (48 * 1024) // lds_item)
-        want = min(max_v, 4096 if max_item <= 4 else 2048 if max_item == 8 else 1024)
+        unit_first = all(cs[first] == a.dtype.itemsize for a, cs in s_arrays)
+        # elements of a tile: what the LDS image of the staged inputs allows, and
+        # enough for a few accesses per thread
+        limit = 32768 // max_item
+        max_v = limit if not lds_item else min(limit, (48 * 1024) // lds_item)
+        want = min(max_v, 16384 // max_item)
+        run = max(32, 256 // max_item)
         while True:
-            mult = [1] * nd
-            mult[last] = vec
-            mult[first] = max(mult[first], svec)
-            cap = [-(-e // m) * m for e, m in zip(cshape, mult)]
-            run = max(32, 256 // max_item)
-            while True:
-                tile = list(mult)
+            tile = [1] * nd
 
-                def grow(order):
-                    have = 1
-                    for ax in order:
-                        if have >= run:
-                            break
-                        need = -(-run // have)
-                        tile[ax] = max(tile[ax], min(cap[ax], -(-need // mult[ax]) * mult[ax]))
-                        have *= tile[ax]
-                        if tile[ax] < cshape[ax]:
-                            break
-                grow(out_order)
-                grow(in_order)
-                volume = internal.prod(tile)
-                if volume <= max_v or run <= 1:
-                    break
-                run //= 2
-            if volume > max_v:
-                return None
-            turn = 0
-            while internal.prod(tile) * 2 <= want:
-                for k in range(2):
-                    order = (out_order, in_order)[(turn + k) % 2]
-                    ax = next((x for x in order if tile[x] < cshape[x]), None)
-                    if ax is not None:
-                        tile[ax] = min(cap[ax], tile[ax] * 2)
-                        turn = (turn + k + 1) % 2
+            def grow(order):
+                have = 1
+                for ax in order:
+                    if have >= run:
                         break
+                    tile[ax] = max(tile[ax], min(cshape[ax], -(-run // have)))
+                    have *= tile[ax]
+                    if tile[ax] < cshape[ax]:
+                        break
+            grow(out_order)
+            grow(in_order)
+            if internal.prod(tile) <= max_v or run <= 1:
+                break
+            run //= 2
+        if internal.prod(tile) > max_v:
+            return None
+        turn = 0
+        while internal.prod(tile) * 2 <= want:
+            for k in range(2):
+                order = (out_order, in_order)[(turn + k) % 2]
+                ax = next((x for x in order if tile[x] < cshape[x]), None)
+                if ax is not None:
+                    tile[ax] = min(cshape[ax], tile[ax] * 2)
+                    turn = (turn + k + 1) % 2
+                    break
+            else:
+                break
+        # an axis cut in two unequal parts: whole if there is room, else in
+        # equal parts
+        for ax in range(nd):
+            if 1 < tile[ax] < cshape[ax]:
+                if cshape[ax] < 2 * tile[ax] and (
+                        internal.prod(tile) // tile[ax] * cshape[ax] <= max_v):
+                    tile[ax] = cshape[ax]
                 else:
-                    break
-            # an axis cut in two unequal parts: whole if there is room, else in
-            # equal parts
-            for ax in range(nd):
-                if 1 < tile[ax] < cshape[ax]:
-                    if cshape[ax] < 2 * tile[ax] and (
-                            internal.prod(tile) // tile[ax] * cap[ax] <= max_v):
-                        tile[ax] = cap[ax]
-                    else:
-                        parts = -(-cshape[ax] // tile[ax])
-                        even = -(-(-(-cshape[ax] // parts)) // mult[ax]) * mult[ax]
-                        tile[ax] = min(tile[ax], even)
-            # a tile that reaches past an axis that is no whole number of
-            # vectors would have no interior: narrower vectors there
-            if vec > 1 and tile[last] > cshape[last]:
-                vec //= 2
-                continue
-            if svec > 1 and tile[first] > cshape[first]:
-                svec //= 2
-                continue
-            break
-        # The first axes of the staged inputs that lie in them as one piece
-        group = 1
-        if s_arrays and all(cs[first] == a.dtype.itemsize for a, cs in s_arrays):
-            while group < nd:
-                a, b = in_order[group - 1], in_order[group]
+                    parts = -(-cshape[ax] // tile[ax])
+                    tile[ax] = min(tile[ax], -(-cshape[ax] // parts))
+
+        def piece_axes(order, members, others):
+            """How many of the first axes of ``order`` lie in ``members`` as one
+            contiguous piece within a tile (``others`` do not move along them)."""
+            count = 1
+            while count < nd:
+                a, b = order[count - 1], order[count]
                 if tile[a] != cshape[a] or tile[b] == 1 or not all(
-                        cs[b] == cs[a] * cshape[a] for arr, cs in s_arrays):
+                        cs[b] == cs[a] * cshape[a] for arr, cs in members) or any(
+                        cs[b] for arr, cs in others):
                     break
-                group += 1
-            if group > 1:
-                piece = internal.prod(tile[ax] for ax in in_order[:group])
-                svec = max(1, 16 // s_item)
-                while svec > 1 and (piece % svec or not all(
-                        _aligned(arr.data.ptr, svec * arr.dtype.itemsize) and all(
-                            _aligned(cs[ax], svec * arr.dtype.itemsize)
-                            for ax in in_order[group:])
-                        for arr, cs in s_arrays)):
-                    svec //= 2
-        unit_first = all(cs[first] == arr.dtype.itemsize for arr, cs in s_arrays)
-        return tuple(tile), tuple(in_order), staged, zero_last, vec, svec, group, unit_first
+                count += 1
+            return count
+
+        def widen(order, count, members, item):
+            """Widest access that divides the piece, the axis that cuts the piece
+            made a multiple of what that takes where it is not spanned whole."""
+            width = max(1, 16 // item)
+            cut = order[count - 1]
+            inner = internal.prod(tile[ax] for ax in order[:count - 1])
+            while width > 1:
+                step = width // math.gcd(inner, width)
+                if tile[cut] < cshape[cut] and tile[cut] % step:
+                    up = -(-tile[cut] // step) * step
+                    down = tile[cut] // step * step
+                    room = internal.prod(tile) // tile[cut]
+                    if up <= cshape[cut] and room * up <= max_v:
+                        tile[cut] = up
+                    elif down:
+                        tile[cut] = down
+                ok = (inner * tile[cut]) % width == 0
+                for arr, cs in members:
+                    nb = width * arr.dtype.itemsize
+                    if not _aligned(arr.data.ptr, nb) or not all(
+                            _aligned(cs[ax], nb) for ax in order[count:]):
+                        ok = False
+                if ok:
+                    break
+                width //= 2
+            return width
+
+        group, svec = 1, 1
+        if s_arrays and unit_first:
+            group = piece_axes(in_order, s_arrays, ())
+            svec = widen(in_order, group, s_arrays, max(a.dtype.itemsize for a, cs in s_arrays))
+        ogroup = piece_axes(out_order, direct, zeros)
+        vec = widen(out_order, ogroup, direct, max_item)
+        # (the second widening may have moved the axis the first one relied on)
+        if s_arrays and unit_first:
+            while svec > 1 and internal.prod(tile[ax] for ax in in_order[:group]) % svec:
+                svec //= 2
+        return (tuple(tile), tuple(in_order), staged, zero_last, vec, svec, group, ogroup,
+                unit_first)
 
     def _launch_packed(self, dev_id, args, nin, arrays, cshape, cstrides, plan, var_types,
                        typedefs, casts, force_read_out, stream_ptr, kernel_name, rec):
-        tile, in_order, staged, zero_last, vec, svec, group, unit_first = plan
+        tile, in_order, staged, zero_last, vec, svec, group, ogroup, unit_first = plan
         nd = len(cshape)
         threads = 256
         ntiles = 1
@@ -1110,8 +1109,8 @@ class _ElementwisePlanner:
         if staged and _tuning.get('packed_order') == 'in':
             tile_order = in_order
         key = ('packed', tile_order, tuple(o.key() for o in operands), typedefs, tile, in_order, staged,
-               zero_last, vec, svec, group, unit_first, idx64, dev_id, stream_hint, threads,
-               xcd)
+               zero_last, vec, svec, group, ogroup, unit_first, idx64, dev_id, stream_hint,
+               threads, xcd)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
@@ -1119,7 +1118,7 @@ class _ElementwisePlanner:
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, tile=tile, in_order=in_order,
                 staged=staged, zero_last=zero_last, vec=vec, svec=svec, group=group,
-                unit_first=unit_first, threads=threads, idx64=idx64, stream_hint=stream_hint,
+                ogroup=ogroup, unit_first=unit_first, threads=threads, idx64=idx64, stream_hint=stream_hint,
                 xcd=xcd, tile_order=tile_order)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'
