@@ -955,11 +955,17 @@ class _AbstractReductionKernel:
         ins = [in_args[i] for i in in_arr_idx]
         cus = _device.get_compute_units(device_id)
         vec = _max_vector_width([a.dtype.itemsize for a in ins])
+        # A lane keeps one state per column of its vector: 16 one-byte values
+        # with the four doubles of a variance each would be 512 bytes of
+        # registers, and 128 KiB of LDS for the fold across the waves
+        # (var over the middle axis of 2647 x 14 x 1780 int8: 435 us)
+        state_bytes = _reduce_type_bytes(reduce_type, typedefs)
+        while vec > 1 and vec * state_bytes > _tuning.get('cols_state_bytes_per_lane'):
+            vec //= 2
         if not batch and len(ins) == len([a for a in in_args if isinstance(a, ndarray)]):
             flat = self._cols_flat_geometry(
                 ins, n_out, n_red, so_in, sr, so_out, [out_args[i] for i in out_arr_idx], vec,
-                (map_expr, reduce_expr, post_map_expr),
-                _reduce_type_bytes(reduce_type, typedefs))
+                (map_expr, reduce_expr, post_map_expr), state_bytes)
             if flat is not None:
                 return self._launch_cols_flat(
                     flat, in_args, out_args, in_arr_idx, out_arr_idx, n_out, n_red, so_in, sr,

@@ -98,6 +98,7 @@ _params = {
     # of memory when reduced down their columns, the columns a lane meets
     # repeating from trip to trip.  'always': every width, whatever the column
     # kernel would make of it (for tests).
+    'cols_state_bytes_per_lane': 128,   # column reductions: widest vector whose per-column states fit this many bytes of a lane's registers
     'cols_flat': True,
     'cols_flat_min_bytes': 1 << 20,
     # ... every workgroup a run of consecutive trips (one contiguous piece of
