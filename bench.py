@@ -453,6 +453,30 @@ def build_layout_cases(cp):
         run('odd1', lambda: cp.cumsum(dflat[:n - 1])), lambda: np.cumsum(flat[:n - 1]),
         lambda: close(res['odd1'], np.cumsum(flat[:n - 1], dtype=np.float64), 1e-5,
                       np.cumsum(np.abs(flat[:n - 1]), dtype=np.float64)), 'cupy_scan_chain')
+    # ---- small trailing axes under a permutation: tiles that span several axes ------------------
+    m88, dm88 = flat.reshape(n // 64, 8, 8), dflat.reshape(n // 64, 8, 8)
+    add('(2^20,8,8) -> matrices transposed, copy f32', 2 * m88.nbytes,
+        run('m88', lambda: cp.ascontiguousarray(dm88.transpose(0, 2, 1))),
+        lambda: np.ascontiguousarray(m88.transpose(0, 2, 1)),
+        lambda: same(res['m88'], np.ascontiguousarray(m88.transpose(0, 2, 1))), 'cupy_copy')
+    nb43 = n // 12
+    h43 = flat[:nb43 * 12].astype(np.float16).reshape(nb43, 4, 3)
+    d43 = cp.asarray(h43)
+    add('(N,4,3) -> (N,3,4) copy f16', 2 * h43.nbytes,
+        run('m43', lambda: cp.ascontiguousarray(d43.transpose(0, 2, 1))),
+        lambda: np.ascontiguousarray(h43.transpose(0, 2, 1)),
+        lambda: same(res['m43'], np.ascontiguousarray(h43.transpose(0, 2, 1))), 'cupy_copy')
+    q4, dq4 = flat.reshape(4, n // 16, 4), dflat.reshape(4, n // 16, 4)
+    add('(4,2^22,4) -> axes reversed, copy f32', 2 * q4.nbytes,
+        run('q4', lambda: cp.ascontiguousarray(dq4.transpose(2, 1, 0))),
+        lambda: np.ascontiguousarray(q4.transpose(2, 1, 0)),
+        lambda: same(res['q4'], np.ascontiguousarray(q4.transpose(2, 1, 0))), 'cupy_copy')
+    r164 = flat.reshape(n // 64, 16, 4)
+    dr164 = dflat.reshape(n // 64, 16, 4)
+    mid = rng.standard_normal((n // 64, 1, 4), dtype=np.float32)
+    dmid = cp.asarray(mid)
+    add('(2^20,16,4) + (2^20,1,4) f32', 2 * r164.nbytes + mid.nbytes, run('mid', lambda: dr164 + dmid),
+        lambda: r164 + mid, lambda: same(res['mid'], r164 + mid), 'cupy_add')
     return cases
 
 

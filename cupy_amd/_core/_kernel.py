@@ -455,19 +455,17 @@ class _ElementwisePlanner:
                             dev_id, args, nin, arrays, plan, var_types, typedefs, casts,
                             force_read_out, stream_ptr, kernel_name, rec)
                     plan = self._plan_batched(arrays, cshape, cstrides, args, nin)
-                # Tiles over several axes (emit_packed) wherever they apply,
-                # except for large tiles of two axes in arrays whose rows do not
-                # start on cache lines: the tiled kernel walks those in strips
-                # that keep neighbours on one die (2^26 float32 over permuted
-                # copies, us, tiles of two axes / of several: (524288, 8, 8) to
-                # (.., 8, 8) transposed 806 / 39; (4, 2^21, 4) reversed 3124 / 38;
-                # (256, 512, 512) as (0, 2, 1) 90 / 76; (255, 511, 513) as
-                # (0, 2, 1) 114 / 136; (4226, 68, 4, 29) as (2, 1, 3, 0) 59 / 97)
+                # Tiles over several axes (emit_packed) where tiles of two axes
+                # would be small or narrow: those are mostly edge, or one tile per
+                # small matrix (2^26 float32 over rotating buffers, us, tiles of
+                # two axes / of several: (2^20, 8, 8) with its matrices transposed
+                # 1591 / 86; (2^18, 16, 16) 340 / 86; (4, 2^22, 4) reversed
+                # 6271 / 102; large tiles of two axes stay ahead: (256, 512, 512)
+                # as (0, 2, 1) 87 / 94, as (2, 1, 0) 94 / 112)
                 mode_p = _tuning.get('packed_tiles')
                 if mode_p and not (mode_p == 'auto' and plan is not None
                                    and plan[0][0] * plan[0][1] >= _tuning.get('packed_tiles_below')
-                                   and min(plan[0]) >= 16
-                                   and _off_lines(arrays, cstrides)):
+                                   and min(plan[0]) >= 16):
                     packed = self._plan_packed(arrays, cshape, cstrides, args, nin)
                     if packed is not None:
                         return self._launch_packed(
@@ -1100,8 +1098,11 @@ class _ElementwisePlanner:
             # tiles share the cache lines at their borders wherever a run is no
             # whole number of lines: plain accesses let the cache put them together
             item = min(a.dtype.itemsize for a in arrays)
-            whole = (tile[-1] * item) % 128 == 0 and not _off_lines(arrays, cstrides)
-            stream_hint = (stream_hint[0] and whole and not staged, stream_hint[1] and whole)
+            aligned = not _off_lines(arrays, cstrides)
+            piece_in = internal.prod(tile[ax] for ax in in_order[:group]) * item
+            piece_out = internal.prod(tile[ax] for ax in range(nd - ogroup, nd)) * item
+            stream_hint = (stream_hint[0] and aligned and piece_in % 128 == 0,
+                           stream_hint[1] and aligned and piece_out % 128 == 0)
         # tiles whose borders fall inside cache lines: neighbours on one die
         mode = _tuning.get('packed_xcd')
         xcd = bool(mode) and (mode is True or _off_lines(arrays, cstrides))
