@@ -933,8 +933,8 @@ def emit_tiled2d(name, operands, operation, typedefs='', preamble='',
 
 def emit_packed(name, operands, operation, typedefs='', preamble='',
                 loop_prep='', after_loop='', tile=(), in_order=(), staged=(),
-                zero_last=(), vec=1, svec=1, group=1, ogroup=1, unit_first=True,
-                threads=256, idx64=False, stream_hint=True, xcd=False, tile_order=None):
+                zero_last=(), zero_moving=(), vec=1, svec=1, group=1, ogroup=1,
+                unit_first=True, threads=256, idx64=False, stream_hint=True, xcd=False, tile_order=None):
     """Kernel for an index space of ``len(tile)`` axes whose arrays are
     permuted differently, with a tile that spans SEVERAL axes: as many of the
     last axes as give the outputs a long contiguous run, and as many of the
@@ -960,8 +960,10 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
     of its axes, and every element finds its own place in the image.
     ``unit_first``: every staged input has unit stride along ``in_order[0]``
     (else ``svec`` and ``group`` are 1 and the stride is applied).  ``ogroup``:
-    the same for the last axes and the arrays of the second pass (the inputs of
-    ``zero_last`` have zero stride along all of these axes).  At the border of
+    the same for the last axes and the arrays of the second pass; the inputs of
+    ``zero_last`` give one value per access, those also named in
+    ``zero_moving`` (a value per row under a piece of several rows) one per
+    element.  At the border of
     the array a piece is shorter, never split: only its last axis can be cut.
 
     ``tile[a]`` elements along axis a; tiles are numbered along the axes of
@@ -1140,11 +1142,22 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
     def address(op):
         return '(_b_%s + %s)' % (op.name, rest_offset(op, rest, '_j'))
 
+    # inputs with zero stride along the last axis: one value per access where
+    # they do not move along the other axes of the piece either (``_s<a>`` may
+    # be anything there: the host says which), else one per element
+    def zero_value(op):
+        if op.name not in zero_moving:
+            return '_z_%s' % op.name
+        idx = split(g_axes, '_g + _k')
+        terms = ['(ptrdiff_t)%s * _s%d_%s' % (idx[a], a, op.name)
+                 for a in g_axes[1:] if tile[a] > 1]
+        return '%s[%s]' % (address(op), ' + '.join(terms) or '0')
+
     def full_load(op):
         if op.name in staged:
             return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
         if op.name in zero_last:
-            return '_z_%s' % op.name
+            return zero_value(op)
         return '_l_%s.v[_k]' % op.name
 
     def full_store(op, value):
@@ -1154,7 +1167,7 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
         if op.name in staged:
             return '_t_%s[%s]' % (op.name, pad('_pos + _k'))
         if op.name in zero_last:
-            return '_z_%s' % op.name
+            return zero_value(op)
         return '%s[_g + _k]' % address(op)
 
     def edge_store(op, value):
@@ -1162,7 +1175,7 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
 
     src.append('      if (%s(_interior || (%s))) {' % (guard, rest_inside(rest, '_j')))
     for op in d_ops:
-        if op.name in zero_last:
+        if op.name in zero_last and op.name not in zero_moving:
             src.append('        const %s _z_%s = *%s;' % (op.store_t, op.name, address(op)))
     src.append('        if (_g + %d <= _len_j) {' % vec)
     for op in d_ops:

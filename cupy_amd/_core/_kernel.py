@@ -272,23 +272,28 @@ def _get_out_args_with_params(out_args, out_types, out_shape, out_params,
 def _canonical_dims(arrays, shape):
     """Merges axes that every array walks back to back and drops unit axes.
     Returns (shape, [strides per array]) of the equivalent smaller problem."""
+    return _merge_axes(shape, [a._strides for a in arrays])
+
+
+def _merge_axes(shape, strides):
+    """``_canonical_dims`` for a shape and the strides of every array along it."""
     cshape = []
-    cstrides = [[] for _ in arrays]
+    cstrides = [[] for _ in strides]
     for d, ext in enumerate(shape):
         if ext == 1:
             continue
         if cshape:
-            for cs, a in zip(cstrides, arrays):
-                if cs[-1] != a._strides[d] * ext:
+            for cs, st in zip(cstrides, strides):
+                if cs[-1] != st[d] * ext:
                     break
             else:
                 cshape[-1] *= ext
-                for cs, a in zip(cstrides, arrays):
-                    cs[-1] = a._strides[d]
+                for cs, st in zip(cstrides, strides):
+                    cs[-1] = st[d]
                 continue
         cshape.append(ext)
-        for cs, a in zip(cstrides, arrays):
-            cs.append(a._strides[d])
+        for cs, st in zip(cstrides, strides):
+            cs.append(st[d])
     return tuple(cshape), [tuple(cs) for cs in cstrides]
 
 
@@ -417,6 +422,22 @@ class _ElementwisePlanner:
         if not (force_generic or self._force_generic) and arrays:
             cshape, cstrides = _canonical_dims(arrays, shape)
             nd = len(cshape)
+            if nd >= 3 and not self._uses_i and not self._uses_ind and _tuning.get(
+                    'order_by_outputs'):
+                # An elementwise operation may visit its elements in any order:
+                # the axes are taken in the order the OUTPUTS are stored in, so
+                # that a permuted destination (dst.transpose(...)[...] = x) is
+                # the array that is walked along its memory, and x the permuted one
+                outs = args[nin:]
+                ref = next((cs for a, cs in zip(arrays, cstrides)
+                            if any(a is o for o in outs)), None)
+                if ref is not None:
+                    order = sorted(range(nd), key=lambda ax: -abs(ref[ax]))
+                    if order != list(range(nd)):
+                        cshape, cstrides = _merge_axes(
+                            [cshape[ax] for ax in order],
+                            [[cs[ax] for ax in order] for cs in cstrides])
+                        nd = len(cshape)
             if nd <= 1:
                 ok = True
                 for a, cs in zip(arrays, cstrides):
@@ -440,6 +461,20 @@ class _ElementwisePlanner:
                         dev_id, args, nin, arrays, cstrides, size, var_types, typedefs,
                         casts, force_read_out, stream_ptr, kernel_name, rec,
                         partial=part, nc=cshape[1])
+                # rows of a few one- or two-byte elements that do not follow one
+                # another without gaps (windows of narrow matrices): tiles of many
+                # rows, the inputs staged through the LDS, the outputs written as
+                # one piece (float16 (11184809, 6), x[:-1, :-1] - x[1:, 1:]: 99 us
+                # row by row, 65 so; four- and eight-byte elements gain nothing)
+                if (not self._uses_i and _tuning.get('packed_tiles')
+                        and min(a.dtype.itemsize for a in arrays) < 4
+                        and cshape[1] * max(a.dtype.itemsize for a in arrays)
+                        < _tuning.get('packed_short_rows_bytes')):
+                    packed = self._plan_packed(arrays, cshape, cstrides, args, nin)
+                    if packed is not None:
+                        return self._launch_packed(
+                            dev_id, args, nin, arrays, cshape, cstrides, packed, var_types,
+                            typedefs, casts, force_read_out, stream_ptr, kernel_name, rec)
                 plan = self._plan_rows2d(arrays, cshape, cstrides, args, nin)
                 if plan is not None:
                     return self._launch_rows2d(
@@ -927,7 +962,7 @@ class _ElementwisePlanner:
         vector (zero stride along it), are read straight from memory; the
         other inputs are staged through the LDS in their own order.  Returns
         (tile, order of the axes for staging, staged names, zero-stride names,
-        vec, svec, axes of the contiguous pieces of the two passes, unit stride
+        those of them that move within a piece, vec, svec, axes of the contiguous pieces of the two passes, unit stride
         along the first axis of the staging?) or None."""
         nd = len(cshape)
         names = [p.name for a, p in zip(args, self.params)
@@ -975,7 +1010,6 @@ class _ElementwisePlanner:
             in_order = out_order
         first = in_order[0]
         direct = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'D']
-        zeros = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'Z']
         s_arrays = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'S']
         unit_first = all(cs[first] == a.dtype.itemsize for a, cs in s_arrays)
         # elements of a tile: what the LDS image of the staged inputs allows, and
@@ -1069,18 +1103,22 @@ class _ElementwisePlanner:
         if s_arrays and unit_first:
             group = piece_axes(in_order, s_arrays, ())
             svec = widen(in_order, group, s_arrays, max(a.dtype.itemsize for a, cs in s_arrays))
-        ogroup = piece_axes(out_order, direct, zeros)
+        ogroup = piece_axes(out_order, direct, ())
+        zero_moving = tuple(sorted(
+            nm for (a, cs, nm) in zip(arrays, cstrides, names)
+            if kinds[nm] == 'Z' and any(cs[ax] for ax in out_order[1:ogroup])))
         vec = widen(out_order, ogroup, direct, max_item)
         # (the second widening may have moved the axis the first one relied on)
         if s_arrays and unit_first:
             while svec > 1 and internal.prod(tile[ax] for ax in in_order[:group]) % svec:
                 svec //= 2
-        return (tuple(tile), tuple(in_order), staged, zero_last, vec, svec, group, ogroup,
-                unit_first)
+        return (tuple(tile), tuple(in_order), staged, zero_last, zero_moving, vec, svec, group,
+                ogroup, unit_first)
 
     def _launch_packed(self, dev_id, args, nin, arrays, cshape, cstrides, plan, var_types,
                        typedefs, casts, force_read_out, stream_ptr, kernel_name, rec):
-        tile, in_order, staged, zero_last, vec, svec, group, ogroup, unit_first = plan
+        (tile, in_order, staged, zero_last, zero_moving, vec, svec, group, ogroup,
+         unit_first) = plan
         nd = len(cshape)
         threads = 256
         ntiles = 1
@@ -1110,16 +1148,16 @@ class _ElementwisePlanner:
         if staged and _tuning.get('packed_order') == 'in':
             tile_order = in_order
         key = ('packed', tile_order, tuple(o.key() for o in operands), typedefs, tile, in_order, staged,
-               zero_last, vec, svec, group, ogroup, unit_first, idx64, dev_id, stream_hint,
-               threads, xcd)
+               zero_last, zero_moving, vec, svec, group, ogroup, unit_first, idx64, dev_id,
+               stream_hint, threads, xcd)
         entry = self._memo.get(key)
         if entry is None:
             name = kernel_name or self.name
             code = _cg.emit_packed(
                 name, operands, self.operation, typedefs, self.preamble,
                 self.loop_prep, self.after_loop, tile=tile, in_order=in_order,
-                staged=staged, zero_last=zero_last, vec=vec, svec=svec, group=group,
-                ogroup=ogroup, unit_first=unit_first, threads=threads, idx64=idx64, stream_hint=stream_hint,
+                staged=staged, zero_last=zero_last, zero_moving=zero_moving, vec=vec, svec=svec,
+                group=group, ogroup=ogroup, unit_first=unit_first, threads=threads, idx64=idx64, stream_hint=stream_hint,
                 xcd=xcd, tile_order=tile_order)
             fn = compiler.compile_with_cache(code, self.options).get_function(name)
             ic = 'q' if idx64 else 'i'

@@ -59,8 +59,10 @@ _params = {
     'tiled_tile': None,         # (rows, columns, threads) of a staged tile; None: by shape
     'tiled_xcd': 'auto',        # tiles numbered die by die: 'auto' (operands off the cache lines), True, False
     'tiled_xcd_strip': 16,      # ... a die walking strips of this many tiles across (transposed copy of 8191 x 8193 float32: 136 us in diagonal order, 116 / 110 / 108 / 105 / 118 with strips of 2 / 4 / 8 / 16 / 64)
+    'order_by_outputs': True,   # problems of three and more axes are walked in the order their outputs are stored in
     'packed_tiles': 'auto',     # tiles over several axes for 3-d and 4-d problems: 'auto' where tiles of two axes would be small, True wherever they apply, False never
     'packed_order': 'out',      # ... numbered along the axes of the outputs ('out') or of the staged inputs ('in'), fastest first
+    'packed_short_rows_bytes': 64,   # ... also for matrices whose rows are shorter than this and do not merge into one run
     'packed_xcd': 'auto',       # ... numbered die by die: 'auto' where their borders fall inside cache lines
     'packed_tiles_below': 2048,  # ... 'auto': where the two tiled axes together hold fewer elements than this
     'tiled_big_min': 256,       # extent of both tile axes from which tiles are 128 x 128

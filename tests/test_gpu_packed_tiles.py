@@ -15,7 +15,8 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(autouse=True)
 def _restore_settings():
     yield
-    _tuning.set(packed_tiles='auto', packed_xcd='auto', packed_tiles_below=2048)
+    _tuning.set(packed_tiles='auto', packed_xcd='auto', packed_tiles_below=2048,
+                order_by_outputs=True, packed_short_rows_bytes=64)
 
 
 def _values(shape, dtype, seed=0):
@@ -148,3 +149,62 @@ def test_large_batches_of_small_matrices_transposed():
                                       np.ascontiguousarray(h.transpose(perm)))
         np.testing.assert_array_equal((d.transpose(perm) + d.transpose(perm)).get(),
                                       h.transpose(perm) * 2)
+
+
+@pytest.mark.parametrize('by_outputs', [True, False])
+def test_permuted_destinations(by_outputs):
+    _tuning.set(order_by_outputs=by_outputs)
+    rng = np.random.default_rng(3)
+    for shape in [(37, 9, 14, 4), (120, 5, 33), (6, 7, 8, 9, 3), (2, 300, 4, 3)]:
+        nd = len(shape)
+        h = _values(shape, 'float32')
+        d = cp.asarray(h)
+        for trial in range(8):
+            perm = tuple(int(p) for p in rng.permutation(nd))
+            base = cp.zeros(tuple(shape[p] for p in np.argsort(perm)), 'float64')
+            dst = base.transpose(perm)
+            assert dst.shape == shape
+            cp.copyto(dst, d)
+            np.testing.assert_array_equal(base.get(), np.ascontiguousarray(h.transpose(np.argsort(perm))),
+                                          err_msg='%s %s' % (shape, perm))
+            # two inputs stored in other orders again, written into the permuted destination
+            other = tuple(int(p) for p in rng.permutation(nd))
+            hb = _values(tuple(shape[p] for p in np.argsort(other)), 'float32', 9).transpose(other)
+            db = cp.asarray(np.ascontiguousarray(hb.transpose(np.argsort(other)))).transpose(other)
+            cp.multiply(d, db, out=dst)
+            np.testing.assert_array_equal(dst.get(), h * hb)
+
+
+def test_a_value_per_row_under_pieces_of_several_rows():
+    for shape, dtype in [((3, 15983, 7), 'float32'), ((4001, 5, 3), 'float64'), ((2, 9, 1001, 6), 'float16')]:
+        h = _values(shape, dtype)
+        d = cp.asarray(h)
+        for axis in range(len(shape) - 1):
+            mshape = [1] * len(shape)
+            mshape[axis] = shape[axis]
+            hm = _values(tuple(mshape), dtype, 4)
+            dm = cp.asarray(hm)
+            np.testing.assert_array_equal((d - dm).get(), h - hm)
+            fused = cp.fuse(lambda a, b, c: (a - b) * c)
+            np.testing.assert_array_equal(fused(d, dm, dm).get(), (h - hm) * hm)
+            # one value per row of the two last axes together
+            mshape[-1] = shape[-1]
+            hm = _values(tuple(mshape), dtype, 5)
+            np.testing.assert_array_equal((d + cp.asarray(hm)).get(), h + hm)
+
+
+def test_windows_of_narrow_matrices_of_small_elements():
+    for dtype in ('uint8', 'float16', 'int16', 'bool'):
+        for shape in [(100003, 6), (50001, 13), (33333, 31), (70001, 2)]:
+            h = _values(shape, dtype)
+            d = cp.asarray(h)
+            if dtype == 'bool':
+                np.testing.assert_array_equal((d[:-1, :-1] ^ d[1:, 1:]).get(), h[:-1, :-1] ^ h[1:, 1:])
+            else:
+                np.testing.assert_array_equal((d[:-1, :-1] - d[1:, 1:]).get(), h[:-1, :-1] - h[1:, 1:])
+            np.testing.assert_array_equal((d[:, 1:] + d[:, :-1]).get(), h[:, 1:] + h[:, :-1])
+            out = cp.zeros((shape[0], shape[1] + 2), dtype)
+            cp.copyto(out[:, 1:-1], d)
+            want = np.zeros((shape[0], shape[1] + 2), dtype)
+            want[:, 1:-1] = h
+            np.testing.assert_array_equal(out.get(), want)
