@@ -1051,8 +1051,10 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
         g_len = 1
         for a in g_axes:
             g_len *= tile[a]
-        assert g_len % width == 0
-        slots = volume // width
+        # (a piece that is no whole number of accesses ends in a partial one,
+        # which goes element by element like those at the border of the array)
+        per = -(-g_len // width)
+        slots = (volume // g_len) * per
         trips = -(-slots // threads)
         cut = g_axes[-1]
         src.append('    const int _len%s = %d * (int)((_e%d - _o%d < %d) ? (_e%d - _o%d) : %d);' % (
@@ -1060,8 +1062,8 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
         src.append(unroll(trips))
         src.append('    for (int _it = 0; _it < %d; ++_it) {' % trips)
         src.append('      const int _v = threadIdx.x + _it * %d;' % threads)
-        src.append('      const int _g = (_v %% %d) * %d; int _r = _v / %d;' % (
-            g_len // width, width, g_len // width))
+        src.append('      const int _g = (_v %% %d) * %d; int _r = _v / %d;' % (per, width, per))
+        src.append('      const int _first = _r * %d + _g;' % g_len)
         for n, a in enumerate(rest):
             if tile[a] == 1:
                 src.append('      const int %s%d = 0;' % (prefix, a))
@@ -1136,7 +1138,7 @@ def emit_packed(name, operands, operation, typedefs='', preamble='',
 
     # ---- second pass: the tile in the order of the outputs ---------------------------------------
     g_axes, rest, slots, trips = one_pass(out_order, ogroup, vec, '_j')
-    src.append('      const int _pos = _v * %d;' % vec)
+    src.append('      const int _pos = _first;')
     guard = '' if slots % threads == 0 else '_v < %d && ' % slots
 
     def address(op):

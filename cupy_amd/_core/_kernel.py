@@ -498,9 +498,11 @@ class _ElementwisePlanner:
                 # 6271 / 102; large tiles of two axes stay ahead: (256, 512, 512)
                 # as (0, 2, 1) 87 / 94, as (2, 1, 0) 94 / 112)
                 mode_p = _tuning.get('packed_tiles')
+                # (rows shorter than a tile of two axes is wide make every such
+                # tile an edge tile, which goes element by element)
                 if mode_p and not (mode_p == 'auto' and plan is not None
                                    and plan[0][0] * plan[0][1] >= _tuning.get('packed_tiles_below')
-                                   and min(plan[0]) >= 16):
+                                   and min(plan[0]) >= 16 and plan[0][1] >= 64):
                     packed = self._plan_packed(arrays, cshape, cstrides, args, nin)
                     if packed is not None:
                         return self._launch_packed(
@@ -1088,7 +1090,8 @@ class _ElementwisePlanner:
                         tile[cut] = up
                     elif down:
                         tile[cut] = down
-                ok = (inner * tile[cut]) % width == 0
+                # (a piece of several accesses may end in a partial one)
+                ok = (inner * tile[cut]) % width == 0 or inner * tile[cut] >= 4 * width
                 for arr, cs in members:
                     nb = width * arr.dtype.itemsize
                     if not _aligned(arr.data.ptr, nb) or not all(
@@ -1110,7 +1113,8 @@ class _ElementwisePlanner:
         vec = widen(out_order, ogroup, direct, max_item)
         # (the second widening may have moved the axis the first one relied on)
         if s_arrays and unit_first:
-            while svec > 1 and internal.prod(tile[ax] for ax in in_order[:group]) % svec:
+            piece = internal.prod(tile[ax] for ax in in_order[:group])
+            while svec > 1 and piece % svec and piece < 4 * svec:
                 svec //= 2
         return (tuple(tile), tuple(in_order), staged, zero_last, zero_moving, vec, svec, group,
                 ogroup, unit_first)
