@@ -32,7 +32,7 @@ from cupy_amd._core._kernel import (
     _get_out_args_from_optionals, _get_out_args_with_params,
     _check_peer_access, _scalar_struct_code, _make_packer, _max_blocks, _max_vector_width, _aligned)
 from cupy_amd._core._scalar import CScalar, get_typename as _get_typename
-from cupy_amd._core.core import ndarray, _convert_from_cupy_like
+from cupy_amd._core.core import ndarray, _ascontiguous, _convert_from_cupy_like
 from cupy_amd.cuda import compiler
 from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import memory as _memory
@@ -359,6 +359,46 @@ class _AbstractReductionKernel:
                     [a.dtype.itemsize for a in outs], map_expr, reduce_expr,
                     post_map_expr, reduce_type, typedefs, device_id, stream_ptr, rec,
                     batch=(n_batch, n_inner, [os_[0] for os_ in o_in]))
+        # Kept and reduced axes interleaved with an innermost axis of a few
+        # elements: the indexer kernel would walk the input in pieces of a few
+        # bytes, and the staged form below would fold very many partial results
+        # per output.  The input is copied once with the reduced axes last --
+        # the permuted copy runs near the streaming rate -- and reduced row by
+        # row: three passes over the data, and still ahead (us, before / so:
+        # any over axes (1, 3) of 833 x 126 x 80 x 4 int32 149 / 61; sum over
+        # (0, 3) of 1000 x 64 x 256 x 3 float16 133 / 52).  Longer innermost
+        # axes are better off as they are (sum over (1, 3) of 64 x 100 x 64 x 100
+        # float32 63 / 85), and so are one-byte elements (their copies are slow).
+        if (in_arr_idx and len(in_arr_idx) == 1 and not has_raw and not needs_indexers
+                and n_r and out_axis and _tuning.get('reduce_via_copy')
+                and not any(uses_identifier(e, '_J') for e in exprs)):
+            src = in_args[in_arr_idx[0]]
+            size = internal.prod(a_shape)
+            item = src.dtype.itemsize
+            special = len(rshape) <= 1 and len(oshape) <= 2
+            if (not special and item >= 2 and a_shape[-1] * item < 64
+                    and tuple(src._shape) == tuple(a_shape)
+                    and _tuning.get('reduce_via_copy_min') <= size
+                    and src.nbytes <= (8 << 30)):
+                perm = tuple(out_axis) + tuple(reduce_axis)
+                if stream is None:
+                    tmp = _ascontiguous(src.transpose(perm))
+                else:
+                    with stream:
+                        tmp = _ascontiguous(src.transpose(perm))
+                new_in = list(in_args)
+                new_in[in_arr_idx[0]] = tmp
+                new_out = list(out_args)
+                if keepdims:
+                    for i in out_arr_idx:
+                        o = out_args[i]
+                        new_out[i] = o._view(kept_shape, tuple(o._strides[d] for d in out_axis))
+                n_k = len(out_axis)
+                return self._launch(
+                    new_in, new_out, tuple(a_shape[p] for p in perm),
+                    tuple(range(n_k, len(perm))), tuple(range(n_k)), False,
+                    map_expr, reduce_expr, post_map_expr, reduce_type, typedefs,
+                    device_id, stream, None)
         # reduction over an outer and the innermost axis, in[r0, c, r1] -> out[c]
         # (e.g. per-channel statistics of a batch of images): the rows kernel
         # reduces r1 for every (r0, c) into partial results, which the combine

@@ -100,6 +100,8 @@ _params = {
     # of memory when reduced down their columns, the columns a lane meets
     # repeating from trip to trip.  'always': every width, whatever the column
     # kernel would make of it (for tests).
+    'reduce_via_copy': True,    # reductions over interleaved kept and reduced axes: copy with the reduced axes last, then reduce rows
+    'reduce_via_copy_min': 1 << 18,   # ... from this many elements
     'cols_state_bytes_per_lane': 128,   # column reductions: widest vector whose per-column states fit this many bytes of a lane's registers
     'cols_flat': True,
     'cols_flat_min_bytes': 1 << 20,

@@ -615,3 +615,50 @@ def test_column_blocks_numbered_die_by_die(shape, axis, mode):
         assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(scale, 1))
     finally:
         _tuning.set(cols_xcd='auto')
+
+
+@pytest.mark.parametrize('via_copy', [True, False])
+def test_interleaved_kept_and_reduced_axes_with_a_tiny_innermost_axis(via_copy):
+    # kept and reduced axes alternate and the last axis holds a few elements: the
+    # input is copied with the reduced axes last and reduced row by row
+    from cupy_amd._core import _tuning
+    _tuning.set(reduce_via_copy=via_copy)
+    try:
+        rng = np.random.default_rng(17)
+        for shape, dtype in [((83, 126, 40, 4), 'int32'), ((100, 64, 50, 3), 'float32'),
+                             ((3000, 50, 3, 2), 'float64'), ((257, 33, 65, 5), 'float16'),
+                             ((70000, 8, 5), 'float32')]:
+            h = rng.integers(-3, 4, size=shape).astype(dtype)
+            d = cp.asarray(h)
+            nd = len(shape)
+            axes = [(1, 3), (0, 2), (0, 1, 3), (0, 3), (1, 2)] if nd == 4 else [(0, 2)]
+            for axis in axes:
+                for keepdims in (False, True):
+                    got = d.sum(axis=axis, keepdims=keepdims)
+                    want = h.sum(axis=axis, keepdims=keepdims, dtype=np.float64 if h.dtype.kind == 'f' else None)
+                    assert got.shape == want.shape
+                    np.testing.assert_allclose(got.get().astype(np.float64), want, rtol=2e-3)
+                np.testing.assert_array_equal(d.max(axis=axis).get(), h.max(axis=axis))
+                np.testing.assert_array_equal(d.any(axis=axis).get(), h.any(axis=axis))
+                if h.dtype.kind == 'f' and h.dtype.itemsize >= 4:
+                    np.testing.assert_allclose(d.var(axis=axis).get(), h.var(axis=axis, dtype=np.float64),
+                                               rtol=1e-4)
+                    np.testing.assert_allclose(d.mean(axis=axis).get(), h.mean(axis=axis, dtype=np.float64),
+                                               rtol=1e-5, atol=1e-6)
+            # into a given output, on another stream, from a view
+            axis = axes[0]
+            out = cp.zeros(h.sum(axis=axis).shape, d.sum(axis=axis).dtype)
+            with cp.cuda.Stream() as s:
+                v = d[1:]
+                v.sum(axis=axis, out=out[1:] if 0 not in axis else out)
+                s.synchronize()
+            want = h[1:].sum(axis=axis)
+            np.testing.assert_allclose((out[1:] if 0 not in axis else out).get().astype(np.float64),
+                                       want.astype(np.float64), rtol=2e-3)
+            # the same call again (nothing of the copy may be replayed from a record)
+            h2 = h + 1
+            d2 = cp.asarray(h2)
+            for _ in range(2):
+                np.testing.assert_array_equal(d2.max(axis=axes[0]).get(), h2.max(axis=axes[0]))
+    finally:
+        _tuning.set(reduce_via_copy=True)
