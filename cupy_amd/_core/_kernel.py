@@ -1018,7 +1018,7 @@ class _ElementwisePlanner:
         # enough for a few accesses per thread
         limit = 32768 // max_item
         max_v = limit if not lds_item else min(limit, (48 * 1024) // lds_item)
-        want = min(max_v, 16384 // max_item)
+        want = min(max_v, _tuning.get('packed_tile_bytes') // max_item)
         run = max(32, 256 // max_item)
         while True:
             tile = [1] * nd
@@ -1124,7 +1124,7 @@ class _ElementwisePlanner:
         (tile, in_order, staged, zero_last, zero_moving, vec, svec, group, ogroup,
          unit_first) = plan
         nd = len(cshape)
-        threads = 256
+        threads = _tuning.get('packed_threads')
         ntiles = 1
         span = 0
         for e, t in zip(cshape, tile):

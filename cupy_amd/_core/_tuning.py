@@ -63,6 +63,8 @@ _params = {
     'packed_tiles': 'auto',     # tiles over several axes for 3-d and 4-d problems: 'auto' where tiles of two axes would be small, True wherever they apply, False never
     'packed_order': 'out',      # ... numbered along the axes of the outputs ('out') or of the staged inputs ('in'), fastest first
     'packed_short_rows_bytes': 64,   # ... also for matrices whose rows are shorter than this and do not merge into one run
+    'packed_tile_bytes': 16384,  # ... of about this many bytes per array
+    'packed_threads': 256,      # ... a workgroup of this many threads each
     'packed_xcd': 'auto',       # ... numbered die by die: 'auto' where their borders fall inside cache lines
     'packed_tiles_below': 2048,  # ... 'auto': where the two tiled axes together hold fewer elements than this
     'tiled_big_min': 256,       # extent of both tile axes from which tiles are 128 x 128
