@@ -964,8 +964,9 @@ class _ElementwisePlanner:
         vector (zero stride along it), are read straight from memory; the
         other inputs are staged through the LDS in their own order.  Returns
         (tile, order of the axes for staging, staged names, zero-stride names,
-        those of them that move within a piece, vec, svec, axes of the contiguous pieces of the two passes, unit stride
-        along the first axis of the staging?) or None."""
+        those of them that move within a piece, vec, svec, axes of the
+        contiguous pieces of the two passes, unit stride along the first axis
+        of the staging?) or None."""
         nd = len(cshape)
         names = [p.name for a, p in zip(args, self.params)
                  if isinstance(a, ndarray) and not p.raw]
