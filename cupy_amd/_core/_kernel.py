@@ -1107,7 +1107,16 @@ class _ElementwisePlanner:
         if s_arrays and unit_first:
             group = piece_axes(in_order, s_arrays, ())
             svec = widen(in_order, group, s_arrays, max(a.dtype.itemsize for a, cs in s_arrays))
-        ogroup = piece_axes(out_order, direct, ())
+        # Inputs with a value per row: pieces of whole rows where a row is a
+        # long enough run by itself (the value is then read once per access),
+        # pieces of several rows with the value looked up per element where rows
+        # are a few elements (float16 (171840, 5, 78) with a value per middle
+        # index: 160 us per element, rows of 7 float32 the other way round)
+        zeros = [(a, cs) for a, cs, nm in zip(arrays, cstrides, names) if kinds[nm] == 'Z']
+        ogroup = piece_axes(out_order, direct, zeros)
+        if zeros and internal.prod(tile[ax] for ax in out_order[:ogroup]) * min(
+                a.dtype.itemsize for a, cs in direct) < 64:
+            ogroup = piece_axes(out_order, direct, ())
         zero_moving = tuple(sorted(
             nm for (a, cs, nm) in zip(arrays, cstrides, names)
             if kinds[nm] == 'Z' and any(cs[ax] for ax in out_order[1:ogroup])))
