@@ -381,11 +381,17 @@ class _AbstractReductionKernel:
                     and _tuning.get('reduce_via_copy_min') <= size
                     and src.nbytes <= (8 << 30)):
                 perm = tuple(out_axis) + tuple(reduce_axis)
-                if stream is None:
-                    tmp = _ascontiguous(src.transpose(perm))
-                else:
-                    with stream:
+                try:
+                    if stream is None:
                         tmp = _ascontiguous(src.transpose(perm))
+                    else:
+                        with stream:
+                            tmp = _ascontiguous(src.transpose(perm))
+                except MemoryError:
+                    tmp = None        # no room for the copy: the input as it is
+            else:
+                tmp = None
+            if tmp is not None:
                 new_in = list(in_args)
                 new_in[in_arr_idx[0]] = tmp
                 new_out = list(out_args)
