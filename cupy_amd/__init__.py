@@ -20,7 +20,12 @@ __version__ = '0.1.0'
 from numpy import (  # noqa
     bool_, int8, int16, int32, int64, uint8, uint16, uint32, uint64,
     float16, float32, float64, complex64, complex128, dtype, newaxis, inf, nan, pi, e)
-from numpy import result_type, can_cast, promote_types  # noqa
+from numpy import (  # noqa
+    result_type, can_cast, promote_types, broadcast_shapes, issubdtype, finfo, iinfo,
+    min_scalar_type, isdtype,
+    generic, number, integer, signedinteger, unsignedinteger, inexact, floating,
+    complexfloating, byte, ubyte, short, ushort, intc, uintc, int_, uint, intp, uintp,
+    longlong, ulonglong, half, single, double, csingle, cdouble, euler_gamma)
 from numpy.exceptions import AxisError, ComplexWarning  # noqa
 
 # -- memory pool -------------------------------------------------------------------
@@ -97,6 +102,12 @@ from cupy_amd._core._routines_logic import all, any  # noqa
 from cupy_amd._core._scan import cumsum, cumprod, nancumsum, nancumprod  # noqa
 from cupy_amd._creation import (  # noqa
     empty, empty_like, zeros, zeros_like, ones, ones_like, full, full_like, arange)
+
+from cupy_amd._manipulation import (  # noqa
+    shape, ndim, size, squeeze, swapaxes, moveaxis, rollaxis, expand_dims,
+    atleast_1d, atleast_2d, atleast_3d, broadcast_arrays, flip, fliplr, flipud,
+    astype, asanyarray, asfortranarray, isscalar, cumulative_sum, cumulative_prod,
+    isneginf, isposinf, array_equal, array_equiv, average, linspace)
 
 max = amax
 min = amin

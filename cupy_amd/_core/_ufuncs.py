@@ -608,6 +608,22 @@ _is_close = create_ufunc(
     }
     ''')
 
+# complex operands: the same test with the modulus in place of fabs
+# (reference: cupy/_logic/comparison.py:24-41)
+_is_close_complex = create_ufunc(
+    'cupy_is_close_complex',
+    (('FFff?->?', None), ('DDdd?->?', None)),
+    '''
+    bool equal_nan = in4;
+    if (isfinite(in0) && isfinite(in1)) {
+      out0 = abs(in0 - in1) <= in3 + in2 * abs(in1);
+    } else if (equal_nan) {
+      out0 = (in0 == in1) || (isnan(in0) && isnan(in1));
+    } else {
+      out0 = (in0 == in1);
+    }
+    ''')
+
 _nan_to_num = create_ufunc(
     'cupy_nan_to_num_',
     tuple(('%s%s%s%s->%s' % (c, c, c, c, c), 'out0 = in0') for c in '?' + _INTS) +
@@ -625,6 +641,10 @@ def isclose(a, b, rtol=1.e-5, atol=1.e-8, equal_nan=False):
     a = array(a, copy=False)
     b = array(b, copy=False)
     dt = numpy.result_type(a.dtype, b.dtype)
+    if dt.kind == 'c':
+        real = numpy.dtype('float32' if dt == numpy.complex64 else 'float64').type
+        return _is_close_complex(a.astype(dt, copy=False), b.astype(dt, copy=False),
+                                 real(rtol), real(atol), bool(equal_nan))
     if dt.kind != 'f':
         dt = numpy.dtype('float64')
     return _is_close(a.astype(dt, copy=False), b.astype(dt, copy=False),

@@ -7,6 +7,7 @@ consumes is here (cupy/_core/core.pyx:134-301 construction and flags,
 """
 import ctypes
 import operator
+import pickle
 
 builtins_type = type
 
@@ -587,6 +588,44 @@ class ndarray:
     def tolist(self):
         return self.get().tolist()
 
+    def tobytes(self, order='C'):
+        """The elements as a Python bytes object (reference: core.pyx:708-710)."""
+        return self.get().tobytes(order)
+
+    def tofile(self, fid, sep='', format='%s'):
+        """Writes the array to a file as numpy.ndarray.tofile does
+        (reference: core.pyx:712-718)."""
+        self.get().tofile(fid, sep, format)
+
+    def dump(self, file):
+        """Pickles the array into an open file (reference: core.pyx:720-727)."""
+        pickle.dump(self, file, -1)
+
+    def dumps(self):
+        """The array's pickle as bytes (reference: core.pyx:729-731)."""
+        return pickle.dumps(self, -1)
+
+    # a pickle holds the host copy; loading it uploads to the current device
+    # (reference: core.pyx:1796-1797)
+    def __reduce__(self):
+        return array, (self.get(order='A'),)
+
+    def __copy__(self):
+        return self.copy()
+
+    def __deepcopy__(self, memo):
+        # the copy is made on the array's own device (reference: core.pyx:1787-1794)
+        with self.device:
+            return self.copy()
+
+    def __iter__(self):
+        if not self._shape:
+            raise TypeError('iteration over a 0-d array')
+        return (self[i] for i in range(self._shape[0]))
+
+    def __complex__(self):
+        return complex(self.get().reshape(()))
+
     def __bool__(self):
         if self.size != 1:
             raise ValueError('The truth value of an array with more than one '
@@ -690,11 +729,25 @@ class ndarray:
     def __rfloordiv__(self, other):
         return self._binary('floor_divide', other, True)
 
+    def __ifloordiv__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.floor_divide(self, other, self)
+
     def __mod__(self, other):
         return self._binary('remainder', other)
 
     def __rmod__(self, other):
         return self._binary('remainder', other, True)
+
+    def __imod__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.remainder(self, other, self)
+
+    def __divmod__(self, other):
+        return self._binary('divmod', other)
+
+    def __rdivmod__(self, other):
+        return self._binary('divmod', other, True)
 
     def __pow__(self, other, modulo=None):
         if modulo is not None:
@@ -744,11 +797,19 @@ class ndarray:
     def __rand__(self, other):
         return self._binary('bitwise_and', other, True)
 
+    def __iand__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.bitwise_and(self, other, self)
+
     def __or__(self, other):
         return self._binary('bitwise_or', other)
 
     def __ror__(self, other):
         return self._binary('bitwise_or', other, True)
+
+    def __ior__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.bitwise_or(self, other, self)
 
     def __xor__(self, other):
         return self._binary('bitwise_xor', other)
@@ -756,11 +817,29 @@ class ndarray:
     def __rxor__(self, other):
         return self._binary('bitwise_xor', other, True)
 
+    def __ixor__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.bitwise_xor(self, other, self)
+
     def __lshift__(self, other):
         return self._binary('left_shift', other)
 
+    def __rlshift__(self, other):
+        return self._binary('left_shift', other, True)
+
+    def __ilshift__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.left_shift(self, other, self)
+
     def __rshift__(self, other):
         return self._binary('right_shift', other)
+
+    def __rrshift__(self, other):
+        return self._binary('right_shift', other, True)
+
+    def __irshift__(self, other):
+        from cupy_amd._core import _ufuncs
+        return _ufuncs.right_shift(self, other, self)
 
     def __lt__(self, other):
         return self._binary('less', other)
@@ -1068,10 +1147,14 @@ def array(obj, dtype=None, copy=True, order='K', subok=False, ndmin=0):
     if isinstance(obj, ndarray) or hasattr(obj, '__cuda_array_interface__') \
             or hasattr(obj, '__cupy_get_ndarray__'):
         src = _convert_from_cupy_like(obj)
-        if dtype is None or _dtype.get_dtype(dtype) == src.dtype:
-            out = src.copy() if copy else src
+        want = (order or 'K').upper()
+        if dtype is not None and _dtype.get_dtype(dtype) != src.dtype:
+            out = src.astype(dtype, order=want)
+        elif copy or (want == 'C' and not src._c_contiguous) \
+                or (want == 'F' and not src._f_contiguous):
+            out = src.copy(order=want)
         else:
-            out = src.astype(dtype)
+            out = src
     else:
         host = numpy.asarray(obj, dtype=dtype)
         _dtype.check_supported_dtype(host.dtype)
