@@ -477,6 +477,22 @@ def build_layout_cases(cp):
     dmid = cp.asarray(mid)
     add('(2^20,16,4) + (2^20,1,4) f32', 2 * r164.nbytes + mid.nbytes, run('mid', lambda: dr164 + dmid),
         lambda: r164 + mid, lambda: same(res['mid'], r164 + mid), 'cupy_add')
+    # ---- joining, tiling, rolling: copies into windows of the result ---------------------------------
+    h2, dh2 = flat.reshape(8192, 8192)[:, :4096], dsq[:, :4096]
+    g2, dg2 = flat.reshape(8192, 8192)[:, 4096:], dsq[:, 4096:]
+    add('concatenate two (8192,4096) f32 windows along axis 0', 2 * (h2.nbytes + g2.nbytes),
+        run('cat0', lambda: cp.concatenate([dh2, dg2])), lambda: np.concatenate([h2, g2]),
+        lambda: same(res['cat0'], np.concatenate([h2, g2])), 'cupy_copy')
+    t1, dt1 = flat[:1 << 25].reshape(4096, 8192), dflat[:1 << 25].reshape(4096, 8192)
+    t2, dt2 = flat[1 << 25:].reshape(4096, 8192), dflat[1 << 25:].reshape(4096, 8192)
+    add('concatenate two (4096,8192) f32 along axis 1', 2 * flat.nbytes,
+        run('cat1', lambda: cp.concatenate([dt1, dt2], axis=1)), lambda: np.concatenate([t1, t2], axis=1),
+        lambda: same(res['cat1'], np.concatenate([t1, t2], axis=1)), 'cupy_copy')
+    tl, dtl = flat[:1 << 24].reshape(4096, 4096), dflat[:1 << 24].reshape(4096, 4096)
+    add('tile (4096,4096) f32 by (2,2)', 5 * tl.nbytes, run('tile', lambda: cp.tile(dtl, (2, 2))),
+        lambda: np.tile(tl, (2, 2)), lambda: same(res['tile'], np.tile(tl, (2, 2))), 'cupy_copy')
+    add('roll f32 8192x8192 by (1,1)', 2 * sq.nbytes, run('roll', lambda: cp.roll(dsq, (1, 1), (0, 1))),
+        lambda: np.roll(sq, (1, 1), (0, 1)), lambda: same(res['roll'], np.roll(sq, (1, 1), (0, 1))), 'cupy_copy')
     return cases
 
 

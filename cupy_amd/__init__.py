@@ -108,6 +108,9 @@ from cupy_amd._manipulation import (  # noqa
     atleast_1d, atleast_2d, atleast_3d, broadcast_arrays, flip, fliplr, flipud,
     astype, asanyarray, asfortranarray, isscalar, cumulative_sum, cumulative_prod,
     isneginf, isposinf, array_equal, array_equiv, average, linspace)
+from cupy_amd._join import (  # noqa
+    concatenate, stack, hstack, vstack, row_stack, dstack, column_stack,
+    array_split, split, hsplit, vsplit, dsplit, tile, repeat, roll, rot90)
 
 max = amax
 min = amin

@@ -1,0 +1,330 @@
+"""Joining, splitting, tiling and rolling arrays.  Splits are views; the others
+allocate the result once and fill it piece by piece with the package's own
+copy kernel (each piece is a strided window of the result, which the
+elementwise planner turns into rows or tiles), so every element is read once
+and written once.  Each function cites the reference function whose
+arguments and errors it keeps."""
+import functools
+import itertools
+import operator
+
+import numpy
+
+from cupy_amd._core import internal
+from cupy_amd._core import _dtype
+from cupy_amd._core.core import ndarray, asarray
+from cupy_amd._core._ufuncs import elementwise_copy
+
+
+def _window(arr, axis, start, stop):
+    return arr[tuple(slice(start, stop) if ax == axis else slice(None) for ax in range(arr.ndim))]
+
+
+def _concatenate(arrays, axis, out, dtype, casting):
+    """reference: cupy/_core/_routines_manipulation.pyx:652-760 (concatenate_method)"""
+    arrays = list(arrays)
+    if not arrays:
+        raise ValueError('Cannot concatenate from empty tuple')
+    for a in arrays:
+        if not isinstance(a, ndarray):
+            raise TypeError('Only cupy arrays can be concatenated')
+    for a in arrays:
+        if a.ndim == 0:
+            raise TypeError('zero-dimensional arrays cannot be concatenated')
+    first = arrays[0]
+    nd = first.ndim
+    if any(a.ndim != nd for a in arrays):
+        raise ValueError('All arrays to concatenate must have the same ndim')
+    axis = internal._normalize_axis_index(axis, nd)
+    shape = list(first.shape)
+    for a in arrays[1:]:
+        if any(ax != axis and shape[ax] != a.shape[ax] for ax in range(nd)):
+            raise ValueError('All arrays must have same shape except the axis to concatenate')
+        shape[axis] += a.shape[axis]
+    shape = tuple(shape)
+    if out is None:
+        if dtype is None:
+            kinds = {a.dtype for a in arrays}
+            dtype = first.dtype if len(kinds) == 1 else functools.reduce(numpy.promote_types, kinds)
+        else:
+            dtype = _dtype.get_dtype(dtype)
+    else:
+        if dtype is not None:
+            raise TypeError('concatenate() only takes `out` or `dtype` as an '
+                            'argument, but both were provided.')
+        dtype = out.dtype
+    for a in arrays:
+        _dtype._raise_if_invalid_cast(a.dtype, dtype, casting)
+    if out is None:
+        out = ndarray(shape, dtype)
+    else:
+        if out.ndim != nd:
+            raise ValueError('Output array has wrong dimensionality')
+        if out.shape != shape:
+            raise ValueError('Output array is the wrong shape')
+    at = 0
+    for a in arrays:
+        ext = a.shape[axis]
+        if a.size:
+            elementwise_copy(a, _window(out, axis, at, at + ext), casting=casting)
+        at += ext
+    return out
+
+
+def concatenate(tup, axis=0, out=None, *, dtype=None, casting='same_kind'):
+    """Joins arrays along an existing axis (``axis=None``: their flattened forms)
+    (reference: cupy/_manipulation/join.py:39-64)."""
+    if axis is None:
+        tup = [a.ravel() if isinstance(a, ndarray) else a for a in tup]
+        axis = 0
+    return _concatenate(tup, axis, out, dtype, casting)
+
+
+def stack(tup, axis=0, out=None, *, dtype=None, casting='same_kind'):
+    """Joins arrays along a new axis (reference: cupy/_manipulation/join.py:147-170)."""
+    tup = list(tup)
+    for a in tup:
+        if not isinstance(a, ndarray):
+            raise TypeError('Only cupy arrays can be stacked')
+    if tup and any(a.shape != tup[0].shape for a in tup):
+        raise ValueError('all input arrays must have the same shape')
+    if tup:
+        axis = internal._normalize_axis_index(axis, tup[0].ndim + 1)
+    from cupy_amd._manipulation import expand_dims
+    return _concatenate([expand_dims(a, axis) for a in tup], axis, out, dtype, casting)
+
+
+def hstack(tup, *, dtype=None, casting='same_kind'):
+    """reference: cupy/_manipulation/join.py:83-108"""
+    from cupy_amd._manipulation import atleast_1d
+    arrs = [atleast_1d(a) for a in tup]
+    axis = 0 if arrs and arrs[0].ndim == 1 else 1
+    return _concatenate(arrs, axis, None, dtype, casting)
+
+
+def vstack(tup, *, dtype=None, casting='same_kind'):
+    """reference: cupy/_manipulation/join.py:111-134"""
+    from cupy_amd._manipulation import atleast_2d
+    return _concatenate([atleast_2d(a) for a in tup], 0, None, dtype, casting)
+
+
+row_stack = vstack
+
+
+def dstack(tup):
+    """reference: cupy/_manipulation/join.py:67-80"""
+    from cupy_amd._manipulation import atleast_3d
+    return _concatenate([atleast_3d(a) for a in tup], 2, None, None, 'same_kind')
+
+
+def column_stack(tup):
+    """1-d arrays become the columns of a matrix, 2-d arrays are joined as
+    they are (reference: cupy/_manipulation/join.py:9-36)."""
+    if any(not isinstance(a, ndarray) for a in tup):
+        raise TypeError('Only cupy arrays can be column stacked')
+    cols = []
+    for a in tup:
+        if a.ndim == 1:
+            a = a[:, None]
+        elif a.ndim != 2:
+            raise ValueError('Only 1 or 2 dimensional arrays can be column stacked')
+        cols.append(a)
+    return _concatenate(cols, 1, None, None, 'same_kind')
+
+
+# ---------------------------------------------------------------------------------
+# splitting: views
+# ---------------------------------------------------------------------------------
+
+def array_split(ary, indices_or_sections, axis=0):
+    """Views of consecutive pieces of one axis; a count that does not divide
+    the axis gives the first pieces one element more
+    (reference: cupy/_core/_routines_manipulation.pyx `array_split`)."""
+    nd = ary.ndim
+    if not -nd <= axis < nd:
+        raise IndexError('Axis exceeds ndim')
+    axis %= nd
+    size = ary.shape[axis]
+    if numpy.isscalar(indices_or_sections):
+        sections = operator.index(indices_or_sections)
+        if sections <= 0:
+            raise ValueError('number sections must be larger than 0.')
+        each, extra = divmod(size, sections)
+        cuts = list(itertools.accumulate([each + 1] * extra + [each] * (sections - extra)))[:-1]
+    else:
+        cuts = [operator.index(i) for i in indices_or_sections]
+    pieces, prev = [], 0
+    for cut in cuts + [size]:
+        # NumPy's slicing rules: negative cuts count from the end, cuts out of
+        # range or out of order give empty pieces
+        piece = _window(ary, axis, prev, cut)
+        pieces.append(piece)
+        prev = cut
+    return pieces
+
+
+def split(ary, indices_or_sections, axis=0):
+    """reference: cupy/_manipulation/split.py:51-80"""
+    if ary.ndim <= axis:
+        raise IndexError('Axis exceeds ndim')
+    if numpy.isscalar(indices_or_sections):
+        if ary.shape[axis] % indices_or_sections != 0:
+            raise ValueError(
+                'indices_or_sections must divide the size along the axes.\n'
+                'If you want to split the array into non-equally-sized '
+                'arrays, use array_split instead.')
+    return array_split(ary, indices_or_sections, axis)
+
+
+def hsplit(ary, indices_or_sections):
+    """reference: cupy/_manipulation/split.py:34-48"""
+    if ary.ndim == 0:
+        raise ValueError('Cannot hsplit a zero-dimensional array')
+    return split(ary, indices_or_sections, 0 if ary.ndim == 1 else 1)
+
+
+def vsplit(ary, indices_or_sections):
+    """reference: cupy/_manipulation/split.py:83-94"""
+    if ary.ndim <= 1:
+        raise ValueError('Cannot vsplit an array with less than 2 dimensions')
+    return split(ary, indices_or_sections, 0)
+
+
+def dsplit(ary, indices_or_sections):
+    """reference: cupy/_manipulation/split.py:21-31"""
+    if ary.ndim <= 2:
+        raise ValueError('Cannot dsplit an array with less than 3 dimensions')
+    return split(ary, indices_or_sections, 2)
+
+
+# ---------------------------------------------------------------------------------
+# tiling
+# ---------------------------------------------------------------------------------
+
+def tile(A, reps):
+    """The array repeated ``reps`` times along each axis: ONE broadcast copy
+    into a result seen as (rep, extent) pairs of axes
+    (reference: cupy/_manipulation/tiling.py:7-55)."""
+    reps = tuple(reps) if isinstance(reps, (tuple, list)) else (reps,)
+    reps = tuple(operator.index(r) for r in reps)
+    a = asarray(A)
+    nd = max(a.ndim, len(reps))
+    if all(r == 1 for r in reps):
+        return a.reshape((1,) * (nd - a.ndim) + a.shape).copy()
+    shape = (1,) * (nd - a.ndim) + a.shape
+    reps = (1,) * (nd - len(reps)) + reps
+    out = ndarray(tuple(s * r for s, r in zip(shape, reps)), a.dtype)
+    if out.size == 0:
+        return out
+    a = a.reshape(shape)
+    # result axis k of extent r*s is the pair (r, s); the source has a step of 0 over r
+    paired = out.reshape(tuple(itertools.chain.from_iterable(zip(reps, shape))))
+    src = a._view(tuple(itertools.chain.from_iterable(zip(reps, shape))),
+                  tuple(itertools.chain.from_iterable((0, st) for st in a.strides)))
+    elementwise_copy(src, paired)
+    return out
+
+
+def repeat(a, repeats, axis=None):
+    """Every element repeated: one count for all (a broadcast copy) or a count
+    per element given on the host (a copy per run)
+    (reference: cupy/_manipulation/tiling.py:58-75,
+    cupy/_core/_routines_manipulation.pyx `_repeat`)."""
+    if isinstance(repeats, ndarray):
+        raise ValueError('cupy.ndaray cannot be specified as `repeats` argument.')
+    if axis is None:
+        a = a.ravel()
+        axis = 0
+    else:
+        axis = internal._normalize_axis_index(axis, a.ndim)
+    if isinstance(repeats, (int, numpy.integer)):
+        counts = [operator.index(repeats)]
+    else:
+        counts = [operator.index(r) for r in repeats]
+    if any(c < 0 for c in counts):
+        raise ValueError("'repeats' should not be negative: {}".format(repeats))
+    n = a.shape[axis]
+    if len(counts) == 1:
+        r = counts[0]
+        shape = a.shape[:axis] + (n * r,) + a.shape[axis + 1:]
+        out = ndarray(shape, a.dtype)
+        if out.size:
+            paired = out.reshape(a.shape[:axis] + (n, r) + a.shape[axis + 1:])
+            src = a._view(paired.shape, a.strides[:axis] + (a.strides[axis], 0) + a.strides[axis + 1:])
+            elementwise_copy(src, paired)
+        return out
+    if len(counts) != n:
+        raise ValueError("'repeats' and 'axis' of 'a' should be same length: {} != {}".format(
+            n, len(counts)))
+    shape = a.shape[:axis] + (sum(counts),) + a.shape[axis + 1:]
+    out = ndarray(shape, a.dtype)
+    at = 0
+    for i, c in enumerate(counts):
+        if c and out.size:
+            dst = _window(out, axis, at, at + c)
+            src = _window(a, axis, i, i + 1)
+            elementwise_copy(src._view(dst.shape, src.strides[:axis] + (0,) + src.strides[axis + 1:]), dst)
+        at += c
+    return out
+
+
+# ---------------------------------------------------------------------------------
+# rolling and quarter turns
+# ---------------------------------------------------------------------------------
+
+def roll(a, shift, axis=None):
+    """Elements shifted along the axes, those pushed out re-enter at the other
+    end; shifts are host integers (reference: cupy/_manipulation/rearrange.py:75-147)."""
+    if isinstance(shift, ndarray):
+        raise NotImplementedError('roll with a device array of shifts is not part of this build')
+    if axis is None:
+        return roll(a.ravel(), shift, 0).reshape(a.shape)
+    axes = (axis,) if numpy.isscalar(axis) else tuple(axis)
+    axes = tuple(internal._normalize_axis_index(ax, a.ndim) for ax in axes)
+    pairs = numpy.broadcast(shift, axes)
+    if pairs.nd > 1:
+        raise ValueError("'shift' and 'axis' should be scalars or 1D sequences")
+    total = dict.fromkeys(range(a.ndim), 0)
+    for sh, ax in pairs:
+        total[ax] += int(sh)
+    # per axis: the (source, destination) windows the shift cuts it into
+    cuts = []
+    for ax in range(a.ndim):
+        off = total[ax] % (a.shape[ax] or 1)
+        if off:
+            cuts.append(((slice(None, -off), slice(off, None)), (slice(-off, None), slice(None, off))))
+        else:
+            cuts.append(((slice(None), slice(None)),))
+    out = ndarray(a.shape, a.dtype)
+    if out.size == 0:
+        return out
+    for combo in itertools.product(*cuts):
+        src, dst = zip(*combo)
+        elementwise_copy(a[src], out[dst])
+    return out
+
+
+def rot90(a, k=1, axes=(0, 1)):
+    """View turned by quarter turns in the plane of two axes
+    (reference: cupy/_manipulation/rearrange.py:150-193)."""
+    nd = a.ndim
+    if nd < 2:
+        raise ValueError('Input must be >= 2-d')
+    axes = tuple(axes)
+    if len(axes) != 2:
+        raise ValueError('len(axes) must be 2')
+    if axes[0] == axes[1] or abs(axes[0] - axes[1]) == nd:
+        raise ValueError('axes must be different')
+    if not (-nd <= axes[0] < nd and -nd <= axes[1] < nd):
+        raise ValueError('axes must be >= %d and < %d' % (-nd, nd))
+    from cupy_amd._manipulation import flip
+    k %= 4
+    if k == 0:
+        return a[:]
+    if k == 2:
+        return flip(a, axes)
+    order = list(range(nd))
+    order[axes[0]], order[axes[1]] = order[axes[1]], order[axes[0]]
+    if k == 1:
+        return flip(a, axes[1]).transpose(order)
+    return flip(a.transpose(order), axes[1])
