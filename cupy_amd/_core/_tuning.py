@@ -28,6 +28,17 @@ _params = {
     # matrices whose rows are spaced apart (windows, every second row or
     # column) are walked row by row in vectors instead of in square tiles
     'rows2d': True,
+    # ndarray.copy() of an array stored in one piece: the driver's device-to-device
+    # copy below this many bytes, the flat elementwise kernel from there on
+    # (64 MiB: 23.8 -> 19.8 us, 256 MiB: 98.4 -> 85.5 us; under 32 MiB the call is
+    # bound by the host either way and the driver's copy costs it 1.5 us less)
+    'copy_kernel_min_bytes': 1 << 25,
+    # the pieces of a concatenation whose layouts allow it are copied by one
+    # launch (up to eight per launch) instead of a launch each
+    'concatenate_one_launch': True,
+    # ... by workgroups of this many threads, each moving this many vectors
+    'concatenate_block': 256,
+    'concatenate_unroll': 1,
     # ... with shorter vectors for rows of fewer than 12 vectors, so that no row
     # ends in a partial one (window of 7 columns: 235 -> 142 us; from 12
     # vectors per row on, the partial vector costs less than shorter accesses)

@@ -16,6 +16,7 @@ import numpy
 from cupy_amd import _dryrun
 from cupy_amd import _rt
 from cupy_amd._core import _dtype
+from cupy_amd._core import _tuning
 from cupy_amd._core import internal
 from cupy_amd.cuda import device as _device
 from cupy_amd.cuda import memory as _memory
@@ -532,7 +533,8 @@ class ndarray:
                 out = out._retype(type(self), self)
             if self.size == 0:
                 return out
-            if self._c_contiguous:
+            if self._c_contiguous and (self.nbytes < _tuning.get('copy_kernel_min_bytes')
+                                       or self.dtype.fields is not None):
                 out.data.copy_from_device_async(self.data, self.nbytes)
             else:
                 from cupy_amd._core._ufuncs import elementwise_copy

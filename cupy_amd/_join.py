@@ -7,17 +7,219 @@ arguments and errors it keeps."""
 import functools
 import itertools
 import operator
+import struct
 
 import numpy
 
 from cupy_amd._core import internal
 from cupy_amd._core import _dtype
+from cupy_amd._core import _tuning
 from cupy_amd._core.core import ndarray, asarray
 from cupy_amd._core._ufuncs import elementwise_copy
 
 
 def _window(arr, axis, start, stop):
     return arr[tuple(slice(start, stop) if ax == axis else slice(None) for ax in range(arr.ndim))]
+
+
+# ---------------------------------------------------------------------------------
+# the pieces of a concatenation in one launch
+# ---------------------------------------------------------------------------------
+# Seen from the joined axis, a piece whose trailing axes are stored one after
+# the other is a matrix: rows = the axes before the joined one, a row = one
+# contiguous run of (extent along the axis) x (elements behind it), and its
+# place in the result is the same matrix with the result's row pitch.  One
+# kernel copies up to _MAX_PIECES such matrices: workgroups are dealt out to
+# the pieces in proportion to their sizes (a table of first workgroups in the
+# argument block), a thread moves a vector or a few, all requested before the
+# first is stored.  A launch per piece costs a ramp and a tail each: two
+# windows of 128 MiB took 95.7 us in two launches.
+
+_MAX_PIECES = 8
+
+_PIECES_SOURCE = r"""
+#include <cupy/carray.cuh>
+struct Piece {
+  const ITEM_T* src;
+  ITEM_T* dst;
+  long long src_pitch;      // elements between rows
+  long long dst_pitch;
+  unsigned int vecs_per_row;
+  unsigned int n_vecs;      // rows * vecs_per_row
+  unsigned int first_block;
+  unsigned int pad;
+};
+struct Pieces { Piece p[MAX_PIECES]; };
+
+extern "C" __global__ void __launch_bounds__(BLOCK)
+cupy_concatenate_pieces(const Pieces ps, const int n_pieces) {
+  int k = 0;
+#pragma unroll
+  for (int j = 1; j < MAX_PIECES; ++j)
+    if (j < n_pieces && blockIdx.x >= ps.p[j].first_block) k = j;
+  const Piece pc = ps.p[k];
+  const unsigned int base = (blockIdx.x - pc.first_block) * (BLOCK * UNROLL) + threadIdx.x;
+  cupy::Vec<ITEM_T, NV> v[UNROLL];
+  long long to[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const unsigned int i = base + u * BLOCK;
+    if (i < pc.n_vecs) {
+      const unsigned int r = i / pc.vecs_per_row;
+      const unsigned int c = (i - r * pc.vecs_per_row) * NV;
+      v[u] = cupy::load_vec<ITEM_T, NV, STREAM_IN>(pc.src + r * pc.src_pitch + c);
+      to[u] = r * pc.dst_pitch + c;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u)
+    if (base + u * BLOCK < pc.n_vecs)
+      cupy::store_vec<ITEM_T, NV, STREAM_OUT>(pc.dst + to[u], v[u]);
+}
+"""
+
+_PIECE_STRUCT = struct.Struct('<QQqqIIII')     # struct Piece of the kernel source
+
+
+class _ArgBytes:
+    """Bytes passed by value as one kernel argument."""
+
+    def __init__(self, data):
+        self._data = data
+
+    def _kernel_arg_bytes(self):
+        return self._data
+
+
+_ITEM_TYPES = {1: 'unsigned char', 2: 'unsigned short', 4: 'unsigned int',
+               8: 'unsigned long long'}
+
+_pieces_kernels = {}
+
+
+def _geometry():
+    """(threads per workgroup, vectors per thread) of the kernel."""
+    return _tuning.get('concatenate_block'), _tuning.get('concatenate_unroll')
+
+
+def _pieces_kernel(itemsize, nv, stream_in, stream_out):
+    _BLOCK, _UNROLL = _geometry()
+    key = (itemsize, nv, stream_in, stream_out, _BLOCK, _UNROLL)
+    ker = _pieces_kernels.get(key)
+    if ker is None:
+        from cupy_amd._core.raw import RawKernel
+        defines = (('ITEM_T', 'item_t'), ('NV', nv), ('MAX_PIECES', _MAX_PIECES),
+                   ('BLOCK', _BLOCK), ('UNROLL', _UNROLL),
+                   ('STREAM_IN', 'true' if stream_in else 'false'),
+                   ('STREAM_OUT', 'true' if stream_out else 'false'))
+        source = 'typedef %s item_t;\n' % _ITEM_TYPES[itemsize] + _PIECES_SOURCE
+        ker = _pieces_kernels[key] = RawKernel(
+            source, 'cupy_concatenate_pieces', tuple('-D%s=%s' % d for d in defines))
+    return ker
+
+
+def _as_rows(shape, strides, item, lead):
+    """(rows, elements per row, elements between rows) of a layout whose axes
+    from ``lead`` on are stored one after the other and whose axes before it
+    step evenly and forwards; None for any other layout."""
+    run = item
+    for k in range(len(shape) - 1, lead - 1, -1):
+        if shape[k] != 1 and strides[k] != run:
+            return None
+        run *= shape[k]
+    rows, pitch = 1, run
+    for k in range(lead - 1, -1, -1):
+        ext = shape[k]
+        if ext == 1:
+            continue
+        st = strides[k]
+        if rows == 1:
+            if st < run or st % item:
+                return None
+            pitch = st
+        elif st != pitch * rows:
+            return None
+        rows *= ext
+    return rows, run // item, pitch // item
+
+
+def _plan_pieces(pieces, dtype):
+    """What the one-launch kernel needs to copy ``pieces``, a list of (shape,
+    strides and address of the source, strides and address of its place in
+    the result), all of element type ``dtype``: (bytes per word, words per
+    vector, [(source address, destination address, rows, words per row, words
+    between the rows of the source, of the destination)]), or None if a
+    piece does not fit the kernel (a layout that is no matrix of contiguous
+    rows, rows of a few elements, 2**31 words or more)."""
+    if len(pieces) < 2 or dtype.fields is not None:
+        return None
+    item = dtype.itemsize
+    # 16-byte elements travel as pairs of 8-byte words
+    word, words = (8, 2) if item == 16 else (item, 1)
+    if word not in _ITEM_TYPES:
+        return None
+    nv = 16 // word
+    forms = []
+    for shape, sstrides, sptr, dstrides, dptr in pieces:
+        # the longest rows both sides have
+        for lead in range(len(shape) + 1):
+            fs = _as_rows(shape, sstrides, item, lead)
+            if fs is None:
+                continue
+            fd = _as_rows(shape, dstrides, item, lead)
+            if fd is not None:
+                break
+        else:
+            return None
+        rows, row = fs[0], fs[1] * words
+        if rows > 1 and row * word < 64:
+            # a few elements per row: the tiled kernels do these better
+            return None
+        sp, dp = fs[2] * words, fd[2] * words
+        if sp == row and dp == row:
+            # rows follow each other on both sides: one long row
+            rows, row = 1, rows * row
+            sp = dp = row
+        while row % nv:
+            nv //= 2
+        if rows * row >= 1 << 31:
+            return None
+        forms.append((sptr, dptr, rows, row, sp, dp))
+    return word, nv, forms
+
+
+def _piece_tables(nv, forms):
+    """The argument tables of the launches that copy ``forms``, eight pieces a
+    launch: [(table bytes, pieces in it, workgroups)]."""
+    block, unroll = _geometry()
+    per_block = block * unroll
+    launches = []
+    for lo in range(0, len(forms), _MAX_PIECES):
+        batch = forms[lo:lo + _MAX_PIECES]
+        table = bytearray(_MAX_PIECES * _PIECE_STRUCT.size)
+        blocks = 0
+        for k, (sptr, dptr, rows, row, sp, dp) in enumerate(batch):
+            n_vecs = rows * (row // nv)
+            _PIECE_STRUCT.pack_into(table, k * _PIECE_STRUCT.size,
+                                    sptr, dptr, sp, dp, row // nv, n_vecs, blocks, 0)
+            blocks += (n_vecs + per_block - 1) // per_block
+        launches.append((bytes(table), len(batch), blocks))
+    return launches
+
+
+def _copy_pieces(pieces, dtype, nbytes):
+    """Copies the pieces with the one-launch kernel; False, with nothing
+    done, if they do not fit it."""
+    plan = _plan_pieces(pieces, dtype)
+    if plan is None:
+        return False
+    word, nv, forms = plan
+    stream_in, stream_out = _tuning.stream_policy(_tuning.get('flat_stream'), nbytes, nbytes)
+    ker = _pieces_kernel(word, nv, stream_in, stream_out)
+    block = _geometry()[0]
+    for table, n_pieces, blocks in _piece_tables(nv, forms):
+        ker((blocks,), (block,), (_ArgBytes(table), numpy.int32(n_pieces)))
+    return True
 
 
 def _concatenate(arrays, axis, out, dtype, casting):
@@ -62,12 +264,22 @@ def _concatenate(arrays, axis, out, dtype, casting):
             raise ValueError('Output array has wrong dimensionality')
         if out.shape != shape:
             raise ValueError('Output array is the wrong shape')
-    at = 0
+    # (source, first index along the axis) of the pieces that hold anything
+    placed, at = [], 0
     for a in arrays:
-        ext = a.shape[axis]
         if a.size:
-            elementwise_copy(a, _window(out, axis, at, at + ext), casting=casting)
-        at += ext
+            placed.append((a, at))
+        at += a.shape[axis]
+    if not placed:
+        return out
+    step = out.strides[axis]
+    same_type = all(a.dtype == dtype for a, _ in placed)
+    if same_type and _tuning.get('concatenate_one_launch') and _copy_pieces(
+            [(a.shape, a.strides, a.data.ptr, out.strides, out.data.ptr + at * step)
+             for a, at in placed], dtype, sum(a.nbytes for a, _ in placed)):
+        return out
+    for a, at in placed:
+        elementwise_copy(a, _window(out, axis, at, at + a.shape[axis]), casting=casting)
     return out
 
 

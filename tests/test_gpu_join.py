@@ -172,3 +172,36 @@ def test_roll_and_quarter_turns():
         cp.rot90(d, 1, (0, 0))
     with pytest.raises(ValueError):
         cp.rot90(d[0, 0])
+
+
+@pytest.mark.parametrize('dtype', ['int8', 'float16', 'float32', 'float64', 'complex128'])
+def test_one_launch_and_piecewise_concatenation_agree(dtype):
+    """Layouts the one-launch kernel takes (windows with contiguous rows, whole
+    arrays, many ragged pieces), with the kernel on and off."""
+    from cupy_amd._core import _tuning
+    rng = np.random.default_rng(11)
+    hbase = rng.integers(-9, 10, size=(37, 21, 130)).astype(dtype)
+    dbase = cp.asarray(hbase)
+    cases = [
+        ([np.s_[:], np.s_[3:9], np.s_[30:]], 0),
+        ([np.s_[:, 1:], np.s_[:, :3], np.s_[:, 5:6]], 1),
+        ([np.s_[:, :, :64], np.s_[:, :, 65:], np.s_[:, :, 1:128]], 2),
+        ([np.s_[::2, :, 2:], np.s_[1:19, :, :128]], 0),
+        ([np.s_[i:i + 1 + i % 3] for i in range(0, 36, 2)], 0),
+        ([np.s_[:, :, 3:]] * 9, -1),
+    ]
+    try:
+        for slices, axis in cases:
+            want = np.concatenate([hbase[s] for s in slices], axis=axis)
+            for on in (True, False):
+                _tuning.set(concatenate_one_launch=on)
+                same(cp.concatenate([dbase[s] for s in slices], axis=axis), want)
+            big = cp.zeros(tuple(e + 2 for e in want.shape), dtype)
+            inner = tuple(slice(1, -1) for _ in want.shape)
+            _tuning.set(concatenate_one_launch=True)
+            cp.concatenate([dbase[s] for s in slices], axis=axis, out=big[inner])
+            hbig = np.zeros(big.shape, dtype)
+            hbig[inner] = want
+            same(big, hbig)
+    finally:
+        _tuning.set(concatenate_one_launch=True)
