@@ -47,7 +47,8 @@ struct Piece {
   unsigned int vecs_per_row;
   unsigned int n_vecs;      // rows * vecs_per_row
   unsigned int first_block;
-  unsigned int pad;
+  unsigned int n_rep;       // copies of the piece in the result ...
+  long long rep_step;       // ... this many elements apart
 };
 struct Pieces { Piece p[MAX_PIECES]; };
 
@@ -74,11 +75,12 @@ cupy_concatenate_pieces(const Pieces ps, const int n_pieces) {
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u)
     if (base + u * BLOCK < pc.n_vecs)
-      cupy::store_vec<ITEM_T, NV, STREAM_OUT>(pc.dst + to[u], v[u]);
+      for (unsigned int j = 0; j < pc.n_rep; ++j)
+        cupy::store_vec<ITEM_T, NV, STREAM_OUT>(pc.dst + to[u] + j * pc.rep_step, v[u]);
 }
 """
 
-_PIECE_STRUCT = struct.Struct('<QQqqIIII')     # struct Piece of the kernel source
+_PIECE_STRUCT = struct.Struct('<QQqqIIIIq')    # struct Piece of the kernel source
 
 
 class _ArgBytes:
@@ -143,15 +145,16 @@ def _as_rows(shape, strides, item, lead):
     return rows, run // item, pitch // item
 
 
-def _plan_pieces(pieces, dtype):
+def _plan_pieces(pieces, dtype, copies=1, copy_step=0):
     """What the one-launch kernel needs to copy ``pieces``, a list of (shape,
     strides and address of the source, strides and address of its place in
-    the result), all of element type ``dtype``: (bytes per word, words per
-    vector, [(source address, destination address, rows, words per row, words
-    between the rows of the source, of the destination)]), or None if a
-    piece does not fit the kernel (a layout that is no matrix of contiguous
-    rows, rows of a few elements, 2**31 words or more)."""
-    if len(pieces) < 2 or dtype.fields is not None:
+    the result), all of element type ``dtype``, each to ``copies`` places
+    ``copy_step`` bytes apart: (bytes per word, words per vector, [(source
+    address, destination address, rows, words per row, words between the rows
+    of the source, of the destination, copies, words between them)]), or None
+    if a piece does not fit the kernel (a layout that is no matrix of
+    contiguous rows, rows of a few elements, 2**31 words or more)."""
+    if len(pieces) * copies < 2 or dtype.fields is not None:
         return None
     item = dtype.itemsize
     # 16-byte elements travel as pairs of 8-byte words
@@ -159,6 +162,8 @@ def _plan_pieces(pieces, dtype):
     if word not in _ITEM_TYPES:
         return None
     nv = 16 // word
+    if copy_step % word:
+        return None
     forms = []
     for shape, sstrides, sptr, dstrides, dptr in pieces:
         # the longest rows both sides have
@@ -184,7 +189,7 @@ def _plan_pieces(pieces, dtype):
             nv //= 2
         if rows * row >= 1 << 31:
             return None
-        forms.append((sptr, dptr, rows, row, sp, dp))
+        forms.append((sptr, dptr, rows, row, sp, dp, copies, copy_step // word))
     return word, nv, forms
 
 
@@ -198,23 +203,24 @@ def _piece_tables(nv, forms):
         batch = forms[lo:lo + _MAX_PIECES]
         table = bytearray(_MAX_PIECES * _PIECE_STRUCT.size)
         blocks = 0
-        for k, (sptr, dptr, rows, row, sp, dp) in enumerate(batch):
+        for k, (sptr, dptr, rows, row, sp, dp, copies, step) in enumerate(batch):
             n_vecs = rows * (row // nv)
             _PIECE_STRUCT.pack_into(table, k * _PIECE_STRUCT.size,
-                                    sptr, dptr, sp, dp, row // nv, n_vecs, blocks, 0)
+                                    sptr, dptr, sp, dp, row // nv, n_vecs, blocks, copies, step)
             blocks += (n_vecs + per_block - 1) // per_block
         launches.append((bytes(table), len(batch), blocks))
     return launches
 
 
-def _copy_pieces(pieces, dtype, nbytes):
-    """Copies the pieces with the one-launch kernel; False, with nothing
-    done, if they do not fit it."""
-    plan = _plan_pieces(pieces, dtype)
+def _copy_pieces(pieces, dtype, nbytes, copies=1, copy_step=0):
+    """Copies the pieces (``nbytes`` in all), each to ``copies`` places, with
+    the one-launch kernel; False, with nothing done, if they do not fit it."""
+    plan = _plan_pieces(pieces, dtype, copies, copy_step)
     if plan is None:
         return False
     word, nv, forms = plan
-    stream_in, stream_out = _tuning.stream_policy(_tuning.get('flat_stream'), nbytes, nbytes)
+    stream_in, stream_out = _tuning.stream_policy(
+        _tuning.get('flat_stream'), nbytes, nbytes * copies)
     ker = _pieces_kernel(word, nv, stream_in, stream_out)
     block = _geometry()[0]
     for table, n_pieces, blocks in _piece_tables(nv, forms):
@@ -430,11 +436,28 @@ def tile(A, reps):
         return out
     a = a.reshape(shape)
     # result axis k of extent r*s is the pair (r, s); the source has a step of 0 over r
-    paired = out.reshape(tuple(itertools.chain.from_iterable(zip(reps, shape))))
-    src = a._view(tuple(itertools.chain.from_iterable(zip(reps, shape))),
-                  tuple(itertools.chain.from_iterable((0, st) for st in a.strides)))
+    pair_shape = tuple(itertools.chain.from_iterable(zip(reps, shape)))
+    paired = out.reshape(pair_shape)
+    if _tuning.get('concatenate_one_launch') and _tile_pieces(a, paired, reps):
+        return out
+    src = a._view(pair_shape, tuple(itertools.chain.from_iterable((0, st) for st in a.strides)))
     elementwise_copy(src, paired)
     return out
+
+
+def _tile_pieces(a, paired, reps):
+    """The tiles written by the kernel that copies pieces: the source is read
+    once per tile along all axes but the one with most repetitions, whose
+    tiles are stored from the same registers."""
+    most = max(range(len(reps)), key=lambda k: reps[k])
+    others = [range(r) if k != most else range(1) for k, r in enumerate(reps)]
+    if internal.prod([len(o) for o in others]) > 64:
+        return False
+    rep_strides, own_strides = paired.strides[0::2], paired.strides[1::2]
+    pieces = [(a.shape, a.strides, a.data.ptr, own_strides,
+               paired.data.ptr + sum(i * st for i, st in zip(combo, rep_strides)))
+              for combo in itertools.product(*others)]
+    return _copy_pieces(pieces, a.dtype, a.nbytes * len(pieces), reps[most], rep_strides[most])
 
 
 def repeat(a, repeats, axis=None):
@@ -462,8 +485,13 @@ def repeat(a, repeats, axis=None):
         out = ndarray(shape, a.dtype)
         if out.size:
             paired = out.reshape(a.shape[:axis] + (n, r) + a.shape[axis + 1:])
-            src = a._view(paired.shape, a.strides[:axis] + (a.strides[axis], 0) + a.strides[axis + 1:])
-            elementwise_copy(src, paired)
+            own = paired.strides[:axis + 1] + paired.strides[axis + 2:]
+            if not (_tuning.get('concatenate_one_launch') and _copy_pieces(
+                    [(a.shape, a.strides, a.data.ptr, own, paired.data.ptr)], a.dtype, a.nbytes,
+                    r, paired.strides[axis + 1])):
+                src = a._view(paired.shape,
+                              a.strides[:axis] + (a.strides[axis], 0) + a.strides[axis + 1:])
+                elementwise_copy(src, paired)
         return out
     if len(counts) != n:
         raise ValueError("'repeats' and 'axis' of 'a' should be same length: {} != {}".format(

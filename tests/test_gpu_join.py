@@ -205,3 +205,27 @@ def test_one_launch_and_piecewise_concatenation_agree(dtype):
             same(big, hbig)
     finally:
         _tuning.set(concatenate_one_launch=True)
+
+
+@pytest.mark.parametrize('dtype', ['int8', 'float32', 'complex128'])
+def test_tile_and_repeat_through_the_pieces_kernel(dtype):
+    """Rows of 64 bytes and more: the tiles and the repeated rows are stored
+    from the registers that hold the source (kernel on), or by a broadcast
+    copy (kernel off); both must give NumPy's result."""
+    from cupy_amd._core import _tuning
+    rng = np.random.default_rng(4)
+    h = rng.integers(-9, 10, size=(6, 5, 64)).astype(dtype)
+    d = cp.asarray(h)
+    try:
+        for on in (True, False):
+            _tuning.set(concatenate_one_launch=on)
+            for reps in (2, (2, 3), (3, 1, 2), (1, 4, 1), (2, 2, 2), (5, 1, 1, 1), (70, 1, 1)):
+                same(cp.tile(d, reps), np.tile(h, reps))
+            same(cp.tile(d[:, 1:3, 8:], (2, 2, 2)), np.tile(h[:, 1:3, 8:], (2, 2, 2)))
+            same(cp.tile(d[0, 0], 7), np.tile(h[0, 0], 7))
+            for axis in (0, 1):
+                same(cp.repeat(d, 3, axis), np.repeat(h, 3, axis))
+                same(cp.repeat(d[1:, :, 16:], 2, axis), np.repeat(h[1:, :, 16:], 2, axis))
+            same(cp.repeat(d, 1, 0), np.repeat(h, 1, 0))
+    finally:
+        _tuning.set(concatenate_one_launch=True)

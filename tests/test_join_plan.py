@@ -11,17 +11,17 @@ from cupy_amd import _join
 # struct Piece of the kernel source
 PIECE = np.dtype([('src', np.uint64), ('dst', np.uint64), ('src_pitch', np.int64),
                   ('dst_pitch', np.int64), ('vecs_per_row', np.uint32), ('n_vecs', np.uint32),
-                  ('first_block', np.uint32), ('pad', np.uint32)])
+                  ('first_block', np.uint32), ('n_rep', np.uint32), ('rep_step', np.int64)])
 
 
 def describe(pairs):
     return [(s.shape, s.strides, s.ctypes.data, d.strides, d.ctypes.data) for s, d in pairs]
 
 
-def replay(pairs, sbase, dbase):
+def replay(pairs, sbase, dbase, copies=1, copy_step=0):
     """Runs the kernel's arithmetic over host buffers.  Returns False if the
     planner declines the pairs."""
-    plan = _join._plan_pieces(describe(pairs), pairs[0][1].dtype)
+    plan = _join._plan_pieces(describe(pairs), pairs[0][1].dtype, copies, copy_step)
     if plan is None:
         return False
     word, nv, forms = plan
@@ -30,7 +30,7 @@ def replay(pairs, sbase, dbase):
     block, unroll = _join._geometry()
     per_block = block * unroll
     for table, n_pieces, blocks in _join._piece_tables(nv, forms):
-        assert len(table) == 48 * _join._MAX_PIECES and n_pieces <= _join._MAX_PIECES
+        assert len(table) == 56 * _join._MAX_PIECES and n_pieces <= _join._MAX_PIECES
         table = np.frombuffer(table, PIECE)
         firsts = [int(table[k]['first_block']) for k in range(n_pieces)]
         assert firsts == sorted(firsts) and firsts[0] == 0
@@ -46,8 +46,11 @@ def replay(pairs, sbase, dbase):
             dst = int(pc['dst']) - d0 + (r * int(pc['dst_pitch']) + c) * word
             assert src.min() >= 0 and src.max() + nv * word <= sw.size
             assert dst.min() >= 0 and dst.max() + nv * word <= dw.size
-            for b in range(nv * word):
-                dw[dst + b] = sw[src + b]
+            for j in range(int(pc['n_rep'])):
+                at = dst + j * int(pc['rep_step']) * word
+                assert at.min() >= 0 and at.max() + nv * word <= dw.size
+                for b in range(nv * word):
+                    dw[at + b] = sw[src + b]
         # every vector of every piece has a workgroup
         assert blocks == sum(-(-int(table[k]['n_vecs']) // per_block) for k in range(n_pieces))
     return True
@@ -123,3 +126,28 @@ def test_row_decomposition():
     assert rows(a[:, :1], 1) == (6, 10, 80)
     assert rows(a.transpose(1, 0, 2), 2) is None
     assert rows(np.broadcast_to(a[:1], (3, 8, 10)), 1) is None
+
+
+@pytest.mark.parametrize('shape,reps,dtype', [
+    ((6, 32), (2, 3), 'float32'), ((6, 64), (3, 2), 'int8'), ((5, 4, 16), (2, 1, 4), 'float64'),
+    ((40,), (7,), 'complex128'), ((3, 64), (1, 5), 'int16'),
+])
+def test_tiles_as_pieces_with_copies(shape, reps, dtype):
+    rng = np.random.default_rng(1)
+    sbase = rng.integers(0, 100, size=shape).astype(dtype)
+    want = np.tile(sbase, reps)
+    dbase = np.zeros((want.shape[0] + 2,) + want.shape[1:], dtype)
+    out = dbase[1:-1]
+    pair_shape = tuple(x for rs in zip(reps, shape) for x in rs)
+    paired = out.reshape(pair_shape)
+    assert np.shares_memory(paired, out)
+    most = max(range(len(reps)), key=lambda k: reps[k])
+    rep_strides, own = paired.strides[0::2], paired.strides[1::2]
+    pairs = []
+    for combo in np.ndindex(*[r if k != most else 1 for k, r in enumerate(reps)]):
+        index = tuple(x for ci in combo for x in (ci, slice(None)))
+        pairs.append((sbase, paired[index]))
+        assert paired[index].strides == own
+    assert replay(pairs, sbase, dbase, reps[most], rep_strides[most])
+    assert np.array_equal(out, want)
+    assert not dbase[0].any() and not dbase[-1].any()
