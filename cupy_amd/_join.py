@@ -32,10 +32,12 @@ def _window(arr, axis, start, stop):
 # kernel copies up to _MAX_PIECES such matrices: workgroups are dealt out to
 # the pieces in proportion to their sizes (a table of first workgroups in the
 # argument block), a thread moves a vector or a few, all requested before the
-# first is stored.  A launch per piece costs a ramp and a tail each: two
+# first is stored; a row's last vector may be a partial one, done element by
+# element.  A launch per piece costs a ramp and a tail each: two
 # windows of 128 MiB took 95.7 us in two launches.
 
 _MAX_PIECES = 8
+_NARROW_PIECE_BYTES = 1 << 20
 
 _PIECES_SOURCE = r"""
 #include <cupy/carray.cuh>
@@ -44,11 +46,13 @@ struct Piece {
   ITEM_T* dst;
   long long src_pitch;      // elements between rows
   long long dst_pitch;
-  unsigned int vecs_per_row;
+  unsigned int vecs_per_row;  // the last vector of a row may be a partial one
   unsigned int n_vecs;      // rows * vecs_per_row
   unsigned int first_block;
   unsigned int n_rep;       // copies of the piece in the result ...
   long long rep_step;       // ... this many elements apart
+  unsigned int row_len;     // elements per row
+  unsigned int pad;
 };
 struct Pieces { Piece p[MAX_PIECES]; };
 
@@ -62,25 +66,42 @@ cupy_concatenate_pieces(const Pieces ps, const int n_pieces) {
   const unsigned int base = (blockIdx.x - pc.first_block) * (BLOCK * UNROLL) + threadIdx.x;
   cupy::Vec<ITEM_T, NV> v[UNROLL];
   long long to[UNROLL];
+  unsigned int have[UNROLL];    // elements of the vector inside the row
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const unsigned int i = base + u * BLOCK;
+    have[u] = 0;
     if (i < pc.n_vecs) {
       const unsigned int r = i / pc.vecs_per_row;
       const unsigned int c = (i - r * pc.vecs_per_row) * NV;
-      v[u] = cupy::load_vec<ITEM_T, NV, STREAM_IN>(pc.src + r * pc.src_pitch + c);
+      const ITEM_T* from = pc.src + r * pc.src_pitch + c;
       to[u] = r * pc.dst_pitch + c;
+      have[u] = pc.row_len - c < NV ? pc.row_len - c : NV;
+      if (have[u] == NV) {
+        v[u] = cupy::load_vec<ITEM_T, NV, STREAM_IN>(from);
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; ++e) if (e < have[u]) v[u].v[e] = from[e];
+      }
     }
   }
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u)
-    if (base + u * BLOCK < pc.n_vecs)
-      for (unsigned int j = 0; j < pc.n_rep; ++j)
-        cupy::store_vec<ITEM_T, NV, STREAM_OUT>(pc.dst + to[u] + j * pc.rep_step, v[u]);
+  for (int u = 0; u < UNROLL; ++u) {
+    if (have[u] == 0) continue;
+    for (unsigned int j = 0; j < pc.n_rep; ++j) {
+      ITEM_T* at = pc.dst + to[u] + j * pc.rep_step;
+      if (have[u] == NV) {
+        cupy::store_vec<ITEM_T, NV, STREAM_OUT>(at, v[u]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; ++e) if (e < have[u]) at[e] = v[u].v[e];
+      }
+    }
+  }
 }
 """
 
-_PIECE_STRUCT = struct.Struct('<QQqqIIIIq')    # struct Piece of the kernel source
+_PIECE_STRUCT = struct.Struct('<QQqqIIIIqII')  # struct Piece of the kernel source
 
 
 class _ArgBytes:
@@ -153,7 +174,7 @@ def _plan_pieces(pieces, dtype, copies=1, copy_step=0):
     address, destination address, rows, words per row, words between the rows
     of the source, of the destination, copies, words between them)]), or None
     if a piece does not fit the kernel (a layout that is no matrix of
-    contiguous rows, rows of a few elements, 2**31 words or more)."""
+    contiguous rows, many rows of a few elements, 2**31 words or more)."""
     if len(pieces) * copies < 2 or dtype.fields is not None:
         return None
     item = dtype.itemsize
@@ -177,17 +198,15 @@ def _plan_pieces(pieces, dtype, copies=1, copy_step=0):
         else:
             return None
         rows, row = fs[0], fs[1] * words
-        if rows > 1 and row * word < 64:
-            # a few elements per row: the tiled kernels do these better
+        if rows > 1 and row * word < 64 and rows * row * word > _NARROW_PIECE_BYTES:
+            # a few elements per row, and many rows: the tiled kernels do these better
             return None
         sp, dp = fs[2] * words, fd[2] * words
         if sp == row and dp == row:
             # rows follow each other on both sides: one long row
             rows, row = 1, rows * row
             sp = dp = row
-        while row % nv:
-            nv //= 2
-        if rows * row >= 1 << 31:
+        if rows * ((row + nv - 1) // nv) * nv >= 1 << 31:
             return None
         forms.append((sptr, dptr, rows, row, sp, dp, copies, copy_step // word))
     return word, nv, forms
@@ -204,9 +223,10 @@ def _piece_tables(nv, forms):
         table = bytearray(_MAX_PIECES * _PIECE_STRUCT.size)
         blocks = 0
         for k, (sptr, dptr, rows, row, sp, dp, copies, step) in enumerate(batch):
-            n_vecs = rows * (row // nv)
-            _PIECE_STRUCT.pack_into(table, k * _PIECE_STRUCT.size,
-                                    sptr, dptr, sp, dp, row // nv, n_vecs, blocks, copies, step)
+            vecs_per_row = (row + nv - 1) // nv
+            n_vecs = rows * vecs_per_row
+            _PIECE_STRUCT.pack_into(table, k * _PIECE_STRUCT.size, sptr, dptr, sp, dp,
+                                    vecs_per_row, n_vecs, blocks, copies, step, row, 0)
             blocks += (n_vecs + per_block - 1) // per_block
         launches.append((bytes(table), len(batch), blocks))
     return launches
@@ -538,9 +558,15 @@ def roll(a, shift, axis=None):
     out = ndarray(a.shape, a.dtype)
     if out.size == 0:
         return out
+    moves = []
     for combo in itertools.product(*cuts):
         src, dst = zip(*combo)
-        elementwise_copy(a[src], out[dst])
+        moves.append((a[src], out[dst]))
+    if not (_tuning.get('concatenate_one_launch') and _copy_pieces(
+            [(s.shape, s.strides, s.data.ptr, d.strides, d.data.ptr) for s, d in moves],
+            a.dtype, a.nbytes)):
+        for s, d in moves:
+            elementwise_copy(s, d)
     return out
 
 

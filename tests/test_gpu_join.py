@@ -160,9 +160,17 @@ def test_repeat(axis):
 
 def test_roll_and_quarter_turns():
     h, d = pair((5, 6, 7))
-    for shift, axis in [(1, None), (-3, None), (0, None), (212, None), (2, 0), (-1, 2), (9, 1),
-                        ((1, 2), (0, 1)), ((1, -2, 3), (0, 1, 2)), (3, (0, 2)), ((1, 1), (1, 1))]:
-        same(cp.roll(d, shift, axis), np.roll(h, shift, axis))
+    from cupy_amd._core import _tuning
+    hw, dw = pair((40, 3, 129), 'float64', seed=3)      # rows that end in partial vectors
+    try:
+        for on in (True, False):
+            _tuning.set(concatenate_one_launch=on)
+            for shift, axis in [(1, None), (-3, None), (0, None), (212, None), (2, 0), (-1, 2), (9, 1),
+                                ((1, 2), (0, 1)), ((1, -2, 3), (0, 1, 2)), (3, (0, 2)), ((1, 1), (1, 1))]:
+                same(cp.roll(d, shift, axis), np.roll(h, shift, axis))
+                same(cp.roll(dw, shift, axis), np.roll(hw, shift, axis))
+    finally:
+        _tuning.set(concatenate_one_launch=True)
     same(cp.roll(d.transpose(2, 0, 1), 3, 1), np.roll(h.transpose(2, 0, 1), 3, 1))
     with pytest.raises(np.exceptions.AxisError):
         cp.roll(d, 1, 3)

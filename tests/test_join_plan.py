@@ -11,7 +11,8 @@ from cupy_amd import _join
 # struct Piece of the kernel source
 PIECE = np.dtype([('src', np.uint64), ('dst', np.uint64), ('src_pitch', np.int64),
                   ('dst_pitch', np.int64), ('vecs_per_row', np.uint32), ('n_vecs', np.uint32),
-                  ('first_block', np.uint32), ('n_rep', np.uint32), ('rep_step', np.int64)])
+                  ('first_block', np.uint32), ('n_rep', np.uint32), ('rep_step', np.int64),
+                  ('row_len', np.uint32), ('pad', np.uint32)])
 
 
 def describe(pairs):
@@ -30,7 +31,7 @@ def replay(pairs, sbase, dbase, copies=1, copy_step=0):
     block, unroll = _join._geometry()
     per_block = block * unroll
     for table, n_pieces, blocks in _join._piece_tables(nv, forms):
-        assert len(table) == 56 * _join._MAX_PIECES and n_pieces <= _join._MAX_PIECES
+        assert len(table) == 64 * _join._MAX_PIECES and n_pieces <= _join._MAX_PIECES
         table = np.frombuffer(table, PIECE)
         firsts = [int(table[k]['first_block']) for k in range(n_pieces)]
         assert firsts == sorted(firsts) and firsts[0] == 0
@@ -42,15 +43,18 @@ def replay(pairs, sbase, dbase, copies=1, copy_step=0):
             assert local.size, 'a workgroup without work'
             r = local // int(pc['vecs_per_row'])
             c = (local - r * int(pc['vecs_per_row'])) * nv
+            assert int(pc['vecs_per_row']) == -(-int(pc['row_len']) // nv)
+            have = np.minimum(int(pc['row_len']) - c, nv)     # the last vector of a row may be partial
+            assert have.min() >= 1
             src = int(pc['src']) - s0 + (r * int(pc['src_pitch']) + c) * word
             dst = int(pc['dst']) - d0 + (r * int(pc['dst_pitch']) + c) * word
-            assert src.min() >= 0 and src.max() + nv * word <= sw.size
-            assert dst.min() >= 0 and dst.max() + nv * word <= dw.size
+            assert src.min() >= 0 and (src + have * word).max() <= sw.size
             for j in range(int(pc['n_rep'])):
                 at = dst + j * int(pc['rep_step']) * word
-                assert at.min() >= 0 and at.max() + nv * word <= dw.size
+                assert at.min() >= 0 and (at + have * word).max() <= dw.size
                 for b in range(nv * word):
-                    dw[at + b] = sw[src + b]
+                    inside = b < have * word
+                    dw[at[inside] + b] = sw[src[inside] + b]
         # every vector of every piece has a workgroup
         assert blocks == sum(-(-int(table[k]['n_vecs']) // per_block) for k in range(n_pieces))
     return True
@@ -67,6 +71,9 @@ CASES = [
     ((4, 5, 96), [np.s_[:, :, :32], np.s_[:, :, 33:80], np.s_[:, :, 64:]], 2, 'float16'),
     ((2050, 3), [np.s_[:1000], np.s_[1000:]], 0, 'uint8'),
     ((300, 17), [np.s_[i * 10:(i + 1) * 10 + (i % 3)] for i in range(19)], 0, 'float32'),
+    ((33, 67), [np.s_[:, 1:], np.s_[:, :66]], 0, 'float32'),          # rows of 66: partial last vectors
+    ((9, 70), [np.s_[:, :33], np.s_[:, 33:36], np.s_[:, 69:]], 1, 'int8'),   # rows of 33, 3 and 1 bytes
+    ((50, 3), [np.s_[:, :2], np.s_[:, 2:]], 1, 'float64'),             # a small piece of narrow rows
 ]
 
 
@@ -99,8 +106,8 @@ def test_layouts_the_kernel_declines():
     # transposed pieces, rows of a few elements, a single piece, reversed rows
     t = np.zeros((50, 80), np.float32)
     assert plan([(base.T, t[:, :40]), (base.T, t[:, 40:])]) is None
-    narrow = np.zeros((40, 3), np.float32)
-    wide = np.zeros((40, 6), np.float32)
+    narrow = np.zeros((100000, 3), np.float32)            # many rows of a few elements
+    wide = np.zeros((100000, 6), np.float32)
     assert plan([(narrow, wide[:, :3]), (narrow, wide[:, 3:])]) is None
     assert plan([(base, out[:40])]) is None
     rev = base[::-1]
