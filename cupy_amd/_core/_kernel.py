@@ -1939,6 +1939,23 @@ def _read_loop_entry(entry, default):
     return signature, None, own
 
 
+def _weak_int_misfits(op, in_args):
+    """Whether a weak Python integer among the inputs lies outside the
+    integer type of its loop input while the loop's result is of another kind
+    than integer (for loops with integer results NumPy raises, and so does the
+    conversion of the scalar later on)."""
+    if op.out_types and numpy.dtype(op.out_types[0]).kind in 'iu':
+        return False
+    for x, t in zip(in_args, op.in_types):
+        if type(x) is CScalar and x.weak_t is int:
+            t = numpy.dtype(t)
+            if t.kind in 'iu':
+                info = numpy.iinfo(t)
+                if not info.min <= x.value <= info.max:
+                    return True
+    return False
+
+
 def _loop_selection_types(in_args):
     """``(dtypes, weak types or None)`` of preprocessed inputs, as loop selection
     sees them: a Python scalar counts as weak only where
@@ -2162,6 +2179,17 @@ class ufunc:
 
         op = self._ops.guess_routine(
             self.name, self._routine_cache, in_args, dtype, self._out_ops)
+        if dtype is None and _weak_int_misfits(op, in_args):
+            # a Python integer outside the integer type the arrays chose, in a
+            # loop that answers in another kind (a comparison, a true division,
+            # a logical function): NumPy computes with the integer's value, so
+            # it counts as a 64-bit integer of its own instead of wrapping or
+            # raising (``uint8_array == -1`` is all False, ``uint8_array / -1``
+            # is negative)
+            in_args = [CScalar(x.value, x.descr) if type(x) is CScalar and x.weak_t is int
+                       else x for x in in_args]
+            op = self._ops.guess_routine(
+                self.name, self._routine_cache, in_args, dtype, self._out_ops)
 
         # outputs are of the first array subclass among the inputs
         template = next((a for a in in_args

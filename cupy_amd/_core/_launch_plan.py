@@ -161,7 +161,7 @@ class FastCall:
     """Recorded call: allocates outputs and temporaries, patches pointers and
     scalar values, launches."""
     __slots__ = ('n_user', 'out_specs', 'temps', 'launches', 'ret', 'overlap', 'quick',
-                 'stream', 'device')
+                 'stream', 'device', 'int_scalars')
 
     def __init__(self, n_user, out_specs, rec, ret, overlap=()):
         self.n_user = n_user
@@ -171,6 +171,12 @@ class FastCall:
         self.ret = ret                        # ref, tuple of refs, or None
         self.overlap = tuple(overlap)         # (input ref, output ref) pairs to check
         self.quick = _quick_launches(self.launches)
+        # scalar arguments that are packed as integers: a Python integer outside
+        # the type takes the full path, which raises or chooses another loop
+        # as NumPy does
+        self.int_scalars = tuple(sorted({
+            (ref, descr) for launch in self.launches for _, ref, descr in launch[6]
+            if descr in _INT_LIMITS}, key=lambda rd: rd[0]))
         self.stream = rec.stream
         self.device = rec.device
 
@@ -192,6 +198,12 @@ class FastCall:
             # reduction is a plain launch, cupy/_core/_reduction.pyx:481-508)
             if not _giveup.usable(self.device, _giveup.REDUCTION):
                 return NotImplemented
+        for ref, descr in self.int_scalars:
+            v = args[ref]
+            if type(v) is int:
+                lo, hi = _INT_LIMITS[descr]
+                if not lo <= v <= hi:
+                    return NotImplemented
         for i, o in self.overlap:
             a, b = args[i], args[o]
             # (arrays of different allocations cannot overlap)

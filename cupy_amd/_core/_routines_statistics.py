@@ -395,13 +395,15 @@ _nanmean_func = create_reduction_func(
     'cupy_nanmean',
     (('e->e', ('nanmean_st<float>(static_cast<float>(in0))', None,
                'out0 = a.value / float(a.count)', 'nanmean_st<float>')),
-     'f->f', 'd->d'),
+     'f->f', 'd->d',
+     ('F->F', (None, None, 'out0 = a.value / float(a.count)', None)),
+     ('D->D', (None, None, 'out0 = a.value / double(a.count)', None))),
     ('nanmean_st<type_out0_raw>(in0)', 'my_nanmean(a, b)',
      'out0 = a.value / type_out0_raw(a.count)', 'nanmean_st<type_out0_raw>'),
     None, _nanmean_preamble)
 
 _count_non_nan = create_reduction_func(
-    'cupy_count_non_nan', ('e->q', 'f->q', 'd->q'),
+    'cupy_count_non_nan', ('e->q', 'f->q', 'd->q', 'F->q', 'D->q'),
     ('(in0 == in0) ? 1 : 0', 'a + b', 'out0 = a', None), 0)
 
 
@@ -584,6 +586,10 @@ template <typename S, typename T>
 __device__ T nanvar_impl(S x, T mean, long long alpha) {
   return ((x != x) ? T(0) : T((x - mean) * (x - mean))) / alpha;
 }
+template <typename S, typename T>
+__device__ T nanvar_impl(complex<S> x, complex<T> mean, long long alpha) {
+  return ((x != x) ? T(0) : T(norm(x - mean))) / alpha;
+}
 '''
 
 _nanvar_cores = {}
@@ -604,6 +610,25 @@ def _nanvar(a, axis, dtype, out, ddof, keepdims):
             'a + b', 'out = a', '0', '_nanvar_core', preamble=_nanvar_preamble)
     count = _count_non_nan(a, axis=axis, keepdims=True)
     arrsum = _routines_math.nansum(a, axis=axis, dtype=dtype, out=None, keepdims=True)
+    if a.dtype.kind == 'c':
+        # the squared modulus of the deviations: a real result
+        # (cupy/_core/_routines_statistics.pyx:751-762, 790-800)
+        real = 'float32' if a.dtype.itemsize == 8 else 'float64'
+        key = 'complex:' + real
+        if key not in _nanvar_cores:
+            ctype = 'float' if real == 'float32' else 'double'
+            _nanvar_cores[key] = ReductionKernel(
+                '%s x, %s sum, int64 _count, int64 ddof' % (a.dtype.name, a.dtype.name),
+                '%s out' % real,
+                'nanvar_impl(x, sum / static_cast<%s>(_count), max(_count - ddof, 0LL))' % ctype,
+                'a + b', 'out = a', '0', '_nanvar_core_' + a.dtype.name, preamble=_nanvar_preamble)
+        var = _nanvar_cores[key](a, arrsum.astype(a.dtype, copy=False), count, ddof,
+                                 axis=axis, keepdims=keepdims)
+        if out is None:
+            return var
+        from cupy_amd._core._ufuncs import elementwise_copy
+        elementwise_copy(var, out)
+        return out
     if out is None:
         return _nanvar_cores['new'](a, arrsum, count, ddof, axis=axis, keepdims=keepdims)
     _nanvar_cores['out'](a, arrsum, count, ddof, out, axis=axis, keepdims=keepdims)

@@ -2,6 +2,8 @@
 nan-variants) against NumPy on the same seeded inputs.  Integer results are
 bit-exact; floating-point results are compared within the reduction tolerance
 (the evaluation order differs from NumPy's)."""
+import warnings
+
 import numpy as np
 import pytest
 
@@ -536,3 +538,34 @@ def test_sums_of_negative_zeros_stay_negative(shape, axis, dtype):
         want = np.nancumsum(hn, axis=axis)
         got = cp.nancumsum(cp.asarray(hn), axis=axis).get()
         assert (np.signbit(got) == np.signbit(want)).all()
+
+
+@pytest.mark.parametrize('dtype', ['complex64', 'complex128'])
+def test_nan_statistics_of_complex_values(dtype):
+    """nanmean / nanvar / nanstd over complex values: an element counts as NaN
+    if either part is; the variance is the mean squared modulus of the
+    deviations, a real number (reference: _routines_statistics.pyx:686-700,
+    732-800)."""
+    rng = np.random.default_rng(8)
+    h = (rng.standard_normal((9, 11, 5)) + 1j * rng.standard_normal((9, 11, 5))).astype(dtype)
+    h[0, 0, 0] = np.nan
+    h[3, 4, 1] = complex(1.0, np.nan)
+    h[:, 7, 2] = np.nan                     # a whole slice along axis 0
+    d = cp.asarray(h)
+    rtol = 2e-5 if dtype == 'complex64' else 1e-12
+    for kwargs in ({}, {'axis': 0}, {'axis': (0, 2)}, {'axis': 1, 'keepdims': True}, {'axis': -1}):
+        for name in ('nanmean', 'nanvar', 'nanstd'):
+            with np.errstate(all='ignore'), warnings.catch_warnings():
+                warnings.simplefilter('ignore')
+                want = getattr(np, name)(h, **kwargs)
+            got = getattr(cp, name)(d, **kwargs)
+            assert got.dtype == want.dtype and got.shape == np.shape(want), (name, kwargs)
+            np.testing.assert_allclose(got.get(), want, rtol=rtol, atol=rtol, equal_nan=True)
+    for name in ('nanvar', 'nanstd'):
+        with np.errstate(all='ignore'):
+            want = getattr(np, name)(h, axis=1, ddof=1)
+        np.testing.assert_allclose(getattr(cp, name)(d, axis=1, ddof=1).get(), want, rtol=rtol, atol=rtol,
+                                   equal_nan=True)
+    out = cp.empty((9, 5), want.dtype)
+    assert cp.nanvar(d, axis=1, out=out) is out
+    np.testing.assert_allclose(out.get(), np.nanvar(h, axis=1), rtol=rtol, atol=rtol, equal_nan=True)

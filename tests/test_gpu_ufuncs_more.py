@@ -178,3 +178,33 @@ def test_around_follows_numpy():
         return cp.around(a * 3, 1) + cp.real(a)
     x32 = x.astype(np.float32)
     assert_exact(f(cp.asarray(x32)).get(), np.around(x32 * 3, 1) + np.real(x32))
+
+
+def test_python_integers_outside_the_arrays_type():
+    """A Python integer that does not fit the arrays' integer type: loops that
+    answer in another kind (comparisons, true division, logical functions)
+    compute with its value as NumPy does; loops with integer results raise as
+    NumPy does."""
+    for dtype in ('uint8', 'int8', 'uint64'):
+        h = np.array([0, 1, 5, 100], dtype)
+        d = cp.asarray(h)
+        for value in (-1, 300, -(1 << 40)):
+            for name in ('equal', 'not_equal', 'less', 'greater_equal', 'true_divide',
+                         'logical_xor', 'logical_and'):
+                with np.errstate(all='ignore'):
+                    want = getattr(np, name)(h, value)
+                    back = getattr(np, name)(value, h)
+                got = getattr(cp, name)(d, value)
+                assert got.dtype == want.dtype, (name, dtype, value)
+                np.testing.assert_array_equal(got.get(), want)
+                np.testing.assert_array_equal(getattr(cp, name)(value, d).get(), back)
+            assert np.array_equal((d == value).get(), h == value)
+            assert np.array_equal((value > d).get(), value > h)
+            for name in ('add', 'maximum', 'floor_divide', 'bitwise_and'):
+                info = np.iinfo(dtype)
+                if info.min <= value <= info.max:
+                    continue
+                with pytest.raises(OverflowError):
+                    getattr(np, name)(h, value)
+                with pytest.raises(OverflowError):
+                    getattr(cp, name)(d, value)

@@ -492,3 +492,20 @@ def test_retired_blocks_are_freed_two_retirements_later():
     finally:
         _reduce_sync._blocks.clear()
         _reduce_sync._blocks.update(saved)
+
+
+def test_a_python_integer_outside_the_recorded_type_is_not_replayed():
+    """A record made with a Python integer that fitted the arrays' type must
+    not pack one that does not: the call goes the full way, which chooses
+    another loop (comparisons) or raises (arithmetic) as NumPy does."""
+    import numpy as np
+    import cupy_amd as cp
+    a = cp.ndarray((5,), np.int8)
+    for value in (-1, -1, -1, 300, 300, -1, 1 << 40):
+        assert (a == value).dtype == np.bool_
+        assert cp.true_divide(a, value).dtype == np.float64
+    for value in (1, 1, 1):
+        assert cp.add(a, value).dtype == np.int8
+    with pytest.raises(OverflowError):
+        cp.add(a, 300)
+    assert cp.add(a, 2).dtype == np.int8
