@@ -1992,7 +1992,7 @@ def _input_fits(given, wanted, weak):
         return False
 
 
-_UFUNC_KEYWORDS = frozenset(('out', '_where', 'dtype', 'casting'))
+_UFUNC_KEYWORDS = frozenset(('out', '_where', 'where', 'dtype', 'casting'))
 
 
 def _preprocess_where(dev_id, where):
@@ -2079,7 +2079,13 @@ class ufunc:
                 raise ValueError(
                     "The 'out' tuple must have exactly one entry per ufunc output"
                     if as_tuple else "'out' must be a tuple of arrays")
-        return (inputs, outputs, kwargs.get('_where'), dtype,
+        where = kwargs.get('_where')
+        if where is None:
+            # NumPy's spelling; True, its default, selects every element
+            where = kwargs.get('where')
+            if where is True:
+                where = None
+        return (inputs, outputs, where, dtype,
                 kwargs.get('casting', self._default_casting))
 
     def __call__(self, *args, **kwargs):
@@ -2179,6 +2185,15 @@ class ufunc:
 
         op = self._ops.guess_routine(
             self.name, self._routine_cache, in_args, dtype, self._out_ops)
+        if dtype is not None:
+            # the loop was chosen by its result: the arrays must be castable
+            # to its inputs under the rule, as NumPy demands (a complex array
+            # does not silently lose its imaginary part to ``dtype=float``)
+            for i, (x, t) in enumerate(zip(in_args, op.in_types)):
+                if isinstance(x, ndarray) and not numpy.can_cast(x.dtype, t, casting):
+                    raise TypeError(
+                        "Cannot cast ufunc '%s' input %d from %r to %r with casting rule '%s'"
+                        % (self.name.replace('cupy_', ''), i, x.dtype, numpy.dtype(t), casting))
         if dtype is None and _weak_int_misfits(op, in_args):
             # a Python integer outside the integer type the arrays chose, in a
             # loop that answers in another kind (a comparison, a true division,

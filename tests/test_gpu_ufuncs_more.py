@@ -3,6 +3,8 @@ inputs: integer and boolean results bit-exact, floating-point results within a
 few ulp (the device's math library is not NumPy's libm: parity of those
 functions is checked to the reference's own tolerance,
 tests/cupy_tests/math_tests/*: ``numpy_cupy_allclose(atol=1e-5)``)."""
+import warnings
+
 import numpy as np
 import pytest
 
@@ -208,3 +210,47 @@ def test_python_integers_outside_the_arrays_type():
                     getattr(np, name)(h, value)
                 with pytest.raises(OverflowError):
                     getattr(cp, name)(d, value)
+
+
+def test_where_keyword_and_input_casts_under_dtype():
+    """``where=`` as NumPy spells it (elements it leaves out keep what ``out``
+    held), and ``dtype=``: the arrays must be castable to the chosen loop's
+    inputs under the casting rule."""
+    rng = np.random.default_rng(2)
+    h = rng.standard_normal((5, 7)).astype(np.float32)
+    g = rng.standard_normal((5, 7)).astype(np.float32)
+    mask = rng.integers(0, 2, (5, 7)).astype(bool)
+    d, e, dm = cp.asarray(h), cp.asarray(g), cp.asarray(mask)
+    want = np.full((5, 7), 9, np.float32)
+    np.add(h, g, out=want, where=mask)
+    out = cp.asarray(np.full((5, 7), 9, np.float32))
+    assert cp.add(d, e, out=out, where=dm) is out
+    np.testing.assert_array_equal(out.get(), want)
+    np.testing.assert_array_equal(cp.add(d, e, where=True).get(), h + g)
+    row = mask[0]
+    want = np.full((5, 7), 3, np.float64)
+    np.multiply(h, 2, out=want, where=row)
+    out = cp.asarray(np.full((5, 7), 3, np.float64))
+    cp.multiply(d, 2, out=out, where=cp.asarray(row))
+    np.testing.assert_array_equal(out.get(), want)
+
+    z = (rng.standard_normal(6) + 1j * rng.standard_normal(6)).astype(np.complex128)
+    dz = cp.asarray(z)
+    for casting in ('same_kind', 'safe'):
+        with pytest.raises(TypeError):
+            np.multiply(z, 2.0, dtype=np.float64, casting=casting)
+        with pytest.raises(TypeError):
+            cp.multiply(dz, 2.0, dtype=np.float64, casting=casting)
+    with warnings.catch_warnings():
+        warnings.simplefilter('ignore')
+        want = np.multiply(z, 2.0, dtype=np.float64, casting='unsafe')
+        got = cp.multiply(dz, 2.0, dtype=np.float64, casting='unsafe')
+    np.testing.assert_array_equal(got.get(), want)
+    i = np.arange(6, dtype=np.int64)
+    with pytest.raises(TypeError):
+        cp.negative(cp.asarray(i), dtype=np.uint8)
+    with pytest.raises(TypeError):
+        cp.true_divide(cp.asarray(i.astype(np.uint64)), cp.asarray(i.astype(np.uint32)), dtype=np.float32,
+                       casting='safe')
+    np.testing.assert_array_equal(cp.add(cp.asarray(i.astype(np.int16)), 1, dtype=np.float64).get(),
+                                  np.add(i.astype(np.int16), 1, dtype=np.float64))
