@@ -2218,6 +2218,20 @@ class ufunc:
         if 0 in shape:
             return ret
 
+        if has_where and any(o.dtype != t for o, t in zip(out_args, core_out_dtypes)):
+            # The kernel keeps what a masked-out element held by reading it as
+            # the loop's result type, which cannot hold every value of another
+            # type (a comparison into an integer array turned every skipped
+            # element into 0 or 1).  Such a call computes into arrays of the
+            # loop's types, converts them, and copies under the mask between
+            # arrays of ONE type.
+            from cupy_amd._core._ufuncs import elementwise_copy
+            plain = {k: v for k, v in kwargs.items() if k in ('dtype', 'casting')}
+            fresh = self(*args[:self.nin], **plain)
+            for o, r in zip(out_args, fresh if self.nout > 1 else (fresh,)):
+                elementwise_copy(r.astype(o.dtype, copy=False), o, _where=where)
+            return ret
+
         for i, t in enumerate(core_in_dtypes):
             if type(in_args[i]) is CScalar:
                 in_args[i].apply_dtype(t)

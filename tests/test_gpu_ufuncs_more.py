@@ -254,3 +254,24 @@ def test_where_keyword_and_input_casts_under_dtype():
                        casting='safe')
     np.testing.assert_array_equal(cp.add(cp.asarray(i.astype(np.int16)), 1, dtype=np.float64).get(),
                                   np.add(i.astype(np.int16), 1, dtype=np.float64))
+
+
+@pytest.mark.parametrize('out_dtype', ['uint64', 'bool', 'int8', 'float32', 'complex64'])
+def test_where_into_an_output_of_another_type_keeps_the_skipped_elements(out_dtype):
+    h = np.arange(0, 12, dtype=np.int8)          # (negative floats into unsigned types are undefined)
+    g = np.full(12, 3, np.int64)
+    mask = (np.arange(12) % 3 != 1)
+    d, e, dm = cp.asarray(h), cp.asarray(g), cp.asarray(mask)
+    for name, casting in (('less', 'same_kind'), ('logical_and', 'unsafe'), ('add', 'unsafe'),
+                          ('true_divide', 'unsafe')):
+        want = np.full(12, 7).astype(out_dtype)
+        try:
+            getattr(np, name)(h, g, out=want, where=mask, casting=casting)
+        except TypeError:
+            with pytest.raises(TypeError):
+                getattr(cp, name)(d, e, out=cp.asarray(np.full(12, 7).astype(out_dtype)), where=dm,
+                                  casting=casting)
+            continue
+        out = cp.asarray(np.full(12, 7).astype(out_dtype))
+        assert getattr(cp, name)(d, e, out=out, where=dm, casting=casting) is out
+        np.testing.assert_array_equal(out.get(), want)
