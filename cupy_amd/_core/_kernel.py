@@ -2186,6 +2186,17 @@ class ufunc:
         op = self._ops.guess_routine(
             self.name, self._routine_cache, in_args, dtype, self._out_ops)
         if dtype is not None:
+            # several loops may give that result type (every comparison gives
+            # bool): NumPy takes the first one the arrays can be cast to safely
+            same_result = [o for o in (self._out_ops or self._ops).ops
+                           if all(t == dtype for t in o.out_types)]
+            if len(same_result) > 1:
+                for candidate in same_result:
+                    if all(not isinstance(x, ndarray) or numpy.can_cast(x.dtype, t, 'safe')
+                           for x, t in zip(in_args, candidate.in_types)):
+                        op = candidate
+                        op.check_valid()
+                        break
             # the loop was chosen by its result: the arrays must be castable
             # to its inputs under the rule, as NumPy demands (a complex array
             # does not silently lose its imaginary part to ``dtype=float``)
