@@ -177,7 +177,7 @@ class Proxy:
         # squaring is a multiply, not a call to pow()
         if type(other) in (int, float):
             kind = self._value.dtype.kind
-            if other == 2 and kind in 'iuf':
+            if other == 2 and (kind in 'fc' or (kind in 'iub' and type(other) is int)):
                 return _u('square')(self)
             if kind == 'f' and other == 0.5:
                 return _u('sqrt')(self)

@@ -766,7 +766,7 @@ class ndarray:
                 return _ufuncs.reciprocal(self)
             if other == 1:
                 return _ufuncs.positive(self)
-        elif type(other) is int and other == 2 and self.dtype.kind in 'iu':
+        elif type(other) is int and other == 2 and self.dtype.kind in 'iub':
             return _ufuncs.square(self)
         return self._binary('power', other)
 

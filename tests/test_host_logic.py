@@ -205,3 +205,15 @@ def test_merge_dims_of_reduction_axes():
     t = a.transpose(1, 0, 2, 3)
     shape, strides = _reduction._merge_dims(t.shape[:2], [t.strides[:2]])
     assert shape == [5, 6]
+
+
+def test_squaring_short_cut_follows_numpy_result_types():
+    """``x ** 2`` with a Python exponent squares (bool gives int8, integers
+    keep their type); a float exponent on integers does not."""
+    import cupy_amd as cp
+    for dt in ('bool', 'int8', 'uint16', 'int64', 'float16', 'float32', 'complex64'):
+        a = cp.ndarray((3,), dt)
+        h = np.ones(3, dt)
+        for e in (2, 3, 0.5) + ((2.0,) if dt != 'bool' else ()):
+            assert (a ** e).dtype == (h ** e).dtype, (dt, e)
+            assert cp.fuse(lambda x: x ** e)(a).dtype == (h ** e).dtype, (dt, e)
