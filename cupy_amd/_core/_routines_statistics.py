@@ -396,8 +396,11 @@ _nanmean_func = create_reduction_func(
     (('e->e', ('nanmean_st<float>(static_cast<float>(in0))', None,
                'out0 = a.value / float(a.count)', 'nanmean_st<float>')),
      'f->f', 'd->d',
-     ('F->F', (None, None, 'out0 = a.value / float(a.count)', None)),
-     ('D->D', (None, None, 'out0 = a.value / double(a.count)', None))),
+     # (the input may be real when ``dtype=`` asked for a complex mean)
+     ('F->F', ('nanmean_st<type_out0_raw>(type_out0_raw(in0))', None,
+               'out0 = a.value / float(a.count)', None)),
+     ('D->D', ('nanmean_st<type_out0_raw>(type_out0_raw(in0))', None,
+               'out0 = a.value / double(a.count)', None))),
     ('nanmean_st<type_out0_raw>(in0)', 'my_nanmean(a, b)',
      'out0 = a.value / type_out0_raw(a.count)', 'nanmean_st<type_out0_raw>'),
     None, _nanmean_preamble)

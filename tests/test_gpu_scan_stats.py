@@ -569,3 +569,17 @@ def test_nan_statistics_of_complex_values(dtype):
     out = cp.empty((9, 5), want.dtype)
     assert cp.nanvar(d, axis=1, out=out) is out
     np.testing.assert_allclose(out.get(), np.nanvar(h, axis=1), rtol=rtol, atol=rtol, equal_nan=True)
+
+
+def test_nanmean_of_real_values_with_a_complex_result_type():
+    rng = np.random.default_rng(12)
+    for dtype in ('float16', 'float32', 'float64'):
+        h = rng.standard_normal((7, 9)).astype(dtype)
+        h[2, 3] = np.nan
+        d = cp.asarray(h)
+        for out in ('complex64', 'complex128'):
+            for kwargs in ({}, {'axis': 0}, {'axis': 1}):
+                want = np.nanmean(h, dtype=out, **kwargs)
+                got = cp.nanmean(d, dtype=out, **kwargs)
+                assert got.dtype == want.dtype
+                np.testing.assert_allclose(got.get(), want, rtol=2e-3 if dtype == 'float16' else 1e-5)
